@@ -1,0 +1,69 @@
+// C ABI of the kernel library.  Every function launches on `stream`, returns 0 on success or a
+// negative value after recording a message for fllm_last_error(), and never allocates device
+// memory.  Element type codes: 0 = float32, 1 = bfloat16.  All tensors are dense row-major
+// unless a stride is given.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char *fllm_last_error(void);
+int fllm_abi_version(void);
+
+// out[r, :] = scale * table[ids[r], :]            out: float32 [rows, width]
+int fllm_embed(const int32_t *ids, const void *table, float *out, int rows, int width, int vocab, int table_dtype,
+               float scale, hipStream_t stream);
+
+// out[i, :] = x[row(i), :] * (rsqrt(mean(x[row(i)]^2) + eps) * weight),  row(i) = rows ? rows[i] : i
+int fllm_rmsnorm(const float *x, const int32_t *rows, const float *weight, void *out, int count, int width, float eps,
+                 int out_dtype, hipStream_t stream);
+
+// y[m, n] = sum_k x[m, k] * w[n, k] (+ bias[n]);   x: [M, K] (row stride ldx), w: [N, K]
+// out_mode 0: store as `dtype`; 1: store float32; 2: add to float32 `out` (row stride ldo)
+int fllm_linear(const void *x, int ldx, const void *w, const float *bias, void *out, int ldo, int M, int N, int K,
+                int dtype, int out_mode, hipStream_t stream);
+
+// out[r, j] = silu(gu[r, j]) * gu[r, I + j]
+int fllm_swiglu(const void *gate_up, void *out, int rows, int inter, int dtype, hipStream_t stream);
+
+// Rotates the query and key heads of qkv rows in place and stores keys and values in pages.
+// qkv: [rows, (heads + 2 kv_heads) * head_dim]; row r belongs to segment row_seg[r] at position
+// row_pos[r]; its page is tables[row_seg[r] * table_stride + row_pos[r] / page_size].
+// K pages: [page][kv_head][token][head_dim]; V pages: [page][kv_head][head_dim][token].
+// pairing 0: lanes (l, l + rope_dims/2); 1: lanes (2l, 2l + 1).  store_kv 0 leaves the pages alone.
+int fllm_rope_kv_store(void *qkv, const int32_t *row_pos, const int32_t *row_seg, const int32_t *tables,
+                       int table_stride, const float *cos_table, const float *sin_table, int table_positions,
+                       void *k_pages, void *v_pages, int num_pages, int rows, int heads, int kv_heads, int head_dim,
+                       int rope_dims, int pairing, int page_size, int dtype, int store_kv, hipStream_t stream);
+
+// Causal attention of each row over the pages of its segment: keys at positions
+// [max(0, pos - window + 1), pos] (window <= 0: from 0).  q: rows of `q_stride` elements, head h at
+// h * head_dim.  out: [rows, heads * head_dim].  `workspace` holds partial results of split
+// contexts (fllm_attention_workspace_bytes()).
+int fllm_attention(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables,
+                   int table_stride, const int32_t *row_pos, const int32_t *row_seg, void *out, int rows, int heads,
+                   int kv_heads, int head_dim, int page_size, int num_pages, float scale, int window, int dtype,
+                   int max_context, int uniform_rows, void *workspace, size_t workspace_bytes, hipStream_t stream);
+size_t fllm_attention_workspace_bytes(int rows, int heads, int head_dim, int max_context);
+
+// out[r] = first index of the largest finite value of logits[r, :]
+int fllm_argmax(const float *logits, int32_t *out, int rows, int vocab, hipStream_t stream);
+
+struct FllmSampleRow {
+    float temperature;   // <= 1e-5: greedy
+    float top_p;         // nucleus; outside (0, 1): off
+    int32_t top_k;       // <= 0: off
+    int32_t pad;
+    uint64_t seed;       // Philox key
+    uint64_t draw;       // number of the draw of this request
+};
+// work: float32 [rows, vocab] scratch (may alias logits)
+int fllm_sample(const float *logits, float *work, const struct FllmSampleRow *params, int32_t *out, int rows, int vocab,
+                hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif

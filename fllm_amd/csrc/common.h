@@ -1,0 +1,71 @@
+// Shared helpers of the gfx950 kernels: element types, wave64 reductions, error reporting.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define FLLM_F32 0
+#define FLLM_BF16 1
+
+typedef __bf16 bf16_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+constexpr int kWave = 64;
+
+// Records the first failure of a call; every entry point returns 0 or a negative code and the
+// text is read back through fllm_last_error().
+void fllm_set_error(const char *fmt, ...);
+int fllm_check_launch(const char *what);
+
+#define FLLM_REQUIRE(cond, ...)            \
+    do {                                   \
+        if (!(cond)) {                     \
+            fllm_set_error(__VA_ARGS__);   \
+            return -1;                     \
+        }                                  \
+    } while (0)
+
+template <typename T> __device__ __forceinline__ float to_f32(T v);
+template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_f32<bf16_t>(bf16_t v) { return (float)v; }
+
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return (bf16_t)v; }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+
+// Sum over a workgroup of NW waves, the same value in every thread; the waves' partial sums
+// are added in wave order, so the result depends only on the data and the launch shape.
+template <int NW> __device__ __forceinline__ float block_sum(float v, float *scratch /* NW floats */) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) scratch[threadIdx.x / kWave] = v;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int i = 0; i < NW; i++) total += scratch[i];
+    return total;
+}
+template <int NW> __device__ __forceinline__ float block_max(float v, float *scratch) {
+    v = wave_max(v);
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) scratch[threadIdx.x / kWave] = v;
+    __syncthreads();
+    float total = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NW; i++) total = fmaxf(total, scratch[i]);
+    return total;
+}

@@ -1,0 +1,26 @@
+// Error reporting shared by the entry points.
+#include "api.h"
+#include "common.h"
+#include <stdarg.h>
+#include <stdio.h>
+
+static thread_local char g_error[512] = "";
+
+void fllm_set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+int fllm_check_launch(const char *what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        fllm_set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+        return -2;
+    }
+    return 0;
+}
+
+extern "C" const char *fllm_last_error(void) { return g_error; }
+extern "C" int fllm_abi_version(void) { return 1; }

@@ -1,0 +1,250 @@
+// Sampling on the device: one workgroup per row of logits.
+//
+// Greedy rows take the first index of the largest finite value.  Other rows follow the
+// reference's device sampler (rust/engine/cuda/sampling.cu:1-13, :253-352): temperature, top-k
+// (ties at the threshold are kept), top-p (smallest set of largest values whose mass reaches
+// top_p, ties kept), then a Gumbel-max draw: argmax of (logit - max) / T - ln(-ln u_i) over the
+// survivors, u_i from Philox-4x32-10 keyed by the request's seed with counter
+// (token id, 0, draw_lo, draw_hi) (rust/engine/src/sampling.rs:155-179).  The result depends on
+// (seed, draw, logits) only: not on the batch, the row or the launch.
+#include "api.h"
+#include "common.h"
+
+namespace {
+
+constexpr int kBlock = 1024;
+constexpr int kWaves = kBlock / kWave;
+
+struct Shared {
+    double dred[kWaves];
+    float fred[kWaves];
+    int ired[kWaves];
+    unsigned hist[256];
+    uint32_t prefix;
+    int remaining;
+};
+
+__device__ __forceinline__ void philox4x32_10(uint32_t c[4], uint32_t k0, uint32_t k1) {
+#pragma unroll
+    for (int i = 0; i < 10; i++) {
+        const uint32_t hi0 = __umulhi(0xD2511F53u, c[0]), lo0 = 0xD2511F53u * c[0];
+        const uint32_t hi1 = __umulhi(0xCD9E8D57u, c[2]), lo1 = 0xCD9E8D57u * c[2];
+        const uint32_t n0 = hi1 ^ c[1] ^ k0, n2 = hi0 ^ c[3] ^ k1;
+        c[0] = n0; c[1] = lo1; c[2] = n2; c[3] = lo0;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+}
+
+// a number in the open interval (0, 1)
+__device__ __forceinline__ float philox_uniform(uint64_t seed, uint64_t draw, uint32_t index) {
+    uint32_t c[4] = {index, 0u, (uint32_t)draw, (uint32_t)(draw >> 32)};
+    philox4x32_10(c, (uint32_t)seed, (uint32_t)(seed >> 32));
+    return ((float)(c[0] >> 8) + 0.5f) / 16777216.0f;
+}
+
+// order-preserving map of floats to unsigned integers (larger float, larger key)
+__device__ __forceinline__ uint32_t f2key(float f) {
+    const uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+__device__ __forceinline__ double block_sum_d(double v, Shared &sh) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) sh.dred[threadIdx.x / kWave] = v;
+    __syncthreads();
+    double total = 0.0;
+#pragma unroll
+    for (int i = 0; i < kWaves; i++) total += sh.dred[i];
+    __syncthreads();
+    return total;
+}
+
+__device__ __forceinline__ float block_max_f(float v, Shared &sh) {
+    v = wave_max(v);
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) sh.fred[threadIdx.x / kWave] = v;
+    __syncthreads();
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < kWaves; i++) m = fmaxf(m, sh.fred[i]);
+    __syncthreads();
+    return m;
+}
+
+// largest value, lowest index on ties; index INT_MAX when nothing qualified
+__device__ __forceinline__ int block_argmax(float v, int idx, Shared &sh) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(v, o, kWave);
+        const int oi = __shfl_xor(idx, o, kWave);
+        if (ov > v || (ov == v && oi < idx)) {
+            v = ov;
+            idx = oi;
+        }
+    }
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        sh.fred[threadIdx.x / kWave] = v;
+        sh.ired[threadIdx.x / kWave] = idx;
+    }
+    __syncthreads();
+    float best = sh.fred[0];
+    int besti = sh.ired[0];
+#pragma unroll
+    for (int i = 1; i < kWaves; i++) {
+        if (sh.fred[i] > best || (sh.fred[i] == best && sh.ired[i] < besti)) {
+            best = sh.fred[i];
+            besti = sh.ired[i];
+        }
+    }
+    __syncthreads();
+    return besti;
+}
+
+__device__ __forceinline__ float sanitize(float v) { return isfinite(v) ? v : -INFINITY; }
+
+__device__ int row_argmax(const float *w, int vocab, Shared &sh) {
+    float best = -INFINITY;
+    int besti = 0x7fffffff;
+    for (int i = threadIdx.x; i < vocab; i += kBlock) {
+        const float v = w[i];
+        if (isfinite(v) && v > best) {   // indices rise, so the first maximum stays
+            best = v;
+            besti = i;
+        }
+    }
+    return block_argmax(best, besti, sh);
+}
+
+// key of the k-th largest value of w (every element counts): radix select, 4 passes of 8 bits
+__device__ uint32_t kth_largest_key(const float *w, int vocab, int k, Shared &sh) {
+    if (threadIdx.x == 0) {
+        sh.prefix = 0;
+        sh.remaining = k;
+    }
+    __syncthreads();
+    for (int pass = 0; pass < 4; pass++) {
+        const int shift = 24 - 8 * pass;
+        for (int i = threadIdx.x; i < 256; i += kBlock) sh.hist[i] = 0;
+        __syncthreads();
+        const uint32_t prefix = sh.prefix;
+        for (int i = threadIdx.x; i < vocab; i += kBlock) {
+            const uint32_t key = f2key(w[i]);
+            const bool match = pass == 0 || (key >> (shift + 8)) == (prefix >> (shift + 8));
+            if (match) atomicAdd(&sh.hist[(key >> shift) & 255u], 1u);
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int acc = 0;
+            const int rem = sh.remaining;
+            uint32_t bin = 0;
+            for (int b = 255; b >= 0; b--) {
+                if (acc + (int)sh.hist[b] >= rem) {
+                    bin = (uint32_t)b;
+                    break;
+                }
+                acc += (int)sh.hist[b];
+            }
+            sh.prefix = prefix | (bin << shift);
+            sh.remaining = rem - acc;
+        }
+        __syncthreads();
+    }
+    return sh.prefix;
+}
+
+__global__ void __launch_bounds__(kBlock)
+argmax_kernel(const float *__restrict__ logits, int32_t *__restrict__ out, int vocab) {
+    __shared__ Shared sh;
+    const int idx = row_argmax(logits + (size_t)blockIdx.x * vocab, vocab, sh);
+    if (threadIdx.x == 0) out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
+}
+
+__global__ void __launch_bounds__(kBlock)
+sample_kernel(const float *logits, float *work, const FllmSampleRow *__restrict__ params,
+              int32_t *__restrict__ out, int vocab) {
+    __shared__ Shared sh;
+    const int row = blockIdx.x;
+    const FllmSampleRow p = params[row];
+    const float *src = logits + (size_t)row * vocab;
+    if (p.temperature <= 1e-5f) {
+        const int idx = row_argmax(src, vocab, sh);
+        if (threadIdx.x == 0) out[row] = idx == 0x7fffffff ? 0 : idx;
+        return;
+    }
+    float *w = work + (size_t)row * vocab;
+    float m = -INFINITY;
+    for (int i = threadIdx.x; i < vocab; i += kBlock) {
+        const float v = sanitize(src[i]);
+        w[i] = v;
+        m = fmaxf(m, v);
+    }
+    m = block_max_f(m, sh);   // its barriers also publish w[]
+    if (!(m > -INFINITY)) {
+        if (threadIdx.x == 0) out[row] = 0;   // no finite logit: the reference's argmax gives index 0 as well
+        return;
+    }
+    const float inv_t = (float)(1.0 / (double)p.temperature);
+    if (p.top_k > 0 && p.top_k < vocab) {
+        const uint32_t t = kth_largest_key(w, vocab, p.top_k, sh);
+        for (int i = threadIdx.x; i < vocab; i += kBlock)
+            if (f2key(w[i]) < t) w[i] = -INFINITY;
+        __syncthreads();
+    }
+    if (p.top_p > 0.f && p.top_p < 1.f) {
+        double part = 0.0;
+        for (int i = threadIdx.x; i < vocab; i += kBlock)
+            if (w[i] > -INFINITY) part += (double)expf((w[i] - m) * inv_t);
+        const double target = (double)p.top_p * block_sum_d(part, sh);
+        // largest key t such that the mass of {key >= t} still reaches the target
+        uint32_t lo = 0, hi = 0xFFFFFFFFu;
+        while (lo < hi) {
+            const uint32_t mid = lo + ((hi - lo) >> 1) + 1;
+            part = 0.0;
+            for (int i = threadIdx.x; i < vocab; i += kBlock) {
+                const float v = w[i];
+                if (v > -INFINITY && f2key(v) >= mid) part += (double)expf((v - m) * inv_t);
+            }
+            if (block_sum_d(part, sh) >= target) lo = mid;
+            else hi = mid - 1;
+        }
+        for (int i = threadIdx.x; i < vocab; i += kBlock)
+            if (w[i] > -INFINITY && f2key(w[i]) < lo) w[i] = -INFINITY;
+        __syncthreads();
+    }
+    float best = -INFINITY;
+    int besti = 0x7fffffff;
+    for (int i = threadIdx.x; i < vocab; i += kBlock) {
+        const float v = w[i];
+        if (!(v > -INFINITY)) continue;
+        const float u = philox_uniform(p.seed, p.draw, (uint32_t)i);
+        const float score = (v - m) * inv_t - logf(-logf(u));
+        if (score > best) {
+            best = score;
+            besti = i;
+        }
+    }
+    const int idx = block_argmax(best, besti, sh);
+    if (threadIdx.x == 0) out[row] = idx == 0x7fffffff ? 0 : idx;
+}
+
+}  // namespace
+
+extern "C" int fllm_argmax(const float *logits, int32_t *out, int rows, int vocab, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && vocab > 0, "argmax: bad sizes rows=%d vocab=%d", rows, vocab);
+    if (rows == 0) return 0;
+    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(kBlock), 0, stream, logits, out, vocab);
+    return fllm_check_launch("argmax");
+}
+
+extern "C" int fllm_sample(const float *logits, float *work, const FllmSampleRow *params, int32_t *out, int rows,
+                           int vocab, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
+    FLLM_REQUIRE(work != nullptr && params != nullptr, "sample: work and params are required");
+    if (rows == 0) return 0;
+    hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(kBlock), 0, stream, logits, work, params, out, vocab);
+    return fllm_check_launch("sample");
+}

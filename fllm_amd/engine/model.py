@@ -1,0 +1,126 @@
+"""A model put together from parts as its `ModelSpec` says, and the plan of its caches."""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..cache import CacheManager, GroupSpec
+from ..config.spec import ModelSpec
+from ..parts.base import KVNeed, StateNeed
+from ..parts.runtime import Runtime
+from ..registry import part_class
+from ..weights.loader import part_weights
+from .context import CacheBinding, StepContext
+
+
+class Model:
+    def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], rt: Runtime):
+        spec.validate()
+        self.spec = spec
+        self.rt = rt
+
+        def make(role, part, **extra):
+            return part_class(role, part.kind)(part, part_weights(part, tensors), rt, **extra)
+
+        self.embedding = make("embedding", spec.embedding)
+        self.blocks = []
+        for layer in spec.layers:
+            norms = {name: make("norm", n) for name, n in layer.norms.items()}
+            mixer = make("mixer", layer.mixer)
+            ffn = make("feed_forward", layer.feed_forward)
+            self.blocks.append(make("block", layer.block, mixer=mixer, feed_forward=ffn, norms=norms))
+        self.final_norm = make("norm", spec.final_norm)
+        self.head = make("head", spec.head)
+        self.bindings: List[CacheBinding] = []
+        self._plan_caches()
+
+    # ---- caches ---------------------------------------------------------------------------
+    def _plan_caches(self) -> None:
+        """Groups cache-owning run entries by what they need; entries that read another entry's
+        cache join that entry's group."""
+        self.kv_needs: List[Optional[KVNeed]] = []
+        self.state_needs: List[Optional[StateNeed]] = []
+        for entry in self.spec.run_order:
+            mixer = self.blocks[entry.layer].mixer
+            self.kv_needs.append(mixer.cache_need())
+            self.state_needs.append(mixer.state_need())
+        keys: List[Tuple] = []
+        self.entry_group: List[Optional[int]] = [None] * len(self.spec.run_order)
+        self.entry_index: List[Optional[int]] = [None] * len(self.spec.run_order)   # index inside the group's tensors
+        members: List[List[int]] = []
+        for i, entry in enumerate(self.spec.run_order):
+            need = self.kv_needs[i]
+            if need is None:
+                continue
+            if entry.reads_cache_of is not None:
+                src = entry.reads_cache_of
+                src_need = self.kv_needs[src]
+                if src_need is None or (src_need.kv_heads, src_need.head_dim) != (need.kv_heads, need.head_dim):
+                    raise ValueError(f"run entry {i} cannot read the cache of entry {src}: different geometry")
+                if src_need.window is not None and (need.window is None or need.window > src_need.window):
+                    raise ValueError(f"run entry {i} needs more keys than entry {src} keeps")
+                self.entry_group[i] = self.entry_group[src]
+                self.entry_index[i] = self.entry_index[src]
+                continue
+            key = (need.kv_heads, need.head_dim, need.window)
+            if key not in keys:
+                keys.append(key)
+                members.append([])
+            g = keys.index(key)
+            self.entry_group[i] = g
+            self.entry_index[i] = len(members[g])
+            members[g].append(i)
+        self.group_keys = keys
+        self.group_members = members
+
+    def group_specs(self, page_size: int) -> List[GroupSpec]:
+        return [GroupSpec(entries=tuple(m), kv_heads=k[0], head_dim=k[1], window=k[2], page_size=page_size)
+                for k, m in zip(self.group_keys, self.group_members)]
+
+    def cache_bytes_per_page(self, page_size: int) -> int:
+        """Bytes one page costs over all groups (a page of every group per `page_size` tokens)."""
+        elem = torch.empty((), dtype=self.rt.dtype).element_size()
+        return sum(2 * len(m) * k[0] * k[1] * page_size * elem for k, m in zip(self.group_keys, self.group_members))
+
+    def allocate_caches(self, page_size: int, pages_per_group: Sequence[int], max_requests: int) -> CacheManager:
+        """Device pages for every group (one page more than the manager hands out: the null page
+        that padding rows of a captured step write to) and the state arenas."""
+        rt = self.rt
+        groups = self.group_specs(page_size)
+        if len(pages_per_group) != len(groups):
+            raise ValueError(f"{len(groups)} cache groups need {len(groups)} page counts")
+        self.page_size = page_size
+        self.null_pages = [int(n) for n in pages_per_group]
+        self.k_store, self.v_store = [], []
+        for g, n in zip(groups, pages_per_group):
+            self.k_store.append(torch.zeros((len(g.entries), n + 1, g.kv_heads, page_size, g.head_dim),
+                                            dtype=rt.dtype, device=rt.device))
+            self.v_store.append(torch.zeros((len(g.entries), n + 1, g.kv_heads, g.head_dim, page_size),
+                                            dtype=rt.dtype, device=rt.device))
+        self.bindings = []
+        for i, entry in enumerate(self.spec.run_order):
+            g = self.entry_group[i]
+            state = None
+            if self.state_needs[i] is not None:
+                need = self.state_needs[i]
+                state = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=rt.device)
+            if g is None:
+                self.bindings.append(CacheBinding(group=-1, k_pages=None, v_pages=None, page_size=page_size,
+                                                  writes=False, state=state))
+                continue
+            idx = self.entry_index[i]
+            self.bindings.append(CacheBinding(group=g, k_pages=self.k_store[g][idx], v_pages=self.v_store[g][idx],
+                                              page_size=page_size, writes=entry.reads_cache_of is None, state=state))
+        return CacheManager(groups, list(pages_per_group), max_requests)
+
+    # ---- forward --------------------------------------------------------------------------
+    def forward(self, ctx: StepContext) -> torch.Tensor:
+        """Logits (float32 [len(logit_rows), vocab]) of the step's wanted rows."""
+        x = self.embedding.forward(ctx, ctx.ids)
+        for entry, binding in zip(self.spec.run_order, self.bindings):
+            self.blocks[entry.layer].forward(ctx, x, binding)
+        if ctx.logit_rows.numel() == 0:
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.rt.device)
+        h = self.final_norm.forward(ctx, x, rows=ctx.logit_rows)
+        return self.head.forward(ctx, h)

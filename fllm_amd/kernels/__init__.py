@@ -1,0 +1,246 @@
+"""The kernel library seen from Python: `Ops` wraps the C ABI of csrc/api.h.
+
+Every method checks on the host that tensors are on the GPU, dense, of the element type and the
+shape the kernel assumes, before anything is launched.  There is no other implementation: if the
+library cannot be loaded or built, constructing `Ops` raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build as _build
+
+F32, BF16 = 0, 1
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+OUT_STORE, OUT_STORE_F32, OUT_ADD_F32 = 0, 1, 2
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+class SampleRow(ctypes.Structure):
+    _fields_ = [("temperature", ctypes.c_float), ("top_p", ctypes.c_float), ("top_k", ctypes.c_int32),
+                ("pad", ctypes.c_int32), ("seed", ctypes.c_uint64), ("draw", ctypes.c_uint64)]
+
+
+SAMPLE_ROW_BYTES = ctypes.sizeof(SampleRow)
+assert SAMPLE_ROW_BYTES == 32
+
+_lib = None
+
+
+def load_library(build_if_missing: bool = True):
+    """The loaded library; builds it first when there is none that matches the sources."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = _build.find_library()
+    if path is None:
+        if not build_if_missing:
+            raise KernelError("the HIP kernel library is not built (run `python -m fllm_amd.kernels.build`)")
+        path = _build.build()
+    try:
+        lib = ctypes.CDLL(path)
+    except OSError as exc:
+        raise KernelError(f"cannot load the HIP kernel library {path}: {exc}") from None
+    c_int, c_void, c_float, c_size = ctypes.c_int, ctypes.c_void_p, ctypes.c_float, ctypes.c_size_t
+    lib.fllm_last_error.restype = ctypes.c_char_p
+    lib.fllm_abi_version.restype = c_int
+    sig = {
+        "fllm_embed": [c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_float, c_void],
+        "fllm_rmsnorm": [c_void, c_void, c_void, c_void, c_int, c_int, c_float, c_int, c_void],
+        "fllm_linear": [c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
+        "fllm_swiglu": [c_void, c_void, c_int, c_int, c_int, c_void],
+        "fllm_rope_kv_store": [c_void, c_void, c_void, c_void, c_int, c_void, c_void, c_int, c_void, c_void, c_int,
+                               c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
+        "fllm_attention": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int,
+                           c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void, c_size, c_void],
+        "fllm_argmax": [c_void, c_void, c_int, c_int, c_void],
+        "fllm_sample": [c_void, c_void, c_void, c_void, c_int, c_int, c_void],
+    }
+    for name, args in sig.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = c_int
+    lib.fllm_attention_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int]
+    lib.fllm_attention_workspace_bytes.restype = c_size
+    _lib = lib
+    return lib
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dense(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
+    _need(t.is_cuda, f"{name} must be on the GPU")
+    _need(t.is_contiguous(), f"{name} must be contiguous")
+    if dtype is not None:
+        _need(t.dtype == dtype, f"{name} must be {dtype}, is {t.dtype}")
+    if shape is not None:
+        _need(tuple(t.shape) == tuple(shape), f"{name} must have shape {tuple(shape)}, has {tuple(t.shape)}")
+
+
+class Ops:
+    """Launches kernels on the current torch stream of the tensors' device."""
+
+    def __init__(self):
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible: the engine runs on gfx950 only")
+        self.lib = load_library()
+
+    def _check(self, code: int) -> None:
+        if code != 0:
+            raise KernelError(self.lib.fllm_last_error().decode("utf-8", "replace"))
+
+    @staticmethod
+    def _stream() -> int:
+        return torch.cuda.current_stream().cuda_stream
+
+    def embed(self, ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+        rows = ids.numel()
+        vocab, width = table.shape
+        _dense(ids, "ids", torch.int32)
+        _dense(table, "table")
+        _need(table.dtype in _DTYPE_CODE, f"table dtype {table.dtype} unsupported")
+        _dense(out, "out", torch.float32, (rows, width))
+        self._check(self.lib.fllm_embed(_ptr(ids), _ptr(table), _ptr(out), rows, width, vocab, _DTYPE_CODE[table.dtype],
+                                        float(scale), self._stream()))
+        return out
+
+    def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        width = x.shape[-1]
+        _dense(x, "x", torch.float32)
+        _dense(weight, "weight", torch.float32, (width,))
+        count = x.shape[0] if rows is None else rows.numel()
+        if rows is not None:
+            _dense(rows, "rows", torch.int32)
+        _dense(out, "out", None, (count, width))
+        _need(out.dtype in _DTYPE_CODE, f"out dtype {out.dtype} unsupported")
+        self._check(self.lib.fllm_rmsnorm(_ptr(x), _ptr(rows), _ptr(weight), _ptr(out), count, width, float(eps),
+                                          _DTYPE_CODE[out.dtype], self._stream()))
+        return out
+
+    def linear(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
+               accumulate: bool = False) -> torch.Tensor:
+        """out = x @ w.T (+ bias); `accumulate` adds into a float32 `out` instead of storing."""
+        _need(x.dim() == 2 and w.dim() == 2 and out.dim() == 2, "linear takes matrices")
+        M, K = x.shape
+        N = w.shape[0]
+        _need(w.shape[1] == K, f"w has {w.shape[1]} columns, x has {K}")
+        _need(x.is_cuda and w.is_cuda and out.is_cuda, "linear operands must be on the GPU")
+        _need(x.dtype == w.dtype and x.dtype in _DTYPE_CODE, f"x is {x.dtype}, w is {w.dtype}")
+        _need(x.stride(1) == 1 and out.stride(1) == 1 and w.is_contiguous(), "linear operands must be row-major")
+        _need(tuple(out.shape) == (M, N), f"out must have shape {(M, N)}, has {tuple(out.shape)}")
+        if accumulate:
+            _need(out.dtype == torch.float32, "accumulate needs a float32 out")
+            mode = OUT_ADD_F32
+        elif out.dtype == x.dtype:
+            mode = OUT_STORE
+        else:
+            _need(out.dtype == torch.float32, f"out must be {x.dtype} or float32")
+            mode = OUT_STORE_F32
+        if bias is not None:
+            _dense(bias, "bias", torch.float32, (N,))
+        ldx = x.stride(0) if M > 1 else K
+        ldo = out.stride(0) if M > 1 else N
+        self._check(self.lib.fllm_linear(_ptr(x), ldx, _ptr(w), _ptr(bias), _ptr(out), ldo, M, N, K, _DTYPE_CODE[x.dtype],
+                                         mode, self._stream()))
+        return out
+
+    def swiglu(self, gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        rows, two_i = gate_up.shape
+        _need(two_i % 2 == 0, "gate_up needs an even width")
+        _dense(gate_up, "gate_up")
+        _need(gate_up.dtype in _DTYPE_CODE, f"dtype {gate_up.dtype} unsupported")
+        _dense(out, "out", gate_up.dtype, (rows, two_i // 2))
+        self._check(self.lib.fllm_swiglu(_ptr(gate_up), _ptr(out), rows, two_i // 2, _DTYPE_CODE[gate_up.dtype],
+                                         self._stream()))
+        return out
+
+    def rope_kv_store(self, qkv: torch.Tensor, row_pos: torch.Tensor, row_seg: torch.Tensor, tables: torch.Tensor,
+                      cos: torch.Tensor, sin: torch.Tensor, k_pages: Optional[torch.Tensor],
+                      v_pages: Optional[torch.Tensor], heads: int, kv_heads: int, head_dim: int, rope_dims: int,
+                      pairing: int, page_size: int) -> None:
+        rows = qkv.shape[0]
+        _dense(qkv, "qkv", None, (rows, (heads + 2 * kv_heads) * head_dim))
+        _need(qkv.dtype in _DTYPE_CODE, f"dtype {qkv.dtype} unsupported")
+        _dense(row_pos, "row_pos", torch.int32, (rows,))
+        _dense(row_seg, "row_seg", torch.int32, (rows,))
+        _dense(tables, "tables", torch.int32)
+        _need(tables.dim() == 2, "tables must be [segments, pages]")
+        half = rope_dims // 2
+        _dense(cos, "cos", torch.float32)
+        _dense(sin, "sin", torch.float32, tuple(cos.shape))
+        _need(cos.dim() == 2 and cos.shape[1] == half, f"rotary tables must be [positions, {half}]")
+        store = k_pages is not None
+        num_pages = 0
+        if store:
+            num_pages = k_pages.shape[0]
+            _dense(k_pages, "k_pages", qkv.dtype, (num_pages, kv_heads, page_size, head_dim))
+            _dense(v_pages, "v_pages", qkv.dtype, (num_pages, kv_heads, head_dim, page_size))
+        self._check(self.lib.fllm_rope_kv_store(
+            _ptr(qkv), _ptr(row_pos), _ptr(row_seg), _ptr(tables), tables.shape[1], _ptr(cos), _ptr(sin), cos.shape[0],
+            _ptr(k_pages), _ptr(v_pages), num_pages, rows, heads, kv_heads, head_dim, rope_dims, pairing, page_size,
+            _DTYPE_CODE[qkv.dtype], 1 if store else 0, self._stream()))
+
+    def attention_workspace_bytes(self, rows: int, heads: int, head_dim: int, max_context: int) -> int:
+        return int(self.lib.fllm_attention_workspace_bytes(rows, heads, head_dim, max_context))
+
+    def attention(self, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, tables: torch.Tensor,
+                  row_pos: torch.Tensor, row_seg: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int,
+                  head_dim: int, page_size: int, scale: float, window: Optional[int], max_context: int,
+                  uniform_rows: int = 0, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """`q` may be a column slice of a wider row-major matrix (the fused qkv buffer).
+        `max_context` bounds pos + 1 over the rows; `uniform_rows` is 1 when every segment has one
+        row (a decode step)."""
+        rows = q.shape[0]
+        _need(q.is_cuda and q.dim() == 2 and q.stride(1) == 1 and q.shape[1] == heads * head_dim,
+              f"q must be [rows, {heads * head_dim}] with unit column stride")
+        _need(q.dtype in _DTYPE_CODE, f"dtype {q.dtype} unsupported")
+        num_pages = k_pages.shape[0]
+        _dense(k_pages, "k_pages", q.dtype, (num_pages, kv_heads, page_size, head_dim))
+        _dense(v_pages, "v_pages", q.dtype, (num_pages, kv_heads, head_dim, page_size))
+        _dense(tables, "tables", torch.int32)
+        _need(tables.dim() == 2, "tables must be [segments, pages]")
+        _dense(row_pos, "row_pos", torch.int32, (rows,))
+        _dense(row_seg, "row_seg", torch.int32, (rows,))
+        _dense(out, "out", q.dtype, (rows, heads * head_dim))
+        ws_ptr, ws_bytes = None, 0
+        if workspace is not None:
+            _need(workspace.is_cuda and workspace.is_contiguous(), "workspace must be a dense GPU tensor")
+            ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+        q_stride = q.stride(0) if rows > 1 else heads * head_dim
+        self._check(self.lib.fllm_attention(
+            _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(tables), tables.shape[1], _ptr(row_pos), _ptr(row_seg),
+            _ptr(out), rows, heads, kv_heads, head_dim, page_size, num_pages, float(scale),
+            int(window) if window else 0, _DTYPE_CODE[q.dtype], int(max_context), int(uniform_rows), ws_ptr, ws_bytes,
+            self._stream()))
+        return out
+
+    def argmax(self, logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        rows, vocab = logits.shape
+        _dense(logits, "logits", torch.float32)
+        _dense(out, "out", torch.int32, (rows,))
+        self._check(self.lib.fllm_argmax(_ptr(logits), _ptr(out), rows, vocab, self._stream()))
+        return out
+
+    def sample(self, logits: torch.Tensor, work: torch.Tensor, params: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """`params`: uint8 GPU tensor [rows, 32] holding `SampleRow` records."""
+        rows, vocab = logits.shape
+        _dense(logits, "logits", torch.float32)
+        _dense(work, "work", torch.float32, (rows, vocab))
+        _dense(params, "params", torch.uint8, (rows, SAMPLE_ROW_BYTES))
+        _dense(out, "out", torch.int32, (rows,))
+        self._check(self.lib.fllm_sample(_ptr(logits), _ptr(work), _ptr(params), _ptr(out), rows, vocab, self._stream()))
+        return out

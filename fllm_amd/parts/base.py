@@ -1,0 +1,93 @@
+"""What every part must offer.
+
+A part is built from a `PartSpec` (its sizes and constants), the tensors the spec names, and the
+runtime (device, precision, kernel library).  It never sees the model configuration.
+
+Roles and their interfaces:
+
+  norm          forward(ctx, x_f32[R,H], out=None, rows=None) -> normed[R or len(rows), H] in the
+                compute dtype; `rows` (int32 device tensor) selects rows first.
+  position      tables(device) -> whatever the mixer's kernels take (rotary: cos/sin tables).
+  mixer         cache_need() / state_need() say what the cache manager must keep for it;
+                forward(ctx, h[R,H], residual_f32[R,H], binding) adds its output to `residual`.
+  feed_forward  forward(ctx, h[R,H], residual_f32[R,H]) adds its output to `residual`.
+  block         forward(ctx, residual_f32[R,H], binding) runs norms, mixer and feed-forward.
+  embedding     forward(ctx, ids[R]) -> residual_f32[R,H].
+  head          forward(ctx, h[L,H]) -> logits_f32[L,V].
+
+The residual stream is float32 in every precision mode; `h` is in the compute dtype.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from ..config.spec import PartSpec
+
+# how random-weights mode fills a tensor
+INIT_MATRIX = "matrix"     # N(0, 0.02)
+INIT_NORM = "norm"         # 1 + U(-0.1, 0.1)
+INIT_BIAS = "bias"         # N(0, 0.02)
+
+
+@dataclass(frozen=True)
+class KVNeed:
+    """Keys and values of `kv_heads` heads of `head_dim` per token; `window` keys back (the
+    token itself included) or all of them when None."""
+    kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """A fixed-size tensor per live request (shape without the request dimension)."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class Part:
+    role = ""
+
+    @classmethod
+    def tensor_shapes(cls, spec: PartSpec) -> Dict[str, Tuple[Tuple[int, ...], str]]:
+        """Own parameter name -> (shape, init kind).  Names that `spec.tensors` lists with a
+        leading '?' are optional in a checkpoint."""
+        return {}
+
+    def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt):
+        self.spec = spec
+        self.rt = rt
+
+
+class Mixer(Part):
+    role = "mixer"
+
+    def cache_need(self) -> Optional[KVNeed]:
+        return None
+
+    def state_need(self) -> Optional[StateNeed]:
+        return None
+
+    def forward(self, ctx, h, residual, binding) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    role = "feed_forward"
+
+    def forward(self, ctx, h, residual) -> None:
+        raise NotImplementedError
+
+
+class Norm(Part):
+    role = "norm"
+
+    def forward(self, ctx, x, out=None, rows=None):
+        raise NotImplementedError
+
+
+class Block(Part):
+    role = "block"

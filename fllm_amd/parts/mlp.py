@@ -1,0 +1,45 @@
+"""Gated feed-forward: x += W_down (silu(W_gate n) * W_up n), silu(g) = g / (1 + exp(-g))
+(rust/engine/src/rust_decoder.rs:8328-8352, :1645; rust/engine/src/cpu_elementwise.rs:3-43).
+Gate and up are one product with the concatenated matrix."""
+from __future__ import annotations
+
+import torch
+
+from ..registry import register_part
+from .base import INIT_BIAS, INIT_MATRIX, FeedForward
+
+
+class GatedMLP(FeedForward):
+    @classmethod
+    def tensor_shapes(cls, spec):
+        h, i = spec["hidden_size"], spec["intermediate_size"]
+        return {"gate": ((i, h), INIT_MATRIX), "up": ((i, h), INIT_MATRIX), "down": ((h, i), INIT_MATRIX),
+                "gate_bias": ((i,), INIT_BIAS), "up_bias": ((i,), INIT_BIAS), "down_bias": ((h,), INIT_BIAS)}
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        if spec.get("activation", "silu") not in ("silu", "swish"):
+            raise ValueError(f"unsupported activation {spec.get('activation')!r}; the gated feed-forward uses silu")
+        self.hidden = int(spec["hidden_size"])
+        self.inter = int(spec["intermediate_size"])
+        self.w_gate_up = torch.cat([rt.matrix(weights["gate"]), rt.matrix(weights["up"])], dim=0).contiguous()
+        self.w_down = rt.matrix(weights["down"])
+        gb, ub = weights.get("gate_bias"), weights.get("up_bias")
+        self.b_gate_up = None
+        if gb is not None or ub is not None:
+            zeros = lambda: torch.zeros(self.inter, dtype=torch.float32, device=rt.device)
+            self.b_gate_up = torch.cat([rt.vector(gb) if gb is not None else zeros(),
+                                        rt.vector(ub) if ub is not None else zeros()]).contiguous()
+        self.b_down = rt.vector(weights["down_bias"]) if weights.get("down_bias") is not None else None
+
+    def forward(self, ctx, h, residual):
+        rt, ops = self.rt, self.rt.ops
+        rows = h.shape[0]
+        gate_up = rt.empty((rows, 2 * self.inter))
+        ops.linear(h, self.w_gate_up, gate_up, bias=self.b_gate_up)
+        act = rt.empty((rows, self.inter))
+        ops.swiglu(gate_up, act)
+        ops.linear(act, self.w_down, residual, bias=self.b_down, accumulate=True)
+
+
+register_part("feed_forward", "gated_mlp", GatedMLP)

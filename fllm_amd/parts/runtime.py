@@ -1,0 +1,47 @@
+"""What parts get to work with: the device, the compute precision and the kernel library."""
+from __future__ import annotations
+
+import weakref
+from typing import Any, Dict, Tuple
+
+import torch
+
+
+class Runtime:
+    """`dtype` is the compute precision: float32 (everything in true 32-bit) or bfloat16
+    (matrices, activations and pages in bfloat16; residual stream, norms, softmax, rotary angles
+    and logits in float32).  `ops` is the kernel library (`fllm_amd.kernels.Ops`)."""
+
+    def __init__(self, device: torch.device, dtype: torch.dtype, ops, max_context: int):
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"compute dtype must be float32 or bfloat16, not {dtype}")
+        self.device = torch.device(device)
+        self.dtype = dtype
+        self.ops = ops
+        self.max_context = int(max_context)
+        # weak: a placed tensor lives as long as a part holds it (pieces of a concatenated matrix are freed)
+        self._placed = weakref.WeakValueDictionary()
+        self.shared: Dict[Any, Any] = {}      # tables several parts share (rotary tables)
+
+    def _place(self, t: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+        key = (t.data_ptr(), tuple(t.shape), t.dtype, dtype)
+        hit = self._placed.get(key)
+        if hit is None:
+            hit = t.to(device=self.device, dtype=dtype).contiguous()
+            self._placed[key] = hit
+        return hit
+
+    def matrix(self, t: torch.Tensor) -> torch.Tensor:
+        """A weight matrix or table on the device in the compute dtype.  The same checkpoint
+        tensor is placed once (a tied head shares the embedding's copy)."""
+        return self._place(t, self.dtype)
+
+    def vector(self, t: torch.Tensor) -> torch.Tensor:
+        """Norm weights and biases: float32 (exact for both storage types)."""
+        return self._place(t, torch.float32)
+
+    def forget_host_tensors(self) -> None:
+        self._placed.clear()
+
+    def empty(self, shape, dtype=None) -> torch.Tensor:
+        return torch.empty(shape, dtype=dtype or self.dtype, device=self.device)

@@ -1,0 +1,264 @@
+"""A plain, slow Llama: whole sequences, no cache, float64, one function per part.
+
+Written from the reference's formulas (file:line cited per function, paths relative to the
+reference's root); it shares no code with `fllm_amd`.  Weights come in as a dict of float64
+NumPy arrays under the checkpoint's tensor names, the configuration as the config.json dict.
+"""
+import math
+
+import numpy as np
+
+
+# ---------------------------------------------------------------------------------------------
+# configuration, read straight from config.json keys (rust/checkpoint/src/plan.rs:1066-1111 sizes,
+# :1222-1236 eps, :1239-1287 window, :92-121 and :1323-1338 rotary base, :1478-1505 llama3)
+# ---------------------------------------------------------------------------------------------
+def read_sizes(cfg):
+    hidden = cfg["hidden_size"]
+    heads = cfg["num_attention_heads"]
+    out = {
+        "hidden": hidden,
+        "layers": cfg["num_hidden_layers"],
+        "heads": heads,
+        "kv_heads": cfg.get("num_key_value_heads", heads),
+        "head_dim": cfg.get("head_dim", hidden // heads),
+        "inter": cfg["intermediate_size"],
+        "vocab": cfg.get("vocab_size", 32000),
+        "eps": cfg.get("rms_norm_eps", 1e-6),
+        "tied": bool(cfg.get("tie_word_embeddings", False)),
+    }
+    scaling = cfg.get("rope_scaling") or {}
+    params = cfg.get("rope_parameters") or {}
+    if params:
+        scaling = params
+    out["theta"] = float(scaling.get("rope_theta", cfg.get("rope_theta", 10000.0)))
+    out["rope_kind"] = str(scaling.get("rope_type", scaling.get("type", "default"))).lower()
+    out["rope_scaling"] = scaling
+    partial = cfg.get("partial_rotary_factor", 1.0)
+    out["rope_dims"] = int(round(out["head_dim"] * partial))
+    window = cfg.get("sliding_window") or 0
+    layers = out["layers"]
+    if window > 0 and cfg.get("use_sliding_window") is not False:
+        types = cfg.get("layer_types")
+        if isinstance(types, list) and len(types) == layers:
+            out["windows"] = [window if t == "sliding_attention" else None for t in types]
+        else:
+            out["windows"] = [window] * layers
+    else:
+        out["windows"] = [None] * layers
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# parts
+# ---------------------------------------------------------------------------------------------
+def rms_norm(x, weight, eps):
+    """rust/engine/src/rust_decoder.rs:1481-1490: inv = 1/sqrt(sum(x^2)/n + eps); x *= inv * w."""
+    x = np.asarray(x, dtype=np.float64)
+    inv = 1.0 / np.sqrt((x * x).sum(axis=-1, keepdims=True) / x.shape[-1] + eps)
+    return x * (inv * np.asarray(weight, dtype=np.float64))
+
+
+def llama3_divisors(dims, theta, factor, low, high, original):
+    """rust/checkpoint/src/plan.rs:1478-1505: float64 per-lane divisors, cast to float32."""
+    out = []
+    low_wavelength = original / low
+    high_wavelength = original / high
+    for i in range(dims // 2):
+        frequency = 1.0 / theta ** ((2 * i) / dims)
+        wavelength = 2.0 * math.pi / frequency
+        if wavelength < high_wavelength:
+            scale = 1.0
+        elif wavelength > low_wavelength:
+            scale = factor
+        else:
+            smooth = (original / wavelength - low) / (high - low)
+            scale = 1.0 / ((1.0 - smooth) / factor + smooth)
+        out.append(np.float32(scale))
+    return np.array(out, dtype=np.float32)
+
+
+def rope_tables(positions, dims, theta, kind="default", scaling=None):
+    """rust/engine/src/rope.rs:38-68: inverse frequencies in float32 (divided by the per-lane
+    divisors when there are any), phase = position * inverse in float32 (`linear` scaling divides
+    the position, :53-62), cos and sin in float64.  Returns float64 [len(positions), dims/2]."""
+    scaling = scaling or {}
+    half = dims // 2
+    lanes = np.arange(half, dtype=np.float32)
+    exponent = (lanes * np.float32(2.0)) / np.float32(dims)
+    inverse = (np.float32(1.0) / np.power(np.float32(theta), exponent)).astype(np.float32)
+    scale = np.float32(1.0)
+    if kind == "llama3":
+        inverse = (inverse / llama3_divisors(dims, theta, float(scaling["factor"]),
+                                             float(scaling.get("low_freq_factor", 1.0)),
+                                             float(scaling.get("high_freq_factor", 4.0)),
+                                             float(scaling["original_max_position_embeddings"]))).astype(np.float32)
+    elif kind == "linear":
+        scale = np.float32(1.0) / np.float32(scaling["factor"])
+    elif kind != "default":
+        raise ValueError(kind)
+    pos = np.asarray(positions, dtype=np.float32) * scale
+    phase = (pos[:, None] * inverse[None, :]).astype(np.float32).astype(np.float64)
+    return np.cos(phase), np.sin(phase)
+
+
+def apply_rope(x, cos, sin, dims, interleaved=False):
+    """rust/engine/src/rust_decoder.rs:1655-1683: rotate lane pairs of the first `dims` values of
+    every head: (a, b) <- (a cos - b sin, b cos + a sin).  The reference pairs (2l, 2l+1) on
+    weights whose q/k rows it permuted at import (rust/checkpoint/src/convert.rs:2713-2745); on the
+    checkpoint's own row order that is the pairing (l, l + dims/2), used here unless `interleaved`.
+    x: [tokens, heads, head_dim]; cos, sin: [tokens, dims/2]."""
+    x = np.array(x, dtype=np.float64, copy=True)
+    half = dims // 2
+    if interleaved:
+        ia, ib = np.arange(half) * 2, np.arange(half) * 2 + 1
+    else:
+        ia, ib = np.arange(half), np.arange(half) + half
+    a, b = x[:, :, ia].copy(), x[:, :, ib].copy()
+    c, s = cos[:, None, :], sin[:, None, :]
+    x[:, :, ia] = a * c - b * s
+    x[:, :, ib] = b * c + a * s
+    return x
+
+
+def attention(q, k, v, scale, window=None):
+    """rust/engine/src/rust_decoder.rs:6065-6166: row r (position r, length n = r + 1) sees keys
+    start..n with start = n - window (0 without a window, :6090-6093); head h uses key/value head
+    h / (heads / kv_heads) (:6121); s = (q . k) * scale; softmax over the visible keys; weights
+    are divided by their sum before they multiply v (:6156-6161).
+    q: [T, heads, d]; k, v: [T, kv_heads, d] -> [T, heads, d]."""
+    T, heads, d = q.shape
+    kv_heads = k.shape[1]
+    group = heads // kv_heads
+    out = np.zeros((T, heads, v.shape[2]), dtype=np.float64)
+    for r in range(T):
+        n = r + 1
+        start = 0 if window is None else max(0, n - window)
+        for h in range(heads):
+            kh = h // group
+            scores = (k[start:n, kh, :] @ q[r, h, :]) * scale
+            e = np.exp(scores - scores.max())
+            w = e / e.sum()
+            out[r, h, :] = w @ v[start:n, kh, :]
+    return out
+
+
+def silu(x):
+    """rust/engine/src/rust_decoder.rs:1645: x / (1 + exp(-x))."""
+    return x / (1.0 + np.exp(-x))
+
+
+def linear(x, weight, bias=None):
+    """rust/engine/src/compute.rs:292-308: y[b][r] = sum_k x[b][k] W[r][k] (+ bias[r])."""
+    y = x @ np.asarray(weight, dtype=np.float64).T
+    if bias is not None:
+        y = y + np.asarray(bias, dtype=np.float64)
+    return y
+
+
+def gated_mlp(x, gate, up, down, gate_bias=None, up_bias=None, down_bias=None):
+    """rust/engine/src/rust_decoder.rs:8328-8352: down(silu(gate x) * (up x))."""
+    return linear(silu(linear(x, gate, gate_bias)) * linear(x, up, up_bias), down, down_bias)
+
+
+def attention_layer(x, weights, prefix, sizes, layer, positions):
+    """rust/engine/src/rust_decoder.rs:8827-8835 (projections), :8895-8898 (rotary on q and k),
+    :8976-9001 (attention), :9025 (output projection)."""
+    T = x.shape[0]
+    heads, kv_heads, d = sizes["heads"], sizes["kv_heads"], sizes["head_dim"]
+    g = lambda n: weights.get(f"{prefix}.self_attn.{n}")
+    q = linear(x, g("q_proj.weight"), g("q_proj.bias")).reshape(T, heads, d)
+    k = linear(x, g("k_proj.weight"), g("k_proj.bias")).reshape(T, kv_heads, d)
+    v = linear(x, g("v_proj.weight"), g("v_proj.bias")).reshape(T, kv_heads, d)
+    cos, sin = rope_tables(positions, sizes["rope_dims"], sizes["theta"], sizes["rope_kind"], sizes["rope_scaling"])
+    q = apply_rope(q, cos, sin, sizes["rope_dims"])
+    k = apply_rope(k, cos, sin, sizes["rope_dims"])
+    o = attention(q, k, v, 1.0 / math.sqrt(d), sizes["windows"][layer])
+    return linear(o.reshape(T, heads * d), g("o_proj.weight"), g("o_proj.bias"))
+
+
+def forward(cfg, weights, token_ids, first_position=0):
+    """Logits [T, vocab] of a whole sequence (rust/engine/src/rust_decoder.rs:8531-8701 and
+    :8706-9117): embedding; per layer x += attention(norm(x)), x += mlp(norm(x)); final norm;
+    head (the embedding table when `tie_word_embeddings`, rust_decoder.rs:2503-2507)."""
+    sizes = read_sizes(cfg)
+    ids = np.asarray(token_ids, dtype=np.int64)
+    positions = np.arange(first_position, first_position + len(ids))
+    x = np.asarray(weights["model.embed_tokens.weight"], dtype=np.float64)[ids]
+    for i in range(sizes["layers"]):
+        p = f"model.layers.{i}"
+        h = rms_norm(x, weights[f"{p}.input_layernorm.weight"], sizes["eps"])
+        x = x + attention_layer(h, weights, p, sizes, i, positions)
+        h = rms_norm(x, weights[f"{p}.post_attention_layernorm.weight"], sizes["eps"])
+        x = x + gated_mlp(h, weights[f"{p}.mlp.gate_proj.weight"], weights[f"{p}.mlp.up_proj.weight"],
+                          weights[f"{p}.mlp.down_proj.weight"], weights.get(f"{p}.mlp.gate_proj.bias"),
+                          weights.get(f"{p}.mlp.up_proj.bias"), weights.get(f"{p}.mlp.down_proj.bias"))
+    x = rms_norm(x, weights["model.norm.weight"], sizes["eps"])
+    head = weights["model.embed_tokens.weight"] if sizes["tied"] else weights["lm_head.weight"]
+    return linear(x, head)
+
+
+# ---------------------------------------------------------------------------------------------
+# sampling
+# ---------------------------------------------------------------------------------------------
+def greedy(logits):
+    """rust/engine/src/sampling.rs:531-552: the first position of the largest value."""
+    logits = np.asarray(logits)
+    return int(np.flatnonzero(logits == logits.max())[0])
+
+
+_M0, _M1, _W0, _W1 = 0xD2511F53, 0xCD9E8D57, 0x9E3779B9, 0xBB67AE85
+
+
+def philox4x32_10(ctr, key):
+    """rust/engine/src/sampling.rs:155-172."""
+    c = [int(v) & 0xFFFFFFFF for v in ctr]
+    k = [int(v) & 0xFFFFFFFF for v in key]
+    for _ in range(10):
+        p0 = _M0 * c[0]
+        p1 = _M1 * c[2]
+        c = [((p1 >> 32) ^ c[1] ^ k[0]) & 0xFFFFFFFF, p1 & 0xFFFFFFFF,
+             ((p0 >> 32) ^ c[3] ^ k[1]) & 0xFFFFFFFF, p0 & 0xFFFFFFFF]
+        k = [(k[0] + _W0) & 0xFFFFFFFF, (k[1] + _W1) & 0xFFFFFFFF]
+    return c
+
+
+def philox_uniform(seed, draw, index):
+    """rust/engine/src/sampling.rs:174-183: ((w >> 8) + 0.5) / 2^24 in float32, in (0, 1)."""
+    w = philox4x32_10([index, 0, draw & 0xFFFFFFFF, draw >> 32], [seed & 0xFFFFFFFF, seed >> 32])[0]
+    return np.float32((np.float32(w >> 8) + np.float32(0.5)) / np.float32(16777216.0))
+
+
+def device_sample(logits, temperature, top_k, top_p, seed, draw):
+    """The reference's device sampler (rust/engine/cuda/sampling.cu:253-352), with sorting in
+    place of its bisections: non-finite logits never win; temperature <= 1e-5 is greedy; top-k
+    keeps everything not below the k-th largest value (ties kept); top-p keeps the largest values
+    until their mass reaches top_p of the total (ties at the threshold kept); the token is the
+    argmax of (logit - max) / T - ln(-ln u_i), u_i = philox_uniform(seed, draw, i), lowest id on
+    ties."""
+    w = np.asarray(logits, dtype=np.float32).copy()
+    w[~np.isfinite(w)] = -np.inf
+    if not np.isfinite(w).any():
+        return 0
+    if temperature <= 1e-5:
+        return greedy(np.where(np.isfinite(w), w, -np.inf))
+    m = w.max()
+    inv_t = np.float32(1.0 / float(temperature))
+    if 0 < top_k < len(w):
+        kth = np.sort(w)[::-1][top_k - 1]
+        w[w < kth] = -np.inf
+    if 0.0 < top_p < 1.0:
+        alive = np.isfinite(w)
+        e = np.where(alive, np.exp(((w - m) * inv_t).astype(np.float32)).astype(np.float64), 0.0)
+        target = float(np.float32(top_p)) * e.sum()
+        values = np.unique(w[alive])[::-1]                      # distinct values, descending
+        mass = np.array([e[w >= v].sum() for v in values])      # mass of {value >= v}
+        threshold = values[np.flatnonzero(mass >= target)[0]]   # largest threshold that still reaches the target
+        w[w < threshold] = -np.inf
+    best, best_i = -np.inf, None
+    for i in np.flatnonzero(np.isfinite(w)):
+        u = philox_uniform(seed, draw, int(i))
+        score = np.float32((w[i] - m) * inv_t) - np.log(-np.log(u, dtype=np.float32), dtype=np.float32)
+        if score > best:
+            best, best_i = score, int(i)
+    return best_i

@@ -1,0 +1,114 @@
+"""Plain PyTorch versions of every kernel of the library, one function per kernel, with the
+kernels' own signatures.  They compute in float64 on whatever device the tensors are on and
+round once to the output type.
+
+Two uses: the GPU tests compare each HIP kernel with its function here, and the CPU tests hand
+a `ReferenceOps` to the engine in place of the kernel library, so that the step function, the
+cache and the scheduler can be exercised without a GPU.  The product never imports this file.
+"""
+import math
+
+import numpy as np
+import torch
+
+import plain_llama
+
+
+class ReferenceOps:
+    def embed(self, ids, table, out, scale=1.0):
+        out.copy_((table[ids.long()].double() * scale).to(out.dtype))
+        return out
+
+    def rmsnorm(self, x, weight, eps, out, rows=None):
+        src = x if rows is None else x[rows.long()]
+        src = src.double()
+        inv = 1.0 / torch.sqrt((src * src).sum(-1, keepdim=True) / src.shape[-1] + eps)
+        out.copy_((src * (inv * weight.double())).to(out.dtype))
+        return out
+
+    def linear(self, x, w, out, bias=None, accumulate=False):
+        y = x.double() @ w.double().T
+        if bias is not None:
+            y = y + bias.double()
+        if accumulate:
+            out.add_(y.to(out.dtype))
+        else:
+            out.copy_(y.to(out.dtype))
+        return out
+
+    def swiglu(self, gate_up, out):
+        inter = gate_up.shape[1] // 2
+        g, u = gate_up[:, :inter].double(), gate_up[:, inter:].double()
+        out.copy_((g / (1.0 + torch.exp(-g)) * u).to(out.dtype))
+        return out
+
+    def rope_kv_store(self, qkv, row_pos, row_seg, tables, cos, sin, k_pages, v_pages, heads, kv_heads, head_dim,
+                      rope_dims, pairing, page_size):
+        rows = qkv.shape[0]
+        half = rope_dims // 2
+        view = qkv.view(rows, heads + 2 * kv_heads, head_dim)
+        for r in range(rows):
+            seg = int(row_seg[r])
+            if seg < 0:
+                continue
+            pos = int(row_pos[r])
+            c, s = cos[pos].double(), sin[pos].double()
+            if pairing == 0:
+                ia, ib = torch.arange(half), torch.arange(half) + half
+            else:
+                ia, ib = torch.arange(half) * 2, torch.arange(half) * 2 + 1
+            ia, ib = ia.to(qkv.device), ib.to(qkv.device)
+            for h in range(heads + kv_heads):
+                a, b = view[r, h, ia].double(), view[r, h, ib].double()
+                view[r, h, ia] = (a * c - b * s).to(qkv.dtype)
+                view[r, h, ib] = (b * c + a * s).to(qkv.dtype)
+            if k_pages is None:
+                continue
+            page = int(tables[seg, pos // page_size])
+            off = pos % page_size
+            k_pages[page, :, off, :] = view[r, heads:heads + kv_heads, :]
+            v_pages[page, :, :, off] = view[r, heads + kv_heads:, :]
+
+    def attention_workspace_bytes(self, rows, heads, head_dim, max_context):
+        return 0
+
+    def attention(self, q, k_pages, v_pages, tables, row_pos, row_seg, out, heads, kv_heads, head_dim, page_size, scale,
+                  window, max_context, uniform_rows=0, workspace=None):
+        rows = q.shape[0]
+        group = heads // kv_heads
+        for r in range(rows):
+            seg = int(row_seg[r])
+            if seg < 0:
+                out[r] = 0
+                continue
+            pos = int(row_pos[r])
+            n = pos + 1
+            lo = max(0, n - window) if window else 0
+            keys = torch.arange(lo, n, device=q.device)
+            pages = tables[seg, (keys // page_size).long()].long()
+            offs = (keys % page_size).long()
+            k = k_pages[pages, :, offs, :].double()          # [n, kv_heads, d]
+            v = v_pages[pages, :, :, offs].double()          # [n, kv_heads, d]
+            qr = q[r].double().view(heads, head_dim)
+            for h in range(heads):
+                s = (k[:, h // group, :] @ qr[h]) * scale
+                p = torch.softmax(s, dim=0)
+                out[r, h * head_dim:(h + 1) * head_dim] = (p @ v[:, h // group, :]).to(out.dtype)
+        return out
+
+    def argmax(self, logits, out):
+        for r in range(logits.shape[0]):
+            row = logits[r].float().cpu().numpy()
+            row = np.where(np.isfinite(row), row, -np.inf)
+            out[r] = 0 if not np.isfinite(row).any() else plain_llama.greedy(row)
+        return out
+
+    def sample(self, logits, work, params, out):
+        raw = params.cpu().numpy().tobytes()
+        rec = np.frombuffer(raw, dtype=np.dtype([("temperature", "<f4"), ("top_p", "<f4"), ("top_k", "<i4"),
+                                                 ("pad", "<i4"), ("seed", "<u8"), ("draw", "<u8")]))
+        for r in range(logits.shape[0]):
+            p = rec[r]
+            out[r] = plain_llama.device_sample(logits[r].float().cpu().numpy(), float(p["temperature"]), int(p["top_k"]),
+                                               float(p["top_p"]), int(p["seed"]), int(p["draw"]))
+        return out

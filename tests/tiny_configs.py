@@ -1,0 +1,40 @@
+"""Tiny Llama configurations for tests.  A and B differ in every size and option; C adds a
+sliding window on some layers, a partial rotary width, linear rotary scaling and biases."""
+import json
+
+import numpy as np
+import torch
+
+TINY_A = {
+    "model_type": "llama", "architectures": ["LlamaForCausalLM"],
+    "num_hidden_layers": 2, "hidden_size": 64, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 16,
+    "intermediate_size": 176, "vocab_size": 256, "rope_theta": 10000.0, "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": False, "max_position_embeddings": 128, "hidden_act": "silu",
+}
+TINY_B = {
+    "model_type": "llama", "architectures": ["LlamaForCausalLM"],
+    "num_hidden_layers": 3, "hidden_size": 160, "num_attention_heads": 5, "num_key_value_heads": 1, "head_dim": 32,
+    "intermediate_size": 432, "vocab_size": 512, "rope_theta": 500000.0, "rms_norm_eps": 1e-6,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 64},
+    "tie_word_embeddings": True, "max_position_embeddings": 256, "hidden_act": "silu",
+}
+TINY_C = {
+    "model_type": "llama", "architectures": ["LlamaForCausalLM"],
+    "num_hidden_layers": 4, "hidden_size": 96, "num_attention_heads": 6, "num_key_value_heads": 3, "head_dim": 48,
+    "intermediate_size": 200, "vocab_size": 300, "rope_theta": 50000.0, "rms_norm_eps": 3e-6,
+    "rope_scaling": {"rope_type": "linear", "factor": 2.0}, "partial_rotary_factor": 0.5,
+    "sliding_window": 24, "layer_types": ["sliding_attention", "full_attention", "sliding_attention", "full_attention"],
+    "tie_word_embeddings": False, "max_position_embeddings": 192, "hidden_act": "silu",
+}
+PAGE_SIZES = {"A": 16, "B": 8, "C": 16}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+
+
+def to_float64(tensors):
+    """Checkpoint tensors (torch, any float type) as float64 NumPy arrays for the plain implementation."""
+    return {n: t.to(torch.float64).numpy() for n, t in tensors.items()}
+
+
+def random_ids(n, vocab, seed):
+    return np.random.default_rng(seed).integers(0, vocab, size=n).tolist()
