@@ -12,6 +12,8 @@ extern "C" {
 
 const char *fllm_last_error(void);
 int fllm_abi_version(void);
+// 0: bfloat16 calls use the plain kernels only (for comparing them with the MFMA kernels); default 1
+void fllm_set_fast_kernels(int on);
 
 // out[r, :] = scale * table[ids[r], :]            out: float32 [rows, width]
 int fllm_embed(const int32_t *ids, const void *table, float *out, int rows, int width, int vocab, int table_dtype,
@@ -41,13 +43,16 @@ int fllm_rope_kv_store(void *qkv, const int32_t *row_pos, const int32_t *row_seg
 
 // Causal attention of each row over the pages of its segment: keys at positions
 // [max(0, pos - window + 1), pos] (window <= 0: from 0).  q: rows of `q_stride` elements, head h at
-// h * head_dim.  out: [rows, heads * head_dim].  `workspace` holds partial results of split
-// contexts (fllm_attention_workspace_bytes()).
+// h * head_dim.  out: [rows, heads * head_dim].  Rows of a segment are consecutive in the batch, at
+// consecutive positions; seg_start[s] is the first row of segment s (seg_start[num_segs] = rows).
+// `max_context` bounds pos + 1; `uniform_rows` says that every segment has one row (a decode
+// step).  `workspace` holds partial results of split contexts (fllm_attention_workspace_bytes()).
 int fllm_attention(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables,
-                   int table_stride, const int32_t *row_pos, const int32_t *row_seg, void *out, int rows, int heads,
-                   int kv_heads, int head_dim, int page_size, int num_pages, float scale, int window, int dtype,
-                   int max_context, int uniform_rows, void *workspace, size_t workspace_bytes, hipStream_t stream);
-size_t fllm_attention_workspace_bytes(int rows, int heads, int head_dim, int max_context);
+                   int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
+                   int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int page_size,
+                   int num_pages, float scale, int window, int dtype, int max_context, int uniform_rows,
+                   void *workspace, size_t workspace_bytes, hipStream_t stream);
+size_t fllm_attention_workspace_bytes(int rows, int heads, int kv_heads, int head_dim, int max_context);
 
 // out[r] = first index of the largest finite value of logits[r, :]
 int fllm_argmax(const float *logits, int32_t *out, int rows, int vocab, hipStream_t stream);

@@ -6,11 +6,11 @@
 #include "common.h"
 
 int fllm_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables,
-                             int table_stride, const int32_t *row_pos, const int32_t *row_seg, void *out, int rows,
-                             int heads, int kv_heads, int head_dim, int page_size, int num_pages, float scale, int window,
-                             int max_context, int uniform_rows, void *workspace, size_t workspace_bytes,
-                             hipStream_t stream);   // attention_mfma.hip; returns 1 when it declines the shape
-size_t fllm_attention_bf16_workspace_bytes(int rows, int heads, int head_dim, int max_context);
+                             int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
+                             int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int page_size,
+                             int num_pages, float scale, int window, int max_context, int uniform_rows, void *workspace,
+                             size_t workspace_bytes, hipStream_t stream);   // attention_mfma.hip; 1: shape declined
+size_t fllm_attention_bf16_workspace_bytes(int rows, int heads, int kv_heads, int head_dim, int max_context);
 
 namespace {
 
@@ -87,24 +87,27 @@ attention_generic_kernel(const T *__restrict__ q, int q_stride, const T *__restr
 
 }  // namespace
 
-extern "C" size_t fllm_attention_workspace_bytes(int rows, int heads, int head_dim, int max_context) {
-    return fllm_attention_bf16_workspace_bytes(rows, heads, head_dim, max_context);
+extern "C" size_t fllm_attention_workspace_bytes(int rows, int heads, int kv_heads, int head_dim, int max_context) {
+    return fllm_attention_bf16_workspace_bytes(rows, heads, kv_heads, head_dim, max_context);
 }
 
 extern "C" int fllm_attention(const void *q, int q_stride, const void *k_pages, const void *v_pages,
                               const int32_t *tables, int table_stride, const int32_t *row_pos, const int32_t *row_seg,
-                              void *out, int rows, int heads, int kv_heads, int head_dim, int page_size, int num_pages,
-                              float scale, int window, int dtype, int max_context, int uniform_rows, void *workspace,
-                              size_t workspace_bytes, hipStream_t stream) {
+                              const int32_t *seg_start, int num_segs, void *out, int rows, int heads, int kv_heads,
+                              int head_dim, int page_size, int num_pages, float scale, int window, int dtype,
+                              int max_context, int uniform_rows, void *workspace, size_t workspace_bytes,
+                              hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && heads > 0 && kv_heads > 0 && head_dim > 0 && page_size > 0 && table_stride > 0 && num_pages > 0,
                  "attention: bad sizes");
     FLLM_REQUIRE(heads % kv_heads == 0, "attention: %d heads are not a multiple of %d key/value heads", heads, kv_heads);
+    FLLM_REQUIRE(num_segs > 0 && seg_start != nullptr, "attention: segment starts are required");
     FLLM_REQUIRE(q_stride >= heads * head_dim, "attention: q_stride %d is shorter than heads*head_dim", q_stride);
     if (rows == 0) return 0;
     if (dtype == FLLM_BF16) {
-        const int fast = fllm_attention_bf16_fast(q, q_stride, k_pages, v_pages, tables, table_stride, row_pos, row_seg, out,
-                                                  rows, heads, kv_heads, head_dim, page_size, num_pages, scale, window,
-                                                  max_context, uniform_rows, workspace, workspace_bytes, stream);
+        const int fast = fllm_attention_bf16_fast(q, q_stride, k_pages, v_pages, tables, table_stride, row_pos, row_seg,
+                                                  seg_start, num_segs, out, rows, heads, kv_heads, head_dim, page_size,
+                                                  num_pages, scale, window, max_context, uniform_rows, workspace,
+                                                  workspace_bytes, stream);
         if (fast <= 0) return fast;
     }
     FLLM_REQUIRE(head_dim <= kBlock * kMaxDimPerThread, "attention: head_dim %d is larger than %d", head_dim,

@@ -1,8 +1,482 @@
+// Paged causal attention in bfloat16 on the MFMA units of gfx950: scores, softmax statistics
+// and output accumulate in float32.
+//
+// Both kernels compute the TRANSPOSED products, so that a lane keeps one query row throughout:
+//   S^T[key][q] = K[key][:] . Q[q][:]          (A = K fragment, B = Q fragment)
+//   O^T[d][q]  += V^T[d][key] * P^T[key][q]     (A = V^T fragment, B = P^T fragment)
+// With v_mfma_f32_16x16x32_bf16 the result tile D[m = 4*(l/16) + i][n = l%16] leaves lane l with
+// four keys of query l%16; the A rows of two consecutive S^T tiles are assigned to keys so that
+// these are the keys 8*(l/16) .. 8*(l/16)+7 of a 32-key block, which is exactly the B operand
+// layout of the second product: probabilities go from the first MFMA to the second without
+// leaving registers, and the running maximum and sum of a query row live in its lanes.
+// Values are stored transposed inside a page ([head_dim][token]) so that V^T fragments are
+// contiguous 16-byte loads.
+//
+//   tile kernel    portions of prompts: a workgroup takes up to 64 (token, head-of-group) rows of
+//                  one segment and one key/value head; keys and values go through LDS in tiles of 64.
+//   decode kernel  one row per segment: a workgroup takes (row, key/value head, context split), its
+//                  four waves stride over 32-key blocks loading K and V^T straight into MFMA
+//                  operands; splits are merged by a second kernel.
 #include "api.h"
 #include "common.h"
-int fllm_attention_bf16_fast(const void *, int, const void *, const void *, const int32_t *, int, const int32_t *,
-                             const int32_t *, void *, int, int, int, int, int, int, float, int, int, int, void *, size_t,
-                             hipStream_t) {
-    return 1;
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = 4;
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct AttnArgs {
+    const bf16_t *q;
+    int q_stride;
+    const bf16_t *kp;
+    const bf16_t *vp;
+    const int32_t *tables;
+    int table_stride;
+    const int32_t *row_pos;
+    const int32_t *row_seg;
+    const int32_t *seg_start;
+    int num_segs;
+    bf16_t *out;
+    int rows, heads, kv_heads, page_size;
+    float scale_log2;
+    int window;
+    float *ws_ml;   // [rows, heads, splits, 2]
+    float *ws_o;    // [rows, heads, splits, D]
+    int splits, keys_per_split;
+};
+
+__device__ __forceinline__ bf16x8_t zero8() {
+    bf16x8_t z;
+#pragma unroll
+    for (int i = 0; i < 8; i++) z[i] = (bf16_t)0.0f;
+    return z;
 }
-size_t fllm_attention_bf16_workspace_bytes(int, int, int, int) { return 0; }
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Online-softmax update of one query row held across the four lane groups of a wave.
+// s: NS score tiles (already scaled and masked with -inf); returns the P^T operands.
+template <int NS>
+__device__ __forceinline__ void softmax_step(f32x4_t (&s)[NS], float &m_run, float &l_run, float &alpha) {
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < NS; t++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) tmax = fmaxf(tmax, s[t][i]);
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+    const float m_new = fmaxf(m_run, tmax);
+    alpha = (m_run == -INFINITY) ? 0.f : fast_exp2(m_run - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int t = 0; t < NS; t++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float p = (s[t][i] == -INFINITY) ? 0.f : fast_exp2(s[t][i] - m_new);
+            s[t][i] = p;
+            psum += p;
+        }
+    psum += __shfl_xor(psum, 16, kWave);
+    psum += __shfl_xor(psum, 32, kWave);
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+}
+
+__device__ __forceinline__ bf16x8_t pack_p(const f32x4_t &lo, const f32x4_t &hi) {
+    bf16x8_t p;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        p[i] = (bf16_t)lo[i];
+        p[4 + i] = (bf16_t)hi[i];
+    }
+    return p;
+}
+
+// ---------------------------------------------------------------------------------------------
+// tile kernel
+// ---------------------------------------------------------------------------------------------
+template <int D>
+__global__ void __launch_bounds__(kThreads)
+attn_tile_kernel(AttnArgs p) {
+    constexpr int KT = 64;          // keys per tile
+    constexpr int KP = D + 8;       // pitch of a key row in LDS
+    constexpr int VP = KT + 8;      // pitch of a value row (one head_dim lane, KT keys) in LDS
+    constexpr int KD = D / 32, DT = D / 16;
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KP];
+    __shared__ __attribute__((aligned(16))) bf16_t Vs[D * VP];
+    __shared__ int s_tile[2];
+    const int G = p.heads / p.kv_heads;
+    const int TQ = 64 / G;          // tokens per tile
+    if (threadIdx.x == 0) {
+        int b = blockIdx.x, seg = -1, t0 = 0;
+        for (int s = 0; s < p.num_segs; s++) {
+            const int n = p.seg_start[s + 1] - p.seg_start[s];
+            const int nt = (n + TQ - 1) / TQ;
+            if (b < nt) {
+                seg = s;
+                t0 = b;
+                break;
+            }
+            b -= nt;
+        }
+        s_tile[0] = seg;
+        s_tile[1] = t0;
+    }
+    __syncthreads();
+    const int seg = s_tile[0];
+    if (seg < 0) return;
+    const int row0 = p.seg_start[seg] + s_tile[1] * TQ;
+    const int ntok = min(TQ, p.seg_start[seg + 1] - row0);
+    const int pos0 = p.row_pos[row0];
+    const int kvh = blockIdx.y;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int c = lane & 15, g = lane >> 4;
+    const int rr = wave * 16 + c;
+    const int tq = rr / G, hg = rr - tq * G;
+    const bool rvalid = tq < ntok;
+    const int prow = rvalid ? pos0 + tq : -1;
+    const int head = kvh * G + hg;
+    const int lo_r = (p.window > 0 && prow - p.window + 1 > 0) ? prow - p.window + 1 : 0;
+    const int ps = p.page_size, nkv = p.kv_heads;
+
+    bf16x8_t qf[KD];
+#pragma unroll
+    for (int kk = 0; kk < KD; kk++)
+        qf[kk] = rvalid ? *(const bf16x8_t *)(p.q + (size_t)(row0 + tq) * p.q_stride + (size_t)head * D + kk * 32 + g * 8)
+                        : zero8();
+
+    const int p_last = pos0 + ntok - 1;
+    const int lo_tile = (p.window > 0 && pos0 - p.window + 1 > 0) ? pos0 - p.window + 1 : 0;
+    const int kbegin = (lo_tile / KT) * KT;
+    const int32_t *tbl = p.tables + (size_t)seg * p.table_stride;
+    const int cpp = ps / 8;   // 16-byte chunks per value row of a page
+
+    f32x4_t o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) o[dt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+
+    for (int k0 = kbegin; k0 <= p_last; k0 += KT) {
+        __syncthreads();   // the previous tile has been read
+        for (int ch = threadIdx.x; ch < KT * D / 8; ch += kThreads) {
+            const int key = ch / (D / 8), dc = ch % (D / 8);
+            const int kabs = k0 + key;
+            bf16x8_t v = zero8();
+            if (kabs >= lo_tile && kabs <= p_last) {
+                const int page = tbl[kabs / ps], off = kabs % ps;
+                v = *(const bf16x8_t *)(p.kp + (((size_t)page * nkv + kvh) * ps + off) * D + dc * 8);
+            }
+            *(bf16x8_t *)(Ks + key * KP + dc * 8) = v;
+        }
+        for (int ch = threadIdx.x; ch < D * KT / 8; ch += kThreads) {
+            const int pg = ch / (D * cpp), rem = ch % (D * cpp);
+            const int d = rem / cpp, hc = rem % cpp;
+            const int koff = pg * ps + hc * 8;
+            const int kabs = k0 + koff;
+            bf16x8_t v = zero8();
+            if (kabs + 7 >= lo_tile && kabs <= p_last) {
+                const int page = tbl[kabs / ps];
+                v = *(const bf16x8_t *)(p.vp + (((size_t)page * nkv + kvh) * D + d) * ps + hc * 8);
+                if (kabs + 7 > p_last) {   // slots past the last token hold whatever an earlier request left
+#pragma unroll
+                    for (int e = 0; e < 8; e++)
+                        if (kabs + e > p_last) v[e] = (bf16_t)0.0f;
+                }
+            }
+            *(bf16x8_t *)(Vs + d * VP + koff) = v;
+        }
+        __syncthreads();
+
+        f32x4_t s[4];
+#pragma unroll
+        for (int st = 0; st < 4; st++) {
+            s[st] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+            const int kb = st >> 1, j = st & 1;
+            const int key_local = kb * 32 + (c >> 2) * 8 + j * 4 + (c & 3);   // A row c of this tile
+#pragma unroll
+            for (int kk = 0; kk < KD; kk++) {
+                const bf16x8_t a = *(const bf16x8_t *)(Ks + key_local * KP + kk * 32 + g * 8);
+                s[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[kk], s[st], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int st = 0; st < 4; st++) {
+            const int kb = st >> 1, j = st & 1;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int key = k0 + kb * 32 + g * 8 + j * 4 + i;
+                const bool vis = key <= prow && key >= lo_r;   // prow = -1 for rows outside the segment
+                s[st][i] = vis ? s[st][i] * p.scale_log2 : -INFINITY;
+            }
+        }
+        float alpha;
+        softmax_step<4>(s, m_run, l_run, alpha);
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) o[dt] *= alpha;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+            const bf16x8_t pf = pack_p(s[kb * 2], s[kb * 2 + 1]);
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) {
+                const bf16x8_t a = *(const bf16x8_t *)(Vs + (dt * 16 + c) * VP + kb * 32 + g * 8);
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf, o[dt], 0, 0, 0);
+            }
+        }
+    }
+    if (rvalid) {
+        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+        bf16_t *dst = p.out + ((size_t)(row0 + tq) * p.heads + head) * D + g * 4;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+            bf16x4_t v;
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[i] = (bf16_t)(o[dt][i] * inv);
+            *(bf16x4_t *)(dst + dt * 16) = v;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// decode kernel
+// ---------------------------------------------------------------------------------------------
+template <int D>
+__global__ void __launch_bounds__(kThreads)
+attn_decode_kernel(AttnArgs p, int qtiles) {
+    constexpr int KD = D / 32, DT = D / 16;
+    constexpr int OP = D + 1;
+    __shared__ float sm_m[kWaves][16], sm_l[kWaves][16];
+    __shared__ float sm_o[kWaves][16][OP];
+    const int row = blockIdx.x;
+    const int qtile = blockIdx.y % qtiles, kvh = blockIdx.y / qtiles;
+    const int split = blockIdx.z;
+    const int G = p.heads / p.kv_heads;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int c = lane & 15, g = lane >> 4;
+    const int hg = qtile * 16 + c;
+    const int seg = p.row_seg[row];
+    const bool qvalid = hg < G && seg >= 0;
+    const int head = kvh * G + (hg < G ? hg : 0);
+    const int n = seg >= 0 ? p.row_pos[row] + 1 : 0;
+    const int lo = (p.window > 0 && n - p.window > 0) ? n - p.window : 0;
+    const int ps = p.page_size, nkv = p.kv_heads;
+    const int begin = (lo / 32) * 32 + split * p.keys_per_split;
+    const int end = min(begin + p.keys_per_split, n);
+    const int32_t *tbl = p.tables + (size_t)(seg >= 0 ? seg : 0) * p.table_stride;
+
+    bf16x8_t qf[KD];
+#pragma unroll
+    for (int kk = 0; kk < KD; kk++)
+        qf[kk] = qvalid ? *(const bf16x8_t *)(p.q + (size_t)row * p.q_stride + (size_t)head * D + kk * 32 + g * 8) : zero8();
+
+    f32x4_t o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) o[dt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+
+    for (int kb = begin + wave * 32; kb < end; kb += kWaves * 32) {
+        // keys: A row c of tile j is key kb + 8*(c/4) + 4*j + c%4; both tiles of a lane lie in one group of 8
+        const int grp = kb + (c >> 2) * 8;
+        const bool gload = grp < n && grp + 8 > lo;
+        const int kpage = gload ? tbl[grp / ps] : 0;
+        f32x4_t s[2];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            s[j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+            const int key = grp + j * 4 + (c & 3);
+            const bool valid = gload && key >= lo && key < n;
+            const bf16_t *kr = p.kp + (((size_t)kpage * nkv + kvh) * ps + (key % ps)) * D + g * 8;
+#pragma unroll
+            for (int kk = 0; kk < KD; kk++) {
+                const bf16x8_t a = valid ? *(const bf16x8_t *)(kr + kk * 32) : zero8();
+                s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[kk], s[j], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int key = kb + g * 8 + j * 4 + i;
+                const bool vis = key >= lo && key < n;
+                s[j][i] = vis ? s[j][i] * p.scale_log2 : -INFINITY;
+            }
+        float alpha;
+        softmax_step<2>(s, m_run, l_run, alpha);
+        const bf16x8_t pf = pack_p(s[0], s[1]);
+        // values: lane (c, g) loads V^T[d = 16 dt + c][keys kb + 8g .. + 7]
+        const int vkey = kb + g * 8;
+        const bool vload = vkey < n && vkey + 8 > lo;
+        const int vpage = vload ? tbl[vkey / ps] : 0;
+        const bf16_t *vr = p.vp + (((size_t)vpage * nkv + kvh) * D + c) * ps + (vkey % ps);
+        const bool tail = vload && vkey + 8 > n;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+            bf16x8_t a = vload ? *(const bf16x8_t *)(vr + (size_t)dt * 16 * ps) : zero8();
+            if (tail) {   // slots past the last token hold whatever an earlier request left
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    if (vkey + e >= n) a[e] = (bf16_t)0.0f;
+            }
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf, o[dt] * alpha, 0, 0, 0);
+        }
+    }
+    // the four waves saw different keys: merge their statistics and outputs
+    if (g == 0) {
+        sm_m[wave][c] = m_run;
+        sm_l[wave][c] = l_run;
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) sm_o[wave][c][dt * 16 + g * 4 + i] = o[dt][i];
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 16 * D; idx += kThreads) {
+        const int qi = idx / D, d = idx - qi * D;
+        const int h = qtile * 16 + qi;
+        if (h >= G) continue;
+        float m = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kWaves; w++) m = fmaxf(m, sm_m[w][qi]);
+        float l = 0.f, acc = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; w++) {
+            const float f = sm_m[w][qi] == -INFINITY ? 0.f : fast_exp2(sm_m[w][qi] - m);
+            l += sm_l[w][qi] * f;
+            acc += sm_o[w][qi][d] * f;
+        }
+        const size_t hrow = (size_t)row * p.heads + kvh * G + h;
+        if (p.splits == 1) {
+            p.out[hrow * D + d] = (bf16_t)(l > 0.f ? acc / l : 0.f);
+        } else {
+            p.ws_o[(hrow * p.splits + split) * D + d] = acc;
+            if (d == 0) {
+                p.ws_ml[(hrow * p.splits + split) * 2] = m;
+                p.ws_ml[(hrow * p.splits + split) * 2 + 1] = l;
+            }
+        }
+    }
+}
+
+template <int D>
+__global__ void __launch_bounds__(kWave)
+attn_merge_kernel(const float *__restrict__ ws_ml, const float *__restrict__ ws_o, bf16_t *__restrict__ out, int heads,
+                  int splits) {
+    const size_t hrow = (size_t)blockIdx.x * heads + blockIdx.y;
+    float m = -INFINITY;
+    for (int s = 0; s < splits; s++) m = fmaxf(m, ws_ml[(hrow * splits + s) * 2]);
+    float l = 0.f;
+    for (int s = 0; s < splits; s++) {
+        const float ms = ws_ml[(hrow * splits + s) * 2];
+        l += ws_ml[(hrow * splits + s) * 2 + 1] * (ms == -INFINITY ? 0.f : fast_exp2(ms - m));
+    }
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    for (int d = threadIdx.x; d < D; d += kWave) {
+        float acc = 0.f;
+        for (int s = 0; s < splits; s++) {
+            const float ms = ws_ml[(hrow * splits + s) * 2];
+            acc += ws_o[(hrow * splits + s) * D + d] * (ms == -INFINITY ? 0.f : fast_exp2(ms - m));
+        }
+        out[hrow * D + d] = (bf16_t)(acc * inv);
+    }
+}
+
+// How a decode step of `rows` rows is split over the context: enough workgroups to fill 256 CUs,
+// at least 128 keys per split.
+void decode_split_plan(int rows, int kv_heads, int qtiles, int max_context, int *splits, int *keys_per_split) {
+    const long base = (long)rows * kv_heads * qtiles;
+    long want = (1024 + base - 1) / base;
+    const long most = (max_context + 127) / 128;
+    if (want > most) want = most;
+    if (want > 64) want = 64;
+    if (want < 1) want = 1;
+    const long span = (long)max_context + 31;   // the first split starts at a multiple of 32 at or below the first key
+    long per = (span + want - 1) / want;
+    per = (per + 127) / 128 * 128;
+    *splits = (int)want;
+    *keys_per_split = (int)per;
+}
+
+bool fast_shape(int heads, int kv_heads, int head_dim, int page_size) {
+    if (head_dim != 32 && head_dim != 64 && head_dim != 128) return false;
+    if (page_size != 8 && page_size != 16 && page_size != 32 && page_size != 64) return false;
+    if (heads / kv_heads > 64) return false;
+    return true;
+}
+
+template <int D>
+int launch(const AttnArgs &a, int uniform_rows, int max_context, void *workspace, size_t workspace_bytes,
+           hipStream_t stream) {
+    const int G = a.heads / a.kv_heads;
+    if (uniform_rows) {
+        const int qtiles = (G + 15) / 16;
+        AttnArgs p = a;
+        decode_split_plan(a.rows, a.kv_heads, qtiles, max_context, &p.splits, &p.keys_per_split);
+        if (p.splits > 1) {
+            const size_t need = (size_t)a.rows * a.heads * p.splits * (D + 2) * sizeof(float);
+            FLLM_REQUIRE(workspace != nullptr && workspace_bytes >= need,
+                         "attention: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+            p.ws_ml = (float *)workspace;
+            p.ws_o = p.ws_ml + (size_t)a.rows * a.heads * p.splits * 2;
+        }
+        FLLM_REQUIRE(a.kv_heads * qtiles <= 65535 && p.splits <= 65535, "attention: grid too large");
+        hipLaunchKernelGGL(attn_decode_kernel<D>, dim3(a.rows, a.kv_heads * qtiles, p.splits), dim3(kThreads), 0, stream, p,
+                           qtiles);
+        if (p.splits > 1)
+            hipLaunchKernelGGL(attn_merge_kernel<D>, dim3(a.rows, a.heads), dim3(kWave), 0, stream, p.ws_ml, p.ws_o, a.out,
+                               a.heads, p.splits);
+        return fllm_check_launch("attention_decode");
+    }
+    const int TQ = 64 / G;
+    const int tiles = (a.rows + TQ - 1) / TQ + a.num_segs;   // upper bound; surplus workgroups leave at once
+    hipLaunchKernelGGL(attn_tile_kernel<D>, dim3(tiles, a.kv_heads), dim3(kThreads), 0, stream, a);
+    return fllm_check_launch("attention_tile");
+}
+
+}  // namespace
+
+size_t fllm_attention_bf16_workspace_bytes(int rows, int heads, int kv_heads, int head_dim, int max_context) {
+    if (rows <= 0 || heads <= 0 || kv_heads <= 0) return 0;
+    const int qtiles = (heads / kv_heads + 15) / 16;
+    int splits, per;
+    decode_split_plan(rows, kv_heads, qtiles, max_context, &splits, &per);
+    if (splits <= 1) return 0;
+    return (size_t)rows * heads * splits * (head_dim + 2) * sizeof(float);
+}
+
+// 0: launched, negative: error, 1: shape declined (the caller uses the plain kernel)
+int fllm_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables,
+                             int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
+                             int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int page_size,
+                             int num_pages, float scale, int window, int max_context, int uniform_rows, void *workspace,
+                             size_t workspace_bytes, hipStream_t stream) {
+    if (!fllm_fast_kernels_enabled()) return 1;
+    (void)num_pages;
+    if (!fast_shape(heads, kv_heads, head_dim, page_size)) return 1;
+    if (q_stride % 8 != 0 || ((uintptr_t)q & 15) != 0) return 1;
+    if (uniform_rows && rows != num_segs) return 1;
+    AttnArgs a;
+    a.q = (const bf16_t *)q;
+    a.q_stride = q_stride;
+    a.kp = (const bf16_t *)k_pages;
+    a.vp = (const bf16_t *)v_pages;
+    a.tables = tables;
+    a.table_stride = table_stride;
+    a.row_pos = row_pos;
+    a.row_seg = row_seg;
+    a.seg_start = seg_start;
+    a.num_segs = num_segs;
+    a.out = (bf16_t *)out;
+    a.rows = rows;
+    a.heads = heads;
+    a.kv_heads = kv_heads;
+    a.page_size = page_size;
+    a.scale_log2 = scale * kLog2e;
+    a.window = window;
+    a.ws_ml = nullptr;
+    a.ws_o = nullptr;
+    a.splits = 1;
+    a.keys_per_split = 0;
+    if (head_dim == 32) return launch<32>(a, uniform_rows, max_context, workspace, workspace_bytes, stream);
+    if (head_dim == 64) return launch<64>(a, uniform_rows, max_context, workspace, workspace_bytes, stream);
+    return launch<128>(a, uniform_rows, max_context, workspace, workspace_bytes, stream);
+}

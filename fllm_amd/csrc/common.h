@@ -19,6 +19,8 @@ constexpr int kWave = 64;
 // text is read back through fllm_last_error().
 void fllm_set_error(const char *fmt, ...);
 int fllm_check_launch(const char *what);
+// 0 when the MFMA kernels are switched off (tests compare them with the plain kernels)
+int fllm_fast_kernels_enabled(void);
 
 #define FLLM_REQUIRE(cond, ...)            \
     do {                                   \

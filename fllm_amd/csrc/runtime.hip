@@ -22,5 +22,9 @@ int fllm_check_launch(const char *what) {
     return 0;
 }
 
+static int g_fast_kernels = 1;
+int fllm_fast_kernels_enabled(void) { return g_fast_kernels; }
+extern "C" void fllm_set_fast_kernels(int on) { g_fast_kernels = on ? 1 : 0; }
+
 extern "C" const char *fllm_last_error(void) { return g_error; }
 extern "C" int fllm_abi_version(void) { return 1; }

@@ -31,6 +31,7 @@ class StepContext:
     ids: torch.Tensor                       # int32 [R]
     row_pos: torch.Tensor                   # int32 [R]
     row_seg: torch.Tensor                   # int32 [R]
+    seg_start: torch.Tensor                 # int32 [S + 1]: first row of each segment, then R
     slots: torch.Tensor                     # int32 [S]
     logit_rows: torch.Tensor                # int32 [L]
     tables: List[torch.Tensor]              # per cache group: int32 [S, max_pages]
@@ -51,9 +52,9 @@ class StepContext:
         cos, sin = rt.shared[key]
         return cos, sin, 0, 0
 
-    def attention_workspace(self, rt, rows: int, heads: int, head_dim: int) -> Optional[torch.Tensor]:
+    def attention_workspace(self, rt, rows: int, heads: int, kv_heads: int, head_dim: int) -> Optional[torch.Tensor]:
         """Scratch for partial results of split contexts, one buffer per step shape."""
-        need = rt.ops.attention_workspace_bytes(rows, heads, head_dim, self.max_context)
+        need = rt.ops.attention_workspace_bytes(rows, heads, kv_heads, head_dim, self.max_context)
         if need == 0:
             return None
         buf = self._scratch.get("attention")

@@ -1,0 +1,185 @@
+"""The engine: requests in, token events out.  `Engine` puts the scheduler and the sampler on
+top of the step function, in the shape of the reference's runtime
+(rust/engine/src/runtime.rs:365-467 `submit*`, :2141-2149 `step`, :2212-3150 `step_round`,
+:3152-3168 `run_until_request_done`; driven without a server as in
+rust/engine/examples/perf_decode.rs:24-46).
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence as Seq, Union
+
+import torch
+
+from ..config.llama import read_config_json
+from ..registry import model_spec_from_config
+from ..sampling import SampleRequest, Sampler, SamplingParams
+from ..weights.loader import load_checkpoint
+from ..weights.random_init import random_tensors
+from .runner import ModelRunner, StepEntry
+from .scheduler import ScheduledStep, Scheduler, SchedulerConfig, Sequence
+
+
+@dataclass
+class TokenEvent:
+    request_id: str
+    token_id: int
+    finished: bool
+    finish_reason: Optional[str] = None     # "stop" | "length"
+
+
+@dataclass
+class EngineStats:
+    """Counters in the manner of the reference's BatchStats (runtime.rs:20-40)."""
+    forward_calls: int = 0
+    rows_total: int = 0
+    max_rows: int = 0
+    prefill_rows: int = 0
+    decode_rows: int = 0
+    preemptions: int = 0
+    scheduler_s: float = 0.0
+    forward_s: float = 0.0
+    postprocess_s: float = 0.0
+
+
+class Engine:
+    def __init__(self, model: Union[str, None] = None, *, config: Optional[dict] = None, seed: int = 0,
+                 dtype: str = "bfloat16", device: str = "cuda:0", ctx: Optional[int] = None, max_seqs: int = 16,
+                 max_batched_tokens: int = 512, block_size: int = 16, num_blocks: Optional[int] = None,
+                 gpu_memory_utilization: float = 0.90, decode_first: bool = True, kv_watermark_blocks: int = 0,
+                 max_num_partial_prefills: int = 0, long_prefill_token_threshold: int = 0,
+                 preemption_mode: str = "recompute", eos_token_ids: Optional[Seq[int]] = None, ops=None):
+        """`model`: a folder with config.json and safetensors; or `config` (a config.json dict)
+        with `seed` for random weights.  Option names follow the reference's server flags
+        (rust/engine/src/bin/serve.rs:530-557, :681-782): ctx, max_seqs, max_batched_tokens,
+        gpu_memory_utilization, kv_watermark_blocks, max_num_partial_prefills,
+        long_prefill_token_threshold, preemption_mode."""
+        if (model is None) == (config is None):
+            raise ValueError("give either a model folder or a config for random weights")
+        if model is not None:
+            config = read_config_json(model)
+        typed, spec = model_spec_from_config(config)
+        if model is not None:
+            tensors = load_checkpoint(model, spec)
+        else:
+            from .runner import parse_dtype
+            tensors = random_tensors(spec, seed, parse_dtype(dtype))
+        self.runner = ModelRunner(spec, tensors, dtype=dtype, device=device, page_size=block_size, num_pages=num_blocks,
+                                  max_requests=max_seqs, max_context=ctx, memory_utilization=gpu_memory_utilization,
+                                  ops=ops, typed_config=typed)
+        del tensors
+        self.config = typed
+        self.max_model_len = self.runner.max_context
+        self.scheduler = Scheduler(
+            SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=max_batched_tokens, decode_first=decode_first,
+                            watermark_pages=kv_watermark_blocks, max_partial_prefills=max_num_partial_prefills,
+                            long_prefill_threshold=long_prefill_token_threshold, preemption=preemption_mode),
+            self.runner.cache, self.max_model_len)
+        self.sampler = Sampler(self.runner.rt)
+        if eos_token_ids is None:
+            eos_token_ids = getattr(typed, "eos_token_ids", ()) or ()
+        self.eos_token_ids = tuple(int(t) for t in eos_token_ids)
+        self.stats = EngineStats()
+        self._requests: Dict[str, int] = {}
+        self._next_seq = 0
+
+    # ---- requests -------------------------------------------------------------------------
+    def add_request(self, request_id: str, prompt_token_ids: Seq[int], sampling: Optional[SamplingParams] = None) -> int:
+        sampling = sampling or SamplingParams()
+        prompt = [int(t) for t in prompt_token_ids]
+        if not request_id or not prompt:
+            raise ValueError("request id, prompt tokens, and max_tokens must be non-empty")
+        if len(prompt) + sampling.max_tokens > self.max_model_len:
+            raise ValueError("prompt plus max_tokens exceeds the configured model context")
+        if request_id in self._requests:
+            raise ValueError(f"request id already active: {request_id}")
+        for t in prompt:
+            if not 0 <= t < self.runner.vocab_size:
+                raise ValueError(f"token id {t} is outside [0, {self.runner.vocab_size})")
+        sid = self._next_seq
+        self._next_seq += 1
+        self.scheduler.add(Sequence(seq_id=sid, req_id=request_id, tokens=prompt, prompt_len=len(prompt), sampling=sampling))
+        self._requests[request_id] = sid
+        return sid
+
+    def abort_request(self, request_id: str) -> None:
+        sid = self._requests.pop(request_id, None)
+        if sid is not None:
+            self.scheduler.finish(sid)
+
+    def has_unfinished(self) -> bool:
+        return self.scheduler.has_work()
+
+    # ---- one round ------------------------------------------------------------------------
+    def step(self) -> List[TokenEvent]:
+        t0 = time.perf_counter()
+        plan = self.scheduler.schedule()
+        t1 = time.perf_counter()
+        self.stats.scheduler_s += t1 - t0
+        self.stats.preemptions = self.scheduler.preemptions
+        if plan is None:
+            if self.scheduler.has_work():
+                raise RuntimeError("scheduler could not make progress with the available KV pool")
+            return []
+        seqs = self.scheduler.sequences
+        entries: List[StepEntry] = []
+        sampled: List[int] = []                  # sequence ids whose row gives a token, in row order
+        for sid, start, count in plan.prefill:
+            seq = seqs[sid]
+            last = start + count == seq.prefill_target
+            entries.append(StepEntry(sid, seq.tokens[start:start + count], [count - 1] if last else []))
+            if last:
+                sampled.append(sid)
+            self.stats.prefill_rows += count
+        for sid in plan.decode:
+            entries.append(StepEntry(sid, [seqs[sid].tokens[-1]], [0]))
+            sampled.append(sid)
+            self.stats.decode_rows += 1
+        logits = self.runner.step(entries)
+        rows = sum(len(e.tokens) for e in entries)
+        self.stats.forward_calls += 1
+        self.stats.rows_total += rows
+        self.stats.max_rows = max(self.stats.max_rows, rows)
+        requests = [SampleRequest(seqs[sid].sampling, seqs[sid].sampling.seed_for(sid), seqs[sid].draws) for sid in sampled]
+        tokens = self.sampler.sample(logits, requests)
+        t2 = time.perf_counter()
+        self.stats.forward_s += t2 - t1
+        for sid, _, count in plan.prefill:
+            self.scheduler.commit_chunk(sid, count)
+        events: List[TokenEvent] = []
+        for sid, token in zip(sampled, tokens):
+            seq = seqs[sid]
+            seq.tokens.append(token)
+            if not seq.sampling.greedy:
+                seq.draws += 1
+            self.scheduler.commit_decode(sid)
+            hit_stop = seq.sampling.stops_on(token, self.eos_token_ids)
+            hit_limit = seq.remaining() == 0
+            reason = "stop" if hit_stop else ("length" if hit_limit else None)
+            if reason:
+                self.scheduler.finish(sid)
+                self._requests.pop(seq.req_id, None)
+            events.append(TokenEvent(seq.req_id, token, reason is not None, reason))
+        self.stats.postprocess_s += time.perf_counter() - t2
+        return events
+
+    # ---- whole requests -------------------------------------------------------------------
+    def generate(self, prompts: Seq[Seq[int]], sampling: Union[SamplingParams, Seq[SamplingParams], None] = None
+                 ) -> List[List[int]]:
+        """Generated token ids of every prompt (token ids in, token ids out)."""
+        if sampling is None or isinstance(sampling, SamplingParams):
+            sampling = [sampling or SamplingParams()] * len(prompts)
+        if len(sampling) != len(prompts):
+            raise ValueError("one SamplingParams per prompt is required")
+        names = []
+        for i, (p, s) in enumerate(zip(prompts, sampling)):
+            name = f"generate-{self._next_seq}-{i}"
+            self.add_request(name, p, s)
+            names.append(name)
+        outputs: Dict[str, List[int]] = {n: [] for n in names}
+        while any(n in self._requests for n in names):
+            for ev in self.step():
+                if ev.request_id in outputs:
+                    outputs[ev.request_id].append(ev.token_id)
+        return [outputs[n] for n in names]

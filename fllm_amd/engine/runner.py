@@ -202,7 +202,10 @@ class ModelRunner:
                 t = self.cache.table(e.req_id, g)
                 flat_tables.extend(t)
                 flat_tables.extend([-1] * (width - len(t)))
-        packed = torch.tensor(ids + row_pos + row_seg + slots + logit_rows + flat_tables, dtype=torch.int32)
+        cu_rows = [0]
+        for n in seg_rows:
+            cu_rows.append(cu_rows[-1] + n)
+        packed = torch.tensor(ids + row_pos + row_seg + cu_rows + slots + logit_rows + flat_tables, dtype=torch.int32)
         packed = packed.to(self.device, non_blocking=False)
         R, L = len(ids), len(logit_rows)
         o = 0
@@ -213,8 +216,9 @@ class ModelRunner:
             o += count
             return out
 
-        t_ids, t_pos, t_seg, t_slots, t_rows = take(R), take(R), take(R), take(S), take(L)
+        t_ids, t_pos, t_seg, t_cu, t_slots, t_rows = take(R), take(R), take(R), take(S + 1), take(S), take(L)
         tables = [take(S * w).view(S, w) for w in widths]
-        return StepContext(num_rows=R, num_segments=S, ids=t_ids, row_pos=t_pos, row_seg=t_seg, slots=t_slots,
+        return StepContext(num_rows=R, num_segments=S, ids=t_ids, row_pos=t_pos, row_seg=t_seg, seg_start=t_cu,
+                           slots=t_slots,
                            logit_rows=t_rows, tables=tables, seg_rows=seg_rows, seg_pos_start=seg_start,
                            seg_slots=slots, max_context=max_context, uniform_rows=all(n == 1 for n in seg_rows))

@@ -1,0 +1,207 @@
+"""Continuous-batching scheduler: admits requests, cuts prompts into portions under a token
+budget, schedules one decode token per running sequence, and decides what happens when pages
+run out.  Behaviour follows the reference's scheduler (rust/engine/src/scheduler.rs):
+
+  admission   first come, first served; a request is admitted when a sequence slot is free and
+              the cache can hold its whole prompt plus one generated token (+ the watermark
+              when others run); the head of the queue blocks those behind it (:494-624, :659-697)
+  portions    each running sequence that still has prompt left gets min(rest, budget) tokens;
+              with `decode_first` one token of the budget is kept per decoding sequence
+              (:340-400)
+  decoding    every running sequence whose prompt is computed gets one row; if no page is left
+              for it the newest running sequence is preempted (:401-455, :647-657)
+  preemption  by recompute: all pages go back, the sequence returns to the FRONT of the queue
+              and later prefills prompt and generated tokens again (:933-968)
+
+The scheduler does the cache bookkeeping (reserve at admission and before a decode row); the
+step function commits what it ran.
+"""
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Deque, Dict, List, Optional, Tuple
+
+from ..cache import CacheManager, OutOfPages
+from ..sampling.params import SamplingParams
+
+
+@dataclass
+class SchedulerConfig:
+    max_num_seqs: int = 16                  # scheduler.rs:225-248 defaults
+    max_num_batched_tokens: int = 512
+    decode_first: bool = False
+    watermark_pages: int = 0
+    max_partial_prefills: int = 0           # 0: no limit
+    long_prefill_threshold: int = 0         # 0: no distinction
+    max_long_partial_prefills: int = 1
+    preemption: str = "recompute"
+
+    def __post_init__(self):
+        if self.max_num_seqs <= 0 or self.max_num_batched_tokens <= 0:
+            raise ValueError("max_num_seqs and max_num_batched_tokens must be positive")
+        if self.preemption not in ("recompute", "none"):
+            raise ValueError("preemption must be 'recompute' or 'none'")
+
+
+@dataclass
+class Sequence:
+    seq_id: int
+    req_id: str
+    tokens: List[int]                       # prompt, then generated tokens
+    prompt_len: int
+    sampling: SamplingParams
+    num_computed: int = 0                   # tokens whose keys and values are in the cache
+    prefill_target: int = 0                 # tokens to run as prompt (all tokens after a preemption)
+    state: str = "waiting"                  # waiting | running | finished
+    preempted: bool = False
+    arrival: int = 0
+    draws: int = 0                          # random draws taken so far
+
+    @property
+    def output_len(self) -> int:
+        return len(self.tokens) - self.prompt_len
+
+    def remaining(self) -> int:
+        return self.sampling.max_tokens - self.output_len
+
+
+@dataclass
+class ScheduledStep:
+    prefill: List[Tuple[int, int, int]] = field(default_factory=list)    # (seq_id, start, count)
+    decode: List[int] = field(default_factory=list)
+
+
+class Scheduler:
+    def __init__(self, cfg: SchedulerConfig, cache: CacheManager, max_model_len: int):
+        self.cfg = cfg
+        self.cache = cache
+        self.max_model_len = max_model_len
+        self.sequences: Dict[int, Sequence] = {}
+        self.waiting: Deque[int] = deque()
+        self.running: List[int] = []
+        self.preemptions = 0
+        self._arrivals = 0
+
+    # ---- queue ----------------------------------------------------------------------------
+    def add(self, seq: Sequence) -> None:
+        seq.arrival = self._arrivals
+        self._arrivals += 1
+        seq.prefill_target = len(seq.tokens)
+        seq.state = "waiting"
+        self.sequences[seq.seq_id] = seq
+        self.waiting.append(seq.seq_id)
+
+    def has_work(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    def _try_admit(self, sid: int) -> bool:
+        seq = self.sequences[sid]
+        if len(seq.tokens) > self.max_model_len:
+            return False
+        self.cache.add_request(sid)
+        total = len(seq.tokens) + 1
+        missing = self.cache.pages_missing(sid, total)
+        watermark = self.cfg.watermark_pages if self.running else 0
+        if any(m + watermark > self.cache.free_pages(g) for g, m in enumerate(missing)):
+            self.cache.free_request(sid)
+            return False
+        self.cache.reserve(sid, total)
+        seq.num_computed = 0
+        return True
+
+    def _admit_waiting(self) -> None:
+        while self.waiting and len(self.running) < self.cfg.max_num_seqs:
+            sid = self.waiting[0]
+            if self.cache.free_slots() == 0 or not self._try_admit(sid):
+                break                       # the head of the queue blocks those behind it
+            self.waiting.popleft()
+            self.sequences[sid].state = "running"
+            self.running.append(sid)
+
+    def _preempt(self, sid: int) -> None:
+        seq = self.sequences[sid]
+        seq.preempted = True
+        self.preemptions += 1
+        self.cache.free_request(sid)
+        seq.num_computed = 0
+        seq.prefill_target = len(seq.tokens)
+        seq.state = "waiting"
+        self.running.remove(sid)
+        self.waiting.appendleft(sid)
+
+    # ---- one step -------------------------------------------------------------------------
+    def schedule(self) -> Optional[ScheduledStep]:
+        self._admit_waiting()
+        if not self.running:
+            return None
+        step = ScheduledStep()
+        budget = self.cfg.max_num_batched_tokens
+        decoders = sum(1 for sid in self.running
+                       if self.sequences[sid].num_computed >= self.sequences[sid].prefill_target
+                       and self.sequences[sid].remaining() > 0)
+        prefill_budget = max(1, budget - decoders) if self.cfg.decode_first else budget
+        long_prefills = 0
+        for sid in list(self.running):
+            if prefill_budget == 0 or budget == 0:
+                break
+            if self.cfg.max_partial_prefills > 0 and len(step.prefill) >= self.cfg.max_partial_prefills:
+                break
+            seq = self.sequences[sid]
+            todo = seq.prefill_target - seq.num_computed
+            if todo <= 0:
+                continue
+            is_long = self.cfg.long_prefill_threshold > 0 and seq.prefill_target > self.cfg.long_prefill_threshold
+            if is_long and long_prefills >= max(1, self.cfg.max_long_partial_prefills):
+                continue
+            chunk = min(todo, prefill_budget)
+            if not self.cache.can_reserve(sid, seq.num_computed + chunk):
+                break
+            self.cache.reserve(sid, seq.num_computed + chunk)
+            step.prefill.append((sid, seq.num_computed, chunk))
+            budget -= chunk
+            prefill_budget -= chunk
+            long_prefills += int(is_long)
+        for sid in list(self.running):
+            if sid not in self.running:
+                continue                    # preempted by an earlier sequence of this loop
+            seq = self.sequences[sid]
+            if seq.num_computed < seq.prefill_target or seq.remaining() <= 0:
+                continue
+            if any(sid == p[0] for p in step.prefill):
+                continue
+            if budget == 0:
+                break
+            total = len(seq.tokens)         # the newest token has no keys yet: it is this row
+            if not self.cache.can_reserve(sid, total):
+                if self.cfg.preemption == "recompute" and len(self.running) > 1:
+                    victim = self.running[-1]
+                    if victim != sid:
+                        self._preempt(victim)
+                        step.decode = [d for d in step.decode if d != victim]
+                        step.prefill = [p for p in step.prefill if p[0] != victim]
+                if not self.cache.can_reserve(sid, total):
+                    continue
+            self.cache.reserve(sid, total)
+            budget -= 1
+            step.decode.append(sid)
+        if not step.prefill and not step.decode:
+            return None
+        return step
+
+    # ---- after the step -------------------------------------------------------------------
+    def commit_chunk(self, sid: int, count: int) -> None:
+        self.sequences[sid].num_computed += count
+
+    def commit_decode(self, sid: int) -> None:
+        seq = self.sequences[sid]
+        seq.num_computed = len(seq.tokens) - 1      # the token just appended is the next decode row
+
+    def finish(self, sid: int) -> None:
+        seq = self.sequences.pop(sid)
+        seq.state = "finished"
+        if sid in self.running:
+            self.running.remove(sid)
+        if sid in self.waiting:
+            self.waiting.remove(sid)
+        self.cache.free_request(sid)

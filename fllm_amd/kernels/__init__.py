@@ -57,8 +57,8 @@ def load_library(build_if_missing: bool = True):
         "fllm_swiglu": [c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_rope_kv_store": [c_void, c_void, c_void, c_void, c_int, c_void, c_void, c_int, c_void, c_void, c_int,
                                c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
-        "fllm_attention": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int,
-                           c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void, c_size, c_void],
+        "fllm_attention": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_int,
+                           c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void, c_size, c_void],
         "fllm_argmax": [c_void, c_void, c_int, c_int, c_void],
         "fllm_sample": [c_void, c_void, c_void, c_void, c_int, c_int, c_void],
     }
@@ -66,7 +66,9 @@ def load_library(build_if_missing: bool = True):
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = c_int
-    lib.fllm_attention_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int]
+    lib.fllm_set_fast_kernels.argtypes = [c_int]
+    lib.fllm_set_fast_kernels.restype = None
+    lib.fllm_attention_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int, c_int]
     lib.fllm_attention_workspace_bytes.restype = c_size
     _lib = lib
     return lib
@@ -97,6 +99,10 @@ class Ops:
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible: the engine runs on gfx950 only")
         self.lib = load_library()
+
+    def set_fast_kernels(self, on: bool) -> None:
+        """Off: bfloat16 calls run the plain kernels (tests compare the two)."""
+        self.lib.fllm_set_fast_kernels(1 if on else 0)
 
     def _check(self, code: int) -> None:
         if code != 0:
@@ -194,11 +200,11 @@ class Ops:
             _ptr(k_pages), _ptr(v_pages), num_pages, rows, heads, kv_heads, head_dim, rope_dims, pairing, page_size,
             _DTYPE_CODE[qkv.dtype], 1 if store else 0, self._stream()))
 
-    def attention_workspace_bytes(self, rows: int, heads: int, head_dim: int, max_context: int) -> int:
-        return int(self.lib.fllm_attention_workspace_bytes(rows, heads, head_dim, max_context))
+    def attention_workspace_bytes(self, rows: int, heads: int, kv_heads: int, head_dim: int, max_context: int) -> int:
+        return int(self.lib.fllm_attention_workspace_bytes(rows, heads, kv_heads, head_dim, max_context))
 
     def attention(self, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, tables: torch.Tensor,
-                  row_pos: torch.Tensor, row_seg: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int,
+                  row_pos: torch.Tensor, row_seg: torch.Tensor, seg_start: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int,
                   head_dim: int, page_size: int, scale: float, window: Optional[int], max_context: int,
                   uniform_rows: int = 0, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
         """`q` may be a column slice of a wider row-major matrix (the fused qkv buffer).
@@ -215,6 +221,9 @@ class Ops:
         _need(tables.dim() == 2, "tables must be [segments, pages]")
         _dense(row_pos, "row_pos", torch.int32, (rows,))
         _dense(row_seg, "row_seg", torch.int32, (rows,))
+        _dense(seg_start, "seg_start", torch.int32)
+        _need(seg_start.numel() >= 2, "seg_start must hold at least one segment")
+        _need(tables.shape[0] >= seg_start.numel() - 1, "tables must have a row per segment")
         _dense(out, "out", q.dtype, (rows, heads * head_dim))
         ws_ptr, ws_bytes = None, 0
         if workspace is not None:
@@ -223,7 +232,7 @@ class Ops:
         q_stride = q.stride(0) if rows > 1 else heads * head_dim
         self._check(self.lib.fllm_attention(
             _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(tables), tables.shape[1], _ptr(row_pos), _ptr(row_seg),
-            _ptr(out), rows, heads, kv_heads, head_dim, page_size, num_pages, float(scale),
+            _ptr(seg_start), seg_start.numel() - 1, _ptr(out), rows, heads, kv_heads, head_dim, page_size, num_pages, float(scale),
             int(window) if window else 0, _DTYPE_CODE[q.dtype], int(max_context), int(uniform_rows), ws_ptr, ws_bytes,
             self._stream()))
         return out

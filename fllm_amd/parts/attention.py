@@ -74,9 +74,10 @@ class PagedAttention(Mixer):
                           binding.k_pages if binding.writes else None, binding.v_pages if binding.writes else None,
                           nh, nkv, d, dims, pairing, binding.page_size)
         out = rt.empty((rows, nh * d))
-        ops.attention(qkv[:, : nh * d], binding.k_pages, binding.v_pages, tables, ctx.row_pos, ctx.row_seg, out,
-                      nh, nkv, d, binding.page_size, self.scale, self.window, ctx.max_context,
-                      uniform_rows=1 if ctx.uniform_rows else 0, workspace=ctx.attention_workspace(rt, rows, nh, d))
+        ops.attention(qkv[:, : nh * d], binding.k_pages, binding.v_pages, tables, ctx.row_pos, ctx.row_seg, ctx.seg_start,
+                      out, nh, nkv, d, binding.page_size, self.scale, self.window, ctx.max_context,
+                      uniform_rows=1 if ctx.uniform_rows else 0,
+                      workspace=ctx.attention_workspace(rt, rows, nh, nkv, d))
         ops.linear(out, self.w_o, residual, bias=self.b_o, accumulate=True)
 
 

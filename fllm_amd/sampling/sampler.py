@@ -1,0 +1,53 @@
+"""Chooses tokens from logits on the device: argmax for greedy rows, the device sampler
+otherwise (temperature, top-k, top-p, Gumbel-max draw keyed by seed and draw number)."""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+from typing import List, Sequence
+
+import torch
+
+from .params import SamplingParams
+
+
+@dataclass
+class SampleRequest:
+    params: SamplingParams
+    seed: int
+    draw: int
+
+
+_RECORD = 32   # bytes of one row record: float temperature, float top_p, int32 top_k, int32 pad, uint64 seed, uint64 draw
+
+
+def pack_rows(rows: Sequence[SampleRequest]) -> torch.Tensor:
+    """The row records the sampling kernel reads, as a uint8 CPU tensor [rows, 32]."""
+    import struct
+    raw = bytearray()
+    for r in rows:
+        p = r.params
+        raw += struct.pack("<ffiiQQ", float(p.temperature), float(p.top_p), int(p.top_k), 0,
+                           int(r.seed) & ((1 << 64) - 1), int(r.draw))
+    return torch.frombuffer(raw, dtype=torch.uint8).view(len(rows), _RECORD).clone()
+
+
+class Sampler:
+    def __init__(self, rt):
+        self.rt = rt
+
+    def sample(self, logits: torch.Tensor, rows: Sequence[SampleRequest]) -> List[int]:
+        """`logits`: float32 [len(rows), vocab] on the device.  Returns one token id per row."""
+        count = logits.shape[0]
+        if count != len(rows):
+            raise ValueError(f"{count} rows of logits for {len(rows)} requests")
+        if count == 0:
+            return []
+        out = torch.empty(count, dtype=torch.int32, device=logits.device)
+        if all(r.params.greedy for r in rows):
+            self.rt.ops.argmax(logits, out)
+        else:
+            params = pack_rows(rows).to(logits.device)
+            work = torch.empty_like(logits)
+            self.rt.ops.sample(logits, work, params, out)
+        return [int(t) for t in out.cpu().tolist()]

@@ -69,10 +69,10 @@ class ReferenceOps:
             k_pages[page, :, off, :] = view[r, heads:heads + kv_heads, :]
             v_pages[page, :, :, off] = view[r, heads + kv_heads:, :]
 
-    def attention_workspace_bytes(self, rows, heads, head_dim, max_context):
+    def attention_workspace_bytes(self, rows, heads, kv_heads, head_dim, max_context):
         return 0
 
-    def attention(self, q, k_pages, v_pages, tables, row_pos, row_seg, out, heads, kv_heads, head_dim, page_size, scale,
+    def attention(self, q, k_pages, v_pages, tables, row_pos, row_seg, seg_start, out, heads, kv_heads, head_dim, page_size, scale,
                   window, max_context, uniform_rows=0, workspace=None):
         rows = q.shape[0]
         group = heads // kv_heads

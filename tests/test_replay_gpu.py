@@ -1,0 +1,115 @@
+"""Replays the same requests whole, with the last 32 tokens one by one, in portions of changing
+size, and mixed with other requests on so few pages that they are used again, in float32 and in
+bfloat16, and compares every logit with the plain implementation."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama
+import tiny_configs as tc
+import trace_tools as tt
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {"A": [5, 17, 31, 70, 128, 100], "B": [1, 9, 40, 100, 256, 130], "C": [3, 50, 190, 77, 120, 64]}
+# |engine - plain| <= tol * max|plain logit| ; float32 engine against a float64 reference, and
+# bfloat16 (8 bits of mantissa in weights, activations and cache) against the same
+TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    """Model folders written with the safetensors library (not the engine's writer), in bfloat16-exact
+    float32 values so that both precisions read the same weights."""
+    from safetensors.torch import save_file
+    import json
+    from fllm_amd.registry import model_spec_from_config
+    from fllm_amd.weights import random_tensors
+    out = {}
+    for name, cfg in tc.CONFIGS.items():
+        _, spec = model_spec_from_config(cfg)
+        tensors = random_tensors(spec, seed=11 + ord(name), dtype=torch.bfloat16, with_optional=(name == "C"))
+        tensors = {k: v.to(torch.float32) for k, v in tensors.items()}
+        folder = str(tmp_path_factory.mktemp(f"tiny_{name}"))
+        with open(os.path.join(folder, "config.json"), "w") as fh:
+            json.dump(cfg, fh)
+        save_file(tensors, os.path.join(folder, "model.safetensors"))
+        requests = {f"r{i}": tc.random_ids(n, cfg["vocab_size"], 100 * ord(name) + i) for i, n in enumerate(LENGTHS[name])}
+        w64 = tc.to_float64(tensors)
+        plain = {rid: plain_llama.forward(cfg, w64, toks) for rid, toks in requests.items()}
+        out[name] = (folder, cfg, requests, plain)
+    return out
+
+
+def check(got, plain, dtype, what):
+    for rid, want in plain.items():
+        assert rid in got, f"{what}: request {rid} missing"
+        assert got[rid].shape == want.shape, f"{what}: {rid} has shape {got[rid].shape}, expected {want.shape}"
+        err = np.abs(got[rid].astype(np.float64) - want)
+        scale = np.abs(want).max()
+        pos = int(err.max(axis=1).argmax())
+        assert err.max() <= TOL[dtype] * scale, (f"{what}: request {rid}: max error {err.max():.3e} at position {pos} "
+                                                 f"(limit {TOL[dtype] * scale:.3e}); first position over the limit: "
+                                                 f"{int(np.argmax(err.max(axis=1) > TOL[dtype] * scale))}")
+
+
+def make_runner(folder, dtype, page_size, max_tokens):
+    from fllm_amd.engine import ModelRunner
+    return ModelRunner.from_folder(folder, dtype=dtype, page_size=page_size, max_tokens=max_tokens, max_requests=8)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("family", ["whole", "last32", "portions", "mixed"])
+def test_replay(models, tmp_path, name, dtype, family):
+    folder, cfg, requests, plain = models[name]
+    steps = {"whole": tt.whole, "last32": tt.last_tokens_one_by_one, "portions": tt.portions,
+             "mixed": lambda r: tt.mixed(r, seed=5)}[family](requests)
+    steps = tt.number(steps)
+    max_tokens = tt.live_tokens_bound(steps)
+    runner = make_runner(folder, dtype, tc.PAGE_SIZES[name], max_tokens)
+    handed_out = tt.record_allocations(runner.cache)
+    got = tt.run_in_process(runner, steps, cfg["vocab_size"], str(tmp_path))
+    check(got, plain, dtype, f"{name} {dtype} {family}")
+    runner.cache.check_invariants()
+    assert all(pool.available == pool.num_pages for pool in runner.cache.pools), "pages were lost"
+    for pages in handed_out:
+        assert len(pages) > len(set(pages)), "the trace was meant to use pages again"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(models, tmp_path, dtype):
+    """bin/trace_run as a user starts it: steps on stdin, `done` lines back, files in --out."""
+    folder, cfg, requests, plain = models["A"]
+    steps = tt.number(tt.mixed(requests, seed=9))
+    got = tt.run_subprocess(folder, dtype, steps, cfg["vocab_size"], str(tmp_path), tt.live_tokens_bound(steps))
+    check(got, plain, dtype, f"trace_run {dtype}")
+
+
+def test_cuts_agree_bit_for_bit_in_float32(models, tmp_path):
+    """float32: every output element is one fixed chain of operations, so the way requests are
+    cut into steps and batched changes nothing at all."""
+    folder, cfg, requests, plain = models["B"]
+    results = []
+    for i, make in enumerate([tt.whole, tt.portions, lambda r: tt.mixed(r, seed=3)]):
+        steps = tt.number(make(requests))
+        runner = make_runner(folder, "float32", 8, tt.live_tokens_bound(steps))
+        sub = tmp_path / str(i)
+        results.append(tt.run_in_process(runner, steps, cfg["vocab_size"], str(sub)))
+    for rid in requests:
+        assert np.array_equal(results[0][rid], results[1][rid]), f"whole vs portions differ for {rid}"
+        assert np.array_equal(results[0][rid], results[2][rid]), f"whole vs mixed differ for {rid}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_and_long_decoding(models, tmp_path, dtype):
+    """A request decoded token by token from its very first token, up to the context limit."""
+    folder, cfg, requests, plain = models["B"]
+    rid = "r4"                                   # 256 tokens: the whole context of config B
+    one = {rid: requests[rid]}
+    steps = tt.number(tt.last_tokens_one_by_one(one, tail=256))
+    runner = make_runner(folder, dtype, 8, 256)
+    got = tt.run_in_process(runner, steps, cfg["vocab_size"], str(tmp_path))
+    check(got, {rid: plain[rid]}, dtype, f"token by token {dtype}")

@@ -1,0 +1,140 @@
+"""Weights: binding by name, the one error that lists everything, the safetensors reader's
+refusals, random-weights mode."""
+import json
+import os
+import struct
+
+import pytest
+import torch
+
+import tiny_configs as tc
+from fllm_amd.registry import model_spec_from_config
+from fllm_amd.weights import (SafetensorsError, SafetensorsFile, WeightsError, check_tensors, expected_tensors,
+                              load_checkpoint, open_checkpoint, random_tensors, write_random_model, write_safetensors)
+
+
+def test_expected_tensors_of_llama():
+    _, spec = model_spec_from_config(tc.TINY_A)
+    required, optional, _ = expected_tensors(spec)
+    assert required["model.embed_tokens.weight"] == (256, 64)
+    assert required["lm_head.weight"] == (256, 64)
+    assert required["model.layers.1.self_attn.k_proj.weight"] == (32, 64)
+    assert required["model.layers.0.mlp.down_proj.weight"] == (64, 176)
+    assert required["model.norm.weight"] == (64,)
+    assert len(required) == 3 + 2 * 9
+    assert optional["model.layers.0.self_attn.q_proj.bias"] == (64,)
+    _, tied = model_spec_from_config(tc.TINY_B)
+    assert "lm_head.weight" not in expected_tensors(tied)[0]
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes():
+    _, spec = model_spec_from_config(tc.TINY_A)
+    shapes = {n: tuple(s) for n, s in expected_tensors(spec)[0].items()}
+    del shapes["model.norm.weight"]
+    del shapes["model.layers.0.mlp.up_proj.weight"]
+    shapes["model.layers.0.self_attn.q_proj.weight"] = (64, 63)
+    shapes["model.layers.7.mlp.up_proj.weight"] = (176, 64)
+    shapes["model.rotary_emb.inv_freq"] = (8,)            # known, ignorable
+    with pytest.raises(WeightsError) as info:
+        check_tensors(spec, shapes)
+    e = info.value
+    assert e.missing == ["model.layers.0.mlp.up_proj.weight", "model.norm.weight"]
+    assert e.unexpected == ["model.layers.7.mlp.up_proj.weight"]
+    assert e.wrong_shape == [("model.layers.0.self_attn.q_proj.weight", (64, 63), (64, 64))]
+    text = str(e)
+    for needle in ("missing tensors (2)", "unexpected tensors (1)", "wrong shapes (1)", "expected [64, 64]"):
+        assert needle in text
+
+
+def test_tied_checkpoint_may_hold_a_head(tmp_path):
+    _, spec = model_spec_from_config(tc.TINY_B)
+    tensors = random_tensors(spec, 1, torch.float32)
+    tensors["lm_head.weight"] = torch.zeros(512, 160)
+    check_tensors(spec, {n: tuple(t.shape) for n, t in tensors.items()})
+
+
+def test_random_model_folder_round_trip(tmp_path):
+    spec = write_random_model(str(tmp_path), tc.TINY_A, seed=3, dtype="bfloat16")
+    assert sorted(os.listdir(tmp_path)) == ["config.json", "model.safetensors"]
+    loaded = load_checkpoint(str(tmp_path), spec)
+    again = random_tensors(spec, 3, torch.bfloat16)
+    assert set(loaded) == set(again)
+    for n in again:
+        assert loaded[n].dtype == torch.bfloat16 and torch.equal(loaded[n], again[n])
+    other = random_tensors(spec, 4, torch.bfloat16)
+    assert not torch.equal(other["model.norm.weight"], again["model.norm.weight"])
+    exact = random_tensors(spec, 3, torch.float32)
+    assert torch.equal(exact["model.norm.weight"].to(torch.bfloat16), again["model.norm.weight"])
+    w = exact["model.layers.0.mlp.up_proj.weight"]
+    assert abs(w.std().item() - 0.02) < 0.002 and abs(w.mean().item()) < 0.002
+    n = exact["model.norm.weight"]
+    assert 0.9 <= n.min().item() and n.max().item() <= 1.1
+
+
+def test_stored_types_are_kept(tmp_path):
+    _, spec = model_spec_from_config(tc.TINY_A)
+    tensors = random_tensors(spec, 1, torch.bfloat16)
+    tensors["model.norm.weight"] = tensors["model.norm.weight"].float()       # a tensor stored in 32-bit stays so
+    os.makedirs(tmp_path, exist_ok=True)
+    write_safetensors(str(tmp_path / "model.safetensors"), tensors)
+    loaded = load_checkpoint(str(tmp_path), spec)
+    assert loaded["model.norm.weight"].dtype == torch.float32
+    assert loaded["lm_head.weight"].dtype == torch.bfloat16
+
+
+def _write_raw(path, header, data=b""):
+    raw = json.dumps(header).encode()
+    with open(path, "wb") as fh:
+        fh.write(struct.pack("<Q", len(raw)) + raw + data)
+
+
+@pytest.mark.parametrize("header,data,text", [
+    ({"a": {"dtype": "F32", "shape": [2], "data_offsets": [0, 8]}}, b"\0" * 12, "trailing bytes"),
+    ({"a": {"dtype": "F32", "shape": [2], "data_offsets": [4, 12]}}, b"\0" * 12, "gap"),
+    ({"a": {"dtype": "F32", "shape": [2], "data_offsets": [0, 8]}, "b": {"dtype": "F32", "shape": [2], "data_offsets": [4, 12]}},
+     b"\0" * 12, "overlaps"),
+    ({"a": {"dtype": "F32", "shape": [3], "data_offsets": [0, 8]}}, b"\0" * 8, "needs 12"),
+    ({"a": {"dtype": "F32", "shape": [2], "data_offsets": [0, 8]}}, b"\0" * 4, "past the end"),
+    ({"a": {"dtype": "F32", "shape": [2], "data_offsets": [8, 0]}}, b"\0" * 8, "start > end"),
+    ({"a": {"dtype": "Q4", "shape": [2], "data_offsets": [0, 8]}}, b"\0" * 8, "unsupported dtype"),
+    ({"a": {"dtype": "F32", "shape": [-2], "data_offsets": [0, 8]}}, b"\0" * 8, "invalid shape"),
+])
+def test_reader_refusals(tmp_path, header, data, text):
+    path = str(tmp_path / "x.safetensors")
+    _write_raw(path, header, data)
+    with pytest.raises(SafetensorsError, match=text):
+        SafetensorsFile(path)
+
+
+def test_reader_refuses_broken_headers(tmp_path):
+    path = str(tmp_path / "x.safetensors")
+    with open(path, "wb") as fh:
+        fh.write(b"\x01\x02")
+    with pytest.raises(SafetensorsError, match="truncated"):
+        SafetensorsFile(path)
+    with open(path, "wb") as fh:
+        fh.write(struct.pack("<Q", 1000) + b"{}")
+    with pytest.raises(SafetensorsError, match="past the end"):
+        SafetensorsFile(path)
+    with open(path, "wb") as fh:
+        fh.write(struct.pack("<Q", 2) + b"[]")
+    with pytest.raises(SafetensorsError, match="not a JSON object"):
+        SafetensorsFile(path)
+
+
+def test_sharded_checkpoint(tmp_path):
+    _, spec = model_spec_from_config(tc.TINY_A)
+    tensors = random_tensors(spec, 1, torch.float32)
+    names = sorted(tensors)
+    half = len(names) // 2
+    shards = {"model-00001-of-00002.safetensors": names[:half], "model-00002-of-00002.safetensors": names[half:]}
+    for shard, held in shards.items():
+        write_safetensors(str(tmp_path / shard), {n: tensors[n] for n in held})
+    with open(tmp_path / "model.safetensors.index.json", "w") as fh:
+        json.dump({"weight_map": {n: s for s, held in shards.items() for n in held}}, fh)
+    loaded = load_checkpoint(str(tmp_path), spec)
+    assert all(torch.equal(loaded[n], tensors[n]) for n in names)
+    with open(tmp_path / "model.safetensors.index.json", "w") as fh:
+        json.dump({"weight_map": {names[0]: "../evil.safetensors"}}, fh)
+    with pytest.raises(SafetensorsError, match="plain file name"):
+        open_checkpoint(str(tmp_path))
