@@ -1,0 +1,161 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on one MI355X, Llama-3.1-8B sizes, random bfloat16
+weights, synthetic token ids.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers N]
+
+A step is one decode step of the whole engine (scheduler, step function, sampling).  The one
+JSON line on standard output holds decoded tokens per second at the default batch (8), the same
+at batch 1 and 64 under "points", a 2,048-token prefill under "prefill" and the decode step's
+share of the HBM roofline under "roofline".
+"""
+import argparse
+import json
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0            # MI355X, published
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
+
+LLAMA_31_8B = {
+    "model_type": "llama", "architectures": ["LlamaForCausalLM"],
+    "num_hidden_layers": 32, "hidden_size": 4096, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+    "intermediate_size": 14336, "vocab_size": 128256, "rope_theta": 500000.0, "rms_norm_eps": 1e-5,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192},
+    "tie_word_embeddings": False, "max_position_embeddings": 131072, "hidden_act": "silu",
+}
+CONTEXT = 8192
+PROMPT_LEN = 1024
+PREFILL_TOKENS = 2048
+PAGE_SIZE = 16
+
+
+def linear_params(cfg, layers):
+    h, nh, nkv, d, i = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"],
+                        cfg["intermediate_size"])
+    per_layer = h * (nh + 2 * nkv) * d + nh * d * h + 3 * h * i
+    return per_layer * layers, cfg["vocab_size"] * h
+
+
+def decode_step_bytes(cfg, layers, contexts, elem=2):
+    """Bytes a decode step has to read: every weight it uses once, and the cache of the live requests."""
+    body, head = linear_params(cfg, layers)
+    norms = (2 * layers + 1) * cfg["hidden_size"] * 4
+    kv = sum(contexts) * layers * 2 * cfg["num_key_value_heads"] * cfg["head_dim"] * elem
+    return (body + head) * elem + norms + kv
+
+
+def prefill_flops(cfg, layers, tokens):
+    body, head = linear_params(cfg, layers)
+    attention = layers * 4 * cfg["num_attention_heads"] * cfg["head_dim"] * (tokens * (tokens + 1) // 2)
+    return 2 * tokens * body + 2 * head + attention          # the head runs on the one wanted row
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=LLAMA_31_8B["num_hidden_layers"],
+                    help="fewer layers than the model has (both numbers are reported)")
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this engine runs on a single MI355X, --gpus {args.gpus} is not supported")
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from fllm_amd import Engine, SamplingParams
+
+    cfg = dict(LLAMA_31_8B, num_hidden_layers=args.layers)
+    steps, warmup = args.steps, args.warmup
+    batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
+    slack = max(batches) + 8          # requests whose prompt is done early decode while the others still prefill
+    need_tokens = max(batches) * (PROMPT_LEN + warmup + steps + slack + PAGE_SIZE) + PREFILL_TOKENS + 64
+    t0 = time.time()
+    engine = Engine(config=cfg, seed=0, dtype="bfloat16", device="cuda:0", ctx=CONTEXT, max_seqs=max(batches),
+                    max_batched_tokens=PREFILL_TOKENS, block_size=PAGE_SIZE, num_blocks=-(-need_tokens // PAGE_SIZE),
+                    decode_first=True, random_weights_on_device=True)
+    print(f"[bench] engine ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
+    rng = np.random.default_rng(0)
+    vocab = cfg["vocab_size"]
+
+    def decode_run(batch):
+        params = SamplingParams(max_tokens=warmup + steps + slack, ignore_eos=True)
+        names = []
+        for i in range(batch):
+            name = f"b{batch}-{i}"
+            engine.add_request(name, rng.integers(0, vocab, PROMPT_LEN).tolist(), params)
+            names.append(name)
+        # prompts first (untimed): until every request has produced its first token
+        produced = {n: 0 for n in names}
+        while min(produced.values()) < 1:
+            for ev in engine.step():
+                produced[ev.request_id] += 1
+        for _ in range(warmup - 1 if warmup > 0 else 0):
+            engine.step()
+        torch.cuda.synchronize()
+        contexts = [engine.runner.cache.length(sid) for sid in engine.scheduler.running]
+        start = time.perf_counter()
+        tokens = 0
+        for _ in range(steps):
+            tokens += len(engine.step())
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - start
+        assert tokens == batch * steps, f"{tokens} tokens from {steps} steps of batch {batch}"
+        for n in names:
+            engine.abort_request(n)
+        mean_contexts = [c + steps / 2.0 for c in contexts]
+        return tokens / elapsed, elapsed / steps * 1e3, mean_contexts
+
+    results = {}
+    for batch in batches:
+        results[batch] = decode_run(batch)
+        print(f"[bench] decode batch {batch}: {results[batch][0]:.1f} tok/s, {results[batch][1]:.3f} ms/step",
+              file=sys.stderr, flush=True)
+
+    value, ms_per_step, contexts = results[args.batch]
+    step_bytes = decode_step_bytes(cfg, args.layers, contexts)
+    achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
+    line = {
+        "metric": "decode tok/s at batch 8 (Llama-3.1-8B shape, 1,024-token prompts); points: batch 1/64; prefill: 2,048 tokens",
+        "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic token ids, random-init weights N(0, 0.02)",
+        "config": {"model": "Llama-3.1-8B shape", "layers": args.layers, "layers_of_model": LLAMA_31_8B["num_hidden_layers"],
+                   "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
+                   "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": vocab,
+                   "global_batch": args.batch, "prompt_len": PROMPT_LEN, "seq_len": CONTEXT, "kv_block": PAGE_SIZE,
+                   "kv_dtype": "bf16", "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+    }
+    if not args.no_points:
+        line["points"] = {"decode_b1": round(results[1][0], 2), "decode_b64": round(results[64][0], 2)}
+        for b in (1, 64):
+            bytes_b = decode_step_bytes(cfg, args.layers, results[b][2])
+            line["points"][f"decode_b{b}_hbm_frac"] = round(bytes_b / (results[b][1] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        # prefill: one request, its 2,048 tokens in one step
+        times = []
+        for i in range(4):
+            engine.add_request(f"prefill-{i}", rng.integers(0, vocab, PREFILL_TOKENS).tolist(),
+                               SamplingParams(max_tokens=1, ignore_eos=True))
+            torch.cuda.synchronize()
+            start = time.perf_counter()
+            events = engine.step()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - start)
+            assert len(events) == 1 and events[0].finished
+        best = float(np.median(times[1:]))
+        flops = prefill_flops(cfg, args.layers, PREFILL_TOKENS)
+        line["prefill"] = {"value": round(PREFILL_TOKENS / best, 1), "tokens": PREFILL_TOKENS, "ms": round(best * 1e3, 3),
+                           "frac": round(flops / best / (MFMA_PEAK_TFLOPS["bf16"] * 1e12), 4)}
+        print(f"[bench] prefill {PREFILL_TOKENS} tokens: {best * 1e3:.2f} ms", file=sys.stderr, flush=True)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -49,9 +49,11 @@ class Engine:
                  max_batched_tokens: int = 512, block_size: int = 16, num_blocks: Optional[int] = None,
                  gpu_memory_utilization: float = 0.90, decode_first: bool = True, kv_watermark_blocks: int = 0,
                  max_num_partial_prefills: int = 0, long_prefill_token_threshold: int = 0,
-                 preemption_mode: str = "recompute", eos_token_ids: Optional[Seq[int]] = None, ops=None):
+                 preemption_mode: str = "recompute", eos_token_ids: Optional[Seq[int]] = None,
+                 random_weights_on_device: bool = False, ops=None):
         """`model`: a folder with config.json and safetensors; or `config` (a config.json dict)
-        with `seed` for random weights.  Option names follow the reference's server flags
+        with `seed` for random weights (drawn on the host, or on the device with a stream of its
+        own when `random_weights_on_device`: large models).  Option names follow the reference's server flags
         (rust/engine/src/bin/serve.rs:530-557, :681-782): ctx, max_seqs, max_batched_tokens,
         gpu_memory_utilization, kv_watermark_blocks, max_num_partial_prefills,
         long_prefill_token_threshold, preemption_mode."""
@@ -64,7 +66,7 @@ class Engine:
             tensors = load_checkpoint(model, spec)
         else:
             from .runner import parse_dtype
-            tensors = random_tensors(spec, seed, parse_dtype(dtype))
+            tensors = random_tensors(spec, seed, parse_dtype(dtype), device=device if random_weights_on_device else "cpu")
         self.runner = ModelRunner(spec, tensors, dtype=dtype, device=device, page_size=block_size, num_pages=num_blocks,
                                   max_requests=max_seqs, max_context=ctx, memory_utilization=gpu_memory_utilization,
                                   ops=ops, typed_config=typed)

@@ -39,6 +39,11 @@ def parse_dtype(name: Union[str, torch.dtype]) -> torch.dtype:
         raise ValueError(f"dtype must be float32 or bfloat16, not {name!r}") from None
 
 
+# Decode steps are padded to these row counts and replayed as HIP graphs (the reference's
+# buckets: rust/engine/src/rust_decoder.rs:1037).
+GRAPH_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64, 128, 256)
+
+
 class StepError(ValueError):
     """A batch the step function refuses before anything is launched."""
 
@@ -55,7 +60,7 @@ class ModelRunner:
     def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype="bfloat16", device="cuda:0",
                  page_size: int = 16, max_tokens: Optional[int] = None, num_pages: Optional[int] = None,
                  max_requests: int = 16, max_context: Optional[int] = None, memory_utilization: float = 0.90,
-                 ops=None, typed_config=None):
+                 ops=None, typed_config=None, use_graphs: bool = True):
         self.spec = spec
         self.config = typed_config
         self.device = torch.device(device)
@@ -83,6 +88,14 @@ class ModelRunner:
         self.cache: CacheManager = self.model.allocate_caches(page_size, [self.num_pages] * num_groups, max_requests)
         self.steps = 0
         self.rows_total = 0
+        # decode steps replay captured graphs when every part can be captured (parts say so with
+        # `graph_safe`; a part that decides on the host per step cannot)
+        parts_ok = all(getattr(b.mixer, "graph_safe", False) and getattr(b.feed_forward, "graph_safe", False)
+                       for b in self.model.blocks)
+        self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and parts_ok
+        self._graphs: Dict[tuple, "_DecodeGraph"] = {}
+        self._graph_pool = None
+        self.graph_replays = 0
 
     # ---- construction ---------------------------------------------------------------------
     @staticmethod
@@ -164,13 +177,66 @@ class ModelRunner:
             for r in added:
                 self.cache.free_request(r)
             raise
-        ctx = self._build_context(entries)
-        logits = self.model.forward(ctx)
+        logits = None
+        if self.use_graphs and all(len(e.tokens) == 1 for e in entries) and len(entries) <= GRAPH_BUCKETS[-1]:
+            logits = self._graph_step(entries)
+        if logits is None:
+            ctx = self._build_context(entries)
+            logits = self.model.forward(ctx)
         for e in entries:
             self.cache.commit(e.req_id, len(e.tokens))
         self.steps += 1
-        self.rows_total += ctx.num_rows
+        self.rows_total += sum(len(e.tokens) for e in entries)
         return logits
+
+    # ---- decode steps as HIP graphs ---------------------------------------------------------
+    def _graph_step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """A step of single-token entries, padded to a bucket and replayed as a graph.  The graph is
+        captured at the first use of a (rows, context bound) pair, after one eager run of the same
+        shape.  Padding rows belong to no segment (row_seg -1): they store nothing and their output
+        is dropped."""
+        import numpy as np
+        count = len(entries)
+        bucket = next(b for b in GRAPH_BUCKETS if b >= count)
+        starts = [self.cache.length(e.req_id) for e in entries]
+        bound = 256
+        while bound < max(starts) + 1:
+            bound *= 2
+        bound = min(bound, self.max_context)
+        widths = [-(-bound // g.page_size) for g in self.cache.groups]
+        key = (bucket, bound)
+        graph = self._graphs.get(key)
+        if graph is None:
+            graph = _DecodeGraph(self, bucket, bound, widths)
+            self._graphs[key] = graph
+        graph.done.synchronize()                  # the previous copy out of the pinned buffer has finished
+        h = graph.host_np
+        h[:] = graph.template
+        B = bucket
+        h[0:count] = [int(e.tokens[0]) for e in entries]
+        h[B:B + count] = starts
+        h[2 * B:2 * B + count] = np.arange(count)
+        h[4 * B + 1:4 * B + 1 + count] = [self.cache.slot(e.req_id) for e in entries]
+        o = 6 * B + 1
+        for g, width in enumerate(widths):
+            tables = h[o:o + B * width].reshape(B, width)
+            for i, e in enumerate(entries):
+                t = self.cache.table(e.req_id, g)
+                tables[i, :len(t)] = t
+            o += B * width
+        graph.device_buf.copy_(graph.host_buf, non_blocking=True)
+        graph.done.record()
+        if graph.graph is None:
+            graph.capture()
+        graph.graph.replay()
+        self.graph_replays += 1
+        wanted = [i for i, e in enumerate(entries) if len(e.want)]
+        if len(wanted) == bucket:
+            return graph.logits
+        if len(wanted) == count and count > 0 and wanted == list(range(count)):
+            return graph.logits[:count]
+        index = torch.tensor(wanted, dtype=torch.long, device=self.device)
+        return graph.logits.index_select(0, index)
 
     def _build_context(self, entries: Sequence[StepEntry]) -> StepContext:
         ids: List[int] = []
@@ -222,3 +288,50 @@ class ModelRunner:
                            slots=t_slots,
                            logit_rows=t_rows, tables=tables, seg_rows=seg_rows, seg_pos_start=seg_start,
                            seg_slots=slots, max_context=max_context, uniform_rows=all(n == 1 for n in seg_rows))
+
+
+class _DecodeGraph:
+    """Static buffers and the captured graph of decode steps of `bucket` rows whose contexts stay
+    within `bound` tokens.  Buffer layout (int32): ids[B], row_pos[B], row_seg[B], seg_start[B+1],
+    slots[B], logit_rows[B], then per cache group tables[B, width]."""
+
+    def __init__(self, runner: "ModelRunner", bucket: int, bound: int, widths):
+        import numpy as np
+        self.runner = runner
+        self.bucket = bucket
+        self.bound = bound
+        B = bucket
+        size = 6 * B + 1 + sum(B * w for w in widths)
+        self.host_buf = torch.zeros(size, dtype=torch.int32, pin_memory=True)
+        self.host_np = self.host_buf.numpy()
+        template = np.zeros(size, dtype=np.int32)
+        template[2 * B:3 * B] = -1                              # row_seg of padding rows
+        template[3 * B:4 * B + 1] = np.arange(B + 1)            # one row per segment
+        template[5 * B + 1:6 * B + 1] = np.arange(B)            # logits of every row
+        self.template = template
+        self.device_buf = torch.zeros(size, dtype=torch.int32, device=runner.device)
+        self.done = torch.cuda.Event()
+        self.done.record()
+        d = self.device_buf
+        o = 6 * B + 1
+        tables = []
+        for w in widths:
+            tables.append(d[o:o + B * w].view(B, w))
+            o += B * w
+        self.ctx = StepContext(num_rows=B, num_segments=B, ids=d[0:B], row_pos=d[B:2 * B], row_seg=d[2 * B:3 * B],
+                               seg_start=d[3 * B:4 * B + 1], slots=d[4 * B + 1:5 * B + 1],
+                               logit_rows=d[5 * B + 1:6 * B + 1], tables=tables, seg_rows=[1] * B,
+                               seg_pos_start=[0] * B, seg_slots=[0] * B, max_context=bound, uniform_rows=True)
+        self.graph = None
+        self.logits = None
+
+    def capture(self) -> None:
+        runner = self.runner
+        runner.model.forward(self.ctx)                  # eager once: every kernel of this shape has run before capture
+        torch.cuda.synchronize(runner.device)
+        if runner._graph_pool is None:
+            runner._graph_pool = torch.cuda.graph_pool_handle()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, pool=runner._graph_pool):
+            self.logits = runner.model.forward(self.ctx)
+        self.graph = graph

@@ -17,6 +17,8 @@ from .base import INIT_BIAS, INIT_MATRIX, KVNeed, Mixer
 
 
 class PagedAttention(Mixer):
+    graph_safe = True      # forward launches kernels only: no per-step decision on the host
+
     @classmethod
     def tensor_shapes(cls, spec):
         h, nh, nkv, d = spec["hidden_size"], spec["num_heads"], spec["num_kv_heads"], spec["head_dim"]

@@ -10,6 +10,8 @@ from .base import INIT_BIAS, INIT_MATRIX, FeedForward
 
 
 class GatedMLP(FeedForward):
+    graph_safe = True      # forward launches kernels only: no per-step decision on the host
+
     @classmethod
     def tensor_shapes(cls, spec):
         h, i = spec["hidden_size"], spec["intermediate_size"]

@@ -229,19 +229,16 @@ def philox_uniform(seed, draw, index):
     return np.float32((np.float32(w >> 8) + np.float32(0.5)) / np.float32(16777216.0))
 
 
-def device_sample(logits, temperature, top_k, top_p, seed, draw):
-    """The reference's device sampler (rust/engine/cuda/sampling.cu:253-352), with sorting in
-    place of its bisections: non-finite logits never win; temperature <= 1e-5 is greedy; top-k
-    keeps everything not below the k-th largest value (ties kept); top-p keeps the largest values
-    until their mass reaches top_p of the total (ties at the threshold kept); the token is the
-    argmax of (logit - max) / T - ln(-ln u_i), u_i = philox_uniform(seed, draw, i), lowest id on
-    ties."""
+def device_survivors(logits, temperature, top_k, top_p):
+    """The tokens the reference's device sampler still draws from, as a float32 array of logits
+    with -inf for the others (rust/engine/cuda/sampling.cu:253-330), with sorting in place of its
+    bisections: non-finite logits never survive; top-k keeps everything not below the k-th
+    largest value (ties kept); top-p keeps the largest values until their mass reaches top_p of the
+    total (ties at the threshold kept)."""
     w = np.asarray(logits, dtype=np.float32).copy()
     w[~np.isfinite(w)] = -np.inf
     if not np.isfinite(w).any():
-        return 0
-    if temperature <= 1e-5:
-        return greedy(np.where(np.isfinite(w), w, -np.inf))
+        return w
     m = w.max()
     inv_t = np.float32(1.0 / float(temperature))
     if 0 < top_k < len(w):
@@ -255,6 +252,22 @@ def device_sample(logits, temperature, top_k, top_p, seed, draw):
         mass = np.array([e[w >= v].sum() for v in values])      # mass of {value >= v}
         threshold = values[np.flatnonzero(mass >= target)[0]]   # largest threshold that still reaches the target
         w[w < threshold] = -np.inf
+    return w
+
+
+def device_sample(logits, temperature, top_k, top_p, seed, draw):
+    """rust/engine/cuda/sampling.cu:253-352: temperature <= 1e-5 is greedy; otherwise the token
+    is the argmax over the survivors of (logit - max) / T - ln(-ln u_i),
+    u_i = philox_uniform(seed, draw, i), lowest id on ties."""
+    raw = np.asarray(logits, dtype=np.float32)
+    finite = np.where(np.isfinite(raw), raw, -np.inf)
+    if not np.isfinite(finite).any():
+        return 0
+    if temperature <= 1e-5:
+        return greedy(finite)
+    w = device_survivors(logits, temperature, top_k, top_p)
+    m = finite.max()
+    inv_t = np.float32(1.0 / float(temperature))
     best, best_i = -np.inf, None
     for i in np.flatnonzero(np.isfinite(w)):
         u = philox_uniform(seed, draw, int(i))

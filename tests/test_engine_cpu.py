@@ -1,0 +1,154 @@
+"""The step function, the scheduler and generation on the CPU, with the plain kernels of
+tests/reference_ops.py in place of the HIP library: what is tested here is the engine's own
+logic (batches, pages, portions, preemption), not the kernels."""
+import numpy as np
+import pytest
+import torch
+
+import plain_llama
+import tiny_configs as tc
+import trace_tools as tt
+from reference_ops import ReferenceOps
+from fllm_amd import Engine, SamplingParams
+from fllm_amd.cache import OutOfPages
+from fllm_amd.engine import ModelRunner, StepEntry, StepError
+from fllm_amd.registry import model_spec_from_config
+from fllm_amd.weights import random_tensors
+
+
+def runner_for(name, max_tokens, **kw):
+    cfg = tc.CONFIGS[name]
+    _, spec = model_spec_from_config(cfg)
+    tensors = random_tensors(spec, 7, torch.float32, with_optional=(name == "C"))
+    r = ModelRunner(spec, tensors, dtype="float32", device="cpu", page_size=tc.PAGE_SIZES[name], max_tokens=max_tokens,
+                    max_requests=8, ops=ReferenceOps(), **kw)
+    return cfg, tc.to_float64(tensors), r
+
+
+@pytest.mark.parametrize("name,lengths", [("A", [5, 17, 40]), ("C", [30, 70])])
+@pytest.mark.parametrize("family", ["whole", "last32", "portions", "mixed"])
+def test_every_way_of_cutting_gives_the_plain_logits(tmp_path, name, lengths, family):
+    requests = {f"r{i}": tc.random_ids(n, tc.CONFIGS[name]["vocab_size"], 50 + i) for i, n in enumerate(lengths)}
+    steps = {"whole": tt.whole, "last32": lambda r: tt.last_tokens_one_by_one(r, 8), "portions": tt.portions,
+             "mixed": lambda r: tt.mixed(r, seed=2, decode_tail=5)}[family](requests)
+    steps = tt.number(steps)
+    cfg, w64, runner = runner_for(name, tt.live_tokens_bound(steps, round_to=16))
+    got = tt.run_in_process(runner, steps, cfg["vocab_size"], str(tmp_path))
+    for rid, toks in requests.items():
+        want = plain_llama.forward(cfg, w64, toks)
+        assert np.abs(got[rid] - want).max() <= 2e-5 * np.abs(want).max(), (family, rid)
+    runner.cache.check_invariants()
+    assert all(p.available == p.num_pages for p in runner.cache.pools)
+
+
+def test_step_refuses_bad_batches():
+    cfg, _, r = runner_for("A", 64)
+    with pytest.raises(StepError, match="at least one entry"):
+        r.step([])
+    with pytest.raises(StepError, match="no tokens"):
+        r.step([StepEntry("a", [], [])])
+    with pytest.raises(StepError, match="outside"):
+        r.step([StepEntry("a", [256], [0])])
+    with pytest.raises(StepError, match="wants logits"):
+        r.step([StepEntry("a", [1, 2], [2])])
+    with pytest.raises(StepError, match="twice"):
+        r.step([StepEntry("a", [1], [0]), StepEntry("a", [2], [0])])
+    with pytest.raises(StepError, match="context"):
+        r.step([StepEntry("a", [1] * 129, [])])
+    assert not r.cache.has_request("a")
+    with pytest.raises(OutOfPages):
+        r.step([StepEntry("a", [1] * 40, []), StepEntry("b", [1] * 40, [])])     # 64 tokens of cache
+    assert not r.cache.has_request("a") and not r.cache.has_request("b")          # nothing changed
+    r.cache.check_invariants()
+    out = r.step([StepEntry("a", [1, 2, 3], [])])
+    assert out.shape == (0, 256) and r.length("a") == 3
+
+
+def make_engine(name="A", **kw):
+    opts = dict(dtype="float32", device="cpu", ctx=tc.CONFIGS[name]["max_position_embeddings"], max_seqs=4,
+                max_batched_tokens=16, block_size=tc.PAGE_SIZES[name], num_blocks=64, ops=ReferenceOps())
+    opts.update(kw)
+    return Engine(config=tc.CONFIGS[name], seed=1, **opts)
+
+
+def plain_greedy(name, prompt, count):
+    cfg = tc.CONFIGS[name]
+    _, spec = model_spec_from_config(cfg)
+    w64 = tc.to_float64(random_tensors(spec, 1, torch.float32))
+    seq = list(prompt)
+    for _ in range(count):
+        seq.append(plain_llama.greedy(plain_llama.forward(cfg, w64, seq)[-1]))
+    return seq[len(prompt):]
+
+
+PROMPTS_A = [tc.random_ids(n, 256, 10 + n) for n in (5, 17, 31)]
+
+
+def test_greedy_generation_matches_the_plain_implementation():
+    """The workload of the first tiny configuration: prompts of 5/17/31 tokens, 16 greedy tokens each."""
+    outs = make_engine().generate(PROMPTS_A, SamplingParams(max_tokens=16))
+    assert outs == [plain_greedy("A", p, 16) for p in PROMPTS_A]
+
+
+def test_few_pages_preempt_and_give_the_same_tokens():
+    roomy = make_engine().generate(PROMPTS_A, SamplingParams(max_tokens=16))
+    tight = make_engine(num_blocks=5)
+    assert tight.generate(PROMPTS_A, SamplingParams(max_tokens=16)) == roomy
+    assert tight.stats.preemptions >= 1
+    tight.runner.cache.check_invariants()
+
+
+def test_no_progress_is_an_error():
+    engine = make_engine(num_blocks=2, max_seqs=1)          # 32 tokens of cache
+    engine.add_request("a", tc.random_ids(30, 256, 1), SamplingParams(max_tokens=8))
+    with pytest.raises(RuntimeError, match="could not make progress"):
+        for _ in range(20):
+            engine.step()
+
+
+def test_seeded_sampling_is_reproducible_and_ignores_the_neighbours():
+    """The second tiny configuration's workload in small: chunked prefill mixed with decode,
+    temperature 0.8 from a fixed seed."""
+    params = SamplingParams(max_tokens=6, temperature=0.8, top_p=0.95, seed=1234)
+    prompts = [tc.random_ids(n, 512, 20 + n) for n in (1, 9, 40)]
+    alone = [make_engine("B", max_batched_tokens=32).generate([p], params)[0] for p in prompts]
+    together = make_engine("B", max_batched_tokens=32).generate(prompts, params)
+    assert together == alone
+    assert make_engine("B", max_batched_tokens=32).generate(prompts, params) == together
+    other = make_engine("B", max_batched_tokens=32).generate(prompts, SamplingParams(max_tokens=6, temperature=0.8, seed=99))
+    assert other != together
+
+
+def test_finish_reasons_and_request_checks():
+    engine = make_engine()
+    first = plain_greedy("A", PROMPTS_A[0], 3)
+    engine.add_request("stop", PROMPTS_A[0], SamplingParams(max_tokens=16, stop_token_ids=(first[2],)))
+    engine.add_request("length", PROMPTS_A[0], SamplingParams(max_tokens=2))
+    events = []
+    while engine.has_unfinished():
+        events += engine.step()
+    done = {e.request_id: e for e in events if e.finished}
+    assert done["stop"].finish_reason == "stop" and done["stop"].token_id == first[2]
+    assert done["length"].finish_reason == "length"
+    assert [e.token_id for e in events if e.request_id == "stop"] == first
+    with pytest.raises(ValueError, match="non-empty"):
+        engine.add_request("x", [], SamplingParams())
+    with pytest.raises(ValueError, match="exceeds the configured model context"):
+        engine.add_request("x", [1] * 120, SamplingParams(max_tokens=16))
+    engine.add_request("dup", [1, 2], SamplingParams(max_tokens=4))
+    with pytest.raises(ValueError, match="already active"):
+        engine.add_request("dup", [1, 2], SamplingParams(max_tokens=4))
+    engine.abort_request("dup")
+    assert not engine.has_unfinished()
+    engine.runner.cache.check_invariants()
+
+
+def test_eos_from_config_stops_unless_ignored():
+    cfg = dict(tc.TINY_A)
+    first = plain_greedy("A", PROMPTS_A[1], 2)
+    cfg["eos_token_id"] = first[1]
+    base = dict(dtype="float32", device="cpu", ctx=128, max_seqs=2, max_batched_tokens=32, block_size=16, num_blocks=16,
+                ops=ReferenceOps())
+    assert Engine(config=cfg, seed=1, **base).generate([PROMPTS_A[1]], SamplingParams(max_tokens=8)) == [first]
+    ignored = Engine(config=cfg, seed=1, **base).generate([PROMPTS_A[1]], SamplingParams(max_tokens=8, ignore_eos=True))
+    assert len(ignored[0]) == 8 and ignored[0][:2] == first

@@ -1,0 +1,110 @@
+"""Greedy and sampled generation through the entry points (Engine.generate, the command line)
+on the GPU, against the plain implementation."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama
+import tiny_configs as tc
+from fllm_amd import Engine, SamplingParams
+from fllm_amd.registry import model_spec_from_config
+from fllm_amd.weights import random_tensors, write_random_model
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PROMPT_LENGTHS = {"A": (5, 17, 31), "B": (1, 9, 40, 100)}
+
+
+def make_engine(name, dtype, **kw):
+    opts = dict(dtype=dtype, ctx=tc.CONFIGS[name]["max_position_embeddings"], max_seqs=4, max_batched_tokens=32,
+                block_size=tc.PAGE_SIZES[name], num_blocks=128)
+    opts.update(kw)
+    return Engine(config=tc.CONFIGS[name], seed=1, **opts)
+
+
+def check_greedy(name, dtype, prompts, outputs):
+    """Every generated token is the plain implementation's choice given the tokens before it, or,
+    where two logits nearly tie, one of the two."""
+    cfg = tc.CONFIGS[name]
+    _, spec = model_spec_from_config(cfg)
+    w64 = tc.to_float64(random_tensors(spec, 1, torch.float32))
+    tol = 2e-5 if dtype == "float32" else 4e-2
+    for prompt, out in zip(prompts, outputs):
+        seq = list(prompt)
+        logits = plain_llama.forward(cfg, w64, seq + list(out))
+        for i, token in enumerate(out):
+            row = logits[len(prompt) - 1 + i]
+            best = plain_llama.greedy(row)
+            assert token == best or row[best] - row[token] <= 2 * tol * np.abs(row).max(), \
+                f"{name} {dtype}: token {i} is {token}, the plain implementation takes {best}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation(name, dtype):
+    prompts = [tc.random_ids(n, tc.CONFIGS[name]["vocab_size"], 10 + n) for n in PROMPT_LENGTHS[name]]
+    count = 16 if name == "A" else 24
+    engine = make_engine(name, dtype)
+    outputs = engine.generate(prompts, SamplingParams(max_tokens=count))
+    assert all(len(o) == count for o in outputs)
+    check_greedy(name, dtype, prompts, outputs)
+    assert engine.runner.graph_replays > 0
+    engine.runner.cache.check_invariants()
+
+
+def test_alone_batched_and_preempted_give_the_same_tokens():
+    prompts = [tc.random_ids(n, 256, 10 + n) for n in PROMPT_LENGTHS["A"]]
+    params = SamplingParams(max_tokens=16)
+    together = make_engine("A", "float32").generate(prompts, params)
+    alone = [make_engine("A", "float32").generate([p], params)[0] for p in prompts]
+    assert together == alone
+    tight = make_engine("A", "float32", num_blocks=5)
+    assert tight.generate(prompts, params) == together and tight.stats.preemptions >= 1
+    eager = make_engine("A", "float32")
+    eager.runner.use_graphs = False
+    assert eager.generate(prompts, params) == together
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sampled_generation_is_reproducible(dtype):
+    """Config B's workload: chunked prefill (portions of 32) mixed with decode, 24 tokens at
+    temperature 0.8 from a fixed seed."""
+    prompts = [tc.random_ids(n, 512, 20 + n) for n in PROMPT_LENGTHS["B"]]
+    params = SamplingParams(max_tokens=24, temperature=0.8, seed=4242)
+    a = make_engine("B", dtype).generate(prompts, params)
+    b = make_engine("B", dtype).generate(prompts, params)
+    assert a == b and all(len(o) == 24 for o in a)
+    if dtype == "float32":
+        alone = [make_engine("B", dtype).generate([p], params)[0] for p in prompts]
+        assert alone == a                                    # the neighbours in the batch do not matter
+        # every token is what the plain sampler draws from the plain logits (near-ties aside)
+        cfg = tc.TINY_B
+        _, spec = model_spec_from_config(cfg)
+        w64 = tc.to_float64(random_tensors(spec, 1, torch.float32))
+        seq = list(prompts[1])
+        agree = 0
+        for draw, token in enumerate(a[1]):
+            logits = plain_llama.forward(cfg, w64, seq)[-1]
+            agree += token == plain_llama.device_sample(logits, 0.8, 0, 1.0, 4242, draw)
+            seq.append(token)
+        assert agree >= 23
+    assert make_engine("B", dtype).generate(prompts, SamplingParams(max_tokens=24, temperature=0.8, seed=1)) != a
+
+
+def test_command_line(tmp_path):
+    folder = str(tmp_path / "model")
+    write_random_model(folder, tc.TINY_A, seed=1, dtype="float32")
+    prompt = tc.random_ids(9, 256, 3)
+    cmd = [sys.executable, "-m", "fllm_amd", "run", folder, "--prompt-ids", ",".join(map(str, prompt)), "--max-tokens", "8",
+           "--dtype", "float32", "--kv-blocks", "16", "--max-seqs", "2"]
+    proc = subprocess.run(cmd, cwd=ROOT, capture_output=True, text=True, timeout=110)
+    assert proc.returncode == 0, proc.stderr
+    record = json.loads(proc.stdout.strip().splitlines()[0])
+    assert record["finish_reason"] == "length" and len(record["token_ids"]) == 8
+    check_greedy("A", "float32", [prompt], [record["token_ids"]])
+    assert "forward_calls=" in proc.stderr

@@ -1,0 +1,247 @@
+"""Pins the plain implementation by what fixes it beside the reference's text: vectors the
+reference's own tests hold, special cases that reduce to a library routine, and invariants, each
+chosen so that a plausible mistake (a wrong sign or pairing, a norm in the wrong place, a head
+mapped to the wrong group) fails it."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_llama as P
+import tiny_configs as tc
+from fllm_amd.registry import model_spec_from_config
+from fllm_amd.weights import random_tensors
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+# ---- RMSNorm ---------------------------------------------------------------------------------
+def test_rms_norm_reduces_to_unit_rms_and_matches_the_library():
+    x = rng(1).normal(size=(5, 48)) * 3
+    w = 1 + 0.1 * rng(2).normal(size=48)
+    y = P.rms_norm(x, w, 1e-12)
+    assert np.allclose(y / w, x / np.linalg.norm(x, axis=-1, keepdims=True) * math.sqrt(48), rtol=1e-9)
+    lib = F.rms_norm(torch.tensor(x), (48,), torch.tensor(w), eps=1e-5).numpy()
+    assert np.allclose(P.rms_norm(x, w, 1e-5), lib, rtol=1e-12)
+    assert np.allclose(P.rms_norm(7.0 * x, w, 1e-12), y, rtol=1e-9)              # scale invariance
+    assert not np.allclose(P.rms_norm(x, w, 1e-5), (x - x.mean(-1, keepdims=True)) / x.std(-1, keepdims=True) * w)
+
+
+def test_rms_norm_eps_is_inside_the_root():
+    x = np.full((1, 4), 1e-3)
+    assert np.allclose(P.rms_norm(x, np.ones(4), 1e-2), x / math.sqrt(1e-6 + 1e-2))
+
+
+# ---- rotary ----------------------------------------------------------------------------------
+def test_rope_tables_reference_vectors():
+    """rust/engine/src/rope.rs:134-142: position 0 is the identity, lane 1 of 8 dims at base
+    10000 turns at frequency 0.1."""
+    cos, sin = P.rope_tables([0, 1, 2], 8, 10000.0)
+    assert cos.shape == (3, 4) and np.all(cos[0] == 1.0) and np.all(sin[0] == 0.0)
+    assert abs(sin[1, 0] - math.sin(1.0)) < 1e-7 and abs(sin[1, 1] - math.sin(0.1)) < 1e-7
+
+
+def test_linear_scaling_divides_the_position():
+    """rust/engine/src/rope.rs:144-151."""
+    plain = P.rope_tables(range(9), 8, 10000.0)[1]
+    linear = P.rope_tables(range(9), 8, 10000.0, "linear", {"factor": 4.0})[1]
+    assert np.allclose(linear[8], plain[2], atol=1e-6)
+
+
+def test_llama3_divisors_reference_vector():
+    """rust/checkpoint/src/plan.rs:3219-3232: head_dim 16, theta 5e5, factor 8, low 1, high 4,
+    original 8192: 8 divisors, the first 1.0, the last 8.0."""
+    d = P.llama3_divisors(16, 500000.0, 8.0, 1.0, 4.0, 8192.0)
+    assert len(d) == 8 and d[0] == 1.0 and d[7] == 8.0
+    assert np.all(np.diff(d) >= 0) and np.all((d >= 1.0) & (d <= 8.0))
+    assert 1.0 < d[4] < 8.0                                      # a lane in the smooth band
+    assert np.all(P.llama3_divisors(16, 500000.0, 8.0, 1.0, 4.0, 1e12) == 1.0)    # huge original context: plain rotary
+
+
+def test_rotation_keeps_norms_and_depends_on_distance_only():
+    q = rng(3).normal(size=(1, 2, 16))
+    k = rng(4).normal(size=(1, 2, 16))
+
+    def dot(pq, pk, **kw):
+        cq, sq = P.rope_tables([pq], 16, 10000.0)
+        ck, sk = P.rope_tables([pk], 16, 10000.0)
+        return (P.apply_rope(q, cq, sq, 16, **kw) * P.apply_rope(k, ck, sk, 16, **kw)).sum(-1)
+
+    c, s = P.rope_tables([5], 16, 10000.0)
+    assert np.allclose(np.linalg.norm(P.apply_rope(q, c, s, 16), axis=-1), np.linalg.norm(q, axis=-1))
+    assert np.allclose(dot(3, 1), dot(12, 10), atol=1e-5) and np.allclose(dot(0, 0), (q * k).sum(-1))
+    assert not np.allclose(dot(3, 1), dot(1, 3), atol=1e-3)      # the sign of the rotation matters
+    # a query ahead of its key by t turns lane 0 by +t radians: <R(t)q, R(0)k> = cos t for q = k = e_0
+    e = np.zeros((1, 1, 16))
+    e[0, 0, 0] = 1.0
+    c2, s2 = P.rope_tables([2], 16, 10000.0)
+    r = P.apply_rope(e, c2, s2, 16)
+    assert abs(r[0, 0, 0] - math.cos(2.0)) < 1e-6 and abs(r[0, 0, 8] - math.sin(2.0)) < 1e-6   # pairs (l, l + 8)
+
+
+def test_half_pairing_equals_the_reference_interleaved_pairing_on_permuted_rows():
+    """rust/checkpoint/src/convert.rs:2713-2745: the importer moves row src < half to 2*src and
+    row src >= half to 2*(src - half) + 1, then rotates pairs (2l, 2l+1)."""
+    d = 16
+    x = rng(5).normal(size=(3, 2, d))
+    cos, sin = P.rope_tables([0, 7, 31], d, 10000.0)
+    dest = np.array([2 * s if s < d // 2 else 2 * (s - d // 2) + 1 for s in range(d)])
+    permuted = np.empty_like(x)
+    permuted[:, :, dest] = x
+    a = P.apply_rope(x, cos, sin, d)
+    b = P.apply_rope(permuted, cos, sin, d, interleaved=True)
+    assert np.allclose(a, b[:, :, dest])
+
+
+def test_partial_rotary_leaves_the_rest_alone():
+    x = rng(6).normal(size=(2, 1, 16))
+    cos, sin = P.rope_tables([3, 4], 8, 10000.0)
+    y = P.apply_rope(x, cos, sin, 8)
+    assert np.array_equal(y[:, :, 8:], x[:, :, 8:]) and not np.allclose(y[:, :, :8], x[:, :, :8])
+
+
+# ---- attention -------------------------------------------------------------------------------
+def test_attention_reduces_to_the_library_routine():
+    T, heads, kv_heads, d = 9, 6, 2, 8
+    q, k, v = (rng(s).normal(size=(T, h, d)) for s, h in ((7, heads), (8, kv_heads), (9, kv_heads)))
+    got = P.attention(q, k, v, 1 / math.sqrt(d))
+    tq, tk, tv = (torch.tensor(a).transpose(0, 1) for a in (q, k, v))
+    lib = F.scaled_dot_product_attention(tq, tk.repeat_interleave(3, 0), tv.repeat_interleave(3, 0), is_causal=True)
+    assert np.allclose(got, lib.transpose(0, 1).numpy(), atol=1e-12)
+    wrong_groups = F.scaled_dot_product_attention(tq, tk.repeat(3, 1, 1), tv.repeat(3, 1, 1), is_causal=True)
+    assert not np.allclose(got, wrong_groups.transpose(0, 1).numpy(), atol=1e-3)       # h -> h // group, not h % kv_heads
+
+
+def test_attention_special_cases():
+    d = 8
+    v = rng(10).normal(size=(5, 1, d))
+    q = rng(11).normal(size=(5, 2, d))
+    one = P.attention(q[:1], np.zeros((1, 1, d)), v[:1], 1.0)
+    assert np.allclose(one[0, 0], v[0, 0])                                             # a single token returns its value
+    flat = P.attention(q, np.zeros((5, 1, d)), v, 1.0)
+    assert np.allclose(flat[4, 1], v[:, 0].mean(0)) and np.allclose(flat[2, 0], v[:3, 0].mean(0))   # equal scores: the mean
+
+
+def test_attention_window_counts_the_token_itself():
+    T, d, w = 12, 8, 4
+    q, k, v = (rng(s).normal(size=(T, 1, d)) for s in (12, 13, 14))
+    got = P.attention(q, k, v, 0.5, window=w)
+    mask = torch.tensor([[0 <= r - c < w for c in range(T)] for r in range(T)])
+    lib = F.scaled_dot_product_attention(*(torch.tensor(a).transpose(0, 1) for a in (q, k, v)), attn_mask=mask, scale=0.5)
+    assert np.allclose(got, lib.transpose(0, 1).numpy(), atol=1e-12)
+    assert np.allclose(P.attention(q, k, v, 0.5, window=T), P.attention(q, k, v, 0.5))
+
+
+# ---- feed-forward ----------------------------------------------------------------------------
+def test_silu_and_gated_mlp():
+    x = np.array([0.0, 40.0, -40.0, 1.5])
+    assert P.silu(x)[0] == 0.0 and abs(P.silu(x)[1] - 40.0) < 1e-12 and abs(P.silu(x)[2]) < 1e-12
+    assert np.allclose(P.silu(x), F.silu(torch.tensor(x)).numpy())
+    h, i = 6, 10
+    xs, g, u, dn = rng(15).normal(size=(3, h)), rng(16).normal(size=(i, h)), rng(17).normal(size=(i, h)), rng(18).normal(size=(h, i))
+    want = (F.silu(torch.tensor(xs @ g.T)) * torch.tensor(xs @ u.T)).numpy() @ dn.T
+    assert np.allclose(P.gated_mlp(xs, g, u, dn), want)
+    assert not np.allclose(P.gated_mlp(xs, u, g, dn), want)                            # the activation sits on the gate
+
+
+# ---- whole model -----------------------------------------------------------------------------
+@pytest.fixture(scope="module")
+def weights():
+    out = {}
+    for name, cfg in tc.CONFIGS.items():
+        _, spec = model_spec_from_config(cfg)
+        out[name] = tc.to_float64(random_tensors(spec, 21, torch.float32, with_optional=(name == "C")))
+    return out
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_a_shift_of_all_positions_changes_nothing(weights, name):
+    """Rotary attention sees distances only (also with per-lane or linear scaling)."""
+    cfg = tc.CONFIGS[name]
+    ids = tc.random_ids(20, cfg["vocab_size"], 1)
+    a = P.forward(cfg, weights[name], ids)
+    b = P.forward(cfg, weights[name], ids, first_position=37)
+    assert np.allclose(a, b, atol=2e-4 * np.abs(a).max())     # float32 phases: the tables differ in the last bits
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_causality_and_the_head(weights, name):
+    cfg = tc.CONFIGS[name]
+    ids = tc.random_ids(24, cfg["vocab_size"], 2)
+    full = P.forward(cfg, weights[name], ids)
+    assert full.shape == (24, cfg["vocab_size"])
+    assert np.allclose(P.forward(cfg, weights[name], ids[:10]), full[:10], atol=1e-12)       # later tokens change nothing
+    other = list(ids)
+    other[3] = (other[3] + 1) % cfg["vocab_size"]
+    changed = P.forward(cfg, weights[name], other)
+    assert np.allclose(changed[:3], full[:3], atol=1e-12) and not np.allclose(changed[3:], full[3:], atol=1e-6)
+
+
+def test_tied_head_is_the_embedding_table(weights):
+    cfg = tc.TINY_B
+    w = dict(weights["B"])
+    ids = tc.random_ids(6, 512, 3)
+    a = P.forward(cfg, w, ids)
+    w["lm_head.weight"] = rng(19).normal(size=(512, 160))       # ignored when tied
+    assert np.array_equal(P.forward(cfg, w, ids), a)
+    untied = dict(cfg, tie_word_embeddings=False)
+    assert not np.allclose(P.forward(untied, w, ids), a)
+
+
+def test_window_config_changes_only_what_lies_beyond_the_window(weights):
+    cfg = tc.TINY_C
+    ids = tc.random_ids(60, 300, 4)
+    with_window = P.forward(cfg, weights["C"], ids)
+    without = P.forward(dict(cfg, sliding_window=None), weights["C"], ids)
+    assert np.allclose(with_window[:24], without[:24], atol=1e-12)      # the first 24 positions see everything either way
+    assert not np.allclose(with_window[30:], without[30:], atol=1e-6)
+
+
+# ---- sampling --------------------------------------------------------------------------------
+def test_philox_known_answers():
+    """rust/engine/src/sampling.rs:1018-1030 (Random123's vectors for philox4x32, 10 rounds)."""
+    assert P.philox4x32_10([0, 0, 0, 0], [0, 0]) == [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]
+    assert P.philox4x32_10([0xFFFFFFFF] * 4, [0xFFFFFFFF] * 2) == [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]
+    pi_digits = P.philox4x32_10([0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0])
+    assert pi_digits == [0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]
+
+
+def test_philox_uniforms():
+    """rust/engine/src/sampling.rs:1032-1046."""
+    us = np.array([P.philox_uniform(42, i, 0) for i in range(4000)])
+    assert us.min() > 0.0 and us.max() < 1.0
+    assert np.all(np.abs(np.histogram(us, bins=8, range=(0, 1))[0] - 500) < 100)
+    assert P.philox_uniform(1, 0, 0) != P.philox_uniform(2, 0, 0) and P.philox_uniform(1, 0, 0) != P.philox_uniform(1, 0, 1)
+    assert P.philox_uniform(7, 3, 9) == P.philox_uniform(7, 3, 9)
+
+
+def test_greedy_takes_the_first_maximum():
+    """rust/engine/src/sampling.rs:763-766."""
+    assert P.greedy([0.1, 0.9, 0.9, -1.0]) == 1
+    assert P.device_sample([0.1, 0.9, 0.9, float("nan")], 0.0, 0, 1.0, 1, 0) == 1
+
+
+def test_filters():
+    """The reference's vectors (rust/engine/src/sampling.rs:1061-1075): logits [3, 2, 1, 0, -1] at
+    temperature 1: top_k 3 keeps ids 0, 1, 2; top_p 0.7 keeps two tokens."""
+    logits = [3.0, 2.0, 1.0, 0.0, -1.0]
+    alive = lambda **kw: np.flatnonzero(np.isfinite(P.device_survivors(logits, 1.0, kw.get("top_k", 0), kw.get("top_p", 1.0)))).tolist()
+    assert alive(top_k=3) == [0, 1, 2] and alive(top_p=0.7) == [0, 1] and alive() == [0, 1, 2, 3, 4]
+    assert alive(top_k=3, top_p=0.7) == [0, 1]
+    assert np.flatnonzero(np.isfinite(P.device_survivors([1.0, 5.0, 5.0, 0.0], 1.0, 1, 1.0))).tolist() == [1, 2]   # ties are kept
+    # a dominant token always survives top-p (sampling.rs:809-823)
+    assert np.flatnonzero(np.isfinite(P.device_survivors([0.0, 20.0, 1.0], 1.0, 0, 0.1))).tolist() == [1]
+
+
+def test_draws_follow_the_distribution_and_depend_on_seed_and_draw_only():
+    logits = np.array([2.0, 1.0, 0.0, -1.0], dtype=np.float32)
+    p = np.exp(logits / 0.8)
+    p /= p.sum()
+    counts = np.bincount([P.device_sample(logits, 0.8, 0, 1.0, 5, d) for d in range(3000)], minlength=4) / 3000
+    assert np.all(np.abs(counts - p) < 0.03)
+    assert P.device_sample(logits, 0.8, 0, 1.0, 5, 17) == P.device_sample(logits, 0.8, 0, 1.0, 5, 17)
+    assert len({P.device_sample(logits, 1.5, 0, 1.0, s, 0) for s in range(40)}) > 1

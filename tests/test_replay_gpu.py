@@ -55,9 +55,10 @@ def check(got, plain, dtype, what):
                                                  f"{int(np.argmax(err.max(axis=1) > TOL[dtype] * scale))}")
 
 
-def make_runner(folder, dtype, page_size, max_tokens):
+def make_runner(folder, dtype, page_size, max_tokens, use_graphs=True):
     from fllm_amd.engine import ModelRunner
-    return ModelRunner.from_folder(folder, dtype=dtype, page_size=page_size, max_tokens=max_tokens, max_requests=8)
+    return ModelRunner.from_folder(folder, dtype=dtype, page_size=page_size, max_tokens=max_tokens, max_requests=8,
+                                   use_graphs=use_graphs)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -113,3 +114,23 @@ def test_first_tokens_and_long_decoding(models, tmp_path, dtype):
     runner = make_runner(folder, dtype, 8, 256)
     got = tt.run_in_process(runner, steps, cfg["vocab_size"], str(tmp_path))
     check(got, {rid: plain[rid]}, dtype, f"token by token {dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_decode_graphs_and_eager_steps_agree(models, tmp_path, name, dtype):
+    """Decode steps replay captured HIP graphs; every replay (with eager steps and synchronisations
+    between them) gives what the eager step gives."""
+    folder, cfg, requests, plain = models[name]
+    steps = tt.number(tt.last_tokens_one_by_one(requests) + tt.mixed(requests, seed=21, decode_tail=40))
+    results = []
+    for i, use_graphs in enumerate((True, False)):
+        runner = make_runner(folder, dtype, tc.PAGE_SIZES[name], tt.live_tokens_bound(steps), use_graphs=use_graphs)
+        results.append(tt.run_in_process(runner, steps, cfg["vocab_size"], str(tmp_path / str(i))))
+        assert (runner.graph_replays > 30) == use_graphs
+    for rid, want in plain.items():
+        a, b = results[0][rid].astype(np.float64), results[1][rid].astype(np.float64)
+        if dtype == "float32":
+            assert np.array_equal(a, b), f"{rid}: graph and eager steps differ in float32"
+        else:
+            assert np.abs(a - b).max() <= TOL[dtype] * np.abs(want).max()

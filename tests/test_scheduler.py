@@ -1,0 +1,151 @@
+"""The scheduler's decisions: admission, portions under the token budget, decode rows, what
+happens when pages run out."""
+import pytest
+
+from fllm_amd.cache import CacheManager, GroupSpec
+from fllm_amd.engine.scheduler import Scheduler, SchedulerConfig, Sequence
+from fllm_amd.sampling import SamplingParams
+
+
+def make(pages, max_seqs=4, budget=8, page_size=4, **kw):
+    cache = CacheManager([GroupSpec(entries=(0,), kv_heads=1, head_dim=16, window=None, page_size=page_size)], [pages],
+                         max_requests=max_seqs)
+    return Scheduler(SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=budget, **kw), cache, max_model_len=64), cache
+
+
+def seq(sid, prompt_len, max_tokens=4):
+    return Sequence(seq_id=sid, req_id=f"r{sid}", tokens=list(range(prompt_len)), prompt_len=prompt_len,
+                    sampling=SamplingParams(max_tokens=max_tokens))
+
+
+def run_step(s, cache, plan, new_token=1):
+    """What the engine does after the forward pass."""
+    for sid, start, count in plan.prefill:
+        cache.commit(sid, count)
+        s.commit_chunk(sid, count)
+        q = s.sequences[sid]
+        if q.num_computed == q.prefill_target:
+            q.tokens.append(new_token)
+            s.commit_decode(sid)
+    for sid in plan.decode:
+        cache.commit(sid, 1)
+        s.sequences[sid].tokens.append(new_token)
+        s.commit_decode(sid)
+
+
+def test_prompt_is_cut_under_the_budget():
+    s, cache = make(pages=16, budget=8)
+    s.add(seq(0, 19))
+    plans = []
+    for _ in range(3):
+        plan = s.schedule()
+        plans.append(plan.prefill)
+        run_step(s, cache, plan)
+    assert plans == [[(0, 0, 8)], [(0, 8, 8)], [(0, 16, 3)]]
+    plan = s.schedule()
+    assert plan.prefill == [] and plan.decode == [0]
+
+
+def test_decode_first_keeps_a_token_per_decoder():
+    """rust/engine/src/scheduler.rs:1381-1397: budget 8 and two decoders leave 6 for the prompt."""
+    for decode_first, expect in ((True, 6), (False, 8)):
+        s, cache = make(pages=32, budget=8, decode_first=decode_first)
+        s.add(seq(0, 3))
+        s.add(seq(1, 3))
+        run_step(s, cache, s.schedule())
+        s.add(seq(2, 20))
+        plan = s.schedule()
+        assert plan.prefill == [(2, 0, expect)]
+        assert plan.decode == ([0, 1] if decode_first else [])       # without it the prompt eats the budget
+
+
+def test_admission_reserves_prompt_plus_one_and_is_first_come_first_served():
+    s, cache = make(pages=4, budget=64)                 # 16 tokens of cache
+    s.add(seq(0, 12))                                   # needs 13 tokens: 4 pages
+    s.add(seq(1, 2))                                    # would fit, but waits behind nobody: the pool is full
+    plan = s.schedule()
+    assert [p[0] for p in plan.prefill] == [0] and list(s.waiting) == [1]
+    assert cache.free_pages() == 0
+    s2, cache2 = make(pages=4, budget=64)
+    s2.add(seq(0, 40))                                  # never fits: blocks the queue (head of line)
+    s2.add(seq(1, 2))
+    assert s2.schedule() is None and list(s2.waiting) == [0, 1]
+
+
+def test_watermark_only_counts_when_others_run():
+    """rust/engine/src/scheduler.rs:1365-1378."""
+    s, cache = make(pages=4, budget=64, watermark_pages=2)
+    s.add(seq(0, 6))                                    # 2 pages; nothing runs, so no watermark
+    plan = s.schedule()
+    assert [p[0] for p in plan.prefill] == [0]
+    run_step(s, cache, plan)
+    s.add(seq(1, 3))                                    # 1 page + watermark 2 > 2 free
+    s.schedule()
+    assert list(s.waiting) == [1]
+
+
+def test_max_num_seqs():
+    s, cache = make(pages=32, max_seqs=2, budget=64)
+    for i in range(3):
+        s.add(seq(i, 3))
+    s.schedule()
+    assert s.running == [0, 1] and list(s.waiting) == [2]
+
+
+def test_partial_prefill_limits():
+    """rust/engine/src/scheduler.rs:1400-1415."""
+    s, cache = make(pages=64, budget=12, max_partial_prefills=2)
+    for i in range(3):
+        s.add(seq(i, 5))
+    assert [p[0] for p in s.schedule().prefill] == [0, 1]
+    s, cache = make(pages=64, budget=64, long_prefill_threshold=8, max_long_partial_prefills=1)
+    s.add(seq(0, 20))
+    s.add(seq(1, 20))
+    s.add(seq(2, 4))
+    assert [p[0] for p in s.schedule().prefill] == [0, 2]   # the second long prompt waits, the short one goes
+
+
+def test_pages_run_out_newest_sequence_is_preempted_and_recomputed():
+    """rust/engine/src/scheduler.rs:933-968, :647-657, :1332."""
+    s, cache = make(pages=4, budget=64, page_size=4)
+    s.add(seq(0, 6, max_tokens=8))                      # 7 tokens reserved: 2 pages
+    s.add(seq(1, 6, max_tokens=8))                      # 2 pages
+    run_step(s, cache, s.schedule())                    # both prompts done, one token each: 7 tokens held
+    for _ in range(2):                                  # positions 6 and 7 fit in the second page of each
+        plan = s.schedule()
+        assert plan.decode == [0, 1]
+        run_step(s, cache, plan)
+    plan = s.schedule()                                 # position 8 needs a third page for both: none left
+    assert plan.decode == [0] and s.preemptions == 1
+    assert list(s.waiting) == [1] and s.running == [0]
+    victim = s.sequences[1]
+    assert victim.num_computed == 0 and victim.prefill_target == len(victim.tokens) == 9 and victim.preempted
+    assert not cache.has_request(1)
+    run_step(s, cache, plan)
+    for _ in range(20):                                 # 0 finishes, then 1 is admitted again and recomputed
+        plan = s.schedule()
+        if plan is None:
+            break
+        run_step(s, cache, plan)
+        for sid in list(s.running):
+            if s.sequences[sid].remaining() <= 0:
+                s.finish(sid)
+    assert not s.has_work() and cache.free_pages() == 4
+    cache.check_invariants()
+
+
+def test_a_single_sequence_is_never_preempted_for_itself():
+    s, cache = make(pages=2, budget=64, page_size=4)
+    s.add(seq(0, 7, max_tokens=8))                      # 8 tokens: both pages
+    run_step(s, cache, s.schedule())
+    run_step(s, cache, s.schedule())                    # the row at position 7 still fits
+    assert s.schedule() is None                         # position 8 has no page; the engine reports no progress
+    assert s.preemptions == 0 and s.running == [0]
+
+
+def test_finish_gives_everything_back():
+    s, cache = make(pages=8, budget=64)
+    s.add(seq(0, 5))
+    run_step(s, cache, s.schedule())
+    s.finish(0)
+    assert cache.free_pages() == 8 and not s.has_work() and cache.free_slots() == 4
