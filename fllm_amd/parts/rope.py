@@ -62,7 +62,9 @@ class Rotary(Part):
         half = self.dims // 2
         lanes = torch.arange(half, dtype=torch.float32)
         exponent = (lanes * 2.0) / float(self.dims)                      # float32, as `(lane*2) as f32 / dims as f32`
-        inv = 1.0 / torch.pow(torch.tensor(self.theta, dtype=torch.float32), exponent)
+        # float32 powf of float32 operands, correctly rounded: evaluated in float64, rounded once
+        base = torch.tensor(self.theta, dtype=torch.float32).double()
+        inv = 1.0 / torch.pow(base, exponent.double()).to(torch.float32)
         if self.scaling == "llama3":
             s = self.spec
             inv = inv / llama3_divisors(self.dims, self.theta, float(s["factor"]), float(s["low_freq_factor"]),

@@ -86,7 +86,9 @@ def rope_tables(positions, dims, theta, kind="default", scaling=None):
     half = dims // 2
     lanes = np.arange(half, dtype=np.float32)
     exponent = (lanes * np.float32(2.0)) / np.float32(dims)
-    inverse = (np.float32(1.0) / np.power(np.float32(theta), exponent)).astype(np.float32)
+    # `base.powf(exponent)` on float32 operands: the correctly rounded float32 power
+    power = np.power(np.float64(np.float32(theta)), exponent.astype(np.float64)).astype(np.float32)
+    inverse = (np.float32(1.0) / power).astype(np.float32)
     scale = np.float32(1.0)
     if kind == "llama3":
         inverse = (inverse / llama3_divisors(dims, theta, float(scaling["factor"]),
