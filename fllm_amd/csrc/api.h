@@ -28,6 +28,24 @@ int fllm_rmsnorm(const float *x, const int32_t *rows, const float *weight, void 
 int fllm_linear(const void *x, int ldx, const void *w, const float *bias, void *out, int ldo, int M, int N, int K,
                 int dtype, int out_mode, hipStream_t stream);
 
+// Fused forms for decode steps in bfloat16 (1..16 rows, K a multiple of 8; fllm_fused_decode_supported).
+// x is the float32 residual stream [M, K]; each computes rmsnorm(x; norm_w, eps) @ w^T (+ bias) and
+//   fllm_norm_linear          stores it as bfloat16 [M, N]
+//   fllm_norm_gate_up_swiglu  w = [gate; up] ([2 I, K]): stores silu(gate) * up as bfloat16 [M, I]
+//   fllm_norm_qkv_rope_store  w = [q; k; v]: rotates query and key lanes in pairs (2l, 2l+1), stores the
+//                             queries as bfloat16 [M, heads * head_dim] and keys and values into the pages
+//                             (layouts and row/segment/table arguments as fllm_rope_kv_store)
+int fllm_fused_decode_supported(int M, int K);
+int fllm_norm_linear(const float *x, const float *norm_w, float eps, const void *w, const float *bias, void *out, int M,
+                     int N, int K, hipStream_t stream);
+int fllm_norm_gate_up_swiglu(const float *x, const float *norm_w, float eps, const void *w_gate_up, const float *bias,
+                             void *out, int M, int inter, int K, hipStream_t stream);
+int fllm_norm_qkv_rope_store(const float *x, const float *norm_w, float eps, const void *w_qkv, const float *bias,
+                             void *q_out, const int32_t *row_pos, const int32_t *row_seg, const int32_t *tables,
+                             int table_stride, const float *cos_table, const float *sin_table, int rope_dims, void *k_pages,
+                             void *v_pages, int M, int heads, int kv_heads, int head_dim, int K, int page_size,
+                             int store_kv, hipStream_t stream);
+
 // out[r, j] = silu(gu[r, j]) * gu[r, I + j]
 int fllm_swiglu(const void *gate_up, void *out, int rows, int inter, int dtype, hipStream_t stream);
 

@@ -15,8 +15,8 @@
 //   tile kernel    portions of prompts: a workgroup takes up to 64 (token, head-of-group) rows of
 //                  one segment and one key/value head; keys and values go through LDS in tiles of 64.
 //   decode kernel  one row per segment: a workgroup takes (row, key/value head, context split), its
-//                  four waves stride over 32-key blocks loading K and V^T straight into MFMA
-//                  operands; splits are merged by a second kernel.
+//                  sixteen waves stride over 32-key blocks loading K and V^T straight into MFMA
+//                  operands; long contexts of small batches are split and merged by a second kernel.
 #include "api.h"
 #include "common.h"
 
@@ -240,17 +240,18 @@ attn_tile_kernel(AttnArgs p) {
 // ---------------------------------------------------------------------------------------------
 // decode kernel
 // ---------------------------------------------------------------------------------------------
-template <int D>
-__global__ void __launch_bounds__(kThreads)
+template <int D, int WAVES>
+__global__ void __launch_bounds__(WAVES * kWave)
 attn_decode_kernel(AttnArgs p, int qtiles) {
     constexpr int KD = D / 32, DT = D / 16;
     constexpr int OP = D + 1;
-    __shared__ float sm_m[kWaves][16], sm_l[kWaves][16];
-    __shared__ float sm_o[kWaves][16][OP];
+    extern __shared__ float dsm[];   // sm_m[WAVES][16], sm_l[WAVES][16], sm_o[WAVES][gq][OP]
     const int row = blockIdx.x;
     const int qtile = blockIdx.y % qtiles, kvh = blockIdx.y / qtiles;
     const int split = blockIdx.z;
     const int G = p.heads / p.kv_heads;
+    const int gq = min(G - qtile * 16, 16);   // query heads of this workgroup
+    float *sm_m = dsm, *sm_l = dsm + WAVES * 16, *sm_o = dsm + 2 * WAVES * 16;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int c = lane & 15, g = lane >> 4;
     const int hg = qtile * 16 + c;
@@ -274,23 +275,35 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
     for (int dt = 0; dt < DT; dt++) o[dt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
 
-    for (int kb = begin + wave * 32; kb < end; kb += kWaves * 32) {
-        // keys: A row c of tile j is key kb + 8*(c/4) + 4*j + c%4; both tiles of a lane lie in one group of 8
+    for (int kb = begin + wave * 32; kb < end; kb += WAVES * 32) {
+        // keys: A row c of tile j is key kb + 8*(c/4) + 4*j + c%4; both tiles of a lane lie in one group of 8.
+        // values: lane (c, g) loads V^T[d = 16 dt + c][keys kb + 8g .. + 7].  All loads of the block are
+        // issued before the first product: one memory latency per block.
         const int grp = kb + (c >> 2) * 8;
         const bool gload = grp < n && grp + 8 > lo;
+        const int vkey = kb + g * 8;
+        const bool vload = vkey < n && vkey + 8 > lo;
         const int kpage = gload ? tbl[grp / ps] : 0;
-        f32x4_t s[2];
+        const int vpage = vload ? tbl[vkey / ps] : 0;
+        bf16x8_t kf[2][KD], vf[DT];
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            s[j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
             const int key = grp + j * 4 + (c & 3);
             const bool valid = gload && key >= lo && key < n;
             const bf16_t *kr = p.kp + (((size_t)kpage * nkv + kvh) * ps + (key % ps)) * D + g * 8;
 #pragma unroll
-            for (int kk = 0; kk < KD; kk++) {
-                const bf16x8_t a = valid ? *(const bf16x8_t *)(kr + kk * 32) : zero8();
-                s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[kk], s[j], 0, 0, 0);
-            }
+            for (int kk = 0; kk < KD; kk++) kf[j][kk] = valid ? *(const bf16x8_t *)(kr + kk * 32) : zero8();
+        }
+        const bf16_t *vr = p.vp + (((size_t)vpage * nkv + kvh) * D + c) * ps + (vkey % ps);
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) vf[dt] = vload ? *(const bf16x8_t *)(vr + (size_t)dt * 16 * ps) : zero8();
+
+        f32x4_t s[2];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            s[j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < KD; kk++) s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[j][kk], qf[kk], s[j], 0, 0, 0);
         }
 #pragma unroll
         for (int j = 0; j < 2; j++)
@@ -303,15 +316,10 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
         float alpha;
         softmax_step<2>(s, m_run, l_run, alpha);
         const bf16x8_t pf = pack_p(s[0], s[1]);
-        // values: lane (c, g) loads V^T[d = 16 dt + c][keys kb + 8g .. + 7]
-        const int vkey = kb + g * 8;
-        const bool vload = vkey < n && vkey + 8 > lo;
-        const int vpage = vload ? tbl[vkey / ps] : 0;
-        const bf16_t *vr = p.vp + (((size_t)vpage * nkv + kvh) * D + c) * ps + (vkey % ps);
         const bool tail = vload && vkey + 8 > n;
 #pragma unroll
         for (int dt = 0; dt < DT; dt++) {
-            bf16x8_t a = vload ? *(const bf16x8_t *)(vr + (size_t)dt * 16 * ps) : zero8();
+            bf16x8_t a = vf[dt];
             if (tail) {   // slots past the last token hold whatever an earlier request left
 #pragma unroll
                 for (int e = 0; e < 8; e++)
@@ -320,29 +328,30 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf, o[dt] * alpha, 0, 0, 0);
         }
     }
-    // the four waves saw different keys: merge their statistics and outputs
+    // the waves saw different keys: merge their statistics and outputs
     if (g == 0) {
-        sm_m[wave][c] = m_run;
-        sm_l[wave][c] = l_run;
+        sm_m[wave * 16 + c] = m_run;
+        sm_l[wave * 16 + c] = l_run;
     }
+    if (c < gq) {
 #pragma unroll
-    for (int dt = 0; dt < DT; dt++)
+        for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-        for (int i = 0; i < 4; i++) sm_o[wave][c][dt * 16 + g * 4 + i] = o[dt][i];
+            for (int i = 0; i < 4; i++) sm_o[(wave * gq + c) * OP + dt * 16 + g * 4 + i] = o[dt][i];
+    }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < 16 * D; idx += kThreads) {
+    for (int idx = threadIdx.x; idx < gq * D; idx += WAVES * kWave) {
         const int qi = idx / D, d = idx - qi * D;
         const int h = qtile * 16 + qi;
-        if (h >= G) continue;
         float m = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < kWaves; w++) m = fmaxf(m, sm_m[w][qi]);
+        for (int w = 0; w < WAVES; w++) m = fmaxf(m, sm_m[w * 16 + qi]);
         float l = 0.f, acc = 0.f;
 #pragma unroll
-        for (int w = 0; w < kWaves; w++) {
-            const float f = sm_m[w][qi] == -INFINITY ? 0.f : fast_exp2(sm_m[w][qi] - m);
-            l += sm_l[w][qi] * f;
-            acc += sm_o[w][qi][d] * f;
+        for (int w = 0; w < WAVES; w++) {
+            const float f = sm_m[w * 16 + qi] == -INFINITY ? 0.f : fast_exp2(sm_m[w * 16 + qi] - m);
+            l += sm_l[w * 16 + qi] * f;
+            acc += sm_o[(w * gq + qi) * OP + d] * f;
         }
         const size_t hrow = (size_t)row * p.heads + kvh * G + h;
         if (p.splits == 1) {
@@ -380,18 +389,21 @@ attn_merge_kernel(const float *__restrict__ ws_ml, const float *__restrict__ ws_
     }
 }
 
-// How a decode step of `rows` rows is split over the context: enough workgroups to fill 256 CUs,
-// at least 128 keys per split.
+// How a decode step of `rows` rows is split over the context.  A workgroup of 16 waves takes 512 keys
+// per round; contexts are split only when they are long and the rows alone do not fill the machine
+// (a split costs a second kernel that merges the parts).
 void decode_split_plan(int rows, int kv_heads, int qtiles, int max_context, int *splits, int *keys_per_split) {
     const long base = (long)rows * kv_heads * qtiles;
-    long want = (1024 + base - 1) / base;
-    const long most = (max_context + 127) / 128;
-    if (want > most) want = most;
-    if (want > 64) want = 64;
-    if (want < 1) want = 1;
     const long span = (long)max_context + 31;   // the first split starts at a multiple of 32 at or below the first key
+    long want = 1;
+    if (span > 2048 && base < 256) {
+        want = (256 + base - 1) / base;
+        const long most = (span + 2047) / 2048;
+        if (want > most) want = most;
+        if (want > 64) want = 64;
+    }
     long per = (span + want - 1) / want;
-    per = (per + 127) / 128 * 128;
+    per = (per + 511) / 512 * 512;
     *splits = (int)want;
     *keys_per_split = (int)per;
 }
@@ -419,8 +431,18 @@ int launch(const AttnArgs &a, int uniform_rows, int max_context, void *workspace
             p.ws_o = p.ws_ml + (size_t)a.rows * a.heads * p.splits * 2;
         }
         FLLM_REQUIRE(a.kv_heads * qtiles <= 65535 && p.splits <= 65535, "attention: grid too large");
-        hipLaunchKernelGGL(attn_decode_kernel<D>, dim3(a.rows, a.kv_heads * qtiles, p.splits), dim3(kThreads), 0, stream, p,
-                           qtiles);
+        constexpr int WAVES = D >= 128 ? 8 : 16;   // wide heads: fewer waves, so that the operands of a block fit the registers
+        const int gq = G < 16 ? G : 16;
+        const size_t smem = (size_t)(2 * WAVES * 16 + WAVES * gq * (D + 1)) * sizeof(float);
+        static bool attribute_set = false;   // more than the default 64 KiB of dynamic LDS has to be asked for once
+        if (!attribute_set) {
+            const hipError_t e = hipFuncSetAttribute((const void *)attn_decode_kernel<D, WAVES>,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            FLLM_REQUIRE(e == hipSuccess, "attention: cannot raise the LDS limit: %s", hipGetErrorString(e));
+            attribute_set = true;
+        }
+        hipLaunchKernelGGL((attn_decode_kernel<D, WAVES>), dim3(a.rows, a.kv_heads * qtiles, p.splits), dim3(WAVES * kWave),
+                           smem, stream, p, qtiles);
         if (p.splits > 1)
             hipLaunchKernelGGL(attn_merge_kernel<D>, dim3(a.rows, a.heads), dim3(kWave), 0, stream, p.ws_ml, p.ws_o, a.out,
                                a.heads, p.splits);

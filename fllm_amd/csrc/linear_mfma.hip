@@ -1,10 +1,7 @@
 // bfloat16 matrix products y = x w^T on the MFMA units of gfx950, float32 accumulation.
 //
-// Two kernels.  `skinny` (M <= 64 rows, the decode step) streams the weight matrix once: a
-// workgroup owns 16 weight rows, its waves split K between them and add their partial sums in
-// wave order through LDS, so the result is deterministic.  Weight fragments go from global memory
-// straight into MFMA operands (each weight is used once; LDS would only add a hop).  `tiled`
-// (M > 64, prompt portions) is a 128x128x64 LDS-tiled kernel, four waves of 64x64 each on
+// Calls of up to 64 rows (decode steps) go to the weight-streaming kernel of linear_skinny.hip.
+// `tiled` (M > 64, prompt portions) is a 128x128x64 LDS-tiled kernel, four waves of 64x64 each on
 // v_mfma_f32_32x32x16_bf16, with register prefetch of the next tile.
 //
 // MFMA operand layouts used here (wave64):
@@ -14,6 +11,9 @@
 //             D lane l holds D[m = 8*(i/4) + 4*(l/32) + i%4][n = l%32], i = 0..15.
 #include "api.h"
 #include "common.h"
+
+int fllm_linear_bf16_skinny(const void *x, int ldx, const void *w, const float *bias, void *out, int ldo, int M, int N,
+                            int K, int out_mode, hipStream_t stream);   // linear_skinny.hip; 1: shape declined
 
 namespace {
 
@@ -28,80 +28,6 @@ __device__ __forceinline__ void store_out(void *out, size_t o, float v, int out_
     if (out_mode == 0) ((bf16_t *)out)[o] = (bf16_t)v;
     else if (out_mode == 1) ((float *)out)[o] = v;
     else ((float *)out)[o] += v;
-}
-
-// ---------------------------------------------------------------------------------------------
-// skinny: M <= 16 * MT
-// ---------------------------------------------------------------------------------------------
-template <int MT, int WAVES>
-__global__ void __launch_bounds__(WAVES * kWave)
-linear_skinny_kernel(const bf16_t *__restrict__ x, int ldx, const bf16_t *__restrict__ w, const float *__restrict__ bias,
-                     void *__restrict__ out, int ldo, int M, int N, int K, int out_mode) {
-    extern __shared__ float red[];   // [WAVES][MT][64] float4
-    constexpr int U = 4;             // k-steps of 32 per wave iteration
-    constexpr int KCHUNK = 32 * U;
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    const int r = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * 16;
-    int wrow = n0 + r;
-    if (wrow >= N) wrow = N - 1;   // rows past the end are computed from a valid row and never stored
-    const bf16_t *wp = w + (size_t)wrow * K + g * 8;
-    const bf16_t *xp[MT];
-    bool xvalid[MT];
-#pragma unroll
-    for (int t = 0; t < MT; t++) {
-        const int m = t * 16 + r;
-        xvalid[t] = m < M;
-        xp[t] = x + (size_t)(xvalid[t] ? m : 0) * ldx + g * 8;
-    }
-    f32x4_t acc[MT];
-#pragma unroll
-    for (int t = 0; t < MT; t++) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-
-    for (int k0 = wave * KCHUNK; k0 < K; k0 += WAVES * KCHUNK) {
-        bf16x8_t a[U], b[MT][U];
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int k = k0 + u * 32;
-            const bool in = k + g * 8 < K;   // K is a multiple of 8: a lane's 8 values are all inside or all outside
-            a[u] = in ? *(const bf16x8_t *)(wp + k) : zero8();
-#pragma unroll
-            for (int t = 0; t < MT; t++) b[t][u] = (in && xvalid[t]) ? *(const bf16x8_t *)(xp[t] + k) : zero8();
-        }
-#pragma unroll
-        for (int u = 0; u < U; u++)
-#pragma unroll
-            for (int t = 0; t < MT; t++) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[t][u], acc[t], 0, 0, 0);
-    }
-    f32x4_t *red4 = (f32x4_t *)red;
-#pragma unroll
-    for (int t = 0; t < MT; t++) red4[(wave * MT + t) * kWave + lane] = acc[t];
-    __syncthreads();
-    for (int e = threadIdx.x; e < MT * kWave; e += WAVES * kWave) {
-        const int t = e / kWave, l = e % kWave;
-        f32x4_t s = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int wv = 0; wv < WAVES; wv++) s += red4[(wv * MT + t) * kWave + l];
-        const int m = t * 16 + (l & 15);
-        const int nb = n0 + (l >> 4) * 4;
-        if (m >= M) continue;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int n = nb + i;
-            if (n >= N) continue;
-            float v = s[i];
-            if (bias) v += bias[n];
-            store_out(out, (size_t)m * ldo + n, v, out_mode);
-        }
-    }
-}
-
-template <int MT, int WAVES>
-void launch_skinny(const bf16_t *x, int ldx, const bf16_t *w, const float *bias, void *out, int ldo, int M, int N, int K,
-                   int out_mode, hipStream_t stream) {
-    const size_t smem = (size_t)WAVES * MT * kWave * sizeof(f32x4_t);
-    hipLaunchKernelGGL((linear_skinny_kernel<MT, WAVES>), dim3((N + 15) / 16), dim3(WAVES * kWave), smem, stream, x, ldx, w,
-                       bias, out, ldo, M, N, K, out_mode);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -203,18 +129,8 @@ int fllm_linear_bf16_fast(const void *x, int ldx, const void *w, const float *bi
     if (K % 8 != 0 || ldx % 8 != 0 || ((uintptr_t)x & 15) != 0 || ((uintptr_t)w & 15) != 0) return 1;
     const bf16_t *xb = (const bf16_t *)x, *wb = (const bf16_t *)w;
     if (M <= 64) {
-        // few weight-row tiles: more waves per tile keep enough loads in flight
-        const bool wide = (N + 15) / 16 < 1024;
-        const int mt = (M + 15) / 16;
-#define FLLM_SKINNY(MT)                                                                                    \
-    if (wide) launch_skinny<MT, 16>(xb, ldx, wb, bias, out, ldo, M, N, K, out_mode, stream);                \
-    else launch_skinny<MT, 8>(xb, ldx, wb, bias, out, ldo, M, N, K, out_mode, stream)
-        if (mt == 1) { FLLM_SKINNY(1); }
-        else if (mt == 2) { FLLM_SKINNY(2); }
-        else if (mt == 3) { FLLM_SKINNY(3); }
-        else { FLLM_SKINNY(4); }
-#undef FLLM_SKINNY
-        return fllm_check_launch("linear_skinny");
+        const int rc = fllm_linear_bf16_skinny(x, ldx, w, bias, out, ldo, M, N, K, out_mode, stream);
+        if (rc != 1) return rc;
     }
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     hipLaunchKernelGGL(linear_tiled_mfma_kernel, dim3(tiles_m * tiles_n), dim3(kTiledThreads), 0, stream, xb, ldx, wb, bias,

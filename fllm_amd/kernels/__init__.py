@@ -59,6 +59,10 @@ def load_library(build_if_missing: bool = True):
                                c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_attention": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_int,
                            c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void, c_size, c_void],
+        "fllm_norm_linear": [c_void, c_void, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
+        "fllm_norm_gate_up_swiglu": [c_void, c_void, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
+        "fllm_norm_qkv_rope_store": [c_void, c_void, c_float, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void,
+                                     c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_argmax": [c_void, c_void, c_int, c_int, c_void],
         "fllm_sample": [c_void, c_void, c_void, c_void, c_int, c_int, c_void],
     }
@@ -66,6 +70,8 @@ def load_library(build_if_missing: bool = True):
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = c_int
+    lib.fllm_fused_decode_supported.argtypes = [c_int, c_int]
+    lib.fllm_fused_decode_supported.restype = c_int
     lib.fllm_set_fast_kernels.argtypes = [c_int]
     lib.fllm_set_fast_kernels.restype = None
     lib.fllm_attention_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int, c_int]
@@ -163,6 +169,63 @@ class Ops:
         self._check(self.lib.fllm_linear(_ptr(x), ldx, _ptr(w), _ptr(bias), _ptr(out), ldo, M, N, K, _DTYPE_CODE[x.dtype],
                                          mode, self._stream()))
         return out
+
+    # ---- fused forms of decode steps (bfloat16, at most 16 rows) ---------------------------------
+    def fused_decode_supported(self, rows: int, width: int) -> bool:
+        return bool(self.lib.fllm_fused_decode_supported(int(rows), int(width)))
+
+    def _fused_operands(self, x, norm_weight, w, bias, n_rows_w):
+        M, K = x.shape
+        _dense(x, "x", torch.float32)
+        _dense(norm_weight, "norm_weight", torch.float32, (K,))
+        _dense(w, "w", torch.bfloat16, (n_rows_w, K))
+        if bias is not None:
+            _dense(bias, "bias", torch.float32, (n_rows_w,))
+        _need(self.fused_decode_supported(M, K), f"the fused decode kernels take 1..16 rows and widths in steps of 8, not {M} x {K}")
+        return M, K
+
+    def norm_linear(self, x, norm_weight, eps, w, out, bias=None):
+        """out = rmsnorm(x) @ w.T (+ bias); x float32 [M, K], w bfloat16 [N, K], out bfloat16 [M, N]."""
+        N = w.shape[0]
+        M, K = self._fused_operands(x, norm_weight, w, bias, N)
+        _dense(out, "out", torch.bfloat16, (M, N))
+        self._check(self.lib.fllm_norm_linear(_ptr(x), _ptr(norm_weight), float(eps), _ptr(w), _ptr(bias), _ptr(out), M, N, K,
+                                              self._stream()))
+        return out
+
+    def norm_gate_up_swiglu(self, x, norm_weight, eps, w_gate_up, out, bias=None):
+        """out = silu(rmsnorm(x) @ gate.T) * (rmsnorm(x) @ up.T); w_gate_up = [gate; up], out bfloat16 [M, I]."""
+        two_i = w_gate_up.shape[0]
+        _need(two_i % 2 == 0, "w_gate_up needs an even number of rows")
+        M, K = self._fused_operands(x, norm_weight, w_gate_up, bias, two_i)
+        _dense(out, "out", torch.bfloat16, (M, two_i // 2))
+        self._check(self.lib.fllm_norm_gate_up_swiglu(_ptr(x), _ptr(norm_weight), float(eps), _ptr(w_gate_up), _ptr(bias),
+                                                      _ptr(out), M, two_i // 2, K, self._stream()))
+        return out
+
+    def norm_qkv_rope_store(self, x, norm_weight, eps, w_qkv, q_out, row_pos, row_seg, tables, cos, sin, k_pages, v_pages,
+                            heads, kv_heads, head_dim, rope_dims, page_size, bias=None):
+        """q, k, v = rmsnorm(x) @ w_qkv.T; rotary on pairs (2l, 2l+1) of q and k; q to `q_out`
+        (bfloat16 [M, heads * head_dim]), k and v into the pages (None: not stored)."""
+        M, K = self._fused_operands(x, norm_weight, w_qkv, bias, (heads + 2 * kv_heads) * head_dim)
+        _dense(q_out, "q_out", torch.bfloat16, (M, heads * head_dim))
+        _dense(row_pos, "row_pos", torch.int32, (M,))
+        _dense(row_seg, "row_seg", torch.int32, (M,))
+        _dense(tables, "tables", torch.int32)
+        _need(tables.dim() == 2, "tables must be [segments, pages]")
+        _dense(cos, "cos", torch.float32)
+        _dense(sin, "sin", torch.float32, tuple(cos.shape))
+        _need(cos.dim() == 2 and cos.shape[1] == rope_dims // 2, f"rotary tables must be [positions, {rope_dims // 2}]")
+        store = k_pages is not None
+        if store:
+            pages = k_pages.shape[0]
+            _dense(k_pages, "k_pages", torch.bfloat16, (pages, kv_heads, page_size, head_dim))
+            _dense(v_pages, "v_pages", torch.bfloat16, (pages, kv_heads, head_dim, page_size))
+        self._check(self.lib.fllm_norm_qkv_rope_store(
+            _ptr(x), _ptr(norm_weight), float(eps), _ptr(w_qkv), _ptr(bias), _ptr(q_out), _ptr(row_pos), _ptr(row_seg),
+            _ptr(tables), tables.shape[1], _ptr(cos), _ptr(sin), rope_dims, _ptr(k_pages), _ptr(v_pages), M, heads, kv_heads,
+            head_dim, K, page_size, 1 if store else 0, self._stream()))
+        return q_out
 
     def swiglu(self, gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         rows, two_i = gate_up.shape

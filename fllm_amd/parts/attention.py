@@ -47,16 +47,41 @@ class PagedAttention(Mixer):
             position = dict(position)
             kind = position.pop("kind")
             self.position = part_class("position", kind)(PartSpec(kind, position), {}, rt)
+        # Rotary with the checkpoint's pairing (l, l + dims/2): the rows of the q and k projections are
+        # reordered inside every head so that the partners sit next to each other (2l, 2l + 1), the
+        # pairing the kernels rotate.  q . k does not change when both are reordered alike
+        # (the reference's importer does the same: rust/checkpoint/src/convert.rs:2713-2745).
+        self.pairing = 1
+        order_q = order_k = None
+        if self.position is not None and self.position.pairing == 0:
+            order_q = self._pair_order(self.heads, self.head_dim, self.position.dims).to(rt.device)
+            order_k = self._pair_order(self.kv_heads, self.head_dim, self.position.dims).to(rt.device)
+        elif self.position is not None:
+            self.pairing = self.position.pairing
+        reorder = lambda t, order: t if order is None or t is None else t.index_select(0, order)
         # one matrix for q, k and v: the normed input is read once
-        self.w_qkv = torch.cat([rt.matrix(weights["q"]), rt.matrix(weights["k"]), rt.matrix(weights["v"])], dim=0).contiguous()
+        self.w_qkv = torch.cat([reorder(rt.matrix(weights["q"]), order_q), reorder(rt.matrix(weights["k"]), order_k),
+                                rt.matrix(weights["v"])], dim=0).contiguous()
         self.w_o = rt.matrix(weights["o"])
-        biases = [weights.get(n) for n in ("q_bias", "k_bias", "v_bias")]
+        biases = [reorder(None if weights.get("q_bias") is None else rt.vector(weights["q_bias"]), order_q),
+                  reorder(None if weights.get("k_bias") is None else rt.vector(weights["k_bias"]), order_k),
+                  None if weights.get("v_bias") is None else rt.vector(weights["v_bias"])]
         self.b_qkv = None
         if any(b is not None for b in biases):
             sizes = (self.heads * self.head_dim, self.kv_heads * self.head_dim, self.kv_heads * self.head_dim)
-            self.b_qkv = torch.cat([rt.vector(b) if b is not None else torch.zeros(n, dtype=torch.float32, device=rt.device)
+            self.b_qkv = torch.cat([b if b is not None else torch.zeros(n, dtype=torch.float32, device=rt.device)
                                     for b, n in zip(biases, sizes)]).contiguous()
         self.b_o = rt.vector(weights["o_bias"]) if weights.get("o_bias") is not None else None
+
+    @staticmethod
+    def _pair_order(heads: int, head_dim: int, rope_dims: int) -> torch.Tensor:
+        """New row -> old row: inside every head, row 2l comes from l and row 2l + 1 from l + rope_dims/2."""
+        half = rope_dims // 2
+        one = []
+        for l in range(half):
+            one += [l, l + half]
+        one += list(range(rope_dims, head_dim))
+        return torch.tensor([h * head_dim + j for h in range(heads) for j in one], dtype=torch.long)
 
     def cache_need(self):
         return KVNeed(self.kv_heads, self.head_dim, self.window)
@@ -69,14 +94,43 @@ class PagedAttention(Mixer):
         ops.linear(h, self.w_qkv, qkv, bias=self.b_qkv)
         tables = ctx.tables[binding.group]
         if self.position is not None:
-            cos, sin, dims, pairing = self.position.cos, self.position.sin, self.position.dims, self.position.pairing
+            cos, sin, dims, pairing = self.position.cos, self.position.sin, self.position.dims, self.pairing
         else:
             cos, sin, dims, pairing = ctx.no_rotation(rt)
         ops.rope_kv_store(qkv, ctx.row_pos, ctx.row_seg, tables, cos, sin,
                           binding.k_pages if binding.writes else None, binding.v_pages if binding.writes else None,
                           nh, nkv, d, dims, pairing, binding.page_size)
+        self._attend_and_project(ctx, qkv[:, : nh * d], residual, binding)
+
+    def forward_from_residual(self, ctx, residual, norm, binding) -> bool:
+        """Decode-sized steps in bfloat16: the norm before the mixer, the q/k/v product, rotary and the
+        cache store are one kernel.  False: not taken, the block runs norm and `forward`."""
+        rt, ops = self.rt, self.rt.ops
+        rows = residual.shape[0]
+        if (rt.dtype != torch.bfloat16 or self.pairing != 1 or getattr(norm, "spec", None) is None or norm.spec.kind != "rms"
+                or not hasattr(ops, "norm_qkv_rope_store") or not ops.fused_decode_supported(rows, self.hidden)
+                or self.head_dim % 4 != 0):
+            return False
+        nh, nkv, d = self.heads, self.kv_heads, self.head_dim
+        if self.position is not None:
+            cos, sin, dims = self.position.cos, self.position.sin, self.position.dims
+        else:
+            cos, sin, dims, _ = ctx.no_rotation(rt)
+        q = rt.empty((rows, nh * d))
+        ops.norm_qkv_rope_store(residual, norm.weight, norm.eps, self.w_qkv, q, ctx.row_pos, ctx.row_seg,
+                                ctx.tables[binding.group], cos, sin, binding.k_pages if binding.writes else None,
+                                binding.v_pages if binding.writes else None, nh, nkv, d, dims, binding.page_size,
+                                bias=self.b_qkv)
+        self._attend_and_project(ctx, q, residual, binding)
+        return True
+
+    def _attend_and_project(self, ctx, q, residual, binding):
+        rt, ops = self.rt, self.rt.ops
+        rows = q.shape[0]
+        nh, nkv, d = self.heads, self.kv_heads, self.head_dim
+        tables = ctx.tables[binding.group]
         out = rt.empty((rows, nh * d))
-        ops.attention(qkv[:, : nh * d], binding.k_pages, binding.v_pages, tables, ctx.row_pos, ctx.row_seg, ctx.seg_start,
+        ops.attention(q, binding.k_pages, binding.v_pages, tables, ctx.row_pos, ctx.row_seg, ctx.seg_start,
                       out, nh, nkv, d, binding.page_size, self.scale, self.window, ctx.max_context,
                       uniform_rows=1 if ctx.uniform_rows else 0,
                       workspace=ctx.attention_workspace(rt, rows, nh, nkv, d))

@@ -15,10 +15,15 @@ class PreNormBlock(Block):
         self.feed_forward_norm = norms["feed_forward"]
 
     def forward(self, ctx, residual, binding):
-        h = self.mixer_norm.forward(ctx, residual)
-        self.mixer.forward(ctx, h, residual, binding)
-        h = self.feed_forward_norm.forward(ctx, residual)
-        self.feed_forward.forward(ctx, h, residual)
+        # a part may take the residual stream and the norm before it in one fused kernel
+        fused = getattr(self.mixer, "forward_from_residual", None)
+        if fused is None or not fused(ctx, residual, self.mixer_norm, binding):
+            h = self.mixer_norm.forward(ctx, residual)
+            self.mixer.forward(ctx, h, residual, binding)
+        fused = getattr(self.feed_forward, "forward_from_residual", None)
+        if fused is None or not fused(ctx, residual, self.feed_forward_norm):
+            h = self.feed_forward_norm.forward(ctx, residual)
+            self.feed_forward.forward(ctx, h, residual)
 
 
 register_part("block", "prenorm", PreNormBlock)

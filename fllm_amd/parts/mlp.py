@@ -34,6 +34,19 @@ class GatedMLP(FeedForward):
                                         rt.vector(ub) if ub is not None else zeros()]).contiguous()
         self.b_down = rt.vector(weights["down_bias"]) if weights.get("down_bias") is not None else None
 
+    def forward_from_residual(self, ctx, residual, norm) -> bool:
+        """Decode-sized steps in bfloat16: norm, gate/up product and activation are one kernel.
+        False: not taken, the block runs norm and `forward`."""
+        rt, ops = self.rt, self.rt.ops
+        rows = residual.shape[0]
+        if (rt.dtype != torch.bfloat16 or getattr(norm, "spec", None) is None or norm.spec.kind != "rms"
+                or not hasattr(ops, "norm_gate_up_swiglu") or not ops.fused_decode_supported(rows, self.hidden)):
+            return False
+        act = rt.empty((rows, self.inter))
+        ops.norm_gate_up_swiglu(residual, norm.weight, norm.eps, self.w_gate_up, act, bias=self.b_gate_up)
+        ops.linear(act, self.w_down, residual, bias=self.b_down, accumulate=True)
+        return True
+
     def forward(self, ctx, h, residual):
         rt, ops = self.rt, self.rt.ops
         rows = h.shape[0]

@@ -36,6 +36,43 @@ class ReferenceOps:
             out.copy_(y.to(out.dtype))
         return out
 
+    # fused forms of decode steps: the same formulas, composed
+    def fused_decode_supported(self, rows, width):
+        return 1 <= rows <= 16 and width % 8 == 0
+
+    def _normed(self, x, norm_weight, eps):
+        x = x.double()
+        return x * (torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * norm_weight.double())
+
+    def norm_linear(self, x, norm_weight, eps, w, out, bias=None):
+        y = self._normed(x, norm_weight, eps) @ w.double().T
+        out.copy_((y if bias is None else y + bias.double()).to(out.dtype))
+        return out
+
+    def norm_gate_up_swiglu(self, x, norm_weight, eps, w_gate_up, out, bias=None):
+        y = self._normed(x, norm_weight, eps) @ w_gate_up.double().T
+        if bias is not None:
+            y = y + bias.double()
+        inter = y.shape[1] // 2
+        g, u = y[:, :inter], y[:, inter:]
+        out.copy_((g / (1.0 + torch.exp(-g)) * u).to(out.dtype))
+        return out
+
+    def norm_qkv_rope_store(self, x, norm_weight, eps, w_qkv, q_out, row_pos, row_seg, tables, cos, sin, k_pages, v_pages,
+                            heads, kv_heads, head_dim, rope_dims, page_size, bias=None):
+        y = self._normed(x, norm_weight, eps) @ w_qkv.double().T
+        if bias is not None:
+            y = y + bias.double()
+        qkv = y.clone()                 # rotated in float64, rounded once when stored
+        kp = None if k_pages is None else k_pages.double()
+        vp = None if v_pages is None else v_pages.double()
+        self.rope_kv_store(qkv, row_pos, row_seg, tables, cos, sin, kp, vp, heads, kv_heads, head_dim, rope_dims, 1, page_size)
+        q_out.copy_(qkv[:, : heads * head_dim].to(q_out.dtype))
+        if k_pages is not None:
+            k_pages.copy_(kp.to(k_pages.dtype))
+            v_pages.copy_(vp.to(v_pages.dtype))
+        return q_out
+
     def swiglu(self, gate_up, out):
         inter = gate_up.shape[1] // 2
         g, u = gate_up[:, :inter].double(), gate_up[:, inter:].double()

@@ -142,6 +142,89 @@ def test_linear_bf16_strided_input(ops, ref):
     close(got, want, 1e-5, 1e-5, "strided")
 
 
+# ---- fused forms of decode steps ----------------------------------------------------------------
+FUSED_SHAPES = [(1, 4096, 4096), (1, 64, 136), (8, 6144, 4096), (5, 100, 72), (16, 520, 264), (13, 128, 128), (2, 1000, 4096),
+                (16, 4096, 4096), (9, 96, 14336), (3, 256, 20000), (16, 48, 40000)]
+
+
+def _fused_inputs(M, K, seed):
+    g = gen(seed)
+    x = torch.randn(M, K, generator=g) * torch.rand(M, 1, generator=g) * 8      # rows of different scale
+    nw = 1 + 0.1 * torch.randn(K, generator=g)
+    return g, x, nw
+
+
+@pytest.mark.parametrize("M,N,K", FUSED_SHAPES)
+@pytest.mark.parametrize("bias", [False, True])
+def test_norm_linear(ops, ref, M, N, K, bias):
+    g, x, nw = _fused_inputs(M, K, 30)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g) if bias else None
+    want = ref.norm_linear(x, nw, 1e-5, w, torch.empty(M, N, dtype=torch.float64), bias=b)
+    got = ops.norm_linear(x.to(DEV), nw.to(DEV), 1e-5, w.to(DEV), torch.empty(M, N, dtype=torch.bfloat16, device=DEV),
+                          bias=None if b is None else b.to(DEV))
+    # the normed operand is rounded to bfloat16 before the product: sqrt(K) * 2^-9 relative to the row's scale
+    close(got, want, 2 * BF16_EPS, 3e-2, f"norm_linear M{M} N{N} K{K}")
+
+
+@pytest.mark.parametrize("M,inter,K", [(1, 14336, 4096), (1, 176, 64), (8, 432, 160), (13, 1000, 4096), (16, 200, 96), (4, 512, 36000)])
+def test_norm_gate_up_swiglu(ops, ref, M, inter, K):
+    g, x, nw = _fused_inputs(M, K, 31)
+    w = (torch.randn(2 * inter, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    b = torch.randn(2 * inter, generator=g) * 0.1
+    want = ref.norm_gate_up_swiglu(x, nw, 1e-6, w, torch.empty(M, inter, dtype=torch.float64), bias=b)
+    got = ops.norm_gate_up_swiglu(x.to(DEV), nw.to(DEV), 1e-6, w.to(DEV), torch.empty(M, inter, dtype=torch.bfloat16, device=DEV),
+                                  bias=b.to(DEV))
+    close(got, want, 2 * BF16_EPS, 4e-2, f"norm_gate_up_swiglu M{M} I{inter} K{K}")
+
+
+@pytest.mark.parametrize("heads,kv_heads,head_dim,rope_dims,page_size,K", [(4, 2, 16, 16, 16, 64), (5, 1, 32, 32, 8, 160),
+                                                                           (6, 3, 48, 24, 16, 96), (32, 8, 128, 128, 16, 4096),
+                                                                           (2, 2, 16, 0, 16, 64)])
+@pytest.mark.parametrize("segs", [[(0, 1)], [(14, 1), (15, 1), (16, 1), (100, 1), (7, 1)], [(5, 3), (40, 2), (127, 1)]])
+def test_norm_qkv_rope_store(ops, ref, heads, kv_heads, head_dim, rope_dims, page_size, K, segs):
+    g, _, _ = _fused_inputs(1, 8, 32)
+    rows = sum(n for _, n in segs)
+    _, x, nw = _fused_inputs(rows, K, 33)
+    positions = 128
+    pages_each = positions // page_size
+    num_pages = len(segs) * pages_each + 3
+    tables = scattered_tables(g, len(segs), pages_each, num_pages)
+    row_pos = torch.tensor([p + i for p, n in segs for i in range(n)], dtype=torch.int32)
+    row_seg = torch.tensor([s for s, (_, n) in enumerate(segs) for _ in range(n)], dtype=torch.int32)
+    row_seg[-1] = -1 if rows > 3 else row_seg[-1]             # a padding row stores nothing
+    angle = torch.rand(positions, rope_dims // 2, generator=g, dtype=torch.float64) * 6.28
+    cos, sin = torch.cos(angle).float(), torch.sin(angle).float()
+    N = (heads + 2 * kv_heads) * head_dim
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g) * 0.1
+    k0, v0 = make_pages(g, num_pages, kv_heads, page_size, head_dim, torch.bfloat16)
+    k_ref, v_ref = k0.clone(), v0.clone()
+    q_ref = ref.norm_qkv_rope_store(x, nw, 1e-5, w, torch.zeros(rows, heads * head_dim, dtype=torch.float64), row_pos, row_seg,
+                                    tables, cos, sin, k_ref, v_ref, heads, kv_heads, head_dim, rope_dims, page_size, bias=b)
+    k_gpu, v_gpu = k0.to(DEV), v0.to(DEV)
+    q_gpu = ops.norm_qkv_rope_store(x.to(DEV), nw.to(DEV), 1e-5, w.to(DEV), torch.zeros(rows, heads * head_dim, dtype=torch.bfloat16, device=DEV),
+                                    row_pos.to(DEV), row_seg.to(DEV), tables.to(DEV), cos.to(DEV), sin.to(DEV), k_gpu, v_gpu,
+                                    heads, kv_heads, head_dim, rope_dims, page_size, bias=b.to(DEV))
+    live = (row_seg >= 0)
+    close(q_gpu[live.to(DEV)], q_ref[live], 2 * BF16_EPS, 4e-2, "fused q")
+    close(k_gpu, k_ref, 2 * BF16_EPS, 4e-2, "fused k pages")
+    close(v_gpu, v_ref, 2 * BF16_EPS, 4e-2, "fused v pages")
+    # slots of other tokens keep their bits
+    untouched = torch.ones(num_pages, page_size, dtype=torch.bool)
+    for r in range(rows):
+        if row_seg[r] >= 0:
+            untouched[int(tables[int(row_seg[r]), int(row_pos[r]) // page_size]), int(row_pos[r]) % page_size] = False
+    assert torch.equal(k_gpu.cpu().permute(0, 2, 1, 3)[untouched], k0.permute(0, 2, 1, 3)[untouched])
+    assert torch.equal(v_gpu.cpu().permute(0, 3, 1, 2)[untouched], v0.permute(0, 3, 1, 2)[untouched])
+    # reading another entry's cache: queries only
+    k2, v2 = k0.to(DEV), v0.to(DEV)
+    q2 = ops.norm_qkv_rope_store(x.to(DEV), nw.to(DEV), 1e-5, w.to(DEV), torch.zeros(rows, heads * head_dim, dtype=torch.bfloat16, device=DEV),
+                                 row_pos.to(DEV), row_seg.to(DEV), tables.to(DEV), cos.to(DEV), sin.to(DEV), None, None,
+                                 heads, kv_heads, head_dim, rope_dims, page_size, bias=b.to(DEV))
+    assert torch.equal(q2[live.to(DEV)], q_gpu[live.to(DEV)])
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("rows,inter", [(1, 176), (13, 432), (3, 14336)])
 def test_swiglu(ops, ref, dtype, rows, inter):
