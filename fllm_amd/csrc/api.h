@@ -23,6 +23,10 @@ int fllm_embed(const int32_t *ids, const void *table, float *out, int rows, int 
 int fllm_rmsnorm(const float *x, const int32_t *rows, const float *weight, void *out, int count, int width, float eps,
                  int out_dtype, hipStream_t stream);
 
+// x[r, :] += branch[r, :] (float32 sum, written back), then out[r, :] = rmsnorm(x[r, :]) as above
+int fllm_add_rmsnorm(float *x, const void *branch, int branch_dtype, const float *weight, void *out, int count, int width,
+                     float eps, int out_dtype, hipStream_t stream);
+
 // y[m, n] = sum_k x[m, k] * w[n, k] (+ bias[n]);   x: [M, K] (row stride ldx), w: [N, K]
 // out_mode 0: store as `dtype`; 1: store float32; 2: add to float32 `out` (row stride ldo)
 int fllm_linear(const void *x, int ldx, const void *w, const float *bias, void *out, int ldo, int M, int N, int K,
@@ -45,6 +49,9 @@ int fllm_norm_qkv_rope_store(const float *x, const float *norm_w, float eps, con
                              int table_stride, const float *cos_table, const float *sin_table, int rope_dims, void *k_pages,
                              void *v_pages, int M, int heads, int kv_heads, int head_dim, int K, int page_size,
                              int store_kv, hipStream_t stream);
+
+// residual[r, :] += branch[r, :]   (residual float32 [rows, width], branch of type `dtype`)
+int fllm_add_residual(float *residual, const void *branch, int rows, int width, int dtype, hipStream_t stream);
 
 // out[r, j] = silu(gu[r, j]) * gu[r, I + j]
 int fllm_swiglu(const void *gate_up, void *out, int rows, int inter, int dtype, hipStream_t stream);

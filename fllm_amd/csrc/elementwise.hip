@@ -21,36 +21,103 @@ embed_kernel(const int32_t *__restrict__ ids, const T *__restrict__ table, float
 }
 
 // One workgroup per output row.  The sum of squares is taken in a fixed order (thread t adds
-// elements t, t + 256, ...; then lanes, then waves), so a row gives the same bits whatever else
-// is in the batch.
-template <typename T>
+// the elements of its groups of four, groups t, t + 256, ...; then lanes, then waves), so a row
+// gives the same bits whatever else is in the batch.  With `branch` the kernel first adds it to
+// the row (x += branch, in float32, written back): residual add and the next norm in one pass.
+// Rows of up to 256 * 4 * VEC values stay in registers between the two uses.
+template <typename T, typename B, int VEC>
 __global__ void __launch_bounds__(kBlock)
-rmsnorm_kernel(const float *__restrict__ x, const int32_t *__restrict__ rows, const float *__restrict__ weight,
-               T *__restrict__ out, int width, float eps) {
+rmsnorm_kernel(float *__restrict__ x, const B *__restrict__ branch, const int32_t *__restrict__ rows,
+               const float *__restrict__ weight, T *__restrict__ out, int width, float eps) {
     __shared__ float scratch[kWaves];
     const int i = blockIdx.x;
     const int r = rows ? rows[i] : i;
-    const float *src = x + (size_t)r * width;
-    float ss = 0.f;
-    for (int c = threadIdx.x; c < width; c += kBlock) {
-        const float v = src[c];
-        ss += v * v;
-    }
-    ss = block_sum<kWaves>(ss, scratch);
-    const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+    float *src = x + (size_t)r * width;
+    const B *br = branch ? branch + (size_t)r * width : nullptr;
     T *dst = out + (size_t)i * width;
-    for (int c = threadIdx.x; c < width; c += kBlock) dst[c] = from_f32<T>(src[c] * (inv * weight[c]));
+    if constexpr (VEC > 0) {   // width is a multiple of 4 and at most 1024 * VEC
+        f32x4_t v[VEC > 0 ? VEC : 1];
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            const int c = (threadIdx.x + j * kBlock) * 4;
+            if (c < width) {
+                v[j] = *(const f32x4_t *)(src + c);
+                if (br) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[j][e] += to_f32<B>(br[c + e]);
+                    *(f32x4_t *)(src + c) = v[j];
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) ss += v[j][e] * v[j][e];
+            }
+        }
+        ss = block_sum<kWaves>(ss, scratch);
+        const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            const int c = (threadIdx.x + j * kBlock) * 4;
+            if (c < width) {
+                const f32x4_t w = *(const f32x4_t *)(weight + c);
+#pragma unroll
+                for (int e = 0; e < 4; e++) dst[c + e] = from_f32<T>(v[j][e] * (inv * w[e]));
+            }
+        }
+    } else {
+        float ss = 0.f;
+        for (int c = threadIdx.x; c < width; c += kBlock) {
+            float v = src[c];
+            if (br) {
+                v += to_f32<B>(br[c]);
+                src[c] = v;
+            }
+            ss += v * v;
+        }
+        ss = block_sum<kWaves>(ss, scratch);   // its barriers also order the row's writes before the reads below
+        const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+        for (int c = threadIdx.x; c < width; c += kBlock) dst[c] = from_f32<T>(src[c] * (inv * weight[c]));
+    }
 }
 
 template <typename T>
 __global__ void __launch_bounds__(kBlock)
-swiglu_kernel(const T *__restrict__ gu, T *__restrict__ out, int rows, int inter) {
-    const size_t total = (size_t)rows * inter;
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (size_t)gridDim.x * kBlock) {
-        const size_t r = i / inter, j = i - r * inter;
-        const float g = to_f32<T>(gu[r * 2 * inter + j]);
-        const float u = to_f32<T>(gu[r * 2 * inter + inter + j]);
-        out[i] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+swiglu_kernel(const T *__restrict__ gu, T *__restrict__ out, int inter) {
+    const size_t r = blockIdx.y;
+    const T *g = gu + r * 2 * inter, *u = g + inter;
+    T *o = out + r * inter;
+    constexpr int V = 16 / sizeof(T);   // values per 16-byte access
+    typedef __attribute__((ext_vector_type(V))) T vec_t;
+    const int c = (blockIdx.x * kBlock + threadIdx.x) * V;
+    if (c + V <= inter && inter % V == 0) {
+        const vec_t gv = *(const vec_t *)(g + c), uv = *(const vec_t *)(u + c);
+        vec_t ov;
+#pragma unroll
+        for (int e = 0; e < V; e++) {
+            const float gf = to_f32<T>(gv[e]);
+            ov[e] = from_f32<T>(gf / (1.0f + expf(-gf)) * to_f32<T>(uv[e]));
+        }
+        *(vec_t *)(o + c) = ov;
+    } else {
+        for (int e = c; e < c + V && e < inter; e++) {
+            const float gf = to_f32<T>(g[e]);
+            o[e] = from_f32<T>(gf / (1.0f + expf(-gf)) * to_f32<T>(u[e]));
+        }
+    }
+}
+
+// residual[r, :] += branch[r, :], the sum in float32
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+add_residual_kernel(float *__restrict__ residual, const T *__restrict__ branch, size_t total) {
+    for (size_t i = ((size_t)blockIdx.x * kBlock + threadIdx.x) * 4; i < total; i += (size_t)gridDim.x * kBlock * 4) {
+        if (i + 4 <= total) {
+            f32x4_t r = *(const f32x4_t *)(residual + i);
+#pragma unroll
+            for (int j = 0; j < 4; j++) r[j] += to_f32<T>(branch[i + j]);
+            *(f32x4_t *)(residual + i) = r;
+        } else {
+            for (size_t j = i; j < total; j++) residual[j] += to_f32<T>(branch[j]);
+        }
     }
 }
 
@@ -125,36 +192,87 @@ extern "C" int fllm_embed(const int32_t *ids, const void *table, float *out, int
     return fllm_check_launch("embed");
 }
 
+namespace {
+
+template <typename T, typename B>
+void launch_rmsnorm(float *x, const B *branch, const int32_t *rows, const float *weight, T *out, int count, int width,
+                    float eps, hipStream_t stream) {
+    const bool vec = width % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)weight & 15) == 0;
+#define FLLM_NORM(V) hipLaunchKernelGGL((rmsnorm_kernel<T, B, V>), dim3(count), dim3(kBlock), 0, stream, x, branch, rows, weight, out, width, eps)
+    if (vec && width <= 1024) FLLM_NORM(1);
+    else if (vec && width <= 2048) FLLM_NORM(2);
+    else if (vec && width <= 4096) FLLM_NORM(4);
+    else if (vec && width <= 8192) FLLM_NORM(8);
+    else FLLM_NORM(0);
+#undef FLLM_NORM
+}
+
+template <typename B>
+int dispatch_rmsnorm(float *x, const B *branch, const int32_t *rows, const float *weight, void *out, int count, int width,
+                     float eps, int out_dtype, hipStream_t stream) {
+    if (out_dtype == FLLM_F32) launch_rmsnorm<float, B>(x, branch, rows, weight, (float *)out, count, width, eps, stream);
+    else if (out_dtype == FLLM_BF16) launch_rmsnorm<bf16_t, B>(x, branch, rows, weight, (bf16_t *)out, count, width, eps, stream);
+    else FLLM_REQUIRE(false, "rmsnorm: unknown dtype %d", out_dtype);
+    return fllm_check_launch("rmsnorm");
+}
+
+}  // namespace
+
 extern "C" int fllm_rmsnorm(const float *x, const int32_t *rows, const float *weight, void *out, int count, int width,
                             float eps, int out_dtype, hipStream_t stream) {
     FLLM_REQUIRE(count >= 0 && width > 0, "rmsnorm: bad sizes count=%d width=%d", count, width);
     FLLM_REQUIRE(eps > 0.f, "rmsnorm: eps must be positive");
     if (count == 0) return 0;
-    if (out_dtype == FLLM_F32)
-        hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(count), dim3(kBlock), 0, stream, x, rows, weight, (float *)out,
-                           width, eps);
-    else if (out_dtype == FLLM_BF16)
-        hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(count), dim3(kBlock), 0, stream, x, rows, weight, (bf16_t *)out,
-                           width, eps);
-    else
-        FLLM_REQUIRE(false, "rmsnorm: unknown dtype %d", out_dtype);
-    return fllm_check_launch("rmsnorm");
+    return dispatch_rmsnorm<float>(const_cast<float *>(x), nullptr, rows, weight, out, count, width, eps, out_dtype, stream);
+}
+
+extern "C" int fllm_add_rmsnorm(float *x, const void *branch, int branch_dtype, const float *weight, void *out, int count,
+                                int width, float eps, int out_dtype, hipStream_t stream) {
+    FLLM_REQUIRE(count >= 0 && width > 0, "add_rmsnorm: bad sizes count=%d width=%d", count, width);
+    FLLM_REQUIRE(eps > 0.f && branch != nullptr, "add_rmsnorm: eps must be positive and the branch given");
+    if (count == 0) return 0;
+    if (branch_dtype == FLLM_F32)
+        return dispatch_rmsnorm<float>(x, (const float *)branch, nullptr, weight, out, count, width, eps, out_dtype, stream);
+    FLLM_REQUIRE(branch_dtype == FLLM_BF16, "add_rmsnorm: unknown dtype %d", branch_dtype);
+    return dispatch_rmsnorm<bf16_t>(x, (const bf16_t *)branch, nullptr, weight, out, count, width, eps, out_dtype, stream);
 }
 
 extern "C" int fllm_swiglu(const void *gate_up, void *out, int rows, int inter, int dtype, hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && inter > 0, "swiglu: bad sizes rows=%d inter=%d", rows, inter);
     if (rows == 0) return 0;
-    const size_t total = (size_t)rows * inter;
-    const int grid = (int)((total + kBlock - 1) / kBlock < 65535 ? (total + kBlock - 1) / kBlock : 65535);
-    if (dtype == FLLM_F32)
-        hipLaunchKernelGGL(swiglu_kernel<float>, dim3(grid), dim3(kBlock), 0, stream, (const float *)gate_up, (float *)out,
-                           rows, inter);
-    else if (dtype == FLLM_BF16)
-        hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3(grid), dim3(kBlock), 0, stream, (const bf16_t *)gate_up,
-                           (bf16_t *)out, rows, inter);
-    else
-        FLLM_REQUIRE(false, "swiglu: unknown dtype %d", dtype);
+    FLLM_REQUIRE(rows <= 65535 * 32, "swiglu: too many rows");
+    for (int r0 = 0; r0 < rows; r0 += 65535) {   // grid.y is limited to 65535
+        const int nr = rows - r0 < 65535 ? rows - r0 : 65535;
+        if (dtype == FLLM_F32) {
+            const dim3 grid((inter + kBlock * 4 - 1) / (kBlock * 4), nr);
+            hipLaunchKernelGGL(swiglu_kernel<float>, grid, dim3(kBlock), 0, stream, (const float *)gate_up + (size_t)r0 * 2 * inter,
+                               (float *)out + (size_t)r0 * inter, inter);
+        } else if (dtype == FLLM_BF16) {
+            const dim3 grid((inter + kBlock * 8 - 1) / (kBlock * 8), nr);
+            hipLaunchKernelGGL(swiglu_kernel<bf16_t>, grid, dim3(kBlock), 0, stream,
+                               (const bf16_t *)gate_up + (size_t)r0 * 2 * inter, (bf16_t *)out + (size_t)r0 * inter, inter);
+        } else {
+            FLLM_REQUIRE(false, "swiglu: unknown dtype %d", dtype);
+        }
+    }
     return fllm_check_launch("swiglu");
+}
+
+extern "C" int fllm_add_residual(float *residual, const void *branch, int rows, int width, int dtype, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && width > 0, "add_residual: bad sizes rows=%d width=%d", rows, width);
+    FLLM_REQUIRE(((uintptr_t)residual & 15) == 0, "add_residual: the residual must be 16-byte aligned");
+    if (rows == 0) return 0;
+    const size_t total = (size_t)rows * width;
+    const size_t groups = (total + 4 * kBlock - 1) / (4 * kBlock);
+    const int grid = (int)(groups < 16384 ? groups : 16384);
+    if (dtype == FLLM_F32)
+        hipLaunchKernelGGL(add_residual_kernel<float>, dim3(grid), dim3(kBlock), 0, stream, residual, (const float *)branch, total);
+    else if (dtype == FLLM_BF16)
+        hipLaunchKernelGGL(add_residual_kernel<bf16_t>, dim3(grid), dim3(kBlock), 0, stream, residual, (const bf16_t *)branch,
+                           total);
+    else
+        FLLM_REQUIRE(false, "add_residual: unknown dtype %d", dtype);
+    return fllm_check_launch("add_residual");
 }
 
 extern "C" int fllm_rope_kv_store(void *qkv, const int32_t *row_pos, const int32_t *row_seg, const int32_t *tables,

@@ -55,6 +55,8 @@ def load_library(build_if_missing: bool = True):
         "fllm_rmsnorm": [c_void, c_void, c_void, c_void, c_int, c_int, c_float, c_int, c_void],
         "fllm_linear": [c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_swiglu": [c_void, c_void, c_int, c_int, c_int, c_void],
+        "fllm_add_residual": [c_void, c_void, c_int, c_int, c_int, c_void],
+        "fllm_add_rmsnorm": [c_void, c_void, c_int, c_void, c_void, c_int, c_int, c_float, c_int, c_void],
         "fllm_rope_kv_store": [c_void, c_void, c_void, c_void, c_int, c_void, c_void, c_int, c_void, c_void, c_int,
                                c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_attention": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_int,
@@ -99,12 +101,18 @@ def _dense(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
 
 
 class Ops:
-    """Launches kernels on the current torch stream of the tensors' device."""
+    """Launches kernels on the current torch stream of the tensors' device.
 
-    def __init__(self):
+    `library_gemm_from`: bfloat16 products of at least this many rows (prompt portions, large
+    decode batches) go to the vendor's GEMM library through `torch.matmul`, as the reference sends
+    its prompt-sized dense products to a library (rust/engine/cuda/cublaslt_gemm.cu:1-20).  None:
+    every product runs the hand-written kernels."""
+
+    def __init__(self, library_gemm_from: Optional[int] = 17):
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible: the engine runs on gfx950 only")
         self.lib = load_library()
+        self.library_gemm_from = library_gemm_from
 
     def set_fast_kernels(self, on: bool) -> None:
         """Off: bfloat16 calls run the plain kernels (tests compare the two)."""
@@ -143,6 +151,19 @@ class Ops:
                                           _DTYPE_CODE[out.dtype], self._stream()))
         return out
 
+    def add_rmsnorm(self, x: torch.Tensor, branch: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor) -> torch.Tensor:
+        """x += branch (float32 sum, in place), out = rmsnorm(x): the residual add and the norm after it in one pass."""
+        rows, width = x.shape
+        _dense(x, "x", torch.float32)
+        _dense(branch, "branch", None, (rows, width))
+        _need(branch.dtype in _DTYPE_CODE, f"branch dtype {branch.dtype} unsupported")
+        _dense(weight, "weight", torch.float32, (width,))
+        _dense(out, "out", None, (rows, width))
+        _need(out.dtype in _DTYPE_CODE, f"out dtype {out.dtype} unsupported")
+        self._check(self.lib.fllm_add_rmsnorm(_ptr(x), _ptr(branch), _DTYPE_CODE[branch.dtype], _ptr(weight), _ptr(out), rows,
+                                              width, float(eps), _DTYPE_CODE[out.dtype], self._stream()))
+        return out
+
     def linear(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
                accumulate: bool = False) -> torch.Tensor:
         """out = x @ w.T (+ bias); `accumulate` adds into a float32 `out` instead of storing."""
@@ -164,6 +185,13 @@ class Ops:
             mode = OUT_STORE_F32
         if bias is not None:
             _dense(bias, "bias", torch.float32, (N,))
+        if (self.library_gemm_from is not None and M >= self.library_gemm_from and x.dtype == torch.bfloat16
+                and bias is None and mode != OUT_STORE_F32):
+            if mode == OUT_STORE:
+                torch.matmul(x, w.t(), out=out)
+            else:
+                self.add_residual(out, torch.matmul(x, w.t()))
+            return out
         ldx = x.stride(0) if M > 1 else K
         ldo = out.stride(0) if M > 1 else N
         self._check(self.lib.fllm_linear(_ptr(x), ldx, _ptr(w), _ptr(bias), _ptr(out), ldo, M, N, K, _DTYPE_CODE[x.dtype],
@@ -226,6 +254,15 @@ class Ops:
             _ptr(tables), tables.shape[1], _ptr(cos), _ptr(sin), rope_dims, _ptr(k_pages), _ptr(v_pages), M, heads, kv_heads,
             head_dim, K, page_size, 1 if store else 0, self._stream()))
         return q_out
+
+    def add_residual(self, residual: torch.Tensor, branch: torch.Tensor) -> torch.Tensor:
+        """residual += branch, summed in float32."""
+        _dense(residual, "residual", torch.float32)
+        _dense(branch, "branch", None, tuple(residual.shape))
+        _need(branch.dtype in _DTYPE_CODE and residual.dim() == 2, "add_residual takes matrices of float32 / bfloat16")
+        self._check(self.lib.fllm_add_residual(_ptr(residual), _ptr(branch), residual.shape[0], residual.shape[1],
+                                               _DTYPE_CODE[branch.dtype], self._stream()))
+        return residual
 
     def swiglu(self, gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         rows, two_i = gate_up.shape

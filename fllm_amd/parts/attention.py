@@ -86,7 +86,7 @@ class PagedAttention(Mixer):
     def cache_need(self):
         return KVNeed(self.kv_heads, self.head_dim, self.window)
 
-    def forward(self, ctx, h, residual, binding):
+    def forward(self, ctx, h, residual, binding, branch=None):
         rt, ops = self.rt, self.rt.ops
         rows = h.shape[0]
         nh, nkv, d = self.heads, self.kv_heads, self.head_dim
@@ -100,7 +100,7 @@ class PagedAttention(Mixer):
         ops.rope_kv_store(qkv, ctx.row_pos, ctx.row_seg, tables, cos, sin,
                           binding.k_pages if binding.writes else None, binding.v_pages if binding.writes else None,
                           nh, nkv, d, dims, pairing, binding.page_size)
-        self._attend_and_project(ctx, qkv[:, : nh * d], residual, binding)
+        self._attend_and_project(ctx, qkv[:, : nh * d], residual, binding, branch=branch)
 
     def forward_from_residual(self, ctx, residual, norm, binding) -> bool:
         """Decode-sized steps in bfloat16: the norm before the mixer, the q/k/v product, rotary and the
@@ -124,7 +124,20 @@ class PagedAttention(Mixer):
         self._attend_and_project(ctx, q, residual, binding)
         return True
 
-    def _attend_and_project(self, ctx, q, residual, binding):
+    def forward_branch(self, ctx, h, binding):
+        """The mixer's output as a tensor of its own instead of a sum into the residual stream, when
+        that lets the block fold the residual add into the next norm (large bfloat16 steps whose
+        products go to the GEMM library, which has no residual epilogue).  None: not taken."""
+        rt, ops = self.rt, self.rt.ops
+        rows = h.shape[0]
+        start = getattr(ops, "library_gemm_from", None)
+        if rt.dtype != torch.bfloat16 or start is None or rows < start or self.b_o is not None:
+            return None
+        branch = rt.empty((rows, self.hidden))
+        self.forward(ctx, h, None, binding, branch=branch)
+        return branch
+
+    def _attend_and_project(self, ctx, q, residual, binding, branch=None):
         rt, ops = self.rt, self.rt.ops
         rows = q.shape[0]
         nh, nkv, d = self.heads, self.kv_heads, self.head_dim
@@ -134,7 +147,10 @@ class PagedAttention(Mixer):
                       out, nh, nkv, d, binding.page_size, self.scale, self.window, ctx.max_context,
                       uniform_rows=1 if ctx.uniform_rows else 0,
                       workspace=ctx.attention_workspace(rt, rows, nh, nkv, d))
-        ops.linear(out, self.w_o, residual, bias=self.b_o, accumulate=True)
+        if branch is not None:
+            ops.linear(out, self.w_o, branch, bias=self.b_o)
+        else:
+            ops.linear(out, self.w_o, residual, bias=self.b_o, accumulate=True)
 
 
 register_part("mixer", "attention", PagedAttention)

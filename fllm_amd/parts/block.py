@@ -16,9 +16,18 @@ class PreNormBlock(Block):
 
     def forward(self, ctx, residual, binding):
         # a part may take the residual stream and the norm before it in one fused kernel
+        h = None
         fused = getattr(self.mixer, "forward_from_residual", None)
         if fused is None or not fused(ctx, residual, self.mixer_norm, binding):
             h = self.mixer_norm.forward(ctx, residual)
+            # a mixer may hand back its output instead of adding it: the add then rides on the next norm
+            as_branch = getattr(self.mixer, "forward_branch", None)
+            add_norm = getattr(self.feed_forward_norm, "add_forward", None)
+            branch = as_branch(ctx, h, binding) if as_branch is not None and add_norm is not None else None
+            if branch is not None:
+                h = add_norm(ctx, residual, branch)
+                self.feed_forward.forward(ctx, h, residual)
+                return
             self.mixer.forward(ctx, h, residual, binding)
         fused = getattr(self.feed_forward, "forward_from_residual", None)
         if fused is None or not fused(ctx, residual, self.feed_forward_norm):

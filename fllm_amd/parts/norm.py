@@ -26,4 +26,11 @@ class RMSNorm(Norm):
         return self.rt.ops.rmsnorm(x, self.weight, self.eps, out, rows=rows)
 
 
+    def add_forward(self, ctx, x, branch, out=None):
+        """x += branch, then the norm of the sum: one pass over the row."""
+        if out is None:
+            out = self.rt.empty((x.shape[0], self.size))
+        return self.rt.ops.add_rmsnorm(x, branch, self.weight, self.eps, out)
+
+
 register_part("norm", "rms", RMSNorm)

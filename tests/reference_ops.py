@@ -73,6 +73,14 @@ class ReferenceOps:
             v_pages.copy_(vp.to(v_pages.dtype))
         return q_out
 
+    def add_rmsnorm(self, x, branch, weight, eps, out):
+        x.add_(branch.to(x.dtype))
+        return self.rmsnorm(x, weight, eps, out)
+
+    def add_residual(self, residual, branch):
+        residual.add_(branch.to(residual.dtype))
+        return residual
+
     def swiglu(self, gate_up, out):
         inter = gate_up.shape[1] // 2
         g, u = gate_up[:, :inter].double(), gate_up[:, inter:].double()

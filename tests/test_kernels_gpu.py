@@ -18,7 +18,13 @@ DEV = "cuda:0"
 @pytest.fixture(scope="module")
 def ops():
     from fllm_amd.kernels import Ops
-    return Ops()
+    return Ops(library_gemm_from=None)      # the hand-written kernels at every size
+
+
+@pytest.fixture(scope="module")
+def library_ops():
+    from fllm_amd.kernels import Ops
+    return Ops()                            # large bfloat16 products through the GEMM library
 
 
 @pytest.fixture(scope="module")
@@ -75,6 +81,22 @@ def test_rmsnorm(ops, ref, out_dtype, rows, width, eps):
     close(got, want[sel.long()], tol, tol * 1e-3, "rmsnorm rows")
 
 
+@pytest.mark.parametrize("branch_dtype,out_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16)])
+@pytest.mark.parametrize("rows,width", [(1, 64), (13, 4096), (5, 5140), (3, 8192), (2, 9000), (4, 1001)])
+def test_add_rmsnorm(ops, ref, branch_dtype, out_dtype, rows, width):
+    g = gen(41)
+    x = torch.randn(rows, width, generator=g) * 2
+    branch = torch.randn(rows, width, generator=g).to(branch_dtype)
+    w = 1.0 + 0.1 * torch.randn(width, generator=g)
+    x_ref = x.double()
+    want = ref.add_rmsnorm(x_ref, branch, w, 1e-5, torch.empty(rows, width, dtype=torch.float64))
+    x_gpu = x.to(DEV)
+    got = ops.add_rmsnorm(x_gpu, branch.to(DEV), w.to(DEV), 1e-5, torch.empty(rows, width, dtype=out_dtype, device=DEV))
+    assert torch.equal(x_gpu.cpu(), x + branch.float())
+    tol = 2e-6 if out_dtype == torch.float32 else BF16_EPS
+    close(got, want, tol, tol * 1e-3, "add_rmsnorm")
+
+
 def test_rmsnorm_row_is_the_same_alone_and_in_a_batch(ops):
     g = gen(3)
     x = torch.randn(9, 1000, generator=g).to(DEV)
@@ -84,7 +106,7 @@ def test_rmsnorm_row_is_the_same_alone_and_in_a_batch(ops):
     assert torch.equal(full[4:5], one)
 
 
-def _linear_case(ops, ref, dtype, M, N, K, mode, bias, seed=4):
+def _linear_case(ops, ref, dtype, M, N, K, mode, bias, seed=4, branch_rounded=False):
     g = gen(seed)
     x = (torch.randn(M, K, generator=g)).to(dtype)
     w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dtype)
@@ -102,6 +124,8 @@ def _linear_case(ops, ref, dtype, M, N, K, mode, bias, seed=4):
     mag = (x.double().abs() @ w.double().abs().T).max().item()
     atol = 4e-7 * mag + 1e-6
     rtol = BF16_EPS if out_dtype == torch.bfloat16 else 1e-6
+    if branch_rounded:      # the library product is rounded to bfloat16 before it is added
+        atol += BF16_EPS * (want - base.double()).abs().max().item()
     close(out, want, rtol, atol + (BF16_EPS * 1e-2 if out_dtype == torch.bfloat16 else 0), f"linear {dtype} M{M} N{N} K{K} {mode}")
 
 
@@ -130,6 +154,22 @@ PLAIN = [(3, 50, 100), (70, 64, 36)]      # K not a multiple of 8: the plain ker
 @pytest.mark.parametrize("mode,bias", [("store", False), ("f32", True), ("add", True)])
 def test_linear_bf16(ops, ref, M, N, K, mode, bias):
     _linear_case(ops, ref, torch.bfloat16, M, N, K, mode, bias)
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 128, 128), (64, 4096, 4096), (200, 6144, 4096), (300, 130, 136)])
+@pytest.mark.parametrize("mode,bias", [("store", False), ("add", False), ("f32", False), ("add", True)])
+def test_linear_bf16_library_path(library_ops, ref, M, N, K, mode, bias):
+    _linear_case(library_ops, ref, torch.bfloat16, M, N, K, mode, bias, branch_rounded=(mode == "add" and not bias))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,width", [(1, 64), (13, 4099), (300, 4096)])
+def test_add_residual(ops, dtype, rows, width):
+    g = gen(40)
+    residual = torch.randn(rows, width, generator=g)
+    branch = torch.randn(rows, width, generator=g).to(dtype)
+    got = ops.add_residual(residual.to(DEV), branch.to(DEV))
+    assert torch.equal(got.cpu(), residual + branch.float())
 
 
 def test_linear_bf16_strided_input(ops, ref):
