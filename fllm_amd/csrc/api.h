@@ -14,6 +14,8 @@ const char *fllm_last_error(void);
 int fllm_abi_version(void);
 // 0: bfloat16 calls use the plain kernels only (for comparing them with the MFMA kernels); default 1
 void fllm_set_fast_kernels(int on);
+// Switches a kernel variant (for measurements and tests): "attention.tile32" 0/1.  0 on success.
+int fllm_set_option(const char *name, int value);
 
 // out[r, :] = scale * table[ids[r], :]            out: float32 [rows, width]
 int fllm_embed(const int32_t *ids, const void *table, float *out, int rows, int width, int vocab, int table_dtype,

@@ -14,6 +14,7 @@
 //
 //   tile kernel    portions of prompts: a workgroup takes up to 64 (token, head-of-group) rows of
 //                  one segment and one key/value head; keys and values go through LDS in tiles of 64.
+//   tile32 kernel  long portions: 128 rows per workgroup on 32x32x16 products (described at the kernel).
 //   decode kernel  one row per segment: a workgroup takes (row, key/value head, context split), its
 //                  sixteen waves stride over 32-key blocks loading K and V^T straight into MFMA
 //                  operands; long contexts of small batches are split and merged by a second kernel.
@@ -39,6 +40,7 @@ struct AttnArgs {
     int num_segs;
     bf16_t *out;
     int rows, heads, kv_heads, page_size;
+    int ps_shift;   // page_size = 1 << ps_shift
     float scale_log2;
     int window;
     float *ws_ml;   // [rows, heads, splits, 2]
@@ -138,7 +140,7 @@ attn_tile_kernel(AttnArgs p) {
     const int prow = rvalid ? pos0 + tq : -1;
     const int head = kvh * G + hg;
     const int lo_r = (p.window > 0 && prow - p.window + 1 > 0) ? prow - p.window + 1 : 0;
-    const int ps = p.page_size, nkv = p.kv_heads;
+    const int ps = p.page_size, psh = p.ps_shift, pmask = ps - 1, nkv = p.kv_heads;
 
     bf16x8_t qf[KD];
 #pragma unroll
@@ -150,7 +152,8 @@ attn_tile_kernel(AttnArgs p) {
     const int lo_tile = (p.window > 0 && pos0 - p.window + 1 > 0) ? pos0 - p.window + 1 : 0;
     const int kbegin = (lo_tile / KT) * KT;
     const int32_t *tbl = p.tables + (size_t)seg * p.table_stride;
-    const int cpp = ps / 8;   // 16-byte chunks per value row of a page
+    const int cps = psh - 3;   // log2 of the 16-byte chunks per value row of a page
+    constexpr int LD = D == 32 ? 5 : D == 64 ? 6 : 7;   // log2(D)
 
     f32x4_t o[DT];
 #pragma unroll
@@ -164,19 +167,19 @@ attn_tile_kernel(AttnArgs p) {
             const int kabs = k0 + key;
             bf16x8_t v = zero8();
             if (kabs >= lo_tile && kabs <= p_last) {
-                const int page = tbl[kabs / ps], off = kabs % ps;
+                const int page = tbl[kabs >> psh], off = kabs & pmask;
                 v = *(const bf16x8_t *)(p.kp + (((size_t)page * nkv + kvh) * ps + off) * D + dc * 8);
             }
             *(bf16x8_t *)(Ks + key * KP + dc * 8) = v;
         }
         for (int ch = threadIdx.x; ch < D * KT / 8; ch += kThreads) {
-            const int pg = ch / (D * cpp), rem = ch % (D * cpp);
-            const int d = rem / cpp, hc = rem % cpp;
-            const int koff = pg * ps + hc * 8;
+            const int pg = ch >> (LD + cps), rem = ch & ((D << cps) - 1);
+            const int d = rem >> cps, hc = rem & ((1 << cps) - 1);
+            const int koff = (pg << psh) + hc * 8;
             const int kabs = k0 + koff;
             bf16x8_t v = zero8();
             if (kabs + 7 >= lo_tile && kabs <= p_last) {
-                const int page = tbl[kabs / ps];
+                const int page = tbl[kabs >> psh];
                 v = *(const bf16x8_t *)(p.vp + (((size_t)page * nkv + kvh) * D + d) * ps + hc * 8);
                 if (kabs + 7 > p_last) {   // slots past the last token hold whatever an earlier request left
 #pragma unroll
@@ -238,6 +241,219 @@ attn_tile_kernel(AttnArgs p) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// tile kernel on 32x32x16 products: 128 (token, head-of-group) rows per workgroup
+// ---------------------------------------------------------------------------------------------
+// v_mfma_f32_32x32x16_bf16: A lane l holds A[m = l%32][k = 8*(l/32) .. +7], B lane l holds
+// B[k = 8*(l/32) .. +7][n = l%32], D lane l holds D[m = 8*(i/4) + 4*(l/32) + i%4][n = l%32], i = 0..15.
+// A wave owns 32 query rows (n).  The A rows of a 32-key block of S^T are assigned to keys so that
+// the sixteen sums of a lane, taken eight at a time, are the keys 16 s + 8 (l/32) .. + 7: the B
+// operand of the P V product for that half block, with no exchange between lanes:
+//   A row a = 16 s + 8 b + 4 h + i  <->  key 16 s + 8 h + 4 b + i      (s, b, h in {0, 1}, i in 0..3)
+// Each K and V fragment read from LDS feeds 32 query rows instead of 16, the next tile is on its way
+// from global memory into registers while the current one is multiplied, the scale is folded into
+// the exponent (one fused multiply-add per score), tiles wholly below the diagonal skip the mask,
+// and the outputs are rescaled only when a row's maximum moved.
+template <int D>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+attn_tile32_kernel(AttnArgs p) {
+    constexpr int KT = 64;          // keys per tile
+    constexpr int KP = D + 8;       // pitch of a key row in LDS
+    constexpr int VP = KT + 8;      // pitch of a value row (one head_dim lane, KT keys) in LDS
+    constexpr int DS = D / 16, DB = D / 32;
+    constexpr int CH = KT * D / 8 / kThreads;   // 16-byte chunks per thread and tile (K and V each)
+    constexpr int LD = D == 64 ? 6 : 7;         // log2(D)
+    static_assert(CH >= 1 && (D == 64 || D == 128), "this tiling takes head_dim 64 or 128");
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KP];
+    __shared__ __attribute__((aligned(16))) bf16_t Vs[D * VP];
+    __shared__ int s_tile[2];
+    const int G = p.heads / p.kv_heads;
+    const int TQ = 128 / G;         // tokens per tile
+    if (threadIdx.x == 0) {
+        int b = blockIdx.x, seg = -1, t0 = 0;
+        for (int s = 0; s < p.num_segs; s++) {
+            const int n = p.seg_start[s + 1] - p.seg_start[s];
+            const int nt = (n + TQ - 1) / TQ;
+            if (b < nt) {
+                seg = s;
+                t0 = nt - 1 - b;    // the tiles with the longest contexts start first
+                break;
+            }
+            b -= nt;
+        }
+        s_tile[0] = seg;
+        s_tile[1] = t0;
+    }
+    __syncthreads();
+    const int seg = s_tile[0];
+    if (seg < 0) return;
+    const int row0 = p.seg_start[seg] + s_tile[1] * TQ;
+    const int ntok = min(TQ, p.seg_start[seg + 1] - row0);
+    const int pos0 = p.row_pos[row0];
+    const int kvh = blockIdx.y;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int q = lane & 31, h = lane >> 5;
+    const int rr = wave * 32 + q;
+    const int tq = rr / G, hg = rr - tq * G;
+    const bool rvalid = tq < ntok;
+    const int prow = rvalid ? pos0 + tq : -1;
+    const int head = kvh * G + hg;
+    const int lo_r = (p.window > 0 && prow - p.window + 1 > 0) ? prow - p.window + 1 : 0;
+    const int ps = p.page_size, psh = p.ps_shift, pmask = ps - 1, nkv = p.kv_heads;
+    const int cps = psh - 3;        // log2 of the 16-byte chunks per value row of a page
+
+    bf16x8_t qf[DS];
+#pragma unroll
+    for (int ds = 0; ds < DS; ds++)
+        qf[ds] = rvalid ? *(const bf16x8_t *)(p.q + (size_t)(row0 + tq) * p.q_stride + (size_t)head * D + ds * 16 + h * 8)
+                        : zero8();
+
+    const int p_last = pos0 + ntok - 1;
+    const int lo_tile = (p.window > 0 && pos0 - p.window + 1 > 0) ? pos0 - p.window + 1 : 0;
+    // from this key on every row of the workgroup sees every key up to pos0 (no window edge inside)
+    const int lo_all = (p.window > 0 && p_last - p.window + 1 > 0) ? p_last - p.window + 1 : 0;
+    const int kbegin = (lo_tile / KT) * KT;
+    const int32_t *tbl = p.tables + (size_t)seg * p.table_stride;
+
+    // What of a chunk's address does not change from tile to tile (tiles start at multiples of 64 >= page size)
+    int k_key[CH], v_koff[CH];
+    size_t k_in_page[CH], v_in_page[CH], k_lds[CH], v_lds[CH];
+#pragma unroll
+    for (int c = 0; c < CH; c++) {
+        const int ch = threadIdx.x + c * kThreads;
+        const int key = ch >> (LD - 3), dc = ch & (D / 8 - 1);
+        k_key[c] = key;
+        k_in_page[c] = ((size_t)kvh * ps + (key & pmask)) * D + dc * 8;
+        k_lds[c] = key * KP + dc * 8;
+        const int pg = ch >> (LD + cps), rem = ch & ((D << cps) - 1);
+        const int d = rem >> cps, hc = rem & ((1 << cps) - 1);
+        v_koff[c] = (pg << psh) + hc * 8;
+        v_in_page[c] = ((size_t)kvh * D + d) * ps + hc * 8;
+        v_lds[c] = d * VP + v_koff[c];
+    }
+    const size_t page_elems = (size_t)nkv * ps * D;
+
+    bf16x8_t kreg[CH], vreg[CH];
+    auto fetch = [&](int k0) {   // tile k0 .. k0 + 63 from the pages into registers
+        const bool inside = k0 >= lo_tile && k0 + KT - 1 <= p_last;   // no edge of the context in this tile
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int kabs = k0 + k_key[c];
+            bf16x8_t v = zero8();
+            if (inside || (kabs >= lo_tile && kabs <= p_last))
+                v = *(const bf16x8_t *)(p.kp + (size_t)tbl[kabs >> psh] * page_elems + k_in_page[c]);
+            kreg[c] = v;
+            const int vabs = k0 + v_koff[c];
+            v = zero8();
+            if (inside || (vabs + 7 >= lo_tile && vabs <= p_last)) {
+                v = *(const bf16x8_t *)(p.vp + (size_t)tbl[vabs >> psh] * page_elems + v_in_page[c]);
+                if (!inside && vabs + 7 > p_last) {   // slots past the last token hold whatever an earlier request left
+#pragma unroll
+                    for (int e = 0; e < 8; e++)
+                        if (vabs + e > p_last) v[e] = (bf16_t)0.0f;
+                }
+            }
+            vreg[c] = v;
+        }
+    };
+
+    f32x16_t o[DB];
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[db][i] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;   // the running maximum is kept in raw units (before the scale)
+    const float sc = p.scale_log2;
+    // A row q of a 32-key block is this key of the block (see the table above)
+    const int a_key = 16 * (q >> 4) + 8 * ((q >> 2) & 1) + 4 * ((q >> 3) & 1) + (q & 3);
+
+    fetch(kbegin);
+    for (int k0 = kbegin; k0 <= p_last; k0 += KT) {
+        __syncthreads();   // the previous tile has been read
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            *(bf16x8_t *)(Ks + k_lds[c]) = kreg[c];
+            *(bf16x8_t *)(Vs + v_lds[c]) = vreg[c];
+        }
+        __syncthreads();
+        if (k0 + KT <= p_last) fetch(k0 + KT);   // in flight while this tile is multiplied
+
+        f32x16_t s[2];
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) s[rb][i] = 0.f;
+            const bf16_t *krow = Ks + (rb * 32 + a_key) * KP + h * 8;
+#pragma unroll
+            for (int ds = 0; ds < DS; ds++)
+                s[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t *)(krow + ds * 16), qf[ds], s[rb], 0, 0, 0);
+        }
+        // tiles wholly below the diagonal and above every window edge need no mask (the same for all rows here)
+        if (!(k0 + KT - 1 <= pos0 && k0 >= lo_all)) {
+#pragma unroll
+            for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int key = k0 + rb * 32 + 16 * (i >> 3) + 8 * h + (i & 7);
+                    if (!(key <= prow && key >= lo_r)) s[rb][i] = -INFINITY;   // prow = -1 for rows outside the segment
+                }
+        }
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, s[rb][i]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+        const float m_new = fmaxf(m_run, tmax);
+        const float mc = m_new == -INFINITY ? 0.f : m_new * sc;   // nothing seen yet: exp2(-inf - 0) = 0 below
+        const float alpha = m_run == -INFINITY ? 0.f : fast_exp2(m_run * sc - mc);
+        float psum = 0.f;
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const float pv = fast_exp2(fmaf(s[rb][i], sc, -mc));   // masked: exp2(-inf) = 0
+                s[rb][i] = pv;
+                psum += pv;
+            }
+        psum += __shfl_xor(psum, 32, kWave);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (__any(alpha != 1.0f)) {   // once the maximum has settled the outputs need no rescaling
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) o[db][i] *= alpha;
+        }
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) {
+                bf16x8_t pf;
+#pragma unroll
+                for (int e = 0; e < 8; e++) pf[e] = (bf16_t)s[rb][8 * s2 + e];
+#pragma unroll
+                for (int db = 0; db < DB; db++) {
+                    const bf16x8_t a = *(const bf16x8_t *)(Vs + (db * 32 + q) * VP + rb * 32 + 16 * s2 + 8 * h);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf, o[db], 0, 0, 0);
+                }
+            }
+    }
+    if (rvalid) {
+        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+        bf16_t *dst = p.out + ((size_t)(row0 + tq) * p.heads + head) * D + 4 * h;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                bf16x4_t v;
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[i] = (bf16_t)(o[db][4 * j + i] * inv);
+                *(bf16x4_t *)(dst + db * 32 + 8 * j) = v;
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // decode kernel
 // ---------------------------------------------------------------------------------------------
 template <int D, int WAVES>
@@ -260,7 +476,7 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
     const int head = kvh * G + (hg < G ? hg : 0);
     const int n = seg >= 0 ? p.row_pos[row] + 1 : 0;
     const int lo = (p.window > 0 && n - p.window > 0) ? n - p.window : 0;
-    const int ps = p.page_size, nkv = p.kv_heads;
+    const int ps = p.page_size, psh = p.ps_shift, pmask = ps - 1, nkv = p.kv_heads;
     const int begin = (lo / 32) * 32 + split * p.keys_per_split;
     const int end = min(begin + p.keys_per_split, n);
     const int32_t *tbl = p.tables + (size_t)(seg >= 0 ? seg : 0) * p.table_stride;
@@ -283,18 +499,18 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
         const bool gload = grp < n && grp + 8 > lo;
         const int vkey = kb + g * 8;
         const bool vload = vkey < n && vkey + 8 > lo;
-        const int kpage = gload ? tbl[grp / ps] : 0;
-        const int vpage = vload ? tbl[vkey / ps] : 0;
+        const int kpage = gload ? tbl[grp >> psh] : 0;
+        const int vpage = vload ? tbl[vkey >> psh] : 0;
         bf16x8_t kf[2][KD], vf[DT];
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int key = grp + j * 4 + (c & 3);
             const bool valid = gload && key >= lo && key < n;
-            const bf16_t *kr = p.kp + (((size_t)kpage * nkv + kvh) * ps + (key % ps)) * D + g * 8;
+            const bf16_t *kr = p.kp + (((size_t)kpage * nkv + kvh) * ps + (key & pmask)) * D + g * 8;
 #pragma unroll
             for (int kk = 0; kk < KD; kk++) kf[j][kk] = valid ? *(const bf16x8_t *)(kr + kk * 32) : zero8();
         }
-        const bf16_t *vr = p.vp + (((size_t)vpage * nkv + kvh) * D + c) * ps + (vkey % ps);
+        const bf16_t *vr = p.vp + (((size_t)vpage * nkv + kvh) * D + c) * ps + (vkey & pmask);
 #pragma unroll
         for (int dt = 0; dt < DT; dt++) vf[dt] = vload ? *(const bf16x8_t *)(vr + (size_t)dt * 16 * ps) : zero8();
 
@@ -396,7 +612,7 @@ void decode_split_plan(int rows, int kv_heads, int qtiles, int max_context, int 
     const long base = (long)rows * kv_heads * qtiles;
     const long span = (long)max_context + 31;   // the first split starts at a multiple of 32 at or below the first key
     long want = 1;
-    if (span > 2048 && base < 256) {
+    if (max_context > 2048 && base < 256) {
         want = (256 + base - 1) / base;
         const long most = (span + 2047) / 2048;
         if (want > most) want = most;
@@ -448,6 +664,12 @@ int launch(const AttnArgs &a, int uniform_rows, int max_context, void *workspace
                                a.heads, p.splits);
         return fllm_check_launch("attention_decode");
     }
+    if (D >= 64 && G <= 64 && a.rows >= 96 && fllm_option_tile32()) {   // long portions: 128 rows per workgroup on 32x32x16 products
+        const int TQ = 128 / G;
+        const int tiles = (a.rows + TQ - 1) / TQ + a.num_segs;   // upper bound; surplus workgroups leave at once
+        hipLaunchKernelGGL(attn_tile32_kernel<(D >= 64 ? D : 64)>, dim3(tiles, a.kv_heads), dim3(kThreads), 0, stream, a);
+        return fllm_check_launch("attention_tile32");
+    }
     const int TQ = 64 / G;
     const int tiles = (a.rows + TQ - 1) / TQ + a.num_segs;   // upper bound; surplus workgroups leave at once
     hipLaunchKernelGGL(attn_tile_kernel<D>, dim3(tiles, a.kv_heads), dim3(kThreads), 0, stream, a);
@@ -492,6 +714,7 @@ int fllm_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, c
     a.heads = heads;
     a.kv_heads = kv_heads;
     a.page_size = page_size;
+    a.ps_shift = page_size == 8 ? 3 : page_size == 16 ? 4 : page_size == 32 ? 5 : 6;
     a.scale_log2 = scale * kLog2e;
     a.window = window;
     a.ws_ml = nullptr;

@@ -374,8 +374,10 @@ int launch_resident(SkinnyArgs a, hipStream_t stream) {
     const int n_out = EPI == EPI_SWIGLU ? a.N / 2 : a.N;
     const int ntiles = (n_out + 15) / 16;
     const int per_cu = smem <= 76 * 1024 ? 2 : 1;
-    int grid = device_cus() * per_cu;
-    if (grid > ntiles) grid = ntiles;
+    // every workgroup takes the same number of tiles (or one fewer): 896 tiles on 512 slots run as 448 x 2
+    const int slots = device_cus() * per_cu;
+    const int rounds = (ntiles + slots - 1) / slots;
+    const int grid = (ntiles + rounds - 1) / rounds;
     static bool attribute_set = false;   // more than the default 64 KiB of dynamic LDS has to be asked for once
     if (!attribute_set) {
         const hipError_t e = hipFuncSetAttribute((const void *)skinny_resident_kernel<PRO, EPI>,

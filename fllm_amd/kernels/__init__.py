@@ -74,6 +74,8 @@ def load_library(build_if_missing: bool = True):
         fn.restype = c_int
     lib.fllm_fused_decode_supported.argtypes = [c_int, c_int]
     lib.fllm_fused_decode_supported.restype = c_int
+    lib.fllm_set_option.argtypes = [ctypes.c_char_p, c_int]
+    lib.fllm_set_option.restype = c_int
     lib.fllm_set_fast_kernels.argtypes = [c_int]
     lib.fllm_set_fast_kernels.restype = None
     lib.fllm_attention_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int, c_int]
@@ -117,6 +119,10 @@ class Ops:
     def set_fast_kernels(self, on: bool) -> None:
         """Off: bfloat16 calls run the plain kernels (tests compare the two)."""
         self.lib.fllm_set_fast_kernels(1 if on else 0)
+
+    def set_option(self, name: str, value: int) -> None:
+        """Switches a kernel variant, for measurements and for tests that compare variants."""
+        self._check(self.lib.fllm_set_option(name.encode(), int(value)))
 
     def _check(self, code: int) -> None:
         if code != 0:

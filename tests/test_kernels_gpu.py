@@ -381,7 +381,7 @@ SHAPES = [(4, 2, 16, 16), (5, 1, 32, 8), (6, 3, 48, 16), (8, 2, 64, 16), (32, 8,
 DECODE_SEGS = [[(0, 1)], [(14, 1), (15, 1), (16, 1), (17, 1)], [(126, 1), (127, 1), (128, 1), (1, 1), (63, 1)],
                [(999, 1), (5, 1), (640, 1)]]
 CHUNK_SEGS = [[(0, 5)], [(0, 64)], [(0, 70)], [(100, 17), (37, 1), (0, 33)], [(3, 70), (200, 2), (15, 2), (16, 1)],
-              [(0, 300)], [(250, 50), (0, 1)]]
+              [(0, 300)], [(250, 50), (0, 1)], [(100, 120), (0, 40), (37, 1)], [(0, 2048)]]
 
 
 @pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", SHAPES)
@@ -405,7 +405,8 @@ def test_attention_bf16_plain_kernel(ops, ref, heads, kv_heads, head_dim, page_s
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(6, 3, 48, 16), (8, 2, 64, 16), (32, 8, 128, 16), (5, 1, 32, 8)])
 @pytest.mark.parametrize("window", [1, 24, 100])
-@pytest.mark.parametrize("segs", [DECODE_SEGS[1], DECODE_SEGS[3], CHUNK_SEGS[3], CHUNK_SEGS[4], CHUNK_SEGS[6]])
+@pytest.mark.parametrize("segs", [DECODE_SEGS[1], DECODE_SEGS[3], CHUNK_SEGS[3], CHUNK_SEGS[4], CHUNK_SEGS[5], CHUNK_SEGS[6],
+                                  CHUNK_SEGS[7]])
 def test_attention_window(ops, ref, dtype, heads, kv_heads, head_dim, page_size, window, segs):
     attention_case(ops, ref, dtype, heads, kv_heads, head_dim, page_size, segs, window, 12)
 
