@@ -61,6 +61,8 @@ def main():
     ap.add_argument("--layers", type=int, default=LLAMA_31_8B["num_hidden_layers"],
                     help="fewer layers than the model has (both numbers are reported)")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run the 2,048-token prefill steps alone and print their time (for profiling); no JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine runs on a single MI355X, --gpus {args.gpus} is not supported")
@@ -72,7 +74,7 @@ def main():
 
     cfg = dict(LLAMA_31_8B, num_hidden_layers=args.layers)
     steps, warmup = args.steps, args.warmup
-    batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
+    batches = [args.batch] if args.no_points or args.prefill_only else sorted({1, args.batch, 64})
     slack = max(batches) + 8          # requests whose prompt is done early decode while the others still prefill
     need_tokens = max(batches) * (PROMPT_LEN + warmup + steps + slack + PAGE_SIZE) + PREFILL_TOKENS + 64
     t0 = time.time()
@@ -111,6 +113,25 @@ def main():
         mean_contexts = [c + steps / 2.0 for c in contexts]
         return tokens / elapsed, elapsed / steps * 1e3, mean_contexts
 
+    def prefill_run(repeats=4):
+        """One request, its 2,048 tokens in one step; the median of the repeats after the first."""
+        times = []
+        for i in range(repeats):
+            engine.add_request(f"prefill-{i}", rng.integers(0, vocab, PREFILL_TOKENS).tolist(),
+                               SamplingParams(max_tokens=1, ignore_eos=True))
+            torch.cuda.synchronize()
+            start = time.perf_counter()
+            events = engine.step()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - start)
+            assert len(events) == 1 and events[0].finished
+        return float(np.median(times[1:]))
+
+    if args.prefill_only:
+        best = prefill_run(max(2, steps))
+        print(f"[bench] prefill {PREFILL_TOKENS} tokens: {best * 1e3:.2f} ms", file=sys.stderr, flush=True)
+        return
+
     results = {}
     for batch in batches:
         results[batch] = decode_run(batch)
@@ -138,18 +159,7 @@ def main():
         for b in (1, 64):
             bytes_b = decode_step_bytes(cfg, args.layers, results[b][2])
             line["points"][f"decode_b{b}_hbm_frac"] = round(bytes_b / (results[b][1] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
-        # prefill: one request, its 2,048 tokens in one step
-        times = []
-        for i in range(4):
-            engine.add_request(f"prefill-{i}", rng.integers(0, vocab, PREFILL_TOKENS).tolist(),
-                               SamplingParams(max_tokens=1, ignore_eos=True))
-            torch.cuda.synchronize()
-            start = time.perf_counter()
-            events = engine.step()
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - start)
-            assert len(events) == 1 and events[0].finished
-        best = float(np.median(times[1:]))
+        best = prefill_run()
         flops = prefill_flops(cfg, args.layers, PREFILL_TOKENS)
         line["prefill"] = {"value": round(PREFILL_TOKENS / best, 1), "tokens": PREFILL_TOKENS, "ms": round(best * 1e3, 3),
                            "frac": round(flops / best / (MFMA_PEAK_TFLOPS["bf16"] * 1e12), 4)}

@@ -14,7 +14,8 @@ const char *fllm_last_error(void);
 int fllm_abi_version(void);
 // 0: bfloat16 calls use the plain kernels only (for comparing them with the MFMA kernels); default 1
 void fllm_set_fast_kernels(int on);
-// Switches a kernel variant (for measurements and tests): "attention.tile32" 0/1.  0 on success.
+// Switches a kernel variant (for measurements and tests): "attention.tile32" 0/1; "linear.slices" n
+// (0: chosen by shape); "linear.dual_k" 0/1; "attention.fused_merge" 0/1.  0 on success.
 int fllm_set_option(const char *name, int value);
 
 // out[r, :] = scale * table[ids[r], :]            out: float32 [rows, width]
@@ -33,6 +34,14 @@ int fllm_add_rmsnorm(float *x, const void *branch, int branch_dtype, const float
 // out_mode 0: store as `dtype`; 1: store float32; 2: add to float32 `out` (row stride ldo)
 int fllm_linear(const void *x, int ldx, const void *w, const float *bias, void *out, int ldo, int M, int N, int K,
                 int dtype, int out_mode, hipStream_t stream);
+
+// Device memory for kernels that meet across workgroups: the decode-shaped products (1..16 rows), whose K
+// dimension is cut into slices over workgroups when the activations of all of K do not fit into LDS, and
+// decode attention over split contexts.  Its first 64 KiB are counters, which must be zero when it is handed
+// over and are zero again after every launch; partial sums follow.  One per device (the current one);
+// work that would need more than it holds runs another way.  Launches on different streams of one device
+// must not overlap while it is set.  nullptr takes it away.
+int fllm_set_device_workspace(void *workspace, size_t bytes);
 
 // Fused forms for decode steps in bfloat16 (1..16 rows, K a multiple of 8; fllm_fused_decode_supported).
 // x is the float32 residual stream [M, K]; each computes rmsnorm(x; norm_w, eps) @ w^T (+ bias) and

@@ -18,6 +18,7 @@
 //   decode kernel  one row per segment: a workgroup takes (row, key/value head, context split), its
 //                  sixteen waves stride over 32-key blocks loading K and V^T straight into MFMA
 //                  operands; long contexts of small batches are split and merged by a second kernel.
+#include <algorithm>
 #include "api.h"
 #include "common.h"
 
@@ -46,6 +47,7 @@ struct AttnArgs {
     float *ws_ml;   // [rows, heads, splits, 2]
     float *ws_o;    // [rows, heads, splits, D]
     int splits, keys_per_split;
+    int *counters;  // one per (row, key/value head, query tile), zero between launches: the last split to arrive merges; null: a merge kernel does
 };
 
 __device__ __forceinline__ bf16x8_t zero8() {
@@ -477,8 +479,12 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
     const int n = seg >= 0 ? p.row_pos[row] + 1 : 0;
     const int lo = (p.window > 0 && n - p.window > 0) ? n - p.window : 0;
     const int ps = p.page_size, psh = p.ps_shift, pmask = ps - 1, nkv = p.kv_heads;
-    const int begin = (lo / 32) * 32 + split * p.keys_per_split;
+    const int first = (lo / 32) * 32;
+    const int begin = first + split * p.keys_per_split;
     const int end = min(begin + p.keys_per_split, n);
+    // the splits that hold keys of this row; the others have nothing to add and leave at once
+    const int live_splits = p.counters ? max(1, (n - first + p.keys_per_split - 1) / p.keys_per_split) : p.splits;
+    if (p.counters && split >= live_splits) return;
     const int32_t *tbl = p.tables + (size_t)(seg >= 0 ? seg : 0) * p.table_stride;
 
     bf16x8_t qf[KD];
@@ -570,8 +576,14 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
             acc += sm_o[(w * gq + qi) * OP + d] * f;
         }
         const size_t hrow = (size_t)row * p.heads + kvh * G + h;
-        if (p.splits == 1) {
+        if (live_splits == 1) {
             p.out[hrow * D + d] = (bf16_t)(l > 0.f ? acc / l : 0.f);
+        } else if (p.counters) {   // read by another workgroup of this launch: straight to the device's point of coherence
+            __hip_atomic_store(p.ws_o + (hrow * p.splits + split) * D + d, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (d == 0) {
+                __hip_atomic_store(p.ws_ml + (hrow * p.splits + split) * 2, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(p.ws_ml + (hrow * p.splits + split) * 2 + 1, l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         } else {
             p.ws_o[(hrow * p.splits + split) * D + d] = acc;
             if (d == 0) {
@@ -579,6 +591,35 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
                 p.ws_ml[(hrow * p.splits + split) * 2 + 1] = l;
             }
         }
+    }
+    if (!p.counters || live_splits == 1) return;
+    // The split that arrives last adds the parts up, in the order of the splits: the result does not depend on
+    // which one that is.  Its partial sums have arrived before it is counted.
+    __shared__ int s_seen;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    int *counter = p.counters + ((size_t)row * p.kv_heads + kvh) * qtiles + qtile;
+    if (threadIdx.x == 0) s_seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (s_seen != live_splits - 1) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+    for (int idx = threadIdx.x; idx < gq * D; idx += WAVES * kWave) {
+        const int qi = idx / D, d = idx - qi * D;
+        const size_t hrow = (size_t)row * p.heads + kvh * G + qtile * 16 + qi;
+        const float *ml = p.ws_ml + hrow * p.splits * 2;
+        float m = -INFINITY;
+        for (int sp = 0; sp < live_splits; sp++)
+            m = fmaxf(m, __hip_atomic_load(ml + sp * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        float l = 0.f, acc = 0.f;
+        for (int sp = 0; sp < live_splits; sp++) {
+            const float ms = __hip_atomic_load(ml + sp * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float f = ms == -INFINITY ? 0.f : fast_exp2(ms - m);
+            l += __hip_atomic_load(ml + sp * 2 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
+            acc += __hip_atomic_load(p.ws_o + (hrow * p.splits + sp) * D + d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
+        }
+        p.out[hrow * D + d] = (bf16_t)(l > 0.f ? acc / l : 0.f);
     }
 }
 
@@ -605,22 +646,28 @@ attn_merge_kernel(const float *__restrict__ ws_ml, const float *__restrict__ ws_
     }
 }
 
-// How a decode step of `rows` rows is split over the context.  A workgroup of 16 waves takes 512 keys
-// per round; contexts are split only when they are long and the rows alone do not fill the machine
-// (a split costs a second kernel that merges the parts).
-void decode_split_plan(int rows, int kv_heads, int qtiles, int max_context, int *splits, int *keys_per_split) {
+// How a decode step of `rows` rows is split over the context.  A workgroup takes `unit` keys per round (32 a
+// wave).  Contexts are split when the rows alone do not fill the machine: down to one round per workgroup when
+// the parts are merged by the split that arrives last (`fused`), and only for long contexts when merging costs
+// a second kernel.
+void decode_split_plan(int rows, int kv_heads, int qtiles, int max_context, int unit, bool fused, int *splits,
+                       int *keys_per_split) {
     const long base = (long)rows * kv_heads * qtiles;
     const long span = (long)max_context + 31;   // the first split starts at a multiple of 32 at or below the first key
     long want = 1;
-    if (max_context > 2048 && base < 256) {
+    if (fused) {
+        if (base < 512) want = (512 + base - 1) / base;
+        const long most = (span + unit - 1) / unit;
+        if (want > most) want = most;
+    } else if (max_context > 2048 && base < 256) {
         want = (256 + base - 1) / base;
         const long most = (span + 2047) / 2048;
         if (want > most) want = most;
-        if (want > 64) want = 64;
     }
+    if (want > 64) want = 64;
     long per = (span + want - 1) / want;
-    per = (per + 511) / 512 * 512;
-    *splits = (int)want;
+    per = (per + unit - 1) / unit * unit;
+    *splits = (int)((span + per - 1) / per);
     *keys_per_split = (int)per;
 }
 
@@ -638,7 +685,13 @@ int launch(const AttnArgs &a, int uniform_rows, int max_context, void *workspace
     if (uniform_rows) {
         const int qtiles = (G + 15) / 16;
         AttnArgs p = a;
-        decode_split_plan(a.rows, a.kv_heads, qtiles, max_context, &p.splits, &p.keys_per_split);
+        constexpr int WAVES = D >= 128 ? 8 : 16;   // wide heads: fewer waves, so that the operands of a block fit the registers
+        void *dev_ws = nullptr;
+        size_t dev_ws_bytes = 0;
+        const bool fused = fllm_device_workspace(&dev_ws, &dev_ws_bytes) &&
+                           (size_t)a.rows * a.kv_heads * qtiles * sizeof(int) <= kWorkspaceCounterBytes && fllm_option_fused_merge();
+        decode_split_plan(a.rows, a.kv_heads, qtiles, max_context, WAVES * 32, fused, &p.splits, &p.keys_per_split);
+        p.counters = fused && p.splits > 1 ? (int *)dev_ws : nullptr;
         if (p.splits > 1) {
             const size_t need = (size_t)a.rows * a.heads * p.splits * (D + 2) * sizeof(float);
             FLLM_REQUIRE(workspace != nullptr && workspace_bytes >= need,
@@ -647,19 +700,18 @@ int launch(const AttnArgs &a, int uniform_rows, int max_context, void *workspace
             p.ws_o = p.ws_ml + (size_t)a.rows * a.heads * p.splits * 2;
         }
         FLLM_REQUIRE(a.kv_heads * qtiles <= 65535 && p.splits <= 65535, "attention: grid too large");
-        constexpr int WAVES = D >= 128 ? 8 : 16;   // wide heads: fewer waves, so that the operands of a block fit the registers
         const int gq = G < 16 ? G : 16;
         const size_t smem = (size_t)(2 * WAVES * 16 + WAVES * gq * (D + 1)) * sizeof(float);
         static bool attribute_set = false;   // more than the default 64 KiB of dynamic LDS has to be asked for once
         if (!attribute_set) {
             const hipError_t e = hipFuncSetAttribute((const void *)attn_decode_kernel<D, WAVES>,
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 159 * 1024);   // a few static bytes come on top
             FLLM_REQUIRE(e == hipSuccess, "attention: cannot raise the LDS limit: %s", hipGetErrorString(e));
             attribute_set = true;
         }
         hipLaunchKernelGGL((attn_decode_kernel<D, WAVES>), dim3(a.rows, a.kv_heads * qtiles, p.splits), dim3(WAVES * kWave),
                            smem, stream, p, qtiles);
-        if (p.splits > 1)
+        if (p.splits > 1 && !p.counters)
             hipLaunchKernelGGL(attn_merge_kernel<D>, dim3(a.rows, a.heads), dim3(kWave), 0, stream, p.ws_ml, p.ws_o, a.out,
                                a.heads, p.splits);
         return fllm_check_launch("attention_decode");
@@ -682,9 +734,13 @@ size_t fllm_attention_bf16_workspace_bytes(int rows, int heads, int kv_heads, in
     if (rows <= 0 || heads <= 0 || kv_heads <= 0) return 0;
     const int qtiles = (heads / kv_heads + 15) / 16;
     int splits, per;
-    decode_split_plan(rows, kv_heads, qtiles, max_context, &splits, &per);
-    if (splits <= 1) return 0;
-    return (size_t)rows * heads * splits * (head_dim + 2) * sizeof(float);
+    // the larger of the two plans (with and without the device workspace): which one runs is decided at the launch
+    size_t most = 0;
+    for (int fused = 0; fused < 2; fused++) {
+        decode_split_plan(rows, kv_heads, qtiles, max_context, (head_dim >= 128 ? 8 : 16) * 32, fused != 0, &splits, &per);
+        if (splits > 1) most = std::max(most, (size_t)rows * heads * splits * (head_dim + 2) * sizeof(float));
+    }
+    return most;
 }
 
 // 0: launched, negative: error, 1: shape declined (the caller uses the plain kernel)
@@ -721,6 +777,7 @@ int fllm_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, c
     a.ws_o = nullptr;
     a.splits = 1;
     a.keys_per_split = 0;
+    a.counters = nullptr;
     if (head_dim == 32) return launch<32>(a, uniform_rows, max_context, workspace, workspace_bytes, stream);
     if (head_dim == 64) return launch<64>(a, uniform_rows, max_context, workspace, workspace_bytes, stream);
     return launch<128>(a, uniform_rows, max_context, workspace, workspace_bytes, stream);

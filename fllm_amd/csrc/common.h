@@ -23,6 +23,17 @@ int fllm_check_launch(const char *what);
 int fllm_fast_kernels_enabled(void);
 // 1: prompt portions of 96+ rows use the 128-row attention kernel (default); 0: the 64-row kernel
 int fllm_option_tile32(void);
+// 0: the decode-shaped products choose their number of K slices themselves (default); n: n slices where that is possible
+int fllm_option_linear_slices(void);
+// 1: the parts of a split decode context are merged by the split that arrives last (default); 0: by a second kernel
+int fllm_option_fused_merge(void);
+// 1: decode-shaped products of up to 8 rows use 8-row weight tiles with two K halves a product (default); 0: 16-row tiles
+int fllm_option_dual_k(void);
+
+// The device workspace of the current device (fllm_set_device_workspace): its first kWorkspaceCounterBytes are
+// counters that every kernel leaves at zero, the rest is for partial results of the kernel that is running.
+constexpr size_t kWorkspaceCounterBytes = 64 * 1024;
+bool fllm_device_workspace(void **base, size_t *bytes);
 
 #define FLLM_REQUIRE(cond, ...)            \
     do {                                   \

@@ -34,8 +34,11 @@ struct SkinnyArgs {
     void *out;
     int ldo;
     int M, N, K;
-    int kc;        // K chunk staged in LDS, a multiple of 128
+    int S, slice;  // K is cut into S slices of `slice` elements (a multiple of 128); a workgroup stages one slice
     int ssq_off;   // byte offset of the sums of squares in LDS (behind the staging / reduction area)
+    float *ws;     // S > 1: partial sums [tile][slice][RT][64 lanes][4], then sums of squares [tile][slice][16]
+    float *ws_ssq;
+    int *counters; // S > 1: items of a tile counted so far (zero between launches)
     // QKV epilogue
     const int32_t *row_pos, *row_seg, *tables;
     int table_stride;
@@ -52,250 +55,319 @@ __device__ __forceinline__ bf16x8_t zero8() {
     return z;
 }
 
-// The epilogue of one output group: row m, columns nb .. nb + 3, sums s[t] (t: weight row tile).
-template <int MT, int WAVES, int PRO, int EPI, int RT>
-__device__ __forceinline__ void finish_group(const SkinnyArgs &a, const f32x4_t *red, const float *ssq_part, int mt, int l,
-                                             int n0, int n_out) {
-    const int M = a.M, N = a.N, K = a.K;
-    do {
-        const int m = mt * 16 + (l & 15);
-        const int nb = n0 + (l >> 4) * 4;   // four consecutive output columns
-        if (m >= M || nb >= n_out) continue;
-        f32x4_t s[RT];
+// The sums of one output group (row m, columns nb .. nb + 3) over the waves of a workgroup, in wave order.
+template <int WAVES, int RT>
+__device__ __forceinline__ void sum_waves(const f32x4_t *red, int stride_t, int idx, f32x4_t (&s)[RT]) {
 #pragma unroll
-        for (int t = 0; t < RT; t++) {
-            s[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < RT; t++) {
+        s[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int wv = 0; wv < WAVES; wv++) s[t] += red[((wv * RT + t) * MT + mt) * kWave + l];
+        for (int wv = 0; wv < WAVES; wv++) s[t] += red[(wv * RT + t) * stride_t + idx];
+    }
+}
+
+// What happens to the finished sums of one output group: row scale of the norm, bias, then the store.
+// ss: the row's sum of squares (norm prologue).
+template <int PRO, int EPI, int RT>
+__device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], float ss, int m, int nb, int n_out) {
+    const int N = a.N, K = a.K;
+    if (PRO == PRO_NORM_F32) {
+        const float inv = 1.0f / sqrtf(ss / (float)K + a.eps);
+#pragma unroll
+        for (int t = 0; t < RT; t++) s[t] *= inv;
+    }
+    if (a.bias) {
+#pragma unroll
+        for (int t = 0; t < RT; t++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (nb + i < n_out) s[t][i] += a.bias[t * n_out + nb + i];
+    }
+    if (EPI == EPI_STORE || EPI == EPI_STORE_F32 || EPI == EPI_ADD) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int n = nb + i;
+            if (n >= N) continue;
+            const size_t o = (size_t)m * a.ldo + n;
+            if (EPI == EPI_STORE) ((bf16_t *)a.out)[o] = (bf16_t)s[0][i];
+            else if (EPI == EPI_STORE_F32) ((float *)a.out)[o] = s[0][i];
+            else ((float *)a.out)[o] += s[0][i];
         }
-        if (PRO == PRO_NORM_F32) {
-            float ss = 0.f;
+    } else if (EPI == EPI_SWIGLU) {
 #pragma unroll
-            for (int wv = 0; wv < WAVES; wv++) ss += ssq_part[wv * 16 * MT + m];
-            const float inv = 1.0f / sqrtf(ss / (float)K + a.eps);
-#pragma unroll
-            for (int t = 0; t < RT; t++) s[t] *= inv;
+        for (int i = 0; i < 4; i++) {
+            const int n = nb + i;
+            if (n >= n_out) continue;
+            const float gt = s[0][i], up = s[RT - 1][i];
+            ((bf16_t *)a.out)[(size_t)m * a.ldo + n] = (bf16_t)(gt / (1.0f + expf(-gt)) * up);
         }
-        if (a.bias) {
+    } else {   // EPI_QKV: N = (heads + 2 kv_heads) * head_dim, head_dim a multiple of 4, so nb..nb+3 lie in one head
+        const int seg = a.row_seg[m];
+        if (seg < 0) return;
+        const int pos = a.row_pos[m];
+        const int d = a.head_dim;
+        const int hd = nb / d, j = nb - hd * d;          // head (q heads, then k heads, then v heads), lane in head
+        float v[4] = {s[0][0], s[0][1], s[0][2], s[0][3]};
+        if (hd < a.heads + a.kv_heads && j < a.rope_dims) {   // rope_dims is even; j is a multiple of 4
+            const float *cs = a.cos_t + (size_t)pos * (a.rope_dims / 2), *sn = a.sin_t + (size_t)pos * (a.rope_dims / 2);
 #pragma unroll
-            for (int t = 0; t < RT; t++)
+            for (int p = 0; p < 2; p++) {
+                if (j + 2 * p < a.rope_dims) {
+                    const int l2 = (j + 2 * p) / 2;
+                    const float x0 = v[2 * p], x1 = v[2 * p + 1];
+                    v[2 * p] = x0 * cs[l2] - x1 * sn[l2];
+                    v[2 * p + 1] = x1 * cs[l2] + x0 * sn[l2];
+                }
+            }
+        }
+        if (hd < a.heads) {
+            bf16_t *q = (bf16_t *)a.out + (size_t)m * a.ldo + nb;
+#pragma unroll
+            for (int i = 0; i < 4; i++) q[i] = (bf16_t)v[i];
+        } else if (a.store_kv) {
+            const int page = a.tables[(size_t)seg * a.table_stride + pos / a.page_size];
+            const int off = pos % a.page_size;
+            if (hd < a.heads + a.kv_heads) {
+                const int kvh = hd - a.heads;
+                bf16_t *kd = a.k_pages + (((size_t)page * a.kv_heads + kvh) * a.page_size + off) * d + j;
+#pragma unroll
+                for (int i = 0; i < 4; i++) kd[i] = (bf16_t)v[i];
+            } else {
+                const int kvh = hd - a.heads - a.kv_heads;
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    if (nb + i < n_out) s[t][i] += a.bias[t * n_out + nb + i];
-        }
-        if (EPI == EPI_STORE || EPI == EPI_STORE_F32 || EPI == EPI_ADD) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int n = nb + i;
-                if (n >= N) continue;
-                const size_t o = (size_t)m * a.ldo + n;
-                if (EPI == EPI_STORE) ((bf16_t *)a.out)[o] = (bf16_t)s[0][i];
-                else if (EPI == EPI_STORE_F32) ((float *)a.out)[o] = s[0][i];
-                else ((float *)a.out)[o] += s[0][i];
-            }
-        } else if (EPI == EPI_SWIGLU) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int n = nb + i;
-                if (n >= n_out) continue;
-                const float gt = s[0][i], up = s[RT - 1][i];
-                ((bf16_t *)a.out)[(size_t)m * a.ldo + n] = (bf16_t)(gt / (1.0f + expf(-gt)) * up);
-            }
-        } else {   // EPI_QKV: N = (heads + 2 kv_heads) * head_dim, head_dim a multiple of 4, so nb..nb+3 lie in one head
-            const int seg = a.row_seg[m];
-            if (seg < 0) continue;
-            const int pos = a.row_pos[m];
-            const int d = a.head_dim;
-            const int hd = nb / d, j = nb - hd * d;          // head (q heads, then k heads, then v heads), lane in head
-            float v[4] = {s[0][0], s[0][1], s[0][2], s[0][3]};
-            if (hd < a.heads + a.kv_heads && j < a.rope_dims) {   // rope_dims is even; j is a multiple of 4
-                const float *cs = a.cos_t + (size_t)pos * (a.rope_dims / 2), *sn = a.sin_t + (size_t)pos * (a.rope_dims / 2);
-#pragma unroll
-                for (int p = 0; p < 2; p++) {
-                    if (j + 2 * p < a.rope_dims) {
-                        const int l2 = (j + 2 * p) / 2;
-                        const float x0 = v[2 * p], x1 = v[2 * p + 1];
-                        v[2 * p] = x0 * cs[l2] - x1 * sn[l2];
-                        v[2 * p + 1] = x1 * cs[l2] + x0 * sn[l2];
-                    }
-                }
-            }
-            if (hd < a.heads) {
-                bf16_t *q = (bf16_t *)a.out + (size_t)m * a.ldo + nb;
-#pragma unroll
-                for (int i = 0; i < 4; i++) q[i] = (bf16_t)v[i];
-            } else if (a.store_kv) {
-                const int page = a.tables[(size_t)seg * a.table_stride + pos / a.page_size];
-                const int off = pos % a.page_size;
-                if (hd < a.heads + a.kv_heads) {
-                    const int kvh = hd - a.heads;
-                    bf16_t *kd = a.k_pages + (((size_t)page * a.kv_heads + kvh) * a.page_size + off) * d + j;
-#pragma unroll
-                    for (int i = 0; i < 4; i++) kd[i] = (bf16_t)v[i];
-                } else {
-                    const int kvh = hd - a.heads - a.kv_heads;
-#pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        a.v_pages[(((size_t)page * a.kv_heads + kvh) * d + j + i) * a.page_size + off] = (bf16_t)v[i];
-                }
+                    a.v_pages[(((size_t)page * a.kv_heads + kvh) * d + j + i) * a.page_size + off] = (bf16_t)v[i];
             }
         }
-        } while (false);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
 // up to 16 rows: activations stay in LDS, workgroups walk over the weight row tiles
 // ---------------------------------------------------------------------------------------------
-// A workgroup of 8 waves stages the activations once (all of K when they fit, which is the case of
-// the model's own shapes; else K chunk by K chunk for every tile) and then takes weight row tiles
-// blockIdx.x, blockIdx.x + gridDim.x, ...: its waves split K, read their B operands from LDS and
-// stream the weights with one block of loads in flight ahead of the products, across tile borders.
-template <int PRO, int EPI>
-__global__ void __launch_bounds__(8 * kWave) __attribute__((amdgpu_waves_per_eu(4, 4)))   // two workgroups per CU: 128 registers
+// The product is cut into items (weight row tile, K slice).  Workgroup b of the grid owns slice
+// b % S and the tiles b / S, b / S + G / S, ...  Its 8 waves split the slice into contiguous ranges;
+// every wave stages the activations of its own range in LDS (for the norm prologue: x * norm_weight
+// as bfloat16, and its part of every row's sum of squares) and needs nobody else's, so no wave waits
+// for another before the end of an item.  The weights go from global memory straight into MFMA A
+// operands, two blocks of loads (8 KiB a wave) in flight ahead of the products, across tile borders.
+//
+// What the 16 A rows of a product are (TM):
+//   TM_ROWS16  16 weight rows, one K range                                   (16 outputs a row)
+//   TM_DUALK   up to 8 activation rows: 8 weight rows, each with two K ranges (the halves of the wave's
+//              range): A row r and B column r take K half r / 8, so D[r][c] is a partial sum where
+//              r / 8 == c / 8, and the two are added at the end               (8 outputs a row)
+//   TM_GATEUP  8 gate rows and the 8 up rows that belong to them              (8 outputs a row)
+// The smaller tiles are what fills the chip evenly: 16-row tiles of the model's projections come to
+// 1.5 or 3.5 a compute-unit slot.
+//
+// At the end of an item the waves' sums meet in LDS; one wave (they take turns) adds them in wave
+// order.  With S = 1 it runs the epilogue.  With S > 1 (only when the activations of all of K do not
+// fit into LDS) it leaves the item's sums in the workspace and counts the item; the workgroup that
+// counts a tile's last item adds the S partial sums in slice order and runs the epilogue, so the
+// result does not depend on which workgroup came last.
+enum { TM_ROWS16 = 0, TM_DUALK = 1, TM_GATEUP = 2 };
+
+template <int PRO, int EPI, int TM, int WAVES>
+__global__ void __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4, 4)))   // 16 waves a CU: 128 registers
 skinny_resident_kernel(SkinnyArgs a, int red_off) {
-    constexpr int MT = 1, WAVES = 8;
+    constexpr int U = 4;                           // k-steps of 32 per block: four 16-byte loads per lane
+    constexpr int KB = 32 * U;                     // K elements of one range per block
+    constexpr int NT = TM == TM_ROWS16 ? 16 : 8;   // outputs per row and tile
     constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
-    constexpr int THREADS = WAVES * kWave;
-    constexpr int U = 4 / RT;                      // k-steps of 32 per wave iteration: four weight loads in flight, four ahead
+    static_assert((EPI == EPI_SWIGLU) == (TM == TM_GATEUP), "gate/up tiles belong to the SwiGLU epilogue");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int r = lane & 15, g = lane >> 4;
-    const int M = a.M, N = a.N, K = a.K;
+    const int M = a.M, N = a.N, K = a.K, S = a.S;
     const int n_out = EPI == EPI_SWIGLU ? N / 2 : N;
-    const int ntiles = (n_out + 15) / 16;
-    const int pitch = a.kc + 8;
+    const int ntiles = (n_out + NT - 1) / NT;
+    const int pitch = a.slice + 8;
     bf16_t *xs = (bf16_t *)smem;                                  // [M][pitch]
-    f32x4_t *red = (f32x4_t *)(smem + red_off);                   // [WAVES][RT][64]
+    f32x4_t *red = (f32x4_t *)(smem + red_off);                   // [WAVES][64]
     float *ssq_part = (float *)(smem + a.ssq_off);                // [WAVES][16]
-    const bool resident = a.kc >= K;                              // one chunk: staged once for all tiles
-    const int kstep = WAVES * 32 * U;
 
-    auto row_pointers = [&](int tile, const bf16_t *(&wp)[RT]) {
-#pragma unroll
-        for (int t = 0; t < RT; t++) {
-            int row = tile * 16 + r;
-            if (row >= n_out) row = n_out - 1;    // past the end: computed from a valid row, never stored
-            wp[t] = a.w + (size_t)(row + t * n_out) * K + g * 8;
-        }
-    };
-    auto load_w = [&](bf16x8_t (&wf)[RT][U], const bf16_t *const (&wp)[RT], int kabs, int kend) {
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const bool in = kabs + u * 32 + g * 8 < kend;
-#pragma unroll
-            for (int t = 0; t < RT; t++) wf[t][u] = in ? *(const bf16x8_t *)(wp[t] + kabs + u * 32) : zero8();
-        }
-    };
+    const int sl = blockIdx.x % S;
+    const int tile0 = blockIdx.x / S, tstride = gridDim.x / S;
+    const int ks0 = sl * a.slice;
+    const int kcn = min(K, ks0 + a.slice) - ks0;                  // a multiple of 8
+    const int my_items = tile0 < ntiles ? (ntiles - tile0 + tstride - 1) / tstride : 0;
+    // the wave's contiguous part of the slice (relative to ks0), in steps of 64, and its blocks (the same number for every wave)
+    const int kwlen = ((kcn + WAVES - 1) / WAVES + 63) / 64 * 64;
+    const int kw0 = min(kcn, wave * kwlen), kw1 = min(kcn, kw0 + kwlen);
+    const int half = TM == TM_DUALK ? kwlen / 2 : kwlen;          // the K range that one A row covers in an item
+    const int nbw = (half + KB - 1) / KB;
+    // this lane's A row and B column: weight row in the tile, activation row, and where its K range starts
+    const int wrow_in_tile = TM == TM_ROWS16 ? r : (r & 7) + (TM == TM_GATEUP ? (r >> 3) * n_out : 0);
+    const int xrow_i = TM == TM_DUALK ? (r & 7) : r;
+    const int kr0 = kw0 + (TM == TM_DUALK ? (r >> 3) * half : 0) + g * 8;      // relative to ks0
+    const int kr1 = TM == TM_DUALK ? min(kw1, kw0 + ((r >> 3) + 1) * half) : kw1;
+    const int row_limit = TM == TM_GATEUP ? n_out : N;            // weight rows past it are clamped (never stored)
 
-    int tile = blockIdx.x;
-    const bf16_t *wp[RT];
-    row_pointers(tile, wp);
-    bf16x8_t wnext[RT][U];
-    int have_tile = tile, have_k = wave * 32 * U;         // which block of weights `wnext` holds
-    load_w(wnext, wp, wave * 32 * U, min(a.kc, K));     // in flight while the activations are staged
+    // cursor of the loads: (item, block in item) of the next block to ask for
+    int l_item = 0, l_j = 0;
+    auto issue = [&](bf16x8_t (&buf)[U]) {
+        if (l_item < my_items) {
+            int row = (tile0 + l_item * tstride) * NT + (TM == TM_ROWS16 ? r : (r & 7));
+            if (row >= row_limit) row = row_limit - 1;
+            if (TM == TM_GATEUP) row += (r >> 3) * n_out;
+            const int kb = kr0 + l_j * KB;
+            const bf16_t *wp = a.w + (size_t)row * K + ks0 + kb;
+#pragma unroll
+            for (int u = 0; u < U; u++) buf[u] = kb + u * 32 < kr1 ? *(const bf16x8_t *)(wp + u * 32) : zero8();
+        }
+        if (++l_j == nbw) l_j = 0, l_item++;
+    };
+    (void)wrow_in_tile;
+    bf16x8_t b0[U], b1[U];
+    issue(b0);      // in flight while the activations are staged
+    issue(b1);
+
+    // the wave's own columns kw0 .. kw1 of every row
     if (PRO == PRO_NORM_F32 && lane < 16) ssq_part[wave * 16 + lane] = 0.f;
-    bool staged = false;
-
-    for (; tile < ntiles; tile += gridDim.x) {
-        const bf16_t *wp_next[RT];
-        row_pointers(tile + gridDim.x < ntiles ? tile + gridDim.x : tile, wp_next);
-        f32x4_t acc[RT];
+    __builtin_amdgcn_wave_barrier();
+    for (int cw = kw0; cw < kw1; cw += kWave * 8) {   // the same trips for every lane: the sums below are over the wave
+        const int c0 = cw + lane * 8;
+        const bool in = c0 < kw1;
+        if (PRO == PRO_BF16) {
+            const bf16_t *x = (const bf16_t *)a.x + ks0 + c0;
+            for (int m0 = 0; m0 < M; m0 += 4) {
+                bf16x8_t v[4];
 #pragma unroll
-        for (int t = 0; t < RT; t++) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-        for (int kc0 = 0; kc0 < K; kc0 += a.kc) {
-            const int kcn = min(a.kc, K - kc0);           // a multiple of 8
-            if (!staged) {
-                __syncthreads();                           // whoever still reads the staging area is done
-                if (PRO == PRO_BF16) {
-                    const bf16_t *x = (const bf16_t *)a.x;
-                    const int per_row = kcn / 8;
-                    for (int idx = threadIdx.x; idx < M * per_row; idx += THREADS) {
-                        const int m = idx / per_row, c = idx - m * per_row;
-                        *(bf16x8_t *)(xs + m * pitch + c * 8) = *(const bf16x8_t *)(x + (size_t)m * a.ldx + kc0 + c * 8);
-                    }
-                } else {
-                    const float *x = (const float *)a.x;
-                    const int per_row = kcn / 8;
-                    const int per_row_pad = (per_row + kWave - 1) / kWave * kWave;   // a wave never straddles two rows
-                    const int total = M * per_row_pad;
-                    constexpr int PASSES = 2;                                         // loads of two passes are in flight together
-                    for (int base = threadIdx.x; base < total; base += PASSES * THREADS) {
-                        f32x4_t xv[PASSES][2], wv[PASSES][2];
-                        int mrow[PASSES], col[PASSES];
-                        bool ok[PASSES];
+                for (int i = 0; i < 4; i++)
+                    if (in && m0 + i < M) v[i] = *(const bf16x8_t *)(x + (size_t)(m0 + i) * a.ldx);
 #pragma unroll
-                        for (int j = 0; j < PASSES; j++) {
-                            const int idx = base + j * THREADS;
-                            mrow[j] = idx / per_row_pad;
-                            col[j] = (idx - mrow[j] * per_row_pad) * 8;
-                            ok[j] = idx < total && col[j] < kcn;
-                            if (ok[j]) {
-                                const float *xp = x + (size_t)mrow[j] * a.ldx + kc0 + col[j];
-                                xv[j][0] = *(const f32x4_t *)xp;
-                                xv[j][1] = *(const f32x4_t *)(xp + 4);
-                                wv[j][0] = *(const f32x4_t *)(a.norm_w + kc0 + col[j]);
-                                wv[j][1] = *(const f32x4_t *)(a.norm_w + kc0 + col[j] + 4);
-                            }
-                        }
-#pragma unroll
-                        for (int j = 0; j < PASSES; j++) {
-                            if (base - threadIdx.x + j * THREADS + wave * kWave >= total) continue;   // the whole wave is past the end
-                            float ss = 0.f;
-                            if (ok[j]) {
-                                bf16x8_t v;
-#pragma unroll
-                                for (int i = 0; i < 4; i++) {
-                                    ss += xv[j][0][i] * xv[j][0][i] + xv[j][1][i] * xv[j][1][i];
-                                    v[i] = (bf16_t)(xv[j][0][i] * wv[j][0][i]);
-                                    v[4 + i] = (bf16_t)(xv[j][1][i] * wv[j][1][i]);
-                                }
-                                *(bf16x8_t *)(xs + mrow[j] * pitch + col[j]) = v;
-                            }
-                            ss = wave_sum(ss);
-                            if (lane == 0) ssq_part[wave * 16 + mrow[j]] += ss;
-                        }
-                    }
-                }
-                __syncthreads();
-                staged = resident;
+                for (int i = 0; i < 4; i++)
+                    if (in && m0 + i < M) *(bf16x8_t *)(xs + (m0 + i) * pitch + c0) = v[i];
             }
-            for (int k0 = wave * 32 * U; k0 < kcn; k0 += kstep) {
-                bf16x8_t wf[RT][U], xf[U];
-                if (have_tile != tile || have_k != kc0 + k0) load_w(wnext, wp, kc0 + k0, kc0 + kcn);   // not prefetched
+        } else {
+            const float *x = (const float *)a.x + ks0 + c0;
+            f32x4_t w0 = {0.f, 0.f, 0.f, 0.f}, w1 = w0;
+            if (in) w0 = *(const f32x4_t *)(a.norm_w + ks0 + c0), w1 = *(const f32x4_t *)(a.norm_w + ks0 + c0 + 4);
+            for (int m0 = 0; m0 < M; m0 += 4) {
+                f32x4_t xv[4][2];
 #pragma unroll
-                for (int t = 0; t < RT; t++)
-#pragma unroll
-                    for (int u = 0; u < U; u++) wf[t][u] = wnext[t][u];
-                // the next weights of this wave: the rest of this chunk, the next chunk, or the next tile
-                if (k0 + kstep < kcn) {
-                    load_w(wnext, wp, kc0 + k0 + kstep, kc0 + kcn);
-                    have_tile = tile, have_k = kc0 + k0 + kstep;
-                } else if (kc0 + a.kc < K) {
-                    load_w(wnext, wp, kc0 + a.kc + wave * 32 * U, min(kc0 + 2 * a.kc, K));
-                    have_tile = tile, have_k = kc0 + a.kc + wave * 32 * U;
-                } else if (tile + gridDim.x < ntiles) {
-                    load_w(wnext, wp_next, wave * 32 * U, min(a.kc, K));
-                    have_tile = tile + gridDim.x, have_k = wave * 32 * U;
+                for (int i = 0; i < 4; i++) {
+                    xv[i][0] = xv[i][1] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+                    if (in && m0 + i < M) {
+                        xv[i][0] = *(const f32x4_t *)(x + (size_t)(m0 + i) * a.ldx);
+                        xv[i][1] = *(const f32x4_t *)(x + (size_t)(m0 + i) * a.ldx + 4);
+                    }
                 }
 #pragma unroll
-                for (int u = 0; u < U; u++) {
-                    const int k = k0 + u * 32 + g * 8;
-                    xf[u] = (k < kcn && r < M) ? *(const bf16x8_t *)(xs + r * pitch + k) : zero8();
+                for (int i = 0; i < 4; i++) {
+                    if (m0 + i >= M) break;
+                    bf16x8_t v;
+                    float ss = 0.f;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        ss += xv[i][0][e] * xv[i][0][e] + xv[i][1][e] * xv[i][1][e];
+                        v[e] = (bf16_t)(xv[i][0][e] * w0[e]);
+                        v[4 + e] = (bf16_t)(xv[i][1][e] * w1[e]);
+                    }
+                    if (in) *(bf16x8_t *)(xs + (m0 + i) * pitch + c0) = v;
+                    ss = wave_sum(ss);
+                    if (lane == 0) ssq_part[wave * 16 + m0 + i] += ss;
                 }
-#pragma unroll
-                for (int u = 0; u < U; u++)
-#pragma unroll
-                    for (int t = 0; t < RT; t++) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t][u], xf[u], acc[t], 0, 0, 0);
             }
         }
+    }
+    __builtin_amdgcn_wave_barrier();   // the wave reads what its own lanes wrote: LDS keeps a wave's accesses in order
+
+    // cursor of the products
+    int item = 0, j = 0;
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    const bf16_t *xrow = xs + xrow_i * pitch + kr0;
+    const bool xvalid = xrow_i < M;
+
+    auto step = [&](bf16x8_t (&buf)[U]) {
+        bf16x8_t xf[U];
+        const int kb = kr0 + j * KB;
 #pragma unroll
-        for (int t = 0; t < RT; t++) red[(wave * RT + t) * kWave + lane] = acc[t];
+        for (int u = 0; u < U; u++) xf[u] = (kb + u * 32 < kr1 && xvalid) ? *(const bf16x8_t *)(xrow + j * KB + u * 32) : zero8();
+#pragma unroll
+        for (int u = 0; u < U; u++) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(buf[u], xf[u], acc, 0, 0, 0);
+        issue(buf);      // the block two ahead takes this one's registers
+        if (++j < nbw) return;
+        // the item is complete: the waves' sums meet in LDS; one wave (they take turns) adds them up and goes on
+        // to the epilogue while the others start the next item
+        j = 0;
+        red[wave * kWave + lane] = acc;
+        acc = (f32x4_t){0.f, 0.f, 0.f, 0.f};
         __syncthreads();
-        if (threadIdx.x < kWave) finish_group<MT, WAVES, PRO, EPI, RT>(a, red, ssq_part, 0, threadIdx.x, tile * 16, n_out);
-        __syncthreads();      // the sums have been read: the next tile may overwrite them
-        if (PRO == PRO_NORM_F32 && !resident && lane < 16) ssq_part[wave * 16 + lane] = 0.f;
+        const int tile = tile0 + item * tstride;
+        const bool finisher = wave == (item & (WAVES - 1));
+        // D[row 4 g + i][column r]: for the 8-output tiles the lanes g < 2 hold outputs 4 g + i, and their partners
+        // sit 32 lanes on (TM_GATEUP: the up rows) or 32 + 8 lanes on (TM_DUALK: the other K half)
+        const bool owner = TM == TM_ROWS16 ? true : (g < 2 && (TM == TM_GATEUP || r < 8));
+        f32x4_t s[RT];
+        if (finisher && owner) {
 #pragma unroll
-        for (int t = 0; t < RT; t++) wp[t] = wp_next[t];
+            for (int t = 0; t < RT; t++) s[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int wv = 0; wv < WAVES; wv++) {
+                s[0] += red[wv * kWave + lane];
+                if (TM == TM_DUALK) s[0] += red[wv * kWave + lane + 40];
+                if (TM == TM_GATEUP) s[RT - 1] += red[wv * kWave + lane + 32];
+            }
+        }
+        __syncthreads();      // the sums have been read: the next item may overwrite them
+        if (finisher) {
+            do {
+                const int m = TM == TM_DUALK ? (r & 7) : r, nb = tile * NT + g * 4;
+                float ss = 0.f;
+                if (PRO == PRO_NORM_F32) {
+#pragma unroll
+                    for (int wv = 0; wv < WAVES; wv++) ss += ssq_part[wv * 16 + m];
+                }
+                if (S > 1) {
+                    float *part = a.ws + ((size_t)(tile * S + sl) * RT * kWave + lane) * 4;
+                    if (owner && m < M) {
+#pragma unroll
+                        for (int t = 0; t < RT; t++)
+#pragma unroll
+                            for (int i = 0; i < 4; i++)
+                                __hip_atomic_store(part + t * kWave * 4 + i, s[t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (PRO == PRO_NORM_F32 && g == 0)
+                            __hip_atomic_store(a.ws_ssq + (size_t)(tile * S + sl) * 16 + m, ss, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    // Every access to the workspace goes to the device's point of coherence by itself (agent-scope
+                    // atomics), so no cache has to be written back or dropped: it is enough that the wave's partial
+                    // sums have arrived there before the item is counted.
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                    __builtin_amdgcn_s_waitcnt(0);
+                    int seen = 0;
+                    if (lane == 0) seen = __hip_atomic_fetch_add(a.counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    seen = __shfl(seen, 0, kWave);
+                    if (seen != S - 1) break;       // another workgroup finishes this tile
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                    if (lane == 0) __hip_atomic_store(a.counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+                    if (!owner || m >= M) break;
+#pragma unroll
+                    for (int t = 0; t < RT; t++) s[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+                    ss = 0.f;
+                    for (int s2 = 0; s2 < S; s2++) {
+                        const float *src = a.ws + ((size_t)(tile * S + s2) * RT * kWave + lane) * 4;
+#pragma unroll
+                        for (int t = 0; t < RT; t++)
+#pragma unroll
+                            for (int i = 0; i < 4; i++)
+                                s[t][i] += __hip_atomic_load(src + t * kWave * 4 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (PRO == PRO_NORM_F32)
+                            ss += __hip_atomic_load(a.ws_ssq + (size_t)(tile * S + s2) * 16 + m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                }
+                if (!owner || m >= M || nb >= n_out) break;
+                epilogue<PRO, EPI, RT>(a, s, ss, m, nb, n_out);
+            } while (false);
+        }
+        item++;
+    };
+
+    const int total = my_items * nbw;
+    for (int q = 0; q < total; q += 2) {
+        step(b0);
+        if (q + 1 < total) step(b1);
     }
 }
 
@@ -340,8 +412,14 @@ skinny_direct_kernel(SkinnyArgs a) {
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) red[(wave * MT + mt) * kWave + lane] = acc[mt];
     __syncthreads();
-    for (int e = threadIdx.x; e < MT * kWave; e += THREADS)
-        finish_group<MT, WAVES, PRO, EPI, RT>(a, red, nullptr, e / kWave, e % kWave, n0, N);
+    for (int e = threadIdx.x; e < MT * kWave; e += THREADS) {
+        const int mt = e / kWave, l = e % kWave;
+        const int m = mt * 16 + (l & 15), nb = n0 + (l >> 4) * 4;
+        if (m >= M || nb >= N) continue;
+        f32x4_t s[RT];
+        sum_waves<WAVES, RT>(red, MT * kWave, mt * kWave + l, s);
+        epilogue<PRO, EPI, RT>(a, s, 0.f, m, nb, N);
+    }
 }
 
 int device_cus() {
@@ -355,38 +433,108 @@ int device_cus() {
     return cus;
 }
 
-template <int PRO, int EPI>
-int launch_resident(SkinnyArgs a, hipStream_t stream) {
-    constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
-    constexpr int WAVES = 8;
-    const int kpad = (a.K + 127) / 128 * 128;
-    // all of K when the rows fit into 136 KiB (one workgroup per CU; two when they fit into 64 KiB), else chunks of 64 KiB
-    int kc = kpad;
-    if ((size_t)a.M * (kpad + 8) * sizeof(bf16_t) > 136 * 1024) {
-        kc = ((int)(64 * 1024 / sizeof(bf16_t) / a.M) - 8) / 128 * 128;
-        if (kc < 128) return 1;
+// Workspace of the K-sliced products: the device workspace, if the host program has set one.
+struct Workspace {
+    float *base = nullptr;
+    size_t bytes = 0;
+};
+constexpr size_t kCounterBytes = kWorkspaceCounterBytes;
+constexpr int kMaxSlices = 32;
+
+// What a launch of the resident kernel looks like for a shape: K slices, waves per workgroup, workgroups per CU.
+struct ResidentPlan {
+    int S = 0, slice = 0, waves = 8, per_cu = 0;
+    size_t stage = 0, red = 0, smem = 0;
+};
+
+// The fewest K slices whose activations fit into LDS (slicing costs more than it gains wherever it is not needed):
+// twice into a compute unit's as two workgroups of 8 waves, else once as one workgroup of 16 waves, so that as
+// many loads are in flight.
+ResidentPlan plan_resident(int M, int K, int ntiles, int rt, const Workspace &ws) {
+    const int forced = fllm_option_linear_slices();
+    ResidentPlan best;
+    for (int S = 1; S <= kMaxSlices; S *= 2) {
+        const int slice = ((K + S - 1) / S + 127) / 128 * 128;
+        if (S > 1 && (slice < 1024 || (S - 1) * slice >= K)) break;
+        if (S > 1) {
+            const size_t need = kCounterBytes + (size_t)ntiles * S * (rt * kWave * 4 + 16) * sizeof(float);
+            if (ws.base == nullptr || need > ws.bytes || (size_t)ntiles * sizeof(int) > kCounterBytes) break;
+        }
+        ResidentPlan p;
+        p.S = S;
+        p.slice = slice;
+        p.stage = ((size_t)M * (slice + 8) * sizeof(bf16_t) + 15) / 16 * 16;
+        const size_t small = p.stage + 8 * (kWave * sizeof(f32x4_t) + 16 * sizeof(float));
+        const size_t large = p.stage + 16 * (kWave * sizeof(f32x4_t) + 16 * sizeof(float));
+        if (small <= 76 * 1024) p.waves = 8, p.per_cu = 2, p.smem = small;
+        else if (large <= 160 * 1024) p.waves = 16, p.per_cu = 1, p.smem = large;
+        else continue;
+        p.red = (size_t)p.waves * kWave * sizeof(f32x4_t);
+        if (forced == 0 || S == forced || best.S == 0) best = p;
+        if (forced == 0 || S == forced) break;
     }
-    a.kc = kc;
-    const size_t stage = ((size_t)a.M * (kc + 8) * sizeof(bf16_t) + 15) / 16 * 16;
-    const size_t red = (size_t)WAVES * RT * kWave * sizeof(f32x4_t);
-    const size_t smem = stage + red + (size_t)WAVES * 16 * sizeof(float);
-    a.ssq_off = (int)(stage + red);
-    const int n_out = EPI == EPI_SWIGLU ? a.N / 2 : a.N;
-    const int ntiles = (n_out + 15) / 16;
-    const int per_cu = smem <= 76 * 1024 ? 2 : 1;
-    // every workgroup takes the same number of tiles (or one fewer): 896 tiles on 512 slots run as 448 x 2
-    const int slots = device_cus() * per_cu;
-    const int rounds = (ntiles + slots - 1) / slots;
-    const int grid = (ntiles + rounds - 1) / rounds;
+    return best;
+}
+
+template <int PRO, int EPI, int TM, int WAVES>
+int launch_resident_plan(SkinnyArgs a, const ResidentPlan &p, int ntiles, const Workspace &ws, hipStream_t stream) {
+    constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
+    a.S = p.S;
+    a.slice = p.slice;
+    a.ssq_off = (int)(p.stage + p.red);
+    if (p.S > 1) {
+        a.counters = (int *)ws.base;
+        a.ws = (float *)((unsigned char *)ws.base + kCounterBytes);
+        a.ws_ssq = a.ws + (size_t)ntiles * p.S * RT * kWave * 4;
+    }
+    // One workgroup per slot of the chip and slice, tiles dealt out in turn: the first slots of the
+    // compute units get one tile more than the second ones when the tiles do not divide evenly.
+    int groups = device_cus() * p.per_cu / p.S;
+    if (groups < 1) groups = 1;
+    if (groups > ntiles) groups = ntiles;
     static bool attribute_set = false;   // more than the default 64 KiB of dynamic LDS has to be asked for once
     if (!attribute_set) {
-        const hipError_t e = hipFuncSetAttribute((const void *)skinny_resident_kernel<PRO, EPI>,
+        const hipError_t e = hipFuncSetAttribute((const void *)skinny_resident_kernel<PRO, EPI, TM, WAVES>,
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         FLLM_REQUIRE(e == hipSuccess, "linear_skinny: cannot raise the LDS limit: %s", hipGetErrorString(e));
         attribute_set = true;
     }
-    hipLaunchKernelGGL((skinny_resident_kernel<PRO, EPI>), dim3(grid), dim3(WAVES * kWave), smem, stream, a, (int)stage);
+    hipLaunchKernelGGL((skinny_resident_kernel<PRO, EPI, TM, WAVES>), dim3(groups * p.S), dim3(WAVES * kWave), p.smem, stream,
+                       a, (int)p.stage);
     return fllm_check_launch("linear_skinny");
+}
+
+template <int PRO, int EPI>
+int launch_resident(const SkinnyArgs &a, hipStream_t stream) {
+    constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
+    Workspace ws;
+    {
+        void *base = nullptr;
+        size_t bytes = 0;
+        if (fllm_device_workspace(&base, &bytes)) ws.base = (float *)base, ws.bytes = bytes;
+    }
+    const int n_out = EPI == EPI_SWIGLU ? a.N / 2 : a.N;
+    const int tiles16 = (n_out + 15) / 16, tiles8 = (n_out + 7) / 8;
+    if constexpr (EPI == EPI_SWIGLU) {
+        const ResidentPlan p = plan_resident(a.M, a.K, tiles8, RT, ws);
+        if (p.S == 0) return 1;
+        if (p.waves == 8) return launch_resident_plan<PRO, EPI, TM_GATEUP, 8>(a, p, tiles8, ws, stream);
+        return launch_resident_plan<PRO, EPI, TM_GATEUP, 16>(a, p, tiles8, ws, stream);
+    } else {
+        ResidentPlan p = plan_resident(a.M, a.K, tiles16, RT, ws);
+        if (p.S == 0) return 1;
+        // 8-row tiles (two K halves a product) when the rows allow it and the 16-row tiles come to between half a
+        // tile and two tiles per slot, unevenly: 384 tiles on 512 slots run as long as 512 would
+        const int slots = device_cus() * p.per_cu;
+        const bool dual = a.M <= 8 && p.S == 1 && fllm_option_dual_k() && 2 * tiles16 > slots && tiles16 < 2 * slots &&
+                          tiles16 % slots != 0;
+        if (dual) {
+            if (p.waves == 8) return launch_resident_plan<PRO, EPI, TM_DUALK, 8>(a, p, tiles8, ws, stream);
+            return launch_resident_plan<PRO, EPI, TM_DUALK, 16>(a, p, tiles8, ws, stream);
+        }
+        if (p.waves == 8) return launch_resident_plan<PRO, EPI, TM_ROWS16, 8>(a, p, tiles16, ws, stream);
+        return launch_resident_plan<PRO, EPI, TM_ROWS16, 16>(a, p, tiles16, ws, stream);
+    }
 }
 
 template <int MT, int WAVES, int EPI>
@@ -435,7 +583,9 @@ int fllm_linear_bf16_skinny(const void *x, int ldx, const void *w, const float *
 }
 
 // The fused forms read the float32 rows once per workgroup: worth it while there are few rows.
-extern "C" int fllm_fused_decode_supported(int M, int K) { return (M >= 1 && M <= 16 && K % 8 == 0) ? 1 : 0; }
+extern "C" int fllm_fused_decode_supported(int M, int K) {
+    return (M >= 1 && M <= 16 && K % 8 == 0 && K >= 8 && K <= 65536) ? 1 : 0;
+}
 
 extern "C" int fllm_norm_linear(const float *x, const float *norm_w, float eps, const void *w, const float *bias, void *out,
                                 int M, int N, int K, hipStream_t stream) {

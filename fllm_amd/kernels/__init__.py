@@ -76,6 +76,8 @@ def load_library(build_if_missing: bool = True):
     lib.fllm_fused_decode_supported.restype = c_int
     lib.fllm_set_option.argtypes = [ctypes.c_char_p, c_int]
     lib.fllm_set_option.restype = c_int
+    lib.fllm_set_device_workspace.argtypes = [c_void, c_size]
+    lib.fllm_set_device_workspace.restype = c_int
     lib.fllm_set_fast_kernels.argtypes = [c_int]
     lib.fllm_set_fast_kernels.restype = None
     lib.fllm_attention_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int, c_int]
@@ -115,6 +117,20 @@ class Ops:
             raise KernelError("no GPU is visible: the engine runs on gfx950 only")
         self.lib = load_library()
         self.library_gemm_from = library_gemm_from
+        self._device_workspace(torch.cuda.current_device())
+
+    _WORKSPACE_BYTES = 32 << 20
+    _workspaces = {}         # device index -> tensor; lives as long as the process: the library keeps its address
+
+    def _device_workspace(self, device: int) -> None:
+        """Hands the library the memory in which workgroups of one kernel meet (counters, partial sums): once per device."""
+        if device in Ops._workspaces:
+            return
+        with torch.cuda.device(device):
+            buf = torch.zeros(Ops._WORKSPACE_BYTES, dtype=torch.uint8, device=f"cuda:{device}")
+            torch.cuda.synchronize()
+            self._check(self.lib.fllm_set_device_workspace(_ptr(buf), buf.numel()))
+        Ops._workspaces[device] = buf
 
     def set_fast_kernels(self, on: bool) -> None:
         """Off: bfloat16 calls run the plain kernels (tests compare the two)."""

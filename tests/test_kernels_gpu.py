@@ -145,7 +145,11 @@ def test_linear_f32_row_is_the_same_alone_and_in_a_batch(ops):
 
 
 SKINNY = [(1, 16, 64), (1, 4096, 4096), (2, 100, 136), (5, 6144, 4096), (8, 4096, 14336), (16, 520, 264),
-          (17, 128, 128), (33, 1000, 4096), (64, 4096, 4096), (48, 30, 72)]
+          (17, 128, 128), (33, 1000, 4096), (64, 4096, 4096), (48, 30, 72),
+          # 8-row weight tiles with two K halves (up to 8 rows, 4,100 to 16,000 outputs), ragged in N and K
+          (3, 5001, 64), (7, 6148, 200), (8, 4104, 1096), (1, 9000, 520),
+          # K in slices over workgroups (the rows of all of K do not fit into LDS), 8 and 16 waves
+          (16, 136, 14336), (5, 1000, 30008), (12, 72, 65536)]
 TILED = [(65, 128, 64), (128, 200, 200), (200, 6144, 4096), (300, 130, 136), (2048, 512, 4096), (129, 4096, 14336)]
 PLAIN = [(3, 50, 100), (70, 64, 36)]      # K not a multiple of 8: the plain kernel
 
@@ -170,6 +174,42 @@ def test_add_residual(ops, dtype, rows, width):
     branch = torch.randn(rows, width, generator=g).to(dtype)
     got = ops.add_residual(residual.to(DEV), branch.to(DEV))
     assert torch.equal(got.cpu(), residual + branch.float())
+
+
+@pytest.mark.parametrize("M,N,K,option,values", [
+    (8, 6144, 4096, "linear.dual_k", (0, 1)), (3, 5001, 200, "linear.dual_k", (0, 1)),
+    (8, 4096, 14336, "linear.slices", (0, 2, 4, 8)), (2, 1000, 4096, "linear.slices", (0, 2, 4)),
+    (16, 264, 8192, "linear.slices", (0, 4))])
+def test_linear_bf16_variants_agree(ops, ref, M, N, K, option, values):
+    """The ways of cutting a decode-shaped product (tile shape, K slices) give the same sums up to the order
+    of float32 additions, each of them the same bits on every call."""
+    g = gen(44)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    want = ref.linear(x, w, torch.zeros(M, N, dtype=torch.float64))
+    mag = (x.double().abs() @ w.double().abs().T).max().item()
+    xg, wg = x.to(DEV), w.to(DEV)
+    try:
+        for value in values:
+            ops.set_option(option, value)
+            outs = [ops.linear(xg, wg, torch.empty(M, N, dtype=torch.float32, device=DEV)) for _ in range(4)]
+            close(outs[0], want, 1e-6, 4e-7 * mag + 1e-6, f"{option}={value}")
+            for other in outs[1:]:
+                assert torch.equal(other, outs[0]), f"{option}={value}: two calls differ"
+    finally:
+        ops.set_option(option, 1 if option == "linear.dual_k" else 0)
+
+
+def test_sliced_products_leave_their_counters_at_zero(ops, ref):
+    """Products of different shapes share the counters of the K-sliced form: each must hand them back at zero."""
+    g = gen(45)
+    for M, N, K in [(8, 4096, 14336), (5, 1000, 30008), (16, 136, 14336), (8, 4096, 14336), (9, 96, 14336)]:
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+        want = ref.linear(x, w, torch.zeros(M, N, dtype=torch.float64))
+        mag = (x.double().abs() @ w.double().abs().T).max().item()
+        got = ops.linear(x.to(DEV), w.to(DEV), torch.empty(M, N, dtype=torch.float32, device=DEV))
+        close(got, want, 1e-6, 4e-7 * mag + 1e-6, f"sliced M{M} N{N} K{K}")
 
 
 def test_linear_bf16_strided_input(ops, ref):
@@ -328,8 +368,10 @@ def test_rope_kv_store(ops, ref, dtype, heads, kv_heads, head_dim, rope_dims, pa
 
 
 # ---------------------------------------------------------------------------------------------
-def attention_case(ops, ref, dtype, heads, kv_heads, head_dim, page_size, segs, window, seed, fast=True, spike=False):
-    """segs: (first position, rows) per segment."""
+def attention_case(ops, ref, dtype, heads, kv_heads, head_dim, page_size, segs, window, seed, fast=True, spike=False,
+                   bound=None, calls=1):
+    """segs: (first position, rows) per segment.  bound: the context bound handed to the kernel (a decode graph's
+    is larger than any context of the step); calls: launches in a row, which must give the same bits."""
     g = gen(seed)
     rows = sum(n for _, n in segs)
     max_context = max(p + n for p, n in segs)
@@ -362,12 +404,17 @@ def attention_case(ops, ref, dtype, heads, kv_heads, head_dim, page_size, segs, 
     uniform = int(all(n == 1 for _, n in segs))
     ops.set_fast_kernels(fast)
     try:
-        nbytes = ops.attention_workspace_bytes(rows, heads, kv_heads, head_dim, max_context)
+        bound = max_context if bound is None else bound
+        nbytes = ops.attention_workspace_bytes(rows, heads, kv_heads, head_dim, bound)
         ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=DEV)
-        got = ops.attention(qkv.to(DEV)[:, : heads * head_dim], k.to(DEV), v.to(DEV), tables.to(DEV), row_pos.to(DEV),
-                            row_seg.to(DEV), seg_start.to(DEV), torch.empty(rows, heads * head_dim, dtype=dtype, device=DEV),
-                            heads, kv_heads, head_dim, page_size, scale, window, max_context, uniform_rows=uniform,
-                            workspace=ws)
+        args = (qkv.to(DEV)[:, : heads * head_dim], k.to(DEV), v.to(DEV), tables.to(DEV), row_pos.to(DEV), row_seg.to(DEV),
+                seg_start.to(DEV))
+        got = None
+        for _ in range(calls):
+            out = ops.attention(*args, torch.empty(rows, heads * head_dim, dtype=dtype, device=DEV),
+                                heads, kv_heads, head_dim, page_size, scale, window, bound, uniform_rows=uniform, workspace=ws)
+            assert got is None or torch.equal(out, got), "two launches of the same attention differ"
+            got = out
     finally:
         ops.set_fast_kernels(True)
     if dtype == torch.float32:
@@ -417,6 +464,21 @@ def test_attention_window(ops, ref, dtype, heads, kv_heads, head_dim, page_size,
 def test_attention_far_key_stands_out(ops, ref, dtype, segs, window):
     attention_case(ops, ref, dtype, 8, 2, 64, 16, segs, window, 13, spike=True)
     attention_case(ops, ref, dtype, 32, 8, 128, 16, segs, window, 14, spike=True)
+
+
+@pytest.mark.parametrize("fused_merge", [1, 0])
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(8, 2, 64, 16), (32, 8, 128, 16), (5, 1, 32, 8)])
+@pytest.mark.parametrize("segs,bound,window", [([(999, 1), (5, 1), (640, 1)], 2048, None), ([(1100, 1)], 4096, None),
+                                                ([(300, 1), (2500, 1)], 8192, 700), ([(0, 1)], 1024, None)])
+def test_attention_decode_split_contexts(ops, ref, fused_merge, heads, kv_heads, head_dim, page_size, segs, bound, window):
+    """A decode step splits its contexts over workgroups by the bound of the step, not by the contexts themselves:
+    splits without keys, one split alone, and the merge by the last split or by a second kernel."""
+    ops.set_option("attention.fused_merge", fused_merge)
+    try:
+        attention_case(ops, ref, torch.bfloat16, heads, kv_heads, head_dim, page_size, segs, window, 16, spike=True,
+                       bound=bound, calls=3)
+    finally:
+        ops.set_option("attention.fused_merge", 1)
 
 
 def test_attention_row_is_the_same_alone_and_in_a_batch(ops, ref):
