@@ -66,10 +66,48 @@ __device__ __forceinline__ void sum_waves(const f32x4_t *red, int stride_t, int 
     }
 }
 
+// What an epilogue reads from global memory besides the sums.  The resident kernel asks for it while the
+// products of the item are still running, so that the end of an item waits for no load.
+struct EpilogueOperands {
+    bool have = false;     // resid / cs / sn hold this item's values
+    f32x4_t resid;         // EPI_ADD: out[m, nb .. nb + 3]
+    float cs[2], sn[2];    // EPI_QKV: cosine and sine of the two pairs at nb, nb + 2
+    int seg = -1, pos = 0, page = 0;   // EPI_QKV: the row's segment, position and page (do not depend on the item)
+};
+
+template <int EPI>
+__device__ __forceinline__ void load_row_operands(const SkinnyArgs &a, int m, EpilogueOperands &e) {
+    if (EPI != EPI_QKV || m >= a.M) return;
+    e.seg = a.row_seg[m];
+    e.pos = a.row_pos[m];
+    if (e.seg >= 0 && a.store_kv) e.page = a.tables[(size_t)e.seg * a.table_stride + e.pos / a.page_size];
+}
+
+template <int EPI>
+__device__ __forceinline__ void load_item_operands(const SkinnyArgs &a, int m, int nb, int n_out, EpilogueOperands &e) {
+    e.have = false;
+    if (m >= a.M || nb >= n_out) return;
+    if (EPI == EPI_ADD) {
+        if (nb + 3 < n_out && (a.ldo & 3) == 0 && ((uintptr_t)a.out & 15) == 0) {
+            e.resid = *(const f32x4_t *)((const float *)a.out + (size_t)m * a.ldo + nb);
+            e.have = true;
+        }
+    } else if (EPI == EPI_QKV) {
+        const int d = a.head_dim;
+        const int hd = nb / d, j = nb - hd * d;
+        if (e.seg >= 0 && hd < a.heads + a.kv_heads && j + 3 < a.rope_dims) {
+            const float *cs = a.cos_t + (size_t)e.pos * (a.rope_dims / 2) + j / 2, *sn = a.sin_t + (size_t)e.pos * (a.rope_dims / 2) + j / 2;
+            e.cs[0] = cs[0], e.cs[1] = cs[1], e.sn[0] = sn[0], e.sn[1] = sn[1];
+            e.have = true;
+        }
+    }
+}
+
 // What happens to the finished sums of one output group: row scale of the norm, bias, then the store.
 // ss: the row's sum of squares (norm prologue).
 template <int PRO, int EPI, int RT>
-__device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], float ss, int m, int nb, int n_out) {
+__device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], float ss, int m, int nb, int n_out,
+                                         const EpilogueOperands &e) {
     const int N = a.N, K = a.K;
     if (PRO == PRO_NORM_F32) {
         const float inv = 1.0f / sqrtf(ss / (float)K + a.eps);
@@ -83,7 +121,9 @@ __device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], 
             for (int i = 0; i < 4; i++)
                 if (nb + i < n_out) s[t][i] += a.bias[t * n_out + nb + i];
     }
-    if (EPI == EPI_STORE || EPI == EPI_STORE_F32 || EPI == EPI_ADD) {
+    if (EPI == EPI_ADD && e.have) {
+        *(f32x4_t *)((float *)a.out + (size_t)m * a.ldo + nb) = e.resid + s[0];
+    } else if (EPI == EPI_STORE || EPI == EPI_STORE_F32 || EPI == EPI_ADD) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int n = nb + i;
@@ -102,9 +142,9 @@ __device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], 
             ((bf16_t *)a.out)[(size_t)m * a.ldo + n] = (bf16_t)(gt / (1.0f + expf(-gt)) * up);
         }
     } else {   // EPI_QKV: N = (heads + 2 kv_heads) * head_dim, head_dim a multiple of 4, so nb..nb+3 lie in one head
-        const int seg = a.row_seg[m];
+        const int seg = e.seg;
         if (seg < 0) return;
-        const int pos = a.row_pos[m];
+        const int pos = e.pos;
         const int d = a.head_dim;
         const int hd = nb / d, j = nb - hd * d;          // head (q heads, then k heads, then v heads), lane in head
         float v[4] = {s[0][0], s[0][1], s[0][2], s[0][3]};
@@ -114,9 +154,10 @@ __device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], 
             for (int p = 0; p < 2; p++) {
                 if (j + 2 * p < a.rope_dims) {
                     const int l2 = (j + 2 * p) / 2;
+                    const float c = e.have ? e.cs[p] : cs[l2], sv = e.have ? e.sn[p] : sn[l2];
                     const float x0 = v[2 * p], x1 = v[2 * p + 1];
-                    v[2 * p] = x0 * cs[l2] - x1 * sn[l2];
-                    v[2 * p + 1] = x1 * cs[l2] + x0 * sn[l2];
+                    v[2 * p] = x0 * c - x1 * sv;
+                    v[2 * p + 1] = x1 * c + x0 * sv;
                 }
             }
         }
@@ -125,7 +166,7 @@ __device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], 
 #pragma unroll
             for (int i = 0; i < 4; i++) q[i] = (bf16_t)v[i];
         } else if (a.store_kv) {
-            const int page = a.tables[(size_t)seg * a.table_stride + pos / a.page_size];
+            const int page = e.page;
             const int off = pos % a.page_size;
             if (hd < a.heads + a.kv_heads) {
                 const int kvh = hd - a.heads;
@@ -222,6 +263,17 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
     bf16x8_t b0[U], b1[U];
     issue(b0);      // in flight while the activations are staged
     issue(b1);
+    // what the epilogue reads besides the sums: the part that belongs to this lane's row now, the part that belongs
+    // to an item when the wave whose turn it is to finish the item starts on it
+    const int m_out = TM == TM_DUALK ? (r & 7) : r;
+    const bool owner = TM == TM_ROWS16 ? true : (g < 2 && (TM == TM_GATEUP || r < 8));
+    EpilogueOperands eo;
+    load_row_operands<EPI>(a, m_out, eo);
+    auto item_operands = [&](int it) {
+        if (S == 1 && it < my_items && wave == (it & (WAVES - 1)) && owner)
+            load_item_operands<EPI>(a, m_out, (tile0 + it * tstride) * NT + g * 4, n_out, eo);
+    };
+    item_operands(0);
 
     // the wave's own columns kw0 .. kw1 of every row
     if (PRO == PRO_NORM_F32 && lane < 16) ssq_part[wave * 16 + lane] = 0.f;
@@ -297,9 +349,8 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
         __syncthreads();
         const int tile = tile0 + item * tstride;
         const bool finisher = wave == (item & (WAVES - 1));
-        // D[row 4 g + i][column r]: for the 8-output tiles the lanes g < 2 hold outputs 4 g + i, and their partners
-        // sit 32 lanes on (TM_GATEUP: the up rows) or 32 + 8 lanes on (TM_DUALK: the other K half)
-        const bool owner = TM == TM_ROWS16 ? true : (g < 2 && (TM == TM_GATEUP || r < 8));
+        // D[row 4 g + i][column r]: for the 8-output tiles the lanes g < 2 (`owner`) hold outputs 4 g + i, and their
+        // partners sit 32 lanes on (TM_GATEUP: the up rows) or 32 + 8 lanes on (TM_DUALK: the other K half)
         f32x4_t s[RT];
         if (finisher && owner) {
 #pragma unroll
@@ -314,7 +365,7 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
         __syncthreads();      // the sums have been read: the next item may overwrite them
         if (finisher) {
             do {
-                const int m = TM == TM_DUALK ? (r & 7) : r, nb = tile * NT + g * 4;
+                const int m = m_out, nb = tile * NT + g * 4;
                 float ss = 0.f;
                 if (PRO == PRO_NORM_F32) {
 #pragma unroll
@@ -358,10 +409,12 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
                     }
                 }
                 if (!owner || m >= M || nb >= n_out) break;
-                epilogue<PRO, EPI, RT>(a, s, ss, m, nb, n_out);
+                if (S > 1) eo.have = false;     // the tile was finished by whoever came last: nothing was asked for ahead
+                epilogue<PRO, EPI, RT>(a, s, ss, m, nb, n_out, eo);
             } while (false);
         }
         item++;
+        item_operands(item);
     };
 
     const int total = my_items * nbw;
@@ -418,7 +471,9 @@ skinny_direct_kernel(SkinnyArgs a) {
         if (m >= M || nb >= N) continue;
         f32x4_t s[RT];
         sum_waves<WAVES, RT>(red, MT * kWave, mt * kWave + l, s);
-        epilogue<PRO, EPI, RT>(a, s, 0.f, m, nb, N);
+        EpilogueOperands eo;
+        load_row_operands<EPI>(a, m, eo);
+        epilogue<PRO, EPI, RT>(a, s, 0.f, m, nb, N, eo);
     }
 }
 

@@ -163,6 +163,48 @@ argmax_kernel(const float *__restrict__ logits, int32_t *__restrict__ out, int v
     if (threadIdx.x == 0) out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
 }
 
+// The same over `parts` workgroups a row: each takes a stretch of the vocabulary and leaves its best (value,
+// index) in `partial`; the one that arrives last (counted in counters[row], zero before and after) picks the
+// largest value, on ties the lowest index, so the answer does not depend on who that is.
+__global__ void __launch_bounds__(kBlock)
+argmax_split_kernel(const float *__restrict__ logits, int32_t *__restrict__ out, int vocab, int parts, int per_part,
+                    float *partial_v, int *partial_i, int *counters) {
+    __shared__ Shared sh;
+    __shared__ int s_seen;
+    const int row = blockIdx.x, part = blockIdx.y;
+    const int lo = part * per_part, hi = min(vocab, lo + per_part);
+    const float *w = logits + (size_t)row * vocab;
+    float best = -INFINITY;
+    int besti = 0x7fffffff;
+    for (int i = lo + threadIdx.x; i < hi; i += kBlock) {
+        const float v = w[i];
+        if (isfinite(v) && v > best) {
+            best = v;
+            besti = i;
+        }
+    }
+    besti = block_argmax(best, besti, sh);
+    if (threadIdx.x == 0) {
+        const float bv = besti == 0x7fffffff ? -INFINITY : w[besti];
+        __hip_atomic_store(partial_v + (size_t)row * parts + part, bv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(partial_i + (size_t)row * parts + part, besti, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);      // the part has arrived before it is counted
+        s_seen = __hip_atomic_fetch_add(counters + row, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (s_seen != parts - 1) return;
+    if (threadIdx.x == 0) __hip_atomic_store(counters + row, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    float v = -INFINITY;
+    int idx = 0x7fffffff;
+    if ((int)threadIdx.x < parts) {
+        v = __hip_atomic_load(partial_v + (size_t)row * parts + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        idx = __hip_atomic_load(partial_i + (size_t)row * parts + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    idx = block_argmax(v, idx, sh);
+    if (threadIdx.x == 0) out[row] = idx == 0x7fffffff ? 0 : idx;
+}
+
 __global__ void __launch_bounds__(kBlock)
 sample_kernel(const float *logits, float *work, const FllmSampleRow *__restrict__ params,
               int32_t *__restrict__ out, int vocab) {
@@ -236,6 +278,21 @@ sample_kernel(const float *logits, float *work, const FllmSampleRow *__restrict_
 extern "C" int fllm_argmax(const float *logits, int32_t *out, int rows, int vocab, hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && vocab > 0, "argmax: bad sizes rows=%d vocab=%d", rows, vocab);
     if (rows == 0) return 0;
+    // few rows of a wide vocabulary: several workgroups a row, if the device workspace is there for them to meet in
+    void *ws = nullptr;
+    size_t ws_bytes = 0;
+    int parts = (vocab + 8191) / 8192;
+    if (parts > 64) parts = 64;
+    if (parts * rows > 2048) parts = 2048 / rows;
+    if (parts > 1 && fllm_device_workspace(&ws, &ws_bytes) && (size_t)rows * sizeof(int) <= kWorkspaceCounterBytes &&
+        kWorkspaceCounterBytes + (size_t)rows * parts * 8 <= ws_bytes) {
+        const int per_part = (vocab + parts - 1) / parts;
+        float *pv = (float *)((unsigned char *)ws + kWorkspaceCounterBytes);
+        int *pi = (int *)(pv + (size_t)rows * parts);
+        hipLaunchKernelGGL(argmax_split_kernel, dim3(rows, parts), dim3(kBlock), 0, stream, logits, out, vocab, parts, per_part,
+                           pv, pi, (int *)ws);
+        return fllm_check_launch("argmax");
+    }
     hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(kBlock), 0, stream, logits, out, vocab);
     return fllm_check_launch("argmax");
 }
