@@ -10,6 +10,7 @@ flags; rust/engine/src/tiny_model.rs:168-195 `make-tiny-model`; rust/engine/src/
     make-tiny-model OUT [--seed N] [--config FILE] [--dtype float32|bfloat16]
     selftest-gpu [--only GROUPS] [--list]                                   kernels against PyTorch on the device
     replay --model DIR --dtype D --out DIR --max-tokens N                   same as bin/trace_run
+    trace-summary DIR [--steps N]                                           per-kernel time of the last steps of a rocprofv3 trace
 """
 from __future__ import annotations
 
@@ -156,7 +157,12 @@ def cmd_replay(argv: List[str]) -> int:
     return main(argv)
 
 
-COMMANDS = {"run": cmd_run, "inspect": cmd_inspect, "make-tiny-model": cmd_make_tiny_model,
+def cmd_trace_summary(argv: List[str]) -> int:
+    from .kernels.trace_summary import main
+    return main(argv)
+
+
+COMMANDS = {"trace-summary": cmd_trace_summary, "run": cmd_run, "inspect": cmd_inspect, "make-tiny-model": cmd_make_tiny_model,
             "selftest-gpu": cmd_selftest, "replay": cmd_replay}
 
 

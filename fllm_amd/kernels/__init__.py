@@ -208,9 +208,11 @@ class Ops:
         if bias is not None:
             _dense(bias, "bias", torch.float32, (N,))
         if (self.library_gemm_from is not None and M >= self.library_gemm_from and x.dtype == torch.bfloat16
-                and bias is None and mode != OUT_STORE_F32):
+                and bias is None):
             if mode == OUT_STORE:
                 torch.matmul(x, w.t(), out=out)
+            elif mode == OUT_STORE_F32:
+                torch.mm(x, w.t(), out_dtype=torch.float32, out=out)     # bfloat16 operands, float32 sums stored as they are
             else:
                 self.add_residual(out, torch.matmul(x, w.t()))
             return out
