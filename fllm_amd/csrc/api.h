@@ -15,7 +15,7 @@ int fllm_abi_version(void);
 // 0: bfloat16 calls use the plain kernels only (for comparing them with the MFMA kernels); default 1
 void fllm_set_fast_kernels(int on);
 // Switches a kernel variant (for measurements and tests): "attention.tile32" 0/1; "linear.slices" n
-// (0: chosen by shape); "linear.dual_k" 0/1; "attention.fused_merge" 0/1.  0 on success.
+// (0: chosen by shape); "linear.dual_k" 0/1; "linear.x_direct" 0/1; "attention.fused_merge" 0/1.  0 on success.
 int fllm_set_option(const char *name, int value);
 
 // out[r, :] = scale * table[ids[r], :]            out: float32 [rows, width]

@@ -27,6 +27,8 @@ int fllm_option_tile32(void);
 int fllm_option_linear_slices(void);
 // 1: the parts of a split decode context are merged by the split that arrives last (default); 0: by a second kernel
 int fllm_option_fused_merge(void);
+// 1: decode-shaped products read bfloat16 activations straight from global memory (default); 0: they stage them in LDS
+int fllm_option_x_direct(void);
 // 1: decode-shaped products of up to 8 rows use 8-row weight tiles with two K halves a product (default); 0: 16-row tiles
 int fllm_option_dual_k(void);
 

@@ -209,11 +209,13 @@ __device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], 
 // result does not depend on which workgroup came last.
 enum { TM_ROWS16 = 0, TM_DUALK = 1, TM_GATEUP = 2 };
 
-template <int PRO, int EPI, int TM, int WAVES>
+template <int PRO, int EPI, int TM, int WAVES, bool XD>
 __global__ void __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4, 4)))   // 16 waves a CU: 128 registers
 skinny_resident_kernel(SkinnyArgs a, int red_off) {
+    static_assert(!XD || PRO == PRO_BF16, "activations straight from global memory: the bfloat16 prologue only");
     constexpr int U = 4;                           // k-steps of 32 per block: four 16-byte loads per lane
     constexpr int KB = 32 * U;                     // K elements of one range per block
+    constexpr int RB = 4;                          // rows of activations staged at a time (more would spill registers)
     constexpr int NT = TM == TM_ROWS16 ? 16 : 8;   // outputs per row and tile
     constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
     static_assert((EPI == EPI_SWIGLU) == (TM == TM_GATEUP), "gate/up tiles belong to the SwiGLU epilogue");
@@ -240,14 +242,20 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
     const int nbw = (half + KB - 1) / KB;
     // this lane's A row and B column: weight row in the tile, activation row, and where its K range starts
     const int wrow_in_tile = TM == TM_ROWS16 ? r : (r & 7) + (TM == TM_GATEUP ? (r >> 3) * n_out : 0);
-    const int xrow_i = TM == TM_DUALK ? (r & 7) : r;
     const int kr0 = kw0 + (TM == TM_DUALK ? (r >> 3) * half : 0) + g * 8;      // relative to ks0
     const int kr1 = TM == TM_DUALK ? min(kw1, kw0 + ((r >> 3) + 1) * half) : kw1;
     const int row_limit = TM == TM_GATEUP ? n_out : N;            // weight rows past it are clamped (never stored)
 
     // cursor of the loads: (item, block in item) of the next block to ask for
     int l_item = 0, l_j = 0;
-    auto issue = [&](bf16x8_t (&buf)[U]) {
+    const int xrow_i = TM == TM_DUALK ? (r & 7) : r;
+    const bool xvalid = xrow_i < M;
+    // XD: the activations are not staged; a block's B operands come from global memory (L2) together with its weights
+    struct Block {
+        bf16x8_t w[U];
+        bf16x8_t x[XD ? U : 1];
+    };
+    auto issue = [&](Block &buf) {
         if (l_item < my_items) {
             int row = (tile0 + l_item * tstride) * NT + (TM == TM_ROWS16 ? r : (r & 7));
             if (row >= row_limit) row = row_limit - 1;
@@ -255,12 +263,17 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
             const int kb = kr0 + l_j * KB;
             const bf16_t *wp = a.w + (size_t)row * K + ks0 + kb;
 #pragma unroll
-            for (int u = 0; u < U; u++) buf[u] = kb + u * 32 < kr1 ? *(const bf16x8_t *)(wp + u * 32) : zero8();
+            for (int u = 0; u < U; u++) buf.w[u] = kb + u * 32 < kr1 ? *(const bf16x8_t *)(wp + u * 32) : zero8();
+            if (XD) {
+                const bf16_t *xp = (const bf16_t *)a.x + (size_t)xrow_i * a.ldx + ks0 + kb;
+#pragma unroll
+                for (int u = 0; u < U; u++) buf.x[XD ? u : 0] = (kb + u * 32 < kr1 && xvalid) ? *(const bf16x8_t *)(xp + u * 32) : zero8();
+            }
         }
         if (++l_j == nbw) l_j = 0, l_item++;
     };
     (void)wrow_in_tile;
-    bf16x8_t b0[U], b1[U];
+    Block b0, b1;
     issue(b0);      // in flight while the activations are staged
     issue(b1);
     // what the epilogue reads besides the sums: the part that belongs to this lane's row now, the part that belongs
@@ -278,7 +291,7 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
     // the wave's own columns kw0 .. kw1 of every row
     if (PRO == PRO_NORM_F32 && lane < 16) ssq_part[wave * 16 + lane] = 0.f;
     __builtin_amdgcn_wave_barrier();
-    for (int cw = kw0; cw < kw1; cw += kWave * 8) {   // the same trips for every lane: the sums below are over the wave
+    for (int cw = kw0; cw < (XD ? 0 : kw1); cw += kWave * 8) {   // the same trips for every lane: the sums below are over the wave
         const int c0 = cw + lane * 8;
         const bool in = c0 < kw1;
         if (PRO == PRO_BF16) {
@@ -296,10 +309,10 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
             const float *x = (const float *)a.x + ks0 + c0;
             f32x4_t w0 = {0.f, 0.f, 0.f, 0.f}, w1 = w0;
             if (in) w0 = *(const f32x4_t *)(a.norm_w + ks0 + c0), w1 = *(const f32x4_t *)(a.norm_w + ks0 + c0 + 4);
-            for (int m0 = 0; m0 < M; m0 += 4) {
-                f32x4_t xv[4][2];
+            for (int m0 = 0; m0 < M; m0 += RB) {   // the loads of RB rows are in flight together
+                f32x4_t xv[RB][2];
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
+                for (int i = 0; i < RB; i++) {
                     xv[i][0] = xv[i][1] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
                     if (in && m0 + i < M) {
                         xv[i][0] = *(const f32x4_t *)(x + (size_t)(m0 + i) * a.ldx);
@@ -307,7 +320,7 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
                     }
                 }
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
+                for (int i = 0; i < RB; i++) {
                     if (m0 + i >= M) break;
                     bf16x8_t v;
                     float ss = 0.f;
@@ -330,15 +343,17 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
     int item = 0, j = 0;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
     const bf16_t *xrow = xs + xrow_i * pitch + kr0;
-    const bool xvalid = xrow_i < M;
 
-    auto step = [&](bf16x8_t (&buf)[U]) {
+    auto step = [&](Block &buf) {
         bf16x8_t xf[U];
         const int kb = kr0 + j * KB;
 #pragma unroll
-        for (int u = 0; u < U; u++) xf[u] = (kb + u * 32 < kr1 && xvalid) ? *(const bf16x8_t *)(xrow + j * KB + u * 32) : zero8();
+        for (int u = 0; u < U; u++) {
+            if (XD) xf[u] = buf.x[XD ? u : 0];
+            else xf[u] = (kb + u * 32 < kr1 && xvalid) ? *(const bf16x8_t *)(xrow + j * KB + u * 32) : zero8();
+        }
 #pragma unroll
-        for (int u = 0; u < U; u++) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(buf[u], xf[u], acc, 0, 0, 0);
+        for (int u = 0; u < U; u++) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(buf.w[u], xf[u], acc, 0, 0, 0);
         issue(buf);      // the block two ahead takes this one's registers
         if (++j < nbw) return;
         // the item is complete: the waves' sums meet in LDS; one wave (they take turns) adds them up and goes on
@@ -505,9 +520,19 @@ struct ResidentPlan {
 // The fewest K slices whose activations fit into LDS (slicing costs more than it gains wherever it is not needed):
 // twice into a compute unit's as two workgroups of 8 waves, else once as one workgroup of 16 waves, so that as
 // many loads are in flight.
-ResidentPlan plan_resident(int M, int K, int ntiles, int rt, const Workspace &ws) {
+ResidentPlan plan_resident(int M, int K, int ntiles, int rt, const Workspace &ws, bool x_direct) {
     const int forced = fllm_option_linear_slices();
     ResidentPlan best;
+    if (x_direct) {   // nothing is staged: one slice, two workgroups of 8 waves a compute unit
+        best.S = 1;
+        best.slice = (K + 127) / 128 * 128;
+        best.waves = 8;
+        best.per_cu = 2;
+        best.stage = 0;
+        best.red = 8 * kWave * sizeof(f32x4_t);
+        best.smem = best.red + 8 * 16 * sizeof(float);
+        return best;
+    }
     for (int S = 1; S <= kMaxSlices; S *= 2) {
         const int slice = ((K + S - 1) / S + 127) / 128 * 128;
         if (S > 1 && (slice < 1024 || (S - 1) * slice >= K)) break;
@@ -531,7 +556,7 @@ ResidentPlan plan_resident(int M, int K, int ntiles, int rt, const Workspace &ws
     return best;
 }
 
-template <int PRO, int EPI, int TM, int WAVES>
+template <int PRO, int EPI, int TM, int WAVES, bool XD = false>
 int launch_resident_plan(SkinnyArgs a, const ResidentPlan &p, int ntiles, const Workspace &ws, hipStream_t stream) {
     constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
     a.S = p.S;
@@ -549,12 +574,12 @@ int launch_resident_plan(SkinnyArgs a, const ResidentPlan &p, int ntiles, const 
     if (groups > ntiles) groups = ntiles;
     static bool attribute_set = false;   // more than the default 64 KiB of dynamic LDS has to be asked for once
     if (!attribute_set) {
-        const hipError_t e = hipFuncSetAttribute((const void *)skinny_resident_kernel<PRO, EPI, TM, WAVES>,
+        const hipError_t e = hipFuncSetAttribute((const void *)skinny_resident_kernel<PRO, EPI, TM, WAVES, XD>,
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         FLLM_REQUIRE(e == hipSuccess, "linear_skinny: cannot raise the LDS limit: %s", hipGetErrorString(e));
         attribute_set = true;
     }
-    hipLaunchKernelGGL((skinny_resident_kernel<PRO, EPI, TM, WAVES>), dim3(groups * p.S), dim3(WAVES * kWave), p.smem, stream,
+    hipLaunchKernelGGL((skinny_resident_kernel<PRO, EPI, TM, WAVES, XD>), dim3(groups * p.S), dim3(WAVES * kWave), p.smem, stream,
                        a, (int)p.stage);
     return fllm_check_launch("linear_skinny");
 }
@@ -571,18 +596,28 @@ int launch_resident(const SkinnyArgs &a, hipStream_t stream) {
     const int n_out = EPI == EPI_SWIGLU ? a.N / 2 : a.N;
     const int tiles16 = (n_out + 15) / 16, tiles8 = (n_out + 7) / 8;
     if constexpr (EPI == EPI_SWIGLU) {
-        const ResidentPlan p = plan_resident(a.M, a.K, tiles8, RT, ws);
+        const ResidentPlan p = plan_resident(a.M, a.K, tiles8, RT, ws, false);
         if (p.S == 0) return 1;
         if (p.waves == 8) return launch_resident_plan<PRO, EPI, TM_GATEUP, 8>(a, p, tiles8, ws, stream);
         return launch_resident_plan<PRO, EPI, TM_GATEUP, 16>(a, p, tiles8, ws, stream);
     } else {
-        ResidentPlan p = plan_resident(a.M, a.K, tiles16, RT, ws);
+        // bfloat16 activations are read where they lie when a workgroup sees few tiles (it reads each of them once
+        // per tile: no dearer than staging for a tile or two, and nothing waits for the staging); with many tiles a
+        // workgroup, and for the norm prologue, they are staged in LDS
+        const bool x_direct = PRO == PRO_BF16 && fllm_option_x_direct() && a.ldx % 8 == 0 && tiles16 <= 4 * device_cus();
+        ResidentPlan p = plan_resident(a.M, a.K, tiles16, RT, ws, x_direct);
         if (p.S == 0) return 1;
         // 8-row tiles (two K halves a product) when the rows allow it and the 16-row tiles come to between half a
         // tile and two tiles per slot, unevenly: 384 tiles on 512 slots run as long as 512 would
         const int slots = device_cus() * p.per_cu;
         const bool dual = a.M <= 8 && p.S == 1 && fllm_option_dual_k() && 2 * tiles16 > slots && tiles16 < 2 * slots &&
                           tiles16 % slots != 0;
+        if constexpr (PRO == PRO_BF16) {
+            if (x_direct) {
+                if (dual) return launch_resident_plan<PRO, EPI, TM_DUALK, 8, true>(a, p, tiles8, ws, stream);
+                return launch_resident_plan<PRO, EPI, TM_ROWS16, 8, true>(a, p, tiles16, ws, stream);
+            }
+        }
         if (dual) {
             if (p.waves == 8) return launch_resident_plan<PRO, EPI, TM_DUALK, 8>(a, p, tiles8, ws, stream);
             return launch_resident_plan<PRO, EPI, TM_DUALK, 16>(a, p, tiles8, ws, stream);

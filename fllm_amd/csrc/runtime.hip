@@ -31,6 +31,8 @@ extern "C" void fllm_set_fast_kernels(int on) { g_fast_kernels = on ? 1 : 0; }
 static int g_tile32 = 1;
 static int g_linear_slices = 0;
 static int g_dual_k = 1;
+static int g_x_direct = 1;
+int fllm_option_x_direct(void) { return g_x_direct; }
 static int g_fused_merge = 1;
 int fllm_option_fused_merge(void) { return g_fused_merge; }
 int fllm_option_dual_k(void) { return g_dual_k; }
@@ -39,6 +41,10 @@ int fllm_option_linear_slices(void) { return g_linear_slices; }
 extern "C" int fllm_set_option(const char *name, int value) {
     if (strcmp(name, "attention.fused_merge") == 0) {
         g_fused_merge = value ? 1 : 0;
+        return 0;
+    }
+    if (strcmp(name, "linear.x_direct") == 0) {
+        g_x_direct = value ? 1 : 0;
         return 0;
     }
     if (strcmp(name, "linear.dual_k") == 0) {

@@ -178,6 +178,7 @@ def test_add_residual(ops, dtype, rows, width):
 
 @pytest.mark.parametrize("M,N,K,option,values", [
     (8, 6144, 4096, "linear.dual_k", (0, 1)), (3, 5001, 200, "linear.dual_k", (0, 1)),
+    (8, 4096, 14336, "linear.x_direct", (0, 1)), (16, 1000, 520, "linear.x_direct", (0, 1)), (3, 5001, 200, "linear.x_direct", (0, 1)),
     (8, 4096, 14336, "linear.slices", (0, 2, 4, 8)), (2, 1000, 4096, "linear.slices", (0, 2, 4)),
     (16, 264, 8192, "linear.slices", (0, 4))])
 def test_linear_bf16_variants_agree(ops, ref, M, N, K, option, values):
@@ -190,6 +191,8 @@ def test_linear_bf16_variants_agree(ops, ref, M, N, K, option, values):
     mag = (x.double().abs() @ w.double().abs().T).max().item()
     xg, wg = x.to(DEV), w.to(DEV)
     try:
+        if option == "linear.slices":
+            ops.set_option("linear.x_direct", 0)      # slices exist for staged activations only
         for value in values:
             ops.set_option(option, value)
             outs = [ops.linear(xg, wg, torch.empty(M, N, dtype=torch.float32, device=DEV)) for _ in range(4)]
@@ -197,12 +200,21 @@ def test_linear_bf16_variants_agree(ops, ref, M, N, K, option, values):
             for other in outs[1:]:
                 assert torch.equal(other, outs[0]), f"{option}={value}: two calls differ"
     finally:
-        ops.set_option(option, 1 if option == "linear.dual_k" else 0)
+        ops.set_option(option, 0 if option == "linear.slices" else 1)
+        ops.set_option("linear.x_direct", 1)
 
 
 def test_sliced_products_leave_their_counters_at_zero(ops, ref):
     """Products of different shapes share the counters of the K-sliced form: each must hand them back at zero."""
     g = gen(45)
+    ops.set_option("linear.x_direct", 0)
+    try:
+        _sliced_products(ops, ref, g)
+    finally:
+        ops.set_option("linear.x_direct", 1)
+
+
+def _sliced_products(ops, ref, g):
     for M, N, K in [(8, 4096, 14336), (5, 1000, 30008), (16, 136, 14336), (8, 4096, 14336), (9, 96, 14336)]:
         x = torch.randn(M, K, generator=g).to(torch.bfloat16)
         w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
