@@ -118,8 +118,18 @@ class Model:
     def forward(self, ctx: StepContext) -> torch.Tensor:
         """Logits (float32 [len(logit_rows), vocab]) of the step's wanted rows."""
         x = self.embedding.forward(ctx, ctx.ids)
+        pending = None      # a block's output that the next block adds together with its first norm
         for entry, binding in zip(self.spec.run_order, self.bindings):
-            self.blocks[entry.layer].forward(ctx, x, binding)
+            block = self.blocks[entry.layer]
+            if getattr(block, "takes_pending", False):
+                pending = block.forward(ctx, x, binding, pending)
+            else:
+                if pending is not None:
+                    self.rt.ops.add_residual(x, pending)
+                pending = None
+                block.forward(ctx, x, binding)
+        if pending is not None:
+            self.rt.ops.add_residual(x, pending)
         if ctx.logit_rows.numel() == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.rt.device)
         h = self.final_norm.forward(ctx, x, rows=ctx.logit_rows)

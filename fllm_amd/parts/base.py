@@ -11,7 +11,10 @@ Roles and their interfaces:
   mixer         cache_need() / state_need() say what the cache manager must keep for it;
                 forward(ctx, h[R,H], residual_f32[R,H], binding) adds its output to `residual`.
   feed_forward  forward(ctx, h[R,H], residual_f32[R,H]) adds its output to `residual`.
-  block         forward(ctx, residual_f32[R,H], binding) runs norms, mixer and feed-forward.
+  block         forward(ctx, residual_f32[R,H], binding) runs norms, mixer and feed-forward.  A block
+                with `takes_pending = True` is called as forward(ctx, residual, binding, pending): `pending`
+                is a branch [R,H] that the block before left for it to add (or None), and it returns its
+                own such branch or None.
   embedding     forward(ctx, ids[R]) -> residual_f32[R,H].
   head          forward(ctx, h[L,H]) -> logits_f32[L,V].
 

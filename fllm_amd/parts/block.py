@@ -14,25 +14,43 @@ class PreNormBlock(Block):
         self.mixer_norm = norms["mixer"]
         self.feed_forward_norm = norms["feed_forward"]
 
-    def forward(self, ctx, residual, binding):
+    takes_pending = True     # forward accepts a branch that the block before has not added yet, and may hand one on
+
+    def forward(self, ctx, residual, binding, pending=None):
+        """Runs the layer on the residual stream.  `pending`: the output of the block before, still
+        to be added; the return value is this block's own such output, or None when everything has
+        been added.  Where a sum can ride on the norm that follows it, it costs no pass of its own."""
+        ops = self.rt.ops
+        add_mixer_norm = getattr(self.mixer_norm, "add_forward", None)
+        add_ff_norm = getattr(self.feed_forward_norm, "add_forward", None)
         # a part may take the residual stream and the norm before it in one fused kernel
-        h = None
         fused = getattr(self.mixer, "forward_from_residual", None)
+        if pending is not None and (fused is not None or add_mixer_norm is None):
+            # the fused kernels read the finished residual stream; they serve steps of few rows, where the
+            # block before hands on nothing in practice
+            ops.add_residual(residual, pending)
+            pending = None
         if fused is None or not fused(ctx, residual, self.mixer_norm, binding):
-            h = self.mixer_norm.forward(ctx, residual)
+            if pending is not None:
+                h = add_mixer_norm(ctx, residual, pending)
+            else:
+                h = self.mixer_norm.forward(ctx, residual)
             # a mixer may hand back its output instead of adding it: the add then rides on the next norm
             as_branch = getattr(self.mixer, "forward_branch", None)
-            add_norm = getattr(self.feed_forward_norm, "add_forward", None)
-            branch = as_branch(ctx, h, binding) if as_branch is not None and add_norm is not None else None
+            branch = as_branch(ctx, h, binding) if as_branch is not None and add_ff_norm is not None else None
             if branch is not None:
-                h = add_norm(ctx, residual, branch)
-                self.feed_forward.forward(ctx, h, residual)
-                return
+                h = add_ff_norm(ctx, residual, branch)
+                ff_branch = getattr(self.feed_forward, "forward_branch", None)
+                out = ff_branch(ctx, h) if ff_branch is not None else None
+                if out is None:
+                    self.feed_forward.forward(ctx, h, residual)
+                return out
             self.mixer.forward(ctx, h, residual, binding)
         fused = getattr(self.feed_forward, "forward_from_residual", None)
         if fused is None or not fused(ctx, residual, self.feed_forward_norm):
             h = self.feed_forward_norm.forward(ctx, residual)
             self.feed_forward.forward(ctx, h, residual)
+        return None
 
 
 register_part("block", "prenorm", PreNormBlock)

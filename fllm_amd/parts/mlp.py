@@ -47,6 +47,23 @@ class GatedMLP(FeedForward):
         ops.linear(act, self.w_down, residual, bias=self.b_down, accumulate=True)
         return True
 
+    def forward_branch(self, ctx, h):
+        """The output as a tensor of its own instead of a sum into the residual stream (large bfloat16
+        steps whose products go to the GEMM library, which has no residual epilogue): the block lets
+        the sum ride on the next norm.  None: not taken."""
+        rt, ops = self.rt, self.rt.ops
+        rows = h.shape[0]
+        start = getattr(ops, "library_gemm_from", None)
+        if rt.dtype != torch.bfloat16 or start is None or rows < start or self.b_down is not None:
+            return None
+        gate_up = rt.empty((rows, 2 * self.inter))
+        ops.linear(h, self.w_gate_up, gate_up, bias=self.b_gate_up)
+        act = rt.empty((rows, self.inter))
+        ops.swiglu(gate_up, act)
+        out = rt.empty((rows, self.hidden))
+        ops.linear(act, self.w_down, out)
+        return out
+
     def forward(self, ctx, h, residual):
         rt, ops = self.rt, self.rt.ops
         rows = h.shape[0]
