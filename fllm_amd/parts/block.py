@@ -25,11 +25,12 @@ class PreNormBlock(Block):
         add_ff_norm = getattr(self.feed_forward_norm, "add_forward", None)
         # a part may take the residual stream and the norm before it in one fused kernel
         fused = getattr(self.mixer, "forward_from_residual", None)
-        if pending is not None and (fused is not None or add_mixer_norm is None):
-            # the fused kernels read the finished residual stream; they serve steps of few rows, where the
-            # block before hands on nothing in practice
-            ops.add_residual(residual, pending)
-            pending = None
+        if pending is not None:
+            if add_mixer_norm is None:
+                ops.add_residual(residual, pending)
+                pending = None
+            else:
+                fused = None     # the fused kernels read the finished residual stream: the sum rides on the norm instead
         if fused is None or not fused(ctx, residual, self.mixer_norm, binding):
             if pending is not None:
                 h = add_mixer_norm(ctx, residual, pending)
