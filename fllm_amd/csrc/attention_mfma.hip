@@ -335,19 +335,32 @@ attn_tile32_kernel(AttnArgs p) {
     const size_t page_elems = (size_t)nkv * ps * D;
 
     bf16x8_t kreg[CH], vreg[CH];
-    auto fetch = [&](int k0) {   // tile k0 .. k0 + 63 from the pages into registers
+    // A tile's loads depend on its page numbers: those are asked for one tile earlier than the tile's keys and
+    // values, which are asked for one tile before they are multiplied, so neither wait lies on the path.
+    int pgk[CH], pgv[CH];
+    auto pages = [&](int k0) {   // page numbers of tile k0 .. k0 + 63 (0 where the tile has no token)
+        if (k0 > p_last) return;
+        const bool inside = k0 >= lo_tile && k0 + KT - 1 <= p_last;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int kabs = k0 + k_key[c], vabs = k0 + v_koff[c];
+            pgk[c] = (inside || (kabs >= lo_tile && kabs <= p_last)) ? tbl[kabs >> psh] : 0;
+            pgv[c] = (inside || (vabs + 7 >= lo_tile && vabs <= p_last)) ? tbl[vabs >> psh] : 0;
+        }
+    };
+    auto fetch = [&](int k0) {   // tile k0 .. k0 + 63 from the pages into registers; pages(k0) has run
         const bool inside = k0 >= lo_tile && k0 + KT - 1 <= p_last;   // no edge of the context in this tile
 #pragma unroll
         for (int c = 0; c < CH; c++) {
             const int kabs = k0 + k_key[c];
             bf16x8_t v = zero8();
             if (inside || (kabs >= lo_tile && kabs <= p_last))
-                v = *(const bf16x8_t *)(p.kp + (size_t)tbl[kabs >> psh] * page_elems + k_in_page[c]);
+                v = *(const bf16x8_t *)(p.kp + (size_t)pgk[c] * page_elems + k_in_page[c]);
             kreg[c] = v;
             const int vabs = k0 + v_koff[c];
             v = zero8();
             if (inside || (vabs + 7 >= lo_tile && vabs <= p_last)) {
-                v = *(const bf16x8_t *)(p.vp + (size_t)tbl[vabs >> psh] * page_elems + v_in_page[c]);
+                v = *(const bf16x8_t *)(p.vp + (size_t)pgv[c] * page_elems + v_in_page[c]);
                 if (!inside && vabs + 7 > p_last) {   // slots past the last token hold whatever an earlier request left
 #pragma unroll
                     for (int e = 0; e < 8; e++)
@@ -368,7 +381,9 @@ attn_tile32_kernel(AttnArgs p) {
     // A row q of a 32-key block is this key of the block (see the table above)
     const int a_key = 16 * (q >> 4) + 8 * ((q >> 2) & 1) + 4 * ((q >> 3) & 1) + (q & 3);
 
+    pages(kbegin);
     fetch(kbegin);
+    pages(kbegin + KT);
     for (int k0 = kbegin; k0 <= p_last; k0 += KT) {
         __syncthreads();   // the previous tile has been read
 #pragma unroll
@@ -377,7 +392,10 @@ attn_tile32_kernel(AttnArgs p) {
             *(bf16x8_t *)(Vs + v_lds[c]) = vreg[c];
         }
         __syncthreads();
-        if (k0 + KT <= p_last) fetch(k0 + KT);   // in flight while this tile is multiplied
+        if (k0 + KT <= p_last) {   // in flight while this tile is multiplied
+            fetch(k0 + KT);
+            pages(k0 + 2 * KT);
+        }
 
         f32x16_t s[2];
 #pragma unroll
