@@ -14,7 +14,9 @@
 //
 //   tile kernel    portions of prompts: a workgroup takes up to 64 (token, head-of-group) rows of
 //                  one segment and one key/value head; keys and values go through LDS in tiles of 64.
-//   tile32 kernel  long portions: 128 rows per workgroup on 32x32x16 products (described at the kernel).
+//   tile32 kernel  head sizes 64 and 128: 128 rows per workgroup on 32x32x16 products, the next tile on its way
+//                  while the current one is multiplied (described at the kernel); faster than the tile kernel
+//                  for portions of any length.
 //   decode kernel  one row per segment: a workgroup takes (row, key/value head, context split), its
 //                  sixteen waves stride over 32-key blocks loading K and V^T straight into MFMA
 //                  operands; long contexts of small batches are split and merged by a second kernel.
@@ -515,6 +517,15 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
     for (int dt = 0; dt < DT; dt++) o[dt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
 
+    // The page numbers of a block are asked for one block ahead, so that a block waits for one memory latency
+    // (its keys and values), not for two in a row.
+    auto block_pages = [&](int kb, int &kpage, int &vpage) {
+        const int grp = kb + (c >> 2) * 8, vkey = kb + g * 8;
+        kpage = (kb < end && grp < n && grp + 8 > lo) ? tbl[grp >> psh] : 0;
+        vpage = (kb < end && vkey < n && vkey + 8 > lo) ? tbl[vkey >> psh] : 0;
+    };
+    int kpage_next, vpage_next;
+    block_pages(begin + wave * 32, kpage_next, vpage_next);
     for (int kb = begin + wave * 32; kb < end; kb += WAVES * 32) {
         // keys: A row c of tile j is key kb + 8*(c/4) + 4*j + c%4; both tiles of a lane lie in one group of 8.
         // values: lane (c, g) loads V^T[d = 16 dt + c][keys kb + 8g .. + 7].  All loads of the block are
@@ -523,8 +534,8 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
         const bool gload = grp < n && grp + 8 > lo;
         const int vkey = kb + g * 8;
         const bool vload = vkey < n && vkey + 8 > lo;
-        const int kpage = gload ? tbl[grp >> psh] : 0;
-        const int vpage = vload ? tbl[vkey >> psh] : 0;
+        const int kpage = kpage_next, vpage = vpage_next;
+        block_pages(kb + WAVES * 32, kpage_next, vpage_next);
         bf16x8_t kf[2][KD], vf[DT];
 #pragma unroll
         for (int j = 0; j < 2; j++) {
@@ -734,7 +745,7 @@ int launch(const AttnArgs &a, int uniform_rows, int max_context, void *workspace
                                a.heads, p.splits);
         return fllm_check_launch("attention_decode");
     }
-    if (D >= 64 && G <= 64 && a.rows >= 96 && fllm_option_tile32()) {   // long portions: 128 rows per workgroup on 32x32x16 products
+    if (D >= 64 && G <= 64 && fllm_option_tile32()) {   // 128 rows per workgroup on 32x32x16 products
         const int TQ = 128 / G;
         const int tiles = (a.rows + TQ - 1) / TQ + a.num_segs;   // upper bound; surplus workgroups leave at once
         hipLaunchKernelGGL(attn_tile32_kernel<(D >= 64 ? D : 64)>, dim3(tiles, a.kv_heads), dim3(kThreads), 0, stream, a);

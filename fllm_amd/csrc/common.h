@@ -21,7 +21,7 @@ void fllm_set_error(const char *fmt, ...);
 int fllm_check_launch(const char *what);
 // 0 when the MFMA kernels are switched off (tests compare them with the plain kernels)
 int fllm_fast_kernels_enabled(void);
-// 1: prompt portions of 96+ rows use the 128-row attention kernel (default); 0: the 64-row kernel
+// 1: prompt portions of heads of 64 and 128 use the 128-row attention kernel (default); 0: the 64-row kernel
 int fllm_option_tile32(void);
 // 0: the decode-shaped products choose their number of K slices themselves (default); n: n slices where that is possible
 int fllm_option_linear_slices(void);

@@ -478,6 +478,18 @@ def test_attention_far_key_stands_out(ops, ref, dtype, segs, window):
     attention_case(ops, ref, dtype, 32, 8, 128, 16, segs, window, 14, spike=True)
 
 
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(8, 2, 64, 16), (32, 8, 128, 16), (8, 8, 64, 32), (16, 1, 128, 16)])
+@pytest.mark.parametrize("segs,window", [(CHUNK_SEGS[3], None), (CHUNK_SEGS[4], None), (CHUNK_SEGS[5], None), (CHUNK_SEGS[7], 100),
+                                          ([(640, 64)], 300)])
+def test_attention_bf16_tile_kernel_of_64_rows(ops, ref, heads, kv_heads, head_dim, page_size, segs, window):
+    """Heads of 64 and 128 go to the 128-row kernel by default; the 64-row kernel serves them when that is switched off."""
+    ops.set_option("attention.tile32", 0)
+    try:
+        attention_case(ops, ref, torch.bfloat16, heads, kv_heads, head_dim, page_size, segs, window, 17, spike=True)
+    finally:
+        ops.set_option("attention.tile32", 1)
+
+
 @pytest.mark.parametrize("fused_merge", [1, 0])
 @pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(8, 2, 64, 16), (32, 8, 128, 16), (5, 1, 32, 8)])
 @pytest.mark.parametrize("segs,bound,window", [([(999, 1), (5, 1), (640, 1)], 2048, None), ([(1100, 1)], 4096, None),
