@@ -8,7 +8,7 @@ from typing import Callable, Dict, List, Optional
 
 import torch
 
-GROUPS = ["embedding", "norm", "linear", "activation", "rope_kv", "attention", "sampling"]
+GROUPS = ["embedding", "norm", "linear", "fused", "activation", "rope_kv", "attention", "sampling"]
 
 
 def _err(got: torch.Tensor, want: torch.Tensor) -> float:
@@ -33,12 +33,33 @@ def _norm(ops, dev, report):
 
 def _linear(ops, dev, report):
     for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 1e-5)):
-        for M, N, K in ((1, 4096, 4096), (5, 520, 264), (64, 1000, 4096), (200, 384, 1024), (13, 100, 72)):
+        for M, N, K in ((1, 4096, 4096), (5, 520, 264), (8, 6144, 4096), (8, 4096, 14336), (64, 1000, 4096), (200, 384, 1024),
+                        (13, 100, 72)):
             x = torch.randn(M, K, device=dev).to(dtype)
             w = (torch.randn(N, K, device=dev) / math.sqrt(K)).to(dtype)
             want = x.double() @ w.double().T
             got = ops.linear(x, w, torch.empty(M, N, device=dev, dtype=torch.float32))
             report(f"linear {dtype} {M}x{N}x{K}", _err(got, want), tol)
+
+
+def _fused(ops, dev, report):
+    """The decode forms: RMSNorm folded into the product, SwiGLU in its epilogue."""
+    for M, N, K in ((1, 4096, 4096), (8, 6144, 4096), (16, 520, 264), (9, 96, 14336)):
+        x = torch.randn(M, K, device=dev) * (1 + 4 * torch.rand(M, 1, device=dev))
+        nw = 1 + 0.1 * torch.randn(K, device=dev)
+        w = (torch.randn(N, K, device=dev) / math.sqrt(K)).to(torch.bfloat16)
+        normed = x.double() * (torch.rsqrt((x.double() ** 2).mean(-1, keepdim=True) + 1e-5) * nw.double())
+        got = ops.norm_linear(x, nw, 1e-5, w, torch.empty(M, N, device=dev, dtype=torch.bfloat16))
+        report(f"norm_linear {M}x{N}x{K}", _err(got, normed @ w.double().T), 2 ** -6)
+    for M, inter, K in ((1, 14336, 4096), (8, 432, 160), (13, 1000, 4096)):
+        x = torch.randn(M, K, device=dev) * 2
+        nw = 1 + 0.1 * torch.randn(K, device=dev)
+        w = (torch.randn(2 * inter, K, device=dev) / math.sqrt(K)).to(torch.bfloat16)
+        normed = x.double() * (torch.rsqrt((x.double() ** 2).mean(-1, keepdim=True) + 1e-5) * nw.double())
+        gu = normed @ w.double().T
+        g, u = gu[:, :inter], gu[:, inter:]
+        got = ops.norm_gate_up_swiglu(x, nw, 1e-5, w, torch.empty(M, inter, device=dev, dtype=torch.bfloat16))
+        report(f"norm_gate_up_swiglu {M}x{inter}x{K}", _err(got, g * torch.sigmoid(g) * u), 2 ** -6)
 
 
 def _activation(ops, dev, report):
@@ -115,7 +136,7 @@ def _sampling(ops, dev, report):
     report("argmax first maximum", 0.0 if ok else 1.0, 0.0)
 
 
-_CHECKS: Dict[str, Callable] = {"embedding": _embedding, "norm": _norm, "linear": _linear, "activation": _activation,
+_CHECKS: Dict[str, Callable] = {"embedding": _embedding, "norm": _norm, "linear": _linear, "fused": _fused, "activation": _activation,
                                 "rope_kv": _rope_kv, "attention": _attention, "sampling": _sampling}
 
 
