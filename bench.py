@@ -4,7 +4,8 @@ weights, synthetic token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers N]
 
-A step is one decode step of the whole engine (scheduler, step function, sampling).  The one
+A step is one decode step of the whole engine (scheduler, step function, sampling), with steps
+launched ahead of the tokens of the step before them (--no-ahead: each step waits for the last).  The one
 JSON line on standard output holds decoded tokens per second at the default batch (8), the same
 at batch 1 and 64 under "points", a 2,048-token prefill under "prefill" and the decode step's
 share of the HBM roofline under "roofline".
@@ -61,6 +62,7 @@ def main():
     ap.add_argument("--layers", type=int, default=LLAMA_31_8B["num_hidden_layers"],
                     help="fewer layers than the model has (both numbers are reported)")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    ap.add_argument("--no-ahead", action="store_true", help="every step waits for the tokens of the step before it")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run the 2,048-token prefill steps alone and print their time (for profiling); no JSON line")
     args = ap.parse_args()
@@ -80,7 +82,7 @@ def main():
     t0 = time.time()
     engine = Engine(config=cfg, seed=0, dtype="bfloat16", device="cuda:0", ctx=CONTEXT, max_seqs=max(batches),
                     max_batched_tokens=PREFILL_TOKENS, block_size=PAGE_SIZE, num_blocks=-(-need_tokens // PAGE_SIZE),
-                    decode_first=True, random_weights_on_device=True)
+                    decode_first=True, random_weights_on_device=True, ahead=not args.no_ahead)
     print(f"[bench] engine ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
     rng = np.random.default_rng(0)
     vocab = cfg["vocab_size"]
@@ -122,6 +124,8 @@ def main():
             torch.cuda.synchronize()
             start = time.perf_counter()
             events = engine.step()
+            while not events:               # with steps launched ahead the token is handed out by the next call
+                events = engine.step()
             torch.cuda.synchronize()
             times.append(time.perf_counter() - start)
             assert len(events) == 1 and events[0].finished

@@ -106,18 +106,16 @@ class CacheManager:
         return max(0, length - group.window + 1) // group.page_size
 
     def pages_missing(self, req_id, total: int) -> List[int]:
-        """Pages each group would have to hand out so that positions below `total` are covered."""
+        """Pages each group would have to hand out so that positions below `total` are covered.
+        Every table entry from the first page still needed to the end of the table holds a page
+        (`reserve` fills them, `commit` takes pages away only below that point, `trim` only at the
+        end), so what is missing is the stretch behind the table."""
         req = self._get(req_id)
         out = []
         for g, group in enumerate(self.groups):
             need_upto = -(-total // group.page_size)
-            table = req.tables[g]
-            first = self._first_needed_page(group, req.length)
-            missing = 0
-            for i in range(first, need_upto):
-                if i >= len(table) or table[i] < 0:
-                    missing += 1
-            out.append(missing)
+            have_upto = max(len(req.tables[g]), self._first_needed_page(group, req.length))
+            out.append(max(0, need_upto - have_upto))
         return out
 
     def can_reserve(self, req_id, total: int) -> bool:
@@ -134,11 +132,11 @@ class CacheManager:
             need_upto = -(-total // group.page_size)
             table = req.tables[g]
             first = self._first_needed_page(group, req.length)
+            start = max(first, len(table))          # entries below `first` are never read again: they stay empty
             while len(table) < need_upto:
                 table.append(-1)
-            for i in range(first, need_upto):
-                if table[i] < 0:
-                    table[i] = self.pools[g].alloc()
+            for i in range(start, need_upto):
+                table[i] = self.pools[g].alloc()
 
     def commit(self, req_id, count: int) -> None:
         """The request holds `count` more tokens; pages a window has passed go back."""
@@ -190,6 +188,11 @@ class CacheManager:
                                          f"tables hold it {held.get(page, 0)} times")
                 if (pool.refcounts[page] == 0) != (page in set(free)):
                     raise AssertionError(f"group {g}: page {page} is neither free nor held, or both")
+        for req_id, req in self._requests.items():
+            for g, group in enumerate(self.groups):
+                first = self._first_needed_page(group, req.length)
+                if any(page < 0 for page in req.tables[g][first:]):
+                    raise AssertionError(f"group {g}: request {req_id!r} misses a page it may still read")
         slots = [r.slot for r in self._requests.values()]
         if len(set(slots)) != len(slots) or set(slots) & set(self._free_slots):
             raise AssertionError("a state slot is held twice")

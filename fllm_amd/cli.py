@@ -35,6 +35,7 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--long-prefill-token-threshold", type=int, default=0)
     ap.add_argument("--preemption-mode", default="recompute", choices=["recompute", "none"])
     ap.add_argument("--chunked-prefill-policy", default="decode-first", choices=["decode-first", "prefill-first"])
+    ap.add_argument("--ahead", action="store_true", help="launch a step before the tokens of the step before it are read")
 
 
 def _make_engine(args, model):
@@ -44,7 +45,7 @@ def _make_engine(args, model):
                   gpu_memory_utilization=args.gpu_memory_utilization, kv_watermark_blocks=args.kv_watermark_blocks,
                   max_num_partial_prefills=args.max_num_partial_prefills,
                   long_prefill_token_threshold=args.long_prefill_token_threshold, preemption_mode=args.preemption_mode,
-                  decode_first=args.chunked_prefill_policy == "decode-first")
+                  decode_first=args.chunked_prefill_policy == "decode-first", ahead=args.ahead)
 
 
 def cmd_run(argv: List[str]) -> int:

@@ -90,6 +90,11 @@ int fllm_attention(const void *q, int q_stride, const void *k_pages, const void 
                    void *workspace, size_t workspace_bytes, hipStream_t stream);
 size_t fllm_attention_workspace_bytes(int rows, int heads, int kv_heads, int head_dim, int max_context);
 
+// ids[r] = previous[source[r]] where source[r] >= 0: token ids that an earlier step chose and that have not left
+// the device yet become the input of this step
+int fllm_carry_ids(int32_t *ids, const int32_t *source, const int32_t *previous, int rows, int previous_rows,
+                   hipStream_t stream);
+
 // out[r] = first index of the largest finite value of logits[r, :]
 int fllm_argmax(const float *logits, int32_t *out, int rows, int vocab, hipStream_t stream);
 

@@ -355,3 +355,20 @@ extern "C" int fllm_rope_kv_store(void *qkv, const int32_t *row_pos, const int32
         FLLM_REQUIRE(false, "rope_kv_store: unknown dtype %d", dtype);
     return fllm_check_launch("rope_kv_store");
 }
+
+namespace {
+__global__ void carry_ids_kernel(int32_t *__restrict__ ids, const int32_t *__restrict__ source, const int32_t *__restrict__ previous,
+                                 int rows) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r < rows && source[r] >= 0) ids[r] = previous[source[r]];
+}
+}  // namespace
+
+extern "C" int fllm_carry_ids(int32_t *ids, const int32_t *source, const int32_t *previous, int rows, int previous_rows,
+                              hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && previous_rows >= 0, "carry_ids: bad sizes");
+    (void)previous_rows;      // the host has checked every source against it
+    if (rows == 0) return 0;
+    hipLaunchKernelGGL(carry_ids_kernel, dim3((rows + 255) / 256), dim3(256), 0, stream, ids, source, previous, rows);
+    return fllm_check_launch("carry_ids");
+}

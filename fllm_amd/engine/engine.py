@@ -43,6 +43,18 @@ class EngineStats:
     postprocess_s: float = 0.0
 
 
+PENDING = -1      # stands in a sequence's token list for a token that is still on the device
+
+
+@dataclass
+class _InFlight:
+    """A launched step whose tokens have not been read: sequence ids in row order, where each
+    token goes in its sequence, and the device tensor that will hold them."""
+    sampled: List[int]
+    at: List[int]
+    tokens: torch.Tensor
+
+
 class Engine:
     def __init__(self, model: Union[str, None] = None, *, config: Optional[dict] = None, seed: int = 0,
                  dtype: str = "bfloat16", device: str = "cuda:0", ctx: Optional[int] = None, max_seqs: int = 16,
@@ -50,13 +62,19 @@ class Engine:
                  gpu_memory_utilization: float = 0.90, decode_first: bool = True, kv_watermark_blocks: int = 0,
                  max_num_partial_prefills: int = 0, long_prefill_token_threshold: int = 0,
                  preemption_mode: str = "recompute", eos_token_ids: Optional[Seq[int]] = None,
-                 random_weights_on_device: bool = False, ops=None):
+                 random_weights_on_device: bool = False, ops=None, ahead: bool = False):
         """`model`: a folder with config.json and safetensors; or `config` (a config.json dict)
         with `seed` for random weights (drawn on the host, or on the device with a stream of its
         own when `random_weights_on_device`: large models).  Option names follow the reference's server flags
         (rust/engine/src/bin/serve.rs:530-557, :681-782): ctx, max_seqs, max_batched_tokens,
         gpu_memory_utilization, kv_watermark_blocks, max_num_partial_prefills,
-        long_prefill_token_threshold, preemption_mode."""
+        long_prefill_token_threshold, preemption_mode.
+
+        `ahead`: a step is launched before the tokens of the step before it have reached the host
+        (the reference's ahead step, rust/engine/src/rust_decoder.rs:1165-1266): the device takes
+        them from the earlier step's output, the host plans the next step while the device runs
+        this one, and `step()` returns the events of the step before.  A request that stops at a
+        token (end of sequence, stop id) has one more row in flight by then; that row is dropped."""
         if (model is None) == (config is None):
             raise ValueError("give either a model folder or a config for random weights")
         if model is not None:
@@ -85,6 +103,8 @@ class Engine:
         self.stats = EngineStats()
         self._requests: Dict[str, int] = {}
         self._next_seq = 0
+        self.ahead = bool(ahead)
+        self._in_flight: Optional[_InFlight] = None
 
     # ---- requests -------------------------------------------------------------------------
     def add_request(self, request_id: str, prompt_token_ids: Seq[int], sampling: Optional[SamplingParams] = None) -> int:
@@ -111,22 +131,28 @@ class Engine:
             self.scheduler.finish(sid)
 
     def has_unfinished(self) -> bool:
-        return self.scheduler.has_work()
+        return self.scheduler.has_work() or self._in_flight is not None
 
     # ---- one round ------------------------------------------------------------------------
     def step(self) -> List[TokenEvent]:
+        """Schedules and runs one step.  Returns the tokens it produced; with `ahead`, those of the
+        step before, while this one runs."""
         t0 = time.perf_counter()
         plan = self.scheduler.schedule()
         t1 = time.perf_counter()
         self.stats.scheduler_s += t1 - t0
         self.stats.preemptions = self.scheduler.preemptions
+        earlier, self._in_flight = self._in_flight, None
         if plan is None:
+            if earlier is not None:
+                return self._resolve(earlier)
             if self.scheduler.has_work():
                 raise RuntimeError("scheduler could not make progress with the available KV pool")
             return []
         seqs = self.scheduler.sequences
         entries: List[StepEntry] = []
         sampled: List[int] = []                  # sequence ids whose row gives a token, in row order
+        row_of = {sid: r for r, sid in enumerate(earlier.sampled)} if earlier is not None else {}
         for sid, start, count in plan.prefill:
             seq = seqs[sid]
             last = start + count == seq.prefill_target
@@ -135,35 +161,56 @@ class Engine:
                 sampled.append(sid)
             self.stats.prefill_rows += count
         for sid in plan.decode:
-            entries.append(StepEntry(sid, [seqs[sid].tokens[-1]], [0]))
+            token = seqs[sid].tokens[-1]
+            entries.append(StepEntry(sid, [token], [0], carry=row_of[sid] if token == PENDING else None))
             sampled.append(sid)
             self.stats.decode_rows += 1
-        logits = self.runner.step(entries)
+        logits = self.runner.step(entries, previous_tokens=earlier.tokens if earlier is not None else None)
         rows = sum(len(e.tokens) for e in entries)
         self.stats.forward_calls += 1
         self.stats.rows_total += rows
         self.stats.max_rows = max(self.stats.max_rows, rows)
         requests = [SampleRequest(seqs[sid].sampling, seqs[sid].sampling.seed_for(sid), seqs[sid].draws) for sid in sampled]
-        tokens = self.sampler.sample(logits, requests)
-        t2 = time.perf_counter()
-        self.stats.forward_s += t2 - t1
+        launched = _InFlight(sampled, [], self.sampler.launch(logits, requests))
+        # What does not depend on the tokens' values: the sequences grow by one (a placeholder until the
+        # token is read), the prompt portions count as computed.
         for sid, _, count in plan.prefill:
             self.scheduler.commit_chunk(sid, count)
-        events: List[TokenEvent] = []
-        for sid, token in zip(sampled, tokens):
+        for sid in sampled:
             seq = seqs[sid]
-            seq.tokens.append(token)
+            launched.at.append(len(seq.tokens))
+            seq.tokens.append(PENDING)
             if not seq.sampling.greedy:
                 seq.draws += 1
             self.scheduler.commit_decode(sid)
+        if self.ahead:
+            self._in_flight = launched
+            events = self._resolve(earlier) if earlier is not None else []
+        else:
+            events = self._resolve(launched)
+        self.stats.forward_s += time.perf_counter() - t1
+        return events
+
+    def _resolve(self, step: _InFlight) -> List[TokenEvent]:
+        """Reads a launched step's tokens (waits for the device), puts them where the placeholders
+        are and finishes the requests that end with them."""
+        t0 = time.perf_counter()
+        tokens = self.sampler.read(step.tokens)
+        seqs = self.scheduler.sequences
+        events: List[TokenEvent] = []
+        for sid, at, token in zip(step.sampled, step.at, tokens):
+            seq = seqs.get(sid)
+            if seq is None:
+                continue                         # finished or aborted while this row was in flight
+            seq.tokens[at] = token
             hit_stop = seq.sampling.stops_on(token, self.eos_token_ids)
-            hit_limit = seq.remaining() == 0
+            hit_limit = at + 1 - seq.prompt_len >= seq.sampling.max_tokens
             reason = "stop" if hit_stop else ("length" if hit_limit else None)
             if reason:
                 self.scheduler.finish(sid)
                 self._requests.pop(seq.req_id, None)
             events.append(TokenEvent(seq.req_id, token, reason is not None, reason))
-        self.stats.postprocess_s += time.perf_counter() - t2
+        self.stats.postprocess_s += time.perf_counter() - t0
         return events
 
     # ---- whole requests -------------------------------------------------------------------

@@ -50,10 +50,13 @@ class StepError(ValueError):
 
 @dataclass
 class StepEntry:
-    """A request's next tokens.  `want`: indices into `tokens` whose logits are returned."""
+    """A request's next tokens.  `want`: indices into `tokens` whose logits are returned.
+    `carry`: for an entry of one token that an earlier step chose and that is still on the
+    device, its row in that step's token tensor (`tokens[0]` is then a placeholder)."""
     req_id: object
     tokens: Sequence[int]
     want: Sequence[int] = ()
+    carry: Optional[int] = None
 
 
 class ModelRunner:
@@ -128,7 +131,7 @@ class ModelRunner:
         return self.cache.length(req_id)
 
     # ---- the step -------------------------------------------------------------------------
-    def _validate(self, entries: Sequence[StepEntry]) -> None:
+    def _validate(self, entries: Sequence[StepEntry], previous_tokens: Optional[torch.Tensor] = None) -> None:
         if not entries:
             raise StepError("a step needs at least one entry")
         if len(entries) > self.max_requests:
@@ -141,7 +144,13 @@ class ModelRunner:
             n = len(e.tokens)
             if n == 0:
                 raise StepError(f"request {e.req_id!r} brings no tokens")
-            for t in e.tokens:
+            if e.carry is not None:
+                if n != 1:
+                    raise StepError(f"request {e.req_id!r}: only an entry of one token can take it from an earlier step")
+                if previous_tokens is None or not 0 <= int(e.carry) < previous_tokens.numel():
+                    raise StepError(f"request {e.req_id!r} takes row {e.carry} of an earlier step's tokens, which has "
+                                    f"{0 if previous_tokens is None else previous_tokens.numel()}")
+            for t in (e.tokens if e.carry is None else ()):
                 if not 0 <= int(t) < self.vocab_size:
                     raise StepError(f"token id {t} of request {e.req_id!r} is outside [0, {self.vocab_size})")
             for w in e.want:
@@ -151,11 +160,12 @@ class ModelRunner:
             if start + n > self.max_context:
                 raise StepError(f"request {e.req_id!r} would hold {start + n} tokens, the context is {self.max_context}")
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], previous_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Runs the entries as one batch and returns float32 logits [wanted, vocab] on the device,
         in the order of the entries and of each entry's `want`.  Unknown requests are added.
-        Raises `OutOfPages` (nothing changed) when the pages do not suffice."""
-        self._validate(entries)
+        Raises `OutOfPages` (nothing changed) when the pages do not suffice.
+        `previous_tokens`: the int32 device tensor that entries with `carry` take their token from."""
+        self._validate(entries, previous_tokens)
         added = []
         try:
             for e in entries:
@@ -179,9 +189,9 @@ class ModelRunner:
             raise
         logits = None
         if self.use_graphs and all(len(e.tokens) == 1 for e in entries) and len(entries) <= GRAPH_BUCKETS[-1]:
-            logits = self._graph_step(entries)
+            logits = self._graph_step(entries, previous_tokens)
         if logits is None:
-            ctx = self._build_context(entries)
+            ctx = self._build_context(entries, previous_tokens)
             logits = self.model.forward(ctx)
         for e in entries:
             self.cache.commit(e.req_id, len(e.tokens))
@@ -190,7 +200,8 @@ class ModelRunner:
         return logits
 
     # ---- decode steps as HIP graphs ---------------------------------------------------------
-    def _graph_step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def _graph_step(self, entries: Sequence[StepEntry], previous_tokens: Optional[torch.Tensor] = None
+                    ) -> Optional[torch.Tensor]:
         """A step of single-token entries, padded to a bucket and replayed as a graph.  The graph is
         captured at the first use of a (rows, context bound) pair, after one eager run of the same
         shape.  Padding rows belong to no segment (row_seg -1): they store nothing and their output
@@ -213,7 +224,7 @@ class ModelRunner:
         h = graph.host_np
         h[:] = graph.template
         B = bucket
-        h[0:count] = [int(e.tokens[0]) for e in entries]
+        h[0:count] = [int(e.tokens[0]) if e.carry is None else 0 for e in entries]
         h[B:B + count] = starts
         h[2 * B:2 * B + count] = np.arange(count)
         h[4 * B + 1:4 * B + 1 + count] = [self.cache.slot(e.req_id) for e in entries]
@@ -224,8 +235,13 @@ class ModelRunner:
                 t = self.cache.table(e.req_id, g)
                 tables[i, :len(t)] = t
             o += B * width
+        carried = any(e.carry is not None for e in entries)
+        if carried:
+            h[graph.carry_at:graph.carry_at + count] = [-1 if e.carry is None else int(e.carry) for e in entries]
         graph.device_buf.copy_(graph.host_buf, non_blocking=True)
         graph.done.record()
+        if carried:
+            self.rt.ops.carry_ids(graph.ctx.ids, graph.carry_source, previous_tokens)
         if graph.graph is None:
             graph.capture()
         graph.graph.replay()
@@ -238,19 +254,24 @@ class ModelRunner:
         index = torch.tensor(wanted, dtype=torch.long, device=self.device)
         return graph.logits.index_select(0, index)
 
-    def _build_context(self, entries: Sequence[StepEntry]) -> StepContext:
+    def _build_context(self, entries: Sequence[StepEntry], previous_tokens: Optional[torch.Tensor] = None) -> StepContext:
         ids: List[int] = []
         row_pos: List[int] = []
         row_seg: List[int] = []
         slots: List[int] = []
         logit_rows: List[int] = []
         seg_rows, seg_start = [], []
+        carry: Dict[int, int] = {}              # row -> row of the earlier step's tokens
         max_context = 0
         for s, e in enumerate(entries):
             start = self.cache.length(e.req_id)
             n = len(e.tokens)
             base = len(ids)
-            ids.extend(int(t) for t in e.tokens)
+            if e.carry is not None:
+                carry[base] = int(e.carry)
+                ids.append(0)
+            else:
+                ids.extend(int(t) for t in e.tokens)
             row_pos.extend(range(start, start + n))
             row_seg.extend([s] * n)
             slots.append(self.cache.slot(e.req_id))
@@ -271,9 +292,13 @@ class ModelRunner:
         cu_rows = [0]
         for n in seg_rows:
             cu_rows.append(cu_rows[-1] + n)
-        packed = torch.tensor(ids + row_pos + row_seg + cu_rows + slots + logit_rows + flat_tables, dtype=torch.int32)
-        packed = packed.to(self.device, non_blocking=False)
         R, L = len(ids), len(logit_rows)
+        source = [carry.get(r, -1) for r in range(R)] if carry else []
+        packed = torch.tensor(ids + row_pos + row_seg + cu_rows + slots + logit_rows + flat_tables + source, dtype=torch.int32)
+        if self.device.type == "cuda":   # from pinned memory, so that the copy does not wait for the step before
+            packed = packed.pin_memory().to(self.device, non_blocking=True)
+        else:
+            packed = packed.to(self.device)
         o = 0
 
         def take(count):
@@ -284,6 +309,8 @@ class ModelRunner:
 
         t_ids, t_pos, t_seg, t_cu, t_slots, t_rows = take(R), take(R), take(R), take(S + 1), take(S), take(L)
         tables = [take(S * w).view(S, w) for w in widths]
+        if carry:
+            self.rt.ops.carry_ids(t_ids, take(R), previous_tokens)
         return StepContext(num_rows=R, num_segments=S, ids=t_ids, row_pos=t_pos, row_seg=t_seg, seg_start=t_cu,
                            slots=t_slots,
                            logit_rows=t_rows, tables=tables, seg_rows=seg_rows, seg_pos_start=seg_start,
@@ -301,13 +328,15 @@ class _DecodeGraph:
         self.bucket = bucket
         self.bound = bound
         B = bucket
-        size = 6 * B + 1 + sum(B * w for w in widths)
+        self.carry_at = 6 * B + 1 + sum(B * w for w in widths)     # behind the tables: where each row's token comes from
+        size = self.carry_at + B
         self.host_buf = torch.zeros(size, dtype=torch.int32, pin_memory=True)
         self.host_np = self.host_buf.numpy()
         template = np.zeros(size, dtype=np.int32)
         template[2 * B:3 * B] = -1                              # row_seg of padding rows
         template[3 * B:4 * B + 1] = np.arange(B + 1)            # one row per segment
         template[5 * B + 1:6 * B + 1] = np.arange(B)            # logits of every row
+        template[self.carry_at:self.carry_at + B] = -1          # tokens come from the host
         self.template = template
         self.device_buf = torch.zeros(size, dtype=torch.int32, device=runner.device)
         self.done = torch.cuda.Event()
@@ -322,6 +351,7 @@ class _DecodeGraph:
                                seg_start=d[3 * B:4 * B + 1], slots=d[4 * B + 1:5 * B + 1],
                                logit_rows=d[5 * B + 1:6 * B + 1], tables=tables, seg_rows=[1] * B,
                                seg_pos_start=[0] * B, seg_slots=[0] * B, max_context=bound, uniform_rows=True)
+        self.carry_source = d[self.carry_at:self.carry_at + B]
         self.graph = None
         self.logits = None
 

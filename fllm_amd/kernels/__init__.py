@@ -66,6 +66,7 @@ def load_library(build_if_missing: bool = True):
         "fllm_norm_qkv_rope_store": [c_void, c_void, c_float, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void,
                                      c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_argmax": [c_void, c_void, c_int, c_int, c_void],
+        "fllm_carry_ids": [c_void, c_void, c_void, c_int, c_int, c_void],
         "fllm_sample": [c_void, c_void, c_void, c_void, c_int, c_int, c_void],
     }
     for name, args in sig.items():
@@ -360,6 +361,16 @@ class Ops:
             int(window) if window else 0, _DTYPE_CODE[q.dtype], int(max_context), int(uniform_rows), ws_ptr, ws_bytes,
             self._stream()))
         return out
+
+    def carry_ids(self, ids: torch.Tensor, source: torch.Tensor, previous: torch.Tensor) -> torch.Tensor:
+        """ids[r] = previous[source[r]] where source[r] >= 0 (int32 device tensors): tokens an earlier step chose
+        become this step's input without passing through the host."""
+        rows = ids.numel()
+        _dense(ids, "ids", torch.int32)
+        _dense(source, "source", torch.int32, (rows,))
+        _dense(previous, "previous", torch.int32)
+        self._check(self.lib.fllm_carry_ids(_ptr(ids), _ptr(source), _ptr(previous), rows, previous.numel(), self._stream()))
+        return ids
 
     def argmax(self, logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         rows, vocab = logits.shape

@@ -38,16 +38,28 @@ class Sampler:
 
     def sample(self, logits: torch.Tensor, rows: Sequence[SampleRequest]) -> List[int]:
         """`logits`: float32 [len(rows), vocab] on the device.  Returns one token id per row."""
+        return self.read(self.launch(logits, rows))
+
+    @staticmethod
+    def read(tokens: torch.Tensor) -> List[int]:
+        """The token ids of `launch` on the host (waits for the device)."""
+        return [int(t) for t in tokens.cpu().tolist()]
+
+    def launch(self, logits: torch.Tensor, rows: Sequence[SampleRequest]) -> torch.Tensor:
+        """Starts the choice of one token per row and returns the int32 device tensor that will
+        hold them; nothing waits for the device."""
         count = logits.shape[0]
         if count != len(rows):
             raise ValueError(f"{count} rows of logits for {len(rows)} requests")
-        if count == 0:
-            return []
         out = torch.empty(count, dtype=torch.int32, device=logits.device)
+        if count == 0:
+            return out
         if all(r.params.greedy for r in rows):
             self.rt.ops.argmax(logits, out)
         else:
-            params = pack_rows(rows).to(logits.device)
+            params = pack_rows(rows)
+            if logits.is_cuda:      # from pinned memory, so that the copy does not wait for the device
+                params = params.pin_memory().to(logits.device, non_blocking=True)
             work = torch.empty_like(logits)
             self.rt.ops.sample(logits, work, params, out)
-        return [int(t) for t in out.cpu().tolist()]
+        return out

@@ -141,6 +141,12 @@ class ReferenceOps:
                 out[r, h * head_dim:(h + 1) * head_dim] = (p @ v[:, h // group, :]).to(out.dtype)
         return out
 
+    def carry_ids(self, ids, source, previous):
+        for r in range(ids.numel()):
+            if int(source[r]) >= 0:
+                ids[r] = previous[int(source[r])]
+        return ids
+
     def argmax(self, logits, out):
         for r in range(logits.shape[0]):
             row = logits[r].float().cpu().numpy()

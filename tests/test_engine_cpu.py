@@ -152,3 +152,56 @@ def test_eos_from_config_stops_unless_ignored():
     assert Engine(config=cfg, seed=1, **base).generate([PROMPTS_A[1]], SamplingParams(max_tokens=8)) == [first]
     ignored = Engine(config=cfg, seed=1, **base).generate([PROMPTS_A[1]], SamplingParams(max_tokens=8, ignore_eos=True))
     assert len(ignored[0]) == 8 and ignored[0][:2] == first
+
+
+# ---- steps launched ahead of the tokens of the step before ----------------------------------
+def test_ahead_generation_gives_the_same_tokens():
+    """Greedy and seeded sampling, prompt portions mixed with decode rows, few pages with preemption:
+    launching a step before the last one's tokens are read changes no token."""
+    greedy = SamplingParams(max_tokens=16)
+    assert make_engine(ahead=True).generate(PROMPTS_A, greedy) == [plain_greedy("A", p, 16) for p in PROMPTS_A]
+    tight = make_engine(num_blocks=5, ahead=True)
+    assert tight.generate(PROMPTS_A, greedy) == make_engine().generate(PROMPTS_A, greedy)
+    assert tight.stats.preemptions >= 1
+    tight.runner.cache.check_invariants()
+    params = SamplingParams(max_tokens=6, temperature=0.8, top_p=0.95, seed=1234)
+    prompts = [tc.random_ids(n, 512, 20 + n) for n in (1, 9, 40)]
+    assert (make_engine("B", max_batched_tokens=32, ahead=True).generate(prompts, params)
+            == make_engine("B", max_batched_tokens=32).generate(prompts, params))
+
+
+def test_ahead_events_come_one_step_later_and_stop_where_they_should():
+    first = plain_greedy("A", PROMPTS_A[0], 5)
+    engine = make_engine(ahead=True)
+    engine.add_request("stop", PROMPTS_A[0], SamplingParams(max_tokens=16, stop_token_ids=(first[2],)))
+    engine.add_request("length", PROMPTS_A[1], SamplingParams(max_tokens=2))
+    engine.add_request("long", PROMPTS_A[0], SamplingParams(max_tokens=5))
+    assert engine.step() == []                       # the first step is in flight: nothing to hand out yet
+    events = []
+    while engine.has_unfinished():
+        events += engine.step()
+    by_request = {}
+    for e in events:
+        by_request.setdefault(e.request_id, []).append(e)
+    assert [e.token_id for e in by_request["stop"]] == first[:3]          # the row launched past the stop token is dropped
+    assert by_request["stop"][-1].finish_reason == "stop"
+    assert len(by_request["length"]) == 2 and by_request["length"][-1].finish_reason == "length"
+    assert [e.token_id for e in by_request["long"]] == first and by_request["long"][-1].finish_reason == "length"
+    assert all(not e.finished for evs in by_request.values() for e in evs[:-1])
+    engine.runner.cache.check_invariants()
+    assert engine.runner.cache.requests() == []
+
+
+def test_ahead_abort_drops_the_row_in_flight():
+    engine = make_engine(ahead=True)
+    engine.add_request("a", PROMPTS_A[0], SamplingParams(max_tokens=8))
+    engine.add_request("b", PROMPTS_A[1], SamplingParams(max_tokens=8))
+    engine.step()
+    engine.step()
+    engine.abort_request("a")
+    events = []
+    while engine.has_unfinished():
+        events += engine.step()
+    assert all(e.request_id == "b" for e in events)
+    assert [e.token_id for e in events][-3:] == plain_greedy("A", PROMPTS_A[1], 8)[-3:]
+    engine.runner.cache.check_invariants()

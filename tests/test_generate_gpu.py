@@ -96,6 +96,26 @@ def test_sampled_generation_is_reproducible(dtype):
     assert make_engine("B", dtype).generate(prompts, SamplingParams(max_tokens=24, temperature=0.8, seed=1)) != a
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_launched_ahead_give_the_same_tokens(dtype):
+    """With `ahead` the device takes a decode row's token from the output of the step before; the tokens are the
+    same as when every step waits for the last: greedy and sampled, graphs and eager steps, few pages."""
+    prompts = [tc.random_ids(n, 512, 20 + n) for n in PROMPT_LENGTHS["B"]]
+    for params in (SamplingParams(max_tokens=24), SamplingParams(max_tokens=24, temperature=0.8, top_p=0.9, seed=7)):
+        want = make_engine("B", dtype).generate(prompts, params)
+        ahead = make_engine("B", dtype, ahead=True)
+        assert ahead.generate(prompts, params) == want
+        assert ahead.runner.graph_replays > 0
+        ahead.runner.cache.check_invariants()
+        eager = make_engine("B", dtype, ahead=True)
+        eager.runner.use_graphs = False
+        assert eager.generate(prompts, params) == want
+    tight = make_engine("B", dtype, ahead=True, num_blocks=26)
+    assert tight.generate(prompts, SamplingParams(max_tokens=24)) == make_engine("B", dtype).generate(prompts, SamplingParams(max_tokens=24))
+    assert tight.stats.preemptions >= 1
+    tight.runner.cache.check_invariants()
+
+
 def test_command_line(tmp_path):
     folder = str(tmp_path / "model")
     write_random_model(folder, tc.TINY_A, seed=1, dtype="float32")
