@@ -51,6 +51,9 @@ int fllm_set_device_workspace(void *workspace, size_t bytes);
 //                             queries as bfloat16 [M, heads * head_dim] and keys and values into the pages
 //                             (layouts and row/segment/table arguments as fllm_rope_kv_store)
 int fllm_fused_decode_supported(int M, int K);
+// out = silu(x gate^T) * (x up^T) for bfloat16 rows x [M, K] (1..64 rows, row stride ldx), w = [gate; up] ([2 I, K])
+int fllm_gate_up_swiglu(const void *x, int ldx, const void *w_gate_up, const float *bias, void *out, int M, int inter,
+                        int K, hipStream_t stream);
 int fllm_norm_linear(const float *x, const float *norm_w, float eps, const void *w, const float *bias, void *out, int M,
                      int N, int K, hipStream_t stream);
 int fllm_norm_gate_up_swiglu(const float *x, const float *norm_w, float eps, const void *w_gate_up, const float *bias,

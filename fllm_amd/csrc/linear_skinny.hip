@@ -440,55 +440,178 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// 17 to 64 rows: operands straight from global memory, one weight row tile per workgroup
+// 17 to 64 rows: a workgroup of four waves takes four weight row tiles and a K slice
 // ---------------------------------------------------------------------------------------------
-template <int MT, int WAVES, int EPI>
-__global__ void __launch_bounds__(WAVES * kWave)
-skinny_direct_kernel(SkinnyArgs a) {
-    constexpr int RT = 1, PRO = PRO_BF16;
-    constexpr int THREADS = WAVES * kWave;
-    constexpr int U = 4;
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+// Every wave owns one 16-row weight tile (8 gate + 8 up rows for the SwiGLU form) for the whole K
+// slice of its workgroup, so no sums cross waves.  The activations of the slice pass through LDS in
+// chunks of 256 columns, shared by the four waves, the next chunk on its way from global memory
+// while the current one is multiplied (two buffers, one barrier per chunk).  The weights go from
+// global memory straight into MFMA A operands, two chunks (16 KiB a wave) in flight ahead of the
+// products, across chunk, tile and item borders.  Workgroup b owns slice b % S and the row groups
+// b / S, b / S + G / S, ...  With S > 1 a wave leaves its tile's sums in the workspace and counts
+// the tile; the wave that counts the last slice adds the S partial sums in slice order and runs
+// the epilogue (as in the resident kernel).
+template <int MT, int EPI>
+__global__ void __launch_bounds__(4 * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
+skinny_wide_kernel(SkinnyArgs a) {
+    constexpr int WAVES = 4, THREADS = WAVES * kWave;
+    constexpr int KC = 256;                        // columns per chunk
+    constexpr int KS = KC / 32;                    // MFMA k-steps per chunk
+    constexpr int XP = KC + 8;                     // pitch of an activation row in LDS
+    constexpr int ROWS = MT * 16;
+    constexpr int XL = ROWS * (KC / 8) / THREADS;  // 16-byte activation loads per thread and chunk
+    constexpr int NT = EPI == EPI_SWIGLU ? 8 : 16; // outputs per row and tile
+    constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
+    static_assert(ROWS * (KC / 8) % THREADS == 0, "the chunk divides evenly over the threads");
+    __shared__ __attribute__((aligned(16))) bf16_t xs[2][ROWS * XP];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int r = lane & 15, g = lane >> 4;
-    const int M = a.M, N = a.N, K = a.K;
-    const int n0 = blockIdx.x * 16;
-    int wrow = n0 + r;
-    if (wrow >= N) wrow = N - 1;   // past the end: computed from a valid row, never stored
-    const bf16_t *wp = a.w + (size_t)wrow * K + g * 8;
+    const int M = a.M, N = a.N, K = a.K, S = a.S;
+    const int n_out = EPI == EPI_SWIGLU ? N / 2 : N;
+    const int ntiles = (n_out + NT - 1) / NT;
+    const int ngroups = (ntiles + WAVES - 1) / WAVES;
+    const int sl = blockIdx.x % S;
+    const int rg0 = blockIdx.x / S, rstride = gridDim.x / S;
+    const int ks0 = sl * a.slice;
+    const int kcn = min(K, ks0 + a.slice) - ks0;                  // columns of this slice, a multiple of 8
+    const int nchunks = (kcn + KC - 1) / KC;
+    const int my_items = rg0 < ngroups ? (ngroups - rg0 + rstride - 1) / rstride : 0;
+    const int total = my_items * nchunks;                         // chunk steps of this workgroup, the same for every wave
     const bf16_t *x = (const bf16_t *)a.x;
+
+    // weights: cursor (item, chunk) of the next chunk to ask for
+    int w_item = 0, w_chunk = 0;
+    auto issue_w = [&](bf16x8_t (&buf)[KS]) {
+        if (w_item < my_items) {
+            const int tile = (rg0 + w_item * rstride) * WAVES + wave;
+            int row = tile * NT + (EPI == EPI_SWIGLU ? (r & 7) : r);
+            if (row >= n_out) row = n_out - 1;    // past the end: computed from a valid row, never stored
+            if (EPI == EPI_SWIGLU) row += (r >> 3) * n_out;
+            const int kb = w_chunk * KC + g * 8;
+            const bf16_t *wp = a.w + (size_t)row * K + ks0 + kb;
+#pragma unroll
+            for (int u = 0; u < KS; u++) buf[u] = kb + u * 32 < kcn ? *(const bf16x8_t *)(wp + u * 32) : zero8();
+        }
+        if (++w_chunk == nchunks) w_chunk = 0, w_item++;
+    };
+    // activations: the chunk index within the slice is all that matters (every item walks the same slice)
+    bf16x8_t xr[XL];
+    auto load_x = [&](int chunk) {
+#pragma unroll
+        for (int i = 0; i < XL; i++) {
+            const int idx = threadIdx.x + i * THREADS;
+            const int m = idx / (KC / 8), c = (idx - m * (KC / 8)) * 8 + chunk * KC;
+            xr[i] = (m < M && c < kcn) ? *(const bf16x8_t *)(x + (size_t)m * a.ldx + ks0 + c) : zero8();
+        }
+    };
+    auto store_x = [&](int buffer) {
+#pragma unroll
+        for (int i = 0; i < XL; i++) {
+            const int idx = threadIdx.x + i * THREADS;
+            const int m = idx / (KC / 8), c = (idx - m * (KC / 8)) * 8;
+            *(bf16x8_t *)(&xs[buffer][m * XP + c]) = xr[i];
+        }
+    };
+
+    bf16x8_t wa[KS], wb[KS];
+    issue_w(wa);
+    issue_w(wb);
+    if (total > 0) {
+        load_x(0);
+        store_x(0);
+    }
+    __syncthreads();
+
     f32x4_t acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) acc[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-    for (int k0 = wave * 32 * U; k0 < K; k0 += WAVES * 32 * U) {
-        bf16x8_t wf[U], xf[MT][U];
+    int item = 0, chunk = 0;
+
+    auto step = [&](bf16x8_t (&buf)[KS], int q) {
+        const int next_chunk = chunk + 1 == nchunks ? 0 : chunk + 1;
+        if (q + 1 < total) load_x(next_chunk);      // on its way while this chunk is multiplied
+        const bf16_t *xb = &xs[q & 1][r * XP + g * 8];
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int k = k0 + u * 32 + g * 8;
-            const bool in = k < K;
-            wf[u] = in ? *(const bf16x8_t *)(wp + k0 + u * 32) : zero8();
+        for (int u = 0; u < KS; u++) {
+            bf16x8_t xf[MT];
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++)
-                xf[mt][u] = (in && mt * 16 + r < M) ? *(const bf16x8_t *)(x + (size_t)(mt * 16 + r) * a.ldx + k) : zero8();
+            for (int mt = 0; mt < MT; mt++) xf[mt] = *(const bf16x8_t *)(xb + mt * 16 * XP + u * 32);
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(buf[u], xf[mt], acc[mt], 0, 0, 0);
         }
+        issue_w(buf);      // the chunk two ahead takes this one's registers
+        if (q + 1 < total) store_x((q + 1) & 1);
+        __syncthreads();   // the next chunk is in LDS; everybody has read the one before it
+        chunk = next_chunk;
+        if (chunk != 0) return;
+        // the item is complete: this wave's tile has its sums over the slice
+        const int tile = (rg0 + item * rstride) * WAVES + wave;
+        item++;
+        const bool owner = EPI == EPI_SWIGLU ? g < 2 : true;      // 8-output tiles: lanes g < 2 hold gate rows, g >= 2 the up rows
+        const int nb = tile * NT + g * 4;
 #pragma unroll
-        for (int u = 0; u < U; u++)
+        for (int mt = 0; mt < MT; mt++) {
+            f32x4_t s[RT];
+            s[0] = acc[mt];
+            if (EPI == EPI_SWIGLU) {
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], xf[mt][u], acc[mt], 0, 0, 0);
-    }
-    f32x4_t *red = (f32x4_t *)smem;   // [WAVES][MT][64]
+                for (int i = 0; i < 4; i++) s[RT - 1][i] = __shfl(acc[mt][i], (lane + 32) & 63, kWave);
+            }
+            acc[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+            const int m = mt * 16 + r;
+            bool finish = tile < ntiles;
+            if (S > 1 && tile < ntiles) {       // wave-uniform: the whole wave takes part in the hand-over
+                float *part = a.ws + (((size_t)tile * S + sl) * MT + mt) * RT * kWave * 4 + (size_t)lane * 4;
+                if (owner && m < M) {
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++) red[(wave * MT + mt) * kWave + lane] = acc[mt];
-    __syncthreads();
-    for (int e = threadIdx.x; e < MT * kWave; e += THREADS) {
-        const int mt = e / kWave, l = e % kWave;
-        const int m = mt * 16 + (l & 15), nb = n0 + (l >> 4) * 4;
-        if (m >= M || nb >= N) continue;
-        f32x4_t s[RT];
-        sum_waves<WAVES, RT>(red, MT * kWave, mt * kWave + l, s);
-        EpilogueOperands eo;
-        load_row_operands<EPI>(a, m, eo);
-        epilogue<PRO, EPI, RT>(a, s, 0.f, m, nb, N, eo);
+                    for (int t = 0; t < RT; t++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++)
+                            __hip_atomic_store(part + t * kWave * 4 + i, s[t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                if (mt == MT - 1) {
+                    // every access to the workspace goes to the device's point of coherence by itself: it is enough
+                    // that the wave's partial sums have arrived there before the tile is counted
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                    __builtin_amdgcn_s_waitcnt(0);
+                    int seen = 0;
+                    if (lane == 0) seen = __hip_atomic_fetch_add(a.counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    seen = __shfl(seen, 0, kWave);
+                    if (seen == S - 1) {        // the last slice of this tile: add the parts in slice order
+                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                        if (lane == 0) __hip_atomic_store(a.counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                        for (int mt2 = 0; mt2 < MT; mt2++) {
+                            const int m2 = mt2 * 16 + r;
+                            if (!owner || m2 >= M || nb >= n_out) continue;
+                            f32x4_t t2[RT];
+#pragma unroll
+                            for (int t = 0; t < RT; t++) t2[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+                            for (int s2 = 0; s2 < S; s2++) {
+                                const float *src = a.ws + (((size_t)tile * S + s2) * MT + mt2) * RT * kWave * 4 + (size_t)lane * 4;
+#pragma unroll
+                                for (int t = 0; t < RT; t++)
+#pragma unroll
+                                    for (int i = 0; i < 4; i++)
+                                        t2[t][i] += __hip_atomic_load(src + t * kWave * 4 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            }
+                            EpilogueOperands eo;
+                            epilogue<PRO_BF16, EPI, RT>(a, t2, 0.f, m2, nb, n_out, eo);
+                        }
+                    }
+                }
+                finish = false;
+            }
+            if (finish && owner && m < M && nb < n_out) {
+                EpilogueOperands eo;
+                epilogue<PRO_BF16, EPI, RT>(a, s, 0.f, m, nb, n_out, eo);
+            }
+        }
+    };
+
+    for (int q = 0; q < total; q += 2) {
+        step(wa, q);
+        if (q + 1 < total) step(wb, q + 1);
     }
 }
 
@@ -627,26 +750,58 @@ int launch_resident(const SkinnyArgs &a, hipStream_t stream) {
     }
 }
 
-template <int MT, int WAVES, int EPI>
-int launch_direct(const SkinnyArgs &a, hipStream_t stream) {
-    const size_t smem = (size_t)WAVES * MT * kWave * sizeof(f32x4_t);
-    hipLaunchKernelGGL((skinny_direct_kernel<MT, WAVES, EPI>), dim3((a.N + 15) / 16), dim3(WAVES * kWave), smem, stream, a);
-    return fllm_check_launch("linear_skinny");
+template <int MT, int EPI>
+int launch_wide(SkinnyArgs a, hipStream_t stream) {
+    constexpr int WAVES = 4;
+    constexpr int NT = EPI == EPI_SWIGLU ? 8 : 16;
+    constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
+    const int n_out = EPI == EPI_SWIGLU ? a.N / 2 : a.N;
+    const int ntiles = (n_out + NT - 1) / NT;
+    const int ngroups = (ntiles + WAVES - 1) / WAVES;
+    const int slots = 2 * device_cus();        // two workgroups of four waves a compute unit
+    void *base = nullptr;
+    size_t bytes = 0;
+    const bool have_ws = fllm_device_workspace(&base, &bytes);
+    // K slices: as many as fill the chip with the row groups there are, each at least two chunks long
+    int S = 1;
+    const int forced = fllm_option_linear_slices();
+    while (S < 8 && ngroups * S * 2 <= slots && (a.K + 2 * S - 1) / (2 * S) >= 512) S *= 2;
+    if (forced > 0) S = forced;
+    while (S > 1) {
+        const size_t need = kWorkspaceCounterBytes + (size_t)ntiles * S * MT * RT * kWave * 4 * sizeof(float);
+        if (have_ws && need <= bytes && (size_t)ntiles * sizeof(int) <= kWorkspaceCounterBytes && (a.K + S - 1) / S >= 256) break;
+        S /= 2;
+    }
+    a.S = S;
+    a.slice = ((a.K + S - 1) / S + 255) / 256 * 256;
+    if ((S - 1) * a.slice >= a.K && S > 1) a.S = S = (a.K + a.slice - 1) / a.slice;   // no empty slice
+    if (S > 1) {
+        a.counters = (int *)base;
+        a.ws = (float *)((unsigned char *)base + kWorkspaceCounterBytes);
+    }
+    int per_slice = slots / S;
+    if (per_slice < 1) per_slice = 1;
+    if (per_slice > ngroups) per_slice = ngroups;
+    hipLaunchKernelGGL((skinny_wide_kernel<MT, EPI>), dim3(per_slice * S), dim3(WAVES * kWave), 0, stream, a);
+    return fllm_check_launch("linear_wide");
+}
+
+template <int EPI>
+int dispatch_wide(const SkinnyArgs &a, hipStream_t stream) {
+    const int mt = (a.M + 15) / 16;
+    if (mt == 2) return launch_wide<2, EPI>(a, stream);
+    if (mt == 3) return launch_wide<3, EPI>(a, stream);
+    return launch_wide<4, EPI>(a, stream);
 }
 
 template <int PRO, int EPI>
 int dispatch(const SkinnyArgs &a, hipStream_t stream) {
     const int mt = (a.M + 15) / 16;
     if (mt == 1) return launch_resident<PRO, EPI>(a, stream);
-    if constexpr (PRO == PRO_BF16 && (EPI == EPI_STORE || EPI == EPI_STORE_F32 || EPI == EPI_ADD)) {
-        const bool wide = (a.N + 15) / 16 < 1024;   // few row tiles: more waves per tile keep enough loads in flight
-#define FLLM_GO(MT) return wide ? launch_direct<MT, 16, EPI>(a, stream) : launch_direct<MT, 8, EPI>(a, stream)
-        if (mt == 2) { FLLM_GO(2); }
-        if (mt == 3) { FLLM_GO(3); }
-        FLLM_GO(4);
-#undef FLLM_GO
+    if constexpr (PRO == PRO_BF16 && (EPI == EPI_STORE || EPI == EPI_STORE_F32 || EPI == EPI_ADD || EPI == EPI_SWIGLU)) {
+        return dispatch_wide<EPI>(a, stream);
     }
-    return 1;   // the fused forms are for up to 16 rows
+    return 1;   // the forms with a norm prologue are for up to 16 rows
 }
 
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
@@ -718,6 +873,26 @@ extern "C" int fllm_norm_gate_up_swiglu(const float *x, const float *norm_w, flo
     a.K = K;
     const int rc = dispatch<PRO_NORM_F32, EPI_SWIGLU>(a, stream);
     FLLM_REQUIRE(rc != 1, "norm_gate_up_swiglu: shape M=%d K=%d does not fit the staging area", M, K);
+    return rc;
+}
+
+extern "C" int fllm_gate_up_swiglu(const void *x, int ldx, const void *w_gate_up, const float *bias, void *out, int M,
+                                   int inter, int K, hipStream_t stream) {
+    FLLM_REQUIRE(M >= 1 && M <= 64 && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && inter > 0,
+                 "gate_up_swiglu: takes 1..64 rows and K, ldx in steps of 8 (M=%d K=%d ldx=%d)", M, K, ldx);
+    FLLM_REQUIRE(aligned16(x) && aligned16(w_gate_up), "gate_up_swiglu: operands must be 16-byte aligned");
+    SkinnyArgs a = {};
+    a.x = x;
+    a.ldx = ldx;
+    a.w = (const bf16_t *)w_gate_up;
+    a.bias = bias;
+    a.out = out;
+    a.ldo = inter;
+    a.M = M;
+    a.N = 2 * inter;
+    a.K = K;
+    const int rc = dispatch<PRO_BF16, EPI_SWIGLU>(a, stream);
+    FLLM_REQUIRE(rc != 1, "gate_up_swiglu: shape M=%d K=%d does not fit", M, K);
     return rc;
 }
 

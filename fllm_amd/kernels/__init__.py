@@ -66,6 +66,7 @@ def load_library(build_if_missing: bool = True):
         "fllm_norm_qkv_rope_store": [c_void, c_void, c_float, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void,
                                      c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_argmax": [c_void, c_void, c_int, c_int, c_void],
+        "fllm_gate_up_swiglu": [c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_carry_ids": [c_void, c_void, c_void, c_int, c_int, c_void],
         "fllm_sample": [c_void, c_void, c_void, c_void, c_int, c_int, c_void],
     }
@@ -254,6 +255,23 @@ class Ops:
         _dense(out, "out", torch.bfloat16, (M, two_i // 2))
         self._check(self.lib.fllm_norm_gate_up_swiglu(_ptr(x), _ptr(norm_weight), float(eps), _ptr(w_gate_up), _ptr(bias),
                                                       _ptr(out), M, two_i // 2, K, self._stream()))
+        return out
+
+    GATE_UP_SWIGLU_ROWS = 64
+
+    def gate_up_swiglu(self, x, w_gate_up, out, bias=None):
+        """out = silu(x @ gate.T) * (x @ up.T) for up to 64 bfloat16 rows; w_gate_up = [gate; up], out bfloat16 [M, I]."""
+        M, K = x.shape
+        two_i = w_gate_up.shape[0]
+        _need(two_i % 2 == 0, "w_gate_up needs an even number of rows")
+        _need(x.dtype == torch.bfloat16 and x.is_cuda and x.stride(1) == 1, "x must be bfloat16 rows on the GPU")
+        _dense(w_gate_up, "w_gate_up", torch.bfloat16, (two_i, K))
+        if bias is not None:
+            _dense(bias, "bias", torch.float32, (two_i,))
+        _dense(out, "out", torch.bfloat16, (M, two_i // 2))
+        _need(1 <= M <= self.GATE_UP_SWIGLU_ROWS and K % 8 == 0, f"gate_up_swiglu takes 1..64 rows and widths in steps of 8, not {M} x {K}")
+        self._check(self.lib.fllm_gate_up_swiglu(_ptr(x), x.stride(0) if M > 1 else K, _ptr(w_gate_up), _ptr(bias), _ptr(out), M,
+                                                 two_i // 2, K, self._stream()))
         return out
 
     def norm_qkv_rope_store(self, x, norm_weight, eps, w_qkv, q_out, row_pos, row_seg, tables, cos, sin, k_pages, v_pages,

@@ -49,6 +49,15 @@ class ReferenceOps:
         out.copy_((y if bias is None else y + bias.double()).to(out.dtype))
         return out
 
+    def gate_up_swiglu(self, x, w_gate_up, out, bias=None):
+        y = x.double() @ w_gate_up.double().T
+        if bias is not None:
+            y = y + bias.double()
+        inter = y.shape[1] // 2
+        g, u = y[:, :inter], y[:, inter:]
+        out.copy_((g / (1.0 + torch.exp(-g)) * u).to(out.dtype))
+        return out
+
     def norm_gate_up_swiglu(self, x, norm_weight, eps, w_gate_up, out, bias=None):
         y = self._normed(x, norm_weight, eps) @ w_gate_up.double().T
         if bias is not None:

@@ -24,7 +24,7 @@ def ops():
 @pytest.fixture(scope="module")
 def library_ops():
     from fllm_amd.kernels import Ops
-    return Ops()                            # large bfloat16 products through the GEMM library
+    return Ops(library_gemm_from=17)        # bfloat16 products of 17 rows and more through the GEMM library
 
 
 @pytest.fixture(scope="module")
@@ -148,6 +148,8 @@ SKINNY = [(1, 16, 64), (1, 4096, 4096), (2, 100, 136), (5, 6144, 4096), (8, 4096
           (17, 128, 128), (33, 1000, 4096), (64, 4096, 4096), (48, 30, 72),
           # 8-row weight tiles with two K halves (up to 8 rows, 4,100 to 16,000 outputs), ragged in N and K
           (3, 5001, 64), (7, 6148, 200), (8, 4104, 1096), (1, 9000, 520),
+          # 17 to 64 rows: four waves a workgroup, activations through LDS in chunks, K slices over workgroups
+          (20, 4096, 14336), (64, 6144, 4096), (40, 100, 264), (33, 5001, 72), (64, 48, 8192), (18, 28672, 512),
           # K in slices over workgroups (the rows of all of K do not fit into LDS), 8 and 16 waves
           (16, 136, 14336), (5, 1000, 30008), (12, 72, 65536)]
 TILED = [(65, 128, 64), (128, 200, 200), (200, 6144, 4096), (300, 130, 136), (2048, 512, 4096), (129, 4096, 14336)]
@@ -180,7 +182,7 @@ def test_add_residual(ops, dtype, rows, width):
     (8, 6144, 4096, "linear.dual_k", (0, 1)), (3, 5001, 200, "linear.dual_k", (0, 1)),
     (8, 4096, 14336, "linear.x_direct", (0, 1)), (16, 1000, 520, "linear.x_direct", (0, 1)), (3, 5001, 200, "linear.x_direct", (0, 1)),
     (8, 4096, 14336, "linear.slices", (0, 2, 4, 8)), (2, 1000, 4096, "linear.slices", (0, 2, 4)),
-    (16, 264, 8192, "linear.slices", (0, 4))])
+    (16, 264, 8192, "linear.slices", (0, 4)), (64, 4096, 14336, "linear.slices", (0, 1, 2, 4, 8)), (40, 1000, 4096, "linear.slices", (0, 1, 2))])
 def test_linear_bf16_variants_agree(ops, ref, M, N, K, option, values):
     """The ways of cutting a decode-shaped product (tile shape, K slices) give the same sums up to the order
     of float32 additions, each of them the same bits on every call."""
@@ -268,6 +270,20 @@ def test_norm_gate_up_swiglu(ops, ref, M, inter, K):
     got = ops.norm_gate_up_swiglu(x.to(DEV), nw.to(DEV), 1e-6, w.to(DEV), torch.empty(M, inter, dtype=torch.bfloat16, device=DEV),
                                   bias=b.to(DEV))
     close(got, want, 2 * BF16_EPS, 4e-2, f"norm_gate_up_swiglu M{M} I{inter} K{K}")
+
+
+@pytest.mark.parametrize("M,inter,K", [(17, 14336, 4096), (64, 176, 64), (40, 432, 160), (33, 1000, 4096), (24, 200, 96), (64, 36, 8192),
+                                       (8, 432, 160), (1, 176, 64)])
+def test_gate_up_swiglu(ops, ref, M, inter, K):
+    g = gen(46)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(2 * inter, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    b = torch.randn(2 * inter, generator=g) * 0.1
+    want = ref.gate_up_swiglu(x, w, torch.empty(M, inter, dtype=torch.float64), bias=b)
+    outs = [ops.gate_up_swiglu(x.to(DEV), w.to(DEV), torch.empty(M, inter, dtype=torch.bfloat16, device=DEV), bias=b.to(DEV))
+            for _ in range(3)]
+    close(outs[0], want, 2 * BF16_EPS, 2e-2, f"gate_up_swiglu M{M} I{inter} K{K}")
+    assert torch.equal(outs[1], outs[0]) and torch.equal(outs[2], outs[0])
 
 
 @pytest.mark.parametrize("heads,kv_heads,head_dim,rope_dims,page_size,K", [(4, 2, 16, 16, 16, 64), (5, 1, 32, 32, 8, 160),
