@@ -521,6 +521,15 @@ def test_attention_decode_split_contexts(ops, ref, fused_merge, heads, kv_heads,
         ops.set_option("attention.fused_merge", 1)
 
 
+@pytest.mark.parametrize("segs,bound,window", [([(20000, 1), (70, 1)], 32768, None), ([(40000, 1)], 65536, None),
+                                                ([(16380, 6)], None, None), ([(30000, 3)], None, 4096)])
+def test_attention_long_contexts(ops, ref, segs, bound, window):
+    """Tens of thousands of keys: many splits of a decode row, many tiles of a prompt portion, page tables of
+    thousands of entries; one far key stands out, so a lost split or a wrong page changes the output."""
+    attention_case(ops, ref, torch.bfloat16, 32, 8, 128, 16, segs, window, 18, spike=True, bound=bound)
+    attention_case(ops, ref, torch.bfloat16, 8, 2, 64, 16, segs, window, 19, spike=True, bound=bound)
+
+
 def test_attention_row_is_the_same_alone_and_in_a_batch(ops, ref):
     """float32: the bits of a row do not depend on the batch around it."""
     a = attention_case(ops, ref, torch.float32, 8, 2, 64, 16, [(100, 17), (37, 1), (0, 33)], None, 15)
