@@ -8,7 +8,7 @@ knows which model it is in.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional, Tuple
+from typing import Any, Dict, Optional, Tuple
 
 
 class ConfigError(ValueError):

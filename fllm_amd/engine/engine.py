@@ -7,7 +7,7 @@ rust/engine/examples/perf_decode.rs:24-46).
 from __future__ import annotations
 
 import time
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence as Seq, Union
 
 import torch
@@ -18,7 +18,7 @@ from ..sampling import SampleRequest, Sampler, SamplingParams
 from ..weights.loader import load_checkpoint
 from ..weights.random_init import random_tensors
 from .runner import ModelRunner, StepEntry
-from .scheduler import ScheduledStep, Scheduler, SchedulerConfig, Sequence
+from .scheduler import Scheduler, SchedulerConfig, Sequence
 
 
 @dataclass

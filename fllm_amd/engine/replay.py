@@ -14,8 +14,6 @@ import os
 import sys
 from typing import IO
 
-import numpy as np
-
 from .runner import ModelRunner, StepEntry
 
 

@@ -9,7 +9,6 @@ a batch: rust/engine/src/runtime.rs:2380-2442).
 """
 from __future__ import annotations
 
-import os
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Union
 

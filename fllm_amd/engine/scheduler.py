@@ -22,7 +22,7 @@ from collections import deque
 from dataclasses import dataclass, field
 from typing import Deque, Dict, List, Optional, Tuple
 
-from ..cache import CacheManager, OutOfPages
+from ..cache import CacheManager
 from ..sampling.params import SamplingParams
 
 

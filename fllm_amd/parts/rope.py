@@ -8,7 +8,7 @@ phase = position * inv[l] in float32; cos and sin are evaluated in float64 and s
 from __future__ import annotations
 
 import math
-from typing import Optional, Tuple
+from typing import Tuple
 
 import torch
 

@@ -2,7 +2,7 @@
 from __future__ import annotations
 
 import weakref
-from typing import Any, Dict, Tuple
+from typing import Any, Dict
 
 import torch
 

@@ -6,7 +6,7 @@ is imported (tests register toy parts the same way).
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, List, Optional, Sequence
+from typing import Any, Callable, Dict, List, Sequence
 
 from .config.spec import ConfigError, ModelSpec
 

@@ -2,7 +2,6 @@
 otherwise (temperature, top-k, top-p, Gumbel-max draw keyed by seed and draw number)."""
 from __future__ import annotations
 
-import ctypes
 from dataclasses import dataclass
 from typing import List, Sequence
 
