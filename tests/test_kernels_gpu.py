@@ -363,10 +363,22 @@ def scattered_tables(g, segments, pages_each, num_pages):
                          [(4, 2, 16, 16, 0, 16), (5, 1, 32, 32, 0, 8), (6, 3, 48, 24, 0, 16), (8, 2, 64, 64, 1, 16),
                           (32, 8, 128, 128, 0, 16), (2, 2, 16, 0, 0, 4)])
 def test_rope_kv_store(ops, ref, dtype, heads, kv_heads, head_dim, rope_dims, pairing, page_size):
+    _rope_case(ops, ref, dtype, heads, kv_heads, head_dim, rope_dims, pairing, page_size,
+               [(0, 5), (37, 1), (page_size - 1, 3), (100, 17)], 128)
+
+
+@pytest.mark.parametrize("heads,kv_heads,head_dim,rope_dims,page_size", [(8, 2, 64, 64, 16), (32, 8, 128, 128, 16), (4, 2, 16, 8, 8),
+                                                                         (6, 3, 48, 24, 32)])
+def test_rope_kv_store_prompt_portions(ops, ref, heads, kv_heads, head_dim, rope_dims, page_size):
+    """Hundreds of rows: runs of 8 tokens that start at a multiple of 8 store their values 16 bytes at a time; runs
+    that start elsewhere, single rows and the ends of portions take the other way."""
+    _rope_case(ops, ref, torch.bfloat16, heads, kv_heads, head_dim, rope_dims, 1, page_size,
+               [(0, 300), (37, 1), (13, 40), (8, 64), (509, 3)], 512)
+
+
+def _rope_case(ops, ref, dtype, heads, kv_heads, head_dim, rope_dims, pairing, page_size, segs, positions):
     g = gen(8)
-    segs = [(0, 5), (37, 1), (page_size - 1, 3), (100, 17)]     # (first position, rows)
-    rows = sum(n for _, n in segs)
-    positions = 128
+    rows = sum(n for _, n in segs)             # segs: (first position, rows)
     pages_each = positions // page_size
     num_pages = len(segs) * pages_each + 3
     tables = scattered_tables(g, len(segs), pages_each, num_pages)
