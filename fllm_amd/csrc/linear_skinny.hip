@@ -21,6 +21,10 @@
 
 namespace {
 
+// 16 bytes of zeros in device memory: what a lane loads when it has nothing of its own to load, so that every lane
+// issues every load and no load sits behind a branch.
+__device__ uint4 kZeros = {0u, 0u, 0u, 0u};     // not const: in the same address space as the tensors it stands in for
+
 enum { PRO_BF16 = 0, PRO_NORM_F32 = 1 };
 enum { EPI_STORE = 0, EPI_STORE_F32 = 1, EPI_ADD = 2, EPI_QKV = 3, EPI_SWIGLU = 4 };
 
@@ -481,17 +485,21 @@ skinny_wide_kernel(SkinnyArgs a) {
 
     // weights: cursor (item, chunk) of the next chunk to ask for
     int w_item = 0, w_chunk = 0;
+    // Every lane issues every load: where it has nothing of its own to load (columns behind the slice, rows behind
+    // the last one, items behind the last item) it reads 16 bytes of zeros, or weights that meet zeros on the
+    // activation side.  No load sits behind a branch, so a chunk waits for its own loads only and the loads of the
+    // chunks behind it stay in flight.
+    const bf16_t *zeros = (const bf16_t *)&kZeros;
     auto issue_w = [&](bf16x8_t (&buf)[KS]) {
-        if (w_item < my_items) {
-            const int tile = (rg0 + w_item * rstride) * WAVES + wave;
-            int row = tile * NT + (EPI == EPI_SWIGLU ? (r & 7) : r);
-            if (row >= n_out) row = n_out - 1;    // past the end: computed from a valid row, never stored
-            if (EPI == EPI_SWIGLU) row += (r >> 3) * n_out;
-            const int kb = w_chunk * KC + g * 8;
-            const bf16_t *wp = a.w + (size_t)row * K + ks0 + kb;
+        const bool live = w_item < my_items;
+        const int tile = (rg0 + (live ? w_item : 0) * rstride) * WAVES + wave;
+        int row = tile * NT + (EPI == EPI_SWIGLU ? (r & 7) : r);
+        if (row >= n_out) row = n_out - 1;    // past the end: computed from a valid row, never stored
+        if (EPI == EPI_SWIGLU) row += (r >> 3) * n_out;
+        const int kb = w_chunk * KC + g * 8;
+        const bf16_t *wp = a.w + (size_t)row * K + ks0;
 #pragma unroll
-            for (int u = 0; u < KS; u++) buf[u] = kb + u * 32 < kcn ? *(const bf16x8_t *)(wp + u * 32) : zero8();
-        }
+        for (int u = 0; u < KS; u++) buf[u] = *(const bf16x8_t *)(live ? wp + min(kb + u * 32, kcn - 8) : zeros);
         if (++w_chunk == nchunks) w_chunk = 0, w_item++;
     };
     // activations: the chunk index within the slice is all that matters (every item walks the same slice)
@@ -501,7 +509,7 @@ skinny_wide_kernel(SkinnyArgs a) {
         for (int i = 0; i < XL; i++) {
             const int idx = threadIdx.x + i * THREADS;
             const int m = idx / (KC / 8), c = (idx - m * (KC / 8)) * 8 + chunk * KC;
-            xr[i] = (m < M && c < kcn) ? *(const bf16x8_t *)(x + (size_t)m * a.ldx + ks0 + c) : zero8();
+            xr[i] = *(const bf16x8_t *)((m < M && c < kcn) ? x + (size_t)m * a.ldx + ks0 + c : zeros);
         }
     };
     auto store_x = [&](int buffer) {
@@ -529,7 +537,7 @@ skinny_wide_kernel(SkinnyArgs a) {
 
     auto step = [&](bf16x8_t (&buf)[KS], int q) {
         const int next_chunk = chunk + 1 == nchunks ? 0 : chunk + 1;
-        if (q + 1 < total) load_x(next_chunk);      // on its way while this chunk is multiplied
+        load_x(next_chunk);      // on its way while this chunk is multiplied (once more than needed at the very end)
         const bf16_t *xb = &xs[q & 1][r * XP + g * 8];
 #pragma unroll
         for (int u = 0; u < KS; u++) {
@@ -540,10 +548,10 @@ skinny_wide_kernel(SkinnyArgs a) {
             for (int mt = 0; mt < MT; mt++) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(buf[u], xf[mt], acc[mt], 0, 0, 0);
         }
         issue_w(buf);      // the chunk two ahead takes this one's registers
-        if (q + 1 < total) store_x((q + 1) & 1);
+        store_x((q + 1) & 1);
         __syncthreads();   // the next chunk is in LDS; everybody has read the one before it
         chunk = next_chunk;
-        if (chunk != 0) return;
+        if (chunk != 0 || item >= my_items) return;      // (a step behind the last item multiplies zeros and ends nothing)
         // the item is complete: this wave's tile has its sums over the slice
         const int tile = (rg0 + item * rstride) * WAVES + wave;
         item++;
@@ -609,9 +617,12 @@ skinny_wide_kernel(SkinnyArgs a) {
         }
     };
 
+    // The two buffers take turns without a condition between them (an odd number of steps gets one more, which
+    // multiplies zeros): only then does the compiler see that the loads of one buffer always lie behind those of
+    // the other, and lets them stay in flight.
     for (int q = 0; q < total; q += 2) {
         step(wa, q);
-        if (q + 1 < total) step(wb, q + 1);
+        step(wb, q + 1);
     }
 }
 
