@@ -15,7 +15,8 @@ int fllm_abi_version(void);
 // 0: bfloat16 calls use the plain kernels only (for comparing them with the MFMA kernels); default 1
 void fllm_set_fast_kernels(int on);
 // Switches a kernel variant (for measurements and tests): "attention.tile32" 0/1; "linear.slices" n
-// (0: chosen by shape); "linear.dual_k" 0/1; "linear.x_direct" 0/1; "attention.fused_merge" 0/1.  0 on success.
+// (0: chosen by shape); "linear.dual_k" 0/1; "linear.x_direct" 0/1; "attention.fused_merge" 0/1;
+// "attention.prefill_parts" 0/1.  0 on success.
 int fllm_set_option(const char *name, int value);
 
 // out[r, :] = scale * table[ids[r], :]            out: float32 [rows, width]
@@ -37,7 +38,8 @@ int fllm_linear(const void *x, int ldx, const void *w, const float *bias, void *
 
 // Device memory for kernels that meet across workgroups: the decode-shaped products (1..16 rows), whose K
 // dimension is cut into slices over workgroups when the activations of all of K do not fit into LDS, and
-// decode attention over split contexts.  Its first 64 KiB are counters, which must be zero when it is handed
+// decode attention over split contexts, and prompt attention of few rows over long contexts (the keys of a row
+// tile go to several workgroups: 66 KiB a part for heads of 128).  Its first 64 KiB are counters, which must be zero when it is handed
 // over and are zero again after every launch; partial sums follow.  One per device (the current one);
 // work that would need more than it holds runs another way.  Launches on different streams of one device
 // must not overlap while it is set.  nullptr takes it away.

@@ -16,7 +16,8 @@
 //                  one segment and one key/value head; keys and values go through LDS in tiles of 64.
 //   tile32 kernel  head sizes 64 and 128: 128 rows per workgroup on 32x32x16 products, the next tile on its way
 //                  while the current one is multiplied (described at the kernel); faster than the tile kernel
-//                  for portions of any length.
+//                  for portions of any length.  Few rows over long contexts: several workgroups share a row
+//                  tile's keys and the one that arrives last adds their parts up.
 //   decode kernel  one row per segment: a workgroup takes (row, key/value head, context split), its
 //                  sixteen waves stride over 32-key blocks loading K and V^T straight into MFMA
 //                  operands; long contexts of small batches are split and merged by a second kernel.
@@ -50,6 +51,11 @@ struct AttnArgs {
     float *ws_o;    // [rows, heads, splits, D]
     int splits, keys_per_split;
     int *counters;  // one per (row, key/value head, query tile), zero between launches: the last split to arrive merges; null: a merge kernel does
+    // Prompt portions (tile32 kernel): a row tile with more than part_tiles key tiles is shared by several workgroups
+    // (blockIdx.y), each with a stretch of its key tiles; 0: never.  Their partial results meet in `parts_ws`
+    // ([row tile][key/value head][part][kPartFloats]) and are counted in `counters` ([row tile][key/value head]).
+    int part_tiles;
+    float *parts_ws;
 };
 
 __device__ __forceinline__ bf16x8_t zero8() {
@@ -60,6 +66,10 @@ __device__ __forceinline__ bf16x8_t zero8() {
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// floats that one part of a shared row tile leaves for the merge (tile32 kernel): head_dim / 2 outputs, a maximum
+// and a sum for each of its 256 lanes
+__host__ __device__ constexpr size_t kPartFloats(int head_dim) { return (size_t)kThreads * (head_dim / 2 + 2); }
 
 // Online-softmax update of one query row held across the four lane groups of a wave.
 // s: NS score tiles (already scaled and masked with -inf); returns the P^T operands.
@@ -272,8 +282,11 @@ attn_tile32_kernel(AttnArgs p) {
     __shared__ int s_tile[2];
     const int G = p.heads / p.kv_heads;
     const int TQ = 128 / G;         // tokens per tile
+    // blockIdx.x = (row tile, key/value head), the head fastest: workgroups start in the order of their row tiles,
+    // longest contexts first, whatever their head, and with 8 heads each of the 8 dies sees the keys of one head only
+    const int group = blockIdx.x;
     if (threadIdx.x == 0) {
-        int b = blockIdx.x, seg = -1, t0 = 0;
+        int b = group / p.kv_heads, seg = -1, t0 = 0;
         for (int s = 0; s < p.num_segs; s++) {
             const int n = p.seg_start[s + 1] - p.seg_start[s];
             const int nt = (n + TQ - 1) / TQ;
@@ -293,7 +306,7 @@ attn_tile32_kernel(AttnArgs p) {
     const int row0 = p.seg_start[seg] + s_tile[1] * TQ;
     const int ntok = min(TQ, p.seg_start[seg + 1] - row0);
     const int pos0 = p.row_pos[row0];
-    const int kvh = blockIdx.y;
+    const int kvh = group % p.kv_heads;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int q = lane & 31, h = lane >> 5;
     const int rr = wave * 32 + q;
@@ -315,7 +328,20 @@ attn_tile32_kernel(AttnArgs p) {
     const int lo_tile = (p.window > 0 && pos0 - p.window + 1 > 0) ? pos0 - p.window + 1 : 0;
     // from this key on every row of the workgroup sees every key up to pos0 (no window edge inside)
     const int lo_all = (p.window > 0 && p_last - p.window + 1 > 0) ? p_last - p.window + 1 : 0;
-    const int kbegin = (lo_tile / KT) * KT;
+    int kbegin = (lo_tile / KT) * KT;
+    // Long contexts of few rows: the key tiles of this row tile are dealt out to `parts` workgroups in equal
+    // stretches; a workgroup beyond that number has nothing to do.
+    int parts = 1, k_stop = p_last;    // k_stop: the last key of this workgroup's stretch
+    if (p.part_tiles > 0) {
+        const int nkt = (p_last - kbegin) / KT + 1;
+        parts = min((nkt + p.part_tiles - 1) / p.part_tiles, (int)gridDim.y);
+        const int part = blockIdx.y;
+        if (part >= parts) return;
+        const int base = nkt / parts, rem = nkt - base * parts;
+        const int first_tile = part * base + min(part, rem), count = base + (part < rem ? 1 : 0);
+        kbegin += first_tile * KT;
+        k_stop = min(p_last, kbegin + count * KT - 1);
+    }
     const int32_t *tbl = p.tables + (size_t)seg * p.table_stride;
 
     // What of a chunk's address does not change from tile to tile (tiles start at multiples of 64 >= page size)
@@ -341,7 +367,7 @@ attn_tile32_kernel(AttnArgs p) {
     // values, which are asked for one tile before they are multiplied, so neither wait lies on the path.
     int pgk[CH], pgv[CH];
     auto pages = [&](int k0) {   // page numbers of tile k0 .. k0 + 63 (0 where the tile has no token)
-        if (k0 > p_last) return;
+        if (k0 > k_stop) return;
         const bool inside = k0 >= lo_tile && k0 + KT - 1 <= p_last;
 #pragma unroll
         for (int c = 0; c < CH; c++) {
@@ -386,7 +412,7 @@ attn_tile32_kernel(AttnArgs p) {
     pages(kbegin);
     fetch(kbegin);
     pages(kbegin + KT);
-    for (int k0 = kbegin; k0 <= p_last; k0 += KT) {
+    for (int k0 = kbegin; k0 <= k_stop; k0 += KT) {
         __syncthreads();   // the previous tile has been read
 #pragma unroll
         for (int c = 0; c < CH; c++) {
@@ -394,7 +420,7 @@ attn_tile32_kernel(AttnArgs p) {
             *(bf16x8_t *)(Vs + v_lds[c]) = vreg[c];
         }
         __syncthreads();
-        if (k0 + KT <= p_last) {   // in flight while this tile is multiplied
+        if (k0 + KT <= k_stop) {   // in flight while this tile is multiplied
             fetch(k0 + KT);
             pages(k0 + 2 * KT);
         }
@@ -459,6 +485,52 @@ attn_tile32_kernel(AttnArgs p) {
                     o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf, o[db], 0, 0, 0);
                 }
             }
+    }
+    if (parts > 1) {
+        // Every part leaves its maximum, sum and unnormalized outputs at the device's point of coherence, each lane
+        // its own values (the parts share the assignment of rows to lanes); the part that arrives last adds them up
+        // in the order of the parts, so the result does not depend on which one that is.
+        __shared__ int s_seen;
+        float *slot = p.parts_ws + (size_t)group * gridDim.y * kPartFloats(D);
+        float *mine = slot + (size_t)blockIdx.y * kPartFloats(D);
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+                __hip_atomic_store(mine + (db * 16 + i) * kThreads + threadIdx.x, o[db][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(mine + DB * 16 * kThreads + threadIdx.x, m_run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(mine + (DB * 16 + 1) * kThreads + threadIdx.x, l_run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);      // the part has arrived before it is counted
+        __syncthreads();
+        int *counter = p.counters + group;
+        if (threadIdx.x == 0) s_seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (s_seen != parts - 1) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+        float m_all = -INFINITY;
+        for (int i = 0; i < parts; i++)
+            m_all = fmaxf(m_all, __hip_atomic_load(slot + (size_t)i * kPartFloats(D) + DB * 16 * kThreads + threadIdx.x,
+                                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) o[db][i] = 0.f;
+        l_run = 0.f;
+        for (int i = 0; i < parts; i++) {
+            const float *from = slot + (size_t)i * kPartFloats(D);
+            const float mi = __hip_atomic_load(from + DB * 16 * kThreads + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float f = mi == -INFINITY ? 0.f : fast_exp2((mi - m_all) * sc);
+            l_run = fmaf(__hip_atomic_load(from + (DB * 16 + 1) * kThreads + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT),
+                         f, l_run);
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int j = 0; j < 16; j++)
+                    o[db][j] = fmaf(__hip_atomic_load(from + (db * 16 + j) * kThreads + threadIdx.x, __ATOMIC_RELAXED,
+                                                      __HIP_MEMORY_SCOPE_AGENT), f, o[db][j]);
+        }
     }
     if (rvalid) {
         const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
@@ -707,6 +779,41 @@ bool fast_shape(int heads, int kv_heads, int head_dim, int page_size) {
     return true;
 }
 
+int device_slots() {   // workgroups of the tile32 kernel that the device holds at a time: two a compute unit
+    static int slots = 0;
+    if (slots == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        int cus = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
+        slots = 2 * (cus > 0 ? cus : 256);
+    }
+    return slots;
+}
+
+// How the tile32 kernel shares the key tiles of a row tile among workgroups: the most key tiles one workgroup
+// takes (0: row tiles are not shared) and the most parts a row tile can have.  Row tiles are shared when, one
+// workgroup each, they would leave workgroup slots of the device empty: a part then has about the key tiles that a
+// slot sees in all when every slot is taken, and at least 8, since every part pays for leaving its results and the
+// last one for adding them up (measured: smaller parts lose more to that than they gain).  `room` is the number of
+// parts that the workspace holds.
+int prefill_part_plan(int tiles, int kv_heads, int max_context, int window, size_t room, int *max_parts) {
+    *max_parts = 1;
+    if (window > 0) return 0;     // a window keeps every context short
+    const long groups = (long)tiles * kv_heads;
+    if (groups * (long)sizeof(int) > (long)kWorkspaceCounterBytes) return 0;
+    const long most_tiles = ((long)max_context + 63) / 64;        // key tiles of the longest context
+    const long per_slot = (groups * most_tiles + device_slots() - 1) / device_slots();
+    long per_part = std::max(8L, per_slot);
+    if (fllm_option_prefill_parts() > 1) per_part = fllm_option_prefill_parts();   // set by hand, for measurements
+    const long cap = std::min(16L, (long)(room / (size_t)groups));   // parts a row tile may have
+    if (cap < 2) return 0;
+    per_part = std::max(per_part, (most_tiles + cap - 1) / cap);
+    if (per_part >= most_tiles) return 0;
+    *max_parts = (int)((most_tiles + per_part - 1) / per_part);
+    return (int)per_part;
+}
+
 template <int D>
 int launch(const AttnArgs &a, int uniform_rows, int max_context, void *workspace, size_t workspace_bytes,
            hipStream_t stream) {
@@ -748,7 +855,18 @@ int launch(const AttnArgs &a, int uniform_rows, int max_context, void *workspace
     if (D >= 64 && G <= 64 && fllm_option_tile32()) {   // 128 rows per workgroup on 32x32x16 products
         const int TQ = 128 / G;
         const int tiles = (a.rows + TQ - 1) / TQ + a.num_segs;   // upper bound; surplus workgroups leave at once
-        hipLaunchKernelGGL(attn_tile32_kernel<(D >= 64 ? D : 64)>, dim3(tiles, a.kv_heads), dim3(kThreads), 0, stream, a);
+        AttnArgs p = a;
+        int max_parts = 1;
+        void *dev_ws = nullptr;
+        size_t dev_ws_bytes = 0;
+        if (fllm_option_prefill_parts() && fllm_device_workspace(&dev_ws, &dev_ws_bytes) && dev_ws_bytes > kWorkspaceCounterBytes) {
+            p.part_tiles = prefill_part_plan(tiles, a.kv_heads, max_context, a.window,
+                                             (dev_ws_bytes - kWorkspaceCounterBytes) / (kPartFloats(D) * sizeof(float)), &max_parts);
+            p.counters = (int *)dev_ws;
+            p.parts_ws = (float *)((unsigned char *)dev_ws + kWorkspaceCounterBytes);
+        }
+        FLLM_REQUIRE(tiles >= 1 && (long)tiles * a.kv_heads <= 0x7fffffffL && max_parts <= 65535, "attention: grid too large");
+        hipLaunchKernelGGL(attn_tile32_kernel<(D >= 64 ? D : 64)>, dim3(tiles * a.kv_heads, max_parts), dim3(kThreads), 0, stream, p);
         return fllm_check_launch("attention_tile32");
     }
     const int TQ = 64 / G;
@@ -807,6 +925,8 @@ int fllm_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, c
     a.splits = 1;
     a.keys_per_split = 0;
     a.counters = nullptr;
+    a.part_tiles = 0;
+    a.parts_ws = nullptr;
     if (head_dim == 32) return launch<32>(a, uniform_rows, max_context, workspace, workspace_bytes, stream);
     if (head_dim == 64) return launch<64>(a, uniform_rows, max_context, workspace, workspace_bytes, stream);
     return launch<128>(a, uniform_rows, max_context, workspace, workspace_bytes, stream);

@@ -27,6 +27,8 @@ int fllm_option_tile32(void);
 int fllm_option_linear_slices(void);
 // 1: the parts of a split decode context are merged by the split that arrives last (default); 0: by a second kernel
 int fllm_option_fused_merge(void);
+// 1: prompt portions with long contexts and few rows share a row tile's keys among workgroups (default); 0: one workgroup a row tile
+int fllm_option_prefill_parts(void);
 // 1: decode-shaped products read bfloat16 activations straight from global memory (default); 0: they stage them in LDS
 int fllm_option_x_direct(void);
 // 1: decode-shaped products of up to 8 rows use 8-row weight tiles with two K halves a product (default); 0: 16-row tiles

@@ -35,12 +35,18 @@ static int g_x_direct = 1;
 int fllm_option_x_direct(void) { return g_x_direct; }
 static int g_fused_merge = 1;
 int fllm_option_fused_merge(void) { return g_fused_merge; }
+static int g_prefill_parts = 1;
+int fllm_option_prefill_parts(void) { return g_prefill_parts; }
 int fllm_option_dual_k(void) { return g_dual_k; }
 int fllm_option_tile32(void) { return g_tile32; }
 int fllm_option_linear_slices(void) { return g_linear_slices; }
 extern "C" int fllm_set_option(const char *name, int value) {
     if (strcmp(name, "attention.fused_merge") == 0) {
         g_fused_merge = value ? 1 : 0;
+        return 0;
+    }
+    if (strcmp(name, "attention.prefill_parts") == 0) {
+        g_prefill_parts = value > 0 ? value : 0;
         return 0;
     }
     if (strcmp(name, "linear.x_direct") == 0) {

@@ -121,7 +121,7 @@ class Ops:
         self.library_gemm_from = library_gemm_from
         self._device_workspace(torch.cuda.current_device())
 
-    _WORKSPACE_BYTES = 32 << 20
+    _WORKSPACE_BYTES = 192 << 20
     _workspaces = {}         # device index -> tensor; lives as long as the process: the library keeps its address
 
     def _device_workspace(self, device: int) -> None:

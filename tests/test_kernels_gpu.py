@@ -542,6 +542,25 @@ def test_attention_long_contexts(ops, ref, segs, bound, window):
     attention_case(ops, ref, torch.bfloat16, 8, 2, 64, 16, segs, window, 19, spike=True, bound=bound)
 
 
+@pytest.mark.parametrize("prefill_parts", [1, 0])
+@pytest.mark.parametrize("heads,kv_heads,head_dim", [(32, 8, 128), (8, 2, 64), (6, 3, 64), (16, 1, 128)])
+@pytest.mark.parametrize("segs,bound", [([(1500, 40), (0, 700), (5000, 3)], None), ([(0, 1100)], None), ([(600, 70), (0, 2)], 8192),
+                                        ([(513, 31), (1000, 33)], 1100)])
+def test_attention_prompt_portions_share_long_row_tiles(ops, ref, prefill_parts, heads, kv_heads, head_dim, segs, bound):
+    """Few rows over long contexts: the keys of a row tile are dealt out to several workgroups, by the bound of the
+    step (parts without keys leave at once), and the one that arrives last adds the parts up: the same bits in
+    every launch, and the counters they meet at are left at zero."""
+    ops.set_option("attention.prefill_parts", prefill_parts)
+    try:
+        attention_case(ops, ref, torch.bfloat16, heads, kv_heads, head_dim, 16, segs, None, 21, spike=True, bound=bound, calls=3)
+    finally:
+        ops.set_option("attention.prefill_parts", 1)
+    torch.cuda.synchronize()
+    from fllm_amd.kernels import Ops
+    counters = Ops._workspaces[torch.cuda.current_device()][: 64 * 1024]
+    assert int(counters.to(torch.int64).sum()) == 0
+
+
 def test_attention_row_is_the_same_alone_and_in_a_batch(ops, ref):
     """float32: the bits of a row do not depend on the batch around it."""
     a = attention_case(ops, ref, torch.float32, 8, 2, 64, 16, [(100, 17), (37, 1), (0, 33)], None, 15)
