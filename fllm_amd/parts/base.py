@@ -7,7 +7,9 @@ Roles and their interfaces:
 
   norm          forward(ctx, x_f32[R,H], out=None, rows=None) -> normed[R or len(rows), H] in the
                 compute dtype; `rows` (int32 device tensor) selects rows first.
-  position      tables(device) -> whatever the mixer's kernels take (rotary: cos/sin tables).
+  position      what the mixer's kernels take: for the attention mixer float32 device tables `cos` and `sin`
+                [positions, dims/2], `dims` (lanes of a head that are rotated) and `pairing` (0: lanes l and
+                l + dims/2, 1: lanes 2l and 2l + 1).
   mixer         cache_need() / state_need() say what the cache manager must keep for it;
                 forward(ctx, h[R,H], residual_f32[R,H], binding) adds its output to `residual`.
   feed_forward  forward(ctx, h[R,H], residual_f32[R,H]) adds its output to `residual`.

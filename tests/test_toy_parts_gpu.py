@@ -1,7 +1,8 @@
-"""A toy mixer with state of its own, defined here, is registered, built and stepped without a
-change to the framework's files: a new architecture (its config, its spec, its tensors), a mixer
+"""Toy parts, defined here, are registered, built and stepped without a change to the framework's
+files.  First a toy mixer with state of its own: a new architecture (its config, its spec, its tensors), a mixer
 that keeps a fixed-size state per request in the slot the cache manager hands out, a run order
-that names a layer twice and lets an entry read another entry's cache."""
+that names a layer twice and lets an entry read another entry's cache.  Then a feed-forward with
+routing and another position encoding."""
 import numpy as np
 import pytest
 import torch
@@ -10,7 +11,7 @@ import plain_llama as P
 import tiny_configs as tc
 from fllm_amd.config.spec import LayerSpec, ModelSpec, PartSpec, RunEntry
 from fllm_amd.engine import ModelRunner, StepEntry
-from fllm_amd.parts.base import INIT_MATRIX, Mixer, StateNeed
+from fllm_amd.parts.base import INIT_MATRIX, FeedForward, Mixer, Part, StateNeed
 from fllm_amd.registry import Architecture, model_spec_from_config, register_architecture, register_part
 from fllm_amd.weights import random_tensors
 
@@ -138,4 +139,140 @@ def test_toy_architecture_steps_through_the_engine():
     # the slot of a is handed out again: the new request starts from a cleared state
     got = runner.step([StepEntry("c", b, all_of(b))])
     assert np.abs(got.double().cpu().numpy() - want_b).max() <= 3e-5 * np.abs(want_b).max()
+    runner.cache.check_invariants()
+
+
+# ---------------------------------------------------------------------------------------------
+# A feed-forward with routing and another position encoding, again without touching the framework
+# ---------------------------------------------------------------------------------------------
+class TopOneExperts(FeedForward):
+    """Router logits in float32; the expert with the largest logit runs, weighted by its softmax
+    probability: y = p_e * W2_e relu(W1_e x)."""
+
+    @classmethod
+    def tensor_shapes(cls, spec):
+        e, h, m = spec["experts"], spec["hidden_size"], spec["intermediate_size"]
+        return {"router": ((e, h), INIT_MATRIX), "w1": ((e * m, h), INIT_MATRIX), "w2": ((e * h, m), INIT_MATRIX)}
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        self.e, self.h, self.m = spec["experts"], spec["hidden_size"], spec["intermediate_size"]
+        self.router = weights["router"].to(rt.device, torch.float32)
+        self.w1 = weights["w1"].to(rt.device, torch.float32).view(self.e, self.m, self.h)
+        self.w2 = weights["w2"].to(rt.device, torch.float32).view(self.e, self.h, self.m)
+
+    def forward(self, ctx, h, residual):
+        x = h.float()
+        logits = x @ self.router.T * 40.0          # far apart, so that rounding does not change the choice
+        prob, choice = torch.softmax(logits, dim=-1).max(dim=-1)
+        for e in range(self.e):
+            rows = (choice == e).nonzero().flatten()
+            if rows.numel():
+                y = torch.relu(x[rows] @ self.w1[e].T) @ self.w2[e].T
+                residual.index_add_(0, rows, y * prob[rows, None])
+
+
+class SquareRootAngles(Part):
+    """Rotation by angles sqrt(position + 1) * (lane + 1) * step on interleaved lane pairs of the first `dims`
+    values of a head: what a position part owes the attention mixer is cos/sin tables by position, `dims` and
+    `pairing`."""
+    role = "position"
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        self.dims, self.pairing = int(spec["dims"]), 1
+        pos = torch.arange(int(spec["max_position"]), dtype=torch.float64)
+        lanes = torch.arange(self.dims // 2, dtype=torch.float64)
+        phase = torch.sqrt(pos + 1.0)[:, None] * (lanes + 1.0)[None, :] * float(spec["step"])
+        self.cos = torch.cos(phase).float().to(rt.device).contiguous()
+        self.sin = torch.sin(phase).float().to(rt.device).contiguous()
+
+
+register_part("feed_forward", "top_one_experts", TopOneExperts)
+register_part("position", "sqrt_angles", SquareRootAngles)
+
+
+def routed_spec(cfg):
+    hidden = cfg["hidden_size"]
+    norm = lambda name: PartSpec("rms", {"size": hidden, "eps": 1e-6}, {"weight": name})
+    layers = []
+    for i in range(2):
+        position = {"kind": "sqrt_angles", "dims": 8, "step": cfg["step"], "max_position": 128} if i == 0 else None
+        mixer = PartSpec("attention", {"hidden_size": hidden, "num_heads": 3, "num_kv_heads": 1, "head_dim": 16, "scale": 0.3,
+                                       "window": None, "position": position},
+                         {k: f"layers.{i}.attn.{k}" for k in "qkvo"})
+        if i == 0:
+            ffn = PartSpec("top_one_experts", {"hidden_size": hidden, "intermediate_size": 40, "experts": 3},
+                           {k: f"layers.{i}.moe.{k}" for k in ("router", "w1", "w2")})
+        else:
+            ffn = PartSpec("gated_mlp", {"hidden_size": hidden, "intermediate_size": 56, "activation": "silu"},
+                           {k: f"layers.{i}.mlp.{k}" for k in ("gate", "up", "down")})
+        layers.append(LayerSpec(PartSpec("prenorm"), mixer, ffn, {"mixer": norm(f"layers.{i}.n1"), "feed_forward": norm(f"layers.{i}.n2")}))
+    return ModelSpec("toy-routed", hidden, cfg["vocab_size"], 128,
+                     PartSpec("table", {"vocab_size": cfg["vocab_size"], "hidden_size": hidden}, {"weight": "embed"}),
+                     tuple(layers), (RunEntry(0), RunEntry(1)), norm("final_norm"),
+                     PartSpec("linear", {"vocab_size": cfg["vocab_size"], "hidden_size": hidden}, {"weight": "head"}))
+
+
+register_architecture(Architecture("toy-routed", ("ToyRoutedModel",), lambda c: c, routed_spec))
+ROUTED = {"model_type": "toy-routed", "hidden_size": 48, "vocab_size": 130, "step": 0.37}
+
+
+def plain_routed(w, ids):
+    """The same model, whole sequence, float64; returns the logits, the experts chosen and the smallest gap between
+    the two largest router logits of a token, relative to their size."""
+    x = w["embed"][np.asarray(ids)]
+    T = len(ids)
+    chosen = None
+    for i in range(2):
+        h = P.rms_norm(x, w[f"layers.{i}.n1"], 1e-6)
+        q = (h @ w[f"layers.{i}.attn.q"].T).reshape(T, 3, 16)
+        k = (h @ w[f"layers.{i}.attn.k"].T).reshape(T, 1, 16)
+        v = (h @ w[f"layers.{i}.attn.v"].T).reshape(T, 1, 16)
+        if i == 0:
+            phase = np.sqrt(np.arange(T) + 1.0)[:, None] * (np.arange(4) + 1.0)[None, :] * 0.37
+            q = P.apply_rope(q, np.cos(phase), np.sin(phase), 8, interleaved=True)
+            k = P.apply_rope(k, np.cos(phase), np.sin(phase), 8, interleaved=True)
+        x = x + P.attention(q, k, v, 0.3).reshape(T, 48) @ w[f"layers.{i}.attn.o"].T
+        h = P.rms_norm(x, w[f"layers.{i}.n2"], 1e-6)
+        if i == 0:
+            logits = h @ w["layers.0.moe.router"].T * 40.0
+            prob = np.exp(logits - logits.max(-1, keepdims=True))
+            prob /= prob.sum(-1, keepdims=True)
+            chosen = logits.argmax(-1)
+            top = np.sort(logits, axis=-1)
+            gap = ((top[:, -1] - top[:, -2]) / np.abs(logits).max()).min()
+            w1, w2 = w["layers.0.moe.w1"].reshape(3, 40, 48), w["layers.0.moe.w2"].reshape(3, 48, 40)
+            y = np.stack([np.maximum(h[t] @ w1[e].T, 0.0) @ w2[e].T * prob[t, e] for t, e in enumerate(chosen)])
+            x = x + y
+        else:
+            x = x + P.gated_mlp(h, w["layers.1.mlp.gate"], w["layers.1.mlp.up"], w["layers.1.mlp.down"])
+    return P.rms_norm(x, w["final_norm"], 1e-6) @ w["head"].T, chosen, gap
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 3e-5), ("bfloat16", 4e-2)])
+def test_toy_routed_feed_forward_and_position_encoding(dtype, tol):
+    """A feed-forward that routes every token to one of three experts and a position encoding with its own angles,
+    interleaved pairs and fewer lanes than the head has, beside a layer of attention without positions and the
+    framework's own feed-forward; portions, single tokens and a second request, against the whole sequence."""
+    typed, spec = model_spec_from_config(ROUTED)
+    tensors = random_tensors(spec, 16, torch.float32 if dtype == "float32" else torch.bfloat16)
+    runner = ModelRunner(spec, tensors, dtype=dtype, page_size=16, max_tokens=192, max_requests=2)
+    w64 = tc.to_float64(tensors)
+    a, b = tc.random_ids(61, 130, 7), tc.random_ids(40, 130, 8)
+    (want_a, chosen_a, gap_a), (want_b, chosen_b, gap_b) = plain_routed(w64, a), plain_routed(w64, b)
+    assert len(set(chosen_a.tolist())) == 3 and len(set(chosen_b.tolist())) >= 2     # the router does route
+    assert min(gap_a, gap_b) > 0.02      # no token so close to a tie that bfloat16 rounding could choose otherwise
+    all_of = lambda toks: list(range(len(toks)))
+    got_a, got_b = [], []
+    got_a.append(runner.step([StepEntry("a", a[:19], all_of(a[:19]))]))
+    out = runner.step([StepEntry("b", b[:2], all_of(b[:2])), StepEntry("a", a[19:50], all_of(a[19:50]))])
+    got_b.append(out[:2]); got_a.append(out[2:])
+    out = runner.step([StepEntry("b", b[2:], all_of(b[2:])), StepEntry("a", [a[50]], [0])])
+    got_b.append(out[:38]); got_a.append(out[38:])
+    for i in range(51, 61):
+        got_a.append(runner.step([StepEntry("a", [a[i]], [0])]))
+    for got, want in ((torch.cat(got_a), want_a), (torch.cat(got_b), want_b)):
+        err = np.abs(got.double().cpu().numpy() - want).max()
+        assert err <= tol * np.abs(want).max(), err
     runner.cache.check_invariants()
