@@ -345,51 +345,67 @@ attn_tile32_kernel(AttnArgs p) {
     const int32_t *tbl = p.tables + (size_t)seg * p.table_stride;
 
     // What of a chunk's address does not change from tile to tile (tiles start at multiples of 64 >= page size)
-    int k_key[CH], v_koff[CH];
-    size_t k_in_page[CH], v_in_page[CH], k_lds[CH], v_lds[CH];
+    int k_key[CH], v_koff[CH], k_in_page[CH], v_in_page[CH], k_lds[CH], v_lds[CH];
 #pragma unroll
     for (int c = 0; c < CH; c++) {
         const int ch = threadIdx.x + c * kThreads;
         const int key = ch >> (LD - 3), dc = ch & (D / 8 - 1);
         k_key[c] = key;
-        k_in_page[c] = ((size_t)kvh * ps + (key & pmask)) * D + dc * 8;
+        k_in_page[c] = (kvh * ps + (key & pmask)) * D + dc * 8;
         k_lds[c] = key * KP + dc * 8;
         const int pg = ch >> (LD + cps), rem = ch & ((D << cps) - 1);
         const int d = rem >> cps, hc = rem & ((1 << cps) - 1);
         v_koff[c] = (pg << psh) + hc * 8;
-        v_in_page[c] = ((size_t)kvh * D + d) * ps + hc * 8;
+        v_in_page[c] = (kvh * D + d) * ps + hc * 8;
         v_lds[c] = d * VP + v_koff[c];
     }
-    const size_t page_elems = (size_t)nkv * ps * D;
+    const unsigned page_elems = (unsigned)nkv * ps * D;   // the host has checked that it fits
 
     bf16x8_t kreg[CH], vreg[CH];
     // A tile's loads depend on its page numbers: those are asked for one tile earlier than the tile's keys and
     // values, which are asked for one tile before they are multiplied, so neither wait lies on the path.
+    // Tiles with no edge of the context inside (all but the first of a window and the last one or two) take the
+    // branch without a condition per lane: the address arithmetic of a tile is a few instructions a chunk.
     int pgk[CH], pgv[CH];
     auto pages = [&](int k0) {   // page numbers of tile k0 .. k0 + 63 (0 where the tile has no token)
         if (k0 > k_stop) return;
-        const bool inside = k0 >= lo_tile && k0 + KT - 1 <= p_last;
+        if (k0 >= lo_tile && k0 + KT - 1 <= p_last) {
+            const int32_t *t = tbl + (k0 >> psh);
+#pragma unroll
+            for (int c = 0; c < CH; c++) {
+                pgk[c] = t[k_key[c] >> psh];
+                pgv[c] = t[v_koff[c] >> psh];
+            }
+            return;
+        }
 #pragma unroll
         for (int c = 0; c < CH; c++) {
             const int kabs = k0 + k_key[c], vabs = k0 + v_koff[c];
-            pgk[c] = (inside || (kabs >= lo_tile && kabs <= p_last)) ? tbl[kabs >> psh] : 0;
-            pgv[c] = (inside || (vabs + 7 >= lo_tile && vabs <= p_last)) ? tbl[vabs >> psh] : 0;
+            pgk[c] = (kabs >= lo_tile && kabs <= p_last) ? tbl[kabs >> psh] : 0;
+            pgv[c] = (vabs + 7 >= lo_tile && vabs <= p_last) ? tbl[vabs >> psh] : 0;
         }
     };
     auto fetch = [&](int k0) {   // tile k0 .. k0 + 63 from the pages into registers; pages(k0) has run
-        const bool inside = k0 >= lo_tile && k0 + KT - 1 <= p_last;   // no edge of the context in this tile
+        if (k0 >= lo_tile && k0 + KT - 1 <= p_last) {
+#pragma unroll
+            for (int c = 0; c < CH; c++) {
+                kreg[c] = *(const bf16x8_t *)(p.kp + ((size_t)(unsigned)pgk[c] * page_elems + (unsigned)k_in_page[c]));
+                vreg[c] = *(const bf16x8_t *)(p.vp + ((size_t)(unsigned)pgv[c] * page_elems + (unsigned)v_in_page[c]));
+            }
+            return;
+        }
 #pragma unroll
         for (int c = 0; c < CH; c++) {
             const int kabs = k0 + k_key[c];
             bf16x8_t v = zero8();
-            if (inside || (kabs >= lo_tile && kabs <= p_last))
-                v = *(const bf16x8_t *)(p.kp + (size_t)pgk[c] * page_elems + k_in_page[c]);
+            if (kabs >= lo_tile && kabs <= p_last)
+                v = *(const bf16x8_t *)(p.kp + ((size_t)(unsigned)pgk[c] * page_elems + (unsigned)k_in_page[c]));
             kreg[c] = v;
             const int vabs = k0 + v_koff[c];
             v = zero8();
-            if (inside || (vabs + 7 >= lo_tile && vabs <= p_last)) {
-                v = *(const bf16x8_t *)(p.vp + (size_t)pgv[c] * page_elems + v_in_page[c]);
-                if (!inside && vabs + 7 > p_last) {   // slots past the last token hold whatever an earlier request left
+            if (vabs + 7 >= lo_tile && vabs <= p_last) {
+                v = *(const bf16x8_t *)(p.vp + ((size_t)(unsigned)pgv[c] * page_elems + (unsigned)v_in_page[c]));
+                if (vabs + 7 > p_last) {   // slots past the last token hold whatever an earlier request left
 #pragma unroll
                     for (int e = 0; e < 8; e++)
                         if (vabs + e > p_last) v[e] = (bf16_t)0.0f;
@@ -435,14 +451,18 @@ attn_tile32_kernel(AttnArgs p) {
             for (int ds = 0; ds < DS; ds++)
                 s[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t *)(krow + ds * 16), qf[ds], s[rb], 0, 0, 0);
         }
-        // tiles wholly below the diagonal and above every window edge need no mask (the same for all rows here)
+        // Tiles wholly below the diagonal and above every window edge need no mask (the same for all rows here).
+        // Key k0 + c + 8 h of the others is visible if lo_r <= key <= prow: the constant c is compared with limits
+        // that hold everything else.
         if (!(k0 + KT - 1 <= pos0 && k0 >= lo_all)) {
+            asm volatile("" ::: "memory");   // a branch of its own: folded into selects it would run for every tile
+            const int hi_lim = prow - k0 - 8 * h, lo_lim = lo_r - k0 - 8 * h;   // prow = -1 for rows outside the segment
 #pragma unroll
             for (int rb = 0; rb < 2; rb++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
-                    const int key = k0 + rb * 32 + 16 * (i >> 3) + 8 * h + (i & 7);
-                    if (!(key <= prow && key >= lo_r)) s[rb][i] = -INFINITY;   // prow = -1 for rows outside the segment
+                    const int c = rb * 32 + 16 * (i >> 3) + (i & 7);
+                    if (!(c <= hi_lim && c >= lo_lim)) s[rb][i] = -INFINITY;
                 }
         }
         float tmax = -INFINITY;
@@ -776,6 +796,7 @@ bool fast_shape(int heads, int kv_heads, int head_dim, int page_size) {
     if (head_dim != 32 && head_dim != 64 && head_dim != 128) return false;
     if (page_size != 8 && page_size != 16 && page_size != 32 && page_size != 64) return false;
     if (heads / kv_heads > 64) return false;
+    if (kv_heads > 4096) return false;   // offsets inside a page are kept in 32 bits
     return true;
 }
 

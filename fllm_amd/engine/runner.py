@@ -9,6 +9,7 @@ a batch: rust/engine/src/runtime.rs:2380-2442).
 """
 from __future__ import annotations
 
+import gc
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Union
 
@@ -361,6 +362,16 @@ class _DecodeGraph:
         if runner._graph_pool is None:
             runner._graph_pool = torch.cuda.graph_pool_handle()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, pool=runner._graph_pool):
-            self.logits = runner.model.forward(self.ctx)
+        # No garbage collection while the stream is capturing: a collector that frees what an engine before this
+        # one left behind (its graphs, its pinned buffers) calls into the HIP runtime, which refuses such calls
+        # during a capture, and a failure inside a destructor ends the process.
+        collecting = gc.isenabled()
+        gc.collect()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph, pool=runner._graph_pool):
+                self.logits = runner.model.forward(self.ctx)
+        finally:
+            if collecting:
+                gc.enable()
         self.graph = graph

@@ -116,6 +116,31 @@ def test_steps_launched_ahead_give_the_same_tokens(dtype):
     tight.runner.cache.check_invariants()
 
 
+def test_no_garbage_collection_while_a_graph_is_captured():
+    """Engines that went before leave cycles behind; their collection frees graphs and pinned buffers through the
+    HIP runtime, which must not happen while a stream is capturing: the collector is off for the capture's
+    length and on again after it."""
+    import gc
+    prompts = [tc.random_ids(n, 512, 40 + n) for n in PROMPT_LENGTHS["B"]]
+    params = SamplingParams(max_tokens=6)
+    want = make_engine("B", "bfloat16", ahead=True).generate(prompts, params)     # left behind for the collector
+    engine = make_engine("B", "bfloat16", ahead=True)
+    seen = []
+    forward = engine.runner.model.forward
+
+    def watched(ctx):
+        seen.append((torch.cuda.is_current_stream_capturing(), gc.isenabled()))
+        return forward(ctx)
+
+    engine.runner.model.forward = watched
+    assert gc.isenabled()
+    assert engine.generate(prompts, params) == want
+    assert gc.isenabled()
+    assert any(capturing for capturing, _ in seen)
+    assert all(not collecting for capturing, collecting in seen if capturing)
+    assert any(collecting for capturing, collecting in seen if not capturing)
+
+
 def test_command_line(tmp_path):
     folder = str(tmp_path / "model")
     write_random_model(folder, tc.TINY_A, seed=1, dtype="float32")
