@@ -1,4 +1,4 @@
-// Sampling on the device: one workgroup per row of logits.
+// Sampling on the device: one workgroup per row of logits (greedy rows of a wide vocabulary: several).
 //
 // Greedy rows take the first index of the largest finite value.  Other rows follow the
 // reference's device sampler (rust/engine/cuda/sampling.cu:1-13, :253-352): temperature, top-k
@@ -119,43 +119,6 @@ __device__ int row_argmax(const float *w, int vocab, Shared &sh) {
     return block_argmax(best, besti, sh);
 }
 
-// key of the k-th largest value of w (every element counts): radix select, 4 passes of 8 bits
-__device__ uint32_t kth_largest_key(const float *w, int vocab, int k, Shared &sh) {
-    if (threadIdx.x == 0) {
-        sh.prefix = 0;
-        sh.remaining = k;
-    }
-    __syncthreads();
-    for (int pass = 0; pass < 4; pass++) {
-        const int shift = 24 - 8 * pass;
-        for (int i = threadIdx.x; i < 256; i += kBlock) sh.hist[i] = 0;
-        __syncthreads();
-        const uint32_t prefix = sh.prefix;
-        for (int i = threadIdx.x; i < vocab; i += kBlock) {
-            const uint32_t key = f2key(w[i]);
-            const bool match = pass == 0 || (key >> (shift + 8)) == (prefix >> (shift + 8));
-            if (match) atomicAdd(&sh.hist[(key >> shift) & 255u], 1u);
-        }
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            int acc = 0;
-            const int rem = sh.remaining;
-            uint32_t bin = 0;
-            for (int b = 255; b >= 0; b--) {
-                if (acc + (int)sh.hist[b] >= rem) {
-                    bin = (uint32_t)b;
-                    break;
-                }
-                acc += (int)sh.hist[b];
-            }
-            sh.prefix = prefix | (bin << shift);
-            sh.remaining = rem - acc;
-        }
-        __syncthreads();
-    }
-    return sh.prefix;
-}
-
 __global__ void __launch_bounds__(kBlock)
 argmax_kernel(const float *__restrict__ logits, int32_t *__restrict__ out, int vocab) {
     __shared__ Shared sh;
@@ -205,10 +168,128 @@ argmax_split_kernel(const float *__restrict__ logits, int32_t *__restrict__ out,
     if (threadIdx.x == 0) out[row] = idx == 0x7fffffff ? 0 : idx;
 }
 
+// ---------------------------------------------------------------------------------------------
+// temperature / top-k / top-p / Gumbel-max
+// ---------------------------------------------------------------------------------------------
+// The thresholds of top-k and top-p lie among the few largest logits.  One pass over the vocabulary
+// fills a histogram over the distance from the largest logit, in steps of 1/64 up to 64 (token
+// counts for top-k, probability mass in 40-bit fixed point for top-p: integer sums, so the order of
+// the additions does not matter); the bin in which the threshold falls is read off it, the tokens
+// up to that bin are gathered into a list (in an order that depends on the data only), and the
+// exact thresholds (radix select, bisection over the keys with sums in double precision) and the
+// draw then run over the list.  A threshold further than 64 below the maximum puts every token on
+// the list.
+constexpr int kBins = 4096;
+constexpr float kBinsPerUnit = 64.0f;
+
+// bin of a finite logit v <= m; kBins: further from the maximum than the histogram reaches
+__device__ __forceinline__ int bin_of(float v, float m) {
+    const float d = (m - v) * kBinsPerUnit;
+    return d < (float)kBins ? (int)d : kBins;
+}
+
+// exclusive prefix sum over the threads of the workgroup, and the total
+__device__ __forceinline__ int block_exclusive_scan(int v, Shared &sh, int *total) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    int inc = v;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        const int n = __shfl_up(inc, o, kWave);
+        if (lane >= o) inc += n;
+    }
+    __syncthreads();
+    if (lane == kWave - 1) sh.ired[wave] = inc;
+    __syncthreads();
+    int before = 0, all = 0;
+#pragma unroll
+    for (int i = 0; i < kWaves; i++) {
+        if (i < wave) before += sh.ired[i];
+        all += sh.ired[i];
+    }
+    __syncthreads();
+    *total = all;
+    return before + inc - v;
+}
+
+// The lowest bin b with sum(hist[0..b]) >= target, kBins when the whole histogram falls short; done by the first
+// wave, every lane over 64 bins; the same value in every thread.
+__device__ int find_bin(const unsigned long long *hist, unsigned long long target, Shared &sh) {
+    __syncthreads();
+    if (threadIdx.x < kWave) {
+        const int lane = threadIdx.x;
+        constexpr int PER = kBins / kWave;
+        unsigned long long own = 0;
+        for (int i = 0; i < PER; i++) own += hist[lane * PER + i];
+        unsigned long long below = 0;      // sum of the lanes before this one
+        for (int o = 1; o < kWave; o++) {
+            const unsigned long long other = __shfl(own, (lane - o) & (kWave - 1), kWave);
+            if (lane - o >= 0) below += other;
+        }
+        int found = kBins;
+        if (below < target && below + own >= target) {      // the crossing lies in this lane's bins: one lane, if any
+            unsigned long long cum = below;
+            for (int i = 0; i < PER; i++) {
+                cum += hist[lane * PER + i];
+                if (cum >= target) {
+                    found = lane * PER + i;
+                    break;
+                }
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) found = min(found, __shfl_xor(found, o, kWave));
+        if (lane == 0) sh.remaining = found;
+    }
+    __syncthreads();
+    const int bin = sh.remaining;
+    __syncthreads();
+    return bin;
+}
+
+// key of the k-th largest value among get(0 .. n-1): radix select, 4 passes of 8 bits
+template <typename Get>
+__device__ uint32_t kth_largest_key_of(Get get, int n, int k, Shared &sh) {
+    if (threadIdx.x == 0) {
+        sh.prefix = 0;
+        sh.remaining = k;
+    }
+    __syncthreads();
+    for (int pass = 0; pass < 4; pass++) {
+        const int shift = 24 - 8 * pass;
+        for (int i = threadIdx.x; i < 256; i += kBlock) sh.hist[i] = 0;
+        __syncthreads();
+        const uint32_t prefix = sh.prefix;
+        for (int i = threadIdx.x; i < n; i += kBlock) {
+            const uint32_t key = f2key(get(i));
+            const bool match = pass == 0 || (key >> (shift + 8)) == (prefix >> (shift + 8));
+            if (match) atomicAdd(&sh.hist[(key >> shift) & 255u], 1u);
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int acc = 0;
+            const int rem = sh.remaining;
+            uint32_t bin = 0;
+            for (int b = 255; b >= 0; b--) {
+                if (acc + (int)sh.hist[b] >= rem) {
+                    bin = (uint32_t)b;
+                    break;
+                }
+                acc += (int)sh.hist[b];
+            }
+            sh.prefix = prefix | (bin << shift);
+            sh.remaining = rem - acc;
+        }
+        __syncthreads();
+    }
+    return sh.prefix;
+}
+
+// `work` gives every row `vocab` 32-bit words of its own (the list of token ids); it must not overlap the logits.
 __global__ void __launch_bounds__(kBlock)
-sample_kernel(const float *logits, float *work, const FllmSampleRow *__restrict__ params,
+sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const FllmSampleRow *__restrict__ params,
               int32_t *__restrict__ out, int vocab) {
     __shared__ Shared sh;
+    __shared__ unsigned long long bins[kBins];
     const int row = blockIdx.x;
     const FllmSampleRow p = params[row];
     const float *src = logits + (size_t)row * vocab;
@@ -217,56 +298,101 @@ sample_kernel(const float *logits, float *work, const FllmSampleRow *__restrict_
         if (threadIdx.x == 0) out[row] = idx == 0x7fffffff ? 0 : idx;
         return;
     }
-    float *w = work + (size_t)row * vocab;
+    int *list = (int *)(work + (size_t)row * vocab);
     float m = -INFINITY;
-    for (int i = threadIdx.x; i < vocab; i += kBlock) {
-        const float v = sanitize(src[i]);
-        w[i] = v;
-        m = fmaxf(m, v);
-    }
-    m = block_max_f(m, sh);   // its barriers also publish w[]
+    for (int i = threadIdx.x; i < vocab; i += kBlock) m = fmaxf(m, sanitize(src[i]));
+    m = block_max_f(m, sh);
     if (!(m > -INFINITY)) {
         if (threadIdx.x == 0) out[row] = 0;   // no finite logit: the reference's argmax gives index 0 as well
         return;
     }
     const float inv_t = (float)(1.0 / (double)p.temperature);
-    if (p.top_k > 0 && p.top_k < vocab) {
-        const uint32_t t = kth_largest_key(w, vocab, p.top_k, sh);
-        for (int i = threadIdx.x; i < vocab; i += kBlock)
-            if (f2key(w[i]) < t) w[i] = -INFINITY;
+    const bool use_k = p.top_k > 0 && p.top_k < vocab;
+    const bool use_p = p.top_p > 0.f && p.top_p < 1.f;
+    int count = vocab;                       // tokens the draw looks at: all of them, or the list
+    uint32_t threshold = 0;                  // key below which a listed token is out
+    if (use_k || use_p) {
+        for (int i = threadIdx.x; i < kBins; i += kBlock) bins[i] = 0;
         __syncthreads();
-    }
-    if (p.top_p > 0.f && p.top_p < 1.f) {
-        double part = 0.0;
-        for (int i = threadIdx.x; i < vocab; i += kBlock)
-            if (w[i] > -INFINITY) part += (double)expf((w[i] - m) * inv_t);
-        const double target = (double)p.top_p * block_sum_d(part, sh);
-        // largest key t such that the mass of {key >= t} still reaches the target
-        uint32_t lo = 0, hi = 0xFFFFFFFFu;
-        while (lo < hi) {
-            const uint32_t mid = lo + ((hi - lo) >> 1) + 1;
-            part = 0.0;
-            for (int i = threadIdx.x; i < vocab; i += kBlock) {
-                const float v = w[i];
-                if (v > -INFINITY && f2key(v) >= mid) part += (double)expf((v - m) * inv_t);
+        double total = 0.0;                  // mass of all finite logits (top-p without top-k)
+        unsigned long long reach = 0;        // what this thread put into the histogram, in its units (top-p)
+        for (int i = threadIdx.x; i < vocab; i += kBlock) {
+            const float v = sanitize(src[i]);
+            if (!(v > -INFINITY)) continue;
+            const int b = bin_of(v, m);
+            if (use_k) {
+                if (b < kBins) atomicAdd(&bins[b], 1ull);
+            } else {
+                const float e = expf((v - m) * inv_t);
+                total += (double)e;
+                const unsigned long long fixed = (unsigned long long)((double)e * 1099511627776.0);
+                reach += fixed;
+                if (b < kBins && fixed != 0) atomicAdd(&bins[b], fixed);
             }
-            if (block_sum_d(part, sh) >= target) lo = mid;
-            else hi = mid - 1;
         }
-        for (int i = threadIdx.x; i < vocab; i += kBlock)
-            if (w[i] > -INFINITY && f2key(w[i]) < lo) w[i] = -INFINITY;
+        int last_bin;
+        if (use_k) {
+            last_bin = find_bin(bins, (unsigned long long)p.top_k, sh);
+        } else {
+            total = block_sum_d(total, sh);
+            // the sum of every thread's share, far tokens included: integers, the same in any order
+            const double all = block_sum_d((double)reach, sh);
+            last_bin = find_bin(bins, (unsigned long long)((double)p.top_p * all), sh);
+            if (last_bin < kBins) last_bin++;   // a bin to spare: the histogram's sums are rounded, the exact ones decide
+        }
+        // gather the tokens up to that bin: thread t's tokens in the order it meets them, behind those of the threads before it
+        int mine = 0;
+        for (int i = threadIdx.x; i < vocab; i += kBlock) {
+            const float v = sanitize(src[i]);
+            mine += (v > -INFINITY && bin_of(v, m) <= last_bin) ? 1 : 0;
+        }
+        int at = block_exclusive_scan(mine, sh, &count);
+        for (int i = threadIdx.x; i < vocab; i += kBlock) {
+            const float v = sanitize(src[i]);
+            if (v > -INFINITY && bin_of(v, m) <= last_bin) list[at++] = i;
+        }
         __syncthreads();
+        auto listed = [&](int i) { return sanitize(src[list[i]]); };
+        if (use_k) {
+            threshold = kth_largest_key_of(listed, count, min(p.top_k, count), sh);
+            if (use_p) {                      // the mass of what top-k left
+                total = 0.0;
+                for (int i = threadIdx.x; i < count; i += kBlock) {
+                    const float v = listed(i);
+                    if (f2key(v) >= threshold) total += (double)expf((v - m) * inv_t);
+                }
+                total = block_sum_d(total, sh);
+            }
+        }
+        if (use_p) {
+            const double target = (double)p.top_p * total;
+            // largest key t such that the mass of {key >= t} still reaches the target
+            uint32_t lo = threshold, hi = 0xFFFFFFFFu;
+            while (lo < hi) {
+                const uint32_t mid = lo + ((hi - lo) >> 1) + 1;
+                double part = 0.0;
+                for (int i = threadIdx.x; i < count; i += kBlock) {
+                    const float v = listed(i);
+                    if (f2key(v) >= mid) part += (double)expf((v - m) * inv_t);
+                }
+                if (block_sum_d(part, sh) >= target) lo = mid;
+                else hi = mid - 1;
+            }
+            threshold = lo;
+        }
     }
     float best = -INFINITY;
     int besti = 0x7fffffff;
-    for (int i = threadIdx.x; i < vocab; i += kBlock) {
-        const float v = w[i];
-        if (!(v > -INFINITY)) continue;
-        const float u = philox_uniform(p.seed, p.draw, (uint32_t)i);
+    const bool whole = !(use_k || use_p);
+    for (int i = threadIdx.x; i < count; i += kBlock) {
+        const int id = whole ? i : list[i];
+        const float v = sanitize(src[id]);
+        if (!(v > -INFINITY) || f2key(v) < threshold) continue;
+        const float u = philox_uniform(p.seed, p.draw, (uint32_t)id);
         const float score = (v - m) * inv_t - logf(-logf(u));
-        if (score > best) {
+        if (score > best || (score == best && id < besti)) {
             best = score;
-            besti = i;
+            besti = id;
         }
     }
     const int idx = block_argmax(best, besti, sh);

@@ -231,6 +231,22 @@ def philox_uniform(seed, draw, index):
     return np.float32((np.float32(w >> 8) + np.float32(0.5)) / np.float32(16777216.0))
 
 
+def philox_uniform_many(seed, draw, indices):
+    """philox_uniform for an array of indices at once (the same arithmetic on uint64 arrays)."""
+    mask = np.uint64(0xFFFFFFFF)
+    c = [np.asarray(indices, dtype=np.uint64) & mask, np.zeros(len(indices), np.uint64),
+         np.full(len(indices), draw & 0xFFFFFFFF, np.uint64), np.full(len(indices), draw >> 32, np.uint64)]
+    k0, k1 = seed & 0xFFFFFFFF, seed >> 32
+    for _ in range(10):
+        p0 = np.uint64(_M0) * c[0]
+        p1 = np.uint64(_M1) * c[2]
+        c = [((p1 >> np.uint64(32)) ^ c[1] ^ np.uint64(k0)) & mask, p1 & mask,
+             ((p0 >> np.uint64(32)) ^ c[3] ^ np.uint64(k1)) & mask, p0 & mask]
+        k0, k1 = (k0 + _W0) & 0xFFFFFFFF, (k1 + _W1) & 0xFFFFFFFF
+    w = (c[0] >> np.uint64(8)).astype(np.float32)
+    return ((w + np.float32(0.5)) / np.float32(16777216.0)).astype(np.float32)
+
+
 def device_survivors(logits, temperature, top_k, top_p):
     """The tokens the reference's device sampler still draws from, as a float32 array of logits
     with -inf for the others (rust/engine/cuda/sampling.cu:253-330), with sorting in place of its
@@ -250,9 +266,10 @@ def device_survivors(logits, temperature, top_k, top_p):
         alive = np.isfinite(w)
         e = np.where(alive, np.exp(((w - m) * inv_t).astype(np.float32)).astype(np.float64), 0.0)
         target = float(np.float32(top_p)) * e.sum()
-        values = np.unique(w[alive])[::-1]                      # distinct values, descending
-        mass = np.array([e[w >= v].sum() for v in values])      # mass of {value >= v}
-        threshold = values[np.flatnonzero(mass >= target)[0]]   # largest threshold that still reaches the target
+        values, inverse = np.unique(w[alive], return_inverse=True)           # distinct values, ascending
+        per_value = np.bincount(inverse, weights=e[alive], minlength=len(values))
+        mass = np.cumsum(per_value[::-1])                       # mass of {value >= v}, v descending
+        threshold = values[::-1][np.flatnonzero(mass >= target)[0]]   # largest threshold that still reaches the target
         w[w < threshold] = -np.inf
     return w
 
@@ -270,10 +287,7 @@ def device_sample(logits, temperature, top_k, top_p, seed, draw):
     w = device_survivors(logits, temperature, top_k, top_p)
     m = finite.max()
     inv_t = np.float32(1.0 / float(temperature))
-    best, best_i = -np.inf, None
-    for i in np.flatnonzero(np.isfinite(w)):
-        u = philox_uniform(seed, draw, int(i))
-        score = np.float32((w[i] - m) * inv_t) - np.log(-np.log(u, dtype=np.float32), dtype=np.float32)
-        if score > best:
-            best, best_i = score, int(i)
-    return best_i
+    alive = np.flatnonzero(np.isfinite(w))
+    u = philox_uniform_many(seed, draw, alive)
+    score = ((w[alive] - m) * inv_t).astype(np.float32) - np.log(-np.log(u, dtype=np.float32), dtype=np.float32)
+    return int(alive[np.flatnonzero(score == score.max())[0]])

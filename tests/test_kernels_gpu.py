@@ -602,6 +602,40 @@ def test_sample_matches_the_plain_sampler(ops):
             assert int(out[i]) == want, (draw, i)
 
 
+@pytest.mark.parametrize("vocab", [50000, 128256])
+def test_sample_thresholds_on_wide_vocabularies(ops, vocab):
+    """Thresholds among the few largest logits, thresholds further from the maximum than the sampler's histogram
+    reaches, ties at the threshold, flat rows, rows with holes: the token is the plain sampler's in every draw."""
+    from fllm_amd.sampling import SampleRequest, SamplingParams, pack_rows
+    g = gen(23)
+    rows = {
+        "normal": torch.randn(vocab, generator=g) * 3.0,
+        "wide": torch.randn(vocab, generator=g) * 60.0,                      # thresholds far below the maximum
+        "flat": torch.zeros(vocab),                                          # all tied
+        "steps": torch.randint(0, 12, (vocab,), generator=g).float() * 0.5,  # many ties at every level
+        "holes": torch.randn(vocab, generator=g) * 2.0,
+        "peak": torch.randn(vocab, generator=g),
+    }
+    rows["holes"][::3] = float("-inf")
+    rows["holes"][5] = float("nan")
+    rows["holes"][11] = float("inf")
+    rows["peak"][vocab - 7] = 30.0
+    cases = [SamplingParams(temperature=0.8), SamplingParams(temperature=1.0, top_k=1), SamplingParams(temperature=0.6, top_k=5),
+             SamplingParams(temperature=1.1, top_k=64), SamplingParams(temperature=1.0, top_k=vocab - 1),
+             SamplingParams(temperature=0.7, top_p=0.01), SamplingParams(temperature=1.0, top_p=0.5),
+             SamplingParams(temperature=2.5, top_p=0.9), SamplingParams(temperature=4.0, top_p=0.999),
+             SamplingParams(temperature=1.3, top_k=50, top_p=0.5), SamplingParams(temperature=0.9, top_k=2000, top_p=0.95)]
+    for name, row in rows.items():
+        logits = row.view(1, vocab).expand(len(cases), vocab).contiguous()
+        for draw in range(2):
+            reqs = [SampleRequest(p, seed=99 + i, draw=draw) for i, p in enumerate(cases)]
+            out = torch.empty(len(cases), dtype=torch.int32, device=DEV)
+            ops.sample(logits.to(DEV), torch.empty(len(cases), vocab, device=DEV), pack_rows(reqs).to(DEV), out)
+            for i, p in enumerate(cases):
+                want = plain_llama.device_sample(row.numpy(), p.temperature, p.top_k, p.top_p, 99 + i, draw)
+                assert int(out[i]) == want, (name, draw, i)
+
+
 def test_sample_depends_only_on_seed_draw_and_logits(ops):
     from fllm_amd.sampling import SampleRequest, SamplingParams, pack_rows
     g = gen(18)

@@ -217,6 +217,9 @@ def test_philox_uniforms():
     assert np.all(np.abs(np.histogram(us, bins=8, range=(0, 1))[0] - 500) < 100)
     assert P.philox_uniform(1, 0, 0) != P.philox_uniform(2, 0, 0) and P.philox_uniform(1, 0, 0) != P.philox_uniform(1, 0, 1)
     assert P.philox_uniform(7, 3, 9) == P.philox_uniform(7, 3, 9)
+    many = P.philox_uniform_many((5 << 40) + 77, (3 << 33) + 9, np.array([0, 1, 2, 70000, 0xFFFFFFFF]))
+    assert many.dtype == np.float32
+    assert many.tolist() == [P.philox_uniform((5 << 40) + 77, (3 << 33) + 9, i) for i in (0, 1, 2, 70000, 0xFFFFFFFF)]
 
 
 def test_greedy_takes_the_first_maximum():
