@@ -276,8 +276,9 @@ extern "C" int fllm_add_residual(float *residual, const void *branch, int rows, 
 }
 
 // bfloat16 rows, pairs (2l, 2l+1), head_dim and rope_dims in steps of 8: every thread takes 8 neighbouring lanes of
-// a head (16-byte loads and stores; cosines and sines as two 16-byte loads each).  A workgroup takes 8 rows; where
-// they are 8 consecutive tokens of one request that start at a multiple of 8 (a prompt portion), their values go
+// a head (16-byte loads and stores; cosines and sines as two 16-byte loads each).  Prompt portions: four workgroups
+// share 8 rows (a read and a write of the same buffer cannot overlap inside a thread, so many short threads beat few
+// long ones); where the rows are 8 consecutive tokens of one request that start at a multiple of 8 (a prompt portion), their values go
 // into the transposed page as one 16-byte store per head lane instead of eight 2-byte ones.
 template <int RB>
 __global__ void __launch_bounds__(kBlock)
@@ -291,55 +292,66 @@ rope_kv_store_vec_kernel(bf16_t *__restrict__ qkv, const int32_t *__restrict__ r
     const int per_head = head_dim / 8;
     const int rot_heads = store_kv ? heads + kv_heads : heads;
     const size_t row_elems = (size_t)(heads + 2 * kv_heads) * head_dim;
-    const int seg0 = row_seg[r0], pos0 = row_pos[r0];
-    bool run = RB == 8 && store_kv && nrows == RB && seg0 >= 0 && (pos0 & (RB - 1)) == 0 && page_size % RB == 0;
-    for (int i = 1; i < RB && run; i++) run = row_seg[r0 + i] == seg0 && row_pos[r0 + i] == pos0 + i;
+    // position (-1: padding row), page and slot of the workgroup's rows
+    __shared__ int s_pos[RB], s_page[RB], s_off[RB], s_run;
+    if ((int)threadIdx.x < nrows) {
+        const int r = r0 + threadIdx.x;
+        const int seg = row_seg[r], pos = row_pos[r];
+        s_pos[threadIdx.x] = seg < 0 ? -1 : pos;
+        s_page[threadIdx.x] = (store_kv && seg >= 0) ? tables[(size_t)seg * table_stride + pos / page_size] : 0;
+        s_off[threadIdx.x] = pos % page_size;
+    }
+    if (threadIdx.x == 0) {
+        const int seg0 = row_seg[r0], pos0 = row_pos[r0];
+        bool run = RB == 8 && store_kv && nrows == RB && seg0 >= 0 && (pos0 & (RB - 1)) == 0 && page_size % RB == 0;
+        for (int i = 1; i < RB && run; i++) run = row_seg[r0 + i] == seg0 && row_pos[r0 + i] == pos0 + i;
+        s_run = run;
+    }
+    __syncthreads();
+    const bool run = s_run != 0;
 
-    for (int i = 0; i < nrows; i++) {
-        const int r = r0 + i;
-        const int seg = row_seg[r];
-        if (seg < 0) continue;   // padding row
-        const int pos = row_pos[r];
-        const float *cs = cos_table + (size_t)pos * half;
-        const float *sn = sin_table + (size_t)pos * half;
-        bf16_t *row = qkv + (size_t)r * row_elems;
-        int page = 0, off = 0;
-        if (store_kv) {
-            page = tables[(size_t)seg * table_stride + pos / page_size];
-            off = pos % page_size;
-        }
-        for (int t = threadIdx.x; t < rot_heads * per_head; t += kBlock) {
-            const int h = t / per_head, c = (t - h * per_head) * 8;
-            bf16x8_t v = *(const bf16x8_t *)(row + (size_t)h * head_dim + c);
-            if (c < rope_dims) {   // rope_dims is a multiple of 8: the chunk is rotated as a whole
-                const f32x4_t c4 = *(const f32x4_t *)(cs + c / 2), s4 = *(const f32x4_t *)(sn + c / 2);
+    // queries and keys: every (row, 16-byte chunk) is a piece of work of its own, so that a thread has several in flight
+    const int per_row = rot_heads * per_head;
+    const int first = blockIdx.y * kBlock + threadIdx.x, stride = gridDim.y * kBlock;   // the workgroups of a row group share its pieces
+    for (int it = first; it < nrows * per_row; it += stride) {
+        const int i = RB == 1 ? 0 : it / per_row, t = it - i * per_row;
+        const int pos = s_pos[i];
+        if (pos < 0) continue;   // padding row
+        const int h = t / per_head, c = (t - h * per_head) * 8;
+        bf16_t *row = qkv + (size_t)(r0 + i) * row_elems;
+        bf16x8_t v = *(const bf16x8_t *)(row + (size_t)h * head_dim + c);
+        if (c < rope_dims) {   // rope_dims is a multiple of 8: the chunk is rotated as a whole
+            const f32x4_t c4 = *(const f32x4_t *)(cos_table + (size_t)pos * half + c / 2);
+            const f32x4_t s4 = *(const f32x4_t *)(sin_table + (size_t)pos * half + c / 2);
 #pragma unroll
-                for (int p = 0; p < 4; p++) {
-                    const float a = (float)v[2 * p], b = (float)v[2 * p + 1];
-                    v[2 * p] = (bf16_t)(a * c4[p] - b * s4[p]);
-                    v[2 * p + 1] = (bf16_t)(b * c4[p] + a * s4[p]);
-                }
+            for (int p = 0; p < 4; p++) {
+                const float a = (float)v[2 * p], b = (float)v[2 * p + 1];
+                v[2 * p] = (bf16_t)(a * c4[p] - b * s4[p]);
+                v[2 * p + 1] = (bf16_t)(b * c4[p] + a * s4[p]);
             }
-            if (h < heads) *(bf16x8_t *)(row + (size_t)h * head_dim + c) = v;
-            else *(bf16x8_t *)(k_pages + (((size_t)page * kv_heads + (h - heads)) * page_size + off) * head_dim + c) = v;
         }
-        if (!store_kv || run) continue;
+        if (h < heads) *(bf16x8_t *)(row + (size_t)h * head_dim + c) = v;
+        else *(bf16x8_t *)(k_pages + (((size_t)s_page[i] * kv_heads + (h - heads)) * page_size + s_off[i]) * head_dim + c) = v;
+    }
+    if (!store_kv) return;
+    if (!run) {
         // values, stored transposed inside the page: [head_dim][token]
-        const bf16_t *vrow = row + (size_t)(heads + kv_heads) * head_dim;
-        for (int t = threadIdx.x; t < kv_heads * per_head; t += kBlock) {
+        const int v_per_row = kv_heads * per_head;
+        for (int it = first; it < nrows * v_per_row; it += stride) {
+            const int i = RB == 1 ? 0 : it / v_per_row, t = it - i * v_per_row;
+            if (s_pos[i] < 0) continue;
             const int h = t / per_head, c = (t - h * per_head) * 8;
-            const bf16x8_t v = *(const bf16x8_t *)(vrow + (size_t)h * head_dim + c);
-            bf16_t *dst = v_pages + (((size_t)page * kv_heads + h) * head_dim + c) * page_size + off;
+            const bf16x8_t v = *(const bf16x8_t *)(qkv + (size_t)(r0 + i) * row_elems + (size_t)(heads + kv_heads + h) * head_dim + c);
+            bf16_t *dst = v_pages + (((size_t)s_page[i] * kv_heads + h) * head_dim + c) * page_size + s_off[i];
 #pragma unroll
             for (int e = 0; e < 8; e++) dst[(size_t)e * page_size] = v[e];
         }
+        return;
     }
-    if (!run) return;
     // the values of the 8 tokens, one head lane at a time: 16 contiguous bytes of the transposed page
-    const int page = tables[(size_t)seg0 * table_stride + pos0 / page_size];
-    const int off = pos0 % page_size;
+    const int page = s_page[0], off = s_off[0];
     const bf16_t *vbase = qkv + (size_t)r0 * row_elems + (size_t)(heads + kv_heads) * head_dim;
-    for (int t = threadIdx.x; t < kv_heads * head_dim; t += kBlock) {
+    for (int t = first; t < kv_heads * head_dim; t += stride) {
         const int h = t / head_dim, c = t - h * head_dim;
         bf16x8_t v;
 #pragma unroll
@@ -371,7 +383,7 @@ extern "C" int fllm_rope_kv_store(void *qkv, const int32_t *row_pos, const int32
         // prompt portions: 8 rows a workgroup, so that runs of 8 tokens store their values 16 bytes at a time; few rows
         // (decode steps): a workgroup a row
         if (rows >= 256)
-            hipLaunchKernelGGL(rope_kv_store_vec_kernel<8>, dim3((rows + 7) / 8), dim3(kBlock), 0, stream, (bf16_t *)qkv, row_pos,
+            hipLaunchKernelGGL(rope_kv_store_vec_kernel<8>, dim3((rows + 7) / 8, 4), dim3(kBlock), 0, stream, (bf16_t *)qkv, row_pos,
                                row_seg, tables, table_stride, cos_table, sin_table, (bf16_t *)k_pages, (bf16_t *)v_pages, rows,
                                heads, kv_heads, head_dim, rope_dims, page_size, store_kv);
         else
