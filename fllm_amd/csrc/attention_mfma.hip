@@ -352,7 +352,10 @@ attn_tile32_kernel(AttnArgs p) {
         const int key = ch >> (LD - 3), dc = ch & (D / 8 - 1);
         k_key[c] = key;
         k_in_page[c] = (kvh * ps + (key & pmask)) * D + dc * 8;
-        k_lds[c] = key * KP + dc * 8;
+        // A key's row in LDS: bits 2 and 3 of the key swapped, which is where the products read it (row q of a 32-key
+        // block is key 16 (q / 16) + 8 (q / 4 % 2) + 4 (q / 8 % 2) + q % 4, see the table above, and that map is this swap): the 8 lanes of a 128-byte LDS access then read 8
+        // consecutive rows, 16 bytes further along the banks each, instead of hitting every bank twice.
+        k_lds[c] = ((key & ~12) | ((key & 4) << 1) | ((key & 8) >> 1)) * KP + dc * 8;
         const int pg = ch >> (LD + cps), rem = ch & ((D << cps) - 1);
         const int d = rem >> cps, hc = rem & ((1 << cps) - 1);
         v_koff[c] = (pg << psh) + hc * 8;
@@ -422,8 +425,6 @@ attn_tile32_kernel(AttnArgs p) {
         for (int i = 0; i < 16; i++) o[db][i] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;   // the running maximum is kept in raw units (before the scale)
     const float sc = p.scale_log2;
-    // A row q of a 32-key block is this key of the block (see the table above)
-    const int a_key = 16 * (q >> 4) + 8 * ((q >> 2) & 1) + 4 * ((q >> 3) & 1) + (q & 3);
 
     pages(kbegin);
     fetch(kbegin);
@@ -446,7 +447,7 @@ attn_tile32_kernel(AttnArgs p) {
         for (int rb = 0; rb < 2; rb++) {
 #pragma unroll
             for (int i = 0; i < 16; i++) s[rb][i] = 0.f;
-            const bf16_t *krow = Ks + (rb * 32 + a_key) * KP + h * 8;
+            const bf16_t *krow = Ks + (rb * 32 + q) * KP + h * 8;
 #pragma unroll
             for (int ds = 0; ds < DS; ds++)
                 s[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t *)(krow + ds * 16), qf[ds], s[rb], 0, 0, 0);
