@@ -65,6 +65,8 @@ def main():
     ap.add_argument("--no-ahead", action="store_true", help="every step waits for the tokens of the step before it")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run the 2,048-token prefill steps alone and print their time (for profiling); no JSON line")
+    ap.add_argument("--prompt-tokens", type=int, default=PREFILL_TOKENS,
+                    help="with --prefill-only: length of the prompt; longer ones run in portions of 2,048 tokens")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine runs on a single MI355X, --gpus {args.gpus} is not supported")
@@ -78,9 +80,10 @@ def main():
     steps, warmup = args.steps, args.warmup
     batches = [args.batch] if args.no_points or args.prefill_only else sorted({1, args.batch, 64})
     slack = max(batches) + 8          # requests whose prompt is done early decode while the others still prefill
-    need_tokens = max(batches) * (PROMPT_LEN + warmup + steps + slack + PAGE_SIZE) + PREFILL_TOKENS + 64
+    prompt_tokens = args.prompt_tokens if args.prefill_only else PREFILL_TOKENS
+    need_tokens = max(batches) * (PROMPT_LEN + warmup + steps + slack + PAGE_SIZE) + prompt_tokens + 64
     t0 = time.time()
-    engine = Engine(config=cfg, seed=0, dtype="bfloat16", device="cuda:0", ctx=CONTEXT, max_seqs=max(batches),
+    engine = Engine(config=cfg, seed=0, dtype="bfloat16", device="cuda:0", ctx=max(CONTEXT, prompt_tokens + 64), max_seqs=max(batches),
                     max_batched_tokens=PREFILL_TOKENS, block_size=PAGE_SIZE, num_blocks=-(-need_tokens // PAGE_SIZE),
                     decode_first=True, random_weights_on_device=True, ahead=not args.no_ahead)
     print(f"[bench] engine ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
@@ -116,10 +119,11 @@ def main():
         return tokens / elapsed, elapsed / steps * 1e3, mean_contexts
 
     def prefill_run(repeats=4):
-        """One request, its 2,048 tokens in one step; the median of the repeats after the first."""
+        """One request, its 2,048 tokens in one step (a longer prompt: in portions of 2,048); the median of the repeats
+        after the first."""
         times = []
         for i in range(repeats):
-            engine.add_request(f"prefill-{i}", rng.integers(0, vocab, PREFILL_TOKENS).tolist(),
+            engine.add_request(f"prefill-{i}", rng.integers(0, vocab, prompt_tokens).tolist(),
                                SamplingParams(max_tokens=1, ignore_eos=True))
             torch.cuda.synchronize()
             start = time.perf_counter()
@@ -133,7 +137,8 @@ def main():
 
     if args.prefill_only:
         best = prefill_run(max(2, steps))
-        print(f"[bench] prefill {PREFILL_TOKENS} tokens: {best * 1e3:.2f} ms", file=sys.stderr, flush=True)
+        print(f"[bench] prefill {prompt_tokens} tokens: {best * 1e3:.2f} ms, {prompt_tokens / best:.0f} tokens/s",
+              file=sys.stderr, flush=True)
         return
 
     results = {}
