@@ -425,6 +425,7 @@ attn_tile32_kernel(AttnArgs p) {
         for (int i = 0; i < 16; i++) o[db][i] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;   // the running maximum is kept in raw units (before the scale)
     const float sc = p.scale_log2;
+    const float tau = 8.0f / sc;
 
     pages(kbegin);
     fetch(kbegin);
@@ -472,7 +473,11 @@ attn_tile32_kernel(AttnArgs p) {
 #pragma unroll
             for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, s[rb][i]);
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-        const float m_new = fmaxf(m_run, tmax);
+        // The reference point of the exponents follows the maximum only when that has grown by more than 2^8 in the
+        // exponent's units: until then the probabilities are at most 256 times their final size, which float32 sums and
+        // bfloat16 operands hold as well, and the outputs need no rescaling (with it at every new maximum, short
+        // contexts rescaled in most tiles).
+        const float m_new = tmax > m_run + tau ? tmax : m_run;
         const float mc = m_new == -INFINITY ? 0.f : m_new * sc;   // nothing seen yet: exp2(-inf - 0) = 0 below
         const float alpha = m_run == -INFINITY ? 0.f : fast_exp2(m_run * sc - mc);
         float psum = 0.f;
