@@ -13,7 +13,8 @@ import trace_tools as tt
 
 pytestmark = pytest.mark.gpu
 
-LENGTHS = {"A": [5, 17, 31, 70, 128, 100], "B": [1, 9, 40, 100, 256, 130], "C": [3, 50, 190, 77, 120, 64]}
+LENGTHS = {"A": [5, 17, 31, 70, 128, 100], "B": [1, 9, 40, 100, 256, 130], "C": [3, 50, 190, 77, 120, 64],
+           "D": [700, 3, 130, 1000, 64]}
 # |engine - plain| <= tol * max|plain logit| ; float32 engine against a float64 reference, and
 # bfloat16 (8 bits of mantissa in weights, activations and cache) against the same
 TOL = {"float32": 2e-5, "bfloat16": 4e-2}
@@ -62,7 +63,7 @@ def make_runner(folder, dtype, page_size, max_tokens, use_graphs=True):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("family", ["whole", "last32", "portions", "mixed"])
 def test_replay(models, tmp_path, name, dtype, family):
     folder, cfg, requests, plain = models[name]

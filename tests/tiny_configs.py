@@ -1,5 +1,7 @@
 """Tiny Llama configurations for tests.  A and B differ in every size and option; C adds a
-sliding window on some layers, a partial rotary width, linear rotary scaling and biases."""
+sliding window on some layers, a partial rotary width, linear rotary scaling and biases; D has heads
+of 64 (the head size of the 128-row prompt attention kernel) and room for a thousand positions, so that
+a portion of a prompt meets contexts of many key tiles."""
 import json
 
 import numpy as np
@@ -27,8 +29,16 @@ TINY_C = {
     "sliding_window": 24, "layer_types": ["sliding_attention", "full_attention", "sliding_attention", "full_attention"],
     "tie_word_embeddings": False, "max_position_embeddings": 192, "hidden_act": "silu",
 }
-PAGE_SIZES = {"A": 16, "B": 8, "C": 16}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+TINY_D = {
+    "model_type": "llama", "architectures": ["LlamaForCausalLM"],
+    "num_hidden_layers": 2, "hidden_size": 128, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 64,
+    "intermediate_size": 320, "vocab_size": 384, "rope_theta": 100000.0, "rms_norm_eps": 1e-5,
+    "rope_scaling": {"rope_type": "llama3", "factor": 4.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 256},
+    "tie_word_embeddings": False, "max_position_embeddings": 1024, "hidden_act": "silu",
+}
+PAGE_SIZES = {"A": 16, "B": 8, "C": 16, "D": 16}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 
 
 def to_float64(tensors):
