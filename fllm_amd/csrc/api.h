@@ -86,12 +86,14 @@ int fllm_rope_kv_store(void *qkv, const int32_t *row_pos, const int32_t *row_seg
 // [max(0, pos - window + 1), pos] (window <= 0: from 0).  q: rows of `q_stride` elements, head h at
 // h * head_dim.  out: [rows, heads * head_dim].  Rows of a segment are consecutive in the batch, at
 // consecutive positions; seg_start[s] is the first row of segment s (seg_start[num_segs] = rows).
-// `max_context` bounds pos + 1; `uniform_rows` says that every segment has one row (a decode
-// step).  `workspace` holds partial results of split contexts (fllm_attention_workspace_bytes()).
+// `max_context` bounds pos + 1.  The segments from `single_from` on have one row each (0: every segment, a decode
+// step; num_segs: none is known to): rows of long contexts among them are split over workgroups, which portions
+// of prompts are not.  `workspace` holds partial results of split contexts (fllm_attention_workspace_bytes() of
+// the number of single rows).
 int fllm_attention(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables,
                    int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
                    int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int page_size,
-                   int num_pages, float scale, int window, int dtype, int max_context, int uniform_rows,
+                   int num_pages, float scale, int window, int dtype, int max_context, int single_from,
                    void *workspace, size_t workspace_bytes, hipStream_t stream);
 size_t fllm_attention_workspace_bytes(int rows, int heads, int kv_heads, int head_dim, int max_context);
 

@@ -8,7 +8,7 @@
 int fllm_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables,
                              int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
                              int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int page_size,
-                             int num_pages, float scale, int window, int max_context, int uniform_rows, void *workspace,
+                             int num_pages, float scale, int window, int max_context, int single_from, void *workspace,
                              size_t workspace_bytes, hipStream_t stream);   // attention_mfma.hip; 1: shape declined
 size_t fllm_attention_bf16_workspace_bytes(int rows, int heads, int kv_heads, int head_dim, int max_context);
 
@@ -95,18 +95,19 @@ extern "C" int fllm_attention(const void *q, int q_stride, const void *k_pages, 
                               const int32_t *tables, int table_stride, const int32_t *row_pos, const int32_t *row_seg,
                               const int32_t *seg_start, int num_segs, void *out, int rows, int heads, int kv_heads,
                               int head_dim, int page_size, int num_pages, float scale, int window, int dtype,
-                              int max_context, int uniform_rows, void *workspace, size_t workspace_bytes,
+                              int max_context, int single_from, void *workspace, size_t workspace_bytes,
                               hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && heads > 0 && kv_heads > 0 && head_dim > 0 && page_size > 0 && table_stride > 0 && num_pages > 0,
                  "attention: bad sizes");
     FLLM_REQUIRE(heads % kv_heads == 0, "attention: %d heads are not a multiple of %d key/value heads", heads, kv_heads);
     FLLM_REQUIRE(num_segs > 0 && seg_start != nullptr, "attention: segment starts are required");
+    FLLM_REQUIRE(single_from >= 0 && single_from <= num_segs, "attention: single_from %d is outside 0..%d", single_from, num_segs);
     FLLM_REQUIRE(q_stride >= heads * head_dim, "attention: q_stride %d is shorter than heads*head_dim", q_stride);
     if (rows == 0) return 0;
     if (dtype == FLLM_BF16) {
         const int fast = fllm_attention_bf16_fast(q, q_stride, k_pages, v_pages, tables, table_stride, row_pos, row_seg,
                                                   seg_start, num_segs, out, rows, heads, kv_heads, head_dim, page_size,
-                                                  num_pages, scale, window, max_context, uniform_rows, workspace,
+                                                  num_pages, scale, window, max_context, single_from, workspace,
                                                   workspace_bytes, stream);
         if (fast <= 0) return fast;
     }

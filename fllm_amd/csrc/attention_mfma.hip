@@ -921,13 +921,15 @@ size_t fllm_attention_bf16_workspace_bytes(int rows, int heads, int kv_heads, in
 int fllm_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables,
                              int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
                              int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int page_size,
-                             int num_pages, float scale, int window, int max_context, int uniform_rows, void *workspace,
+                             int num_pages, float scale, int window, int max_context, int single_from, void *workspace,
                              size_t workspace_bytes, hipStream_t stream) {
     if (!fllm_fast_kernels_enabled()) return 1;
     (void)num_pages;
     if (!fast_shape(heads, kv_heads, head_dim, page_size)) return 1;
     if (q_stride % 8 != 0 || ((uintptr_t)q & 15) != 0) return 1;
-    if (uniform_rows && rows != num_segs) return 1;
+    const int singles = num_segs - single_from;       // segments of one row each, at the end of the batch
+    if (single_from == 0 && rows != num_segs) return 1;
+    if (singles > rows) return 1;
     AttnArgs a;
     a.q = (const bf16_t *)q;
     a.q_stride = q_stride;
@@ -954,7 +956,27 @@ int fllm_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, c
     a.counters = nullptr;
     a.part_tiles = 0;
     a.parts_ws = nullptr;
-    if (head_dim == 32) return launch<32>(a, uniform_rows, max_context, workspace, workspace_bytes, stream);
-    if (head_dim == 64) return launch<64>(a, uniform_rows, max_context, workspace, workspace_bytes, stream);
-    return launch<128>(a, uniform_rows, max_context, workspace, workspace_bytes, stream);
+    auto run = [&](const AttnArgs &part, int uniform) {
+        if (head_dim == 32) return launch<32>(part, uniform, max_context, workspace, workspace_bytes, stream);
+        if (head_dim == 64) return launch<64>(part, uniform, max_context, workspace, workspace_bytes, stream);
+        return launch<128>(part, uniform, max_context, workspace, workspace_bytes, stream);
+    };
+    if (single_from == 0 || singles == 0) return run(a, single_from == 0);
+    // Portions of prompts beside single tokens: the portions go to the tile kernel, the single rows behind them to
+    // the decode kernel, which splits long contexts over workgroups (one row of a long context is a poor tile).
+    const int first = rows - singles;
+    AttnArgs portions = a;
+    portions.rows = first;
+    portions.num_segs = single_from;
+    const int rc = run(portions, 0);
+    if (rc != 0) return rc;
+    AttnArgs single = a;
+    single.q = a.q + (size_t)first * q_stride;
+    single.row_pos = row_pos + first;
+    single.row_seg = row_seg + first;
+    single.seg_start = seg_start + single_from;
+    single.num_segs = singles;
+    single.out = a.out + (size_t)first * heads * head_dim;
+    single.rows = singles;
+    return run(single, 1);
 }

@@ -41,6 +41,8 @@ class StepContext:
     seg_slots: List[int] = field(default_factory=list)
     max_context: int = 0                    # largest position + 1 in the step
     uniform_rows: bool = False              # every segment has exactly one row
+    single_from: Optional[int] = None       # the segments from this one on have one row each (None: unknown)
+    single_max_context: int = 0             # largest position + 1 among those single rows
     _scratch: Dict = field(default_factory=dict)
 
     def no_rotation(self, rt):
@@ -52,9 +54,17 @@ class StepContext:
         cos, sin = rt.shared[key]
         return cos, sin, 0, 0
 
+    def single_rows_from(self) -> int:
+        """Index of the first segment from which every segment has one row."""
+        if self.uniform_rows:
+            return 0
+        return self.num_segments if self.single_from is None else self.single_from
+
     def attention_workspace(self, rt, rows: int, heads: int, kv_heads: int, head_dim: int) -> Optional[torch.Tensor]:
-        """Scratch for partial results of split contexts, one buffer per step shape."""
-        need = rt.ops.attention_workspace_bytes(rows, heads, kv_heads, head_dim, self.max_context)
+        """Scratch for partial results of split contexts, one buffer per step shape: sized for the single rows of the
+        step, which are the ones whose contexts are split."""
+        singles = self.num_segments - self.single_rows_from()
+        need = max(rt.ops.attention_workspace_bytes(n, heads, kv_heads, head_dim, self.max_context) for n in {rows, singles} if n > 0)
         if need == 0:
             return None
         buf = self._scratch.get("attention")

@@ -263,10 +263,15 @@ class ModelRunner:
         seg_rows, seg_start = [], []
         carry: Dict[int, int] = {}              # row -> row of the earlier step's tokens
         max_context = 0
-        for s, e in enumerate(entries):
+        # Segments of several rows first, single rows behind them (attention treats the two kinds differently); the
+        # logits keep the order of the caller's entries.
+        order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens) == 1)
+        base_of = {}
+        for s, i in enumerate(order):
+            e = entries[i]
             start = self.cache.length(e.req_id)
             n = len(e.tokens)
-            base = len(ids)
+            base = base_of[i] = len(ids)
             if e.carry is not None:
                 carry[base] = int(e.carry)
                 ids.append(0)
@@ -275,10 +280,14 @@ class ModelRunner:
             row_pos.extend(range(start, start + n))
             row_seg.extend([s] * n)
             slots.append(self.cache.slot(e.req_id))
-            logit_rows.extend(base + int(w) for w in e.want)
             seg_rows.append(n)
             seg_start.append(start)
             max_context = max(max_context, start + n)
+        for i, e in enumerate(entries):
+            logit_rows.extend(base_of[i] + int(w) for w in e.want)
+        single_from = sum(1 for n in seg_rows if n != 1)
+        single_max_context = max((start + 1 for start, n in zip(seg_start, seg_rows) if n == 1), default=0)
+        entries = [entries[i] for i in order]       # the tables below follow the segments
         S = len(entries)
         widths = []
         flat_tables: List[int] = []
@@ -314,7 +323,8 @@ class ModelRunner:
         return StepContext(num_rows=R, num_segments=S, ids=t_ids, row_pos=t_pos, row_seg=t_seg, seg_start=t_cu,
                            slots=t_slots,
                            logit_rows=t_rows, tables=tables, seg_rows=seg_rows, seg_pos_start=seg_start,
-                           seg_slots=slots, max_context=max_context, uniform_rows=all(n == 1 for n in seg_rows))
+                           seg_slots=slots, max_context=max_context, uniform_rows=all(n == 1 for n in seg_rows),
+                           single_from=single_from, single_max_context=single_max_context)
 
 
 class _DecodeGraph:

@@ -349,10 +349,10 @@ class Ops:
     def attention(self, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, tables: torch.Tensor,
                   row_pos: torch.Tensor, row_seg: torch.Tensor, seg_start: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int,
                   head_dim: int, page_size: int, scale: float, window: Optional[int], max_context: int,
-                  uniform_rows: int = 0, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  uniform_rows: int = 0, workspace: Optional[torch.Tensor] = None, single_from: Optional[int] = None) -> torch.Tensor:
         """`q` may be a column slice of a wider row-major matrix (the fused qkv buffer).
-        `max_context` bounds pos + 1 over the rows; `uniform_rows` is 1 when every segment has one
-        row (a decode step)."""
+        `max_context` bounds pos + 1 over the rows; the segments from `single_from` on have one row each
+        (`uniform_rows` = 1 is `single_from` = 0: a decode step; by default no segment is known to)."""
         rows = q.shape[0]
         _need(q.is_cuda and q.dim() == 2 and q.stride(1) == 1 and q.shape[1] == heads * head_dim,
               f"q must be [rows, {heads * head_dim}] with unit column stride")
@@ -373,10 +373,14 @@ class Ops:
             _need(workspace.is_cuda and workspace.is_contiguous(), "workspace must be a dense GPU tensor")
             ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
         q_stride = q.stride(0) if rows > 1 else heads * head_dim
+        num_segs = seg_start.numel() - 1
+        if single_from is None:
+            single_from = 0 if uniform_rows else num_segs
+        _need(0 <= single_from <= num_segs and num_segs - single_from <= rows, f"single_from {single_from} does not fit {num_segs} segments of {rows} rows")
         self._check(self.lib.fllm_attention(
             _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(tables), tables.shape[1], _ptr(row_pos), _ptr(row_seg),
             _ptr(seg_start), seg_start.numel() - 1, _ptr(out), rows, heads, kv_heads, head_dim, page_size, num_pages, float(scale),
-            int(window) if window else 0, _DTYPE_CODE[q.dtype], int(max_context), int(uniform_rows), ws_ptr, ws_bytes,
+            int(window) if window else 0, _DTYPE_CODE[q.dtype], int(max_context), int(single_from), ws_ptr, ws_bytes,
             self._stream()))
         return out
 

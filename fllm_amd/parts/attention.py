@@ -137,15 +137,22 @@ class PagedAttention(Mixer):
         self.forward(ctx, h, None, binding, branch=branch)
         return branch
 
+    SPLIT_SINGLE_ROWS_FROM = 3072      # context length (measured: equal cost at about 4,000 keys)
+
     def _attend_and_project(self, ctx, q, residual, binding, branch=None):
         rt, ops = self.rt, self.rt.ops
         rows = q.shape[0]
         nh, nkv, d = self.heads, self.kv_heads, self.head_dim
         tables = ctx.tables[binding.group]
         out = rt.empty((rows, nh * d))
+        # Single rows behind portions of prompts: with long contexts they go to the kernel that splits a context over
+        # workgroups (a second launch); with short ones they ride along in the portions' launch, which is faster then.
+        single_from = ctx.single_rows_from()
+        if 0 < single_from < ctx.num_segments and ctx.single_max_context < self.SPLIT_SINGLE_ROWS_FROM:
+            single_from = ctx.num_segments
         ops.attention(q, binding.k_pages, binding.v_pages, tables, ctx.row_pos, ctx.row_seg, ctx.seg_start,
                       out, nh, nkv, d, binding.page_size, self.scale, self.window, ctx.max_context,
-                      uniform_rows=1 if ctx.uniform_rows else 0,
+                      single_from=single_from,
                       workspace=ctx.attention_workspace(rt, rows, nh, nkv, d))
         if branch is not None:
             ops.linear(out, self.w_o, branch, bias=self.b_o)

@@ -127,7 +127,7 @@ class ReferenceOps:
         return 0
 
     def attention(self, q, k_pages, v_pages, tables, row_pos, row_seg, seg_start, out, heads, kv_heads, head_dim, page_size, scale,
-                  window, max_context, uniform_rows=0, workspace=None):
+                  window, max_context, uniform_rows=0, workspace=None, single_from=None):
         rows = q.shape[0]
         group = heads // kv_heads
         for r in range(rows):

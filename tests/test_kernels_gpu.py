@@ -409,7 +409,7 @@ def _rope_case(ops, ref, dtype, heads, kv_heads, head_dim, rope_dims, pairing, p
 
 # ---------------------------------------------------------------------------------------------
 def attention_case(ops, ref, dtype, heads, kv_heads, head_dim, page_size, segs, window, seed, fast=True, spike=False,
-                   bound=None, calls=1):
+                   bound=None, calls=1, mark_single_rows=True):
     """segs: (first position, rows) per segment.  bound: the context bound handed to the kernel (a decode graph's
     is larger than any context of the step); calls: launches in a row, which must give the same bits."""
     g = gen(seed)
@@ -442,17 +442,22 @@ def attention_case(ops, ref, dtype, heads, kv_heads, head_dim, page_size, segs, 
     want = ref.attention(q, k, v, tables, row_pos, row_seg, seg_start, torch.empty(rows, heads * head_dim, dtype=torch.float64),
                          heads, kv_heads, head_dim, page_size, scale, window, max_context)
     uniform = int(all(n == 1 for _, n in segs))
+    single_from = len(segs)
+    while single_from > 0 and segs[single_from - 1][1] == 1:
+        single_from -= 1
+    if not mark_single_rows:
+        single_from = 0 if uniform else len(segs)
     ops.set_fast_kernels(fast)
     try:
         bound = max_context if bound is None else bound
-        nbytes = ops.attention_workspace_bytes(rows, heads, kv_heads, head_dim, bound)
+        nbytes = max(ops.attention_workspace_bytes(n, heads, kv_heads, head_dim, bound) for n in {rows, len(segs) - single_from} if n > 0)
         ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=DEV)
         args = (qkv.to(DEV)[:, : heads * head_dim], k.to(DEV), v.to(DEV), tables.to(DEV), row_pos.to(DEV), row_seg.to(DEV),
                 seg_start.to(DEV))
         got = None
         for _ in range(calls):
             out = ops.attention(*args, torch.empty(rows, heads * head_dim, dtype=dtype, device=DEV),
-                                heads, kv_heads, head_dim, page_size, scale, window, bound, uniform_rows=uniform, workspace=ws)
+                                heads, kv_heads, head_dim, page_size, scale, window, bound, single_from=single_from, workspace=ws)
             assert got is None or torch.equal(out, got), "two launches of the same attention differ"
             got = out
     finally:
@@ -559,6 +564,19 @@ def test_attention_prompt_portions_share_long_row_tiles(ops, ref, prefill_parts,
     from fllm_amd.kernels import Ops
     counters = Ops._workspaces[torch.cuda.current_device()][: 64 * 1024]
     assert int(counters.to(torch.int64).sum()) == 0
+
+
+@pytest.mark.parametrize("mark_single_rows", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv_heads,head_dim", [(32, 8, 128), (8, 2, 64), (5, 1, 32), (6, 3, 48)])
+@pytest.mark.parametrize("segs,window", [([(0, 300), (5000, 1), (37, 1), (999, 1)], None), ([(100, 17), (0, 33), (640, 1)], None),
+                                         ([(3, 70), (700, 2), (2000, 1), (15, 1), (0, 1)], None), ([(250, 50), (900, 1), (30, 1)], 100)])
+def test_attention_portions_beside_single_rows(ops, ref, mark_single_rows, dtype, heads, kv_heads, head_dim, segs, window):
+    """Portions of prompts with single rows behind them, as a step of the engine lays them out: the single rows go
+    to the kernel that splits long contexts when the caller says where they begin, and to the tile kernel with the
+    portions when it does not; either way every row is right."""
+    attention_case(ops, ref, dtype, heads, kv_heads, head_dim, 16, segs, window, 24, spike=True, calls=2,
+                   mark_single_rows=mark_single_rows)
 
 
 def test_attention_row_is_the_same_alone_and_in_a_batch(ops, ref):

@@ -82,6 +82,21 @@ def test_replay(models, tmp_path, name, dtype, family):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_single_rows_beside_portions_take_the_decode_kernel(models, tmp_path, monkeypatch, name, dtype):
+    """In a step that mixes portions of prompts with single tokens the single rows go to the decode kernel once their
+    contexts are long; here from the first key on, so that the tiny models take that way."""
+    from fllm_amd.parts.attention import PagedAttention
+    monkeypatch.setattr(PagedAttention, "SPLIT_SINGLE_ROWS_FROM", 0)
+    folder, cfg, requests, plain = models[name]
+    steps = tt.number(tt.mixed(requests, seed=13, decode_tail=40))
+    runner = make_runner(folder, dtype, tc.PAGE_SIZES[name], tt.live_tokens_bound(steps))
+    got = tt.run_in_process(runner, steps, cfg["vocab_size"], str(tmp_path))
+    check(got, plain, dtype, f"{name} {dtype} mixed, single rows apart")
+    runner.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(models, tmp_path, dtype):
     """bin/trace_run as a user starts it: steps on stdin, `done` lines back, files in --out."""
     folder, cfg, requests, plain = models["A"]
