@@ -1,0 +1,64 @@
+"""Sizes that fit no fast kernel, through the whole engine: heads of 80 and of 256, a width and an intermediate
+size that are no multiple of 8, an odd vocabulary, seven heads with a key/value head each, twelve heads on one
+key/value head.  Every request whole and mixed with others, in both precisions, against the plain implementation:
+a size is served by a slower kernel or refused, never answered wrongly."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama
+import tiny_configs as tc
+import trace_tools as tt
+
+pytestmark = pytest.mark.gpu
+
+BASE = {"model_type": "llama", "rope_theta": 10000.0, "rms_norm_eps": 1e-5, "hidden_act": "silu"}
+ODD = {
+    "head80": dict(BASE, num_hidden_layers=2, hidden_size=104, num_attention_heads=3, num_key_value_heads=1, head_dim=80,
+                   intermediate_size=250, vocab_size=1001, tie_word_embeddings=False, max_position_embeddings=300),
+    "width100": dict(BASE, num_hidden_layers=2, hidden_size=100, num_attention_heads=7, num_key_value_heads=7, head_dim=16,
+                     intermediate_size=36, vocab_size=77, tie_word_embeddings=True, max_position_embeddings=200),
+    "head256": dict(BASE, num_hidden_layers=1, hidden_size=256, num_attention_heads=2, num_key_value_heads=1, head_dim=256,
+                    intermediate_size=264, vocab_size=513, tie_word_embeddings=False, max_position_embeddings=300),
+    "group12": dict(BASE, num_hidden_layers=1, hidden_size=192, num_attention_heads=12, num_key_value_heads=1, head_dim=64,
+                    intermediate_size=512, vocab_size=300, tie_word_embeddings=False, max_position_embeddings=700),
+}
+TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+
+
+@pytest.fixture(scope="module")
+def odd_models(tmp_path_factory):
+    from safetensors.torch import save_file
+    from fllm_amd.registry import model_spec_from_config
+    from fllm_amd.weights import random_tensors
+    out = {}
+    for name, cfg in ODD.items():
+        _, spec = model_spec_from_config(cfg)
+        tensors = {k: v.to(torch.float32) for k, v in random_tensors(spec, seed=3, dtype=torch.bfloat16).items()}
+        folder = str(tmp_path_factory.mktemp(f"odd_{name}"))
+        with open(os.path.join(folder, "config.json"), "w") as fh:
+            json.dump(cfg, fh)
+        save_file(tensors, os.path.join(folder, "model.safetensors"))
+        longest = cfg["max_position_embeddings"]
+        requests = {f"r{i}": tc.random_ids(n, cfg["vocab_size"], 7 + i) for i, n in enumerate([5, 33, longest, 70, longest // 2])}
+        w64 = tc.to_float64(tensors)
+        out[name] = (folder, cfg, requests, {rid: plain_llama.forward(cfg, w64, toks) for rid, toks in requests.items()})
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("family", ["whole", "mixed"])
+@pytest.mark.parametrize("name", list(ODD))
+def test_odd_sizes(odd_models, tmp_path, name, family, dtype):
+    from fllm_amd.engine import ModelRunner
+    folder, cfg, requests, plain = odd_models[name]
+    steps = tt.number(tt.whole(requests) if family == "whole" else tt.mixed(requests, seed=5))
+    runner = ModelRunner.from_folder(folder, dtype=dtype, page_size=16, max_tokens=tt.live_tokens_bound(steps), max_requests=8)
+    got = tt.run_in_process(runner, steps, cfg["vocab_size"], str(tmp_path))
+    for rid, want in plain.items():
+        err = np.abs(got[rid].astype(np.float64) - want).max()
+        assert err <= TOL[dtype] * np.abs(want).max(), f"{name} {dtype} {family}: request {rid}: error {err:.3e}"
+    runner.cache.check_invariants()
