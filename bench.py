@@ -2,13 +2,14 @@
 """Decode and prefill throughput of the engine on one MI355X, Llama-3.1-8B sizes, random bfloat16
 weights, synthetic token ids.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers N]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers N] [--shape 8b|1b|70b]
 
 A step is one decode step of the whole engine (scheduler, step function, sampling), with steps
 launched ahead of the tokens of the step before them (--no-ahead: each step waits for the last).  The one
 JSON line on standard output holds decoded tokens per second at the default batch (8), the same
 at batch 1 and 64 under "points", a 2,048-token prefill under "prefill" and the decode step's
-share of the HBM roofline under "roofline".
+share of the HBM roofline under "roofline": of the published peaks (8 TB/s, 2.5 PFLOP/s), and under "measured_peak" /
+"frac_measured" of what a kernel that only reads, or only issues MFMA products, gets out of this device.
 """
 import argparse
 import json
@@ -26,6 +27,16 @@ LLAMA_31_8B = {
                      "original_max_position_embeddings": 8192},
     "tie_word_embeddings": False, "max_position_embeddings": 131072, "hidden_act": "silu",
 }
+SHAPES = {
+    "8b": LLAMA_31_8B,
+    "1b": dict(LLAMA_31_8B, num_hidden_layers=16, hidden_size=2048, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
+               intermediate_size=8192, tie_word_embeddings=True,
+               rope_scaling={"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                             "original_max_position_embeddings": 8192}),
+    "70b": dict(LLAMA_31_8B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64, num_key_value_heads=8, head_dim=128,
+                intermediate_size=28672),
+}
+SHAPE_NAMES = {"8b": "Llama-3.1-8B shape", "1b": "Llama-3.2-1B shape", "70b": "Llama-3.1-70B shape"}
 CONTEXT = 8192
 PROMPT_LEN = 1024
 PREFILL_TOKENS = 2048
@@ -59,8 +70,12 @@ def main():
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=LLAMA_31_8B["num_hidden_layers"],
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="8b",
+                    help="layer sizes: Llama-3.1-8B (the default, the headline configuration), Llama-3.2-1B or Llama-3.1-70B")
+    ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the model has (both numbers are reported)")
+    ap.add_argument("--no-ceilings", action="store_true",
+                    help="do not measure what the device delivers to a kernel that only reads or only multiplies")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     ap.add_argument("--no-ahead", action="store_true", help="every step waits for the tokens of the step before it")
     ap.add_argument("--prefill-only", action="store_true",
@@ -76,7 +91,10 @@ def main():
     import torch
     from fllm_amd import Engine, SamplingParams
 
-    cfg = dict(LLAMA_31_8B, num_hidden_layers=args.layers)
+    shape = SHAPES[args.shape]
+    if args.layers is None:
+        args.layers = shape["num_hidden_layers"]
+    cfg = dict(shape, num_hidden_layers=args.layers)
     steps, warmup = args.steps, args.warmup
     batches = [args.batch] if args.no_points or args.prefill_only else sorted({1, args.batch, 64})
     slack = max(batches) + 8          # requests whose prompt is done early decode while the others still prefill
@@ -151,11 +169,11 @@ def main():
     step_bytes = decode_step_bytes(cfg, args.layers, contexts)
     achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
     line = {
-        "metric": "decode tok/s at batch 8 (Llama-3.1-8B shape, 1,024-token prompts); points: batch 1/64; prefill: 2,048 tokens",
+        "metric": f"decode tok/s at batch {args.batch} ({SHAPE_NAMES[args.shape]}, 1,024-token prompts); points: batch 1/64; prefill: 2,048 tokens",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic token ids, random-init weights N(0, 0.02)",
-        "config": {"model": "Llama-3.1-8B shape", "layers": args.layers, "layers_of_model": LLAMA_31_8B["num_hidden_layers"],
+        "config": {"model": SHAPE_NAMES[args.shape], "layers": args.layers, "layers_of_model": shape["num_hidden_layers"],
                    "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
                    "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": vocab,
                    "global_batch": args.batch, "prompt_len": PROMPT_LEN, "seq_len": CONTEXT, "kv_block": PAGE_SIZE,
@@ -173,6 +191,16 @@ def main():
         line["prefill"] = {"value": round(PREFILL_TOKENS / best, 1), "tokens": PREFILL_TOKENS, "ms": round(best * 1e3, 3),
                            "frac": round(flops / best / (MFMA_PEAK_TFLOPS["bf16"] * 1e12), 4)}
         print(f"[bench] prefill {PREFILL_TOKENS} tokens: {best * 1e3:.2f} ms", file=sys.stderr, flush=True)
+    if not args.no_ceilings:
+        # beside the published peaks: what a kernel that only reads, or only multiplies, gets out of this device
+        measured = engine.runner.rt.ops.measured_ceilings()
+        line["roofline"]["measured_peak"] = round(measured["hbm_read_gbs"], 1)
+        line["roofline"]["frac_measured"] = round(achieved / measured["hbm_read_gbs"], 4)
+        if "prefill" in line:
+            line["prefill"]["measured_peak_tflops"] = round(measured["mfma_bf16_tflops"], 1)
+            line["prefill"]["frac_measured"] = round(flops / best / (measured["mfma_bf16_tflops"] * 1e12), 4)
+        print(f"[bench] measured ceilings: {measured['hbm_read_gbs']:.0f} GB/s read, {measured['mfma_bf16_tflops']:.0f} TFLOP/s bf16 MFMA",
+              file=sys.stderr, flush=True)
     print(json.dumps(line), flush=True)
 
 

@@ -102,6 +102,12 @@ size_t fllm_attention_workspace_bytes(int rows, int heads, int kv_heads, int hea
 int fllm_carry_ids(int32_t *ids, const int32_t *source, const int32_t *previous, int rows, int previous_rows,
                    hipStream_t stream);
 
+// Probes for measurements: a kernel that only reads `bytes` from `src` (`sink`: 4 bytes a workgroup, left alone),
+// and one that only multiplies (32x32x16 bfloat16 MFMA, `blocks` workgroups of 8 waves; `sink`: 2 KiB a workgroup;
+// returns the floating-point operations of the launch, negative on error).  The caller times them.
+int fllm_probe_read(const void *src, size_t bytes, void *sink, int blocks, hipStream_t stream);
+double fllm_probe_mfma_bf16(void *sink, int blocks, int iters, hipStream_t stream);
+
 // out[r] = first index of the largest finite value of logits[r, :]
 int fllm_argmax(const float *logits, int32_t *out, int rows, int vocab, hipStream_t stream);
 

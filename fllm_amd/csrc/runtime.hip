@@ -94,5 +94,75 @@ extern "C" int fllm_set_device_workspace(void *workspace, size_t bytes) {
     return 0;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Probes of what the device delivers, for measurements that state a share of a measured ceiling beside the share
+// of the published one.
+// ---------------------------------------------------------------------------------------------
+namespace {
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
+
+// every workgroup reads a contiguous stretch with 16-byte loads, eight of them in flight a lane
+__global__ void __launch_bounds__(256) probe_read_kernel(const u32x4_t *__restrict__ src, size_t chunks, unsigned int *sink) {
+    const size_t per_block = (chunks + gridDim.x - 1) / gridDim.x;
+    const size_t begin = (size_t)blockIdx.x * per_block, end = begin + per_block < chunks ? begin + per_block : chunks;
+    u32x4_t acc = {0u, 0u, 0u, 0u};
+    size_t i = begin + threadIdx.x;
+    for (; i + 7 * 256 < end; i += 8 * 256) {
+        u32x4_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = __builtin_nontemporal_load(src + i + u * 256);
+#pragma unroll
+        for (int u = 0; u < 8; u++) acc ^= v[u];
+    }
+    for (; i < end; i += 256) acc ^= src[i];
+    const unsigned int x = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+    if (x == 0x9e3779b9u) sink[blockIdx.x] = x;     // keeps the loads alive; written next to never
+}
+
+// four independent chains of 32x32x16 bfloat16 products a wave, two waves a SIMD
+__global__ void __launch_bounds__(512) probe_mfma_kernel(float *sink, int iters) {
+    bf16x8_t a, b;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        a[i] = (bf16_t)(0.001f * (float)((threadIdx.x + i) & 15));
+        b[i] = (bf16_t)(0.002f * (float)((threadIdx.x * 3 + i) & 7));
+    }
+    f32x16_t acc[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[c][i] = 0.f;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[c], 0, 0, 0);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) s += acc[c][i];
+    if (s == 12345.678f) sink[blockIdx.x * 512 + threadIdx.x] = s;
+}
+}  // namespace
+
+extern "C" int fllm_probe_read(const void *src, size_t bytes, void *sink, int blocks, hipStream_t stream) {
+    FLLM_REQUIRE(src != nullptr && sink != nullptr && bytes >= 16 && ((uintptr_t)src & 15) == 0, "probe_read: a 16-byte aligned buffer is required");
+    FLLM_REQUIRE(blocks > 0 && blocks <= 65535 * 16, "probe_read: bad number of workgroups %d", blocks);
+    hipLaunchKernelGGL(probe_read_kernel, dim3(blocks), dim3(256), 0, stream, (const u32x4_t *)src, bytes / 16, (unsigned int *)sink);
+    return fllm_check_launch("probe_read");
+}
+
+extern "C" double fllm_probe_mfma_bf16(void *sink, int blocks, int iters, hipStream_t stream) {
+    if (sink == nullptr || blocks <= 0 || iters <= 0) {
+        fllm_set_error("probe_mfma: bad arguments");
+        return -1.0;
+    }
+    hipLaunchKernelGGL(probe_mfma_kernel, dim3(blocks), dim3(512), 0, stream, (float *)sink, iters);
+    if (fllm_check_launch("probe_mfma") != 0) return -1.0;
+    return 2.0 * 32 * 32 * 16 * 16.0 * iters * 8.0 * blocks;      // floating-point operations of the launch
+}
+
 extern "C" const char *fllm_last_error(void) { return g_error; }
 extern "C" int fllm_abi_version(void) { return 1; }

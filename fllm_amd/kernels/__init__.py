@@ -80,6 +80,10 @@ def load_library(build_if_missing: bool = True):
     lib.fllm_set_option.restype = c_int
     lib.fllm_set_device_workspace.argtypes = [c_void, c_size]
     lib.fllm_set_device_workspace.restype = c_int
+    lib.fllm_probe_read.argtypes = [c_void, c_size, c_void, c_int, c_void]
+    lib.fllm_probe_read.restype = c_int
+    lib.fllm_probe_mfma_bf16.argtypes = [c_void, c_int, c_int, c_void]
+    lib.fllm_probe_mfma_bf16.restype = ctypes.c_double
     lib.fllm_set_fast_kernels.argtypes = [c_int]
     lib.fllm_set_fast_kernels.restype = None
     lib.fllm_attention_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int, c_int]
@@ -383,6 +387,32 @@ class Ops:
             int(window) if window else 0, _DTYPE_CODE[q.dtype], int(max_context), int(single_from), ws_ptr, ws_bytes,
             self._stream()))
         return out
+
+    def measured_ceilings(self, read_bytes: int = 4 << 30, repeats: int = 5) -> dict:
+        """What the device delivers to kernels that do nothing else: GB/s of a kernel that only reads a buffer much larger
+        than the caches, TFLOP/s of a kernel that only issues bfloat16 MFMA products.  The best of `repeats` timings."""
+        dev = torch.device("cuda", torch.cuda.current_device())
+        props = torch.cuda.get_device_properties(dev)
+        blocks = props.multi_processor_count * 8
+        buf = torch.zeros(read_bytes, dtype=torch.uint8, device=dev)
+        sink = torch.zeros(max(blocks, 2 * props.multi_processor_count * 512), dtype=torch.float32, device=dev)
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        best_read, best_mfma = 0.0, 0.0
+        iters, mfma_blocks = 4096, 2 * props.multi_processor_count
+        for _ in range(repeats + 1):
+            start.record()
+            self._check(self.lib.fllm_probe_read(_ptr(buf), buf.numel(), _ptr(sink), blocks, self._stream()))
+            end.record()
+            end.synchronize()
+            best_read = max(best_read, buf.numel() / (start.elapsed_time(end) * 1e-3) / 1e9)
+            start.record()
+            flops = self.lib.fllm_probe_mfma_bf16(_ptr(sink), mfma_blocks, iters, self._stream())
+            end.record()
+            end.synchronize()
+            if flops < 0:
+                raise KernelError(self.lib.fllm_last_error().decode("utf-8", "replace"))
+            best_mfma = max(best_mfma, flops / (start.elapsed_time(end) * 1e-3) / 1e12)
+        return {"hbm_read_gbs": best_read, "mfma_bf16_tflops": best_mfma}
 
     def carry_ids(self, ids: torch.Tensor, source: torch.Tensor, previous: torch.Tensor) -> torch.Tensor:
         """ids[r] = previous[source[r]] where source[r] >= 0 (int32 device tensors): tokens an earlier step chose
