@@ -64,6 +64,38 @@ def prefill_flops(cfg, layers, tokens):
     return 2 * tokens * body + 2 * head + attention          # the head runs on the one wanted row
 
 
+def mixed_run(cfg, args):
+    """Continuous batching under load: 64 requests at once, prompts of 64 to 2,048 tokens, 128 generated tokens each."""
+    import numpy as np
+    import torch
+    from fllm_amd import Engine, SamplingParams
+    rng = np.random.default_rng(1)
+    lengths = rng.integers(64, 2049, 64).tolist()
+    generate = 128
+    need_tokens = sum(n + generate + PAGE_SIZE for n in lengths) + 64
+    engine = Engine(config=cfg, seed=0, dtype="bfloat16", device="cuda:0", ctx=4096, max_seqs=64, max_batched_tokens=PREFILL_TOKENS,
+                    block_size=PAGE_SIZE, num_blocks=-(-need_tokens // PAGE_SIZE), decode_first=True, random_weights_on_device=True,
+                    ahead=not args.no_ahead)
+    vocab = cfg["vocab_size"]
+    results = []
+    for run in range(2):            # the first run captures the graphs
+        for i, n in enumerate(lengths):
+            engine.add_request(f"m{run}-{i}", rng.integers(0, vocab, n).tolist(), SamplingParams(max_tokens=generate, ignore_eos=True))
+        torch.cuda.synchronize()
+        start, tokens, rounds = time.perf_counter(), 0, 0
+        while engine.has_unfinished():
+            tokens += len(engine.step())
+            rounds += 1
+        torch.cuda.synchronize()
+        results.append((time.perf_counter() - start, tokens, rounds))
+    elapsed, tokens, rounds = results[-1]
+    assert tokens == 64 * generate
+    print(json.dumps({"workload": "64 requests at once, prompts of 64..2,048 tokens, 128 generated tokens each", "model": SHAPE_NAMES[args.shape],
+                      "seconds": round(elapsed, 3), "steps": rounds, "prompt_tokens": int(sum(lengths)),
+                      "generated_tokens": tokens, "generated_tokens_per_s": round(tokens / elapsed, 1),
+                      "all_tokens_per_s": round((tokens + sum(lengths)) / elapsed, 1), "preemptions": engine.stats.preemptions}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -74,6 +106,10 @@ def main():
                     help="layer sizes: Llama-3.1-8B (the default, the headline configuration), Llama-3.2-1B or Llama-3.1-70B")
     ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the model has (both numbers are reported)")
+    ap.add_argument("--mixed", action="store_true",
+                    help="instead of the headline run: 64 requests with prompts of 64 to 2,048 tokens and 128 generated tokens each, "
+                         "all submitted at once (continuous batching, prompts in portions beside decoding requests); prints a "
+                         "line of its own")
     ap.add_argument("--no-ceilings", action="store_true",
                     help="do not measure what the device delivers to a kernel that only reads or only multiplies")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
@@ -96,6 +132,8 @@ def main():
         args.layers = shape["num_hidden_layers"]
     cfg = dict(shape, num_hidden_layers=args.layers)
     steps, warmup = args.steps, args.warmup
+    if args.mixed:
+        return mixed_run(cfg, args)
     batches = [args.batch] if args.no_points or args.prefill_only else sorted({1, args.batch, 64})
     slack = max(batches) + 8          # requests whose prompt is done early decode while the others still prefill
     prompt_tokens = args.prompt_tokens if args.prefill_only else PREFILL_TOKENS
