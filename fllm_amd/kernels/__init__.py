@@ -33,6 +33,9 @@ assert SAMPLE_ROW_BYTES == 32
 _lib = None
 
 
+ABI_VERSION = 2
+
+
 def load_library(build_if_missing: bool = True):
     """The loaded library; builds it first when there is none that matches the sources."""
     global _lib
@@ -50,6 +53,9 @@ def load_library(build_if_missing: bool = True):
     c_int, c_void, c_float, c_size = ctypes.c_int, ctypes.c_void_p, ctypes.c_float, ctypes.c_size_t
     lib.fllm_last_error.restype = ctypes.c_char_p
     lib.fllm_abi_version.restype = c_int
+    if lib.fllm_abi_version() != ABI_VERSION:
+        raise KernelError(f"the HIP kernel library {path} has interface version {lib.fllm_abi_version()}, this package needs "
+                          f"{ABI_VERSION}: build it again (python -m fllm_amd.kernels.build)")
     sig = {
         "fllm_embed": [c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_float, c_void],
         "fllm_rmsnorm": [c_void, c_void, c_void, c_void, c_int, c_int, c_float, c_int, c_void],
