@@ -536,9 +536,16 @@ attn_tile32_kernel(AttnArgs p) {
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
         float m_all = -INFINITY;
-        for (int i = 0; i < parts; i++)
-            m_all = fmaxf(m_all, __hip_atomic_load(slot + (size_t)i * kPartFloats(D) + DB * 16 * kThreads + threadIdx.x,
-                                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        for (int i0 = 0; i0 < parts; i0 += 8) {       // eight loads in flight at a time
+            float mp[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                mp[i] = i0 + i < parts ? __hip_atomic_load(slot + (size_t)(i0 + i) * kPartFloats(D) + DB * 16 * kThreads + threadIdx.x,
+                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                       : -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 8; i++) m_all = fmaxf(m_all, mp[i]);
+        }
 #pragma unroll
         for (int db = 0; db < DB; db++)
 #pragma unroll
@@ -732,19 +739,39 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
     if (s_seen != live_splits - 1) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+    // The parts are read eight at a time, all loads of a group asked for before the first is used: two round trips to
+    // memory a group instead of two a part.
+    constexpr int GRP = 8;
     for (int idx = threadIdx.x; idx < gq * D; idx += WAVES * kWave) {
         const int qi = idx / D, d = idx - qi * D;
         const size_t hrow = (size_t)row * p.heads + kvh * G + qtile * 16 + qi;
         const float *ml = p.ws_ml + hrow * p.splits * 2;
+        const float *po = p.ws_o + hrow * p.splits * D + d;
         float m = -INFINITY;
-        for (int sp = 0; sp < live_splits; sp++)
-            m = fmaxf(m, __hip_atomic_load(ml + sp * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        for (int s0 = 0; s0 < live_splits; s0 += GRP) {
+            float ms[GRP];
+#pragma unroll
+            for (int i = 0; i < GRP; i++)
+                ms[i] = s0 + i < live_splits ? __hip_atomic_load(ml + (s0 + i) * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;
+#pragma unroll
+            for (int i = 0; i < GRP; i++) m = fmaxf(m, ms[i]);
+        }
         float l = 0.f, acc = 0.f;
-        for (int sp = 0; sp < live_splits; sp++) {
-            const float ms = __hip_atomic_load(ml + sp * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const float f = ms == -INFINITY ? 0.f : fast_exp2(ms - m);
-            l += __hip_atomic_load(ml + sp * 2 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
-            acc += __hip_atomic_load(p.ws_o + (hrow * p.splits + sp) * D + d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
+        for (int s0 = 0; s0 < live_splits; s0 += GRP) {
+            float ms[GRP], ls[GRP], os[GRP];
+#pragma unroll
+            for (int i = 0; i < GRP; i++) {
+                const bool live = s0 + i < live_splits;
+                ms[i] = live ? __hip_atomic_load(ml + (s0 + i) * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;
+                ls[i] = live ? __hip_atomic_load(ml + (s0 + i) * 2 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+                os[i] = live ? __hip_atomic_load(po + (size_t)(s0 + i) * D, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < GRP; i++) {       // in the order of the parts
+                const float f = ms[i] == -INFINITY ? 0.f : fast_exp2(ms[i] - m);
+                l += ls[i] * f;
+                acc += os[i] * f;
+            }
         }
         p.out[hrow * D + d] = (bf16_t)(l > 0.f ? acc / l : 0.f);
     }

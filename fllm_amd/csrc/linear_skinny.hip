@@ -416,15 +416,30 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
 #pragma unroll
                     for (int t = 0; t < RT; t++) s[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
                     ss = 0.f;
-                    for (int s2 = 0; s2 < S; s2++) {
-                        const float *src = a.ws + ((size_t)(tile * S + s2) * RT * kWave + lane) * 4;
+                    // four slices at a time: their loads are all asked for before the first is added (in slice order)
+                    for (int s0 = 0; s0 < S; s0 += 4) {
+                        float pv[4][RT][4], ps[4];
 #pragma unroll
-                        for (int t = 0; t < RT; t++)
+                        for (int j = 0; j < 4; j++) {
+                            const bool live = s0 + j < S;
+                            const float *src = a.ws + ((size_t)(tile * S + (live ? s0 + j : s0)) * RT * kWave + lane) * 4;
 #pragma unroll
-                            for (int i = 0; i < 4; i++)
-                                s[t][i] += __hip_atomic_load(src + t * kWave * 4 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        if (PRO == PRO_NORM_F32)
-                            ss += __hip_atomic_load(a.ws_ssq + (size_t)(tile * S + s2) * 16 + m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            for (int t = 0; t < RT; t++)
+#pragma unroll
+                                for (int i = 0; i < 4; i++)
+                                    pv[j][t][i] = live ? __hip_atomic_load(src + t * kWave * 4 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+                            ps[j] = (PRO == PRO_NORM_F32 && live)
+                                        ? __hip_atomic_load(a.ws_ssq + (size_t)(tile * S + s0 + j) * 16 + m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                        : 0.f;
+                        }
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+#pragma unroll
+                            for (int t = 0; t < RT; t++)
+#pragma unroll
+                                for (int i = 0; i < 4; i++) s[t][i] += pv[j][t][i];
+                            ss += ps[j];
+                        }
                     }
                 }
                 if (!owner || m >= M || nb >= n_out) break;
