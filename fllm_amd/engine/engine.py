@@ -159,13 +159,19 @@ class Engine:
             entries.append(StepEntry(sid, seq.tokens[start:start + count], [count - 1] if last else []))
             if last:
                 sampled.append(sid)
-            self.stats.prefill_rows += count
         for sid in plan.decode:
             token = seqs[sid].tokens[-1]
             entries.append(StepEntry(sid, [token], [0], carry=row_of[sid] if token == PENDING else None))
             sampled.append(sid)
-            self.stats.decode_rows += 1
-        logits = self.runner.step(entries, previous_tokens=earlier.tokens if earlier is not None else None)
+        try:
+            logits = self.runner.step(entries, previous_tokens=earlier.tokens if earlier is not None else None)
+        except Exception:
+            # nothing was launched: the earlier step stays in flight, so that its tokens still replace their
+            # placeholders (the next call schedules again)
+            self._in_flight = earlier
+            raise
+        self.stats.prefill_rows += sum(count for _, _, count in plan.prefill)
+        self.stats.decode_rows += len(plan.decode)
         rows = sum(len(e.tokens) for e in entries)
         self.stats.forward_calls += 1
         self.stats.rows_total += rows

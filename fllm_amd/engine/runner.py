@@ -232,7 +232,9 @@ class ModelRunner:
         for g, width in enumerate(widths):
             tables = h[o:o + B * width].reshape(B, width)
             for i, e in enumerate(entries):
-                t = self.cache.table(e.req_id, g)
+                # a table may be longer than the graph's rows (pages reserved ahead, for the rest of a prompt or by
+                # the caller): the row at position `start` reads entries up to start / page_size, all below `width`
+                t = self.cache.table(e.req_id, g)[:width]
                 tables[i, :len(t)] = t
             o += B * width
         carried = any(e.carry is not None for e in entries)

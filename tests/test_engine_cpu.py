@@ -205,3 +205,32 @@ def test_ahead_abort_drops_the_row_in_flight():
     assert all(e.request_id == "b" for e in events)
     assert [e.token_id for e in events][-3:] == plain_greedy("A", PROMPTS_A[1], 8)[-3:]
     engine.runner.cache.check_invariants()
+
+
+def test_ahead_step_that_fails_keeps_the_step_before_in_flight():
+    """A step that raises launched nothing: the tokens of the step before still replace their placeholders,
+    and generation goes on as if the failed call had not happened."""
+    want = plain_greedy("A", PROMPTS_A[0], 6)
+    engine = make_engine(ahead=True)
+    engine.add_request("a", PROMPTS_A[0], SamplingParams(max_tokens=6))
+    engine.step()
+    engine.step()
+    real_step, calls = engine.runner.step, []
+
+    def failing_once(entries, previous_tokens=None):
+        if not calls:
+            calls.append(1)
+            raise OutOfPages("forced by the test")
+        return real_step(entries, previous_tokens=previous_tokens)
+
+    engine.runner.step = failing_once
+    with pytest.raises(OutOfPages):
+        engine.step()
+    events = []
+    while engine.has_unfinished():
+        events += engine.step()
+    seq_tokens = [e.token_id for e in events]
+    assert seq_tokens == want[-len(seq_tokens):] and len(seq_tokens) >= 4
+    assert events[-1].finished
+    engine.runner.cache.check_invariants()
+    assert engine.runner.cache.requests() == []

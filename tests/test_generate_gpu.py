@@ -153,3 +153,29 @@ def test_command_line(tmp_path):
     assert record["finish_reason"] == "length" and len(record["token_ids"]) == 8
     check_greedy("A", "float32", [prompt], [record["token_ids"]])
     assert "forward_calls=" in proc.stderr
+
+
+@pytest.mark.parametrize("budget,prompt_len", [(512, 512), (2, 40)])
+def test_single_token_portion_with_pages_reserved_ahead(budget, prompt_len):
+    """A prompt's last portion (or, under a tiny budget, every portion) can be one token: the step is then all
+    single tokens and runs as a graph, while the request's block table already holds the pages of the whole
+    prompt plus one, more entries than the graph's table rows are wide.  The tokens are those of a run that
+    cuts nothing."""
+    first = tc.random_ids(40, 384, 1)
+    second = tc.random_ids(prompt_len, 384, 2)
+    params = SamplingParams(max_tokens=12)
+    base = dict(ctx=1024, max_seqs=4, block_size=16, num_blocks=160, decode_first=True)
+    want = [make_engine("D", "float32", max_batched_tokens=1024, **base).generate([p], params)[0] for p in (first, second)]
+    engine = make_engine("D", "float32", max_batched_tokens=budget, **base)
+    engine.add_request("first", first, params)
+    outputs = {"first": [], "second": []}
+    for _ in range(3 if budget > 2 else 22):          # "first" is decoding when "second" arrives
+        for ev in engine.step():
+            outputs[ev.request_id].append(ev.token_id)
+    engine.add_request("second", second, params)
+    while engine.has_unfinished():
+        for ev in engine.step():
+            outputs[ev.request_id].append(ev.token_id)
+    assert [outputs["first"], outputs["second"]] == want
+    assert engine.runner.graph_replays > 0
+    engine.runner.cache.check_invariants()
