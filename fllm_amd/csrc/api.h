@@ -111,6 +111,15 @@ double fllm_probe_mfma_bf16(void *sink, int blocks, int iters, hipStream_t strea
 // out[r] = first index of the largest finite value of logits[r, :]
 int fllm_argmax(const float *logits, int32_t *out, int rows, int vocab, hipStream_t stream);
 
+// fllm_argmax for callers that cannot allocate device memory and have no workspace to hand over (code under HIP
+// graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+// The workgroups of a row meet in a static device array of 132,096 bytes that every GPU the library runs on holds
+// until the process ends; the call allocates nothing and needs no fllm_set_device_workspace.  At most 256 rows
+// (more are refused; any vocabulary).  Same result as fllm_argmax.  All calls on one GPU share that GPU's array:
+// calls that overlap on one GPU (different streams, different threads) race; calls in stream order do not.  The
+// first call on a device looks up the array's address (once per device); make it outside a graph capture.
+int fllm_argmax_static(const float *logits, int32_t *out, int rows, int vocab, hipStream_t stream);
+
 struct FllmSampleRow {
     float temperature;   // <= 1e-5: greedy
     float top_p;         // nucleus; outside (0, 1): off

@@ -423,6 +423,65 @@ extern "C" int fllm_argmax(const float *logits, int32_t *out, int rows, int voca
     return fllm_check_launch("argmax");
 }
 
+// ---------------------------------------------------------------------------------------------
+// The split argmax for callers that cannot allocate and hand over no workspace.
+// ---------------------------------------------------------------------------------------------
+// Partial results and arrival counters live in a file-scope device array.  Every GPU holds a copy of its own at an
+// address of its own, which the host learns once per device through hipGetSymbolAddress; host code uses that
+// address only, never the array's name.  Layout: kStaticRows counters (int), then kStaticRows * kStaticParts
+// values (float), then as many indices (int).
+constexpr int kStaticRows = 256;         // most rows a call takes
+constexpr int kStaticParts = 64;         // most workgroups a row
+constexpr size_t kStaticBytes = (size_t)kStaticRows * 4 + (size_t)kStaticRows * kStaticParts * 8;     // 132,096 bytes
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];
+
+constexpr int kMaxDevices = 16;
+static void *g_static_scratch[kMaxDevices];     // per device: the address of its copy of `scratch`
+
+// the address of the current device's copy, looked up at the first call on that device
+static int static_scratch_of_current_device(unsigned char **base) {
+    int dev = -1;
+    FLLM_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices, "argmax_static: no current device below %d",
+                 kMaxDevices);
+    void *ptr = __atomic_load_n(&g_static_scratch[dev], __ATOMIC_ACQUIRE);
+    if (ptr == nullptr) {
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        FLLM_REQUIRE(e == hipSuccess && ptr != nullptr, "argmax_static: the device's scratch array was not found: %s",
+                     hipGetErrorString(e));
+        __atomic_store_n(&g_static_scratch[dev], ptr, __ATOMIC_RELEASE);     // threads that race here store the same address
+    }
+    *base = (unsigned char *)ptr;
+    return 0;
+}
+
+__global__ void clear_ints_kernel(int *p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+extern "C" int fllm_argmax_static(const float *logits, int32_t *out, int rows, int vocab, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && vocab > 0, "argmax_static: bad sizes rows=%d vocab=%d", rows, vocab);
+    FLLM_REQUIRE(rows <= kStaticRows, "argmax_static: %d rows, the static scratch array is made for at most %d (use fllm_argmax)",
+                 rows, kStaticRows);
+    if (rows == 0) return 0;
+    FLLM_REQUIRE(logits != nullptr && out != nullptr, "argmax_static: logits and out are required");
+    unsigned char *base = nullptr;
+    if (static_scratch_of_current_device(&base) != 0) return -1;
+    int parts = (vocab + 8191) / 8192;          // the plan of fllm_argmax
+    if (parts > kStaticParts) parts = kStaticParts;
+    if (parts * rows > 2048) parts = 2048 / rows;
+    if (parts < 1) parts = 1;
+    const int per_part = (vocab + parts - 1) / parts;
+    int *counters = (int *)base;
+    float *pv = (float *)(base + (size_t)kStaticRows * 4);
+    int *pi = (int *)(pv + (size_t)kStaticRows * kStaticParts);
+    // the array keeps what the call before left (a call that was cut short may have left counts): the counters start at zero
+    hipLaunchKernelGGL(clear_ints_kernel, dim3((rows + 255) / 256), dim3(256), 0, stream, counters, rows);
+    hipLaunchKernelGGL(argmax_split_kernel, dim3(rows, parts), dim3(kBlock), 0, stream, logits, out, vocab, parts, per_part, pv, pi,
+                       counters);
+    return fllm_check_launch("argmax_static");
+}
+
 extern "C" int fllm_sample(const float *logits, float *work, const FllmSampleRow *params, int32_t *out, int rows,
                            int vocab, hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
