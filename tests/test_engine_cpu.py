@@ -30,10 +30,14 @@ def runner_for(name, max_tokens, **kw):
 def test_every_way_of_cutting_gives_the_plain_logits(tmp_path, name, lengths, family):
     requests = {f"r{i}": tc.random_ids(n, tc.CONFIGS[name]["vocab_size"], 50 + i) for i, n in enumerate(lengths)}
     steps = {"whole": tt.whole, "last32": lambda r: tt.last_tokens_one_by_one(r, 8), "portions": tt.portions,
-             "mixed": lambda r: tt.mixed(r, seed=2, decode_tail=5)}[family](requests)
+             "mixed": lambda r: tt.mixed(r, seed=2, decode_tail=5, refeed=[f"r{len(lengths) - 1}"])}[family](requests)
     steps = tt.number(steps)
     cfg, w64, runner = runner_for(name, tt.live_tokens_bound(steps, round_to=16))
-    got = tt.run_in_process(runner, steps, cfg["vocab_size"], str(tmp_path))
+    given_up = {}
+    got = tt.run_in_process(runner, steps, cfg["vocab_size"], str(tmp_path), given_up)
+    assert (len(given_up) == 1) == (family == "mixed")
+    for rid, feedings in given_up.items():          # ended half way and fed again from the first token: the same logits
+        assert np.array_equal(feedings[0], got[rid][:len(feedings[0])])
     for rid, toks in requests.items():
         want = plain_llama.forward(cfg, w64, toks)
         assert np.abs(got[rid] - want).max() <= 2e-5 * np.abs(want).max(), (family, rid)

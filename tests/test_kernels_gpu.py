@@ -441,6 +441,12 @@ def attention_case(ops, ref, dtype, heads, kv_heads, head_dim, page_size, segs, 
     scale = head_dim ** -0.5
     want = ref.attention(q, k, v, tables, row_pos, row_seg, seg_start, torch.empty(rows, heads * head_dim, dtype=torch.float64),
                          heads, kv_heads, head_dim, page_size, scale, window, max_context)
+    if window:
+        # pages that lie wholly before the window of a segment's first row have been given back: their table entries
+        # are -1, and a kernel that looked at them would read outside the pages
+        tables = tables.clone()
+        for s, (p, n) in enumerate(segs):
+            tables[s, : max(0, p + 1 - window) // page_size] = -1
     uniform = int(all(n == 1 for _, n in segs))
     single_from = len(segs)
     while single_from > 0 and segs[single_from - 1][1] == 1:
@@ -579,12 +585,35 @@ def test_attention_portions_beside_single_rows(ops, ref, mark_single_rows, dtype
                    mark_single_rows=mark_single_rows)
 
 
-def test_attention_row_is_the_same_alone_and_in_a_batch(ops, ref):
-    """float32: the bits of a row do not depend on the batch around it."""
-    a = attention_case(ops, ref, torch.float32, 8, 2, 64, 16, [(100, 17), (37, 1), (0, 33)], None, 15)
-    b = attention_case(ops, ref, torch.float32, 8, 2, 64, 16, [(100, 17)], None, 15)
-    # same seed, same first segment: tables and pages differ, so compare against the reference only
-    assert a.shape[0] == 51 and b.shape[0] == 17
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_row_is_the_same_alone_and_in_a_batch(ops, dtype):
+    """The bits of a row do not depend on the batch around it: a portion of 17 rows alone and with two other segments
+    in the step, on the same pages with the same table."""
+    g = gen(15)
+    heads, kv_heads, head_dim, page_size = 8, 2, 64, 16
+    segs = [(100, 17), (37, 1), (0, 33)]
+    pages_each = 8
+    num_pages = 3 * pages_each + 2
+    tables = scattered_tables(g, 3, pages_each, num_pages)
+    k, v = make_pages(g, num_pages, kv_heads, page_size, head_dim, dtype)
+    q = torch.randn(51, heads * head_dim, generator=g).to(dtype)
+    scale = head_dim ** -0.5
+
+    def run(count):
+        these = segs[:count]
+        rows = sum(n for _, n in these)
+        row_pos = torch.tensor([p + i for p, n in these for i in range(n)], dtype=torch.int32)
+        row_seg = torch.tensor([s for s, (_, n) in enumerate(these) for _ in range(n)], dtype=torch.int32)
+        seg_start = torch.tensor(np.cumsum([0] + [n for _, n in these]), dtype=torch.int32)
+        bound = max(p + n for p, n in these)
+        ws = torch.empty(max(1, ops.attention_workspace_bytes(rows, heads, kv_heads, head_dim, bound)), dtype=torch.uint8, device=DEV)
+        return ops.attention(q[:rows].to(DEV), k.to(DEV), v.to(DEV), tables[:count].contiguous().to(DEV), row_pos.to(DEV),
+                             row_seg.to(DEV), seg_start.to(DEV), torch.empty(rows, heads * head_dim, dtype=dtype, device=DEV),
+                             heads, kv_heads, head_dim, page_size, scale, None, bound, single_from=count, workspace=ws)
+
+    together, alone = run(3), run(1)
+    assert together.shape[0] == 51 and alone.shape[0] == 17
+    assert torch.equal(together[:17], alone), "a row's bits changed with its neighbours"
 
 
 # ---------------------------------------------------------------------------------------------

@@ -26,7 +26,8 @@ ODD = {
     "group12": dict(BASE, num_hidden_layers=1, hidden_size=192, num_attention_heads=12, num_key_value_heads=1, head_dim=64,
                     intermediate_size=512, vocab_size=300, tie_word_embeddings=False, max_position_embeddings=700),
 }
-TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+# about three times the largest error seen on the MI355X (float32 9.2e-7, bfloat16 4.9e-3)
+TOL = {"float32": 3e-6, "bfloat16": 1.5e-2}
 
 
 @pytest.fixture(scope="module")
@@ -60,5 +61,6 @@ def test_odd_sizes(odd_models, tmp_path, name, family, dtype):
     got = tt.run_in_process(runner, steps, cfg["vocab_size"], str(tmp_path))
     for rid, want in plain.items():
         err = np.abs(got[rid].astype(np.float64) - want).max()
+        tt.observe(f"odd sizes {name} {dtype}", err / np.abs(want).max())
         assert err <= TOL[dtype] * np.abs(want).max(), f"{name} {dtype} {family}: request {rid}: error {err:.3e}"
     runner.cache.check_invariants()

@@ -201,6 +201,79 @@ def test_window_config_changes_only_what_lies_beyond_the_window(weights):
     assert not np.allclose(with_window[30:], without[30:], atol=1e-6)
 
 
+def test_llama3_band_interpolates_the_frequency_not_the_divisor():
+    """Inside the band the scaled frequency f / divisor is a straight line in f between f / factor at the band's low end
+    and f at its high end (rust/checkpoint/src/plan.rs:1495-1499), so 1 / divisor is a straight line in the wavelength's
+    inverse: a lane in the middle of the band has divisor 1 / ((1/factor + 1) / 2), not (factor + 1) / 2; the ends join
+    the regions outside without a step."""
+    factor, low, high, original = 8.0, 1.0, 4.0, 8192.0
+    dims = 64
+    d = P.llama3_divisors(dims, 500000.0, factor, low, high, original).astype(np.float64)
+    lanes = np.arange(dims // 2)
+    wavelength = 2 * math.pi * 500000.0 ** (2 * lanes / dims)
+    inside = (wavelength >= original / high) & (wavelength <= original / low)
+    assert inside.sum() >= 3
+    smooth = (original / wavelength[inside] - low) / (high - low)
+    assert np.allclose(1.0 / d[inside], (1 - smooth) / factor + smooth, rtol=1e-6)
+    assert not np.allclose(d[inside], (1 - smooth) * factor + smooth, rtol=1e-2)
+    # a wavelength exactly in the middle of the band (theta chosen so that lane 1 of 4 dims has it)
+    middle = original / ((low + high) / 2)
+    theta = (middle / (2 * math.pi)) ** 2                  # lane 1: wavelength 2 pi theta^(2/4)
+    assert abs(P.llama3_divisors(4, theta, factor, low, high, original)[1] - 1.0 / ((1.0 / factor + 1.0) / 2.0)) < 1e-5
+    # the band's ends
+    for edge, want in ((original / high, 1.0), (original / low, factor)):
+        theta = (edge * (1 + 1e-9) / (2 * math.pi)) ** 2
+        assert abs(P.llama3_divisors(4, theta, factor, low, high, original)[1] - want) < 1e-5
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_one_token_reduces_to_library_routines(weights, name):
+    """A sequence of one token attends to itself alone: the attention weights are 1 whatever q, k and the rotation are,
+    and the model is norms, matrix products, an activation and sums.  Written out with the library's routines in the
+    order of a pre-norm layer (the branch reads the normed stream and adds to the stream that was not normed; the last
+    norm comes before the head), it gives the plain implementation's logits; with a norm in another place it does not."""
+    cfg = tc.CONFIGS[name]
+    w = {k: torch.tensor(v) for k, v in weights[name].items()}
+    sizes = P.read_sizes(cfg)
+    group = sizes["heads"] // sizes["kv_heads"]
+    d = sizes["head_dim"]
+
+    def library(token, prenorm=True):
+        x = w["model.embed_tokens.weight"][token]
+        for i in range(sizes["layers"]):
+            p = f"model.layers.{i}"
+            h = F.rms_norm(x, x.shape, w[f"{p}.input_layernorm.weight"], eps=sizes["eps"])
+            v = F.linear(h if prenorm else x, w[f"{p}.self_attn.v_proj.weight"], w.get(f"{p}.self_attn.v_proj.bias"))
+            per_head = v.reshape(sizes["kv_heads"], d).repeat_interleave(group, dim=0).reshape(-1)
+            x = x + F.linear(per_head, w[f"{p}.self_attn.o_proj.weight"], w.get(f"{p}.self_attn.o_proj.bias"))
+            h = F.rms_norm(x, x.shape, w[f"{p}.post_attention_layernorm.weight"], eps=sizes["eps"])
+            act = F.silu(F.linear(h, w[f"{p}.mlp.gate_proj.weight"], w.get(f"{p}.mlp.gate_proj.bias"))) * \
+                F.linear(h, w[f"{p}.mlp.up_proj.weight"], w.get(f"{p}.mlp.up_proj.bias"))
+            x = x + F.linear(act, w[f"{p}.mlp.down_proj.weight"], w.get(f"{p}.mlp.down_proj.bias"))
+        x = F.rms_norm(x, x.shape, w["model.norm.weight"], eps=sizes["eps"])
+        head = w["model.embed_tokens.weight"] if sizes["tied"] else w["lm_head.weight"]
+        return F.linear(x, head).numpy()
+
+    for token in (0, 7, cfg["vocab_size"] - 1):
+        got = P.forward(cfg, weights[name], [token], first_position=5)[0]
+        assert np.allclose(got, library(token), rtol=1e-9, atol=1e-12)
+        assert not np.allclose(got, library(token, prenorm=False), rtol=1e-3)
+
+
+def test_without_branches_the_model_is_norm_and_head(weights):
+    """Output and down projections of zero: every layer adds nothing and the logits are head(norm(embedding)), for
+    every token of a sequence."""
+    cfg = tc.TINY_A
+    w = dict(weights["A"])
+    for i in range(cfg["num_hidden_layers"]):
+        for n in ("self_attn.o_proj", "mlp.down_proj"):
+            w[f"model.layers.{i}.{n}.weight"] = np.zeros_like(w[f"model.layers.{i}.{n}.weight"])
+    ids = tc.random_ids(9, 256, 8)
+    e = torch.tensor(w["model.embed_tokens.weight"])[ids]
+    want = F.linear(F.rms_norm(e, (64,), torch.tensor(w["model.norm.weight"]), eps=1e-5), torch.tensor(w["lm_head.weight"]))
+    assert np.allclose(P.forward(cfg, w, ids), want.numpy(), rtol=1e-10)
+
+
 # ---- sampling --------------------------------------------------------------------------------
 def test_philox_known_answers():
     """rust/engine/src/sampling.rs:1018-1030 (Random123's vectors for philox4x32, 10 rounds)."""

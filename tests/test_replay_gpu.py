@@ -14,10 +14,11 @@ import trace_tools as tt
 pytestmark = pytest.mark.gpu
 
 LENGTHS = {"A": [5, 17, 31, 70, 128, 100], "B": [1, 9, 40, 100, 256, 130], "C": [3, 50, 190, 77, 120, 64],
-           "D": [700, 3, 130, 1000, 64]}
+           "D": [700, 3, 130, 1000, 64], "E": [300, 45, 130, 500, 64, 90]}
 # |engine - plain| <= tol * max|plain logit| ; float32 engine against a float64 reference, and
-# bfloat16 (8 bits of mantissa in weights, activations and cache) against the same
-TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+# bfloat16 (8 bits of mantissa in weights, activations and cache) against the same.  About three times the largest
+# error any case here has shown on the MI355X (float32 7.0e-7, bfloat16 5.7e-3; the test session prints them).
+TOL = {"float32": 3e-6, "bfloat16": 1.5e-2}
 
 
 @pytest.fixture(scope="module")
@@ -51,6 +52,7 @@ def check(got, plain, dtype, what):
         err = np.abs(got[rid].astype(np.float64) - want)
         scale = np.abs(want).max()
         pos = int(err.max(axis=1).argmax())
+        tt.observe(f"replay {what.split()[0]} {dtype}", err.max() / scale)
         assert err.max() <= TOL[dtype] * scale, (f"{what}: request {rid}: max error {err.max():.3e} at position {pos} "
                                                  f"(limit {TOL[dtype] * scale:.3e}); first position over the limit: "
                                                  f"{int(np.argmax(err.max(axis=1) > TOL[dtype] * scale))}")
@@ -63,18 +65,30 @@ def make_runner(folder, dtype, page_size, max_tokens, use_graphs=True):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 @pytest.mark.parametrize("family", ["whole", "last32", "portions", "mixed"])
 def test_replay(models, tmp_path, name, dtype, family):
     folder, cfg, requests, plain = models[name]
+    refed = [rid for rid, toks in requests.items() if len(toks) >= 60][:2]
     steps = {"whole": tt.whole, "last32": tt.last_tokens_one_by_one, "portions": tt.portions,
-             "mixed": lambda r: tt.mixed(r, seed=5)}[family](requests)
+             "mixed": lambda r: tt.mixed(r, seed=5, refeed=refed)}[family](requests)
     steps = tt.number(steps)
     max_tokens = tt.live_tokens_bound(steps)
     runner = make_runner(folder, dtype, tc.PAGE_SIZES[name], max_tokens)
     handed_out = tt.record_allocations(runner.cache)
-    got = tt.run_in_process(runner, steps, cfg["vocab_size"], str(tmp_path))
+    given_up = {}
+    got = tt.run_in_process(runner, steps, cfg["vocab_size"], str(tmp_path), given_up)
     check(got, plain, dtype, f"{name} {dtype} {family}")
+    if family == "mixed":
+        # a request that was ended half way and fed again from its first token (as after a preemption) gave the same
+        # logits the first time, on other pages and in other company
+        assert sorted(given_up) == sorted(refed)
+        for rid, feedings in given_up.items():
+            for first in feedings:
+                assert len(first) >= len(requests[rid]) // 2
+                if dtype == "float32":
+                    assert np.array_equal(first, got[rid][:len(first)]), f"{rid}: fed again, other logits"
+                check({rid: first}, {rid: plain[rid][:len(first)]}, dtype, f"{name} {dtype} given-up")
     runner.cache.check_invariants()
     assert all(pool.available == pool.num_pages for pool in runner.cache.pools), "pages were lost"
     for pages in handed_out:

@@ -1,7 +1,9 @@
 """Tiny Llama configurations for tests.  A and B differ in every size and option; C adds a
 sliding window on some layers, a partial rotary width, linear rotary scaling and biases; D has heads
 of 64 (the head size of the 128-row prompt attention kernel) and room for a thousand positions, so that
-a portion of a prompt meets contexts of many key tiles."""
+a portion of a prompt meets contexts of many key tiles; E has heads of 64 with a sliding window on two of its three
+layers, so that the matrix-core attention kernels meet windows, pages that were given back (table entries of -1)
+and pages that are used again."""
 import json
 
 import numpy as np
@@ -37,8 +39,15 @@ TINY_D = {
                      "original_max_position_embeddings": 256},
     "tie_word_embeddings": False, "max_position_embeddings": 1024, "hidden_act": "silu",
 }
-PAGE_SIZES = {"A": 16, "B": 8, "C": 16, "D": 16}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+TINY_E = {
+    "model_type": "llama", "architectures": ["LlamaForCausalLM"],
+    "num_hidden_layers": 3, "hidden_size": 192, "num_attention_heads": 6, "num_key_value_heads": 2, "head_dim": 64,
+    "intermediate_size": 272, "vocab_size": 320, "rope_theta": 250000.0, "rms_norm_eps": 2e-6,
+    "sliding_window": 40, "layer_types": ["sliding_attention", "full_attention", "sliding_attention"],
+    "tie_word_embeddings": True, "max_position_embeddings": 512, "hidden_act": "silu",
+}
+PAGE_SIZES = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 16}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
 
 
 def to_float64(tensors):

@@ -10,6 +10,15 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 PORTIONS = [7, 2, 13, 3, 32, 2, 11, 5, 64, 2]
 
 
+# Largest |engine - plain| / max |plain logit| that each group of comparisons saw in this run; the test session prints
+# them at its end (tests/conftest.py), which is where the tolerances of the bfloat16 comparisons come from.
+OBSERVED = {}
+
+
+def observe(group, value):
+    OBSERVED[group] = max(OBSERVED.get(group, 0.0), float(value))
+
+
 def whole(requests):
     """Each request alone, in one step, logits wanted everywhere."""
     steps = []
@@ -46,12 +55,16 @@ def portions(requests, sizes=PORTIONS):
     return steps
 
 
-def mixed(requests, seed, max_live=4, decode_tail=12):
+def mixed(requests, seed, max_live=4, decode_tail=12, refeed=()):
     """Up to `max_live` requests at a time: portions of some beside single tokens of others;
-    a request sometimes sits a step out; finished requests leave and the next one arrives."""
+    a request sometimes sits a step out; finished requests leave and the next one arrives.
+    A request named in `refeed` is ended once it has been fed about half of its tokens (what it holds is given
+    back) and is fed again from its first token under the same name while the others go on, as a scheduler does
+    that preempts a request and computes it again."""
     rng = np.random.default_rng(seed)
     waiting = list(requests.items())
     live = {}      # id -> (tokens, fed)
+    again = set(refeed)
     steps = []
     while waiting or live:
         while waiting and len(live) < max_live:
@@ -72,6 +85,11 @@ def mixed(requests, seed, max_live=4, decode_tail=12):
             if fed + n == len(toks):
                 ends.append(rid)
                 del live[rid]
+            elif rid in again and fed + n >= len(toks) // 2:
+                again.discard(rid)
+                ends.append(rid)                                 # given up half way ...
+                del live[rid]
+                waiting.insert(0, (rid, toks))                   # ... and next in line, from its first token
         if entries:
             steps.append({"entries": entries, "end": ends})
     return steps
@@ -93,30 +111,37 @@ def live_tokens_bound(steps, round_to=64):
     return most
 
 
-def collect(steps, read_step, vocab):
-    """Per request the logits of every position, in position order: id -> [tokens, vocab]."""
+def collect(steps, read_step, vocab, given_up=None):
+    """Per request the logits of every position, in position order: id -> [tokens, vocab].  Of a request that was
+    ended and fed again this is the last feeding; what the feedings before it gave goes to `given_up`
+    (id -> list of [tokens fed, vocab]) when that is a dict."""
     out = {}
+    ended = set()
     for s in steps:
         wanted = sum(len(e["want"]) for e in s["entries"])
-        if not wanted:
-            continue
-        data = read_step(s["step"]).reshape(wanted, vocab)
+        data = read_step(s["step"]).reshape(wanted, vocab) if wanted else None
         o = 0
         for e in s["entries"]:
             n = len(e["want"])
             assert e["want"] == list(range(len(e["tokens"]))), "these traces want every position"
+            if e["id"] in ended:                                  # fed again from its first token
+                ended.discard(e["id"])
+                if given_up is not None:
+                    given_up.setdefault(e["id"], []).append(np.concatenate(out[e["id"]]))
+                out[e["id"]] = []
             out.setdefault(e["id"], []).append(data[o:o + n])
             o += n
+        ended.update(s["end"])
     return {k: np.concatenate(v) for k, v in out.items()}
 
 
-def run_in_process(runner, steps, vocab, out_dir):
+def run_in_process(runner, steps, vocab, out_dir, given_up=None):
     import io
     from fllm_amd.engine.replay import replay
     log = io.StringIO()
     replay(runner, [json.dumps(s) for s in steps], out_dir, out=log)
     assert log.getvalue().split() == [w for s in steps for w in ("done", str(s["step"]))]
-    return collect(steps, lambda i: np.fromfile(os.path.join(out_dir, f"{i}.f32"), dtype="<f4"), vocab)
+    return collect(steps, lambda i: np.fromfile(os.path.join(out_dir, f"{i}.f32"), dtype="<f4"), vocab, given_up)
 
 
 def run_subprocess(model_dir, dtype, steps, vocab, out_dir, max_tokens, env=None):
