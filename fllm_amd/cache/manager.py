@@ -39,11 +39,19 @@ class _Request:
 
 
 class CacheManager:
-    def __init__(self, groups: Sequence[GroupSpec], pages_per_group: Sequence[int], max_requests: int):
+    def __init__(self, groups: Sequence[GroupSpec], pages_per_group: Sequence[int], max_requests: int,
+                 max_step_tokens: Optional[int] = None):
+        """`max_step_tokens`: the most tokens of one request that a step brings, when the caller keeps to such a
+        bound.  A window group then never holds pages further ahead of a request than one step can reach, however
+        far a reservation looks (a whole prompt at admission): its pool can be made for
+        `window_pages_bound` pages a request instead of a whole context."""
         if len(groups) != len(pages_per_group):
             raise ValueError("one page count per group is required")
         if max_requests <= 0:
             raise ValueError("max_requests must be positive")
+        if max_step_tokens is not None and max_step_tokens <= 0:
+            raise ValueError("max_step_tokens must be positive")
+        self.max_step_tokens = max_step_tokens
         self.groups = list(groups)
         self.pools = [PagePool(n) for n in pages_per_group]
         self.max_requests = max_requests
@@ -105,6 +113,19 @@ class CacheManager:
             return 0
         return max(0, length - group.window + 1) // group.page_size
 
+    def _covered_upto(self, group: GroupSpec, length: int, total: int) -> int:
+        """Table entries below this index are to hold pages so that positions below `total` are covered; in a window
+        group no further than the next step can reach."""
+        if group.window is not None and self.max_step_tokens is not None:
+            total = min(total, length + self.max_step_tokens)
+        return -(-total // group.page_size)
+
+    @staticmethod
+    def window_pages_bound(window: int, page_size: int, max_step_tokens: int) -> int:
+        """Most pages a request holds in a window group when no step brings more than `max_step_tokens` of its
+        tokens: the window before the step's first row, the step's rows, and the page edges on both sides."""
+        return -(-(window - 1 + max_step_tokens) // page_size) + 1
+
     def pages_missing(self, req_id, total: int) -> List[int]:
         """Pages each group would have to hand out so that positions below `total` are covered.
         Every table entry from the first page still needed to the end of the table holds a page
@@ -113,7 +134,7 @@ class CacheManager:
         req = self._get(req_id)
         out = []
         for g, group in enumerate(self.groups):
-            need_upto = -(-total // group.page_size)
+            need_upto = self._covered_upto(group, req.length, total)
             have_upto = max(len(req.tables[g]), self._first_needed_page(group, req.length))
             out.append(max(0, need_upto - have_upto))
         return out
@@ -129,7 +150,7 @@ class CacheManager:
                 raise OutOfPages(f"group {g} needs {m} pages, {pool.available} are free")
         req = self._get(req_id)
         for g, group in enumerate(self.groups):
-            need_upto = -(-total // group.page_size)
+            need_upto = self._covered_upto(group, req.length, total)
             table = req.tables[g]
             first = self._first_needed_page(group, req.length)
             start = max(first, len(table))          # entries below `first` are never read again: they stay empty

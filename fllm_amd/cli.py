@@ -102,7 +102,7 @@ def cmd_inspect(argv: List[str]) -> int:
     ap = argparse.ArgumentParser(prog="fllm_amd inspect")
     ap.add_argument("model")
     args = ap.parse_args(argv)
-    from .config.llama import read_config_json
+    from .config.files import read_config_json
     from .registry import model_spec_from_config
     from .weights.loader import check_tensors, expected_tensors
     from .weights.safetensors_io import open_checkpoint

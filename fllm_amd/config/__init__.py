@@ -1,5 +1,6 @@
 from .spec import ConfigError, LayerSpec, ModelSpec, PartSpec, RunEntry, default_run_order
-from .llama import LlamaConfig, RopeScaling, read_config_json
+from .files import read_config_json
+from .llama import LlamaConfig, RopeScaling
 
 __all__ = ["ConfigError", "LayerSpec", "ModelSpec", "PartSpec", "RunEntry", "default_run_order",
            "LlamaConfig", "RopeScaling", "read_config_json"]

@@ -7,12 +7,11 @@ Keys, defaults and error texts follow the reference's checkpoint planner
 """
 from __future__ import annotations
 
-import json
 import math
-import os
 from dataclasses import dataclass
 from typing import Any, Dict, Optional, Tuple
 
+from .files import read_config_json
 from .spec import ConfigError
 
 _EPS_KEYS = ("rms_norm_eps", "layer_norm_eps", "norm_epsilon", "layer_norm_epsilon", "norm_eps", "layernorm_epsilon")
@@ -184,22 +183,6 @@ class LlamaConfig:
         if self.bos_token_id is not None:
             out["bos_token_id"] = self.bos_token_id
         return out
-
-
-def read_config_json(path: str) -> Dict[str, Any]:
-    """`path` is a model folder or a config.json file."""
-    if os.path.isdir(path):
-        path = os.path.join(path, "config.json")
-    try:
-        with open(path, "r", encoding="utf-8") as fh:
-            cfg = json.load(fh)
-    except FileNotFoundError:
-        raise ConfigError(f"{path} not found") from None
-    except json.JSONDecodeError as exc:
-        raise ConfigError(f"{path} is not valid JSON: {exc}") from None
-    if not isinstance(cfg, dict):
-        raise ConfigError(f"{path} must hold a JSON object")
-    return cfg
 
 
 def _first(*values):

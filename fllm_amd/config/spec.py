@@ -33,12 +33,25 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """A block: its arrangement (`block.kind`) and the parts the arrangement places."""
+    """A block: its arrangement (`block.kind`) and the parts the arrangement places.  `mixer` is the part that may own
+    a cache or per-request state; `feed_forward` may be absent; `norms` are named by the arrangement; `extras` are
+    further weight-holding parts of any role that the arrangement knows by name (name -> (role, PartSpec))."""
 
     block: PartSpec
     mixer: PartSpec
-    feed_forward: PartSpec
-    norms: Dict[str, PartSpec]
+    feed_forward: Optional[PartSpec] = None
+    norms: Dict[str, PartSpec] = field(default_factory=dict)
+    extras: Dict[str, Tuple[str, PartSpec]] = field(default_factory=dict)
+
+    def parts(self):
+        """(name, role, PartSpec) of every part the layer places, the block's own spec aside."""
+        for name, norm in self.norms.items():
+            yield f"norm:{name}", "norm", norm
+        yield "mixer", "mixer", self.mixer
+        if self.feed_forward is not None:
+            yield "feed_forward", "feed_forward", self.feed_forward
+        for name, (role, part) in self.extras.items():
+            yield f"extra:{name}", role, part
 
 
 @dataclass(frozen=True)

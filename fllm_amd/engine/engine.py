@@ -12,7 +12,7 @@ from typing import Dict, List, Optional, Sequence as Seq, Union
 
 import torch
 
-from ..config.llama import read_config_json
+from ..config.files import read_config_json
 from ..registry import model_spec_from_config
 from ..sampling import SampleRequest, Sampler, SamplingParams
 from ..weights.loader import load_checkpoint
@@ -87,7 +87,7 @@ class Engine:
             tensors = random_tensors(spec, seed, parse_dtype(dtype), device=device if random_weights_on_device else "cpu")
         self.runner = ModelRunner(spec, tensors, dtype=dtype, device=device, page_size=block_size, num_pages=num_blocks,
                                   max_requests=max_seqs, max_context=ctx, memory_utilization=gpu_memory_utilization,
-                                  ops=ops, typed_config=typed)
+                                  ops=ops, typed_config=typed, max_step_tokens=max_batched_tokens)
         del tensors
         self.config = typed
         self.max_model_len = self.runner.max_context

@@ -28,8 +28,11 @@ class Model:
         for layer in spec.layers:
             norms = {name: make("norm", n) for name, n in layer.norms.items()}
             mixer = make("mixer", layer.mixer)
-            ffn = make("feed_forward", layer.feed_forward)
-            self.blocks.append(make("block", layer.block, mixer=mixer, feed_forward=ffn, norms=norms))
+            ffn = make("feed_forward", layer.feed_forward) if layer.feed_forward is not None else None
+            placed = dict(mixer=mixer, feed_forward=ffn, norms=norms)
+            if layer.extras:            # only an arrangement that names further parts is handed them
+                placed["extras"] = {name: make(role, part) for name, (role, part) in layer.extras.items()}
+            self.blocks.append(make("block", layer.block, **placed))
         self.final_norm = make("norm", spec.final_norm)
         self.head = make("head", spec.head)
         self.bindings: List[CacheBinding] = []
@@ -78,12 +81,13 @@ class Model:
         return [GroupSpec(entries=tuple(m), kv_heads=k[0], head_dim=k[1], window=k[2], page_size=page_size)
                 for k, m in zip(self.group_keys, self.group_members)]
 
-    def cache_bytes_per_page(self, page_size: int) -> int:
-        """Bytes one page costs over all groups (a page of every group per `page_size` tokens)."""
+    def cache_bytes_per_page(self, page_size: int) -> List[int]:
+        """Bytes a page of each group costs (keys and values of all the group's run entries)."""
         elem = torch.empty((), dtype=self.rt.dtype).element_size()
-        return sum(2 * len(m) * k[0] * k[1] * page_size * elem for k, m in zip(self.group_keys, self.group_members))
+        return [2 * len(m) * k[0] * k[1] * page_size * elem for k, m in zip(self.group_keys, self.group_members)]
 
-    def allocate_caches(self, page_size: int, pages_per_group: Sequence[int], max_requests: int) -> CacheManager:
+    def allocate_caches(self, page_size: int, pages_per_group: Sequence[int], max_requests: int,
+                        max_step_tokens: Optional[int] = None) -> CacheManager:
         """Device pages for every group (one page more than the manager hands out: the null page
         that padding rows of a captured step write to) and the state arenas."""
         rt = self.rt
@@ -112,7 +116,17 @@ class Model:
             idx = self.entry_index[i]
             self.bindings.append(CacheBinding(group=g, k_pages=self.k_store[g][idx], v_pages=self.v_store[g][idx],
                                               page_size=page_size, writes=entry.reads_cache_of is None, state=state))
-        return CacheManager(groups, list(pages_per_group), max_requests)
+        return CacheManager(groups, list(pages_per_group), max_requests, max_step_tokens=max_step_tokens)
+
+    def clear_state(self, slot: int) -> None:
+        """Zeros the fixed-size state of every run entry in one request slot (a request's first step)."""
+        for binding in self.bindings:
+            if binding.state is not None:
+                binding.state[slot].zero_()
+
+    @property
+    def has_state(self) -> bool:
+        return any(b.state is not None for b in self.bindings)
 
     # ---- forward --------------------------------------------------------------------------
     def forward(self, ctx: StepContext) -> torch.Tensor:

@@ -16,7 +16,7 @@ from typing import Dict, List, Optional, Sequence, Union
 import torch
 
 from ..cache import CacheManager, OutOfPages
-from ..config.llama import read_config_json
+from ..config.files import read_config_json
 from ..config.spec import ModelSpec
 from ..parts.runtime import Runtime
 from ..registry import model_spec_from_config
@@ -61,9 +61,14 @@ class StepEntry:
 
 class ModelRunner:
     def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype="bfloat16", device="cuda:0",
-                 page_size: int = 16, max_tokens: Optional[int] = None, num_pages: Optional[int] = None,
+                 page_size: int = 16, max_tokens: Optional[int] = None,
+                 num_pages: Union[int, Sequence[int], None] = None,
                  max_requests: int = 16, max_context: Optional[int] = None, memory_utilization: float = 0.90,
-                 ops=None, typed_config=None, use_graphs: bool = True):
+                 ops=None, typed_config=None, use_graphs: bool = True, max_step_tokens: Optional[int] = None):
+        """`num_pages`: pages of every cache group (one number) or of each group (a list); by default what
+        `max_tokens` tokens need, else what fits on the card.  `max_step_tokens`: the most tokens of one request
+        that a step may bring (more are refused); with it, groups that keep a window of keys are made no larger than
+        `max_requests` requests can fill."""
         self.spec = spec
         self.config = typed_config
         self.device = torch.device(device)
@@ -80,20 +85,30 @@ class ModelRunner:
         self.model = Model(spec, tensors, self.rt)
         self.vocab_size = spec.vocab_size
         num_groups = len(self.model.group_keys)
+        self.max_requests = max_requests
+        self.max_step_tokens = None if max_step_tokens is None else int(max_step_tokens)
         if num_pages is None and max_tokens is not None:
             num_pages = -(-int(max_tokens) // page_size)
         if num_pages is None:
-            num_pages = self._pages_that_fit(memory_utilization, max_requests)
-        if num_pages <= 0:
+            pages = self._pages_that_fit(memory_utilization, max_requests)
+        elif isinstance(num_pages, int):
+            pages = [min(num_pages, cap) for cap in self._page_caps(max_requests)]
+        else:
+            pages = [int(n) for n in num_pages]
+            if len(pages) != num_groups:
+                raise ValueError(f"the model has {num_groups} cache groups, {len(pages)} page counts were given")
+        if any(n <= 0 for n in pages):
             raise ValueError("the cache needs at least one page")
-        self.num_pages = int(num_pages)
-        self.max_requests = max_requests
-        self.cache: CacheManager = self.model.allocate_caches(page_size, [self.num_pages] * num_groups, max_requests)
+        self.pages_per_group = pages
+        self.cache: CacheManager = self.model.allocate_caches(page_size, pages, max_requests,
+                                                              max_step_tokens=self.max_step_tokens)
         self.steps = 0
         self.rows_total = 0
         # decode steps replay captured graphs when every part can be captured (parts say so with
         # `graph_safe`; a part that decides on the host per step cannot)
-        parts_ok = all(getattr(b.mixer, "graph_safe", False) and getattr(b.feed_forward, "graph_safe", False)
+        parts_ok = all(getattr(b.mixer, "graph_safe", False)
+                       and (b.feed_forward is None or getattr(b.feed_forward, "graph_safe", False))
+                       and all(getattr(p, "graph_safe", False) for p in getattr(b, "extras", {}).values())
                        for b in self.model.blocks)
         self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and parts_ok
         self._graphs: Dict[tuple, "_DecodeGraph"] = {}
@@ -109,16 +124,36 @@ class ModelRunner:
         tensors = load_checkpoint(model_dir, spec)
         return ModelRunner(spec, tensors, typed_config=typed, **kwargs)
 
-    def _pages_that_fit(self, utilization: float, max_requests: int) -> int:
-        """Pages for what is left of the card after the weights, capped at what `max_requests`
-        requests of full context can use."""
-        per_page = max(1, self.model.cache_bytes_per_page(self.page_size))
-        cap = max_requests * (-(-self.max_context // self.page_size))
+    def _page_caps(self, max_requests: int) -> List[int]:
+        """Per cache group the most pages `max_requests` requests can hold: whole contexts, or, for a group that
+        keeps a window when steps are bounded, the window and one step."""
+        caps = []
+        for key in self.model.group_keys:
+            window = key[2]
+            each = -(-self.max_context // self.page_size)
+            if window is not None and self.max_step_tokens is not None:
+                each = min(each, CacheManager.window_pages_bound(window, self.page_size, self.max_step_tokens))
+            caps.append(max_requests * each)
+        return caps
+
+    def _pages_that_fit(self, utilization: float, max_requests: int) -> List[int]:
+        """Pages for what is left of the card after the weights: window groups get what `max_requests` requests
+        can fill, the other groups share the rest equally (a token needs a page of each), capped likewise."""
+        per_page = self.model.cache_bytes_per_page(self.page_size)
+        caps = self._page_caps(max_requests)
         if self.device.type != "cuda":
-            return cap
+            return caps
         free, total = torch.cuda.mem_get_info(self.device)
         budget = int(free - (1.0 - utilization) * total) - (2 << 30)   # room for activations and logits
-        return max(1, min(cap, budget // per_page))
+        bounded = [key[2] is not None and self.max_step_tokens is not None for key in self.model.group_keys]
+        pages = [cap if b else 0 for cap, b in zip(caps, bounded)]
+        budget -= sum(n * size for n, size in zip(pages, per_page))
+        rest = [g for g, b in enumerate(bounded) if not b]
+        if rest:
+            each = budget // max(1, sum(per_page[g] for g in rest))
+            for g in rest:
+                pages[g] = max(1, min(caps[g], each))
+        return pages
 
     # ---- requests -------------------------------------------------------------------------
     def add_request(self, req_id) -> int:
@@ -156,13 +191,16 @@ class ModelRunner:
             for w in e.want:
                 if not 0 <= int(w) < n:
                     raise StepError(f"request {e.req_id!r} wants logits at {w}, it brings {n} tokens")
+            if self.max_step_tokens is not None and n > self.max_step_tokens:
+                raise StepError(f"request {e.req_id!r} brings {n} tokens, a step takes at most {self.max_step_tokens} of a request")
             start = self.cache.length(e.req_id) if self.cache.has_request(e.req_id) else 0
             if start + n > self.max_context:
                 raise StepError(f"request {e.req_id!r} would hold {start + n} tokens, the context is {self.max_context}")
 
     def step(self, entries: Sequence[StepEntry], previous_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Runs the entries as one batch and returns float32 logits [wanted, vocab] on the device,
-        in the order of the entries and of each entry's `want`.  Unknown requests are added.
+        in the order of the entries and of each entry's `want`; they are valid until the next step (decode steps
+        replay graphs that write them in place).  Unknown requests are added.
         Raises `OutOfPages` (nothing changed) when the pages do not suffice.
         `previous_tokens`: the int32 device tensor that entries with `carry` take their token from."""
         self._validate(entries, previous_tokens)
@@ -187,6 +225,10 @@ class ModelRunner:
             for r in added:
                 self.cache.free_request(r)
             raise
+        if self.model.has_state:
+            for e in entries:                # a request's first step finds its state slot cleared
+                if self.cache.length(e.req_id) == 0:
+                    self.model.clear_state(self.cache.slot(e.req_id))
         logits = None
         if self.use_graphs and all(len(e.tokens) == 1 for e in entries) and len(entries) <= GRAPH_BUCKETS[-1]:
             logits = self._graph_step(entries, previous_tokens)

@@ -107,17 +107,19 @@ class PagedAttention(Mixer):
         cache store are one kernel.  False: not taken, the block runs norm and `forward`."""
         rt, ops = self.rt, self.rt.ops
         rows = residual.shape[0]
-        if (rt.dtype != torch.bfloat16 or self.pairing != 1 or getattr(norm, "spec", None) is None or norm.spec.kind != "rms"
+        prologue = getattr(norm, "fused_prologue", lambda: None)()
+        if (rt.dtype != torch.bfloat16 or self.pairing != 1 or prologue is None
                 or not hasattr(ops, "norm_qkv_rope_store") or not ops.fused_decode_supported(rows, self.hidden)
                 or self.head_dim % 4 != 0):
             return False
+        norm_scale, norm_eps = prologue
         nh, nkv, d = self.heads, self.kv_heads, self.head_dim
         if self.position is not None:
             cos, sin, dims = self.position.cos, self.position.sin, self.position.dims
         else:
             cos, sin, dims, _ = ctx.no_rotation(rt)
         q = rt.empty((rows, nh * d))
-        ops.norm_qkv_rope_store(residual, norm.weight, norm.eps, self.w_qkv, q, ctx.row_pos, ctx.row_seg,
+        ops.norm_qkv_rope_store(residual, norm_scale, norm_eps, self.w_qkv, q, ctx.row_pos, ctx.row_seg,
                                 ctx.tables[binding.group], cos, sin, binding.k_pages if binding.writes else None,
                                 binding.v_pages if binding.writes else None, nh, nkv, d, dims, binding.page_size,
                                 bias=self.b_qkv)

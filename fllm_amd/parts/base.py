@@ -6,14 +6,26 @@ runtime (device, precision, kernel library).  It never sees the model configurat
 Roles and their interfaces:
 
   norm          forward(ctx, x_f32[R,H], out=None, rows=None) -> normed[R or len(rows), H] in the
-                compute dtype; `rows` (int32 device tensor) selects rows first.
+                compute dtype; `rows` (int32 device tensor) selects rows first.  Optional:
+                add_forward(ctx, x, branch, out=None) adds `branch` to x first (one pass over the row), and
+                fused_prologue() -> (scale_f32[H], eps) when the norm is x * rsqrt(mean(x^2) + eps) * scale for some
+                vector `scale` (None otherwise): parts that have a kernel which norms its input on the way in ask the
+                norm for these instead of asking what kind of norm it is.
   position      what the mixer's kernels take: for the attention mixer float32 device tables `cos` and `sin`
                 [positions, dims/2], `dims` (lanes of a head that are rotated) and `pairing` (0: lanes l and
                 l + dims/2, 1: lanes 2l and 2l + 1).
   mixer         cache_need() / state_need() say what the cache manager must keep for it;
                 forward(ctx, h[R,H], residual_f32[R,H], binding) adds its output to `residual`.
+                State of fixed size: `binding.state[slot]` belongs to one live request (slot = ctx.seg_slots[s] on the
+                host, ctx.slots[s] on the device).  The step function hands it over filled with zeros at the first
+                step of a request it has not seen before (also one that was freed and is fed again from position 0),
+                touches it at no other time, and runs a request's rows in position order, `seg_pos_start[s]` being the
+                number of tokens the request held before this step; so the state a mixer finds is the one it left after
+                position seg_pos_start[s] - 1.
   feed_forward  forward(ctx, h[R,H], residual_f32[R,H]) adds its output to `residual`.
-  block         forward(ctx, residual_f32[R,H], binding) runs norms, mixer and feed-forward.  A block
+  block         forward(ctx, residual_f32[R,H], binding) runs norms, mixer and feed-forward.  It is built with
+                mixer=, feed_forward= (None for a layer without one), norms= (by the names the layer's spec
+                uses) and, only when the spec lists any, extras= (further parts by name).  A block
                 with `takes_pending = True` is called as forward(ctx, residual, binding, pending): `pending`
                 is a branch [R,H] that the block before left for it to add (or None), and it returns its
                 own such branch or None.
@@ -92,6 +104,11 @@ class Norm(Part):
 
     def forward(self, ctx, x, out=None, rows=None):
         raise NotImplementedError
+
+    def fused_prologue(self):
+        """(scale, eps) if the norm is x * rsqrt(mean(x^2) + eps) * scale with a float32 device vector `scale`,
+        so that a kernel can apply it to the rows it reads; None if it is anything else."""
+        return None
 
 
 class Block(Part):

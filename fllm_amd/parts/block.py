@@ -12,7 +12,7 @@ class PreNormBlock(Block):
         self.mixer = mixer
         self.feed_forward = feed_forward
         self.mixer_norm = norms["mixer"]
-        self.feed_forward_norm = norms["feed_forward"]
+        self.feed_forward_norm = norms["feed_forward"] if feed_forward is not None else None
 
     takes_pending = True     # forward accepts a branch that the block before has not added yet, and may hand one on
 
@@ -22,7 +22,7 @@ class PreNormBlock(Block):
         been added.  Where a sum can ride on the norm that follows it, it costs no pass of its own."""
         ops = self.rt.ops
         add_mixer_norm = getattr(self.mixer_norm, "add_forward", None)
-        add_ff_norm = getattr(self.feed_forward_norm, "add_forward", None)
+        add_ff_norm = getattr(self.feed_forward_norm, "add_forward", None) if self.feed_forward is not None else None
         # a part may take the residual stream and the norm before it in one fused kernel
         fused = getattr(self.mixer, "forward_from_residual", None)
         if pending is not None:
@@ -47,6 +47,8 @@ class PreNormBlock(Block):
                     self.feed_forward.forward(ctx, h, residual)
                 return out
             self.mixer.forward(ctx, h, residual, binding)
+        if self.feed_forward is None:
+            return None                  # a layer of a mixer alone
         fused = getattr(self.feed_forward, "forward_from_residual", None)
         if fused is None or not fused(ctx, residual, self.feed_forward_norm):
             h = self.feed_forward_norm.forward(ctx, residual)

@@ -39,11 +39,13 @@ class GatedMLP(FeedForward):
         False: not taken, the block runs norm and `forward`."""
         rt, ops = self.rt, self.rt.ops
         rows = residual.shape[0]
-        if (rt.dtype != torch.bfloat16 or getattr(norm, "spec", None) is None or norm.spec.kind != "rms"
+        prologue = getattr(norm, "fused_prologue", lambda: None)()
+        if (rt.dtype != torch.bfloat16 or prologue is None
                 or not hasattr(ops, "norm_gate_up_swiglu") or not ops.fused_decode_supported(rows, self.hidden)):
             return False
+        norm_scale, norm_eps = prologue
         act = rt.empty((rows, self.inter))
-        ops.norm_gate_up_swiglu(residual, norm.weight, norm.eps, self.w_gate_up, act, bias=self.b_gate_up)
+        ops.norm_gate_up_swiglu(residual, norm_scale, norm_eps, self.w_gate_up, act, bias=self.b_gate_up)
         ops.linear(act, self.w_down, residual, bias=self.b_down, accumulate=True)
         return True
 

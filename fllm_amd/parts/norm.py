@@ -25,6 +25,8 @@ class RMSNorm(Norm):
             out = self.rt.empty((count, self.size))
         return self.rt.ops.rmsnorm(x, self.weight, self.eps, out, rows=rows)
 
+    def fused_prologue(self):
+        return self.weight, self.eps
 
     def add_forward(self, ctx, x, branch, out=None):
         """x += branch, then the norm of the sum: one pass over the row."""

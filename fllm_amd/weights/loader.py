@@ -37,10 +37,9 @@ def iter_parts(spec: ModelSpec):
     """(role, PartSpec) of every part of the model, each weight-holding part once."""
     yield "embedding", spec.embedding
     for layer in spec.layers:
-        for norm in layer.norms.values():
-            yield "norm", norm
-        yield "mixer", layer.mixer
-        yield "feed_forward", layer.feed_forward
+        yield "block", layer.block
+        for _, role, part in layer.parts():
+            yield role, part
     yield "norm", spec.final_norm
     yield "head", spec.head
 

@@ -161,3 +161,34 @@ def test_random_orders_keep_the_books(seed):
     m.check_invariants()
     assert m.free_pages(0) == 24 and m.free_pages(1) == 24 and m.free_slots() == 4
     assert finished > 10 and refused > 0
+
+
+def test_window_group_looks_no_further_ahead_than_a_step():
+    """With a bound on the tokens a step brings, a group that keeps a window holds pages for the window and one step,
+    however long the prompt that a reservation covers; a pool made for that bound never runs dry, under random steps."""
+    window, page, step = 10, 4, 7
+    bound = CacheManager.window_pages_bound(window, page, step)
+    assert bound == 5                                  # 9 keys behind the first row + 7 rows = 16 positions, + one edge
+    requests = 3
+    m = CacheManager([full(page), windowed(window, page)], [200, requests * bound], max_requests=requests, max_step_tokens=step)
+    m.add_request("a")
+    assert m.pages_missing("a", 101) == [26, 2]        # admission: the whole prompt in the full group, one step in the other
+    m.reserve("a", 101)
+    assert len([p for p in m.table("a", 1) if p >= 0]) == 2
+    rng = random.Random(3)
+    names = ["a", "b", "c"]
+    m.add_request("b"), m.add_request("c")
+    most = 0
+    for _ in range(400):
+        name = rng.choice(names)
+        n = rng.randint(1, step)
+        m.reserve(name, m.length(name) + n)
+        most = max(most, max(sum(p >= 0 for p in m.table(x, 1)) for x in names))
+        m.commit(name, n)
+        m.check_invariants()
+        if m.length(name) > 150:
+            m.free_request(name)
+            m.add_request(name)
+    assert most == bound                               # the bound is reached, and never passed
+    with pytest.raises(ValueError):
+        m.commit("a", step + 40)                       # more than was reserved: a step longer than the bound

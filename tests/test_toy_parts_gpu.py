@@ -276,3 +276,165 @@ def test_toy_routed_feed_forward_and_position_encoding(dtype, tol):
         err = np.abs(got.double().cpu().numpy() - want).max()
         assert err <= tol * np.abs(want).max(), err
     runner.cache.check_invariants()
+
+
+# ---------------------------------------------------------------------------------------------
+# A norm of another kind, layers without a feed-forward, and a state that the mixer never clears itself
+# ---------------------------------------------------------------------------------------------
+from fllm_amd.parts.base import INIT_NORM, Norm  # noqa: E402
+
+
+class PlusOneNorm(Norm):
+    """y = x * rsqrt(mean(x^2) + eps) * (1 + w): the weight is stored as a distance from one.  It says what a kernel
+    needs to apply it (`fused_prologue`), and so gets the decode kernels that norm their input on the way in."""
+
+    @classmethod
+    def tensor_shapes(cls, spec):
+        return {"weight": ((spec["size"],), INIT_NORM)}
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        self.size, self.eps = int(spec["size"]), float(spec["eps"])
+        self.scale = (rt.vector(weights["weight"]) + 1.0).contiguous()
+
+    def forward(self, ctx, x, out=None, rows=None):
+        count = x.shape[0] if rows is None else rows.numel()
+        out = self.rt.empty((count, self.size)) if out is None else out
+        return self.rt.ops.rmsnorm(x, self.scale, self.eps, out, rows=rows)
+
+    def fused_prologue(self):
+        return self.scale, self.eps
+
+
+class TrustingSum(DecayingSum):
+    """The decaying sum again, but it never clears its state: it relies on the step function handing a request's
+    slot over filled with zeros."""
+
+    def forward(self, ctx, h, residual, binding):
+        row = 0
+        for rows, slot in zip(ctx.seg_rows, ctx.seg_slots):
+            state = binding.state[slot]
+            for r in range(row, row + rows):
+                state.mul_(self.decay).add_(h[r].float())
+                residual[r] += (self.w.float() @ state)
+            row += rows
+
+
+register_part("norm", "rms_plus_one", PlusOneNorm)
+register_part("mixer", "trusting_sum", TrustingSum)
+
+
+def bare_spec(cfg):
+    hidden = cfg["hidden_size"]
+    norm = lambda name: PartSpec("rms_plus_one", {"size": hidden, "eps": 1e-5}, {"weight": name})
+    attention = lambda i: PartSpec("attention", {"hidden_size": hidden, "num_heads": 4, "num_kv_heads": 2, "head_dim": 16,
+                                                 "scale": 0.25, "window": None,
+                                                 "position": {"kind": "rotary", "dims": 16, "theta": 10000.0, "scaling": "none",
+                                                              "pairing": "interleaved", "max_position": 128}},
+                                   {k: f"layers.{i}.attn.{k}" for k in "qkvo"})
+    layers = [LayerSpec(PartSpec("prenorm"), attention(0), norms={"mixer": norm("layers.0.n1")})]      # no feed-forward
+    if cfg["stateful"]:
+        layers.append(LayerSpec(PartSpec("prenorm"), PartSpec("trusting_sum", {"hidden_size": hidden, "decay": 0.5},
+                                                              {"w": "layers.1.mix.w"}), norms={"mixer": norm("layers.1.n1")}))
+    else:
+        ffn = PartSpec("gated_mlp", {"hidden_size": hidden, "intermediate_size": 96, "activation": "silu"},
+                       {k: f"layers.1.mlp.{k}" for k in ("gate", "up", "down")})
+        layers.append(LayerSpec(PartSpec("prenorm"), attention(1), ffn,
+                                {"mixer": norm("layers.1.n1"), "feed_forward": norm("layers.1.n2")}))
+    return ModelSpec("toy-bare", hidden, cfg["vocab_size"], 128,
+                     PartSpec("table", {"vocab_size": cfg["vocab_size"], "hidden_size": hidden}, {"weight": "embed"}),
+                     tuple(layers), (RunEntry(0), RunEntry(1)), norm("final_norm"),
+                     PartSpec("linear", {"vocab_size": cfg["vocab_size"], "hidden_size": hidden}, {"weight": "head"}))
+
+
+register_architecture(Architecture("toy-bare", ("ToyBareModel",), lambda c: c, bare_spec))
+
+
+def plain_bare(w, ids, stateful):
+    x = w["embed"][np.asarray(ids)]
+    T = len(ids)
+    norm = lambda x, name: P.rms_norm(x, 1.0 + w[name], 1e-5)
+    cos, sin = P.rope_tables(range(T), 16, 10000.0)
+
+    def attention(x, i):
+        h = norm(x, f"layers.{i}.n1")
+        q = P.apply_rope((h @ w[f"layers.{i}.attn.q"].T).reshape(T, 4, 16), cos, sin, 16, interleaved=True)
+        k = P.apply_rope((h @ w[f"layers.{i}.attn.k"].T).reshape(T, 2, 16), cos, sin, 16, interleaved=True)
+        v = (h @ w[f"layers.{i}.attn.v"].T).reshape(T, 2, 16)
+        return x + P.attention(q, k, v, 0.25).reshape(T, 64) @ w[f"layers.{i}.attn.o"].T
+
+    x = attention(x, 0)
+    if stateful:
+        h = norm(x, "layers.1.n1")
+        state = np.zeros(64)
+        out = np.zeros_like(x)
+        for t in range(T):
+            state = 0.5 * state + h[t]
+            out[t] = w["layers.1.mix.w"] @ state
+        x = x + out
+    else:
+        x = attention(x, 1)
+        h = norm(x, "layers.1.n2")
+        x = x + P.gated_mlp(h, w["layers.1.mlp.gate"], w["layers.1.mlp.up"], w["layers.1.mlp.down"])
+    return norm(x, "final_norm") @ w["head"].T
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 3e-5), ("bfloat16", 1.5e-2)])
+def test_toy_norm_keeps_the_fused_decode_kernels_and_a_layer_may_lack_a_feed_forward(dtype, tol):
+    cfg = {"model_type": "toy-bare", "hidden_size": 64, "vocab_size": 150, "stateful": False}
+    _, spec = model_spec_from_config(cfg)
+    tensors = {k: v.float() for k, v in random_tensors(spec, 23, torch.bfloat16).items()}
+    runner = ModelRunner(spec, tensors, dtype=dtype, page_size=16, max_tokens=256, max_requests=4)
+    assert runner.use_graphs and runner.model.blocks[0].feed_forward is None
+    calls = {"norm_qkv_rope_store": 0, "norm_gate_up_swiglu": 0}
+    for name in calls:
+        def counted(*args, _fn=getattr(runner.rt.ops, name), _name=name, **kw):
+            calls[_name] += 1
+            return _fn(*args, **kw)
+        setattr(runner.rt.ops, name, counted)
+    try:
+        w64 = tc.to_float64(tensors)
+        a, b = tc.random_ids(40, 150, 3), tc.random_ids(25, 150, 4)
+        want_a, want_b = plain_bare(w64, a, False), plain_bare(w64, b, False)
+        all_of = lambda toks: list(range(len(toks)))
+        got_a = [runner.step([StepEntry("a", a[:30], all_of(a[:30]))])]
+        got_b = [runner.step([StepEntry("b", b[:20], all_of(b[:20]))])]
+        for i in range(5):      # a step's logits are valid until the next step: decode graphs write them in place
+            out = runner.step([StepEntry("a", [a[30 + i]], [0]), StepEntry("b", [b[20 + i]], [0])]).clone()
+            got_a.append(out[:1]); got_b.append(out[1:])
+        for i in range(35, 40):
+            got_a.append(runner.step([StepEntry("a", [a[i]], [0])]).clone())
+    finally:
+        for name in calls:
+            delattr(runner.rt.ops, name)
+    for got, want in ((torch.cat(got_a), want_a), (torch.cat(got_b), want_b)):
+        err = np.abs(got.double().cpu().numpy() - want).max()
+        assert err <= tol * np.abs(want).max(), err
+    if dtype == "bfloat16":      # the decode steps went through the kernels that norm on the way in, and through graphs
+        assert calls["norm_qkv_rope_store"] >= 2 and calls["norm_gate_up_swiglu"] >= 1 and runner.graph_replays >= 8
+    else:
+        assert calls == {"norm_qkv_rope_store": 0, "norm_gate_up_swiglu": 0}
+
+
+def test_state_slot_is_handed_over_cleared():
+    """A mixer that never clears its state: a request's first step finds zeros, also in a slot that another request
+    used before and also when the same request is freed and fed again."""
+    cfg = {"model_type": "toy-bare", "hidden_size": 64, "vocab_size": 150, "stateful": True}
+    _, spec = model_spec_from_config(cfg)
+    tensors = random_tensors(spec, 29, torch.float32)
+    runner = ModelRunner(spec, tensors, dtype="float32", page_size=16, max_tokens=256, max_requests=2)
+    w64 = tc.to_float64(tensors)
+    a, b = tc.random_ids(30, 150, 5), tc.random_ids(21, 150, 6)
+    want_a, want_b = plain_bare(w64, a, True), plain_bare(w64, b, True)
+    all_of = lambda toks: list(range(len(toks)))
+    close = lambda got, want: np.abs(got.double().cpu().numpy() - want).max() <= 3e-5 * np.abs(want).max()
+    first = torch.cat([runner.step([StepEntry("a", a[:11], all_of(a[:11]))]), runner.step([StepEntry("a", a[11:], all_of(a[11:]))])])
+    assert close(first, want_a)
+    slot = runner.cache.slot("a")
+    runner.free_request("a")
+    assert close(runner.step([StepEntry("b", b, all_of(b))]), want_b) and runner.cache.slot("b") == slot
+    runner.free_request("b")
+    half = runner.step([StepEntry("a", a[:15], all_of(a[:15]))])            # given up half way ...
+    runner.free_request("a")
+    again = runner.step([StepEntry("a", a, all_of(a))])                    # ... and fed again from its first token
+    assert close(half, want_a[:15]) and close(again, want_a)
