@@ -15,115 +15,87 @@ namespace {
 constexpr int kBlock = 1024;
 constexpr int kWaves = kBlock / kWave;
 
-struct Shared {
-    double dred[kWaves];
-    float fred[kWaves];
-    int ired[kWaves];
-    unsigned hist[256];
-    uint32_t prefix;
-    int remaining;
+// A candidate for "the largest value, at the lowest index among equals".  kNone marks "nothing qualified".
+constexpr int kNone = 0x7fffffff;
+struct Pick {
+    float value;
+    int index;
+};
+__device__ __forceinline__ Pick better_of(Pick a, Pick b) {
+    const bool take_b = b.value > a.value || (b.value == a.value && b.index < a.index);
+    return take_b ? b : a;
+}
+
+// What the reductions of a workgroup pass through LDS: one cell a wave.
+struct Cells {
+    Pick picks[kWaves];
+    double sums[kWaves];
+    int counts[kWaves];
+    int word;            // a value one thread hands to all
+    uint32_t key;
 };
 
-__device__ __forceinline__ void philox4x32_10(uint32_t c[4], uint32_t k0, uint32_t k1) {
+__device__ __forceinline__ Pick wave_best(Pick p) {
 #pragma unroll
-    for (int i = 0; i < 10; i++) {
-        const uint32_t hi0 = __umulhi(0xD2511F53u, c[0]), lo0 = 0xD2511F53u * c[0];
-        const uint32_t hi1 = __umulhi(0xCD9E8D57u, c[2]), lo1 = 0xCD9E8D57u * c[2];
-        const uint32_t n0 = hi1 ^ c[1] ^ k0, n2 = hi0 ^ c[3] ^ k1;
-        c[0] = n0; c[1] = lo1; c[2] = n2; c[3] = lo0;
-        k0 += 0x9E3779B9u;
-        k1 += 0xBB67AE85u;
+    for (int hop = kWave / 2; hop >= 1; hop /= 2) {
+        Pick other;
+        other.value = __shfl_xor(p.value, hop, kWave);
+        other.index = __shfl_xor(p.index, hop, kWave);
+        p = better_of(p, other);
     }
+    return p;
 }
-
-// a number in the open interval (0, 1)
-__device__ __forceinline__ float philox_uniform(uint64_t seed, uint64_t draw, uint32_t index) {
-    uint32_t c[4] = {index, 0u, (uint32_t)draw, (uint32_t)(draw >> 32)};
-    philox4x32_10(c, (uint32_t)seed, (uint32_t)(seed >> 32));
-    return ((float)(c[0] >> 8) + 0.5f) / 16777216.0f;
-}
-
-// order-preserving map of floats to unsigned integers (larger float, larger key)
-__device__ __forceinline__ uint32_t f2key(float f) {
-    const uint32_t u = __float_as_uint(f);
-    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
-
-__device__ __forceinline__ double block_sum_d(double v, Shared &sh) {
+__device__ __forceinline__ int wave_count(int v) {
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-    __syncthreads();
-    if ((threadIdx.x & (kWave - 1)) == 0) sh.dred[threadIdx.x / kWave] = v;
-    __syncthreads();
-    double total = 0.0;
+    for (int hop = kWave / 2; hop >= 1; hop /= 2) v += __shfl_xor(v, hop, kWave);
+    return v;
+}
+__device__ __forceinline__ double wave_mass(double v) {
 #pragma unroll
-    for (int i = 0; i < kWaves; i++) total += sh.dred[i];
-    __syncthreads();
-    return total;
+    for (int hop = kWave / 2; hop >= 1; hop /= 2) v += __shfl_xor(v, hop, kWave);
+    return v;
 }
 
-__device__ __forceinline__ float block_max_f(float v, Shared &sh) {
-    v = wave_max(v);
+// The best pick of the workgroup, the same in every thread: every wave leaves its best in its cell and all threads
+// fold the cells in wave order.
+__device__ __forceinline__ Pick block_best(Pick p, Cells &cells) {
+    p = wave_best(p);
+    const int wave = threadIdx.x / kWave;
+    __syncthreads();                               // the cells are free again
+    if (threadIdx.x % kWave == 0) cells.picks[wave] = p;
     __syncthreads();
-    if ((threadIdx.x & (kWave - 1)) == 0) sh.fred[threadIdx.x / kWave] = v;
-    __syncthreads();
-    float m = -INFINITY;
+    Pick all = cells.picks[0];
 #pragma unroll
-    for (int i = 0; i < kWaves; i++) m = fmaxf(m, sh.fred[i]);
-    __syncthreads();
-    return m;
+    for (int w = 1; w < kWaves; w++) all = better_of(all, cells.picks[w]);
+    return all;
+}
+__device__ __forceinline__ float block_largest(float v, Cells &cells) {
+    Pick p = {v, 0};
+    return block_best(p, cells).value;
 }
 
-// largest value, lowest index on ties; index INT_MAX when nothing qualified
-__device__ __forceinline__ int block_argmax(float v, int idx, Shared &sh) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const float ov = __shfl_xor(v, o, kWave);
-        const int oi = __shfl_xor(idx, o, kWave);
-        if (ov > v || (ov == v && oi < idx)) {
-            v = ov;
-            idx = oi;
-        }
-    }
-    __syncthreads();
-    if ((threadIdx.x & (kWave - 1)) == 0) {
-        sh.fred[threadIdx.x / kWave] = v;
-        sh.ired[threadIdx.x / kWave] = idx;
-    }
-    __syncthreads();
-    float best = sh.fred[0];
-    int besti = sh.ired[0];
-#pragma unroll
-    for (int i = 1; i < kWaves; i++) {
-        if (sh.fred[i] > best || (sh.fred[i] == best && sh.ired[i] < besti)) {
-            best = sh.fred[i];
-            besti = sh.ired[i];
-        }
-    }
-    __syncthreads();
-    return besti;
-}
+// finite values stay, everything else can never be chosen
+__device__ __forceinline__ float usable(float v) { return fabsf(v) < INFINITY ? v : -INFINITY; }
 
-__device__ __forceinline__ float sanitize(float v) { return isfinite(v) ? v : -INFINITY; }
-
-__device__ int row_argmax(const float *w, int vocab, Shared &sh) {
-    float best = -INFINITY;
-    int besti = 0x7fffffff;
-    for (int i = threadIdx.x; i < vocab; i += kBlock) {
+// the best pick among w[lo .. hi): a thread meets its indices in rising order, so the first of equal values stays
+__device__ __forceinline__ Pick best_in_range(const float *w, int lo, int hi) {
+    Pick mine = {-INFINITY, kNone};
+    for (int i = lo + (int)threadIdx.x; i < hi; i += kBlock) {
         const float v = w[i];
-        if (isfinite(v) && v > best) {   // indices rise, so the first maximum stays
-            best = v;
-            besti = i;
+        if (fabsf(v) < INFINITY && v > mine.value) {
+            mine.value = v;
+            mine.index = i;
         }
     }
-    return block_argmax(best, besti, sh);
+    return mine;
 }
+__device__ __forceinline__ int32_t token_of(Pick p) { return p.index == kNone ? 0 : p.index; }
 
 __global__ void __launch_bounds__(kBlock)
 argmax_kernel(const float *__restrict__ logits, int32_t *__restrict__ out, int vocab) {
-    __shared__ Shared sh;
-    const int idx = row_argmax(logits + (size_t)blockIdx.x * vocab, vocab, sh);
-    if (threadIdx.x == 0) out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
+    __shared__ Cells cells;
+    const Pick best = block_best(best_in_range(logits + (size_t)blockIdx.x * vocab, 0, vocab), cells);
+    if (threadIdx.x == 0) out[blockIdx.x] = token_of(best);
 }
 
 // The same over `parts` workgroups a row: each takes a stretch of the vocabulary and leaves its best (value,
@@ -132,40 +104,67 @@ argmax_kernel(const float *__restrict__ logits, int32_t *__restrict__ out, int v
 __global__ void __launch_bounds__(kBlock)
 argmax_split_kernel(const float *__restrict__ logits, int32_t *__restrict__ out, int vocab, int parts, int per_part,
                     float *partial_v, int *partial_i, int *counters) {
-    __shared__ Shared sh;
-    __shared__ int s_seen;
+    __shared__ Cells cells;
     const int row = blockIdx.x, part = blockIdx.y;
     const int lo = part * per_part, hi = min(vocab, lo + per_part);
-    const float *w = logits + (size_t)row * vocab;
-    float best = -INFINITY;
-    int besti = 0x7fffffff;
-    for (int i = lo + threadIdx.x; i < hi; i += kBlock) {
-        const float v = w[i];
-        if (isfinite(v) && v > best) {
-            best = v;
-            besti = i;
-        }
-    }
-    besti = block_argmax(best, besti, sh);
+    const Pick best = block_best(best_in_range(logits + (size_t)row * vocab, lo, hi), cells);
     if (threadIdx.x == 0) {
-        const float bv = besti == 0x7fffffff ? -INFINITY : w[besti];
-        __hip_atomic_store(partial_v + (size_t)row * parts + part, bv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(partial_i + (size_t)row * parts + part, besti, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(partial_v + (size_t)row * parts + part, best.value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(partial_i + (size_t)row * parts + part, best.index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __builtin_amdgcn_s_waitcnt(0);      // the part has arrived before it is counted
-        s_seen = __hip_atomic_fetch_add(counters + row, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        cells.word = __hip_atomic_fetch_add(counters + row, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
-    if (s_seen != parts - 1) return;
+    if (cells.word != parts - 1) return;
     if (threadIdx.x == 0) __hip_atomic_store(counters + row, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    float v = -INFINITY;
-    int idx = 0x7fffffff;
+    Pick mine = {-INFINITY, kNone};
     if ((int)threadIdx.x < parts) {
-        v = __hip_atomic_load(partial_v + (size_t)row * parts + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        idx = __hip_atomic_load(partial_i + (size_t)row * parts + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        mine.value = __hip_atomic_load(partial_v + (size_t)row * parts + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        mine.index = __hip_atomic_load(partial_i + (size_t)row * parts + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    idx = block_argmax(v, idx, sh);
-    if (threadIdx.x == 0) out[row] = idx == 0x7fffffff ? 0 : idx;
+    const Pick all = block_best(mine, cells);
+    if (threadIdx.x == 0) out[row] = token_of(all);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Random numbers: Philox-4x32 with ten rounds (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3"), the
+// generator the reference keys its draws with (rust/engine/src/sampling.rs:155-183).  A round multiplies two
+// counter words by fixed odd constants and mixes the halves of the products with the other words and the key; the
+// key moves on by the golden-ratio and sqrt(3) - 1 constants.
+// ---------------------------------------------------------------------------------------------
+struct Philox {
+    uint32_t c0, c1, c2, c3;
+    __device__ __forceinline__ void ten_rounds(uint32_t key_lo, uint32_t key_hi) {
+#pragma unroll
+        for (int round = 0; round < 10; round++) {
+            const uint64_t left = (uint64_t)0xD2511F53u * c0;
+            const uint64_t right = (uint64_t)0xCD9E8D57u * c2;
+            const uint32_t next0 = (uint32_t)(right >> 32) ^ c1 ^ key_lo;
+            const uint32_t next2 = (uint32_t)(left >> 32) ^ c3 ^ key_hi;
+            c1 = (uint32_t)right;
+            c3 = (uint32_t)left;
+            c0 = next0;
+            c2 = next2;
+            key_lo += 0x9E3779B9u;
+            key_hi += 0xBB67AE85u;
+        }
+    }
+};
+
+// The uniform number of (seed, draw, token): the counter is (token, 0, draw), the key is the seed; the top 24 bits of
+// the first output word, centred in their cell, so that the number lies strictly between 0 and 1.
+__device__ __forceinline__ float uniform_of(uint64_t seed, uint64_t draw, uint32_t token) {
+    Philox g = {token, 0u, (uint32_t)draw, (uint32_t)(draw >> 32)};
+    g.ten_rounds((uint32_t)seed, (uint32_t)(seed >> 32));
+    return ((float)(g.c0 >> 8) + 0.5f) * (1.0f / 16777216.0f);
+}
+
+// Floats as unsigned integers in the same order: the sign bit is set on positive numbers, all bits are turned
+// over on negative ones.
+__device__ __forceinline__ uint32_t ordered_key(float f) {
+    const uint32_t bits = __float_as_uint(f);
+    return bits ^ ((uint32_t)((int32_t)bits >> 31) | 0x80000000u);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -176,11 +175,17 @@ argmax_split_kernel(const float *__restrict__ logits, int32_t *__restrict__ out,
 // counts for top-k, probability mass in 40-bit fixed point for top-p: integer sums, so the order of
 // the additions does not matter); the bin in which the threshold falls is read off it, the tokens
 // up to that bin are gathered into a list (in an order that depends on the data only), and the
-// exact thresholds (radix select, bisection over the keys with sums in double precision) and the
-// draw then run over the list.  A threshold further than 64 below the maximum puts every token on
-// the list.
+// exact thresholds and the draw then run over the list.  A threshold further than 64 below the maximum puts every
+// token on the list.
+//
+// A threshold is a key t (ordered_key of a logit): the tokens with keys >= t stay.  Both thresholds are the largest
+// t for which a sum over {key >= t} still reaches a target (k tokens; top_p of the mass), and such a t is built
+// bit by bit from the top: a bit stays set if the sum with it set still reaches the target.  A list of up to
+// kStaged candidates is copied into LDS (logit and weight exp((v - max) / T)) and ONE wave runs the 32 + 32 trials
+// over it with shuffles and no barrier; a longer list is walked by the whole workgroup.
 constexpr int kBins = 4096;
 constexpr float kBinsPerUnit = 64.0f;
+constexpr int kStaged = 4096;            // candidates that fit into the LDS the histogram no longer needs
 
 // bin of a finite logit v <= m; kBins: further from the maximum than the histogram reaches
 __device__ __forceinline__ int bin_of(float v, float m) {
@@ -189,7 +194,7 @@ __device__ __forceinline__ int bin_of(float v, float m) {
 }
 
 // exclusive prefix sum over the threads of the workgroup, and the total
-__device__ __forceinline__ int block_exclusive_scan(int v, Shared &sh, int *total) {
+__device__ __forceinline__ int block_exclusive_scan(int v, Cells &cells, int *total) {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     int inc = v;
 #pragma unroll
@@ -198,13 +203,13 @@ __device__ __forceinline__ int block_exclusive_scan(int v, Shared &sh, int *tota
         if (lane >= o) inc += n;
     }
     __syncthreads();
-    if (lane == kWave - 1) sh.ired[wave] = inc;
+    if (lane == kWave - 1) cells.counts[wave] = inc;
     __syncthreads();
     int before = 0, all = 0;
 #pragma unroll
     for (int i = 0; i < kWaves; i++) {
-        if (i < wave) before += sh.ired[i];
-        all += sh.ired[i];
+        if (i < wave) before += cells.counts[i];
+        all += cells.counts[i];
     }
     __syncthreads();
     *total = all;
@@ -213,7 +218,7 @@ __device__ __forceinline__ int block_exclusive_scan(int v, Shared &sh, int *tota
 
 // The lowest bin b with sum(hist[0..b]) >= target, kBins when the whole histogram falls short; done by the first
 // wave, every lane over 64 bins; the same value in every thread.
-__device__ int find_bin(const unsigned long long *hist, unsigned long long target, Shared &sh) {
+__device__ int find_bin(const unsigned long long *hist, unsigned long long target, Cells &cells) {
     __syncthreads();
     if (threadIdx.x < kWave) {
         const int lane = threadIdx.x;
@@ -238,70 +243,113 @@ __device__ int find_bin(const unsigned long long *hist, unsigned long long targe
         }
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) found = min(found, __shfl_xor(found, o, kWave));
-        if (lane == 0) sh.remaining = found;
+        if (lane == 0) cells.word = found;
     }
     __syncthreads();
-    const int bin = sh.remaining;
+    const int bin = cells.word;
     __syncthreads();
     return bin;
 }
 
-// key of the k-th largest value among get(0 .. n-1): radix select, 4 passes of 8 bits
-template <typename Get>
-__device__ uint32_t kth_largest_key_of(Get get, int n, int k, Shared &sh) {
-    if (threadIdx.x == 0) {
-        sh.prefix = 0;
-        sh.remaining = k;
+// Who walks a list of candidates: the first wave alone (sums by shuffles, no barrier; the other waves wait at the
+// next barrier) or the whole workgroup (sums through LDS).  Sums are the same in every thread that takes part.
+struct OneWave {
+    static constexpr int kStride = kWave;
+    __device__ static int sum(int v, Cells &) { return wave_count(v); }
+    __device__ static double sum(double v, Cells &) { return wave_mass(v); }
+};
+struct WholeBlock {
+    static constexpr int kStride = kBlock;
+    __device__ static int sum(int v, Cells &cells) {
+        v = wave_count(v);
+        __syncthreads();
+        if (threadIdx.x % kWave == 0) cells.counts[threadIdx.x / kWave] = v;
+        __syncthreads();
+        int all = 0;
+#pragma unroll
+        for (int w = 0; w < kWaves; w++) all += cells.counts[w];
+        return all;
     }
-    __syncthreads();
-    for (int pass = 0; pass < 4; pass++) {
-        const int shift = 24 - 8 * pass;
-        for (int i = threadIdx.x; i < 256; i += kBlock) sh.hist[i] = 0;
+    __device__ static double sum(double v, Cells &cells) {
+        v = wave_mass(v);
         __syncthreads();
-        const uint32_t prefix = sh.prefix;
-        for (int i = threadIdx.x; i < n; i += kBlock) {
-            const uint32_t key = f2key(get(i));
-            const bool match = pass == 0 || (key >> (shift + 8)) == (prefix >> (shift + 8));
-            if (match) atomicAdd(&sh.hist[(key >> shift) & 255u], 1u);
-        }
+        if (threadIdx.x % kWave == 0) cells.sums[threadIdx.x / kWave] = v;
         __syncthreads();
-        if (threadIdx.x == 0) {
-            int acc = 0;
-            const int rem = sh.remaining;
-            uint32_t bin = 0;
-            for (int b = 255; b >= 0; b--) {
-                if (acc + (int)sh.hist[b] >= rem) {
-                    bin = (uint32_t)b;
-                    break;
-                }
-                acc += (int)sh.hist[b];
-            }
-            sh.prefix = prefix | (bin << shift);
-            sh.remaining = rem - acc;
-        }
-        __syncthreads();
+        double all = 0.0;
+#pragma unroll
+        for (int w = 0; w < kWaves; w++) all += cells.sums[w];      // in wave order: the same in every thread
+        return all;
     }
-    return sh.prefix;
+};
+
+// The largest key t such that at least k of the n candidates have keys >= t (the key of the k-th largest), built
+// from the top bit down.  1 <= k <= n.
+template <typename Who, typename KeyAt>
+__device__ uint32_t key_of_kth_largest(KeyAt key_at, int n, int k, Cells &cells) {
+    uint32_t t = 0;
+    for (int bit = 31; bit >= 0; bit--) {
+        const uint32_t trial = t | (1u << bit);
+        int mine = 0;
+        for (int i = threadIdx.x; i < n; i += Who::kStride) mine += key_at(i) >= trial ? 1 : 0;
+        if (Who::sum(mine, cells) >= k) t = trial;
+    }
+    return t;
+}
+
+// Sum of the weights of the candidates with keys >= t.
+template <typename Who, typename KeyAt, typename WeightAt>
+__device__ double mass_from(KeyAt key_at, WeightAt weight_at, int n, uint32_t t, Cells &cells) {
+    double mine = 0.0;
+    for (int i = threadIdx.x; i < n; i += Who::kStride)
+        if (key_at(i) >= t) mine += (double)weight_at(i);
+    return Who::sum(mine, cells);
+}
+
+// The largest key t >= floor such that the weights of the candidates with keys >= t add up to `target` or more
+// (floor itself if no larger key does).
+template <typename Who, typename KeyAt, typename WeightAt>
+__device__ uint32_t key_of_mass(KeyAt key_at, WeightAt weight_at, int n, uint32_t floor, double target, Cells &cells) {
+    uint32_t t = 0;
+    for (int bit = 31; bit >= 0; bit--) {
+        const uint32_t trial = t | (1u << bit);
+        // below the floor the answer is known: everything from the floor up counts, and that reaches the target
+        if (trial <= floor || mass_from<Who>(key_at, weight_at, n, trial, cells) >= target) t = trial;
+    }
+    return t > floor ? t : floor;
+}
+
+// Both thresholds over one list.  `total` comes in as the mass of all finite logits and is replaced by the mass of
+// what top-k keeps when top-k is on.
+template <typename Who, typename KeyAt, typename WeightAt>
+__device__ uint32_t thresholds(KeyAt key_at, WeightAt weight_at, int n, int top_k, bool use_k, bool use_p, float top_p,
+                               double total, Cells &cells) {
+    uint32_t t = 0;
+    if (use_k) {
+        t = key_of_kth_largest<Who>(key_at, n, min(top_k, n), cells);
+        if (use_p) total = mass_from<Who>(key_at, weight_at, n, t, cells);
+    }
+    if (use_p) t = key_of_mass<Who>(key_at, weight_at, n, t, (double)top_p * total, cells);
+    return t;
 }
 
 // `work` gives every row `vocab` 32-bit words of its own (the list of token ids); it must not overlap the logits.
 __global__ void __launch_bounds__(kBlock)
 sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const FllmSampleRow *__restrict__ params,
               int32_t *__restrict__ out, int vocab) {
-    __shared__ Shared sh;
-    __shared__ unsigned long long bins[kBins];
+    __shared__ Cells cells;
+    __shared__ unsigned long long bins[kBins];       // the histogram; afterwards the staged candidates
     const int row = blockIdx.x;
     const FllmSampleRow p = params[row];
     const float *src = logits + (size_t)row * vocab;
     if (p.temperature <= 1e-5f) {
-        const int idx = row_argmax(src, vocab, sh);
-        if (threadIdx.x == 0) out[row] = idx == 0x7fffffff ? 0 : idx;
+        const Pick best = block_best(best_in_range(src, 0, vocab), cells);
+        if (threadIdx.x == 0) out[row] = token_of(best);
         return;
     }
     int *list = (int *)(work + (size_t)row * vocab);
     float m = -INFINITY;
-    for (int i = threadIdx.x; i < vocab; i += kBlock) m = fmaxf(m, sanitize(src[i]));
-    m = block_max_f(m, sh);
+    for (int i = threadIdx.x; i < vocab; i += kBlock) m = fmaxf(m, usable(src[i]));
+    m = block_largest(m, cells);
     if (!(m > -INFINITY)) {
         if (threadIdx.x == 0) out[row] = 0;   // no finite logit: the reference's argmax gives index 0 as well
         return;
@@ -317,7 +365,7 @@ sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const 
         double total = 0.0;                  // mass of all finite logits (top-p without top-k)
         unsigned long long reach = 0;        // what this thread put into the histogram, in its units (top-p)
         for (int i = threadIdx.x; i < vocab; i += kBlock) {
-            const float v = sanitize(src[i]);
+            const float v = usable(src[i]);
             if (!(v > -INFINITY)) continue;
             const int b = bin_of(v, m);
             if (use_k) {
@@ -332,71 +380,62 @@ sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const 
         }
         int last_bin;
         if (use_k) {
-            last_bin = find_bin(bins, (unsigned long long)p.top_k, sh);
+            last_bin = find_bin(bins, (unsigned long long)p.top_k, cells);
         } else {
-            total = block_sum_d(total, sh);
+            total = WholeBlock::sum(total, cells);
             // the sum of every thread's share, far tokens included: integers, the same in any order
-            const double all = block_sum_d((double)reach, sh);
-            last_bin = find_bin(bins, (unsigned long long)((double)p.top_p * all), sh);
+            const double all = WholeBlock::sum((double)reach, cells);
+            last_bin = find_bin(bins, (unsigned long long)((double)p.top_p * all), cells);
             if (last_bin < kBins) last_bin++;   // a bin to spare: the histogram's sums are rounded, the exact ones decide
         }
         // gather the tokens up to that bin: thread t's tokens in the order it meets them, behind those of the threads before it
         int mine = 0;
         for (int i = threadIdx.x; i < vocab; i += kBlock) {
-            const float v = sanitize(src[i]);
+            const float v = usable(src[i]);
             mine += (v > -INFINITY && bin_of(v, m) <= last_bin) ? 1 : 0;
         }
-        int at = block_exclusive_scan(mine, sh, &count);
+        int at = block_exclusive_scan(mine, cells, &count);
         for (int i = threadIdx.x; i < vocab; i += kBlock) {
-            const float v = sanitize(src[i]);
+            const float v = usable(src[i]);
             if (v > -INFINITY && bin_of(v, m) <= last_bin) list[at++] = i;
         }
-        __syncthreads();
-        auto listed = [&](int i) { return sanitize(src[list[i]]); };
-        if (use_k) {
-            threshold = kth_largest_key_of(listed, count, min(p.top_k, count), sh);
-            if (use_p) {                      // the mass of what top-k left
-                total = 0.0;
-                for (int i = threadIdx.x; i < count; i += kBlock) {
-                    const float v = listed(i);
-                    if (f2key(v) >= threshold) total += (double)expf((v - m) * inv_t);
-                }
-                total = block_sum_d(total, sh);
+        __syncthreads();                     // the list is written (global memory, read back by other threads below)
+        if (count <= kStaged) {
+            // the histogram is done with: its memory takes the candidates' logits and weights, and one wave finds both thresholds
+            float *logit_of = (float *)bins, *weight_of = logit_of + kStaged;
+            for (int i = threadIdx.x; i < count; i += kBlock) {
+                const float v = usable(src[list[i]]);
+                logit_of[i] = v;
+                weight_of[i] = expf((v - m) * inv_t);
             }
-        }
-        if (use_p) {
-            const double target = (double)p.top_p * total;
-            // largest key t such that the mass of {key >= t} still reaches the target
-            uint32_t lo = threshold, hi = 0xFFFFFFFFu;
-            while (lo < hi) {
-                const uint32_t mid = lo + ((hi - lo) >> 1) + 1;
-                double part = 0.0;
-                for (int i = threadIdx.x; i < count; i += kBlock) {
-                    const float v = listed(i);
-                    if (f2key(v) >= mid) part += (double)expf((v - m) * inv_t);
-                }
-                if (block_sum_d(part, sh) >= target) lo = mid;
-                else hi = mid - 1;
+            __syncthreads();
+            if (threadIdx.x < kWave) {
+                const uint32_t t = thresholds<OneWave>([&](int i) { return ordered_key(logit_of[i]); },
+                                                       [&](int i) { return weight_of[i]; }, count, p.top_k, use_k, use_p,
+                                                       p.top_p, total, cells);
+                if (threadIdx.x == 0) cells.key = t;
             }
-            threshold = lo;
+            __syncthreads();
+            threshold = cells.key;
+        } else {
+            threshold = thresholds<WholeBlock>([&](int i) { return ordered_key(usable(src[list[i]])); },
+                                               [&](int i) { return expf((usable(src[list[i]]) - m) * inv_t); }, count,
+                                               p.top_k, use_k, use_p, p.top_p, total, cells);
         }
     }
-    float best = -INFINITY;
-    int besti = 0x7fffffff;
+    // Gumbel-max over what is left: the largest of (v - max) / T - ln(-ln u), u the token's uniform number
+    Pick best = {-INFINITY, kNone};
     const bool whole = !(use_k || use_p);
     for (int i = threadIdx.x; i < count; i += kBlock) {
         const int id = whole ? i : list[i];
-        const float v = sanitize(src[id]);
-        if (!(v > -INFINITY) || f2key(v) < threshold) continue;
-        const float u = philox_uniform(p.seed, p.draw, (uint32_t)id);
-        const float score = (v - m) * inv_t - logf(-logf(u));
-        if (score > best || (score == best && id < besti)) {
-            best = score;
-            besti = id;
-        }
+        const float v = usable(src[id]);
+        if (!(v > -INFINITY) || ordered_key(v) < threshold) continue;
+        const float u = uniform_of(p.seed, p.draw, (uint32_t)id);
+        const Pick here = {(v - m) * inv_t - logf(-logf(u)), id};
+        best = better_of(best, here);
     }
-    const int idx = block_argmax(best, besti, sh);
-    if (threadIdx.x == 0) out[row] = idx == 0x7fffffff ? 0 : idx;
+    best = block_best(best, cells);
+    if (threadIdx.x == 0) out[row] = token_of(best);
 }
 
 }  // namespace

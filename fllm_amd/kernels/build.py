@@ -53,20 +53,22 @@ def _fallback_dir() -> str:
     return os.path.join(tempfile.gettempdir(), f"fllm_amd_build_{os.getuid()}_{_source_digest()}")
 
 
-def find_library() -> Optional[str]:
-    """An existing library that matches the sources (the in-tree one is taken as is when it has
-    no digest file beside it: a library shipped with the tree)."""
-    lib = in_tree_library()
+def _stamp_matches(lib: str) -> bool:
+    """True when `lib` exists and the digest written beside it at build time is that of the present sources."""
     stamp = lib + ".digest"
-    if os.path.isfile(lib):
-        if not os.path.isfile(stamp):
+    if not (os.path.isfile(lib) and os.path.isfile(stamp)):
+        return False
+    with open(stamp) as fh:
+        return fh.read().strip() == _source_digest()
+
+
+def find_library() -> Optional[str]:
+    """A library built from the present sources: the in-tree one, else the one under the temporary folder (whose
+    folder name carries the digest too).  A library without a digest beside it, or with another one, is stale:
+    None is returned and the caller builds."""
+    for lib in (in_tree_library(), os.path.join(_fallback_dir(), LIB_NAME)):
+        if _stamp_matches(lib):
             return lib
-        with open(stamp) as fh:
-            if fh.read().strip() == _source_digest():
-                return lib
-    fb = os.path.join(_fallback_dir(), LIB_NAME)
-    if os.path.isfile(fb):
-        return fb
     return None
 
 
