@@ -36,6 +36,10 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--preemption-mode", default="recompute", choices=["recompute", "none"])
     ap.add_argument("--chunked-prefill-policy", default="decode-first", choices=["decode-first", "prefill-first"])
     ap.add_argument("--ahead", action="store_true", help="launch a step before the tokens of the step before it are read")
+    ap.add_argument("--warm-up", action="store_true",
+                    help="before the first request: capture the decode graphs of every batch size and run the sampler and prompt portions once")
+    ap.add_argument("--check-layers", type=int, default=0, metavar="STEPS",
+                    help="run every layer of the first STEPS steps also with the plain kernels and print their distance layer by layer")
 
 
 def _make_engine(args, model):
@@ -45,7 +49,8 @@ def _make_engine(args, model):
                   gpu_memory_utilization=args.gpu_memory_utilization, kv_watermark_blocks=args.kv_watermark_blocks,
                   max_num_partial_prefills=args.max_num_partial_prefills,
                   long_prefill_token_threshold=args.long_prefill_token_threshold, preemption_mode=args.preemption_mode,
-                  decode_first=args.chunked_prefill_policy == "decode-first", ahead=args.ahead)
+                  decode_first=args.chunked_prefill_policy == "decode-first", ahead=args.ahead,
+                  check_layers=args.check_layers)
 
 
 def cmd_run(argv: List[str]) -> int:
@@ -70,6 +75,11 @@ def cmd_run(argv: List[str]) -> int:
     if not prompts:
         ap.error("give --prompt-ids or --prompts-file")
     engine = _make_engine(args, args.model)
+    if args.warm_up:
+        started = time.perf_counter()
+        count = engine.warm_up()
+        print(f"warm-up: {count} requests, {len(engine.runner._graphs)} decode graphs in {time.perf_counter() - started:.2f}s",
+              file=sys.stderr)
     stops = tuple(int(t) for t in args.stop_token_ids.split(",") if t.strip())
     params = SamplingParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k, seed=args.seed,
                             max_tokens=args.max_tokens, stop_token_ids=stops, ignore_eos=args.ignore_eos)

@@ -62,7 +62,7 @@ class Engine:
                  gpu_memory_utilization: float = 0.90, decode_first: bool = True, kv_watermark_blocks: int = 0,
                  max_num_partial_prefills: int = 0, long_prefill_token_threshold: int = 0,
                  preemption_mode: str = "recompute", eos_token_ids: Optional[Seq[int]] = None,
-                 random_weights_on_device: bool = False, ops=None, ahead: bool = False):
+                 random_weights_on_device: bool = False, ops=None, ahead: bool = False, check_layers: int = 0):
         """`model`: a folder with config.json and safetensors; or `config` (a config.json dict)
         with `seed` for random weights (drawn on the host, or on the device with a stream of its
         own when `random_weights_on_device`: large models).  Option names follow the reference's server flags
@@ -74,7 +74,10 @@ class Engine:
         (the reference's ahead step, rust/engine/src/rust_decoder.rs:1165-1266): the device takes
         them from the earlier step's output, the host plans the next step while the device runs
         this one, and `step()` returns the events of the step before.  A request that stops at a
-        token (end of sequence, stop id) has one more row in flight by then; that row is dropped."""
+        token (end of sequence, stop id) has one more row in flight by then; that row is dropped.
+
+        `check_layers`: the first so many steps run every layer also with the plain kernels and print, layer by
+        layer, how far the two are apart, the largest value, a checksum and NaN/Inf counts (`runner.check_layers`)."""
         if (model is None) == (config is None):
             raise ValueError("give either a model folder or a config for random weights")
         if model is not None:
@@ -105,6 +108,7 @@ class Engine:
         self._next_seq = 0
         self.ahead = bool(ahead)
         self._in_flight: Optional[_InFlight] = None
+        self.layer_check = self.runner.check_layers(check_layers) if check_layers > 0 else None
 
     # ---- requests -------------------------------------------------------------------------
     def add_request(self, request_id: str, prompt_token_ids: Seq[int], sampling: Optional[SamplingParams] = None) -> int:
@@ -218,6 +222,62 @@ class Engine:
             events.append(TokenEvent(seq.req_id, token, reason is not None, reason))
         self.stats.postprocess_s += time.perf_counter() - t0
         return events
+
+    # ---- before the first request ----------------------------------------------------------
+    def warm_up(self, context_bounds: Optional[Seq[int]] = None) -> int:
+        """Runs a few synthetic requests so that what is built at first use exists before the first real request
+        (rust/engine/src/runtime.rs:1085-1173): the decode graph of every batch size that `max_seqs` sequences can
+        reach, the sampler, prompt portions of 128 to 2,048 tokens; then captures the same graphs for longer
+        contexts (`context_bounds`, by default the powers of two up to the context or 32,768).  Nothing of it
+        stays: every request is finished, the counters are put back.  Returns the number of requests run."""
+        if self.scheduler.has_work() or self._in_flight is not None:
+            return 0
+        from .runner import GRAPH_BUCKETS
+        saved = EngineStats(**vars(self.stats))
+        max_seqs = self.scheduler.cfg.max_num_seqs
+        budget = self.scheduler.cfg.max_num_batched_tokens
+        room = self.max_model_len
+        vocab = self.runner.vocab_size
+        sizes = [b for b in GRAPH_BUCKETS if b <= max_seqs]
+        if max_seqs not in sizes:
+            sizes.append(max_seqs)
+        plan = [(rows, 8, 4, False) for rows in sizes] + [(1, 8, 4, True), (min(max_seqs, 16), 8, 4, True)]
+        plan += [(1, tokens, 1, False) for tokens in (128, 256, 512, 1024, 2048) if tokens + 8 <= room and tokens <= budget]
+        ran = serial = 0
+        for count, prompt_len, new_tokens, sampled in plan:
+            if prompt_len + new_tokens > room:
+                continue
+            names = []
+            for _ in range(count):
+                serial += 1
+                prompt = [(serial * 131 + j * 17) % vocab for j in range(prompt_len)]
+                params = SamplingParams(max_tokens=new_tokens, temperature=0.7 if sampled else 0.0,
+                                        top_p=0.9 if sampled else 1.0, ignore_eos=True, seed=serial)
+                name = f"__warmup_{serial}"
+                self.add_request(name, prompt, params)
+                names.append(name)
+            try:
+                while any(n in self._requests for n in names):
+                    self.step()
+                while self._in_flight is not None:
+                    self.step()
+            except Exception:
+                for n in names:
+                    self.abort_request(n)
+                self._in_flight = None
+                self.stats = saved
+                raise
+            ran += len(names)
+        if context_bounds is None:
+            context_bounds = []
+            bound = 512
+            while bound <= min(room, 32768):
+                context_bounds.append(bound)
+                bound *= 2
+        self.runner.capture_graphs(sizes, context_bounds)
+        self.stats = saved
+        self.scheduler.preemptions = saved.preemptions
+        return ran
 
     # ---- whole requests -------------------------------------------------------------------
     def generate(self, prompts: Seq[Seq[int]], sampling: Union[SamplingParams, Seq[SamplingParams], None] = None

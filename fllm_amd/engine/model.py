@@ -36,6 +36,7 @@ class Model:
         self.final_norm = make("norm", spec.final_norm)
         self.head = make("head", spec.head)
         self.bindings: List[CacheBinding] = []
+        self.layer_check = None          # a diagnostics.LayerCheck while layers are being checked
         self._plan_caches()
 
     # ---- caches ---------------------------------------------------------------------------
@@ -133,8 +134,12 @@ class Model:
         """Logits (float32 [len(logit_rows), vocab]) of the step's wanted rows."""
         x = self.embedding.forward(ctx, ctx.ids)
         pending = None      # a block's output that the next block adds together with its first norm
-        for entry, binding in zip(self.spec.run_order, self.bindings):
+        check = self.layer_check if self.layer_check is not None and self.layer_check.active else None
+        for index, (entry, binding) in enumerate(zip(self.spec.run_order, self.bindings)):
             block = self.blocks[entry.layer]
+            if check is not None:
+                check.run_block(self, block, ctx, x, binding, index, entry.layer)
+                continue
             if getattr(block, "takes_pending", False):
                 pending = block.forward(ctx, x, binding, pending)
             else:
@@ -144,6 +149,8 @@ class Model:
                 block.forward(ctx, x, binding)
         if pending is not None:
             self.rt.ops.add_residual(x, pending)
+        if check is not None:
+            check.end_step()
         if ctx.logit_rows.numel() == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.rt.device)
         h = self.final_norm.forward(ctx, x, rows=ctx.logit_rows)

@@ -155,6 +155,13 @@ class ModelRunner:
                 pages[g] = max(1, min(caps[g], each))
         return pages
 
+    def check_layers(self, steps: int = 2, limit: float = 5e-2, out=None):
+        """Switches the layer-by-layer check on for the next `steps` steps (see `diagnostics.LayerCheck`) and returns
+        the object that collects the reports."""
+        from .diagnostics import LayerCheck
+        self.model.layer_check = LayerCheck(steps, limit, out)
+        return self.model.layer_check
+
     # ---- requests -------------------------------------------------------------------------
     def add_request(self, req_id) -> int:
         return self.cache.add_request(req_id)
@@ -230,7 +237,8 @@ class ModelRunner:
                 if self.cache.length(e.req_id) == 0:
                     self.model.clear_state(self.cache.slot(e.req_id))
         logits = None
-        if self.use_graphs and all(len(e.tokens) == 1 for e in entries) and len(entries) <= GRAPH_BUCKETS[-1]:
+        checking = self.model.layer_check is not None and self.model.layer_check.active     # checked steps run eagerly
+        if not checking and self.use_graphs and all(len(e.tokens) == 1 for e in entries) and len(entries) <= GRAPH_BUCKETS[-1]:
             logits = self._graph_step(entries, previous_tokens)
         if logits is None:
             ctx = self._build_context(entries, previous_tokens)
@@ -297,6 +305,34 @@ class ModelRunner:
             return graph.logits[:count]
         index = torch.tensor(wanted, dtype=torch.long, device=self.device)
         return graph.logits.index_select(0, index)
+
+    def capture_graphs(self, row_counts: Sequence[int], context_bounds: Sequence[int]) -> int:
+        """Captures the decode graphs of these (rows, context bound) pairs before a step needs them (rows are rounded up
+        to buckets, bounds to the powers of two from 256 that graphs are keyed by).  Every row of such a capture is a
+        padding row: nothing is stored.  Returns the number of graphs captured."""
+        if not self.use_graphs:
+            return 0
+        made = 0
+        buckets = sorted({next(b for b in GRAPH_BUCKETS if b >= min(n, GRAPH_BUCKETS[-1])) for n in row_counts if n > 0})
+        bounds = set()
+        for limit in context_bounds:
+            bound = 256
+            while bound < limit:
+                bound *= 2
+            bounds.add(min(bound, self.max_context))
+        for bucket in buckets:
+            for bound in sorted(bounds):
+                if (bucket, bound) in self._graphs:
+                    continue
+                widths = [-(-bound // g.page_size) for g in self.cache.groups]
+                graph = _DecodeGraph(self, bucket, bound, widths)
+                graph.host_np[:] = graph.template
+                graph.device_buf.copy_(graph.host_buf, non_blocking=True)
+                graph.done.record()
+                graph.capture()
+                self._graphs[(bucket, bound)] = graph
+                made += 1
+        return made
 
     def _build_context(self, entries: Sequence[StepEntry], previous_tokens: Optional[torch.Tensor] = None) -> StepContext:
         ids: List[int] = []

@@ -238,3 +238,40 @@ def test_ahead_step_that_fails_keeps_the_step_before_in_flight():
     assert events[-1].finished
     engine.runner.cache.check_invariants()
     assert engine.runner.cache.requests() == []
+
+
+def test_warm_up_leaves_nothing_behind():
+    """Synthetic requests of every batch size run before the first real one; afterwards no request, no page and no
+    count of theirs is left, and generation gives what it gives without a warm-up."""
+    engine = make_engine(max_seqs=4, num_blocks=64)
+    ran = engine.warm_up()
+    assert ran >= 1 + 2 + 4 + 1 + 4                      # batch sizes 1, 2, 4, and the sampled runs
+    assert engine.stats.forward_calls == 0 and engine.stats.rows_total == 0
+    assert not engine.has_unfinished() and engine.runner.cache.requests() == []
+    assert all(p.available == p.num_pages for p in engine.runner.cache.pools)
+    engine.runner.cache.check_invariants()
+    greedy = SamplingParams(max_tokens=8)
+    assert engine.generate(PROMPTS_A, greedy) == make_engine(max_seqs=4, num_blocks=64).generate(PROMPTS_A, greedy)
+    busy = make_engine()
+    busy.add_request("x", PROMPTS_A[0], greedy)
+    assert busy.warm_up() == 0                            # only before the first request
+
+
+def test_layer_check_counts_bad_values_per_layer():
+    import io
+    log = io.StringIO()
+    engine = make_engine(check_layers=1)
+    engine.layer_check.out = log
+    engine.generate([PROMPTS_A[0]], SamplingParams(max_tokens=3))
+    reports = engine.layer_check.reports
+    assert [r.entry for r in reports] == [0, 1] and all(r.step == 0 and r.rows == len(PROMPTS_A[0]) for r in reports)
+    assert all(r.bad_values == 0 and r.distance is None and r.largest > 0 for r in reports)      # one kind of kernel here
+    assert not engine.layer_check.active and log.getvalue().count("[layer-check] step 0") == 2
+    assert "none beyond" in log.getvalue()
+    # a weight that is not a number: the first layer that touches it is named
+    broken = make_engine(check_layers=1)
+    broken.layer_check.out = log
+    broken.runner.model.blocks[1].feed_forward.w_down[3, 5] = float("nan")
+    broken.generate([PROMPTS_A[0]], SamplingParams(max_tokens=1))
+    assert [r.bad_values > 0 for r in broken.layer_check.reports] == [False, True]
+    assert "first suspect: step 0, run entry 1" in log.getvalue()

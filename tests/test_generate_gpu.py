@@ -212,3 +212,57 @@ def test_ahead_stop_token_with_pages_that_change_hands(dtype):
     assert len(handed_out[0]) > len(set(handed_out[0])), "no page changed hands"
     engine.runner.cache.check_invariants()
     assert engine.runner.cache.requests() == []
+
+
+def test_warm_up_captures_the_graphs_before_the_first_request():
+    """After `warm_up` the decode graphs of every batch size up to `max_seqs`, for short and long contexts, exist; the
+    first real requests capture nothing, and their tokens are those of an engine that was not warmed up."""
+    prompts = [tc.random_ids(n, 384, 60 + n) for n in (5, 300, 40)]
+    params = SamplingParams(max_tokens=12)
+    want = make_engine("D", "bfloat16", ctx=1024, num_blocks=256).generate(prompts, params)
+    engine = make_engine("D", "bfloat16", ctx=1024, num_blocks=256)
+    assert engine.warm_up() > 0
+    keys = set(engine.runner._graphs)
+    assert {(rows, bound) for rows in (1, 2, 4) for bound in (256, 512, 1024)} <= keys
+    assert engine.stats.forward_calls == 0 and engine.runner.cache.requests() == []
+    assert engine.generate(prompts, params) == want
+    assert set(engine.runner._graphs) == keys, "a graph was captured after the warm-up"
+    engine.runner.cache.check_invariants()
+
+
+def test_layer_check_names_the_layer_that_goes_wrong():
+    """Every layer of the first steps runs with the plain kernels and with the serving kernels on the same input.
+    Healthy: the two stay within bfloat16 rounding of each other.  With the serving run of one layer's attention
+    disturbed, that layer is the first suspect."""
+    import io
+    prompt = tc.random_ids(40, 384, 77)
+    log = io.StringIO()
+    healthy = make_engine("D", "bfloat16", ctx=1024, num_blocks=64, max_batched_tokens=64, check_layers=3)
+    healthy.layer_check.out = log
+    want = make_engine("D", "bfloat16", ctx=1024, num_blocks=64, max_batched_tokens=64).generate([prompt], SamplingParams(max_tokens=6))
+    assert healthy.generate([prompt], SamplingParams(max_tokens=6)) == want          # the check changes no token
+    reports = healthy.layer_check.reports
+    assert len(reports) == 3 * 2 and [r.rows for r in reports] == [40, 40, 1, 1, 1, 1]
+    assert all(r.distance is not None and r.distance < 2e-2 and r.bad_values == 0 for r in reports), log.getvalue()
+    assert healthy.layer_check.suspects() == [] and healthy.runner.graph_replays > 0   # graphs again once the check is over
+
+    broken = make_engine("D", "bfloat16", ctx=1024, num_blocks=64, max_batched_tokens=64, check_layers=1)
+    broken.layer_check.out = log
+    ops = broken.runner.rt.ops
+    calls = []
+    attention = ops.attention
+
+    def disturbed(*args, **kw):
+        out = attention(*args, **kw)
+        calls.append(1)
+        if len(calls) == 4:                   # layer 0 plain, layer 0 serving, layer 1 plain, layer 1 serving
+            out.mul_(1.5)
+        return out
+
+    ops.attention = disturbed
+    try:
+        broken.generate([prompt], SamplingParams(max_tokens=1))
+    finally:
+        del ops.attention
+    suspects = broken.layer_check.suspects()
+    assert [r.entry for r in suspects] == [1] and "first suspect: step 0, run entry 1" in log.getvalue()
