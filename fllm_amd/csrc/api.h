@@ -16,7 +16,7 @@ int fllm_abi_version(void);
 void fllm_set_fast_kernels(int on);
 // Switches a kernel variant (for measurements and tests): "attention.tile32" 0/1; "linear.slices" n
 // (0: chosen by shape); "linear.dual_k" 0/1; "linear.x_direct" 0/1; "attention.fused_merge" 0/1;
-// "attention.prefill_parts" 0/1.  0 on success.
+// "attention.prefill_parts" 0/1; "linear.slab" 0/1/2.  0 on success.
 int fllm_set_option(const char *name, int value);
 
 // out[r, :] = scale * table[ids[r], :]            out: float32 [rows, width]
@@ -45,7 +45,7 @@ int fllm_linear(const void *x, int ldx, const void *w, const float *bias, void *
 // must not overlap while it is set.  nullptr takes it away.
 int fllm_set_device_workspace(void *workspace, size_t bytes);
 
-// Fused forms for decode steps in bfloat16 (1..16 rows, K a multiple of 8; fllm_fused_decode_supported).
+// Fused forms for decode steps in bfloat16 (1..64 rows, K a multiple of 8; fllm_fused_decode_supported).
 // x is the float32 residual stream [M, K]; each computes rmsnorm(x; norm_w, eps) @ w^T (+ bias) and
 //   fllm_norm_linear          stores it as bfloat16 [M, N]
 //   fllm_norm_gate_up_swiglu  w = [gate; up] ([2 I, K]): stores silu(gate) * up as bfloat16 [M, I]

@@ -25,6 +25,24 @@ namespace {
 // issues every load and no load sits behind a branch.
 __device__ uint4 kZeros = {0u, 0u, 0u, 0u};     // not const: in the same address space as the tensors it stands in for
 
+// Partial sums that workgroups hand to each other go through the device workspace in 16-byte pieces that pass by the
+// caches of the compute units and of their die on both ways (the sc0 sc1 forms of the buffer instructions: written
+// through to memory, read from memory), as device-scope atomics do for single words.  The workspace is one buffer
+// for these instructions; offsets are in bytes from its base.
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
+constexpr int kThroughCaches = 17;        // cache policy bits sc0 (1) and sc1 (16)
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t workspace_buffer(float *base) {
+    return __builtin_amdgcn_make_buffer_rsrc(base, 0, 0x7fffffff, 0x00020000);      // raw buffer, offsets up to 2 GiB
+}
+__device__ __forceinline__ void hand_over(__amdgpu_buffer_rsrc_t ws, unsigned int byte_offset, f32x4_t v) {
+    u32x4_t bits = {__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])};
+    __builtin_amdgcn_raw_buffer_store_b128(bits, ws, byte_offset, 0, kThroughCaches);
+}
+__device__ __forceinline__ f32x4_t take_over(__amdgpu_buffer_rsrc_t ws, unsigned int byte_offset) {
+    const u32x4_t bits = __builtin_amdgcn_raw_buffer_load_b128(ws, byte_offset, 0, kThroughCaches);
+    return (f32x4_t){__uint_as_float(bits[0]), __uint_as_float(bits[1]), __uint_as_float(bits[2]), __uint_as_float(bits[3])};
+}
+
 enum { PRO_BF16 = 0, PRO_NORM_F32 = 1 };
 enum { EPI_STORE = 0, EPI_STORE_F32 = 1, EPI_ADD = 2, EPI_QKV = 3, EPI_SWIGLU = 4 };
 
@@ -51,6 +69,13 @@ struct SkinnyArgs {
     bf16_t *k_pages, *v_pages;
     int heads, kv_heads, head_dim, page_size, store_kv;
 };
+
+__device__ __forceinline__ bf16x4_t pack4(f32x4_t v) {
+    bf16x4_t p;
+#pragma unroll
+    for (int i = 0; i < 4; i++) p[i] = (bf16_t)v[i];
+    return p;
+}
 
 __device__ __forceinline__ bf16x8_t zero8() {
     bf16x8_t z;
@@ -125,8 +150,17 @@ __device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], 
             for (int i = 0; i < 4; i++)
                 if (nb + i < n_out) s[t][i] += a.bias[t * n_out + nb + i];
     }
+    // the four outputs of a lane are neighbours in a row: one store where the row's pitch and the base keep them aligned
+    const bool whole = nb + 3 < n_out && (a.ldo & 3) == 0;
     if (EPI == EPI_ADD && e.have) {
         *(f32x4_t *)((float *)a.out + (size_t)m * a.ldo + nb) = e.resid + s[0];
+    } else if (EPI == EPI_ADD && whole && ((uintptr_t)a.out & 15) == 0) {
+        f32x4_t *dst = (f32x4_t *)((float *)a.out + (size_t)m * a.ldo + nb);
+        *dst = *dst + s[0];
+    } else if (EPI == EPI_STORE && whole && ((uintptr_t)a.out & 7) == 0) {
+        *(bf16x4_t *)((bf16_t *)a.out + (size_t)m * a.ldo + nb) = pack4(s[0]);
+    } else if (EPI == EPI_STORE_F32 && whole && ((uintptr_t)a.out & 15) == 0) {
+        *(f32x4_t *)((float *)a.out + (size_t)m * a.ldo + nb) = s[0];
     } else if (EPI == EPI_STORE || EPI == EPI_STORE_F32 || EPI == EPI_ADD) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -138,12 +172,18 @@ __device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], 
             else ((float *)a.out)[o] += s[0][i];
         }
     } else if (EPI == EPI_SWIGLU) {
+        f32x4_t act;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const int n = nb + i;
-            if (n >= n_out) continue;
             const float gt = s[0][i], up = s[RT - 1][i];
-            ((bf16_t *)a.out)[(size_t)m * a.ldo + n] = (bf16_t)(gt / (1.0f + expf(-gt)) * up);
+            act[i] = gt / (1.0f + expf(-gt)) * up;
+        }
+        if (whole && ((uintptr_t)a.out & 7) == 0) {
+            *(bf16x4_t *)((bf16_t *)a.out + (size_t)m * a.ldo + nb) = pack4(act);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (nb + i < n_out) ((bf16_t *)a.out)[(size_t)m * a.ldo + nb + i] = (bf16_t)act[i];
         }
     } else {   // EPI_QKV: N = (heads + 2 kv_heads) * head_dim, head_dim a multiple of 4, so nb..nb+3 lie in one head
         const int seg = e.seg;
@@ -165,18 +205,27 @@ __device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], 
                 }
             }
         }
+        const f32x4_t v4 = {v[0], v[1], v[2], v[3]};
         if (hd < a.heads) {
             bf16_t *q = (bf16_t *)a.out + (size_t)m * a.ldo + nb;
+            if ((a.ldo & 3) == 0 && ((uintptr_t)a.out & 7) == 0) {
+                *(bf16x4_t *)q = pack4(v4);
+            } else {
 #pragma unroll
-            for (int i = 0; i < 4; i++) q[i] = (bf16_t)v[i];
+                for (int i = 0; i < 4; i++) q[i] = (bf16_t)v[i];
+            }
         } else if (a.store_kv) {
             const int page = e.page;
             const int off = pos % a.page_size;
             if (hd < a.heads + a.kv_heads) {
                 const int kvh = hd - a.heads;
                 bf16_t *kd = a.k_pages + (((size_t)page * a.kv_heads + kvh) * a.page_size + off) * d + j;
+                if (((uintptr_t)a.k_pages & 7) == 0) {      // head_dim and j are multiples of 4
+                    *(bf16x4_t *)kd = pack4(v4);
+                } else {
 #pragma unroll
-                for (int i = 0; i < 4; i++) kd[i] = (bf16_t)v[i];
+                    for (int i = 0; i < 4; i++) kd[i] = (bf16_t)v[i];
+                }
             } else {
                 const int kvh = hd - a.heads - a.kv_heads;
 #pragma unroll
@@ -641,6 +690,287 @@ skinny_wide_kernel(SkinnyArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// 17 to 64 rows: the activations of a K slice stay in LDS, one workgroup a compute unit walks over row groups
+// ---------------------------------------------------------------------------------------------
+// With this many rows the activations weigh as much as the weights a workgroup streams past them, so they must not
+// be fetched again for every weight tile.  A workgroup of 8 waves stages ONE K slice of all rows in LDS (up to 1,024
+// columns of 64 rows: 132 KiB; for the norm prologue x * norm_weight as bfloat16, and the slice's part of every row's
+// sum of squares) and keeps it for the whole launch.  It then walks over row groups of 8 weight tiles, one tile a
+// wave (16 weight rows, or 8 gate and 8 up rows), each wave over the whole slice: the weights go from global
+// memory straight into MFMA A operands, two chunks of 256 columns (16 KiB a wave) in flight ahead of the products;
+// the B operands come from LDS.  No wave waits for another after the staging.  Workgroup b owns slice b % S and the
+// row groups b / S, b / S + G / S, ...  With S > 1 a wave leaves its tile's sums (and the slice's sums of squares)
+// in the workspace and counts the tile; the wave that counts the last slice adds the S parts in slice order and
+// runs the epilogue, so the result does not depend on who came last.
+template <int PRO, int EPI, int MT>
+__global__ void __launch_bounds__(8 * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
+skinny_slab_kernel(SkinnyArgs a, int cells_off) {
+    constexpr int WAVES = 8, THREADS = WAVES * kWave;
+    constexpr int KC = 256;                        // columns per chunk of weights
+    constexpr int KS = KC / 32;                    // MFMA k-steps per chunk
+    constexpr int ROWS = MT * 16;
+    constexpr int NT = EPI == EPI_SWIGLU ? 8 : 16; // outputs per row and tile
+    constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int r = lane & 15, g = lane >> 4;
+    const int M = a.M, N = a.N, K = a.K, S = a.S;
+    const int n_out = EPI == EPI_SWIGLU ? N / 2 : N;
+    const int ntiles = (n_out + NT - 1) / NT;
+    const int ngroups = (ntiles + WAVES - 1) / WAVES;
+    const int sl = blockIdx.x % S;
+    const int rg0 = blockIdx.x / S, rstride = gridDim.x / S;
+    const int ks0 = sl * a.slice;
+    const int kcn = min(K, ks0 + a.slice) - ks0;                  // columns of this slice, a multiple of 8
+    const int nchunks = (kcn + KC - 1) / KC;
+    const int my_items = rg0 < ngroups ? (ngroups - rg0 + rstride - 1) / rstride : 0;
+    const int total = my_items * nchunks;                         // chunk steps of every wave of this workgroup
+    const int pitch = a.slice + 8;
+    bf16_t *xs = (bf16_t *)smem;                                  // [ROWS][pitch]; columns from kcn on and rows from M on are zero
+    float *cells = (float *)(smem + cells_off);                   // norm prologue: [ROWS][slice / 512] sums of squares
+    const int cpr = a.slice / 8;                                  // 16-byte pieces of a staged row
+    const int cells_per_row = (a.slice + 511) / 512;
+
+    // weights: cursor (item, chunk) of the next chunk to ask for.  Every lane issues every load (zeros where it has
+    // nothing of its own), so no load sits behind a branch and the chunks behind the current one stay in flight.
+    int w_item = 0, w_chunk = 0;
+    // Every wave walks the chunks of its slice in a circle, starting at a chunk of its own: at any moment the waves of
+    // the device then read different columns, which lie in different memory channels (all waves at the same columns
+    // of rows that are a power of two apart would crowd into a few channels).
+    const int phase = (wave + rg0) % nchunks;
+    const bf16_t *zeros = (const bf16_t *)&kZeros;
+    auto issue_w = [&](bf16x8_t (&buf)[KS]) __attribute__((always_inline)) {
+        const bool live = w_item < my_items;
+        const int tile = (rg0 + (live ? w_item : 0) * rstride) * WAVES + wave;
+        int row = tile * NT + (EPI == EPI_SWIGLU ? (r & 7) : r);
+        if (row >= n_out) row = n_out - 1;    // past the end: computed from a valid row, never stored
+        if (EPI == EPI_SWIGLU) row += (r >> 3) * n_out;
+        const int kb = ((w_chunk + phase) % nchunks) * KC + g * 8;
+        const bf16_t *wp = a.w + (size_t)row * K + ks0;
+#pragma unroll
+        for (int u = 0; u < KS; u++) buf[u] = *(const bf16x8_t *)(live ? wp + min(kb + u * 32, kcn - 8) : zeros);
+        if (++w_chunk == nchunks) w_chunk = 0, w_item++;
+    };
+    bf16x8_t wa[KS], wb[KS];
+    issue_w(wa);      // in flight while the activations are staged
+    issue_w(wb);
+
+    // ---- staging: piece idx of the slice is (row idx / cpr, columns (idx % cpr) * 8 ...) ----
+    if (PRO == PRO_BF16) {
+        const bf16_t *x = (const bf16_t *)a.x;
+        constexpr int B = 8;       // loads in flight a thread
+        for (int i0 = threadIdx.x; i0 < ROWS * cpr; i0 += B * THREADS) {
+            bf16x8_t v[B];
+#pragma unroll
+            for (int i = 0; i < B; i++) {
+                const int idx = i0 + i * THREADS;
+                const int m = idx / cpr, c = (idx - m * cpr) * 8;
+                v[i] = *(const bf16x8_t *)((idx < ROWS * cpr && m < M && c < kcn) ? x + (size_t)m * a.ldx + ks0 + c : zeros);
+            }
+#pragma unroll
+            for (int i = 0; i < B; i++) {
+                const int idx = i0 + i * THREADS;
+                const int m = idx / cpr, c = (idx - m * cpr) * 8;
+                if (idx < ROWS * cpr) *(bf16x8_t *)(xs + m * pitch + c) = v[i];
+            }
+        }
+    } else {
+        // A wave covers 512 consecutive columns of one row at a time (the slice is a multiple of 512 columns), so one
+        // cell holds the squares of exactly one wave's trip: every cell is written once, and a row's sum is the sum of
+        // its cells in order.
+        const float *x = (const float *)a.x;
+        constexpr int B = 4;
+        for (int i0 = threadIdx.x; i0 < ROWS * cpr; i0 += B * THREADS) {
+            f32x4_t xv[B][2], nw[B][2];
+#pragma unroll
+            for (int i = 0; i < B; i++) {
+                const int idx = i0 + i * THREADS;
+                const int m = idx / cpr, c = (idx - m * cpr) * 8;
+                const bool in = idx < ROWS * cpr && m < M && c < kcn;
+                const float *src = in ? x + (size_t)m * a.ldx + ks0 + c : (const float *)zeros;
+                const float *wsrc = in ? a.norm_w + ks0 + c : (const float *)zeros;
+                xv[i][0] = *(const f32x4_t *)src;
+                xv[i][1] = in ? *(const f32x4_t *)(src + 4) : (f32x4_t){0.f, 0.f, 0.f, 0.f};
+                nw[i][0] = *(const f32x4_t *)wsrc;
+                nw[i][1] = in ? *(const f32x4_t *)(wsrc + 4) : (f32x4_t){0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int i = 0; i < B; i++) {
+                const int idx = i0 + i * THREADS;     // the same for all lanes of a wave up to the lane index: no lane leaves the loop early
+                const int m = idx / cpr, c = (idx - m * cpr) * 8;
+                bf16x8_t v;
+                float ss = 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    ss += xv[i][0][e] * xv[i][0][e] + xv[i][1][e] * xv[i][1][e];
+                    v[e] = (bf16_t)(xv[i][0][e] * nw[i][0][e]);
+                    v[4 + e] = (bf16_t)(xv[i][1][e] * nw[i][1][e]);
+                }
+                if (idx < ROWS * cpr) *(bf16x8_t *)(xs + m * pitch + c) = v;
+                ss = wave_sum(ss);
+                if (lane == 0 && idx < ROWS * cpr) cells[m * cells_per_row + c / 512] = ss;
+            }
+        }
+    }
+    __syncthreads();
+
+    f32x4_t acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) acc[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    int item = 0, chunk = 0;
+    const bf16_t *xb = xs + r * pitch + g * 8;
+
+    // ---- what happens to a finished tile ----
+    // One slice (S == 1): the wave runs the epilogue.  Several: the wave leaves its sums and its slice's sums of
+    // squares in the workspace, counts the tile, and whoever counts last adds the S parts in slice order and runs
+    // the epilogue.  None of this may make the wave wait, or the weights stop streaming, so it is spread over three
+    // item ends: the parts are sent at the end of their own item; the tile is counted at the end of the item after,
+    // when the loads that were asked for since have pushed the parts' stores out of the queue of outstanding memory
+    // operations (they complete in the order of their issue, so waiting until only the newest loads are outstanding
+    // is waiting for nothing that is not needed anyway); the count is looked at one item later still.
+    const bool owner = EPI == EPI_SWIGLU ? g < 2 : true;      // 8-output tiles: lanes g < 2 hold gate rows, g >= 2 the up rows
+    const __amdgpu_buffer_rsrc_t wsb = workspace_buffer(a.ws);
+    int sent_tile = -1;                     // parts sent, tile not counted yet
+    int counted_tile = -1, counted_raw = 0; // tile counted; lane 0 holds what the counter said, not looked at yet
+
+    // the epilogue of one 16-row block of a tile
+    auto finish_rows = [&](int tile, int mt, f32x4_t (&s)[RT], float ss) __attribute__((always_inline)) {
+        const int nb = tile * NT + g * 4;
+        const int m = mt * 16 + r;
+        if (!owner || m >= M || nb >= n_out) return;
+        EpilogueOperands eo;
+        load_row_operands<EPI>(a, m, eo);
+        load_item_operands<EPI>(a, m, nb, n_out, eo);
+        epilogue<PRO, EPI, RT>(a, s, ss, m, nb, n_out, eo);
+    };
+    auto look = [&]() __attribute__((always_inline)) {
+        if (counted_tile < 0) return;
+        const int tile = counted_tile;
+        counted_tile = -1;
+        if (__shfl(counted_raw, 0, kWave) != S - 1) return;      // another workgroup finishes this tile
+        asm volatile("" ::: "memory");
+        if (lane == 0) __hip_atomic_store(a.counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+        // one block of 16 rows after the other (few registers: this runs in the middle of the stream of weights); the
+        // parts of two slices are asked for before the first is added, and they are added in slice order
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            const bool mine = owner && mt * 16 + r < M;
+            f32x4_t s[RT];
+#pragma unroll
+            for (int t = 0; t < RT; t++) s[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+            float ss = 0.f;
+            for (int s0 = 0; s0 < S; s0 += 2) {
+                f32x4_t pv[2][RT];
+                float ps[2];
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const bool live = s0 + j < S;
+                    const size_t at = (size_t)tile * S + (live ? s0 + j : s0);
+                    const unsigned int src = (unsigned int)(((at * MT + mt) * RT * kWave + lane) * 16);
+#pragma unroll
+                    for (int t = 0; t < RT; t++) {
+                        const f32x4_t got = take_over(wsb, src + t * kWave * 16);     // every lane loads: no load behind a branch
+                        pv[j][t] = (live && mine) ? got : (f32x4_t){0.f, 0.f, 0.f, 0.f};
+                    }
+                    ps[j] = 0.f;
+                    if (PRO == PRO_NORM_F32) {
+                        const float got = __hip_atomic_load(a.ws_ssq + at * ROWS + mt * 16 + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        ps[j] = live ? got : 0.f;
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+#pragma unroll
+                    for (int t = 0; t < RT; t++) s[t] += pv[j][t];
+                    ss += ps[j];
+                }
+            }
+            finish_rows(tile, mt, s, ss);
+        }
+    };
+    // `drained`: nothing more will be asked for, wait for everything; otherwise wait until only the loads that the
+    // item just finished asked for are outstanding (8 a chunk, up to two chunks): the parts were sent before them.
+    auto count = [&](bool drained) __attribute__((always_inline)) {
+        if (sent_tile < 0) return;
+        if (drained) __builtin_amdgcn_s_waitcnt(0);
+        else if (nchunks >= 2) __builtin_amdgcn_s_waitcnt(0x4F70);      // vmcnt(16), nothing else waited for
+        else __builtin_amdgcn_s_waitcnt(0x0F78);                        // vmcnt(8)
+        asm volatile("" ::: "memory");
+        if (lane == 0) counted_raw = __hip_atomic_fetch_add(a.counters + sent_tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        counted_tile = sent_tile;
+        sent_tile = -1;
+    };
+
+    auto step = [&](bf16x8_t (&buf)[KS]) __attribute__((always_inline)) {
+        const bf16_t *xc = xb + ((chunk + phase) % nchunks) * KC;
+#pragma unroll
+        for (int u = 0; u < KS; u++) {
+            bf16x8_t xf[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) xf[mt] = *(const bf16x8_t *)(xc + mt * 16 * pitch + u * 32);
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(buf[u], xf[mt], acc[mt], 0, 0, 0);
+        }
+        issue_w(buf);      // the chunk two ahead takes this one's registers
+        if (++chunk < nchunks) return;
+        chunk = 0;
+        if (item >= my_items) return;      // (a step behind the last item multiplied zeros and ends nothing)
+        // the item is complete: this wave's tile has its sums over the slice
+        const int tile = (rg0 + item * rstride) * WAVES + wave;
+        item++;
+        if (S > 1) {
+            look();
+            count(false);
+        }
+        f32x4_t s[MT][RT];
+        float ss[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            s[mt][0] = acc[mt];
+            if (EPI == EPI_SWIGLU) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) s[mt][RT - 1][i] = __shfl(acc[mt][i], (lane + 32) & 63, kWave);
+            }
+            acc[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+            ss[mt] = 0.f;
+            if (PRO == PRO_NORM_F32) {
+                for (int c = 0; c < cells_per_row; c++) ss[mt] += cells[(mt * 16 + r) * cells_per_row + c];
+            }
+        }
+        if (tile >= ntiles) return;        // wave-uniform: a wave without a tile in the last row group
+        if (S == 1) {
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) finish_rows(tile, mt, s[mt], ss[mt]);
+            return;
+        }
+        // a tile's part of a slice: [mt][t][lane] pieces of 16 bytes; offsets in bytes from the start of the partial sums
+        const unsigned int part = (unsigned int)((((size_t)tile * S + sl) * MT * RT * kWave + lane) * 16);
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            if (!owner || mt * 16 + r >= M) continue;
+#pragma unroll
+            for (int t = 0; t < RT; t++) hand_over(wsb, part + (mt * RT + t) * kWave * 16, s[mt][t]);
+            if (PRO == PRO_NORM_F32 && g == 0)
+                __hip_atomic_store(a.ws_ssq + ((size_t)tile * S + sl) * ROWS + mt * 16 + r, ss[mt], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        sent_tile = tile;
+    };
+
+    // The two buffers take turns without a condition between them (an odd number of steps gets one more, which
+    // multiplies zeros): only then does the compiler see that the loads of one buffer always lie behind those of
+    // the other, and lets them stay in flight.
+    for (int q = 0; q < total; q += 2) {
+        step(wa);
+        step(wb);
+    }
+    if (S > 1) {       // what the last items left to do
+        look();
+        count(true);
+        look();
+    }
+}
+
 int device_cus() {
     static int cus = 0;
     if (cus == 0) {
@@ -812,6 +1142,89 @@ int launch_wide(SkinnyArgs a, hipStream_t stream) {
     return fllm_check_launch("linear_wide");
 }
 
+// What a launch of the slab kernel looks like: the K slice that a workgroup stages and the grid.
+struct SlabPlan {
+    int S = 0, slice = 0, grid = 0;
+    size_t smem = 0, cells_off = 0;
+};
+
+// The slice length (256 to 1,024 columns; multiples of 512 for the norm prologue, whose sums of squares are kept per
+// 512 columns) that costs a workgroup the fewest bytes: its items' weights, its staged slice, and its share of the
+// partial sums that slices cost.  S == 0: nothing fits (no workspace for the slices, or too many tiles to count).
+SlabPlan plan_slab(int M, int n_tiles, int K, int mt, int rt, bool norm, int nt, size_t ws_bytes, bool have_ws, int cus) {
+    SlabPlan best;
+    double best_cost = 0.0;
+    const int rows = mt * 16;
+    const int ngroups = (n_tiles + 7) / 8;
+    const int forced = fllm_option_linear_slices();
+    for (int slice = 1024; slice >= 256; slice -= 256) {
+        if (norm && slice % 512 != 0) continue;
+        int S = (K + slice - 1) / slice;
+        int len = slice;
+        if (S == 1) len = (K + (norm ? 511 : 255)) / (norm ? 512 : 256) * (norm ? 512 : 256);   // one slice: no longer than K needs
+        if (forced > 0 && S != forced && !(S == 1 && forced == 1)) continue;
+        SlabPlan p;
+        p.S = S;
+        p.slice = len;
+        p.cells_off = ((size_t)rows * (len + 8) * sizeof(bf16_t) + 15) / 16 * 16;
+        p.smem = p.cells_off + (norm ? (size_t)rows * ((len + 511) / 512) * sizeof(float) : 0);
+        if (p.smem > 160 * 1024) continue;
+        if (S > 1) {
+            const size_t need = kWorkspaceCounterBytes + (size_t)n_tiles * S * ((size_t)mt * rt * kWave * 4 + rows) * sizeof(float);
+            if (!have_ws || need > ws_bytes || (size_t)n_tiles * sizeof(int) > kWorkspaceCounterBytes) continue;
+        }
+        int per_slice = cus / S;
+        if (per_slice < 1) per_slice = 1;
+        if (per_slice > ngroups) per_slice = ngroups;
+        p.grid = per_slice * S;
+        const int items = (ngroups + per_slice - 1) / per_slice;
+        const double weights = (double)items * 8 * (rt * nt) * len * 2.0;
+        const double staged = (double)rows * len * (norm ? 4.0 : 2.0);
+        const double parts = S > 1 ? (double)items * 8 * (double)M * rt * nt * 4.0 * 2.0 : 0.0;   // written, and read again by somebody
+        const double cost = weights + staged + parts;
+        if (best.S == 0 || cost < best_cost) best = p, best_cost = cost;
+        if (S == 1) break;      // shorter slices of a K that fits in one gain nothing
+    }
+    return best;
+}
+
+template <int PRO, int EPI, int MT>
+int launch_slab(SkinnyArgs a, hipStream_t stream) {
+    constexpr int NT = EPI == EPI_SWIGLU ? 8 : 16;
+    constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
+    const int n_out = EPI == EPI_SWIGLU ? a.N / 2 : a.N;
+    const int ntiles = (n_out + NT - 1) / NT;
+    void *base = nullptr;
+    size_t bytes = 0;
+    const bool have_ws = fllm_device_workspace(&base, &bytes);
+    const SlabPlan p = plan_slab(a.M, ntiles, a.K, MT, RT, PRO == PRO_NORM_F32, NT, bytes, have_ws, device_cus());
+    if (p.S == 0) return 1;
+    a.S = p.S;
+    a.slice = p.slice;
+    if (p.S > 1) {
+        a.counters = (int *)base;
+        a.ws = (float *)((unsigned char *)base + kWorkspaceCounterBytes);
+        a.ws_ssq = a.ws + (size_t)ntiles * p.S * MT * RT * kWave * 4;
+    }
+    static bool attribute_set = false;   // more than the default 64 KiB of dynamic LDS has to be asked for once
+    if (!attribute_set) {
+        const hipError_t e = hipFuncSetAttribute((const void *)skinny_slab_kernel<PRO, EPI, MT>,
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        FLLM_REQUIRE(e == hipSuccess, "linear_skinny: cannot raise the LDS limit: %s", hipGetErrorString(e));
+        attribute_set = true;
+    }
+    hipLaunchKernelGGL((skinny_slab_kernel<PRO, EPI, MT>), dim3(p.grid), dim3(8 * kWave), p.smem, stream, a, (int)p.cells_off);
+    return fllm_check_launch("linear_slab");
+}
+
+template <int PRO, int EPI>
+int dispatch_slab(const SkinnyArgs &a, hipStream_t stream) {
+    const int mt = (a.M + 15) / 16;
+    if (mt == 2) return launch_slab<PRO, EPI, 2>(a, stream);
+    if (mt == 3) return launch_slab<PRO, EPI, 3>(a, stream);
+    return launch_slab<PRO, EPI, 4>(a, stream);
+}
+
 template <int EPI>
 int dispatch_wide(const SkinnyArgs &a, hipStream_t stream) {
     const int mt = (a.M + 15) / 16;
@@ -824,10 +1237,21 @@ template <int PRO, int EPI>
 int dispatch(const SkinnyArgs &a, hipStream_t stream) {
     const int mt = (a.M + 15) / 16;
     if (mt == 1) return launch_resident<PRO, EPI>(a, stream);
-    if constexpr (PRO == PRO_BF16 && (EPI == EPI_STORE || EPI == EPI_STORE_F32 || EPI == EPI_ADD || EPI == EPI_SWIGLU)) {
-        return dispatch_wide<EPI>(a, stream);
+    // Two kernels serve 17 to 64 rows.  The slab kernel (a K slice of the activations resident in LDS, partial sums
+    // handed over between workgroups) wins where a matrix has few rows, so that row groups alone would not fill the
+    // device (output and down projections: 20 against 32 us and 42 against 51 us at 64 rows of the 8B sizes), and it has
+    // the forms with a norm prologue and the q/k/v epilogue.  The chunk kernel wins on matrices of many rows (gate/up:
+    // 58 against 69 us), where slices only cost.  "linear.slab" 0 / 2 force one of them where both can serve.
+    constexpr bool kChunkCan = PRO == PRO_BF16 && (EPI == EPI_STORE || EPI == EPI_STORE_F32 || EPI == EPI_ADD || EPI == EPI_SWIGLU);
+    const int n_out = EPI == EPI_SWIGLU ? a.N / 2 : a.N;
+    const int pick = fllm_option_slab();
+    const bool slab_first = !kChunkCan || pick == 2 || (pick == 1 && n_out <= 8192);
+    if (slab_first) {
+        const int rc = dispatch_slab<PRO, EPI>(a, stream);
+        if (rc != 1) return rc;
     }
-    return 1;   // the forms with a norm prologue are for up to 16 rows
+    if constexpr (kChunkCan) return dispatch_wide<EPI>(a, stream);
+    return 1;   // the forms with a norm prologue and the q/k/v epilogue need the slab kernel from 17 rows on
 }
 
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
@@ -855,12 +1279,12 @@ int fllm_linear_bf16_skinny(const void *x, int ldx, const void *w, const float *
 
 // The fused forms read the float32 rows once per workgroup: worth it while there are few rows.
 extern "C" int fllm_fused_decode_supported(int M, int K) {
-    return (M >= 1 && M <= 16 && K % 8 == 0 && K >= 8 && K <= 65536) ? 1 : 0;
+    return (M >= 1 && M <= 64 && K % 8 == 0 && K >= 8 && K <= 65536) ? 1 : 0;
 }
 
 extern "C" int fllm_norm_linear(const float *x, const float *norm_w, float eps, const void *w, const float *bias, void *out,
                                 int M, int N, int K, hipStream_t stream) {
-    FLLM_REQUIRE(fllm_fused_decode_supported(M, K), "norm_linear: takes 1..16 rows and K a multiple of 8 (M=%d K=%d)", M, K);
+    FLLM_REQUIRE(fllm_fused_decode_supported(M, K), "norm_linear: takes 1..64 rows and K a multiple of 8 (M=%d K=%d)", M, K);
     FLLM_REQUIRE(aligned16(x) && aligned16(w) && aligned16(norm_w), "norm_linear: operands must be 16-byte aligned");
     FLLM_REQUIRE(eps > 0.f, "norm_linear: eps must be positive");
     SkinnyArgs a = {};
@@ -882,7 +1306,7 @@ extern "C" int fllm_norm_linear(const float *x, const float *norm_w, float eps, 
 
 extern "C" int fllm_norm_gate_up_swiglu(const float *x, const float *norm_w, float eps, const void *w_gate_up,
                                         const float *bias, void *out, int M, int inter, int K, hipStream_t stream) {
-    FLLM_REQUIRE(fllm_fused_decode_supported(M, K), "norm_gate_up_swiglu: takes 1..16 rows and K a multiple of 8 (M=%d K=%d)", M, K);
+    FLLM_REQUIRE(fllm_fused_decode_supported(M, K), "norm_gate_up_swiglu: takes 1..64 rows and K a multiple of 8 (M=%d K=%d)", M, K);
     FLLM_REQUIRE(aligned16(x) && aligned16(w_gate_up) && aligned16(norm_w), "norm_gate_up_swiglu: operands must be 16-byte aligned");
     FLLM_REQUIRE(eps > 0.f && inter > 0, "norm_gate_up_swiglu: bad eps or size");
     SkinnyArgs a = {};
@@ -927,7 +1351,7 @@ extern "C" int fllm_norm_qkv_rope_store(const float *x, const float *norm_w, flo
                                         int table_stride, const float *cos_table, const float *sin_table, int rope_dims,
                                         void *k_pages, void *v_pages, int M, int heads, int kv_heads, int head_dim, int K,
                                         int page_size, int store_kv, hipStream_t stream) {
-    FLLM_REQUIRE(fllm_fused_decode_supported(M, K), "norm_qkv_rope_store: takes 1..16 rows and K a multiple of 8 (M=%d K=%d)", M, K);
+    FLLM_REQUIRE(fllm_fused_decode_supported(M, K), "norm_qkv_rope_store: takes 1..64 rows and K a multiple of 8 (M=%d K=%d)", M, K);
     FLLM_REQUIRE(aligned16(x) && aligned16(w_qkv) && aligned16(norm_w), "norm_qkv_rope_store: operands must be 16-byte aligned");
     FLLM_REQUIRE(head_dim % 4 == 0 && rope_dims % 2 == 0 && rope_dims <= head_dim && rope_dims >= 0,
                  "norm_qkv_rope_store: head_dim %d must be a multiple of 4 and rope_dims %d even and no larger", head_dim, rope_dims);

@@ -119,16 +119,19 @@ def _dense(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
 class Ops:
     """Launches kernels on the current torch stream of the tensors' device.
 
-    `library_gemm_from`: bfloat16 products of at least this many rows (prompt portions, large
-    decode batches) go to the vendor's GEMM library through `torch.matmul`, as the reference sends
-    its prompt-sized dense products to a library (rust/engine/cuda/cublaslt_gemm.cu:1-20).  None:
-    every product runs the hand-written kernels."""
+    `library_gemm_from`: bfloat16 products of at least this many rows (prompt portions, large decode batches) go
+    to the vendor's GEMM library through `torch.matmul`, as the reference sends its prompt-sized dense products
+    to a library (rust/engine/cuda/cublaslt_gemm.cu:1-20).  None: every product runs the hand-written kernels.
+    `fused_decode_rows`: up to this many rows a step uses the kernels that fold the norm, rotary, cache store and
+    activation into the product (the kernels take up to 64 rows; beyond 16 the library products with separate small
+    kernels are faster at the sizes measured)."""
 
-    def __init__(self, library_gemm_from: Optional[int] = 17):
+    def __init__(self, library_gemm_from: Optional[int] = 17, fused_decode_rows: int = 16):
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible: the engine runs on gfx950 only")
         self.lib = load_library()
         self.library_gemm_from = library_gemm_from
+        self.fused_decode_rows = int(fused_decode_rows)
         self._device_workspace(torch.cuda.current_device())
 
     _WORKSPACE_BYTES = 192 << 20
@@ -234,8 +237,13 @@ class Ops:
                                          mode, self._stream()))
         return out
 
-    # ---- fused forms of decode steps (bfloat16, at most 16 rows) ---------------------------------
+    # ---- fused forms of decode steps (bfloat16, at most 64 rows) ---------------------------------
     def fused_decode_supported(self, rows: int, width: int) -> bool:
+        """Whether a step of `rows` rows should take the fused forms: the kernels can (1..64 rows, widths in steps of 8)
+        and `fused_decode_rows` lets them."""
+        return rows <= self.fused_decode_rows and self._fused_kernels_take(rows, width)
+
+    def _fused_kernels_take(self, rows: int, width: int) -> bool:
         return bool(self.lib.fllm_fused_decode_supported(int(rows), int(width)))
 
     def _fused_operands(self, x, norm_weight, w, bias, n_rows_w):
@@ -245,7 +253,7 @@ class Ops:
         _dense(w, "w", torch.bfloat16, (n_rows_w, K))
         if bias is not None:
             _dense(bias, "bias", torch.float32, (n_rows_w,))
-        _need(self.fused_decode_supported(M, K), f"the fused decode kernels take 1..16 rows and widths in steps of 8, not {M} x {K}")
+        _need(self._fused_kernels_take(M, K), f"the fused decode kernels take 1..64 rows and widths in steps of 8, not {M} x {K}")
         return M, K
 
     def norm_linear(self, x, norm_weight, eps, w, out, bias=None):

@@ -148,8 +148,9 @@ SKINNY = [(1, 16, 64), (1, 4096, 4096), (2, 100, 136), (5, 6144, 4096), (8, 4096
           (17, 128, 128), (33, 1000, 4096), (64, 4096, 4096), (48, 30, 72),
           # 8-row weight tiles with two K halves (up to 8 rows, 4,100 to 16,000 outputs), ragged in N and K
           (3, 5001, 64), (7, 6148, 200), (8, 4104, 1096), (1, 9000, 520),
-          # 17 to 64 rows: four waves a workgroup, activations through LDS in chunks, K slices over workgroups
+          # 17 to 64 rows: a K slice of the activations stays in LDS, a workgroup a compute unit, K slices over workgroups
           (20, 4096, 14336), (64, 6144, 4096), (40, 100, 264), (33, 5001, 72), (64, 48, 8192), (18, 28672, 512),
+          (64, 4096, 14336), (64, 28672, 4096), (64, 4096, 8192), (64, 8200, 1000), (17, 16, 24), (50, 1000, 2072),
           # K in slices over workgroups (the rows of all of K do not fit into LDS), 8 and 16 waves
           (16, 136, 14336), (5, 1000, 30008), (12, 72, 65536)]
 TILED = [(65, 128, 64), (128, 200, 200), (200, 6144, 4096), (300, 130, 136), (2048, 512, 4096), (129, 4096, 14336)]
@@ -182,7 +183,9 @@ def test_add_residual(ops, dtype, rows, width):
     (8, 6144, 4096, "linear.dual_k", (0, 1)), (3, 5001, 200, "linear.dual_k", (0, 1)),
     (8, 4096, 14336, "linear.x_direct", (0, 1)), (16, 1000, 520, "linear.x_direct", (0, 1)), (3, 5001, 200, "linear.x_direct", (0, 1)),
     (8, 4096, 14336, "linear.slices", (0, 2, 4, 8)), (2, 1000, 4096, "linear.slices", (0, 2, 4)),
-    (16, 264, 8192, "linear.slices", (0, 4)), (64, 4096, 14336, "linear.slices", (0, 1, 2, 4, 8)), (40, 1000, 4096, "linear.slices", (0, 1, 2))])
+    (16, 264, 8192, "linear.slices", (0, 4)), (64, 4096, 14336, "linear.slices", (0, 1, 2, 4, 8, 14, 19)), (40, 1000, 4096, "linear.slices", (0, 1, 2, 4, 6)),
+    (64, 4096, 14336, "linear.slab", (0, 1, 2)), (33, 5001, 72, "linear.slab", (0, 2)), (48, 6144, 4096, "linear.slab", (0, 2)),
+    (64, 28672, 4096, "linear.slab", (0, 2)), (20, 128256, 1024, "linear.slab", (0, 2))])
 def test_linear_bf16_variants_agree(ops, ref, M, N, K, option, values):
     """The ways of cutting a decode-shaped product (tile shape, K slices) give the same sums up to the order
     of float32 additions, each of them the same bits on every call."""
@@ -238,7 +241,9 @@ def test_linear_bf16_strided_input(ops, ref):
 
 # ---- fused forms of decode steps ----------------------------------------------------------------
 FUSED_SHAPES = [(1, 4096, 4096), (1, 64, 136), (8, 6144, 4096), (5, 100, 72), (16, 520, 264), (13, 128, 128), (2, 1000, 4096),
-                (16, 4096, 4096), (9, 96, 14336), (3, 256, 20000), (16, 48, 40000)]
+                (16, 4096, 4096), (9, 96, 14336), (3, 256, 20000), (16, 48, 40000),
+                # 17 to 64 rows: the slab kernel with the norm folded in
+                (17, 128, 128), (64, 6144, 4096), (33, 1000, 4096), (40, 100, 264), (64, 4096, 14336), (24, 96, 1000), (64, 520, 8192)]
 
 
 def _fused_inputs(M, K, seed):
@@ -261,7 +266,8 @@ def test_norm_linear(ops, ref, M, N, K, bias):
     close(got, want, 2 * BF16_EPS, 3e-2, f"norm_linear M{M} N{N} K{K}")
 
 
-@pytest.mark.parametrize("M,inter,K", [(1, 14336, 4096), (1, 176, 64), (8, 432, 160), (13, 1000, 4096), (16, 200, 96), (4, 512, 36000)])
+@pytest.mark.parametrize("M,inter,K", [(1, 14336, 4096), (1, 176, 64), (8, 432, 160), (13, 1000, 4096), (16, 200, 96), (4, 512, 36000),
+                                       (17, 14336, 4096), (64, 176, 64), (40, 432, 160), (33, 1000, 4096), (64, 100, 8192), (64, 14336, 4096)])
 def test_norm_gate_up_swiglu(ops, ref, M, inter, K):
     g, x, nw = _fused_inputs(M, K, 31)
     w = (torch.randn(2 * inter, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
@@ -289,7 +295,8 @@ def test_gate_up_swiglu(ops, ref, M, inter, K):
 @pytest.mark.parametrize("heads,kv_heads,head_dim,rope_dims,page_size,K", [(4, 2, 16, 16, 16, 64), (5, 1, 32, 32, 8, 160),
                                                                            (6, 3, 48, 24, 16, 96), (32, 8, 128, 128, 16, 4096),
                                                                            (2, 2, 16, 0, 16, 64)])
-@pytest.mark.parametrize("segs", [[(0, 1)], [(14, 1), (15, 1), (16, 1), (100, 1), (7, 1)], [(5, 3), (40, 2), (127, 1)]])
+@pytest.mark.parametrize("segs", [[(0, 1)], [(14, 1), (15, 1), (16, 1), (100, 1), (7, 1)], [(5, 3), (40, 2), (127, 1)],
+                                  [(3, 17)], [(0, 40), (100, 20)], [(i, 1) for i in range(60, 124)]])
 def test_norm_qkv_rope_store(ops, ref, heads, kv_heads, head_dim, rope_dims, page_size, K, segs):
     g, _, _ = _fused_inputs(1, 8, 32)
     rows = sum(n for _, n in segs)
