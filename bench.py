@@ -2,14 +2,17 @@
 """Decode and prefill throughput of the engine on one MI355X, Llama-3.1-8B sizes, random bfloat16
 weights, synthetic token ids.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers N] [--shape 8b|1b|70b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers N] [--shape 8b|1b|70b] [--no-further]
 
 A step is one decode step of the whole engine (scheduler, step function, sampling), with steps
 launched ahead of the tokens of the step before them (--no-ahead: each step waits for the last).  The one
 JSON line on standard output holds decoded tokens per second at the default batch (8), the same
 at batch 1 and 64 under "points", a 2,048-token prefill under "prefill" and the decode step's
 share of the HBM roofline under "roofline": of the published peaks (8 TB/s, 2.5 PFLOP/s), and under "measured_peak" /
-"frac_measured" of what a kernel that only reads, or only issues MFMA products, gets out of this device.
+"frac_measured" of what a kernel that only reads, or only issues MFMA products, gets out of this device.  Further points
+(left out with --no-further): decoding at the default batch at contexts of 8,192 and 32,768 tokens, and at the
+Llama-3.2-1B sizes decoding one request and the mixed workload of 64 requests, each decode point with its share of
+the roofline ("..._hbm_frac").
 """
 import argparse
 import json
@@ -64,7 +67,7 @@ def prefill_flops(cfg, layers, tokens):
     return 2 * tokens * body + 2 * head + attention          # the head runs on the one wanted row
 
 
-def mixed_run(cfg, args):
+def mixed_run(cfg, args, quiet=False):
     """Continuous batching under load: 64 requests at once, prompts of 64 to 2,048 tokens, 128 generated tokens each."""
     import numpy as np
     import torch
@@ -73,7 +76,8 @@ def mixed_run(cfg, args):
     lengths = rng.integers(64, 2049, 64).tolist()
     generate = 128
     need_tokens = sum(n + generate + PAGE_SIZE for n in lengths) + 64
-    engine = Engine(config=cfg, seed=0, dtype="bfloat16", device="cuda:0", ctx=4096, max_seqs=64, max_batched_tokens=PREFILL_TOKENS,
+    model = {k: v for k, v in cfg.items() if not k.startswith("_")}
+    engine = Engine(config=model, seed=0, dtype="bfloat16", device="cuda:0", ctx=4096, max_seqs=64, max_batched_tokens=PREFILL_TOKENS,
                     block_size=PAGE_SIZE, num_blocks=-(-need_tokens // PAGE_SIZE), decode_first=True, random_weights_on_device=True,
                     ahead=not args.no_ahead)
     vocab = cfg["vocab_size"]
@@ -90,16 +94,59 @@ def mixed_run(cfg, args):
         results.append((time.perf_counter() - start, tokens, rounds))
     elapsed, tokens, rounds = results[-1]
     assert tokens == 64 * generate
-    print(json.dumps({"workload": "64 requests at once, prompts of 64..2,048 tokens, 128 generated tokens each", "model": SHAPE_NAMES[args.shape],
-                      "seconds": round(elapsed, 3), "steps": rounds, "prompt_tokens": int(sum(lengths)),
-                      "generated_tokens": tokens, "generated_tokens_per_s": round(tokens / elapsed, 1),
-                      "all_tokens_per_s": round((tokens + sum(lengths)) / elapsed, 1), "preemptions": engine.stats.preemptions}), flush=True)
+    record = {"workload": "64 requests at once, prompts of 64..2,048 tokens, 128 generated tokens each", "model": cfg.get("_name", ""),
+              "seconds": round(elapsed, 3), "steps": rounds, "prompt_tokens": int(sum(lengths)),
+              "generated_tokens": tokens, "generated_tokens_per_s": round(tokens / elapsed, 1),
+              "all_tokens_per_s": round((tokens + sum(lengths)) / elapsed, 1), "preemptions": engine.stats.preemptions}
+    if not quiet:
+        print(json.dumps(record), flush=True)
+    return record, engine
+
+
+def decode_slack(batch, prompt_len):
+    """Tokens a request may generate before the timed steps begin: a request whose prompt is done decodes while the
+    prompts of the others still run, a step of PREFILL_TOKENS tokens at a time."""
+    return batch * -(-prompt_len // PREFILL_TOKENS) + 8
+
+
+def decode_run(engine, rng, vocab, batch, steps, warmup, prompt_len, tag):
+    """`batch` requests with prompts of `prompt_len` tokens; the prompts run untimed, then `warmup` untimed and `steps`
+    timed decode steps.  Returns (tokens/s, ms a step, mean context of each request over the timed steps)."""
+    import torch
+    from fllm_amd import SamplingParams
+    params = SamplingParams(max_tokens=warmup + steps + decode_slack(batch, prompt_len), ignore_eos=True)
+    names = []
+    for i in range(batch):
+        name = f"{tag}-{i}"
+        engine.add_request(name, rng.integers(0, vocab, prompt_len).tolist(), params)
+        names.append(name)
+    # prompts first (untimed): until every request has produced its first token
+    produced = {n: 0 for n in names}
+    while min(produced.values()) < 1:
+        for ev in engine.step():
+            produced[ev.request_id] += 1
+    for _ in range(warmup - 1 if warmup > 0 else 0):
+        engine.step()
+    torch.cuda.synchronize()
+    contexts = [engine.runner.cache.length(sid) for sid in engine.scheduler.running]
+    start = time.perf_counter()
+    tokens = 0
+    for _ in range(steps):
+        tokens += len(engine.step())
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - start
+    assert tokens == batch * steps, f"{tokens} tokens from {steps} steps of batch {batch}"
+    for n in names:
+        engine.abort_request(n)
+    while engine.has_unfinished():          # the step that was launched ahead
+        engine.step()
+    return tokens / elapsed, elapsed / steps * 1e3, [c + steps / 2.0 for c in contexts]
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--steps", type=int, default=248, help="timed decode steps (with the warm-up: 256 generated tokens a request)")
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--shape", choices=sorted(SHAPES), default="8b",
@@ -112,12 +159,16 @@ def main():
                          "line of its own")
     ap.add_argument("--no-ceilings", action="store_true",
                     help="do not measure what the device delivers to a kernel that only reads or only multiplies")
-    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64, the prefill and the further points")
+    ap.add_argument("--no-further", action="store_true",
+                    help="skip the points beyond the headline configuration: decoding at contexts of 8,192 and 32,768 tokens, and "
+                         "the Llama-3.2-1B sizes (decoding at batch 1 and the mixed workload of 64 requests)")
     ap.add_argument("--no-ahead", action="store_true", help="every step waits for the tokens of the step before it")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run the 2,048-token prefill steps alone and print their time (for profiling); no JSON line")
     ap.add_argument("--prompt-tokens", type=int, default=PREFILL_TOKENS,
                     help="with --prefill-only: length of the prompt; longer ones run in portions of 2,048 tokens")
+    ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="prompt length of the decode runs (for profiling other contexts)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine runs on a single MI355X, --gpus {args.gpus} is not supported")
@@ -133,46 +184,24 @@ def main():
     cfg = dict(shape, num_hidden_layers=args.layers)
     steps, warmup = args.steps, args.warmup
     if args.mixed:
-        return mixed_run(cfg, args)
+        mixed_run(dict(cfg, _name=SHAPE_NAMES[args.shape]), args)
+        return
+    further = not (args.no_points or args.no_further or args.prefill_only) and args.shape == "8b"
+    long_contexts = (8192, 32768) if further else ()
+    long_steps = 32
     batches = [args.batch] if args.no_points or args.prefill_only else sorted({1, args.batch, 64})
-    slack = max(batches) + 8          # requests whose prompt is done early decode while the others still prefill
     prompt_tokens = args.prompt_tokens if args.prefill_only else PREFILL_TOKENS
-    need_tokens = max(batches) * (PROMPT_LEN + warmup + steps + slack + PAGE_SIZE) + prompt_tokens + 64
+    runs = [(b, args.prompt_len, steps) for b in batches] + [(args.batch, c, long_steps) for c in long_contexts]
+    held = [prompt + warmup + count + decode_slack(b, prompt) for b, prompt, count in runs]      # tokens a request comes to hold
+    need_tokens = max(b * (h + PAGE_SIZE) for (b, _, _), h in zip(runs, held)) + prompt_tokens + 64
+    most_context = max([CONTEXT, prompt_tokens + 64] + [h + 64 for h in held])
     t0 = time.time()
-    engine = Engine(config=cfg, seed=0, dtype="bfloat16", device="cuda:0", ctx=max(CONTEXT, prompt_tokens + 64), max_seqs=max(batches),
+    engine = Engine(config=cfg, seed=0, dtype="bfloat16", device="cuda:0", ctx=most_context, max_seqs=max(batches),
                     max_batched_tokens=PREFILL_TOKENS, block_size=PAGE_SIZE, num_blocks=-(-need_tokens // PAGE_SIZE),
                     decode_first=True, random_weights_on_device=True, ahead=not args.no_ahead)
     print(f"[bench] engine ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
     rng = np.random.default_rng(0)
     vocab = cfg["vocab_size"]
-
-    def decode_run(batch):
-        params = SamplingParams(max_tokens=warmup + steps + slack, ignore_eos=True)
-        names = []
-        for i in range(batch):
-            name = f"b{batch}-{i}"
-            engine.add_request(name, rng.integers(0, vocab, PROMPT_LEN).tolist(), params)
-            names.append(name)
-        # prompts first (untimed): until every request has produced its first token
-        produced = {n: 0 for n in names}
-        while min(produced.values()) < 1:
-            for ev in engine.step():
-                produced[ev.request_id] += 1
-        for _ in range(warmup - 1 if warmup > 0 else 0):
-            engine.step()
-        torch.cuda.synchronize()
-        contexts = [engine.runner.cache.length(sid) for sid in engine.scheduler.running]
-        start = time.perf_counter()
-        tokens = 0
-        for _ in range(steps):
-            tokens += len(engine.step())
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - start
-        assert tokens == batch * steps, f"{tokens} tokens from {steps} steps of batch {batch}"
-        for n in names:
-            engine.abort_request(n)
-        mean_contexts = [c + steps / 2.0 for c in contexts]
-        return tokens / elapsed, elapsed / steps * 1e3, mean_contexts
 
     def prefill_run(repeats=4):
         """One request, its 2,048 tokens in one step (a longer prompt: in portions of 2,048); the median of the repeats
@@ -197,9 +226,12 @@ def main():
               file=sys.stderr, flush=True)
         return
 
+    def share(result, model=cfg, layers=args.layers):
+        return decode_step_bytes(model, layers, result[2]) / (result[1] * 1e-3) / 1e9 / HBM_PEAK_GBS
+
     results = {}
     for batch in batches:
-        results[batch] = decode_run(batch)
+        results[batch] = decode_run(engine, rng, vocab, batch, steps, warmup, args.prompt_len, f"b{batch}")
         print(f"[bench] decode batch {batch}: {results[batch][0]:.1f} tok/s, {results[batch][1]:.3f} ms/step",
               file=sys.stderr, flush=True)
 
@@ -207,14 +239,14 @@ def main():
     step_bytes = decode_step_bytes(cfg, args.layers, contexts)
     achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
     line = {
-        "metric": f"decode tok/s at batch {args.batch} ({SHAPE_NAMES[args.shape]}, 1,024-token prompts); points: batch 1/64; prefill: 2,048 tokens",
+        "metric": f"decode tok/s at batch {args.batch} ({SHAPE_NAMES[args.shape]}, {args.prompt_len:,}-token prompts); points: batch 1/64; prefill: 2,048 tokens",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic token ids, random-init weights N(0, 0.02)",
         "config": {"model": SHAPE_NAMES[args.shape], "layers": args.layers, "layers_of_model": shape["num_hidden_layers"],
                    "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
                    "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": vocab,
-                   "global_batch": args.batch, "prompt_len": PROMPT_LEN, "seq_len": CONTEXT, "kv_block": PAGE_SIZE,
+                   "global_batch": args.batch, "prompt_len": args.prompt_len, "seq_len": CONTEXT, "kv_block": PAGE_SIZE,
                    "kv_dtype": "bf16", "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
@@ -222,13 +254,19 @@ def main():
     if not args.no_points:
         line["points"] = {"decode_b1": round(results[1][0], 2), "decode_b64": round(results[64][0], 2)}
         for b in (1, 64):
-            bytes_b = decode_step_bytes(cfg, args.layers, results[b][2])
-            line["points"][f"decode_b{b}_hbm_frac"] = round(bytes_b / (results[b][1] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+            line["points"][f"decode_b{b}_hbm_frac"] = round(share(results[b]), 4)
         best = prefill_run()
         flops = prefill_flops(cfg, args.layers, PREFILL_TOKENS)
         line["prefill"] = {"value": round(PREFILL_TOKENS / best, 1), "tokens": PREFILL_TOKENS, "ms": round(best * 1e3, 3),
                            "frac": round(flops / best / (MFMA_PEAK_TFLOPS["bf16"] * 1e12), 4)}
         print(f"[bench] prefill {PREFILL_TOKENS} tokens: {best * 1e3:.2f} ms", file=sys.stderr, flush=True)
+    for context in long_contexts:
+        # the same batch further into its requests: the cache of the live requests outweighs the weights
+        result = decode_run(engine, rng, vocab, args.batch, long_steps, 2, context, f"c{context}")
+        line["points"][f"decode_b{args.batch}_ctx{context}"] = round(result[0], 2)
+        line["points"][f"decode_b{args.batch}_ctx{context}_hbm_frac"] = round(share(result), 4)
+        print(f"[bench] decode batch {args.batch} at context {context}: {result[0]:.1f} tok/s, {result[1]:.3f} ms/step",
+              file=sys.stderr, flush=True)
     if not args.no_ceilings:
         # beside the published peaks: what a kernel that only reads, or only multiplies, gets out of this device
         measured = engine.runner.rt.ops.measured_ceilings()
@@ -239,6 +277,24 @@ def main():
             line["prefill"]["frac_measured"] = round(flops / best / (measured["mfma_bf16_tflops"] * 1e12), 4)
         print(f"[bench] measured ceilings: {measured['hbm_read_gbs']:.0f} GB/s read, {measured['mfma_bf16_tflops']:.0f} TFLOP/s bf16 MFMA",
               file=sys.stderr, flush=True)
+    if further:
+        # the Llama-3.2-1B sizes: decoding one request (the fixed cost of a kernel weighs most there), and continuous
+        # batching under load (64 requests at once, prompts of 64 to 2,048 tokens, 128 generated tokens each)
+        del engine
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+        small = dict(SHAPES["1b"], _name=SHAPE_NAMES["1b"])
+        record, small_engine = mixed_run(small, args, quiet=True)
+        line["points"]["mixed_1b_generated_tok_s"] = record["generated_tokens_per_s"]
+        line["points"]["mixed_1b_all_tok_s"] = record["all_tokens_per_s"]
+        print(f"[bench] 1B sizes, 64 mixed requests: {record['generated_tokens_per_s']:.0f} generated tok/s, "
+              f"{record['all_tokens_per_s']:.0f} tok/s with the prompts", file=sys.stderr, flush=True)
+        model = {k: v for k, v in small.items() if not k.startswith("_")}
+        result = decode_run(small_engine, rng, vocab, 1, steps, warmup, PROMPT_LEN, "s1")
+        line["points"]["decode_1b_b1"] = round(result[0], 2)
+        line["points"]["decode_1b_b1_hbm_frac"] = round(share(result, model, model["num_hidden_layers"]), 4)
+        print(f"[bench] 1B sizes, decode batch 1: {result[0]:.1f} tok/s, {result[1]:.3f} ms/step", file=sys.stderr, flush=True)
     print(json.dumps(line), flush=True)
 
 
