@@ -24,6 +24,7 @@
 #include <algorithm>
 #include "api.h"
 #include "common.h"
+#include "plans.h"
 
 namespace {
 
@@ -69,7 +70,8 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 
 // floats that one part of a shared row tile leaves for the merge (tile32 kernel): head_dim / 2 outputs, a maximum
 // and a sum for each of its 256 lanes
-__host__ __device__ constexpr size_t kPartFloats(int head_dim) { return (size_t)kThreads * (head_dim / 2 + 2); }
+__host__ __device__ constexpr size_t kPartFloats(int head_dim) { return fllm_plan::part_floats(head_dim); }
+static_assert(kThreads == 256, "part_floats counts 256 threads");
 
 // Online-softmax update of one query row held across the four lane groups of a wave.
 // s: NS score tiles (already scaled and masked with -inf); returns the P^T operands.
@@ -800,30 +802,7 @@ attn_merge_kernel(const float *__restrict__ ws_ml, const float *__restrict__ ws_
     }
 }
 
-// How a decode step of `rows` rows is split over the context.  A workgroup takes `unit` keys per round (32 a
-// wave).  Contexts are split when the rows alone do not fill the machine: down to one round per workgroup when
-// the parts are merged by the split that arrives last (`fused`), and only for long contexts when merging costs
-// a second kernel.
-void decode_split_plan(int rows, int kv_heads, int qtiles, int max_context, int unit, bool fused, int *splits,
-                       int *keys_per_split) {
-    const long base = (long)rows * kv_heads * qtiles;
-    const long span = (long)max_context + 31;   // the first split starts at a multiple of 32 at or below the first key
-    long want = 1;
-    if (fused) {
-        if (base < 512) want = (512 + base - 1) / base;
-        const long most = (span + unit - 1) / unit;
-        if (want > most) want = most;
-    } else if (max_context > 2048 && base < 256) {
-        want = (256 + base - 1) / base;
-        const long most = (span + 2047) / 2048;
-        if (want > most) want = most;
-    }
-    if (want > 64) want = 64;
-    long per = (span + want - 1) / want;
-    per = (per + unit - 1) / unit * unit;
-    *splits = (int)((span + per - 1) / per);
-    *keys_per_split = (int)per;
-}
+using fllm_plan::decode_split_plan;      // how a decode step is split over the context (plans.h)
 
 bool fast_shape(int heads, int kv_heads, int head_dim, int page_size) {
     if (head_dim != 32 && head_dim != 64 && head_dim != 128) return false;
@@ -845,27 +824,11 @@ int device_slots() {   // workgroups of the tile32 kernel that the device holds 
     return slots;
 }
 
-// How the tile32 kernel shares the key tiles of a row tile among workgroups: the most key tiles one workgroup
-// takes (0: row tiles are not shared) and the most parts a row tile can have.  Row tiles are shared when, one
-// workgroup each, they would leave workgroup slots of the device empty: a part then has about the key tiles that a
-// slot sees in all when every slot is taken, and at least 8, since every part pays for leaving its results and the
-// last one for adding them up (measured: smaller parts lose more to that than they gain).  `room` is the number of
-// parts that the workspace holds.
+// How the tile32 kernel shares the key tiles of a row tile among workgroups (plans.h), with the device's slots and
+// the option that is set by hand.
 int prefill_part_plan(int tiles, int kv_heads, int max_context, int window, size_t room, int *max_parts) {
-    *max_parts = 1;
-    if (window > 0) return 0;     // a window keeps every context short
-    const long groups = (long)tiles * kv_heads;
-    if (groups * (long)sizeof(int) > (long)kWorkspaceCounterBytes) return 0;
-    const long most_tiles = ((long)max_context + 63) / 64;        // key tiles of the longest context
-    const long per_slot = (groups * most_tiles + device_slots() - 1) / device_slots();
-    long per_part = std::max(8L, per_slot);
-    if (fllm_option_prefill_parts() > 1) per_part = fllm_option_prefill_parts();   // set by hand, for measurements
-    const long cap = std::min(16L, (long)(room / (size_t)groups));   // parts a row tile may have
-    if (cap < 2) return 0;
-    per_part = std::max(per_part, (most_tiles + cap - 1) / cap);
-    if (per_part >= most_tiles) return 0;
-    *max_parts = (int)((most_tiles + per_part - 1) / per_part);
-    return (int)per_part;
+    return fllm_plan::prefill_part_plan(tiles, kv_heads, max_context, window, room, device_slots(), fllm_option_prefill_parts(),
+                                        max_parts);
 }
 
 template <int D>
@@ -883,7 +846,7 @@ int launch(const AttnArgs &a, int uniform_rows, int max_context, void *workspace
         decode_split_plan(a.rows, a.kv_heads, qtiles, max_context, WAVES * 32, fused, &p.splits, &p.keys_per_split);
         p.counters = fused && p.splits > 1 ? (int *)dev_ws : nullptr;
         if (p.splits > 1) {
-            const size_t need = (size_t)a.rows * a.heads * p.splits * (D + 2) * sizeof(float);
+            const size_t need = fllm_plan::decode_workspace_need(a.rows, a.heads, D, p.splits);
             FLLM_REQUIRE(workspace != nullptr && workspace_bytes >= need,
                          "attention: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
             p.ws_ml = (float *)workspace;
@@ -891,7 +854,8 @@ int launch(const AttnArgs &a, int uniform_rows, int max_context, void *workspace
         }
         FLLM_REQUIRE(a.kv_heads * qtiles <= 65535 && p.splits <= 65535, "attention: grid too large");
         const int gq = G < 16 ? G : 16;
-        const size_t smem = (size_t)(2 * WAVES * 16 + WAVES * gq * (D + 1)) * sizeof(float);
+        const size_t smem = fllm_plan::decode_lds_bytes(D, G);
+        static_assert(WAVES == (D >= 128 ? 8 : 16), "the plan's wave count is the kernel's");
         static bool attribute_set = false;   // more than the default 64 KiB of dynamic LDS has to be asked for once
         if (!attribute_set) {
             const hipError_t e = hipFuncSetAttribute((const void *)attn_decode_kernel<D, WAVES>,
@@ -939,7 +903,7 @@ size_t fllm_attention_bf16_workspace_bytes(int rows, int heads, int kv_heads, in
     size_t most = 0;
     for (int fused = 0; fused < 2; fused++) {
         decode_split_plan(rows, kv_heads, qtiles, max_context, (head_dim >= 128 ? 8 : 16) * 32, fused != 0, &splits, &per);
-        if (splits > 1) most = std::max(most, (size_t)rows * heads * splits * (head_dim + 2) * sizeof(float));
+        most = std::max(most, fllm_plan::decode_workspace_need(rows, heads, head_dim, splits));
     }
     return most;
 }

@@ -39,7 +39,7 @@ int fllm_option_dual_k(void);
 
 // The device workspace of the current device (fllm_set_device_workspace): its first kWorkspaceCounterBytes are
 // counters that every kernel leaves at zero, the rest is for partial results of the kernel that is running.
-constexpr size_t kWorkspaceCounterBytes = 64 * 1024;
+constexpr size_t kWorkspaceCounterBytes = 64 * 1024;      // plans.h counts with the same number (checked where both are seen)
 bool fllm_device_workspace(void **base, size_t *bytes);
 
 #define FLLM_REQUIRE(cond, ...)            \

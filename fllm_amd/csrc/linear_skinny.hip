@@ -18,6 +18,7 @@
 // workgroup takes one tile and reads its B operands from global memory.
 #include "api.h"
 #include "common.h"
+#include "plans.h"
 
 namespace {
 
@@ -988,51 +989,12 @@ struct Workspace {
     size_t bytes = 0;
 };
 constexpr size_t kCounterBytes = kWorkspaceCounterBytes;
-constexpr int kMaxSlices = 32;
+static_assert(kWorkspaceCounterBytes == fllm_plan::kCounterBytes, "plans.h and common.h agree on the counters");
+using fllm_plan::ResidentPlan;
 
-// What a launch of the resident kernel looks like for a shape: K slices, waves per workgroup, workgroups per CU.
-struct ResidentPlan {
-    int S = 0, slice = 0, waves = 8, per_cu = 0;
-    size_t stage = 0, red = 0, smem = 0;
-};
-
-// The fewest K slices whose activations fit into LDS (slicing costs more than it gains wherever it is not needed):
-// twice into a compute unit's as two workgroups of 8 waves, else once as one workgroup of 16 waves, so that as
-// many loads are in flight.
+// the plan of a resident launch (plans.h), with the options that are set by hand
 ResidentPlan plan_resident(int M, int K, int ntiles, int rt, const Workspace &ws, bool x_direct) {
-    const int forced = fllm_option_linear_slices();
-    ResidentPlan best;
-    if (x_direct) {   // nothing is staged: one slice, two workgroups of 8 waves a compute unit
-        best.S = 1;
-        best.slice = (K + 127) / 128 * 128;
-        best.waves = 8;
-        best.per_cu = 2;
-        best.stage = 0;
-        best.red = 8 * kWave * sizeof(f32x4_t);
-        best.smem = best.red + 8 * 16 * sizeof(float);
-        return best;
-    }
-    for (int S = 1; S <= kMaxSlices; S *= 2) {
-        const int slice = ((K + S - 1) / S + 127) / 128 * 128;
-        if (S > 1 && (slice < 1024 || (S - 1) * slice >= K)) break;
-        if (S > 1) {
-            const size_t need = kCounterBytes + (size_t)ntiles * S * (rt * kWave * 4 + 16) * sizeof(float);
-            if (ws.base == nullptr || need > ws.bytes || (size_t)ntiles * sizeof(int) > kCounterBytes) break;
-        }
-        ResidentPlan p;
-        p.S = S;
-        p.slice = slice;
-        p.stage = ((size_t)M * (slice + 8) * sizeof(bf16_t) + 15) / 16 * 16;
-        const size_t small = p.stage + 8 * (kWave * sizeof(f32x4_t) + 16 * sizeof(float));
-        const size_t large = p.stage + 16 * (kWave * sizeof(f32x4_t) + 16 * sizeof(float));
-        if (small <= 76 * 1024) p.waves = 8, p.per_cu = 2, p.smem = small;
-        else if (large <= 160 * 1024) p.waves = 16, p.per_cu = 1, p.smem = large;
-        else continue;
-        p.red = (size_t)p.waves * kWave * sizeof(f32x4_t);
-        if (forced == 0 || S == forced || best.S == 0) best = p;
-        if (forced == 0 || S == forced) break;
-    }
-    return best;
+    return fllm_plan::plan_resident(M, K, ntiles, rt, ws.bytes, ws.base != nullptr, x_direct, fllm_option_linear_slices());
 }
 
 template <int PRO, int EPI, int TM, int WAVES, bool XD = false>
@@ -1044,13 +1006,11 @@ int launch_resident_plan(SkinnyArgs a, const ResidentPlan &p, int ntiles, const 
     if (p.S > 1) {
         a.counters = (int *)ws.base;
         a.ws = (float *)((unsigned char *)ws.base + kCounterBytes);
-        a.ws_ssq = a.ws + (size_t)ntiles * p.S * RT * kWave * 4;
+        a.ws_ssq = a.ws + fllm_plan::resident_ssq_offset_floats(ntiles, p.S, RT);
     }
     // One workgroup per slot of the chip and slice, tiles dealt out in turn: the first slots of the
     // compute units get one tile more than the second ones when the tiles do not divide evenly.
-    int groups = device_cus() * p.per_cu / p.S;
-    if (groups < 1) groups = 1;
-    if (groups > ntiles) groups = ntiles;
+    const int groups = fllm_plan::resident_groups(p, ntiles, device_cus());
     static bool attribute_set = false;   // more than the default 64 KiB of dynamic LDS has to be asked for once
     if (!attribute_set) {
         const hipError_t e = hipFuncSetAttribute((const void *)skinny_resident_kernel<PRO, EPI, TM, WAVES, XD>,
@@ -1114,79 +1074,24 @@ int launch_wide(SkinnyArgs a, hipStream_t stream) {
     const int n_out = EPI == EPI_SWIGLU ? a.N / 2 : a.N;
     const int ntiles = (n_out + NT - 1) / NT;
     const int ngroups = (ntiles + WAVES - 1) / WAVES;
-    const int slots = 2 * device_cus();        // two workgroups of four waves a compute unit
     void *base = nullptr;
     size_t bytes = 0;
     const bool have_ws = fllm_device_workspace(&base, &bytes);
-    // K slices: as many as fill the chip with the row groups there are, each at least two chunks long
-    int S = 1;
-    const int forced = fllm_option_linear_slices();
-    while (S < 8 && ngroups * S * 2 <= slots && (a.K + 2 * S - 1) / (2 * S) >= 512) S *= 2;
-    if (forced > 0) S = forced;
-    while (S > 1) {
-        const size_t need = kWorkspaceCounterBytes + (size_t)ntiles * S * MT * RT * kWave * 4 * sizeof(float);
-        if (have_ws && need <= bytes && (size_t)ntiles * sizeof(int) <= kWorkspaceCounterBytes && (a.K + S - 1) / S >= 256) break;
-        S /= 2;
-    }
-    a.S = S;
-    a.slice = ((a.K + S - 1) / S + 255) / 256 * 256;
-    if ((S - 1) * a.slice >= a.K && S > 1) a.S = S = (a.K + a.slice - 1) / a.slice;   // no empty slice
-    if (S > 1) {
+    const fllm_plan::ChunkPlan p = fllm_plan::plan_chunks(a.K, ntiles, MT, RT, bytes, have_ws, device_cus(), fllm_option_linear_slices());
+    a.S = p.S;
+    a.slice = p.slice;
+    if (p.S > 1) {
         a.counters = (int *)base;
         a.ws = (float *)((unsigned char *)base + kWorkspaceCounterBytes);
     }
-    int per_slice = slots / S;
-    if (per_slice < 1) per_slice = 1;
-    if (per_slice > ngroups) per_slice = ngroups;
+    const int per_slice = p.grid / p.S;
+    const int S = p.S;
+    (void)ngroups;
     hipLaunchKernelGGL((skinny_wide_kernel<MT, EPI>), dim3(per_slice * S), dim3(WAVES * kWave), 0, stream, a);
     return fllm_check_launch("linear_wide");
 }
 
-// What a launch of the slab kernel looks like: the K slice that a workgroup stages and the grid.
-struct SlabPlan {
-    int S = 0, slice = 0, grid = 0;
-    size_t smem = 0, cells_off = 0;
-};
-
-// The slice length (256 to 1,024 columns; multiples of 512 for the norm prologue, whose sums of squares are kept per
-// 512 columns) that costs a workgroup the fewest bytes: its items' weights, its staged slice, and its share of the
-// partial sums that slices cost.  S == 0: nothing fits (no workspace for the slices, or too many tiles to count).
-SlabPlan plan_slab(int M, int n_tiles, int K, int mt, int rt, bool norm, int nt, size_t ws_bytes, bool have_ws, int cus) {
-    SlabPlan best;
-    double best_cost = 0.0;
-    const int rows = mt * 16;
-    const int ngroups = (n_tiles + 7) / 8;
-    const int forced = fllm_option_linear_slices();
-    for (int slice = 1024; slice >= 256; slice -= 256) {
-        if (norm && slice % 512 != 0) continue;
-        int S = (K + slice - 1) / slice;
-        int len = slice;
-        if (S == 1) len = (K + (norm ? 511 : 255)) / (norm ? 512 : 256) * (norm ? 512 : 256);   // one slice: no longer than K needs
-        if (forced > 0 && S != forced && !(S == 1 && forced == 1)) continue;
-        SlabPlan p;
-        p.S = S;
-        p.slice = len;
-        p.cells_off = ((size_t)rows * (len + 8) * sizeof(bf16_t) + 15) / 16 * 16;
-        p.smem = p.cells_off + (norm ? (size_t)rows * ((len + 511) / 512) * sizeof(float) : 0);
-        if (p.smem > 160 * 1024) continue;
-        if (S > 1) {
-            const size_t need = kWorkspaceCounterBytes + (size_t)n_tiles * S * ((size_t)mt * rt * kWave * 4 + rows) * sizeof(float);
-            if (!have_ws || need > ws_bytes || (size_t)n_tiles * sizeof(int) > kWorkspaceCounterBytes) continue;
-        }
-        int per_slice = cus / S;
-        if (per_slice < 1) per_slice = 1;
-        if (per_slice > ngroups) per_slice = ngroups;
-        p.grid = per_slice * S;
-        const int items = (ngroups + per_slice - 1) / per_slice;
-        const double weights = (double)items * 8 * (rt * nt) * len * 2.0;
-        const double staged = (double)rows * len * (norm ? 4.0 : 2.0);
-        const double parts = S > 1 ? (double)items * 8 * (double)M * rt * nt * 4.0 * 2.0 : 0.0;   // written, and read again by somebody
-        const double cost = weights + staged + parts;
-        if (best.S == 0 || cost < best_cost) best = p, best_cost = cost;
-        if (S == 1) break;      // shorter slices of a K that fits in one gain nothing
-    }
-    return best;
-}
+using fllm_plan::SlabPlan;
 
 template <int PRO, int EPI, int MT>
 int launch_slab(SkinnyArgs a, hipStream_t stream) {
@@ -1197,14 +1102,15 @@ int launch_slab(SkinnyArgs a, hipStream_t stream) {
     void *base = nullptr;
     size_t bytes = 0;
     const bool have_ws = fllm_device_workspace(&base, &bytes);
-    const SlabPlan p = plan_slab(a.M, ntiles, a.K, MT, RT, PRO == PRO_NORM_F32, NT, bytes, have_ws, device_cus());
+    const SlabPlan p = fllm_plan::plan_slab(a.M, ntiles, a.K, MT, RT, PRO == PRO_NORM_F32, NT, bytes, have_ws, device_cus(),
+                                            fllm_option_linear_slices());
     if (p.S == 0) return 1;
     a.S = p.S;
     a.slice = p.slice;
     if (p.S > 1) {
         a.counters = (int *)base;
         a.ws = (float *)((unsigned char *)base + kWorkspaceCounterBytes);
-        a.ws_ssq = a.ws + (size_t)ntiles * p.S * MT * RT * kWave * 4;
+        a.ws_ssq = a.ws + fllm_plan::slab_ssq_offset_floats(ntiles, p.S, MT, RT);
     }
     static bool attribute_set = false;   // more than the default 64 KiB of dynamic LDS has to be asked for once
     if (!attribute_set) {
