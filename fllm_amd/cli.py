@@ -35,7 +35,9 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--long-prefill-token-threshold", type=int, default=0)
     ap.add_argument("--preemption-mode", default="recompute", choices=["recompute", "none"])
     ap.add_argument("--chunked-prefill-policy", default="decode-first", choices=["decode-first", "prefill-first"])
-    ap.add_argument("--ahead", action="store_true", help="launch a step before the tokens of the step before it are read")
+    ap.add_argument("--no-ahead", dest="ahead", action="store_false",
+                    help="wait for the tokens of every step before the next one is launched (by default a step is launched "
+                         "while the tokens of the step before it are still on their way to the host)")
     ap.add_argument("--warm-up", action="store_true",
                     help="before the first request: capture the decode graphs of every batch size and run the sampler and prompt portions once")
     ap.add_argument("--check-layers", type=int, default=0, metavar="STEPS",

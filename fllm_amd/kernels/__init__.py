@@ -159,9 +159,24 @@ class Ops:
         if code != 0:
             raise KernelError(self.lib.fllm_last_error().decode("utf-8", "replace"))
 
+    _streams = {}            # device index -> the stream on which this process launches the kernels of that device
+
     @staticmethod
     def _stream() -> int:
-        return torch.cuda.current_stream().cuda_stream
+        """The current stream.  Kernels of one device meet in that device's workspace (counters that each launch leaves
+        at zero, partial results behind them), so launches on one device must not overlap: all of them go to one stream
+        (a stream that is capturing a graph stands for the stream the graph will be replayed on).  A launch on a second
+        stream of the same device is refused."""
+        stream = torch.cuda.current_stream()
+        handle, device = stream.cuda_stream, stream.device_index
+        seen = Ops._streams.get(device)
+        if seen is None:
+            if not torch.cuda.is_current_stream_capturing():
+                Ops._streams[device] = handle
+        elif handle != seen and not torch.cuda.is_current_stream_capturing():
+            raise KernelError(f"kernels of device {device} were launched on stream {seen:#x} before and are now asked for on "
+                              f"stream {handle:#x}: they share the device workspace and must stay on one stream")
+        return handle
 
     def embed(self, ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
         rows = ids.numel()

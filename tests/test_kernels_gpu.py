@@ -706,3 +706,26 @@ def test_sample_depends_only_on_seed_draw_and_logits(ops):
     assert int(out[1]) == int(out[3]) == int(alone[0])
     top40 = set(torch.topk(lg[0], 40).indices.tolist())
     assert int(out[0]) in top40
+
+
+def test_a_second_stream_is_refused(ops):
+    """Kernels of a device meet in its workspace: launches on another stream could overlap with those on the first and
+    are refused; a stream that captures a graph is let through (the engine's decode graphs are captured that way)."""
+    from fllm_amd.kernels import KernelError
+    x = torch.randn(4, 64, device=DEV)
+    w = torch.ones(64, device=DEV)
+    out = torch.empty(4, 64, device=DEV)
+    ops.rmsnorm(x, w, 1e-5, out)
+    other = torch.cuda.Stream()
+    with torch.cuda.stream(other):
+        with pytest.raises(KernelError, match="one stream"):
+            ops.rmsnorm(x, w, 1e-5, out)
+    torch.cuda.synchronize()
+    want = out.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.rmsnorm(x, w, 1e-5, out)
+    out.zero_()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
