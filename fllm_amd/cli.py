@@ -10,7 +10,7 @@ flags; rust/engine/src/tiny_model.rs:168-195 `make-tiny-model`; rust/engine/src/
     make-tiny-model OUT [--seed N] [--config FILE] [--dtype float32|bfloat16]
     selftest-gpu [--only GROUPS] [--list]                                   kernels against PyTorch on the device
     replay --model DIR --dtype D --out DIR --max-tokens N                   same as bin/trace_run
-    trace-summary DIR [--steps N]                                           per-kernel time of the last steps of a rocprofv3 trace
+    trace-summary DIR [--steps N | --counters [--last N]]                   per-kernel time of the last steps of a rocprofv3 trace, or counters a dispatch of a --pmc run
 """
 from __future__ import annotations
 

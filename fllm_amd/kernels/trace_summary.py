@@ -44,12 +44,55 @@ def summarize(path: str, steps: int = 8, top: int = 20, marker: str = "embed_ker
     return lines
 
 
+def find_counters(path: str) -> str:
+    if os.path.isfile(path):
+        return path
+    found = sorted(glob.glob(os.path.join(path, "**", "*counter_collection.csv"), recursive=True))
+    if not found:
+        raise FileNotFoundError(f"no *counter_collection.csv under {path}")
+    return found[-1]
+
+
+def summarize_counters(path: str, last: int = 2000, top: int = 8) -> List[str]:
+    """Hardware counters of a `rocprofv3 --pmc ... --output-format csv` run, averaged per dispatch for each kernel over
+    the last `last` dispatches of the run (the decode steps at its end).  One row a kernel, one column a counter."""
+    with open(find_counters(path), newline="") as f:
+        rows = list(csv.DictReader(f))
+    ids = sorted({int(r["Dispatch_Id"]) for r in rows})
+    keep = set(ids[-last:])
+    sums = collections.defaultdict(lambda: collections.defaultdict(float))
+    dispatches = collections.defaultdict(set)
+    names = []
+    for r in rows:
+        if int(r["Dispatch_Id"]) not in keep:
+            continue
+        kernel, counter = r["Kernel_Name"], r["Counter_Name"]
+        if counter not in names:
+            names.append(counter)
+        sums[kernel][counter] += float(r["Counter_Value"])
+        dispatches[kernel].add(int(r["Dispatch_Id"]))
+    order = sorted(sums, key=lambda k: -len(dispatches[k]))[:top]
+    lines = [f"counters a dispatch, averaged over the last {len(keep)} dispatches of the run"]
+    for kernel in order:
+        n = len(dispatches[kernel])
+        lines.append(f"{kernel[:100]}  ({n} dispatches)")
+        for counter in names:
+            lines.append(f"    {counter:32s} {sums[kernel][counter] / n:16.1f}")
+    return lines
+
+
 def main(argv=None) -> int:
     import argparse
     ap = argparse.ArgumentParser(prog="fllm_amd trace-summary")
     ap.add_argument("path", help="a rocprofv3 output folder or a *kernel_trace.csv")
     ap.add_argument("--steps", type=int, default=8, help="engine steps to add up, counted back from the last one")
     ap.add_argument("--top", type=int, default=20)
+    ap.add_argument("--counters", action="store_true",
+                    help="the folder holds a --pmc run: print the counters a dispatch for each kernel instead")
+    ap.add_argument("--last", type=int, default=2000, help="with --counters: dispatches to average over, counted back from the end")
     args = ap.parse_args(argv)
-    print("\n".join(summarize(args.path, args.steps, args.top)))
+    if args.counters:
+        print("\n".join(summarize_counters(args.path, args.last, min(args.top, 8))))
+    else:
+        print("\n".join(summarize(args.path, args.steps, args.top)))
     return 0
