@@ -49,10 +49,12 @@ PENDING = -1      # stands in a sequence's token list for a token that is still 
 @dataclass
 class _InFlight:
     """A launched step whose tokens have not been read: sequence ids in row order, where each
-    token goes in its sequence, and the device tensor that will hold them."""
+    token goes in its sequence, the device tensor that will hold them (the next step takes its input from there),
+    and the copy of them to the host that was queued right behind the step."""
     sampled: List[int]
     at: List[int]
     tokens: torch.Tensor
+    on_host: object = None
 
 
 class Engine:
@@ -182,6 +184,8 @@ class Engine:
         self.stats.max_rows = max(self.stats.max_rows, rows)
         requests = [SampleRequest(seqs[sid].sampling, seqs[sid].sampling.seed_for(sid), seqs[sid].draws) for sid in sampled]
         launched = _InFlight(sampled, [], self.sampler.launch(logits, requests))
+        # queued now, before the next step is launched behind it: reading these tokens must not wait for that step
+        launched.on_host = self.sampler.start_read(launched.tokens)
         # What does not depend on the tokens' values: the sequences grow by one (a placeholder until the
         # token is read), the prompt portions count as computed.
         for sid, _, count in plan.prefill:
@@ -205,7 +209,7 @@ class Engine:
         """Reads a launched step's tokens (waits for the device), puts them where the placeholders
         are and finishes the requests that end with them."""
         t0 = time.perf_counter()
-        tokens = self.sampler.read(step.tokens)
+        tokens = self.sampler.finish_read(step.on_host)
         seqs = self.scheduler.sequences
         events: List[TokenEvent] = []
         for sid, at, token in zip(step.sampled, step.at, tokens):

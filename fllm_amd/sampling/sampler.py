@@ -40,9 +40,30 @@ class Sampler:
         return self.read(self.launch(logits, rows))
 
     @staticmethod
-    def read(tokens: torch.Tensor) -> List[int]:
+    def start_read(tokens: torch.Tensor):
+        """Asks for the tokens of `launch` on the host without waiting: the copy into pinned memory is queued right
+        behind the kernels that choose them, and an event marks its end.  What is launched after this call does not
+        delay the read.  Returns what `finish_read` takes."""
+        if not tokens.is_cuda or tokens.numel() == 0:
+            return tokens, None
+        host = torch.empty(tokens.shape, dtype=tokens.dtype, pin_memory=True)
+        host.copy_(tokens, non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+        return host, done
+
+    @staticmethod
+    def finish_read(pending) -> List[int]:
+        """The token ids on the host; waits until the copy that `start_read` queued has ended."""
+        host, done = pending
+        if done is not None:
+            done.synchronize()
+        return [int(t) for t in host.tolist()]
+
+    @classmethod
+    def read(cls, tokens: torch.Tensor) -> List[int]:
         """The token ids of `launch` on the host (waits for the device)."""
-        return [int(t) for t in tokens.cpu().tolist()]
+        return cls.finish_read(cls.start_read(tokens))
 
     def launch(self, logits: torch.Tensor, rows: Sequence[SampleRequest]) -> torch.Tensor:
         """Starts the choice of one token per row and returns the int32 device tensor that will

@@ -196,6 +196,36 @@ def test_ahead_events_come_one_step_later_and_stop_where_they_should():
     assert engine.runner.cache.requests() == []
 
 
+def test_ahead_asks_for_a_steps_tokens_before_the_next_step_is_launched():
+    """The copy of a step's tokens to the host is queued right behind that step, before the next one is launched: on
+    the device's one stream a copy queued later would wait for the next step, and nothing would run ahead."""
+    engine = make_engine(ahead=True)
+    order = []
+    run_step, start_read, finish_read = engine.runner.step, engine.sampler.start_read, engine.sampler.finish_read
+
+    def spy_step(*a, **k):
+        order.append("launch")
+        return run_step(*a, **k)
+
+    def spy_start(tokens):
+        order.append("ask")
+        return start_read(tokens)
+
+    def spy_finish(pending):
+        order.append("read")
+        return finish_read(pending)
+
+    engine.runner.step, engine.sampler.start_read, engine.sampler.finish_read = spy_step, spy_start, spy_finish
+    engine.add_request("a", PROMPTS_A[0], SamplingParams(max_tokens=3))
+    while engine.has_unfinished():
+        engine.step()
+    assert order[:5] == ["launch", "ask", "launch", "ask", "read"]
+    assert order.count("ask") == order.count("read") == order.count("launch")
+    for i, what in enumerate(order):              # every read follows the launch AND the asking of a later step, or ends the run
+        if what == "read":
+            assert order[:i].count("ask") >= order[:i + 1].count("read")
+
+
 def test_ahead_abort_drops_the_row_in_flight():
     engine = make_engine(ahead=True)
     engine.add_request("a", PROMPTS_A[0], SamplingParams(max_tokens=8))
