@@ -204,21 +204,29 @@ def main():
     vocab = cfg["vocab_size"]
 
     def prefill_run(repeats=4):
-        """One request, its 2,048 tokens in one step (a longer prompt: in portions of 2,048); the median of the repeats
-        after the first."""
-        times = []
-        for i in range(repeats):
-            engine.add_request(f"prefill-{i}", rng.integers(0, vocab, prompt_tokens).tolist(),
+        """Prompts of 2,048 tokens, one request each, one step each (a longer prompt: in portions of 2,048).  All
+        requests wait in the queue before the clock starts and the first one runs untimed, so the timed steps follow one
+        another as they do under load; a device that idled for milliseconds before a step runs its first
+        kernels slower (5 ms of idling cost a 2,048-token step 1.7 ms here).  Returns the seconds a prompt took."""
+        for i in range(repeats + 2):
+            engine.add_request(f"prefill-{prefill_run.serial}-{i}", rng.integers(0, vocab, prompt_tokens).tolist(),
                                SamplingParams(max_tokens=1, ignore_eos=True))
-            torch.cuda.synchronize()
-            start = time.perf_counter()
-            events = engine.step()
-            while not events:               # with steps launched ahead the token is handed out by the next call
-                events = engine.step()
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - start)
-            assert len(events) == 1 and events[0].finished
-        return float(np.median(times[1:]))
+        prefill_run.serial += 1
+        finished = 0
+        while finished < 1:
+            finished += sum(1 for ev in engine.step() if ev.finished)
+        torch.cuda.synchronize()          # what was launched so far (a step ahead, perhaps) has run: it is not timed
+        rows_before = engine.stats.prefill_rows
+        start = time.perf_counter()
+        while finished < repeats + 2:
+            finished += sum(1 for ev in engine.step() if ev.finished)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - start
+        rows = engine.stats.prefill_rows - rows_before
+        assert rows >= repeats * prompt_tokens
+        return elapsed * prompt_tokens / rows
+
+    prefill_run.serial = 0
 
     if args.prefill_only:
         best = prefill_run(max(2, steps))
