@@ -64,7 +64,7 @@ class Engine:
                  gpu_memory_utilization: float = 0.90, decode_first: bool = True, kv_watermark_blocks: int = 0,
                  max_num_partial_prefills: int = 0, long_prefill_token_threshold: int = 0,
                  preemption_mode: str = "recompute", eos_token_ids: Optional[Seq[int]] = None,
-                 random_weights_on_device: bool = False, ops=None, ahead: bool = False, check_layers: int = 0):
+                 random_weights_on_device: bool = False, ops=None, ahead: bool = True, check_layers: int = 0):
         """`model`: a folder with config.json and safetensors; or `config` (a config.json dict)
         with `seed` for random weights (drawn on the host, or on the device with a stream of its
         own when `random_weights_on_device`: large models).  Option names follow the reference's server flags
@@ -72,7 +72,8 @@ class Engine:
         gpu_memory_utilization, kv_watermark_blocks, max_num_partial_prefills,
         long_prefill_token_threshold, preemption_mode.
 
-        `ahead`: a step is launched before the tokens of the step before it have reached the host
+        `ahead` (the default; False: every `step()` waits for its own tokens and returns them, and the host's work per
+        step adds to the step): a step is launched before the tokens of the step before it have reached the host
         (the reference's ahead step, rust/engine/src/rust_decoder.rs:1165-1266): the device takes
         them from the earlier step's output, the host plans the next step while the device runs
         this one, and `step()` returns the events of the step before.  A request that stops at a
