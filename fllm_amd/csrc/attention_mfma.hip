@@ -826,8 +826,8 @@ int device_slots() {   // workgroups of the tile32 kernel that the device holds 
 
 // How the tile32 kernel shares the key tiles of a row tile among workgroups (plans.h), with the device's slots and
 // the option that is set by hand.
-int prefill_part_plan(int tiles, int kv_heads, int max_context, int window, size_t room, int *max_parts) {
-    return fllm_plan::prefill_part_plan(tiles, kv_heads, max_context, window, room, device_slots(), fllm_option_prefill_parts(),
+int prefill_part_plan(int tiles, int kv_heads, int rows, int max_context, int window, size_t room, int *max_parts) {
+    return fllm_plan::prefill_part_plan(tiles, kv_heads, rows, max_context, window, room, device_slots(), fllm_option_prefill_parts(),
                                         max_parts);
 }
 
@@ -878,7 +878,7 @@ int launch(const AttnArgs &a, int uniform_rows, int max_context, void *workspace
         void *dev_ws = nullptr;
         size_t dev_ws_bytes = 0;
         if (fllm_option_prefill_parts() && fllm_device_workspace(&dev_ws, &dev_ws_bytes) && dev_ws_bytes > kWorkspaceCounterBytes) {
-            p.part_tiles = prefill_part_plan(tiles, a.kv_heads, max_context, a.window,
+            p.part_tiles = prefill_part_plan(tiles, a.kv_heads, a.rows, max_context, a.window,
                                              (dev_ws_bytes - kWorkspaceCounterBytes) / (kPartFloats(D) * sizeof(float)), &max_parts);
             p.counters = (int *)dev_ws;
             p.parts_ws = (float *)((unsigned char *)dev_ws + kWorkspaceCounterBytes);

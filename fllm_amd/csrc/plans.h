@@ -197,9 +197,11 @@ constexpr size_t part_floats(int head_dim) { return (size_t)256 * (head_dim / 2 
 // The most key tiles one workgroup takes (0: row tiles are not shared) and the most parts a row tile can have.  Row
 // tiles are shared when, one workgroup each, they would leave workgroup slots of the device empty: a part then has
 // about the key tiles that a slot sees in all when every slot is taken, and at least 8, since every part pays for
-// leaving its results and the last one for adding them up.  `room`: parts that the workspace holds; `by_hand`: key
-// tiles a part when set by hand (> 1).
-inline int prefill_part_plan(int tiles, int kv_heads, int max_context, int window, size_t room, int slots, int by_hand,
+// leaving its results and the last one for adding them up.  A step whose rows are as many as its longest context (a
+// prompt from its first token on) has row tiles of every length up to the longest, half of it on average: up to 2,048
+// tokens the long ones are shared in halves (8 to 16 key tiles a part), or the slots of the short ones would idle
+// through the second half of the launch (longer prompts have row tiles enough to keep every slot busy).  `room`: parts that the workspace holds; `by_hand`: key tiles a part when set by hand (> 1).
+inline int prefill_part_plan(int tiles, int kv_heads, int rows, int max_context, int window, size_t room, int slots, int by_hand,
                              int *max_parts) {
     *max_parts = 1;
     if (window > 0) return 0;     // a window keeps every context short
@@ -208,6 +210,11 @@ inline int prefill_part_plan(int tiles, int kv_heads, int max_context, int windo
     const long most_tiles = ((long)max_context + 63) / 64;        // key tiles of the longest context
     const long per_slot = (groups * most_tiles + slots - 1) / slots;
     long per_part = per_slot > 8 ? per_slot : 8;
+    if (rows + 63 >= max_context && most_tiles <= 32) {       // contexts of every length; measured a gain up to 2,048 tokens only
+        long half = most_tiles / 2;
+        half = half < 8 ? 8 : (half > 16 ? 16 : half);
+        if (half < per_part) per_part = half;
+    }
     if (by_hand > 1) per_part = by_hand;
     long cap = (long)(room / (size_t)groups);   // parts a row tile may have
     if (cap > 16) cap = 16;

@@ -160,9 +160,10 @@ int main() {
                 for (int window : {0, 512})
                     for (size_t room : {(size_t)0, (size_t)40, (size_t)4096, (size_t)1 << 20})
                         for (int slots : {2, 512})
-                            for (int by_hand : {0, 1, 3, 40}) {
+                            for (int by_hand : {0, 1, 3, 40})
+                            for (int rows : {1, context / 2, context, 4 * context}) {
                                 int max_parts = -1;
-                                const int per_part = prefill_part_plan(tiles, kv_heads, context, window, room, slots, by_hand, &max_parts);
+                                const int per_part = prefill_part_plan(tiles, kv_heads, rows, context, window, room, slots, by_hand, &max_parts);
                                 REQUIRE(max_parts >= 1 && max_parts <= 16, "parts %d", max_parts);
                                 if (per_part == 0) {
                                     REQUIRE(max_parts == 1, "an unshared row tile has one part");

@@ -563,9 +563,10 @@ def test_attention_long_contexts(ops, ref, segs, bound, window):
 @pytest.mark.parametrize("prefill_parts", [1, 0])
 @pytest.mark.parametrize("heads,kv_heads,head_dim", [(32, 8, 128), (8, 2, 64), (6, 3, 64), (16, 1, 128)])
 @pytest.mark.parametrize("segs,bound", [([(1500, 40), (0, 700), (5000, 3)], None), ([(0, 1100)], None), ([(600, 70), (0, 2)], 8192),
-                                        ([(513, 31), (1000, 33)], 1100)])
+                                        ([(513, 31), (1000, 33)], 1100), ([(0, 2048)], None)])
 def test_attention_prompt_portions_share_long_row_tiles(ops, ref, prefill_parts, heads, kv_heads, head_dim, segs, bound):
-    """Few rows over long contexts: the keys of a row tile are dealt out to several workgroups, by the bound of the
+    """Few rows over long contexts, and whole prompts (row tiles of every length, the long ones shared in halves): the
+    keys of a row tile are dealt out to several workgroups, by the bound of the
     step (parts without keys leave at once), and the one that arrives last adds the parts up: the same bits in
     every launch, and the counters they meet at are left at zero."""
     ops.set_option("attention.prefill_parts", prefill_parts)
