@@ -96,6 +96,15 @@ int fllm_attention(const void *q, int q_stride, const void *k_pages, const void 
                    int num_pages, float scale, int window, int dtype, int max_context, int single_from,
                    void *workspace, size_t workspace_bytes, hipStream_t stream);
 size_t fllm_attention_workspace_bytes(int rows, int heads, int kv_heads, int head_dim, int max_context);
+// The same attention with a bias on every score that depends on the distance alone: score(row, key) = q . k * scale +
+// head_slopes[head] * (key position - row position), float32 `head_slopes[heads]` (for position encodings that bias
+// scores instead of, or beside, rotating q and k).  Runs the plain kernel (one workgroup a row and head) in both
+// precisions: the MFMA kernels know no bias.
+int fllm_attention_sloped(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables,
+                          int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
+                          int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int page_size,
+                          int num_pages, float scale, int window, int dtype, int max_context, const float *head_slopes,
+                          hipStream_t stream);
 
 // ids[r] = previous[source[r]] where source[r] >= 0: token ids that an earlier step chose and that have not left
 // the device yet become the input of this step

@@ -23,7 +23,8 @@ __global__ void __launch_bounds__(kBlock)
 attention_generic_kernel(const T *__restrict__ q, int q_stride, const T *__restrict__ k_pages,
                          const T *__restrict__ v_pages, const int32_t *__restrict__ tables, int table_stride,
                          const int32_t *__restrict__ row_pos, const int32_t *__restrict__ row_seg, T *__restrict__ out,
-                         int heads, int kv_heads, int head_dim, int page_size, float scale, int window) {
+                         int heads, int kv_heads, int head_dim, int page_size, float scale, int window,
+                         const float *__restrict__ head_slopes) {
     extern __shared__ float smem[];
     float *qs = smem;                   // head_dim
     float *sc = smem + head_dim;        // kBlock
@@ -55,6 +56,7 @@ attention_generic_kernel(const T *__restrict__ q, int q_stride, const T *__restr
             float dot = 0.f;
             for (int c = 0; c < head_dim; c++) dot = fmaf(qs[c], to_f32<T>(kr[c]), dot);
             s = dot * scale;
+            if (head_slopes != nullptr) s = fmaf(head_slopes[h], (float)(key - pos), s);   // a bias by distance (<= 0 keys back)
         }
         const float m_new = fmaxf(m, block_max<kWaves>(s, scratch));
         const float alpha = expf(m - m_new);   // first chunk: exp(-inf) = 0
@@ -91,12 +93,13 @@ extern "C" size_t fllm_attention_workspace_bytes(int rows, int heads, int kv_hea
     return fllm_attention_bf16_workspace_bytes(rows, heads, kv_heads, head_dim, max_context);
 }
 
-extern "C" int fllm_attention(const void *q, int q_stride, const void *k_pages, const void *v_pages,
-                              const int32_t *tables, int table_stride, const int32_t *row_pos, const int32_t *row_seg,
-                              const int32_t *seg_start, int num_segs, void *out, int rows, int heads, int kv_heads,
-                              int head_dim, int page_size, int num_pages, float scale, int window, int dtype,
-                              int max_context, int single_from, void *workspace, size_t workspace_bytes,
-                              hipStream_t stream) {
+namespace {
+int attention_any(const void *q, int q_stride, const void *k_pages, const void *v_pages,
+                  const int32_t *tables, int table_stride, const int32_t *row_pos, const int32_t *row_seg,
+                  const int32_t *seg_start, int num_segs, void *out, int rows, int heads, int kv_heads,
+                  int head_dim, int page_size, int num_pages, float scale, int window, int dtype,
+                  int max_context, int single_from, void *workspace, size_t workspace_bytes, const float *head_slopes,
+                  hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && heads > 0 && kv_heads > 0 && head_dim > 0 && page_size > 0 && table_stride > 0 && num_pages > 0,
                  "attention: bad sizes");
     FLLM_REQUIRE(heads % kv_heads == 0, "attention: %d heads are not a multiple of %d key/value heads", heads, kv_heads);
@@ -104,7 +107,7 @@ extern "C" int fllm_attention(const void *q, int q_stride, const void *k_pages, 
     FLLM_REQUIRE(single_from >= 0 && single_from <= num_segs, "attention: single_from %d is outside 0..%d", single_from, num_segs);
     FLLM_REQUIRE(q_stride >= heads * head_dim, "attention: q_stride %d is shorter than heads*head_dim", q_stride);
     if (rows == 0) return 0;
-    if (dtype == FLLM_BF16) {
+    if (dtype == FLLM_BF16 && head_slopes == nullptr) {     // the MFMA kernels know no bias: biased scores take the plain kernel
         const int fast = fllm_attention_bf16_fast(q, q_stride, k_pages, v_pages, tables, table_stride, row_pos, row_seg,
                                                   seg_start, num_segs, out, rows, heads, kv_heads, head_dim, page_size,
                                                   num_pages, scale, window, max_context, single_from, workspace,
@@ -119,12 +122,35 @@ extern "C" int fllm_attention(const void *q, int q_stride, const void *k_pages, 
     if (dtype == FLLM_F32)
         hipLaunchKernelGGL(attention_generic_kernel<float>, grid, dim3(kBlock), smem, stream, (const float *)q, q_stride,
                            (const float *)k_pages, (const float *)v_pages, tables, table_stride, row_pos, row_seg,
-                           (float *)out, heads, kv_heads, head_dim, page_size, scale, window);
+                           (float *)out, heads, kv_heads, head_dim, page_size, scale, window, head_slopes);
     else if (dtype == FLLM_BF16)
         hipLaunchKernelGGL(attention_generic_kernel<bf16_t>, grid, dim3(kBlock), smem, stream, (const bf16_t *)q, q_stride,
                            (const bf16_t *)k_pages, (const bf16_t *)v_pages, tables, table_stride, row_pos, row_seg,
-                           (bf16_t *)out, heads, kv_heads, head_dim, page_size, scale, window);
+                           (bf16_t *)out, heads, kv_heads, head_dim, page_size, scale, window, head_slopes);
     else
         FLLM_REQUIRE(false, "attention: unknown dtype %d", dtype);
     return fllm_check_launch("attention");
+}
+}  // namespace
+
+extern "C" int fllm_attention(const void *q, int q_stride, const void *k_pages, const void *v_pages,
+                              const int32_t *tables, int table_stride, const int32_t *row_pos, const int32_t *row_seg,
+                              const int32_t *seg_start, int num_segs, void *out, int rows, int heads, int kv_heads,
+                              int head_dim, int page_size, int num_pages, float scale, int window, int dtype,
+                              int max_context, int single_from, void *workspace, size_t workspace_bytes,
+                              hipStream_t stream) {
+    return attention_any(q, q_stride, k_pages, v_pages, tables, table_stride, row_pos, row_seg, seg_start, num_segs, out, rows,
+                         heads, kv_heads, head_dim, page_size, num_pages, scale, window, dtype, max_context, single_from,
+                         workspace, workspace_bytes, nullptr, stream);
+}
+
+extern "C" int fllm_attention_sloped(const void *q, int q_stride, const void *k_pages, const void *v_pages,
+                                     const int32_t *tables, int table_stride, const int32_t *row_pos, const int32_t *row_seg,
+                                     const int32_t *seg_start, int num_segs, void *out, int rows, int heads, int kv_heads,
+                                     int head_dim, int page_size, int num_pages, float scale, int window, int dtype,
+                                     int max_context, const float *head_slopes, hipStream_t stream) {
+    FLLM_REQUIRE(head_slopes != nullptr, "attention_sloped: a slope per head is required");
+    return attention_any(q, q_stride, k_pages, v_pages, tables, table_stride, row_pos, row_seg, seg_start, num_segs, out, rows,
+                         heads, kv_heads, head_dim, page_size, num_pages, scale, window, dtype, max_context, num_segs,
+                         nullptr, 0, head_slopes, stream);
 }

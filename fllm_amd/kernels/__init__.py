@@ -67,6 +67,8 @@ def load_library(build_if_missing: bool = True):
                                c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_attention": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_int,
                            c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void, c_size, c_void],
+        "fllm_attention_sloped": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_int,
+                                  c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void, c_void],
         "fllm_norm_linear": [c_void, c_void, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_norm_gate_up_swiglu": [c_void, c_void, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_norm_qkv_rope_store": [c_void, c_void, c_float, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void,
@@ -382,10 +384,13 @@ class Ops:
     def attention(self, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, tables: torch.Tensor,
                   row_pos: torch.Tensor, row_seg: torch.Tensor, seg_start: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int,
                   head_dim: int, page_size: int, scale: float, window: Optional[int], max_context: int,
-                  uniform_rows: int = 0, workspace: Optional[torch.Tensor] = None, single_from: Optional[int] = None) -> torch.Tensor:
+                  uniform_rows: int = 0, workspace: Optional[torch.Tensor] = None, single_from: Optional[int] = None,
+                  head_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
         """`q` may be a column slice of a wider row-major matrix (the fused qkv buffer).
         `max_context` bounds pos + 1 over the rows; the segments from `single_from` on have one row each
-        (`uniform_rows` = 1 is `single_from` = 0: a decode step; by default no segment is known to)."""
+        (`uniform_rows` = 1 is `single_from` = 0: a decode step; by default no segment is known to).
+        `head_slopes` (float32 [heads]): every score gets head_slopes[head] * (key position - row position) added, for
+        position encodings that bias scores; such a call runs the plain kernel in both precisions."""
         rows = q.shape[0]
         _need(q.is_cuda and q.dim() == 2 and q.stride(1) == 1 and q.shape[1] == heads * head_dim,
               f"q must be [rows, {heads * head_dim}] with unit column stride")
@@ -407,6 +412,13 @@ class Ops:
             ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
         q_stride = q.stride(0) if rows > 1 else heads * head_dim
         num_segs = seg_start.numel() - 1
+        if head_slopes is not None:
+            _dense(head_slopes, "head_slopes", torch.float32, (heads,))
+            self._check(self.lib.fllm_attention_sloped(
+                _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(tables), tables.shape[1], _ptr(row_pos), _ptr(row_seg),
+                _ptr(seg_start), num_segs, _ptr(out), rows, heads, kv_heads, head_dim, page_size, num_pages, float(scale),
+                int(window) if window else 0, _DTYPE_CODE[q.dtype], int(max_context), _ptr(head_slopes), self._stream()))
+            return out
         if single_from is None:
             single_from = 0 if uniform_rows else num_segs
         _need(0 <= single_from <= num_segs and num_segs - single_from <= rows, f"single_from {single_from} does not fit {num_segs} segments of {rows} rows")

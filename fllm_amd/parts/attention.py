@@ -152,10 +152,15 @@ class PagedAttention(Mixer):
         single_from = ctx.single_rows_from()
         if 0 < single_from < ctx.num_segments and ctx.single_max_context < self.SPLIT_SINGLE_ROWS_FROM:
             single_from = ctx.num_segments
-        ops.attention(q, binding.k_pages, binding.v_pages, tables, ctx.row_pos, ctx.row_seg, ctx.seg_start,
-                      out, nh, nkv, d, binding.page_size, self.scale, self.window, ctx.max_context,
-                      single_from=single_from,
-                      workspace=ctx.attention_workspace(rt, rows, nh, nkv, d))
+        slopes = getattr(self.position, "score_slopes", None)      # a position encoding may bias scores by distance
+        if slopes is not None:
+            ops.attention(q, binding.k_pages, binding.v_pages, tables, ctx.row_pos, ctx.row_seg, ctx.seg_start,
+                          out, nh, nkv, d, binding.page_size, self.scale, self.window, ctx.max_context, head_slopes=slopes)
+        else:
+            ops.attention(q, binding.k_pages, binding.v_pages, tables, ctx.row_pos, ctx.row_seg, ctx.seg_start,
+                          out, nh, nkv, d, binding.page_size, self.scale, self.window, ctx.max_context,
+                          single_from=single_from,
+                          workspace=ctx.attention_workspace(rt, rows, nh, nkv, d))
         if branch is not None:
             ops.linear(out, self.w_o, branch, bias=self.b_o)
         else:

@@ -12,8 +12,10 @@ Roles and their interfaces:
                 vector `scale` (None otherwise): parts that have a kernel which norms its input on the way in ask the
                 norm for these instead of asking what kind of norm it is.
   position      what the mixer's kernels take: for the attention mixer float32 device tables `cos` and `sin`
-                [positions, dims/2], `dims` (lanes of a head that are rotated) and `pairing` (0: lanes l and
-                l + dims/2, 1: lanes 2l and 2l + 1).
+                [positions, dims/2], `dims` (lanes of a head that are rotated; 0 with empty tables: none) and `pairing`
+                (0: lanes l and l + dims/2, 1: lanes 2l and 2l + 1).  Optional: `score_slopes`, a float32 device
+                vector [heads]: every score gets score_slopes[head] * (key position - row position) added (an
+                encoding that biases scores by distance; such layers run the plain attention kernel).
   mixer         cache_need() / state_need() say what the cache manager must keep for it;
                 forward(ctx, h[R,H], residual_f32[R,H], binding) adds its output to `residual`.
                 State of fixed size: `binding.state[slot]` belongs to one live request (slot = ctx.seg_slots[s] on the

@@ -127,7 +127,7 @@ class ReferenceOps:
         return 0
 
     def attention(self, q, k_pages, v_pages, tables, row_pos, row_seg, seg_start, out, heads, kv_heads, head_dim, page_size, scale,
-                  window, max_context, uniform_rows=0, workspace=None, single_from=None):
+                  window, max_context, uniform_rows=0, workspace=None, single_from=None, head_slopes=None):
         rows = q.shape[0]
         group = heads // kv_heads
         for r in range(rows):
@@ -146,6 +146,8 @@ class ReferenceOps:
             qr = q[r].double().view(heads, head_dim)
             for h in range(heads):
                 s = (k[:, h // group, :] @ qr[h]) * scale
+                if head_slopes is not None:
+                    s = s + float(head_slopes[h]) * (keys - pos).double()
                 p = torch.softmax(s, dim=0)
                 out[r, h * head_dim:(h + 1) * head_dim] = (p @ v[:, h // group, :]).to(out.dtype)
         return out

@@ -416,7 +416,7 @@ def _rope_case(ops, ref, dtype, heads, kv_heads, head_dim, rope_dims, pairing, p
 
 # ---------------------------------------------------------------------------------------------
 def attention_case(ops, ref, dtype, heads, kv_heads, head_dim, page_size, segs, window, seed, fast=True, spike=False,
-                   bound=None, calls=1, mark_single_rows=True):
+                   bound=None, calls=1, mark_single_rows=True, slopes=None):
     """segs: (first position, rows) per segment.  bound: the context bound handed to the kernel (a decode graph's
     is larger than any context of the step); calls: launches in a row, which must give the same bits."""
     g = gen(seed)
@@ -447,7 +447,7 @@ def attention_case(ops, ref, dtype, heads, kv_heads, head_dim, page_size, segs, 
     q = qkv[:, : heads * head_dim]
     scale = head_dim ** -0.5
     want = ref.attention(q, k, v, tables, row_pos, row_seg, seg_start, torch.empty(rows, heads * head_dim, dtype=torch.float64),
-                         heads, kv_heads, head_dim, page_size, scale, window, max_context)
+                         heads, kv_heads, head_dim, page_size, scale, window, max_context, head_slopes=slopes)
     if window:
         # pages that lie wholly before the window of a segment's first row have been given back: their table entries
         # are -1, and a kernel that looked at them would read outside the pages
@@ -470,7 +470,8 @@ def attention_case(ops, ref, dtype, heads, kv_heads, head_dim, page_size, segs, 
         got = None
         for _ in range(calls):
             out = ops.attention(*args, torch.empty(rows, heads * head_dim, dtype=dtype, device=DEV),
-                                heads, kv_heads, head_dim, page_size, scale, window, bound, single_from=single_from, workspace=ws)
+                                heads, kv_heads, head_dim, page_size, scale, window, bound, single_from=single_from, workspace=ws,
+                                head_slopes=None if slopes is None else slopes.to(DEV))
             assert got is None or torch.equal(out, got), "two launches of the same attention differ"
             got = out
     finally:
@@ -578,6 +579,26 @@ def test_attention_prompt_portions_share_long_row_tiles(ops, ref, prefill_parts,
     from fllm_amd.kernels import Ops
     counters = Ops._workspaces[torch.cuda.current_device()][: 64 * 1024]
     assert int(counters.to(torch.int64).sum()) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv_heads,head_dim", [(8, 2, 128), (5, 1, 32), (6, 3, 48)])
+@pytest.mark.parametrize("segs,window", [([(0, 70), (300, 1), (37, 1)], None), ([(250, 50), (900, 1)], 100)])
+def test_attention_with_scores_biased_by_distance(ops, ref, dtype, heads, kv_heads, head_dim, segs, window):
+    """A slope per head times (key position - row position) on every score, as a position encoding that biases
+    scores asks for: steep slopes, so that a bias left out, of the wrong sign or of the wrong head changes the
+    result (the far key that stands out without the bias no longer does with it)."""
+    slopes = torch.tensor([0.05 * (1 + h % 4) for h in range(heads)], dtype=torch.float32)
+    biased = attention_case(ops, ref, dtype, heads, kv_heads, head_dim, 16, segs, window, 31, spike=True, calls=2, slopes=slopes)
+    plain = attention_case(ops, ref, dtype, heads, kv_heads, head_dim, 16, segs, window, 31, spike=True)
+    assert (biased.float() - plain.float()).abs().max() > 0.05
+    from fllm_amd.kernels import KernelError
+    q = torch.zeros(1, heads * head_dim, dtype=dtype, device=DEV)
+    pages = torch.zeros(2, kv_heads, 16, head_dim, dtype=dtype, device=DEV)
+    ints = lambda *v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    with pytest.raises(KernelError, match="head_slopes"):        # one slope too few
+        ops.attention(q, pages, pages.view(2, kv_heads, head_dim, 16), ints(0).view(1, 1), ints(0), ints(0), ints(0, 1),
+                      torch.empty_like(q), heads, kv_heads, head_dim, 16, 1.0, None, 1, head_slopes=slopes[:-1].to(DEV))
 
 
 @pytest.mark.parametrize("mark_single_rows", [True, False])

@@ -438,3 +438,107 @@ def test_state_slot_is_handed_over_cleared():
     runner.free_request("a")
     again = runner.step([StepEntry("a", a, all_of(a))])                    # ... and fed again from its first token
     assert close(half, want_a[:15]) and close(again, want_a)
+
+
+# ---------------------------------------------------------------------------------------------
+# A position encoding that rotates nothing and biases every score by the distance to the key
+# ---------------------------------------------------------------------------------------------
+class DistanceSlopes(Part):
+    """score(row, key) += slope[head] * (key position - row position), slope[head] = -base ** -(head + 1): what
+    such a part owes the attention mixer is `score_slopes` (float32 [heads] on the device) beside rotary arguments
+    that rotate nothing (`dims` 0, empty tables)."""
+    role = "position"
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        self.dims, self.pairing = 0, 1
+        self.cos = self.sin = torch.zeros((1, 0), dtype=torch.float32, device=rt.device)
+        slopes = [float(spec["base"]) ** -(h + 1) for h in range(int(spec["heads"]))]
+        self.score_slopes = torch.tensor(slopes, dtype=torch.float32, device=rt.device)
+
+
+register_part("position", "distance_slopes", DistanceSlopes)
+
+
+def slopes_spec(cfg):
+    hidden = cfg["hidden_size"]
+    norm = lambda name: PartSpec("rms", {"size": hidden, "eps": 1e-6}, {"weight": name})
+    layers = []
+    for i, window in enumerate((None, 24)):
+        mixer = PartSpec("attention", {"hidden_size": hidden, "num_heads": 4, "num_kv_heads": 2, "head_dim": 16, "scale": 0.25,
+                                       "window": window, "position": {"kind": "distance_slopes", "base": cfg["base"], "heads": 4}},
+                         {k: f"layers.{i}.attn.{k}" for k in "qkvo"})
+        ffn = PartSpec("gated_mlp", {"hidden_size": hidden, "intermediate_size": 56, "activation": "silu"},
+                       {k: f"layers.{i}.mlp.{k}" for k in ("gate", "up", "down")})
+        layers.append(LayerSpec(PartSpec("prenorm"), mixer, ffn, {"mixer": norm(f"layers.{i}.n1"), "feed_forward": norm(f"layers.{i}.n2")}))
+    return ModelSpec("toy-slopes", hidden, cfg["vocab_size"], 256,
+                     PartSpec("table", {"vocab_size": cfg["vocab_size"], "hidden_size": hidden}, {"weight": "embed"}),
+                     tuple(layers), (RunEntry(0), RunEntry(1)), norm("final_norm"),
+                     PartSpec("linear", {"vocab_size": cfg["vocab_size"], "hidden_size": hidden}, {"weight": "head"}))
+
+
+register_architecture(Architecture("toy-slopes", ("ToySlopesModel",), lambda c: c, slopes_spec))
+SLOPES = {"model_type": "toy-slopes", "hidden_size": 40, "vocab_size": 90, "base": 1.6}
+
+
+def biased_attention(q, k, v, scale, slopes, window=None):
+    """P.attention with slopes[h] * (key - row) added to every score (keys behind the row: a negative distance)."""
+    T, heads, d = q.shape
+    group = heads // k.shape[1]
+    out = np.zeros((T, heads, d))
+    for r in range(T):
+        start = 0 if window is None else max(0, r + 1 - window)
+        for h in range(heads):
+            s = (k[start:r + 1, h // group] @ q[r, h]) * scale + slopes[h] * (np.arange(start, r + 1) - r)
+            e = np.exp(s - s.max())
+            out[r, h] = (e / e.sum()) @ v[start:r + 1, h // group]
+    return out
+
+
+def plain_slopes(w, ids, slopes):
+    x = w["embed"][np.asarray(ids)]
+    T = len(ids)
+    for i, window in enumerate((None, 24)):
+        h = P.rms_norm(x, w[f"layers.{i}.n1"], 1e-6)
+        q = (h @ w[f"layers.{i}.attn.q"].T).reshape(T, 4, 16)
+        k = (h @ w[f"layers.{i}.attn.k"].T).reshape(T, 2, 16)
+        v = (h @ w[f"layers.{i}.attn.v"].T).reshape(T, 2, 16)
+        x = x + biased_attention(q, k, v, 0.25, slopes, window).reshape(T, 64) @ w[f"layers.{i}.attn.o"].T
+        h = P.rms_norm(x, w[f"layers.{i}.n2"], 1e-6)
+        x = x + P.gated_mlp(h, w[f"layers.{i}.mlp.gate"], w[f"layers.{i}.mlp.up"], w[f"layers.{i}.mlp.down"])
+    return P.rms_norm(x, w["final_norm"], 1e-6) @ w["head"].T
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 3e-5), ("bfloat16", 4e-2)])
+def test_toy_position_encoding_that_biases_scores(dtype, tol):
+    """A position part that hands the attention mixer a slope per head instead of angles: scores fall off with the
+    distance to the key, in a layer with all keys and in one with a window; portions, single tokens and a second
+    request against the whole sequence.  The plain function equals plain attention at slopes of zero, and the bias
+    matters: without it the logits are far from the ones wanted."""
+    rng = np.random.default_rng(3)
+    q, k, v = rng.standard_normal((9, 4, 16)), rng.standard_normal((9, 2, 16)), rng.standard_normal((9, 2, 16))
+    assert np.allclose(biased_attention(q, k, v, 0.25, np.zeros(4), 5), P.attention(q, k, v, 0.25, 5), atol=1e-12)
+    typed, spec = model_spec_from_config(SLOPES)
+    tensors = random_tensors(spec, 21, torch.float32 if dtype == "float32" else torch.bfloat16)
+    for name in tensors:                       # larger q and k, so that scores and their bias are of one size
+        if name.endswith("attn.q") or name.endswith("attn.k"):
+            tensors[name] = tensors[name] * 8
+    runner = ModelRunner(spec, tensors, dtype=dtype, page_size=16, max_tokens=256, max_requests=2)
+    w64 = tc.to_float64(tensors)
+    slopes = np.array([1.6 ** -(h + 1) for h in range(4)])
+    a, b = tc.random_ids(70, 90, 5), tc.random_ids(33, 90, 6)
+    want_a, want_b = plain_slopes(w64, a, slopes), plain_slopes(w64, b, slopes)
+    assert np.abs(plain_slopes(w64, a, np.zeros(4)) - want_a).max() > 0.05 * np.abs(want_a).max()
+    all_of = lambda toks: list(range(len(toks)))
+    got_a, got_b = [], []
+    got_a.append(runner.step([StepEntry("a", a[:23], all_of(a[:23]))]))
+    out = runner.step([StepEntry("b", b[:2], all_of(b[:2])), StepEntry("a", a[23:60], all_of(a[23:60]))])
+    got_b.append(out[:2]); got_a.append(out[2:])
+    out = runner.step([StepEntry("b", b[2:], all_of(b[2:])), StepEntry("a", [a[60]], [0])])
+    got_b.append(out[:31]); got_a.append(out[31:])
+    for i in range(61, 70):
+        got_a.append(runner.step([StepEntry("a", [a[i]], [0])]).clone())
+    for got, want in ((torch.cat(got_a), want_a), (torch.cat(got_b), want_b)):
+        err = np.abs(got.double().cpu().numpy() - want).max()
+        assert err <= tol * np.abs(want).max(), err
+    runner.cache.check_invariants()
