@@ -293,6 +293,17 @@ class Ops:
         return out
 
     GATE_UP_SWIGLU_ROWS = 64
+    # Beside the GEMM library: up to this many rows, and from this many bytes of gate and up weights on, the own
+    # product with the SwiGLU epilogue is faster than the library's product and a SwiGLU kernel behind it (measured at
+    # 17 and 32 rows: 6.5 and 4.6 us a layer at 235 MB of weights; slower at 64 rows, and at 67 MB of weights).
+    OWN_GATE_UP_ROWS = 32
+    OWN_GATE_UP_BYTES = 128 << 20
+
+    def prefers_own_gate_up(self, rows: int, w_gate_up: torch.Tensor) -> bool:
+        """Whether a bfloat16 step of `rows` rows whose products go to the GEMM library should still take
+        `gate_up_swiglu` for its gate/up product."""
+        return (self.library_gemm_from is not None and self.library_gemm_from <= rows <= self.OWN_GATE_UP_ROWS
+                and w_gate_up.numel() * w_gate_up.element_size() >= self.OWN_GATE_UP_BYTES)
 
     def gate_up_swiglu(self, x, w_gate_up, out, bias=None):
         """out = silu(x @ gate.T) * (x @ up.T) for up to 64 bfloat16 rows; w_gate_up = [gate; up], out bfloat16 [M, I]."""

@@ -58,10 +58,14 @@ class GatedMLP(FeedForward):
         start = getattr(ops, "library_gemm_from", None)
         if rt.dtype != torch.bfloat16 or start is None or rows < start or self.b_down is not None:
             return None
-        gate_up = rt.empty((rows, 2 * self.inter))
-        ops.linear(h, self.w_gate_up, gate_up, bias=self.b_gate_up)
         act = rt.empty((rows, self.inter))
-        ops.swiglu(gate_up, act)
+        if (getattr(ops, "prefers_own_gate_up", None) is not None and ops.prefers_own_gate_up(rows, self.w_gate_up)
+                and self.hidden % 8 == 0 and h.stride(0) % 8 == 0):
+            ops.gate_up_swiglu(h, self.w_gate_up, act, bias=self.b_gate_up)     # the activation as the product's epilogue
+        else:
+            gate_up = rt.empty((rows, 2 * self.inter))
+            ops.linear(h, self.w_gate_up, gate_up, bias=self.b_gate_up)
+            ops.swiglu(gate_up, act)
         out = rt.empty((rows, self.hidden))
         ops.linear(act, self.w_down, out)
         return out

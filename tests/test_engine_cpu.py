@@ -305,3 +305,18 @@ def test_layer_check_counts_bad_values_per_layer():
     broken.generate([PROMPTS_A[0]], SamplingParams(max_tokens=1))
     assert [r.bad_values > 0 for r in broken.layer_check.reports] == [False, True]
     assert "first suspect: step 0, run entry 1" in log.getvalue()
+
+
+def test_own_gate_up_beside_the_library_only_where_it_was_measured_faster():
+    """Up to 32 rows and from 128 MiB of gate and up weights on, a step whose products go to the GEMM library keeps
+    the own gate/up product with the SwiGLU epilogue; not below 17 rows (those steps take the fused kernels
+    anyway), not for small matrices, not without the library."""
+    from types import SimpleNamespace
+    from fllm_amd.kernels import Ops
+    big = torch.empty(0, dtype=torch.bfloat16).new_empty((2 * 14336, 4096), device="meta")
+    small = torch.empty(0, dtype=torch.bfloat16).new_empty((2 * 8192, 2048), device="meta")
+    ops = SimpleNamespace(library_gemm_from=17, OWN_GATE_UP_ROWS=Ops.OWN_GATE_UP_ROWS, OWN_GATE_UP_BYTES=Ops.OWN_GATE_UP_BYTES)
+    prefers = lambda rows, w, o=ops: Ops.prefers_own_gate_up(o, rows, w)
+    assert [prefers(r, big) for r in (16, 17, 32, 33, 64)] == [False, True, True, False, False]
+    assert not prefers(24, small)
+    assert not prefers(24, big, SimpleNamespace(library_gemm_from=None, OWN_GATE_UP_ROWS=32, OWN_GATE_UP_BYTES=1))
