@@ -33,6 +33,8 @@ struct Cells {
     int counts[kWaves];
     int word;            // a value one thread hands to all
     uint32_t key;
+    unsigned long long before;
+    unsigned long long units[kWaves];
 };
 
 __device__ __forceinline__ Pick wave_best(Pick p) {
@@ -182,7 +184,8 @@ __device__ __forceinline__ uint32_t ordered_key(float f) {
 // t for which a sum over {key >= t} still reaches a target (k tokens; top_p of the mass), and such a t is built
 // bit by bit from the top: a bit stays set if the sum with it set still reaches the target.  A list of up to
 // kStaged candidates is copied into LDS (logit and weight exp((v - max) / T)) and ONE wave runs the 32 + 32 trials
-// over it with shuffles and no barrier; a longer list is walked by the whole workgroup.
+// over it with shuffles and no barrier; a longer list (a flat distribution with top-p close to 1) takes three
+// histograms over the bits of the keys instead, with weights in units of 2^-40 (`key_by_histograms`).
 constexpr int kBins = 4096;
 constexpr float kBinsPerUnit = 64.0f;
 constexpr int kStaged = 4096;            // candidates that fit into the LDS the histogram no longer needs
@@ -218,7 +221,8 @@ __device__ __forceinline__ int block_exclusive_scan(int v, Cells &cells, int *to
 
 // The lowest bin b with sum(hist[0..b]) >= target, kBins when the whole histogram falls short; done by the first
 // wave, every lane over 64 bins; the same value in every thread.
-__device__ int find_bin(const unsigned long long *hist, unsigned long long target, Cells &cells) {
+__device__ int find_bin(const unsigned long long *hist, unsigned long long target, Cells &cells,
+                        unsigned long long *before = nullptr) {
     __syncthreads();
     if (threadIdx.x < kWave) {
         const int lane = threadIdx.x;
@@ -231,14 +235,17 @@ __device__ int find_bin(const unsigned long long *hist, unsigned long long targe
             if (lane - o >= 0) below += other;
         }
         int found = kBins;
+        if (lane == 0) cells.before = 0;
         if (below < target && below + own >= target) {      // the crossing lies in this lane's bins: one lane, if any
             unsigned long long cum = below;
             for (int i = 0; i < PER; i++) {
-                cum += hist[lane * PER + i];
-                if (cum >= target) {
+                const unsigned long long here = hist[lane * PER + i];
+                if (cum + here >= target) {
                     found = lane * PER + i;
+                    cells.before = cum;                      // the sum of the bins before the one found
                     break;
                 }
+                cum += here;
             }
         }
 #pragma unroll
@@ -247,6 +254,7 @@ __device__ int find_bin(const unsigned long long *hist, unsigned long long targe
     }
     __syncthreads();
     const int bin = cells.word;
+    if (before != nullptr) *before = cells.before;
     __syncthreads();
     return bin;
 }
@@ -318,6 +326,58 @@ __device__ uint32_t key_of_mass(KeyAt key_at, WeightAt weight_at, int n, uint32_
     return t > floor ? t : floor;
 }
 
+// A candidate's weight in units of 2^-40: integers, whose sums do not depend on the order of the additions.
+__device__ __forceinline__ unsigned long long units_of(float weight) {
+    return (unsigned long long)((double)weight * 1099511627776.0);
+}
+
+// the sum of `v` over the workgroup, the same in every thread
+__device__ __forceinline__ unsigned long long block_units(unsigned long long v, Cells &cells) {
+#pragma unroll
+    for (int hop = kWave / 2; hop >= 1; hop /= 2) v += __shfl_xor(v, hop, kWave);
+    __syncthreads();
+    if (threadIdx.x % kWave == 0) cells.units[threadIdx.x / kWave] = v;
+    __syncthreads();
+    unsigned long long all = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; w++) all += cells.units[w];
+    return all;
+}
+
+// Long lists (more candidates than fit into LDS): the largest key t >= floor such that the candidates with keys in
+// [t, ...) that are not below `floor` weigh `target` or more (MASS: in units of 2^-40; otherwise every candidate
+// weighs 1), found with three histograms over the key's bits, 12, 12 and 8 from the top, instead of 32 walks over
+// the list: each histogram covers the keys that share the bits found so far, its bin 0 holds the largest of them,
+// and the bin at which the running sum reaches what is still missing gives the next bits.  `floor` if no larger
+// key reaches the target.  `hist`: kBins cells of LDS.
+template <bool MASS, typename KeyAt, typename WeightAt>
+__device__ uint32_t key_by_histograms(KeyAt key_at, WeightAt weight_at, int n, uint32_t floor, unsigned long long target,
+                                      unsigned long long *hist, Cells &cells) {
+    uint32_t prefix = 0;
+    int known = 0;                          // bits of the answer found so far, from the top
+    unsigned long long above = 0;           // weight of the candidates whose keys lie above every key that begins with `prefix`
+    for (int round = 0; round < 3; round++) {
+        const int bits = round < 2 ? 12 : 8;
+        const int shift = 32 - known - bits;
+        const uint32_t mask = (1u << bits) - 1;
+        for (int i = threadIdx.x; i < kBins; i += kBlock) hist[i] = 0;
+        __syncthreads();
+        for (int i = threadIdx.x; i < n; i += kBlock) {
+            const uint32_t key = key_at(i);
+            if (key < floor || (known > 0 && (key >> (32 - known)) != prefix)) continue;
+            const unsigned long long w = MASS ? units_of(weight_at(i)) : 1ull;
+            if (w != 0) atomicAdd(&hist[mask - ((key >> shift) & mask)], w);
+        }
+        unsigned long long before = 0;
+        const int bin = find_bin(hist, target - above, cells, &before);
+        if (bin > (int)mask) return floor;   // everything from the floor up falls short of the target (rounding): keep it all
+        above += before;
+        prefix = (prefix << bits) | (mask - (uint32_t)bin);
+        known += bits;
+    }
+    return prefix > floor ? prefix : floor;
+}
+
 // Both thresholds over one list.  `total` comes in as the mass of all finite logits and is replaced by the mass of
 // what top-k keeps when top-k is on.
 template <typename Who, typename KeyAt, typename WeightAt>
@@ -364,6 +424,7 @@ sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const 
         __syncthreads();
         double total = 0.0;                  // mass of all finite logits (top-p without top-k)
         unsigned long long reach = 0;        // what this thread put into the histogram, in its units (top-p)
+        unsigned long long all_units = 0;    // the same over the workgroup
         for (int i = threadIdx.x; i < vocab; i += kBlock) {
             const float v = usable(src[i]);
             if (!(v > -INFINITY)) continue;
@@ -384,8 +445,8 @@ sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const 
         } else {
             total = WholeBlock::sum(total, cells);
             // the sum of every thread's share, far tokens included: integers, the same in any order
-            const double all = WholeBlock::sum((double)reach, cells);
-            last_bin = find_bin(bins, (unsigned long long)((double)p.top_p * all), cells);
+            all_units = block_units(reach, cells);
+            last_bin = find_bin(bins, (unsigned long long)((double)p.top_p * (double)all_units), cells);
             if (last_bin < kBins) last_bin++;   // a bin to spare: the histogram's sums are rounded, the exact ones decide
         }
         // gather the tokens up to that bin: thread t's tokens in the order it meets them, behind those of the threads before it
@@ -418,9 +479,26 @@ sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const 
             __syncthreads();
             threshold = cells.key;
         } else {
-            threshold = thresholds<WholeBlock>([&](int i) { return ordered_key(usable(src[list[i]])); },
-                                               [&](int i) { return expf((usable(src[list[i]]) - m) * inv_t); }, count,
-                                               p.top_k, use_k, use_p, p.top_p, total, cells);
+            // a long list: histograms over the keys' bits, weights in units of 2^-40 (the histogram's memory again)
+            auto key_at = [&](int i) { return ordered_key(usable(src[list[i]])); };
+            auto weight_at = [&](int i) { return expf((usable(src[list[i]]) - m) * inv_t); };
+            uint32_t t = 0;
+            unsigned long long whole = all_units;        // top-p alone: the mass of every finite logit, listed or not
+            if (use_k) {
+                t = key_by_histograms<false>(key_at, weight_at, count, 0u, (unsigned long long)min(p.top_k, count), bins, cells);
+                if (use_p) {
+                    unsigned long long mine = 0;
+                    for (int i = threadIdx.x; i < count; i += kBlock)
+                        if (key_at(i) >= t) mine += units_of(weight_at(i));
+                    whole = block_units(mine, cells);
+                }
+            }
+            if (use_p) {
+                unsigned long long target = (unsigned long long)((double)p.top_p * (double)whole);
+                if (target == 0) target = 1;
+                t = key_by_histograms<true>(key_at, weight_at, count, t, target, bins, cells);
+            }
+            threshold = t;
         }
     }
     // Gumbel-max over what is left: the largest of (v - max) / T - ln(-ln u), u the token's uniform number
