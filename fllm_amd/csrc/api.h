@@ -137,9 +137,10 @@ struct FllmSampleRow {
     uint64_t seed;       // Philox key
     uint64_t draw;       // number of the draw of this request
 };
-// work: float32 [rows, vocab] scratch (may alias logits)
+// work: float32 [rows, vocab] scratch.  kinds: 1 every row has a temperature and neither top-k nor top-p (the draw
+// looks at every token: several workgroups share a row), 2 no row is of that kind, 3 some may be.
 int fllm_sample(const float *logits, float *work, const struct FllmSampleRow *params, int32_t *out, int rows, int vocab,
-                hipStream_t stream);
+                int kinds, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -103,13 +103,11 @@ argmax_kernel(const float *__restrict__ logits, int32_t *__restrict__ out, int v
 // The same over `parts` workgroups a row: each takes a stretch of the vocabulary and leaves its best (value,
 // index) in `partial`; the one that arrives last (counted in counters[row], zero before and after) picks the
 // largest value, on ties the lowest index, so the answer does not depend on who that is.
-__global__ void __launch_bounds__(kBlock)
-argmax_split_kernel(const float *__restrict__ logits, int32_t *__restrict__ out, int vocab, int parts, int per_part,
-                    float *partial_v, int *partial_i, int *counters) {
-    __shared__ Cells cells;
-    const int row = blockIdx.x, part = blockIdx.y;
-    const int lo = part * per_part, hi = min(vocab, lo + per_part);
-    const Pick best = block_best(best_in_range(logits + (size_t)row * vocab, lo, hi), cells);
+// A part's workgroup leaves its best and is counted; true in the workgroup that was counted last, which then holds
+// the best of all parts in `all` (the largest value, on ties the lowest index, whoever it is) and has put the row's
+// counter back to zero.  parts <= kBlock.
+__device__ __forceinline__ bool meet_and_merge(Pick best, int row, int part, int parts, float *partial_v, int *partial_i,
+                                               int *counters, Cells &cells, Pick *all) {
     if (threadIdx.x == 0) {
         __hip_atomic_store(partial_v + (size_t)row * parts + part, best.value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(partial_i + (size_t)row * parts + part, best.index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -118,15 +116,27 @@ argmax_split_kernel(const float *__restrict__ logits, int32_t *__restrict__ out,
         cells.word = __hip_atomic_fetch_add(counters + row, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
-    if (cells.word != parts - 1) return;
+    if (cells.word != parts - 1) return false;
     if (threadIdx.x == 0) __hip_atomic_store(counters + row, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     Pick mine = {-INFINITY, kNone};
     if ((int)threadIdx.x < parts) {
         mine.value = __hip_atomic_load(partial_v + (size_t)row * parts + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         mine.index = __hip_atomic_load(partial_i + (size_t)row * parts + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    const Pick all = block_best(mine, cells);
-    if (threadIdx.x == 0) out[row] = token_of(all);
+    *all = block_best(mine, cells);
+    return true;
+}
+
+__global__ void __launch_bounds__(kBlock)
+argmax_split_kernel(const float *__restrict__ logits, int32_t *__restrict__ out, int vocab, int parts, int per_part,
+                    float *partial_v, int *partial_i, int *counters) {
+    __shared__ Cells cells;
+    const int row = blockIdx.x, part = blockIdx.y;
+    const int lo = part * per_part, hi = min(vocab, lo + per_part);
+    const Pick best = block_best(best_in_range(logits + (size_t)row * vocab, lo, hi), cells);
+    Pick all;
+    if (meet_and_merge(best, row, part, parts, partial_v, partial_i, counters, cells, &all) && threadIdx.x == 0)
+        out[row] = token_of(all);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -392,14 +402,87 @@ __device__ uint32_t thresholds(KeyAt key_at, WeightAt weight_at, int n, int top_
     return t;
 }
 
+// Calls f(token, logit) for every token of a row, each thread of the workgroup with a share of its own: four
+// consecutive tokens a load where the row's alignment allows (two such loads in flight), single tokens at both ends.
+// A thread meets its tokens in the same order in every pass.
+template <typename F>
+__device__ __forceinline__ void for_each_token(const float *__restrict__ src, int vocab, F f) {
+    const int head = min(vocab, (int)((4 - (((uintptr_t)src >> 2) & 3)) & 3));      // tokens before the first 16-byte boundary
+    if ((int)threadIdx.x < head) f((int)threadIdx.x, src[threadIdx.x]);
+    const int quads = (vocab - head) / 4;
+    const f32x4_t *q = (const f32x4_t *)(src + head);
+    int i = threadIdx.x;
+    for (; i + kBlock < quads; i += 2 * kBlock) {
+        const f32x4_t a = q[i], b = q[i + kBlock];
+        const int ta = head + 4 * i, tb = head + 4 * (i + kBlock);
+#pragma unroll
+        for (int e = 0; e < 4; e++) f(ta + e, a[e]);
+#pragma unroll
+        for (int e = 0; e < 4; e++) f(tb + e, b[e]);
+    }
+    if (i < quads) {
+        const f32x4_t a = q[i];
+        const int ta = head + 4 * i;
+#pragma unroll
+        for (int e = 0; e < 4; e++) f(ta + e, a[e]);
+    }
+    const int done = head + 4 * quads;
+    if ((int)threadIdx.x < vocab - done) f(done + (int)threadIdx.x, src[done + threadIdx.x]);
+}
+
+// a row with a temperature and neither top-k nor top-p: the draw looks at every token
+__device__ __forceinline__ bool draws_from_all(const FllmSampleRow &p, int vocab) {
+    return p.temperature > 1e-5f && !(p.top_k > 0 && p.top_k < vocab) && !(p.top_p > 0.f && p.top_p < 1.f);
+}
+
+// Such rows spend their time on the random numbers of all tokens, so several workgroups share a row, in two
+// launches: the largest logit first (`row_max`), then the largest (v - max) / T - ln(-ln u), each as a split argmax.
+// Rows of another kind leave at once.
+template <int PHASE>
+__global__ void __launch_bounds__(kBlock)
+draw_from_all_kernel(const float *__restrict__ logits, const FllmSampleRow *__restrict__ params, int32_t *__restrict__ out,
+                     int vocab, int parts, int per_part, float *partial_v, int *partial_i, int *counters, float *row_max) {
+    __shared__ Cells cells;
+    const int row = blockIdx.x, part = blockIdx.y;
+    const FllmSampleRow p = params[row];
+    if (!draws_from_all(p, vocab)) return;
+    const float *src = logits + (size_t)row * vocab;
+    const int lo = part * per_part, hi = min(vocab, lo + per_part);
+    Pick best = {-INFINITY, kNone}, all;
+    if (PHASE == 0) {
+        best = block_best(best_in_range(src, lo, hi), cells);
+        if (meet_and_merge(best, row, part, parts, partial_v, partial_i, counters, cells, &all) && threadIdx.x == 0)
+            row_max[row] = all.value;
+        return;
+    }
+    const float m = row_max[row];
+    if (!(m > -INFINITY)) {                  // no finite logit: index 0, as the reference's argmax gives
+        if (part == 0 && threadIdx.x == 0) out[row] = 0;
+        return;
+    }
+    const float inv_t = (float)(1.0 / (double)p.temperature);
+    for (int i = lo + (int)threadIdx.x; i < hi; i += kBlock) {
+        const float v = usable(src[i]);
+        if (!(v > -INFINITY)) continue;
+        const float u = uniform_of(p.seed, p.draw, (uint32_t)i);
+        const Pick here = {(v - m) * inv_t - logf(-logf(u)), i};
+        best = better_of(best, here);
+    }
+    best = block_best(best, cells);
+    if (meet_and_merge(best, row, part, parts, partial_v, partial_i, counters, cells, &all) && threadIdx.x == 0)
+        out[row] = token_of(all);
+}
+
 // `work` gives every row `vocab` 32-bit words of its own (the list of token ids); it must not overlap the logits.
+// `skip_draws_from_all`: rows with a temperature and no filter are left to `draw_from_all_kernel`.
 __global__ void __launch_bounds__(kBlock)
 sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const FllmSampleRow *__restrict__ params,
-              int32_t *__restrict__ out, int vocab) {
+              int32_t *__restrict__ out, int vocab, int skip_draws_from_all) {
     __shared__ Cells cells;
     __shared__ unsigned long long bins[kBins];       // the histogram; afterwards the staged candidates
     const int row = blockIdx.x;
     const FllmSampleRow p = params[row];
+    if (skip_draws_from_all && draws_from_all(p, vocab)) return;
     const float *src = logits + (size_t)row * vocab;
     if (p.temperature <= 1e-5f) {
         const Pick best = block_best(best_in_range(src, 0, vocab), cells);
@@ -408,7 +491,7 @@ sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const 
     }
     int *list = (int *)(work + (size_t)row * vocab);
     float m = -INFINITY;
-    for (int i = threadIdx.x; i < vocab; i += kBlock) m = fmaxf(m, usable(src[i]));
+    for_each_token(src, vocab, [&](int, float v) { m = fmaxf(m, usable(v)); });
     m = block_largest(m, cells);
     if (!(m > -INFINITY)) {
         if (threadIdx.x == 0) out[row] = 0;   // no finite logit: the reference's argmax gives index 0 as well
@@ -425,20 +508,20 @@ sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const 
         double total = 0.0;                  // mass of all finite logits (top-p without top-k)
         unsigned long long reach = 0;        // what this thread put into the histogram, in its units (top-p)
         unsigned long long all_units = 0;    // the same over the workgroup
-        for (int i = threadIdx.x; i < vocab; i += kBlock) {
-            const float v = usable(src[i]);
-            if (!(v > -INFINITY)) continue;
+        for_each_token(src, vocab, [&](int, float raw) {
+            const float v = usable(raw);
+            if (!(v > -INFINITY)) return;
             const int b = bin_of(v, m);
             if (use_k) {
                 if (b < kBins) atomicAdd(&bins[b], 1ull);
             } else {
                 const float e = expf((v - m) * inv_t);
                 total += (double)e;
-                const unsigned long long fixed = (unsigned long long)((double)e * 1099511627776.0);
+                const unsigned long long fixed = units_of(e);
                 reach += fixed;
                 if (b < kBins && fixed != 0) atomicAdd(&bins[b], fixed);
             }
-        }
+        });
         int last_bin;
         if (use_k) {
             last_bin = find_bin(bins, (unsigned long long)p.top_k, cells);
@@ -451,15 +534,15 @@ sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const 
         }
         // gather the tokens up to that bin: thread t's tokens in the order it meets them, behind those of the threads before it
         int mine = 0;
-        for (int i = threadIdx.x; i < vocab; i += kBlock) {
-            const float v = usable(src[i]);
+        for_each_token(src, vocab, [&](int, float raw) {
+            const float v = usable(raw);
             mine += (v > -INFINITY && bin_of(v, m) <= last_bin) ? 1 : 0;
-        }
+        });
         int at = block_exclusive_scan(mine, cells, &count);
-        for (int i = threadIdx.x; i < vocab; i += kBlock) {
-            const float v = usable(src[i]);
-            if (v > -INFINITY && bin_of(v, m) <= last_bin) list[at++] = i;
-        }
+        for_each_token(src, vocab, [&](int token, float raw) {
+            const float v = usable(raw);
+            if (v > -INFINITY && bin_of(v, m) <= last_bin) list[at++] = token;
+        });
         __syncthreads();                     // the list is written (global memory, read back by other threads below)
         if (count <= kStaged) {
             // the histogram is done with: its memory takes the candidates' logits and weights, and one wave finds both thresholds
@@ -600,10 +683,31 @@ extern "C" int fllm_argmax_static(const float *logits, int32_t *out, int rows, i
 }
 
 extern "C" int fllm_sample(const float *logits, float *work, const FllmSampleRow *params, int32_t *out, int rows,
-                           int vocab, hipStream_t stream) {
+                           int vocab, int kinds, hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
     FLLM_REQUIRE(work != nullptr && params != nullptr, "sample: work and params are required");
+    FLLM_REQUIRE(kinds >= 1 && kinds <= 3, "sample: kinds %d is none of 1 (rows that draw from all tokens), 2 (other rows), 3 (both)", kinds);
     if (rows == 0) return 0;
-    hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(kBlock), 0, stream, logits, work, params, out, vocab);
+    // rows with a temperature and no filter: several workgroups a row, if the device workspace is there to meet in
+    void *ws = nullptr;
+    size_t ws_bytes = 0;
+    int parts = (vocab + 8191) / 8192;
+    if (parts > 64) parts = 64;
+    if (parts * rows > 2048) parts = 2048 / rows;
+    const bool split = (kinds & 1) && parts > 1 && fllm_device_workspace(&ws, &ws_bytes) &&
+                       (size_t)rows * sizeof(int) <= kWorkspaceCounterBytes &&
+                       kWorkspaceCounterBytes + (size_t)rows * parts * 8 + (size_t)rows * 4 <= ws_bytes;
+    if (split) {
+        const int per_part = (vocab + parts - 1) / parts;
+        float *pv = (float *)((unsigned char *)ws + kWorkspaceCounterBytes);
+        int *pi = (int *)(pv + (size_t)rows * parts);
+        float *row_max = (float *)(pi + (size_t)rows * parts);
+        hipLaunchKernelGGL(draw_from_all_kernel<0>, dim3(rows, parts), dim3(kBlock), 0, stream, logits, params, out, vocab, parts,
+                           per_part, pv, pi, (int *)ws, row_max);
+        hipLaunchKernelGGL(draw_from_all_kernel<1>, dim3(rows, parts), dim3(kBlock), 0, stream, logits, params, out, vocab, parts,
+                           per_part, pv, pi, (int *)ws, row_max);
+        if (!(kinds & 2)) return fllm_check_launch("sample");
+    }
+    hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(kBlock), 0, stream, logits, work, params, out, vocab, split ? 1 : 0);
     return fllm_check_launch("sample");
 }

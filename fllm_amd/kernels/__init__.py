@@ -33,7 +33,7 @@ assert SAMPLE_ROW_BYTES == 32
 _lib = None
 
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 def load_library(build_if_missing: bool = True):
@@ -76,7 +76,7 @@ def load_library(build_if_missing: bool = True):
         "fllm_argmax": [c_void, c_void, c_int, c_int, c_void],
         "fllm_gate_up_swiglu": [c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_carry_ids": [c_void, c_void, c_void, c_int, c_int, c_void],
-        "fllm_sample": [c_void, c_void, c_void, c_void, c_int, c_int, c_void],
+        "fllm_sample": [c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -483,12 +483,15 @@ class Ops:
         self._check(self.lib.fllm_argmax(_ptr(logits), _ptr(out), rows, vocab, self._stream()))
         return out
 
-    def sample(self, logits: torch.Tensor, work: torch.Tensor, params: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-        """`params`: uint8 GPU tensor [rows, 32] holding `SampleRow` records."""
+    def sample(self, logits: torch.Tensor, work: torch.Tensor, params: torch.Tensor, out: torch.Tensor,
+               kinds: int = 3) -> torch.Tensor:
+        """`params`: uint8 GPU tensor [rows, 32] holding `SampleRow` records.  `kinds`: what the caller knows of the rows:
+        1 all of them have a temperature and no top-k or top-p (their draw looks at every token, and several
+        workgroups share a row), 2 none of them is of that kind, 3 (default) some may be."""
         rows, vocab = logits.shape
         _dense(logits, "logits", torch.float32)
         _dense(work, "work", torch.float32, (rows, vocab))
         _dense(params, "params", torch.uint8, (rows, SAMPLE_ROW_BYTES))
         _dense(out, "out", torch.int32, (rows,))
-        self._check(self.lib.fllm_sample(_ptr(logits), _ptr(work), _ptr(params), _ptr(out), rows, vocab, self._stream()))
+        self._check(self.lib.fllm_sample(_ptr(logits), _ptr(work), _ptr(params), _ptr(out), rows, vocab, int(kinds), self._stream()))
         return out

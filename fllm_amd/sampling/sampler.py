@@ -81,5 +81,8 @@ class Sampler:
             if logits.is_cuda:      # from pinned memory, so that the copy does not wait for the device
                 params = params.pin_memory().to(logits.device, non_blocking=True)
             work = torch.empty_like(logits)
-            self.rt.ops.sample(logits, work, params, out)
+            vocab = logits.shape[1]
+            from_all = [(not r.params.greedy) and not (0 < r.params.top_k < vocab) and not (0.0 < r.params.top_p < 1.0) for r in rows]
+            kinds = 1 if all(from_all) else (3 if any(from_all) else 2)
+            self.rt.ops.sample(logits, work, params, out, kinds)
         return out

@@ -165,7 +165,7 @@ class ReferenceOps:
             out[r] = 0 if not np.isfinite(row).any() else plain_llama.greedy(row)
         return out
 
-    def sample(self, logits, work, params, out):
+    def sample(self, logits, work, params, out, kinds=3):
         raw = params.cpu().numpy().tobytes()
         rec = np.frombuffer(raw, dtype=np.dtype([("temperature", "<f4"), ("top_p", "<f4"), ("top_k", "<i4"),
                                                  ("pad", "<i4"), ("seed", "<u8"), ("draw", "<u8")]))

@@ -712,6 +712,40 @@ def test_sample_thresholds_on_wide_vocabularies(ops, vocab):
                 assert int(out[i]) == want, (name, draw, i)
 
 
+@pytest.mark.parametrize("vocab", [1000, 128256])
+def test_sample_rows_that_draw_from_all_tokens_share_workgroups(ops, vocab):
+    """Rows with a temperature and no filter are drawn by several workgroups each (wide vocabularies) in launches of
+    their own; what the caller says it knows of the rows (`kinds`) changes no token, rows of both kinds in one call
+    are each the plain sampler's, and a row without a finite logit gives token 0."""
+    from fllm_amd.sampling import SampleRequest, SamplingParams, pack_rows
+    g = gen(29)
+    plain = [SamplingParams(temperature=t) for t in (0.3, 1.0, 2.5, 1.0)]
+    other = [SamplingParams(temperature=0.9, top_k=7), SamplingParams(temperature=0.0), SamplingParams(temperature=1.2, top_p=0.8)]
+    logits = torch.randn(len(plain) + len(other), vocab, generator=g) * 2.5
+    logits[3] = float("-inf")
+    logits[1, ::5] = float("nan")
+
+    def draw(rows, params, kinds, d):
+        reqs = [SampleRequest(p, seed=70 + i, draw=d) for i, p in zip(rows, params)]
+        out = torch.full((len(rows),), -1, dtype=torch.int32, device=DEV)
+        ops.sample(logits[rows].to(DEV), torch.empty(len(rows), vocab, device=DEV), pack_rows(reqs).to(DEV), out, kinds)
+        return out.cpu().tolist()
+
+    for d in range(3):
+        want = [plain_llama.device_sample(logits[i].numpy(), p.temperature, p.top_k, p.top_p, 70 + i, d)
+                for i, p in enumerate(plain + other)]
+        assert want[3] == 0
+        assert draw(list(range(7)), plain + other, 3, d) == want
+        assert draw([0, 1, 2, 3], plain, 1, d) == want[:4] == draw([0, 1, 2, 3], plain, 3, d)
+        assert draw([4, 5, 6], other, 2, d) == want[4:] == draw([4, 5, 6], other, 3, d)
+    from fllm_amd.kernels import KernelError
+    with pytest.raises(KernelError, match="kinds"):
+        draw([0], plain[:1], 0, 0)
+    counters = type(ops)._workspaces[torch.cuda.current_device()][: 64 * 1024]
+    torch.cuda.synchronize()
+    assert int(counters.to(torch.int64).sum()) == 0
+
+
 def test_sample_depends_only_on_seed_draw_and_logits(ops):
     from fllm_amd.sampling import SampleRequest, SamplingParams, pack_rows
     g = gen(18)
