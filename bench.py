@@ -10,7 +10,7 @@ JSON line on standard output holds decoded tokens per second at the default batc
 at batch 1 and 64 under "points", a 2,048-token prefill under "prefill" and the decode step's
 share of the HBM roofline under "roofline": of the published peaks (8 TB/s, 2.5 PFLOP/s), and under "measured_peak" /
 "frac_measured" of what a kernel that only reads, or only issues MFMA products, gets out of this device.  Further points
-(left out with --no-further): decoding at the default batch at contexts of 8,192 and 32,768 tokens, and at the
+(left out with --no-further): decoding at the default batch with sampled tokens (temperature 0.8, top-k 50, top-p 0.9) and at contexts of 8,192 and 32,768 tokens, and at the
 Llama-3.2-1B sizes decoding one request and the mixed workload of 64 requests, each decode point with its share of
 the roofline ("..._hbm_frac").
 """
@@ -109,12 +109,13 @@ def decode_slack(batch, prompt_len):
     return batch * -(-prompt_len // PREFILL_TOKENS) + 8
 
 
-def decode_run(engine, rng, vocab, batch, steps, warmup, prompt_len, tag):
+def decode_run(engine, rng, vocab, batch, steps, warmup, prompt_len, tag, sampling=None):
     """`batch` requests with prompts of `prompt_len` tokens; the prompts run untimed, then `warmup` untimed and `steps`
-    timed decode steps.  Returns (tokens/s, ms a step, mean context of each request over the timed steps)."""
+    timed decode steps.  `sampling`: temperature, top_k, top_p of every request (greedy without).
+    Returns (tokens/s, ms a step, mean context of each request over the timed steps)."""
     import torch
     from fllm_amd import SamplingParams
-    params = SamplingParams(max_tokens=warmup + steps + decode_slack(batch, prompt_len), ignore_eos=True)
+    params = SamplingParams(max_tokens=warmup + steps + decode_slack(batch, prompt_len), ignore_eos=True, **(sampling or {}))
     names = []
     for i in range(batch):
         name = f"{tag}-{i}"
@@ -268,6 +269,13 @@ def main():
         line["prefill"] = {"value": round(PREFILL_TOKENS / best, 1), "tokens": PREFILL_TOKENS, "ms": round(best * 1e3, 3),
                            "frac": round(flops / best / (MFMA_PEAK_TFLOPS["bf16"] * 1e12), 4)}
         print(f"[bench] prefill {PREFILL_TOKENS} tokens: {best * 1e3:.2f} ms", file=sys.stderr, flush=True)
+    if further:
+        # the same batch with sampled tokens (temperature 0.8, top-k 50, top-p 0.9): what the sampler adds to a step
+        result = decode_run(engine, rng, vocab, args.batch, min(steps, 64), 2, args.prompt_len, "sampled",
+                            sampling={"temperature": 0.8, "top_k": 50, "top_p": 0.9})
+        line["points"][f"decode_b{args.batch}_sampled"] = round(result[0], 2)
+        print(f"[bench] decode batch {args.batch}, temperature 0.8, top-k 50, top-p 0.9: {result[0]:.1f} tok/s, {result[1]:.3f} ms/step",
+              file=sys.stderr, flush=True)
     for context in long_contexts:
         # the same batch further into its requests: the cache of the live requests outweighs the weights
         result = decode_run(engine, rng, vocab, args.batch, long_steps, 2, context, f"c{context}")
