@@ -43,3 +43,12 @@ def test_the_line_of_a_short_run():
     assert (roofline["bound"], roofline["peak"], roofline["unit"]) == ("hbm", 8000.0, "GB/s")
     assert abs(roofline["frac"] - roofline["achieved"] / roofline["peak"]) < 1e-3 and 0 < roofline["frac"] < 1
     assert line["points"]["decode_b1"] > 0 and line["points"]["decode_b64"] > line["points"]["decode_b1"]
+
+
+@pytest.mark.gpu
+def test_the_smoke_run_of_the_entry_file():
+    """`__graft_entry__.smoke()` in a process of its own, as it is run: a few tokens of a tiny random model on the
+    device against the plain implementation."""
+    done = subprocess.run([sys.executable, "-c", "import __graft_entry__ as g; g.smoke()"], capture_output=True, text=True,
+                          timeout=300, cwd=ROOT)
+    assert done.returncode == 0, (done.stdout + done.stderr)[-2000:]
