@@ -31,6 +31,15 @@ def pack_rows(rows: Sequence[SampleRequest]) -> torch.Tensor:
     return torch.frombuffer(raw, dtype=torch.uint8).view(len(rows), _RECORD).clone()
 
 
+def draws_from_all(p: SamplingParams, vocab: int) -> bool:
+    """A temperature and neither top-k nor top-p: the kernel's own test, on the float32 values that the row record
+    holds (a temperature or top-p that rounds across its limit must be judged as the kernel judges it)."""
+    import struct
+    temperature, top_p = struct.unpack("<ff", struct.pack("<ff", float(p.temperature), float(p.top_p)))
+    limit = struct.unpack("<f", struct.pack("<f", 1e-5))[0]
+    return temperature > limit and not (0 < int(p.top_k) < vocab) and not (0.0 < top_p < 1.0)
+
+
 class Sampler:
     def __init__(self, rt):
         self.rt = rt
@@ -82,7 +91,7 @@ class Sampler:
                 params = params.pin_memory().to(logits.device, non_blocking=True)
             work = torch.empty_like(logits)
             vocab = logits.shape[1]
-            from_all = [(not r.params.greedy) and not (0 < r.params.top_k < vocab) and not (0.0 < r.params.top_p < 1.0) for r in rows]
+            from_all = [draws_from_all(r.params, vocab) for r in rows]
             kinds = 1 if all(from_all) else (3 if any(from_all) else 2)
             self.rt.ops.sample(logits, work, params, out, kinds)
         return out

@@ -320,3 +320,16 @@ def test_own_gate_up_beside_the_library_only_where_it_was_measured_faster():
     assert [prefers(r, big) for r in (16, 17, 32, 33, 64)] == [False, True, True, False, False]
     assert not prefers(24, small)
     assert not prefers(24, big, SimpleNamespace(library_gemm_from=None, OWN_GATE_UP_ROWS=32, OWN_GATE_UP_BYTES=1))
+
+
+def test_rows_that_draw_from_all_tokens_are_told_as_the_kernel_tells_them():
+    """What the sampler says it knows of its rows is judged on the float32 values of the row records: a temperature a
+    hair above the greedy limit, or a top-p a hair below one, rounds across the limit there."""
+    from fllm_amd.sampling.sampler import draws_from_all
+    P = SamplingParams
+    assert draws_from_all(P(temperature=0.8), 100) and draws_from_all(P(temperature=0.8, top_k=100), 100)
+    assert draws_from_all(P(temperature=0.8, top_p=1.0), 100)
+    assert not draws_from_all(P(temperature=0.0), 100) and not draws_from_all(P(temperature=0.8, top_k=5), 100)
+    assert not draws_from_all(P(temperature=0.8, top_p=0.9), 100)
+    assert not draws_from_all(P(temperature=1.0000000001e-5), 100)           # float32: the limit itself, greedy in the kernel
+    assert draws_from_all(P(temperature=0.8, top_p=0.999999999), 100)        # float32: one, no filter in the kernel
