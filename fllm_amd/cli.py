@@ -65,6 +65,13 @@ def cmd_run(argv: List[str]) -> int:
     ap.add_argument("--top-p", type=float, default=1.0)
     ap.add_argument("--top-k", type=int, default=0)
     ap.add_argument("--seed", type=int, default=None)
+    ap.add_argument("--min-p", type=float, default=0.0, help="drop what weighs less than this share of the likeliest token")
+    ap.add_argument("--repeat-penalty", type=float, default=1.0, help="repetition penalty on tokens seen before (1: off)")
+    ap.add_argument("--presence-penalty", type=float, default=0.0)
+    ap.add_argument("--frequency-penalty", type=float, default=0.0)
+    ap.add_argument("--repeat-last-n", type=int, default=-1, help="tokens of the history the penalties look at (negative: all)")
+    ap.add_argument("--min-tokens", type=int, default=0, help="no end-of-sequence or stop id before this many generated tokens")
+    ap.add_argument("--logit-bias", default="", help="comma-separated id:value pairs added to the logits")
     ap.add_argument("--stop-token-ids", default="", help="comma-separated")
     ap.add_argument("--ignore-eos", action="store_true")
     _engine_options(ap)
@@ -83,8 +90,12 @@ def cmd_run(argv: List[str]) -> int:
         print(f"warm-up: {count} requests, {len(engine.runner._graphs)} decode graphs in {time.perf_counter() - started:.2f}s",
               file=sys.stderr)
     stops = tuple(int(t) for t in args.stop_token_ids.split(",") if t.strip())
+    bias = tuple((int(t), float(b)) for t, b in (pair.split(":") for pair in args.logit_bias.split(",") if pair.strip()))
     params = SamplingParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k, seed=args.seed,
-                            max_tokens=args.max_tokens, stop_token_ids=stops, ignore_eos=args.ignore_eos)
+                            max_tokens=args.max_tokens, stop_token_ids=stops, ignore_eos=args.ignore_eos, min_p=args.min_p,
+                            repetition_penalty=args.repeat_penalty, presence_penalty=args.presence_penalty,
+                            frequency_penalty=args.frequency_penalty, repeat_last_n=args.repeat_last_n,
+                            min_tokens=args.min_tokens, logit_bias=bias)
     names = [f"prompt-{i}" for i in range(len(prompts))]
     for name, prompt in zip(names, prompts):
         engine.add_request(name, prompt, params)

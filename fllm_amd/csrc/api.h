@@ -133,10 +133,29 @@ struct FllmSampleRow {
     float temperature;   // <= 1e-5: greedy
     float top_p;         // nucleus; outside (0, 1): off
     int32_t top_k;       // <= 0: off
-    int32_t pad;
+    float min_p;         // drops what weighs less than min_p times the likeliest token; <= 0: off
     uint64_t seed;       // Philox key
     uint64_t draw;       // number of the draw of this request
 };
+// What is done to a row of logits before a token is chosen (rust/engine/src/sampling.rs:220-229, :252-274).  The
+// lists live in arrays shared by all rows: seen_ids / seen_counts [seen_off .. + seen_len) are the distinct tokens of
+// the request's history (within its window) and how often each occurs; bias_ids / bias_values; blocked_ids (to -inf).
+// last_row >= 0: last_tokens[last_row] (device memory, written by an earlier launch) is the newest token of the
+// history and not in the lists yet: it counts once more.  A row whose lists are empty and last_row < 0 is left alone.
+struct FllmAdjustRow {
+    float repetition_penalty;   // 1: off
+    float presence_penalty;
+    float frequency_penalty;
+    int32_t seen_off, seen_len;
+    int32_t bias_off, bias_len;
+    int32_t blocked_off, blocked_len;
+    int32_t last_row;           // -1: none
+};
+// logits: float32 [rows, vocab], changed in place; one record a row; the id arrays may be null when no row uses them
+int fllm_adjust_logits(float *logits, int rows, int vocab, const struct FllmAdjustRow *row_records, const int32_t *seen_ids,
+                       const int32_t *seen_counts, const int32_t *bias_ids, const float *bias_values, const int32_t *blocked_ids,
+                       const int32_t *last_tokens, hipStream_t stream);
+
 // work: float32 [rows, vocab] scratch.  kinds: 1 every row has a temperature and neither top-k nor top-p (the draw
 // looks at every token: several workgroups share a row), 2 no row is of that kind, 3 some may be.
 int fllm_sample(const float *logits, float *work, const struct FllmSampleRow *params, int32_t *out, int rows, int vocab,

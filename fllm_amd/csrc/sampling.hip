@@ -374,7 +374,7 @@ __device__ uint32_t key_by_histograms(KeyAt key_at, WeightAt weight_at, int n, u
         __syncthreads();
         for (int i = threadIdx.x; i < n; i += kBlock) {
             const uint32_t key = key_at(i);
-            if (key < floor || (known > 0 && (key >> (32 - known)) != prefix)) continue;
+            if (key == 0 || key < floor || (known > 0 && (key >> (32 - known)) != prefix)) continue;     // key 0: not a candidate
             const unsigned long long w = MASS ? units_of(weight_at(i)) : 1ull;
             if (w != 0) atomicAdd(&hist[mask - ((key >> shift) & mask)], w);
         }
@@ -390,15 +390,18 @@ __device__ uint32_t key_by_histograms(KeyAt key_at, WeightAt weight_at, int n, u
 
 // Both thresholds over one list.  `total` comes in as the mass of all finite logits and is replaced by the mass of
 // what top-k keeps when top-k is on.
+// min-p (`min_p` > 0) stands between the two: a candidate that weighs less than min_p (times the largest weight, which
+// is 1) counts for nothing in top-p; the caller leaves such candidates out of the draw itself.
 template <typename Who, typename KeyAt, typename WeightAt>
 __device__ uint32_t thresholds(KeyAt key_at, WeightAt weight_at, int n, int top_k, bool use_k, bool use_p, float top_p,
-                               double total, Cells &cells) {
+                               float min_p, double total, Cells &cells) {
     uint32_t t = 0;
-    if (use_k) {
-        t = key_of_kth_largest<Who>(key_at, n, min(top_k, n), cells);
-        if (use_p) total = mass_from<Who>(key_at, weight_at, n, t, cells);
+    if (use_k) t = key_of_kth_largest<Who>(key_at, n, min(top_k, n), cells);
+    if (use_p) {
+        auto heavy_key_at = [&](int i) { return weight_at(i) >= min_p ? key_at(i) : 0u; };     // min_p 0: every candidate
+        if (use_k || min_p > 0.f) total = mass_from<Who>(heavy_key_at, weight_at, n, t > 1u ? t : 1u, cells);     // key 0: left out
+        t = key_of_mass<Who>(heavy_key_at, weight_at, n, t, (double)top_p * total, cells);
     }
-    if (use_p) t = key_of_mass<Who>(key_at, weight_at, n, t, (double)top_p * total, cells);
     return t;
 }
 
@@ -430,9 +433,9 @@ __device__ __forceinline__ void for_each_token(const float *__restrict__ src, in
     if ((int)threadIdx.x < vocab - done) f(done + (int)threadIdx.x, src[done + threadIdx.x]);
 }
 
-// a row with a temperature and neither top-k nor top-p: the draw looks at every token
+// a row with a temperature and none of top-k, top-p and min-p: the draw looks at every token
 __device__ __forceinline__ bool draws_from_all(const FllmSampleRow &p, int vocab) {
-    return p.temperature > 1e-5f && !(p.top_k > 0 && p.top_k < vocab) && !(p.top_p > 0.f && p.top_p < 1.f);
+    return p.temperature > 1e-5f && !(p.top_k > 0 && p.top_k < vocab) && !(p.top_p > 0.f && p.top_p < 1.f) && !(p.min_p > 0.f);
 }
 
 // Such rows spend their time on the random numbers of all tokens, so several workgroups share a row, in two
@@ -500,15 +503,23 @@ sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const 
     const float inv_t = (float)(1.0 / (double)p.temperature);
     const bool use_k = p.top_k > 0 && p.top_k < vocab;
     const bool use_p = p.top_p > 0.f && p.top_p < 1.f;
+    const bool use_m = p.min_p > 0.f;
+    const float min_p = use_m ? p.min_p : 0.f;
+    // min-p keeps the tokens with exp((v - max) / T) >= min_p: none of them lies below this bin (one to spare for rounding)
+    int min_p_bin = kBins;
+    if (use_m) {
+        const float reach = -logf(min_p) * p.temperature;      // max - v of the lightest token that stays, about
+        min_p_bin = reach < 63.f ? min(kBins, bin_of(m - reach, m) + 1) : kBins;
+    }
     int count = vocab;                       // tokens the draw looks at: all of them, or the list
     uint32_t threshold = 0;                  // key below which a listed token is out
-    if (use_k || use_p) {
+    if (use_k || use_p || use_m) {
         for (int i = threadIdx.x; i < kBins; i += kBlock) bins[i] = 0;
         __syncthreads();
         double total = 0.0;                  // mass of all finite logits (top-p without top-k)
         unsigned long long reach = 0;        // what this thread put into the histogram, in its units (top-p)
         unsigned long long all_units = 0;    // the same over the workgroup
-        for_each_token(src, vocab, [&](int, float raw) {
+        if (use_k || use_p) for_each_token(src, vocab, [&](int, float raw) {
             const float v = usable(raw);
             if (!(v > -INFINITY)) return;
             const int b = bin_of(v, m);
@@ -522,16 +533,17 @@ sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const 
                 if (b < kBins && fixed != 0) atomicAdd(&bins[b], fixed);
             }
         });
-        int last_bin;
+        int last_bin = kBins;
         if (use_k) {
             last_bin = find_bin(bins, (unsigned long long)p.top_k, cells);
-        } else {
+        } else if (use_p) {
             total = WholeBlock::sum(total, cells);
             // the sum of every thread's share, far tokens included: integers, the same in any order
             all_units = block_units(reach, cells);
             last_bin = find_bin(bins, (unsigned long long)((double)p.top_p * (double)all_units), cells);
             if (last_bin < kBins) last_bin++;   // a bin to spare: the histogram's sums are rounded, the exact ones decide
         }
+        last_bin = min(last_bin, min_p_bin);    // what every filter keeps lies within what any one of them keeps
         // gather the tokens up to that bin: thread t's tokens in the order it meets them, behind those of the threads before it
         int mine = 0;
         for_each_token(src, vocab, [&](int, float raw) {
@@ -556,7 +568,7 @@ sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const 
             if (threadIdx.x < kWave) {
                 const uint32_t t = thresholds<OneWave>([&](int i) { return ordered_key(logit_of[i]); },
                                                        [&](int i) { return weight_of[i]; }, count, p.top_k, use_k, use_p,
-                                                       p.top_p, total, cells);
+                                                       p.top_p, min_p, total, cells);
                 if (threadIdx.x == 0) cells.key = t;
             }
             __syncthreads();
@@ -565,32 +577,38 @@ sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const 
             // a long list: histograms over the keys' bits, weights in units of 2^-40 (the histogram's memory again)
             auto key_at = [&](int i) { return ordered_key(usable(src[list[i]])); };
             auto weight_at = [&](int i) { return expf((usable(src[list[i]]) - m) * inv_t); };
+            // top-p looks at what top-k and min-p left: a candidate below min_p has key 0 there
+            auto heavy_key_at = [&](int i) {
+                const float v = usable(src[list[i]]);
+                return expf((v - m) * inv_t) >= min_p ? ordered_key(v) : 0u;
+            };
             uint32_t t = 0;
             unsigned long long whole = all_units;        // top-p alone: the mass of every finite logit, listed or not
-            if (use_k) {
-                t = key_by_histograms<false>(key_at, weight_at, count, 0u, (unsigned long long)min(p.top_k, count), bins, cells);
-                if (use_p) {
+            if (use_k) t = key_by_histograms<false>(key_at, weight_at, count, 0u, (unsigned long long)min(p.top_k, count), bins, cells);
+            if (use_p) {
+                if (use_k || use_m) {
                     unsigned long long mine = 0;
-                    for (int i = threadIdx.x; i < count; i += kBlock)
-                        if (key_at(i) >= t) mine += units_of(weight_at(i));
+                    for (int i = threadIdx.x; i < count; i += kBlock) {
+                        const uint32_t key = heavy_key_at(i);
+                        if (key != 0 && key >= t) mine += units_of(weight_at(i));
+                    }
                     whole = block_units(mine, cells);
                 }
-            }
-            if (use_p) {
                 unsigned long long target = (unsigned long long)((double)p.top_p * (double)whole);
                 if (target == 0) target = 1;
-                t = key_by_histograms<true>(key_at, weight_at, count, t, target, bins, cells);
+                t = key_by_histograms<true>(heavy_key_at, weight_at, count, t, target, bins, cells);
             }
             threshold = t;
         }
     }
     // Gumbel-max over what is left: the largest of (v - max) / T - ln(-ln u), u the token's uniform number
     Pick best = {-INFINITY, kNone};
-    const bool whole = !(use_k || use_p);
+    const bool whole = !(use_k || use_p || use_m);
     for (int i = threadIdx.x; i < count; i += kBlock) {
         const int id = whole ? i : list[i];
         const float v = usable(src[id]);
         if (!(v > -INFINITY) || ordered_key(v) < threshold) continue;
+        if (use_m && expf((v - m) * inv_t) < min_p) continue;
         const float u = uniform_of(p.seed, p.draw, (uint32_t)id);
         const Pick here = {(v - m) * inv_t - logf(-logf(u)), id};
         best = better_of(best, here);
@@ -680,6 +698,65 @@ extern "C" int fllm_argmax_static(const float *logits, int32_t *out, int rows, i
     hipLaunchKernelGGL(argmax_split_kernel, dim3(rows, parts), dim3(kBlock), 0, stream, logits, out, vocab, parts, per_part, pv, pi,
                        counters);
     return fllm_check_launch("argmax_static");
+}
+
+// ---------------------------------------------------------------------------------------------
+// What a request asks to be done to its logits before a token is chosen
+// ---------------------------------------------------------------------------------------------
+// The reference's order (rust/engine/src/sampling.rs:220-229, :252-274): ids that may not be chosen yet go to -inf;
+// every token seen before is penalised once (divided by the repetition penalty when its logit is positive,
+// multiplied otherwise; then presence + frequency * count taken off); biases are added.  The host lists the tokens
+// seen with their counts; the token that the step before chose may still be on the device only (steps launched
+// ahead): `last_tokens[last_row]` then counts once more, as an entry of its own if the list does not hold it.
+namespace {
+constexpr int kAdjustBlock = 256;
+
+__device__ __forceinline__ float penalised(float v, const FllmAdjustRow &a, int count) {
+    if (fabsf(a.repetition_penalty - 1.f) >= 1e-5f) v = v > 0.f ? v / a.repetition_penalty : v * a.repetition_penalty;
+    return v - (a.presence_penalty + a.frequency_penalty * (float)count);
+}
+
+__global__ void __launch_bounds__(kAdjustBlock)
+adjust_logits_kernel(float *__restrict__ logits, int vocab, const FllmAdjustRow *__restrict__ rows, const int32_t *__restrict__ seen_ids,
+                     const int32_t *__restrict__ seen_counts, const int32_t *__restrict__ bias_ids, const float *__restrict__ bias_values,
+                     const int32_t *__restrict__ blocked_ids, const int32_t *__restrict__ last_tokens) {
+    __shared__ int last_was_listed;
+    const FllmAdjustRow a = rows[blockIdx.x];
+    float *w = logits + (size_t)blockIdx.x * vocab;
+    const int last = a.last_row >= 0 ? last_tokens[a.last_row] : -1;
+    if (threadIdx.x == 0) last_was_listed = 0;
+    __syncthreads();
+    for (int j = threadIdx.x; j < a.seen_len; j += kAdjustBlock) {        // ids of a row are distinct: no two threads meet
+        const int id = seen_ids[a.seen_off + j];
+        if (id < 0 || id >= vocab) continue;
+        int count = seen_counts[a.seen_off + j];
+        if (id == last) count++, last_was_listed = 1;
+        w[id] = penalised(w[id], a, count);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0 && last >= 0 && last < vocab && !last_was_listed) w[last] = penalised(w[last], a, 1);
+    __syncthreads();
+    for (int j = threadIdx.x; j < a.bias_len; j += kAdjustBlock) {
+        const int id = bias_ids[a.bias_off + j];
+        if (id >= 0 && id < vocab) w[id] += bias_values[a.bias_off + j];
+    }
+    __syncthreads();
+    for (int j = threadIdx.x; j < a.blocked_len; j += kAdjustBlock) {
+        const int id = blocked_ids[a.blocked_off + j];
+        if (id >= 0 && id < vocab) w[id] = -INFINITY;
+    }
+}
+}  // namespace
+
+extern "C" int fllm_adjust_logits(float *logits, int rows, int vocab, const FllmAdjustRow *row_records, const int32_t *seen_ids,
+                                  const int32_t *seen_counts, const int32_t *bias_ids, const float *bias_values,
+                                  const int32_t *blocked_ids, const int32_t *last_tokens, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && vocab > 0, "adjust_logits: bad sizes rows=%d vocab=%d", rows, vocab);
+    if (rows == 0) return 0;
+    FLLM_REQUIRE(logits != nullptr && row_records != nullptr, "adjust_logits: logits and row records are required");
+    hipLaunchKernelGGL(adjust_logits_kernel, dim3(rows), dim3(kAdjustBlock), 0, stream, logits, vocab, row_records, seen_ids,
+                       seen_counts, bias_ids, bias_values, blocked_ids, last_tokens);
+    return fllm_check_launch("adjust_logits");
 }
 
 extern "C" int fllm_sample(const float *logits, float *work, const FllmSampleRow *params, int32_t *out, int rows,

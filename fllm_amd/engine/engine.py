@@ -184,6 +184,7 @@ class Engine:
         self.stats.rows_total += rows
         self.stats.max_rows = max(self.stats.max_rows, rows)
         requests = [SampleRequest(seqs[sid].sampling, seqs[sid].sampling.seed_for(sid), seqs[sid].draws) for sid in sampled]
+        self._adjust(logits, sampled, row_of, earlier)
         launched = _InFlight(sampled, [], self.sampler.launch(logits, requests))
         # queued now, before the next step is launched behind it: reading these tokens must not wait for that step
         launched.on_host = self.sampler.start_read(launched.tokens)
@@ -205,6 +206,23 @@ class Engine:
             events = self._resolve(launched)
         self.stats.forward_s += time.perf_counter() - t1
         return events
+
+    def _adjust(self, logits, sampled: List[int], row_of: Dict[int, int], earlier: Optional[_InFlight]) -> None:
+        """Penalties, biases and blocked ids of the requests that ask for any, on the step's logits before a token is
+        chosen.  A request whose newest token is still a placeholder (the step in flight chose it) has it counted on
+        the device, from that step's tokens."""
+        seqs = self.scheduler.sequences
+        if not any(seqs[sid].sampling.adjusts_logits(seqs[sid].output_len) for sid in sampled):
+            return
+        from ..sampling.adjust import SeenTokens, row_for
+        rows = []
+        for sid in sampled:
+            seq = seqs[sid]
+            pending = row_of[sid] if seq.tokens[-1] == PENDING else None
+            if seq.seen is None and seq.sampling.penalizes:
+                seq.seen = SeenTokens()
+            rows.append(row_for(seq.sampling, seq.tokens, seq.prompt_len, pending, self.eos_token_ids, seq.seen))
+        self.sampler.adjust(logits, rows, earlier.tokens if earlier is not None else None)
 
     def _resolve(self, step: _InFlight) -> List[TokenEvent]:
         """Reads a launched step's tokens (waits for the device), puts them where the placeholders

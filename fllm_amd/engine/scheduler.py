@@ -57,6 +57,7 @@ class Sequence:
     preempted: bool = False
     arrival: int = 0
     draws: int = 0                          # random draws taken so far
+    seen: Optional[object] = None           # counts of the tokens so far, kept by the engine for requests with penalties
 
     @property
     def output_len(self) -> int:

@@ -7,7 +7,7 @@ library cannot be loaded or built, constructing `Ops` raises.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+from typing import Optional, Sequence
 
 import torch
 
@@ -24,10 +24,11 @@ class KernelError(RuntimeError):
 
 class SampleRow(ctypes.Structure):
     _fields_ = [("temperature", ctypes.c_float), ("top_p", ctypes.c_float), ("top_k", ctypes.c_int32),
-                ("pad", ctypes.c_int32), ("seed", ctypes.c_uint64), ("draw", ctypes.c_uint64)]
+                ("min_p", ctypes.c_float), ("seed", ctypes.c_uint64), ("draw", ctypes.c_uint64)]
 
 
 SAMPLE_ROW_BYTES = ctypes.sizeof(SampleRow)
+ADJUST_ROW_WORDS = 10         # int32 words of one FllmAdjustRow
 assert SAMPLE_ROW_BYTES == 32
 
 _lib = None
@@ -77,6 +78,7 @@ def load_library(build_if_missing: bool = True):
         "fllm_gate_up_swiglu": [c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_carry_ids": [c_void, c_void, c_void, c_int, c_int, c_void],
         "fllm_sample": [c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
+        "fllm_adjust_logits": [c_void, c_int, c_int, c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_void],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -482,6 +484,30 @@ class Ops:
         _dense(out, "out", torch.int32, (rows,))
         self._check(self.lib.fllm_argmax(_ptr(logits), _ptr(out), rows, vocab, self._stream()))
         return out
+
+    def adjust_logits(self, logits: torch.Tensor, packed: torch.Tensor, sections: Sequence[int],
+                      last_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Penalties, biases and blocked ids on float32 logits [rows, vocab], in place (fllm_adjust_logits).  `packed`: one
+        int32 device tensor holding, one behind the other, the row records (10 words a row: the three penalties as
+        float bits, then seen_off, seen_len, bias_off, bias_len, blocked_off, blocked_len, last_row), the seen ids, the
+        seen counts, the bias ids, the bias values (float bits) and the blocked ids; `sections`: (entries of the seen
+        lists, entries of the bias lists, blocked ids), each over all rows.
+        `last_tokens`: int32 device tensor that the records' last_row points into."""
+        rows, vocab = logits.shape
+        seen, bias, blocked = (int(n) for n in sections)
+        _dense(logits, "logits", torch.float32)
+        _dense(packed, "packed", torch.int32, (rows * ADJUST_ROW_WORDS + 2 * seen + 2 * bias + blocked,))
+        if last_tokens is not None:
+            _dense(last_tokens, "last_tokens", torch.int32)
+        base = packed.data_ptr()
+        at = rows * ADJUST_ROW_WORDS
+        seen_ids, seen_counts = base + 4 * at, base + 4 * (at + seen)
+        at += 2 * seen
+        bias_ids, bias_values = base + 4 * at, base + 4 * (at + bias)
+        at += 2 * bias
+        self._check(self.lib.fllm_adjust_logits(_ptr(logits), rows, vocab, base, seen_ids, seen_counts, bias_ids, bias_values,
+                                                base + 4 * at, _ptr(last_tokens), self._stream()))
+        return logits
 
     def sample(self, logits: torch.Tensor, work: torch.Tensor, params: torch.Tensor, out: torch.Tensor,
                kinds: int = 3) -> torch.Tensor:

@@ -20,6 +20,13 @@ class SamplingParams:
     max_tokens: int = 16              # generated tokens at most
     stop_token_ids: Tuple[int, ...] = ()
     ignore_eos: bool = False
+    min_p: float = 0.0                # drops what weighs less than min_p times the likeliest token; 0: off
+    repetition_penalty: float = 1.0   # logits of tokens seen before: divided by it when positive, multiplied otherwise; 1: off
+    presence_penalty: float = 0.0     # taken off the logit of every token seen before
+    frequency_penalty: float = 0.0    # taken off once for every time the token was seen
+    repeat_last_n: int = -1           # tokens of the history (prompt and generated) the penalties look at; negative: all
+    logit_bias: Tuple[Tuple[int, float], ...] = ()   # (token id, what is added to its logit)
+    min_tokens: int = 0               # no end-of-sequence or stop id before this many tokens were generated
 
     def __post_init__(self):
         if self.temperature < 0.0:
@@ -30,7 +37,27 @@ class SamplingParams:
             raise ValueError("top_k must be nonnegative")
         if self.max_tokens <= 0:
             raise ValueError("max_tokens must be positive")
+        if not 0.0 <= self.min_p <= 1.0:
+            raise ValueError("min_p must be in [0, 1]")
+        if not self.repetition_penalty > 0.0:
+            raise ValueError("repetition_penalty must be positive")
+        if self.min_tokens < 0:
+            raise ValueError("min_tokens must be nonnegative")
         object.__setattr__(self, "stop_token_ids", tuple(int(t) for t in self.stop_token_ids))
+        bias = tuple((int(t), float(b)) for t, b in self.logit_bias)
+        if any(t < 0 for t, _ in bias) or len({t for t, _ in bias}) != len(bias):
+            raise ValueError("logit_bias needs nonnegative token ids, each once")
+        object.__setattr__(self, "logit_bias", bias)
+
+    @property
+    def penalizes(self) -> bool:
+        """Whether tokens seen before change the logits (sampling.rs:98-107: what keeps a request off the plain argmax)."""
+        return abs(self.repetition_penalty - 1.0) >= 1e-5 or self.presence_penalty != 0.0 or self.frequency_penalty != 0.0
+
+    def adjusts_logits(self, generated: int) -> bool:
+        """Whether the logits of the next token are changed before a token is chosen: penalties, biases, or
+        end and stop ids that `min_tokens` still blocks after `generated` tokens."""
+        return self.penalizes or bool(self.logit_bias) or generated < self.min_tokens
 
     @property
     def greedy(self) -> bool:

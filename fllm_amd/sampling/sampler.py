@@ -17,7 +17,7 @@ class SampleRequest:
     draw: int
 
 
-_RECORD = 32   # bytes of one row record: float temperature, float top_p, int32 top_k, int32 pad, uint64 seed, uint64 draw
+_RECORD = 32   # bytes of one row record: float temperature, float top_p, int32 top_k, float min_p, uint64 seed, uint64 draw
 
 
 def pack_rows(rows: Sequence[SampleRequest]) -> torch.Tensor:
@@ -26,23 +26,36 @@ def pack_rows(rows: Sequence[SampleRequest]) -> torch.Tensor:
     raw = bytearray()
     for r in rows:
         p = r.params
-        raw += struct.pack("<ffiiQQ", float(p.temperature), float(p.top_p), int(p.top_k), 0,
+        raw += struct.pack("<ffifQQ", float(p.temperature), float(p.top_p), int(p.top_k), float(p.min_p),
                            int(r.seed) & ((1 << 64) - 1), int(r.draw))
     return torch.frombuffer(raw, dtype=torch.uint8).view(len(rows), _RECORD).clone()
 
 
 def draws_from_all(p: SamplingParams, vocab: int) -> bool:
-    """A temperature and neither top-k nor top-p: the kernel's own test, on the float32 values that the row record
+    """A temperature and none of top-k, top-p and min-p: the kernel's own test, on the float32 values that the row record
     holds (a temperature or top-p that rounds across its limit must be judged as the kernel judges it)."""
     import struct
-    temperature, top_p = struct.unpack("<ff", struct.pack("<ff", float(p.temperature), float(p.top_p)))
+    temperature, top_p, min_p = struct.unpack("<fff", struct.pack("<fff", float(p.temperature), float(p.top_p), float(p.min_p)))
     limit = struct.unpack("<f", struct.pack("<f", 1e-5))[0]
-    return temperature > limit and not (0 < int(p.top_k) < vocab) and not (0.0 < top_p < 1.0)
+    return temperature > limit and not (0 < int(p.top_k) < vocab) and not (0.0 < top_p < 1.0) and not min_p > 0.0
 
 
 class Sampler:
     def __init__(self, rt):
         self.rt = rt
+
+    def adjust(self, logits: torch.Tensor, rows, last_tokens=None) -> torch.Tensor:
+        """Penalties, biases and blocked ids of the rows that ask for any (`rows`: one `AdjustRow` or None a row of
+        `logits`), on the logits in place; nothing is launched when no row asks.  `last_tokens`: the device tensor that
+        the rows' `last_row` points into."""
+        if all(r is None for r in rows):
+            return logits
+        from .adjust import pack
+        packed, sections = pack(rows)
+        if logits.is_cuda:
+            packed = packed.pin_memory().to(logits.device, non_blocking=True)
+        self.rt.ops.adjust_logits(logits, packed, sections, last_tokens)
+        return logits
 
     def sample(self, logits: torch.Tensor, rows: Sequence[SampleRequest]) -> List[int]:
         """`logits`: float32 [len(rows), vocab] on the device.  Returns one token id per row."""

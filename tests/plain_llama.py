@@ -247,12 +247,48 @@ def philox_uniform_many(seed, draw, indices):
     return ((w + np.float32(0.5)) / np.float32(16777216.0)).astype(np.float32)
 
 
-def device_survivors(logits, temperature, top_k, top_p):
+def apply_generation_controls(logits, min_tokens, generated, eos_ids, stop_token_ids):
+    """rust/engine/src/sampling.rs:220-229: while fewer than `min_tokens` tokens were generated, neither an
+    end-of-sequence id nor a stop id can be chosen.  Returns a float32 copy."""
+    out = np.asarray(logits, dtype=np.float32).copy()
+    if generated < min_tokens:
+        for t in list(eos_ids) + list(stop_token_ids):
+            if 0 <= t < len(out):
+                out[t] = -np.inf
+    return out
+
+
+def apply_penalties(logits, history, repetition_penalty=1.0, presence_penalty=0.0, frequency_penalty=0.0, repeat_last_n=-1,
+                    logit_bias=()):
+    """rust/engine/src/sampling.rs:252-274 and :579-598: over the last `repeat_last_n` tokens of the history (all of
+    them when negative): every distinct token's logit is divided by the repetition penalty when positive and multiplied
+    by it otherwise (once a token, and only if the penalty differs from 1 by 1e-5 or more); then presence +
+    frequency * count is taken off; then the biases are added.  float32 arithmetic; returns a copy."""
+    out = np.asarray(logits, dtype=np.float32).copy()
+    tokens = list(history) if repeat_last_n < 0 else list(history)[max(0, len(history) - repeat_last_n):]
+    tokens = [t for t in tokens if 0 <= t < len(out)]
+    counts = {}
+    for t in tokens:
+        counts[t] = counts.get(t, 0) + 1
+    rep = np.float32(repetition_penalty)
+    if abs(float(rep) - 1.0) >= 1e-5:
+        for t in counts:
+            out[t] = out[t] / rep if out[t] > 0 else out[t] * rep
+    for t, n in counts.items():
+        out[t] = out[t] - (np.float32(presence_penalty) + np.float32(frequency_penalty) * np.float32(n))
+    for t, b in logit_bias:
+        if 0 <= t < len(out):
+            out[t] = out[t] + np.float32(b)
+    return out
+
+
+def device_survivors(logits, temperature, top_k, top_p, min_p=0.0):
     """The tokens the reference's device sampler still draws from, as a float32 array of logits
     with -inf for the others (rust/engine/cuda/sampling.cu:253-330), with sorting in place of its
     bisections: non-finite logits never survive; top-k keeps everything not below the k-th
-    largest value (ties kept); top-p keeps the largest values until their mass reaches top_p of the
-    total (ties at the threshold kept)."""
+    largest value (ties kept); min-p (:294-300) then drops what weighs less than min_p times the
+    largest weight, exp((v - max) / T) < min_p in float32; top-p keeps the largest values until their mass
+    reaches top_p of the total of what is left (ties at the threshold kept)."""
     w = np.asarray(logits, dtype=np.float32).copy()
     w[~np.isfinite(w)] = -np.inf
     if not np.isfinite(w).any():
@@ -262,6 +298,13 @@ def device_survivors(logits, temperature, top_k, top_p):
     if 0 < top_k < len(w):
         kth = np.sort(w)[::-1][top_k - 1]
         w[w < kth] = -np.inf
+    if min_p > 0.0:
+        alive = np.isfinite(w)
+        e = np.exp(((w[alive] - m) * inv_t).astype(np.float32)).astype(np.float32)
+        keep = np.flatnonzero(alive)[e >= np.float32(min_p)]
+        cut = np.full(len(w), -np.inf, dtype=np.float32)
+        cut[keep] = w[keep]
+        w = cut
     if 0.0 < top_p < 1.0:
         alive = np.isfinite(w)
         e = np.where(alive, np.exp(((w - m) * inv_t).astype(np.float32)).astype(np.float64), 0.0)
@@ -274,7 +317,7 @@ def device_survivors(logits, temperature, top_k, top_p):
     return w
 
 
-def device_sample(logits, temperature, top_k, top_p, seed, draw):
+def device_sample(logits, temperature, top_k, top_p, seed, draw, min_p=0.0):
     """rust/engine/cuda/sampling.cu:253-352: temperature <= 1e-5 is greedy; otherwise the token
     is the argmax over the survivors of (logit - max) / T - ln(-ln u_i),
     u_i = philox_uniform(seed, draw, i), lowest id on ties."""
@@ -284,7 +327,7 @@ def device_sample(logits, temperature, top_k, top_p, seed, draw):
         return 0
     if temperature <= 1e-5:
         return greedy(finite)
-    w = device_survivors(logits, temperature, top_k, top_p)
+    w = device_survivors(logits, temperature, top_k, top_p, min_p)
     m = finite.max()
     inv_t = np.float32(1.0 / float(temperature))
     alive = np.flatnonzero(np.isfinite(w))

@@ -165,12 +165,38 @@ class ReferenceOps:
             out[r] = 0 if not np.isfinite(row).any() else plain_llama.greedy(row)
         return out
 
+    def adjust_logits(self, logits, packed, sections, last_tokens=None):
+        """The packed lists of `Ops.adjust_logits`, taken apart here and applied with the plain functions."""
+        rows, vocab = logits.shape
+        seen, bias, blocked = (int(n) for n in sections)
+        words = packed.cpu().numpy().astype(np.int32)
+        at = rows * 10
+        seen_ids, seen_counts = words[at:at + seen], words[at + seen:at + 2 * seen]
+        at += 2 * seen
+        bias_ids, bias_values = words[at:at + bias], words[at + bias:at + 2 * bias].view(np.float32)
+        blocked_ids = words[at + 2 * bias:at + 2 * bias + blocked]
+        for r in range(rows):
+            rec = words[r * 10:(r + 1) * 10]
+            rep, pres, freq = (float(v) for v in rec[:3].view(np.float32))
+            seen_off, seen_len, bias_off, bias_len, blocked_off, blocked_len, last_row = (int(v) for v in rec[3:])
+            history = []
+            for t, n in zip(seen_ids[seen_off:seen_off + seen_len], seen_counts[seen_off:seen_off + seen_len]):
+                history += [int(t)] * int(n)
+            if last_row >= 0:
+                history.append(int(last_tokens[last_row]))
+            row = plain_llama.apply_penalties(logits[r].float().cpu().numpy(), history, rep, pres, freq, -1,
+                                              list(zip(bias_ids[bias_off:bias_off + bias_len].tolist(),
+                                                       bias_values[bias_off:bias_off + bias_len].tolist())))
+            row[[int(t) for t in blocked_ids[blocked_off:blocked_off + blocked_len] if 0 <= t < vocab]] = -np.inf
+            logits[r] = torch.from_numpy(row).to(logits.dtype)
+        return logits
+
     def sample(self, logits, work, params, out, kinds=3):
         raw = params.cpu().numpy().tobytes()
         rec = np.frombuffer(raw, dtype=np.dtype([("temperature", "<f4"), ("top_p", "<f4"), ("top_k", "<i4"),
-                                                 ("pad", "<i4"), ("seed", "<u8"), ("draw", "<u8")]))
+                                                 ("min_p", "<f4"), ("seed", "<u8"), ("draw", "<u8")]))
         for r in range(logits.shape[0]):
             p = rec[r]
             out[r] = plain_llama.device_sample(logits[r].float().cpu().numpy(), float(p["temperature"]), int(p["top_k"]),
-                                               float(p["top_p"]), int(p["seed"]), int(p["draw"]))
+                                               float(p["top_p"]), int(p["seed"]), int(p["draw"]), float(p["min_p"]))
         return out

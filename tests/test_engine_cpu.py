@@ -333,3 +333,62 @@ def test_rows_that_draw_from_all_tokens_are_told_as_the_kernel_tells_them():
     assert not draws_from_all(P(temperature=0.8, top_p=0.9), 100)
     assert not draws_from_all(P(temperature=1.0000000001e-5), 100)           # float32: the limit itself, greedy in the kernel
     assert draws_from_all(P(temperature=0.8, top_p=0.999999999), 100)        # float32: one, no filter in the kernel
+
+
+def plain_generate(name, prompt, params, eos=()):
+    """Tokens of one request chosen the plain way: the whole sequence through the plain model for every token, then
+    the reference's order of hard controls, penalties and the draw (rust/engine/src/sampling.rs:220-229, :252-274,
+    cuda/sampling.cu)."""
+    cfg = tc.CONFIGS[name]
+    _, spec = model_spec_from_config(cfg)
+    w64 = tc.to_float64(random_tensors(spec, 1, torch.float32))
+    seq = list(prompt)
+    for draw in range(params.max_tokens):
+        row = plain_llama.forward(cfg, w64, seq)[-1].astype(np.float32)
+        row = plain_llama.apply_generation_controls(row, params.min_tokens, len(seq) - len(prompt), eos, params.stop_token_ids)
+        row = plain_llama.apply_penalties(row, seq, params.repetition_penalty, params.presence_penalty, params.frequency_penalty,
+                                          params.repeat_last_n, params.logit_bias)
+        token = plain_llama.device_sample(row, params.temperature, params.top_k, params.top_p, params.seed or 0, draw, params.min_p)
+        seq.append(token)
+        if params.stops_on(token, eos):
+            break
+    return seq[len(prompt):]
+
+
+@pytest.mark.parametrize("ahead", [False, True])
+def test_penalties_biases_min_tokens_and_min_p_match_the_plain_order(ahead):
+    """Requests that ask for what else the reference samples with: penalties on the tokens seen (prompt and
+    generated, all of them or a window), biases, end and stop ids blocked for the first tokens, min-p; beside a
+    request that asks for nothing.  With steps launched ahead the newest token of a request is counted on the device."""
+    plain = SamplingParams(max_tokens=12)
+    free = plain_generate("A", PROMPTS_A[1], plain)
+    loops = SamplingParams(max_tokens=12, repetition_penalty=1.6, presence_penalty=0.4, frequency_penalty=0.3)
+    window = SamplingParams(max_tokens=12, repetition_penalty=1.3, frequency_penalty=0.5, repeat_last_n=3)
+    eos = (free[0], free[1])
+    held = SamplingParams(max_tokens=8, min_tokens=5, stop_token_ids=(free[2],), logit_bias=((free[3], 4.0), (7, -2.0)))
+    drawn = SamplingParams(max_tokens=10, temperature=0.9, top_k=30, min_p=0.08, top_p=0.9, seed=77, presence_penalty=0.6)
+    cases = [("loops", PROMPTS_A[1], loops), ("window", PROMPTS_A[2], window), ("held", PROMPTS_A[1], held),
+             ("drawn", PROMPTS_A[0], drawn), ("plain", PROMPTS_A[1], plain)]
+    engine = make_engine(ahead=ahead, eos_token_ids=eos)
+    for name, prompt, params in cases:
+        engine.add_request(name, prompt, params)
+    got = {name: [] for name, _, _ in cases}
+    while engine.has_unfinished():
+        for ev in engine.step():
+            got[ev.request_id].append(ev.token_id)
+    for name, prompt, params in cases:
+        assert got[name] == plain_generate("A", prompt, params, eos), name
+    assert got["loops"] != free and got["window"] != free            # the penalties do change the tokens
+    assert len(got["held"]) >= 5 and not set(got["held"][:5]) & (set(eos) | {free[2]})
+    assert got["plain"] == free[:1]                                  # the first token the model gives is an end id here
+    engine.runner.cache.check_invariants()
+
+
+def test_sampling_params_refuse_what_makes_no_sense():
+    for bad in (dict(min_p=1.5), dict(min_p=-0.1), dict(repetition_penalty=0.0), dict(min_tokens=-1),
+                dict(logit_bias=((3, 1.0), (3, 2.0))), dict(logit_bias=((-1, 1.0),))):
+        with pytest.raises(ValueError):
+            SamplingParams(**bad)
+    p = SamplingParams(presence_penalty=0.5, min_tokens=2)
+    assert p.penalizes and p.adjusts_logits(0) and SamplingParams(min_tokens=2).adjusts_logits(1)
+    assert not SamplingParams(min_tokens=2).adjusts_logits(2) and not SamplingParams(repetition_penalty=1.000001).penalizes

@@ -103,7 +103,7 @@ def test_steps_launched_ahead_give_the_same_tokens(dtype):
     same as when every step waits for the last: greedy and sampled, graphs and eager steps, few pages."""
     prompts = [tc.random_ids(n, 512, 20 + n) for n in PROMPT_LENGTHS["B"]]
     for params in (SamplingParams(max_tokens=24), SamplingParams(max_tokens=24, temperature=0.8, top_p=0.9, seed=7)):
-        want = make_engine("B", dtype).generate(prompts, params)
+        want = make_engine("B", dtype, ahead=False).generate(prompts, params)
         ahead = make_engine("B", dtype, ahead=True)
         assert ahead.generate(prompts, params) == want
         assert ahead.runner.graph_replays > 0
@@ -112,9 +112,57 @@ def test_steps_launched_ahead_give_the_same_tokens(dtype):
         eager.runner.use_graphs = False
         assert eager.generate(prompts, params) == want
     tight = make_engine("B", dtype, ahead=True, num_blocks=26)
-    assert tight.generate(prompts, SamplingParams(max_tokens=24)) == make_engine("B", dtype).generate(prompts, SamplingParams(max_tokens=24))
+    assert tight.generate(prompts, SamplingParams(max_tokens=24)) == make_engine("B", dtype, ahead=False).generate(prompts, SamplingParams(max_tokens=24))
     assert tight.stats.preemptions >= 1
     tight.runner.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_penalties_biases_min_tokens_and_min_p(dtype):
+    """What else the reference samples with, on the device: penalties over the tokens seen (all of them, or a
+    window), biases, end and stop ids blocked for the first tokens, min-p.  Steps launched ahead (the newest token of
+    a request is counted from the device's copy) give the tokens of steps that wait; in float32 they are the plain
+    order's tokens, computed from the plain model's logits."""
+    cfg = tc.CONFIGS["A"]
+    prompts = [tc.random_ids(n, cfg["vocab_size"], 10 + n) for n in PROMPT_LENGTHS["A"]]
+    free = make_engine("A", dtype).generate([prompts[1]], SamplingParams(max_tokens=12))[0]
+    eos = (free[0], free[1])
+    cases = [("loops", prompts[1], SamplingParams(max_tokens=12, repetition_penalty=1.6, presence_penalty=0.4, frequency_penalty=0.3)),
+             ("window", prompts[2], SamplingParams(max_tokens=12, repetition_penalty=1.3, frequency_penalty=0.5, repeat_last_n=3)),
+             ("held", prompts[1], SamplingParams(max_tokens=8, min_tokens=5, stop_token_ids=(free[2],), logit_bias=((free[3], 4.0), (7, -2.0)))),
+             ("drawn", prompts[0], SamplingParams(max_tokens=10, temperature=0.9, top_k=30, min_p=0.08, top_p=0.9, seed=77, presence_penalty=0.6)),
+             ("plain", prompts[1], SamplingParams(max_tokens=12))]
+
+    def run(ahead, graphs=True):
+        engine = make_engine("A", dtype, ahead=ahead, eos_token_ids=eos, max_seqs=8)
+        engine.runner.use_graphs = graphs
+        for name, prompt, params in cases:
+            engine.add_request(name, prompt, params)
+        got = {name: [] for name, _, _ in cases}
+        while engine.has_unfinished():
+            for ev in engine.step():
+                got[ev.request_id].append(ev.token_id)
+        engine.runner.cache.check_invariants()
+        return got
+
+    waited = run(False)
+    assert run(True) == waited and run(True, graphs=False) == waited
+    assert waited["loops"] != free and waited["window"] != free and waited["plain"] == free[:1]
+    assert len(waited["held"]) >= 5 and not set(waited["held"][:5]) & (set(eos) | {free[2]})
+    if dtype == "float32":
+        _, spec = model_spec_from_config(cfg)
+        w64 = tc.to_float64(random_tensors(spec, 1, torch.float32))
+        for name, prompt, params in cases:
+            seq, agree = list(prompt), 0
+            for draw, token in enumerate(waited[name]):
+                row = plain_llama.forward(cfg, w64, seq)[-1].astype(np.float32)
+                row = plain_llama.apply_generation_controls(row, params.min_tokens, draw, eos, params.stop_token_ids)
+                row = plain_llama.apply_penalties(row, seq, params.repetition_penalty, params.presence_penalty,
+                                                  params.frequency_penalty, params.repeat_last_n, params.logit_bias)
+                agree += token == plain_llama.device_sample(row, params.temperature, params.top_k, params.top_p, params.seed or 0,
+                                                            draw, params.min_p)
+                seq.append(token)
+            assert agree >= len(waited[name]) - 1, name          # a near-tie may fall the other way
 
 
 def test_no_garbage_collection_while_a_graph_is_captured():
@@ -154,6 +202,19 @@ def test_command_line(tmp_path):
     assert record["finish_reason"] == "length" and len(record["token_ids"]) == 8
     check_greedy("A", "float32", [prompt], [record["token_ids"]])
     assert "forward_calls=" in proc.stderr
+    # the further sampling options, by the reference's flag names: the tokens of the same options through the entry point
+    first = record["token_ids"]
+    flags = ["--repeat-penalty", "1.5", "--presence-penalty", "0.3", "--frequency-penalty", "0.2", "--repeat-last-n", "6",
+             "--min-tokens", "3", "--stop-token-ids", str(first[0]), "--logit-bias", f"{first[1]}:-5,3:0.5", "--min-p", "0.1",
+             "--temperature", "0.7", "--seed", "5"]
+    proc = subprocess.run(cmd + flags, cwd=ROOT, capture_output=True, text=True, timeout=110)
+    assert proc.returncode == 0, proc.stderr
+    record = json.loads(proc.stdout.strip().splitlines()[0])
+    params = SamplingParams(max_tokens=8, temperature=0.7, seed=5, min_p=0.1, repetition_penalty=1.5, presence_penalty=0.3,
+                            frequency_penalty=0.2, repeat_last_n=6, min_tokens=3, stop_token_ids=(first[0],),
+                            logit_bias=((first[1], -5.0), (3, 0.5)))
+    engine = Engine(folder, dtype="float32", num_blocks=16, max_seqs=2)
+    assert record["token_ids"] == engine.generate([prompt], params)[0] and first[0] not in record["token_ids"][:3]
 
 
 @pytest.mark.parametrize("budget,prompt_len", [(512, 512), (2, 40)])

@@ -667,14 +667,16 @@ def test_sample_matches_the_plain_sampler(ops):
     vocab = 1000
     cases = [SamplingParams(temperature=0.8), SamplingParams(temperature=1.0, top_k=5),
              SamplingParams(temperature=0.7, top_p=0.9), SamplingParams(temperature=1.3, top_k=50, top_p=0.5),
-             SamplingParams(temperature=0.0), SamplingParams(temperature=0.8, top_p=0.01)]
+             SamplingParams(temperature=0.0), SamplingParams(temperature=0.8, top_p=0.01),
+             SamplingParams(temperature=1.0, min_p=0.05), SamplingParams(temperature=1.5, top_k=40, min_p=0.2, top_p=0.8),
+             SamplingParams(temperature=0.9, min_p=0.3, top_p=0.6), SamplingParams(temperature=0.7, min_p=1.0)]
     logits = torch.randn(len(cases), vocab, generator=g) * 2.0
     for draw in range(6):
         reqs = [SampleRequest(p, seed=1234 + i, draw=draw) for i, p in enumerate(cases)]
         out = torch.empty(len(cases), dtype=torch.int32, device=DEV)
         ops.sample(logits.to(DEV), torch.empty(len(cases), vocab, device=DEV), pack_rows(reqs).to(DEV), out)
         for i, p in enumerate(cases):
-            want = plain_llama.device_sample(logits[i].numpy(), p.temperature, p.top_k, p.top_p, 1234 + i, draw)
+            want = plain_llama.device_sample(logits[i].numpy(), p.temperature, p.top_k, p.top_p, 1234 + i, draw, p.min_p)
             assert int(out[i]) == want, (draw, i)
 
 
@@ -700,7 +702,10 @@ def test_sample_thresholds_on_wide_vocabularies(ops, vocab):
              SamplingParams(temperature=1.1, top_k=64), SamplingParams(temperature=1.0, top_k=vocab - 1),
              SamplingParams(temperature=0.7, top_p=0.01), SamplingParams(temperature=1.0, top_p=0.5),
              SamplingParams(temperature=2.5, top_p=0.9), SamplingParams(temperature=4.0, top_p=0.999),
-             SamplingParams(temperature=1.3, top_k=50, top_p=0.5), SamplingParams(temperature=0.9, top_k=2000, top_p=0.95)]
+             SamplingParams(temperature=1.3, top_k=50, top_p=0.5), SamplingParams(temperature=0.9, top_k=2000, top_p=0.95),
+             SamplingParams(temperature=1.0, min_p=0.1), SamplingParams(temperature=3.0, min_p=0.001),       # a long list
+             SamplingParams(temperature=3.0, min_p=0.002, top_p=0.9), SamplingParams(temperature=1.2, top_k=3000, min_p=0.01, top_p=0.9),
+             SamplingParams(temperature=40.0, min_p=1e-30)]                                               # further than the histogram reaches
     for name, row in rows.items():
         logits = row.view(1, vocab).expand(len(cases), vocab).contiguous()
         for draw in range(2):
@@ -708,7 +713,7 @@ def test_sample_thresholds_on_wide_vocabularies(ops, vocab):
             out = torch.empty(len(cases), dtype=torch.int32, device=DEV)
             ops.sample(logits.to(DEV), torch.empty(len(cases), vocab, device=DEV), pack_rows(reqs).to(DEV), out)
             for i, p in enumerate(cases):
-                want = plain_llama.device_sample(row.numpy(), p.temperature, p.top_k, p.top_p, 99 + i, draw)
+                want = plain_llama.device_sample(row.numpy(), p.temperature, p.top_k, p.top_p, 99 + i, draw, p.min_p)
                 assert int(out[i]) == want, (name, draw, i)
 
 
@@ -744,6 +749,37 @@ def test_sample_rows_that_draw_from_all_tokens_share_workgroups(ops, vocab):
     counters = type(ops)._workspaces[torch.cuda.current_device()][: 64 * 1024]
     torch.cuda.synchronize()
     assert int(counters.to(torch.int64).sum()) == 0
+
+
+def test_adjust_logits(ops):
+    """Penalties, biases and blocked ids on rows of logits against the plain functions: a row with everything, a row
+    whose newest token is on the device only and already in its list (it counts once more), one whose newest token
+    is new to the list, a row left alone, ids outside the vocabulary ignored."""
+    from fllm_amd.sampling import SamplingParams
+    from fllm_amd.sampling.adjust import AdjustRow, pack
+    g = gen(41)
+    vocab = 1000
+    logits = torch.randn(5, vocab, generator=g) * 3.0
+    logits[0, 17] = float("nan")
+    last_tokens = torch.tensor([5, 123, 999], dtype=torch.int32)
+    full = SamplingParams(repetition_penalty=1.7, presence_penalty=0.3, frequency_penalty=0.2, logit_bias=((3, 2.5), (17, 1.0), (4000, 9.0)))
+    rows = [AdjustRow(full, {5: 2, 17: 1, 900: 4, 4000: 1, 44: 3}, blocked=(1, 2, 4000)),
+            AdjustRow(SamplingParams(frequency_penalty=0.5), {123: 2, 7: 1}, last_row=1),
+            AdjustRow(SamplingParams(repetition_penalty=0.5), {7: 1}, last_row=2),
+            None,
+            AdjustRow(SamplingParams(min_tokens=3), {}, blocked=(0, 999))]
+    packed, sections = pack(rows)
+    got = ops.adjust_logits(logits.clone().to(DEV), packed.to(DEV), sections, last_tokens.to(DEV)).cpu()
+    histories = [[5, 5, 17, 900, 900, 900, 900, 4000, 44, 44, 44], [123, 123, 7, 123], [7, 999], [], []]
+    for r, row in enumerate(rows):
+        want = logits[r].numpy()
+        if row is not None:
+            p = row.params
+            want = plain_llama.apply_penalties(want, histories[r], p.repetition_penalty, p.presence_penalty, p.frequency_penalty, -1,
+                                               p.logit_bias)
+            want[[t for t in row.blocked if t < vocab]] = -np.inf
+        assert np.array_equal(got[r].numpy(), want, equal_nan=True), r
+    assert torch.equal(got[3], logits[3])
 
 
 def test_sample_depends_only_on_seed_draw_and_logits(ops):

@@ -313,6 +313,40 @@ def test_filters():
     assert np.flatnonzero(np.isfinite(P.device_survivors([0.0, 20.0, 1.0], 1.0, 0, 0.1))).tolist() == [1]
 
 
+def test_min_p_and_the_order_of_the_filters():
+    """The reference's vectors: logits [3, 2, 1, 0, -1] at temperature 1 with min_p 0.3 keep two tokens
+    (rust/engine/src/sampling.rs:1069-1070: e^-1 = 0.37 stays, e^-2 = 0.14 goes); [5, 3, 0] with min_p 0.5 leave
+    token 0 alone (:842-856).  top-k comes first, min-p next, top-p last, each over what the one before left."""
+    alive = lambda logits, **kw: np.flatnonzero(np.isfinite(P.device_survivors(
+        logits, kw.get("t", 1.0), kw.get("top_k", 0), kw.get("top_p", 1.0), kw.get("min_p", 0.0)))).tolist()
+    assert alive([3.0, 2.0, 1.0, 0.0, -1.0], min_p=0.3) == [0, 1]
+    assert alive([5.0, 3.0, 0.0], min_p=0.5) == [0]
+    assert all(P.device_sample([5.0, 3.0, 0.0], 1.0, 0, 1.0, 1, d, min_p=0.5) == 0 for d in range(50))
+    # the weight is taken at the temperature: at T = 2, e^(-2/2) = 0.37 stays where at T = 1 e^-2 went
+    assert alive([3.0, 2.0, 1.0, 0.0, -1.0], min_p=0.3, t=2.0) == [0, 1, 2]
+    # top-p over what min-p left: of [3, 2] (weights 1, 0.37) top_p 0.7 needs only the first; without min-p, of all five, it needs two
+    assert alive([3.0, 2.0, 1.0, 0.0, -1.0], min_p=0.3, top_p=0.7) == [0]
+    assert alive([3.0, 2.0, 1.0, 0.0, -1.0], top_p=0.7) == [0, 1]
+    assert alive([3.0, 3.0, 2.9, 0.0], top_k=1, min_p=0.5) == [0, 1]        # ties of top-k stay, min-p has nothing to add
+
+
+def test_penalties_and_controls():
+    """The reference's vectors: repetition penalty 2 turns logits [4, 6, 1] with token 1 in the history into a win for
+    token 0 (rust/engine/src/sampling.rs:776-791); frequency 1.0 and presence 0.5 over the last 2 tokens of [0, 1, 1]
+    turn [5, 5] into [5, 2.5] (:857-868).  A negative logit is multiplied, not divided; a token counts once for the
+    repetition penalty however often it occurs; biases come last; min_tokens blocks end and stop ids until reached."""
+    assert P.greedy(P.apply_penalties([4.0, 6.0, 1.0], [1], repetition_penalty=2.0)) == 0
+    assert P.apply_penalties([5.0, 5.0], [0, 1, 1], frequency_penalty=1.0, presence_penalty=0.5, repeat_last_n=2).tolist() == [5.0, 2.5]
+    assert P.apply_penalties([5.0, 5.0], [0, 1, 1], frequency_penalty=1.0, presence_penalty=0.5).tolist() == [3.5, 2.5]
+    assert P.apply_penalties([-2.0, 2.0, 1.0], [0, 0, 1], repetition_penalty=2.0).tolist() == [-4.0, 1.0, 1.0]
+    assert P.apply_penalties([1.0, 1.0], [0], repetition_penalty=1.000001).tolist() == [1.0, 1.0]      # as good as 1: off
+    assert P.apply_penalties([1.0, 1.0, 1.0], [7, -1, 1], presence_penalty=0.25, logit_bias=[(2, -3.0), (9, 1.0)]).tolist() == [1.0, 0.75, -2.0]
+    assert P.apply_penalties([4.0], [0], repetition_penalty=2.0, logit_bias=[(0, 1.0)]).tolist() == [3.0]   # the bias after the penalty
+    blocked = P.apply_generation_controls([1.0, 2.0, 3.0, 4.0], 3, 2, [3], [1])
+    assert np.isneginf(blocked[[1, 3]]).all() and blocked[[0, 2]].tolist() == [1.0, 3.0]
+    assert P.apply_generation_controls([1.0, 2.0, 3.0, 4.0], 3, 3, [3], [1]).tolist() == [1.0, 2.0, 3.0, 4.0]
+
+
 def test_draws_follow_the_distribution_and_depend_on_seed_and_draw_only():
     logits = np.array([2.0, 1.0, 0.0, -1.0], dtype=np.float32)
     p = np.exp(logits / 0.8)
