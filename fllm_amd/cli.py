@@ -34,6 +34,7 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--max-num-partial-prefills", type=int, default=0)
     ap.add_argument("--long-prefill-token-threshold", type=int, default=0)
     ap.add_argument("--preemption-mode", default="recompute", choices=["recompute", "none"])
+    ap.add_argument("--scheduling-policy", default="fcfs", choices=["fcfs", "priority"])
     ap.add_argument("--chunked-prefill-policy", default="decode-first", choices=["decode-first", "prefill-first"])
     ap.add_argument("--no-ahead", dest="ahead", action="store_false",
                     help="wait for the tokens of every step before the next one is launched (by default a step is launched "
@@ -52,6 +53,7 @@ def _make_engine(args, model):
                   max_num_partial_prefills=args.max_num_partial_prefills,
                   long_prefill_token_threshold=args.long_prefill_token_threshold, preemption_mode=args.preemption_mode,
                   decode_first=args.chunked_prefill_policy == "decode-first", ahead=args.ahead,
+                  scheduling_policy=args.scheduling_policy,
                   check_layers=args.check_layers)
 
 

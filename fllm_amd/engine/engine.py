@@ -64,13 +64,16 @@ class Engine:
                  gpu_memory_utilization: float = 0.90, decode_first: bool = True, kv_watermark_blocks: int = 0,
                  max_num_partial_prefills: int = 0, long_prefill_token_threshold: int = 0,
                  preemption_mode: str = "recompute", eos_token_ids: Optional[Seq[int]] = None,
-                 random_weights_on_device: bool = False, ops=None, ahead: bool = True, check_layers: int = 0):
+                 random_weights_on_device: bool = False, ops=None, ahead: bool = True, check_layers: int = 0,
+                 scheduling_policy: str = "fcfs"):
         """`model`: a folder with config.json and safetensors; or `config` (a config.json dict)
         with `seed` for random weights (drawn on the host, or on the device with a stream of its
         own when `random_weights_on_device`: large models).  Option names follow the reference's server flags
         (rust/engine/src/bin/serve.rs:530-557, :681-782): ctx, max_seqs, max_batched_tokens,
         gpu_memory_utilization, kv_watermark_blocks, max_num_partial_prefills,
-        long_prefill_token_threshold, preemption_mode.
+        long_prefill_token_threshold, preemption_mode, scheduling_policy (`fcfs`, or `priority`: requests with the
+        smaller `SamplingParams.priority` first, and a waiting one of better priority takes the place of the worst
+        running one).
 
         `ahead` (the default; False: every `step()` waits for its own tokens and returns them, and the host's work per
         step adds to the step): a step is launched before the tokens of the step before it have reached the host
@@ -100,7 +103,8 @@ class Engine:
         self.scheduler = Scheduler(
             SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=max_batched_tokens, decode_first=decode_first,
                             watermark_pages=kv_watermark_blocks, max_partial_prefills=max_num_partial_prefills,
-                            long_prefill_threshold=long_prefill_token_threshold, preemption=preemption_mode),
+                            long_prefill_threshold=long_prefill_token_threshold, preemption=preemption_mode,
+                            policy=scheduling_policy),
             self.runner.cache, self.max_model_len)
         self.sampler = Sampler(self.runner.rt)
         if eos_token_ids is None:

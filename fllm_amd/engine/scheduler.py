@@ -12,6 +12,10 @@ run out.  Behaviour follows the reference's scheduler (rust/engine/src/scheduler
               for it the newest running sequence is preempted (:401-455, :647-657)
   preemption  by recompute: all pages go back, the sequence returns to the FRONT of the queue
               and later prefills prompt and generated tokens again (:933-968)
+  policy      `fcfs`, or `priority` (:206-219, :625-697): the waiting request with the smallest (priority,
+              arrival) is served first, running sequences are served in that order too, a waiting request of
+              better priority takes the slot or the pages of the worst running sequence (never of an equal one),
+              and when a decode row finds no page the worst sequence gives way instead of the newest
 
 The scheduler does the cache bookkeeping (reserve at admission and before a decode row); the
 step function commits what it ran.
@@ -36,12 +40,15 @@ class SchedulerConfig:
     long_prefill_threshold: int = 0         # 0: no distinction
     max_long_partial_prefills: int = 1
     preemption: str = "recompute"
+    policy: str = "fcfs"                    # fcfs | priority (smaller `SamplingParams.priority` first)
 
     def __post_init__(self):
         if self.max_num_seqs <= 0 or self.max_num_batched_tokens <= 0:
             raise ValueError("max_num_seqs and max_num_batched_tokens must be positive")
         if self.preemption not in ("recompute", "none"):
             raise ValueError("preemption must be 'recompute' or 'none'")
+        if self.policy not in ("fcfs", "priority"):
+            raise ValueError("scheduling policy must be 'fcfs' or 'priority'")
 
 
 @dataclass
@@ -111,12 +118,48 @@ class Scheduler:
         seq.num_computed = 0
         return True
 
+    # ---- order ----------------------------------------------------------------------------
+    def _key(self, sid: int) -> Tuple[int, int]:
+        """The sequence with the smaller key goes first (scheduler.rs:625-631)."""
+        seq = self.sequences[sid]
+        return (seq.sampling.priority if self.cfg.policy == "priority" else 0, seq.arrival)
+
+    def _ordered_running(self) -> List[int]:
+        return sorted(self.running, key=self._key) if self.cfg.policy == "priority" else list(self.running)
+
+    def _pick_waiting(self) -> Optional[int]:
+        if not self.waiting:
+            return None
+        return min(self.waiting, key=self._key) if self.cfg.policy == "priority" else self.waiting[0]
+
+    def _victim(self, needy: int) -> int:
+        """Who gives way to `needy`: the last arrival under FCFS, the running sequence of the worst priority (the
+        newest of them) otherwise (scheduler.rs:646-658)."""
+        if self.cfg.policy == "priority":
+            others = [sid for sid in self.running if sid != needy]
+            return max(others, key=self._key) if others else needy
+        return self.running[-1]
+
     def _admit_waiting(self) -> None:
-        while self.waiting and len(self.running) < self.cfg.max_num_seqs:
-            sid = self.waiting[0]
-            if self.cache.free_slots() == 0 or not self._try_admit(sid):
-                break                       # the head of the queue blocks those behind it
-            self.waiting.popleft()
+        by_priority = self.cfg.policy == "priority" and self.cfg.preemption == "recompute"
+        while True:
+            sid = self._pick_waiting()
+            if sid is None:
+                break
+            if len(self.running) >= self.cfg.max_num_seqs:
+                # all slots taken: a waiting request of better priority takes the slot of the worst running sequence
+                if not (by_priority and self.running and self._key(self._victim(sid))[0] > self._key(sid)[0]):
+                    break
+                self._preempt(self._victim(sid))
+            ok = self.cache.free_slots() > 0 and self._try_admit(sid)
+            if not ok and by_priority and self.running and self.cache.free_slots() > 0:
+                victim = self._victim(sid)          # the pool is full: the pages of a running sequence of worse priority
+                if self._key(victim)[0] > self._key(sid)[0]:
+                    self._preempt(victim)
+                    ok = self._try_admit(sid)
+            if not ok:
+                break                       # the request that is next in line blocks those behind it
+            self.waiting.remove(sid)
             self.sequences[sid].state = "running"
             self.running.append(sid)
 
@@ -143,7 +186,7 @@ class Scheduler:
                        and self.sequences[sid].remaining() > 0)
         prefill_budget = max(1, budget - decoders) if self.cfg.decode_first else budget
         long_prefills = 0
-        for sid in list(self.running):
+        for sid in self._ordered_running():
             if prefill_budget == 0 or budget == 0:
                 break
             if self.cfg.max_partial_prefills > 0 and len(step.prefill) >= self.cfg.max_partial_prefills:
@@ -163,7 +206,7 @@ class Scheduler:
             budget -= chunk
             prefill_budget -= chunk
             long_prefills += int(is_long)
-        for sid in list(self.running):
+        for sid in self._ordered_running():
             if sid not in self.running:
                 continue                    # preempted by an earlier sequence of this loop
             seq = self.sequences[sid]
@@ -176,7 +219,7 @@ class Scheduler:
             total = len(seq.tokens)         # the newest token has no keys yet: it is this row
             if not self.cache.can_reserve(sid, total):
                 if self.cfg.preemption == "recompute" and len(self.running) > 1:
-                    victim = self.running[-1]
+                    victim = self._victim(sid)
                     if victim != sid:
                         self._preempt(victim)
                         step.decode = [d for d in step.decode if d != victim]

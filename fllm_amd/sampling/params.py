@@ -27,6 +27,7 @@ class SamplingParams:
     repeat_last_n: int = -1           # tokens of the history (prompt and generated) the penalties look at; negative: all
     logit_bias: Tuple[Tuple[int, float], ...] = ()   # (token id, what is added to its logit)
     min_tokens: int = 0               # no end-of-sequence or stop id before this many tokens were generated
+    priority: int = 0                 # smaller values are served first under the `priority` scheduling policy
 
     def __post_init__(self):
         if self.temperature < 0.0:

@@ -392,3 +392,22 @@ def test_sampling_params_refuse_what_makes_no_sense():
     p = SamplingParams(presence_penalty=0.5, min_tokens=2)
     assert p.penalizes and p.adjusts_logits(0) and SamplingParams(min_tokens=2).adjusts_logits(1)
     assert not SamplingParams(min_tokens=2).adjusts_logits(2) and not SamplingParams(repetition_penalty=1.000001).penalizes
+
+
+@pytest.mark.parametrize("ahead", [False, True])
+def test_priority_policy_lets_a_better_request_overtake(ahead):
+    """One slot: a request of better priority that arrives later takes it, the one that ran waits and later runs its
+    prompt and what it had generated again; both end with the tokens they would have had alone."""
+    engine = make_engine(max_seqs=1, scheduling_policy="priority", ahead=ahead)
+    engine.add_request("low", PROMPTS_A[1], SamplingParams(max_tokens=8, priority=5))
+    events = []
+    for _ in range(4):
+        events += engine.step()
+    engine.add_request("high", PROMPTS_A[0], SamplingParams(max_tokens=4, priority=0))
+    while engine.has_unfinished():
+        events += engine.step()
+    tokens = {name: [e.token_id for e in events if e.request_id == name] for name in ("low", "high")}
+    assert tokens == {"low": plain_greedy("A", PROMPTS_A[1], 8), "high": plain_greedy("A", PROMPTS_A[0], 4)}
+    finished = [e.request_id for e in events if e.finished]
+    assert finished == ["high", "low"] and engine.stats.preemptions == 1
+    engine.runner.cache.check_invariants()

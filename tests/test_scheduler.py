@@ -149,3 +149,81 @@ def test_finish_gives_everything_back():
     run_step(s, cache, s.schedule())
     s.finish(0)
     assert cache.free_pages() == 8 and not s.has_work() and cache.free_slots() == 4
+
+
+def prioritized(sid, prompt_len, priority, max_tokens=8):
+    return Sequence(seq_id=sid, req_id=f"r{sid}", tokens=list(range(prompt_len)), prompt_len=prompt_len,
+                    sampling=SamplingParams(max_tokens=max_tokens, priority=priority))
+
+
+def test_priority_policy_serves_the_smaller_value_first_and_fcfs_ignores_it():
+    """rust/engine/src/scheduler.rs:1308-1319: two requests of priorities 5 and 1; first come, first served runs both in
+    arrival order; with one slot under the priority policy the smaller value runs."""
+    s, _ = make(pages=64, max_seqs=2, budget=16)
+    s.add(prioritized(1, 4, 5))
+    s.add(prioritized(2, 4, 1))
+    s.schedule()
+    assert s.running == [1, 2]
+    s, _ = make(pages=64, max_seqs=1, budget=16, policy="priority")
+    s.add(prioritized(1, 4, 5))
+    s.add(prioritized(2, 4, 1))
+    s.schedule()
+    assert s.running == [2]
+
+
+def test_a_better_priority_takes_the_slot_of_the_worst_running_sequence():
+    """rust/engine/src/scheduler.rs:1322-1339: the preempted sequence waits again with nothing computed; an equal
+    priority never preempts; first come, first served never preempts for a waiting request (:1341-1350)."""
+    s, cache = make(pages=64, max_seqs=1, budget=16, policy="priority")
+    s.add(prioritized(1, 4, 5))
+    run_step(s, cache, s.schedule())
+    assert s.running == [1]
+    s.add(prioritized(2, 4, 0))
+    plan = s.schedule()
+    assert s.running == [2] and 1 in s.waiting and s.preemptions == 1
+    assert s.sequences[1].num_computed == 0 and not cache.has_request(1)
+    assert plan.prefill == [(2, 0, 4)]
+    s.add(prioritized(3, 4, 0))
+    s.schedule()
+    assert s.running == [2] and s.preemptions == 1
+    cache.check_invariants()
+    s, cache = make(pages=64, max_seqs=1, budget=16)
+    s.add(prioritized(1, 4, 9))
+    s.schedule()
+    s.add(prioritized(2, 4, -9))
+    s.schedule()
+    assert s.running == [1] and s.preemptions == 0
+
+
+def test_a_full_pool_admits_by_priority_through_preemption():
+    """rust/engine/src/scheduler.rs:1352-1363: 4 pages of 4 tokens; a 12-token prompt (3 pages and one for its first
+    token) fills the pool, a better request gets its pages."""
+    s, cache = make(pages=4, max_seqs=4, budget=16, policy="priority")
+    s.add(prioritized(1, 12, 5))
+    s.schedule()
+    assert s.running == [1]
+    s.add(prioritized(2, 12, 0))
+    s.schedule()
+    assert s.running == [2] and s.preemptions == 1
+    cache.check_invariants()
+
+
+def test_priority_orders_the_running_sequences_and_picks_the_worst_when_pages_run_out():
+    """Running sequences are served in (priority, arrival) order, and a decode row that finds no page sends the
+    sequence of the worst priority back to the queue, not the newest."""
+    s, cache = make(pages=3, max_seqs=3, budget=16, policy="priority")
+    s.add(prioritized(1, 3, 7))          # the worst priority, the oldest
+    s.add(prioritized(2, 3, 0))
+    s.add(prioritized(3, 3, 3))
+    plan = s.schedule()
+    assert [p[0] for p in plan.prefill] == [2, 3, 1]
+    run_step(s, cache, plan)
+    plan = s.schedule()
+    assert plan.decode == [2, 3, 1]      # the fourth token of each still fits its one page
+    run_step(s, cache, plan)
+    # The fifth token needs a second page and none is free.  Request 2 is served first and takes the page of the worst
+    # one (1, not the newest, 3); request 3 then finds no page either, and the only other sequence gives way to it,
+    # better though it is: whoever needs a page takes it from the worst of the others (scheduler.rs:433-445, :646-658).
+    plan = s.schedule()
+    assert plan.decode == [3] and s.preemptions == 2 and s.running == [3] and set(s.waiting) == {1, 2}
+    cache.check_invariants()
