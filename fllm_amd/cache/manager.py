@@ -19,6 +19,7 @@ from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence
 
 from .pages import OutOfPages, PagePool
+from .prefix import PrefixIndex, PrefixNode
 
 
 @dataclass(frozen=True)
@@ -36,6 +37,7 @@ class _Request:
     slot: int
     length: int = 0                                   # committed tokens
     tables: List[List[int]] = field(default_factory=list)   # per group
+    shared: List[PrefixNode] = field(default_factory=list)  # the prefix index's nodes for this request's first pages, in order
 
 
 class CacheManager:
@@ -57,6 +59,90 @@ class CacheManager:
         self.max_requests = max_requests
         self._free_slots = list(range(max_requests - 1, -1, -1))
         self._requests: Dict[object, _Request] = {}
+        self.prefix: Optional[PrefixIndex] = None
+        # nodes of the index that no live request holds, in the order in which they may be given up: the one unused
+        # for longest first, and the pages behind a node always before the node itself
+        self._idle: Dict[PrefixNode, None] = {}
+        self.prefix_hit_tokens = 0
+
+    # ---- prefixes shared between requests ---------------------------------------------------
+    def enable_prefix_cache(self) -> None:
+        """From now on full pages stay after their request has ended and serve later requests that begin with the
+        same tokens, until the room is needed.  Only where every group keeps all keys with one page size: a window
+        gives pages back that a later request would need, and a prefix is counted in pages."""
+        if any(g.window is not None for g in self.groups) or len({g.page_size for g in self.groups}) != 1:
+            raise ValueError("the prefix cache needs cache groups that keep all keys, with one page size")
+        if self.prefix is None:
+            self.prefix = PrefixIndex(self.groups[0].page_size)
+
+    def _hold(self, req: _Request, node: PrefixNode) -> None:
+        node.holders += 1
+        self._idle.pop(node, None)
+        req.shared.append(node)
+
+    def adopt_prefix(self, req_id, tokens: Sequence[int]) -> int:
+        """For a request that holds nothing yet: puts the pages of the longest known prefix of `tokens` into its block
+        tables, leaving at least the last token to be computed.  Returns the number of tokens taken over; the request
+        holds them as if it had committed them."""
+        req = self._get(req_id)
+        if self.prefix is None or req.length != 0 or any(req.tables):
+            return 0
+        page_size = self.prefix.page_size
+        for node in self.prefix.match(tokens, (len(tokens) - 1) // page_size):
+            for g, page in enumerate(node.pages):
+                self.pools[g].retain(page)
+                req.tables[g].append(page)
+            self._hold(req, node)
+        req.length = len(req.shared) * page_size
+        self.prefix_hit_tokens += req.length
+        return req.length
+
+    def remember_prefix(self, req_id, tokens: Sequence[int], known: Optional[int] = None) -> None:
+        """Enters the full pages of a request into the index.  `tokens` are the request's tokens from its first on, of
+        which the first `known` are final; pages wholly below that and below the committed length are entered.  Where
+        another request has entered the same tokens meanwhile, this one goes on with that one's pages and gives its
+        own back (same tokens at the same places: same keys and values)."""
+        if self.prefix is None:
+            return
+        req = self._get(req_id)
+        page_size = self.prefix.page_size
+        full = min(len(tokens) if known is None else known, req.length) // page_size
+        while len(req.shared) < full:
+            i = len(req.shared)
+            parent = req.shared[-1] if req.shared else None
+            key = tuple(tokens[i * page_size:(i + 1) * page_size])
+            node = self.prefix.child(parent, key)
+            if node is None:
+                pages = tuple(req.tables[g][i] for g in range(len(self.groups)))
+                for g, page in enumerate(pages):
+                    self.pools[g].retain(page)           # the index's own reference
+                node = self.prefix.insert(parent, key, pages)
+            else:
+                for g, page in enumerate(node.pages):
+                    if req.tables[g][i] != page:
+                        self.pools[g].retain(page)
+                        self.pools[g].release(req.tables[g][i])
+                        req.tables[g][i] = page
+            self._hold(req, node)
+
+    def cached_pages(self) -> int:
+        return self.prefix.size if self.prefix is not None else 0
+
+    def clear_prefixes(self) -> int:
+        """Gives up every known prefix that no request holds; returns how many pages a group got back."""
+        dropped = len(self._idle)
+        for g in range(len(self.groups)):
+            self._make_room(g, self.pools[g].num_pages + 1)
+        return dropped
+
+    def _make_room(self, group: int, needed: int) -> None:
+        """Gives up unused prefixes, the longest unused first and from their ends, until `needed` pages are free."""
+        while self.pools[group].available < needed and self._idle:
+            node = next(iter(self._idle))
+            del self._idle[node]
+            self.prefix.remove(node)
+            for g, page in enumerate(node.pages):
+                self.pools[g].release(page)
 
     # ---- requests -------------------------------------------------------------------------
     def add_request(self, req_id) -> int:
@@ -78,6 +164,10 @@ class CacheManager:
         req = self._requests.pop(req_id, None)
         if req is None:
             return
+        for node in reversed(req.shared):               # the end of a prefix goes before its beginning
+            node.holders -= 1
+            if node.holders == 0:
+                self._idle[node] = None
         for g, table in enumerate(req.tables):
             for page in table:
                 if page >= 0:
@@ -103,7 +193,8 @@ class CacheManager:
         return len(self._free_slots)
 
     def free_pages(self, group: int = 0) -> int:
-        return self.pools[group].available
+        """Pages that a reservation can get: the free ones and those of known prefixes that no request holds."""
+        return self.pools[group].available + len(self._idle)
 
     # ---- pages ----------------------------------------------------------------------------
     def _first_needed_page(self, group: GroupSpec, length: int) -> int:
@@ -140,14 +231,16 @@ class CacheManager:
         return out
 
     def can_reserve(self, req_id, total: int) -> bool:
-        return all(m <= pool.available for m, pool in zip(self.pages_missing(req_id, total), self.pools))
+        return all(m <= self.free_pages(g) for g, m in enumerate(self.pages_missing(req_id, total)))
 
     def reserve(self, req_id, total: int) -> None:
         """Covers positions below `total` in every group, or raises `OutOfPages` and changes nothing."""
         missing = self.pages_missing(req_id, total)
-        for g, (m, pool) in enumerate(zip(missing, self.pools)):
-            if m > pool.available:
-                raise OutOfPages(f"group {g} needs {m} pages, {pool.available} are free")
+        for g, m in enumerate(missing):
+            if m > self.free_pages(g):
+                raise OutOfPages(f"group {g} needs {m} pages, {self.free_pages(g)} are free")
+        for g, m in enumerate(missing):
+            self._make_room(g, m)
         req = self._get(req_id)
         for g, group in enumerate(self.groups):
             need_upto = self._covered_upto(group, req.length, total)
@@ -193,9 +286,37 @@ class CacheManager:
 
     # ---- self check -----------------------------------------------------------------------
     def check_invariants(self) -> None:
-        """No page lost, none held twice, none both free and held; slots likewise."""
+        """No page lost, none held twice, none both free and held; slots likewise.  With shared prefixes: every
+        reference is a block table's or the index's, and the index agrees with the tables."""
+        nodes = self.prefix.nodes() if self.prefix is not None else []
+        holders: Dict[PrefixNode, int] = {}
+        for req_id, req in self._requests.items():
+            for i, node in enumerate(req.shared):
+                holders[node] = holders.get(node, 0) + 1
+                if node.parent is not (req.shared[i - 1] if i else self.prefix.root):
+                    raise AssertionError(f"request {req_id!r}: its shared pages are no chain from the first page on")
+                if any(req.tables[g][i] != page for g, page in enumerate(node.pages)):
+                    raise AssertionError(f"request {req_id!r}: page {i} is shared but its table names another page")
+            if len(req.shared) * (self.prefix.page_size if self.prefix else 0) > req.length:
+                raise AssertionError(f"request {req_id!r} shares pages it has not committed")
+        for node in nodes:
+            if node.holders != holders.get(node, 0):
+                raise AssertionError(f"a prefix node counts {node.holders} holders, {holders.get(node, 0)} requests hold it")
+            if (node.holders == 0) != (node in self._idle):
+                raise AssertionError("a prefix node is unused and not up for reuse, or the other way round")
+        if len(self._idle) != sum(1 for node in nodes if node.holders == 0):
+            raise AssertionError("a node that is up for reuse is not in the index")
+        seen_idle = set()
+        for node in self._idle:
+            if any(child not in seen_idle for child in node.children.values()):
+                raise AssertionError("a prefix would be given up before what lies behind it")
+            seen_idle.add(node)
         for g, pool in enumerate(self.pools):
             held: Dict[int, int] = {}
+            for node in nodes:
+                held[node.pages[g]] = held.get(node.pages[g], 0) + 1
+                if held[node.pages[g]] > 1:
+                    raise AssertionError(f"group {g}: page {node.pages[g]} stands for two prefixes")
             for req in self._requests.values():
                 for page in req.tables[g]:
                     if page >= 0:

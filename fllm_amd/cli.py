@@ -35,6 +35,9 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--long-prefill-token-threshold", type=int, default=0)
     ap.add_argument("--preemption-mode", default="recompute", choices=["recompute", "none"])
     ap.add_argument("--scheduling-policy", default="fcfs", choices=["fcfs", "priority"])
+    ap.add_argument("--prefix-cache", action="store_true", default=None,
+                    help="keep full cache pages after their request and start later requests behind the tokens they share "
+                         "(default: the environment's FLLM_PREFIX_CACHE, else off)")
     ap.add_argument("--chunked-prefill-policy", default="decode-first", choices=["decode-first", "prefill-first"])
     ap.add_argument("--no-ahead", dest="ahead", action="store_false",
                     help="wait for the tokens of every step before the next one is launched (by default a step is launched "
@@ -53,7 +56,7 @@ def _make_engine(args, model):
                   max_num_partial_prefills=args.max_num_partial_prefills,
                   long_prefill_token_threshold=args.long_prefill_token_threshold, preemption_mode=args.preemption_mode,
                   decode_first=args.chunked_prefill_policy == "decode-first", ahead=args.ahead,
-                  scheduling_policy=args.scheduling_policy,
+                  scheduling_policy=args.scheduling_policy, prefix_cache=args.prefix_cache,
                   check_layers=args.check_layers)
 
 
@@ -116,7 +119,7 @@ def cmd_run(argv: List[str]) -> int:
     st = engine.stats
     total = sum(len(v) for v in outputs.values())
     print(f"stats: forward_calls={st.forward_calls} rows_total={st.rows_total} max_rows={st.max_rows} "
-          f"prefill_rows={st.prefill_rows} decode_rows={st.decode_rows} preemptions={st.preemptions} "
+          f"prefill_rows={st.prefill_rows} decode_rows={st.decode_rows} preemptions={st.preemptions} prefix_hit_tokens={st.prefix_hit_tokens} "
           f"scheduler={st.scheduler_s * 1e3:.1f}ms model_forward={st.forward_s * 1e3:.1f}ms "
           f"postprocess={st.postprocess_s * 1e3:.1f}ms; generated {total} tok in {elapsed:.3f}s "
           f"({total / max(elapsed, 1e-9):.1f} tok/s)", file=sys.stderr)

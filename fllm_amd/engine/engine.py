@@ -6,6 +6,7 @@ rust/engine/examples/perf_decode.rs:24-46).
 """
 from __future__ import annotations
 
+import os
 import time
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence as Seq, Union
@@ -38,6 +39,7 @@ class EngineStats:
     prefill_rows: int = 0
     decode_rows: int = 0
     preemptions: int = 0
+    prefix_hit_tokens: int = 0     # prompt tokens that were not computed because the cache knew them
     scheduler_s: float = 0.0
     forward_s: float = 0.0
     postprocess_s: float = 0.0
@@ -65,7 +67,7 @@ class Engine:
                  max_num_partial_prefills: int = 0, long_prefill_token_threshold: int = 0,
                  preemption_mode: str = "recompute", eos_token_ids: Optional[Seq[int]] = None,
                  random_weights_on_device: bool = False, ops=None, ahead: bool = True, check_layers: int = 0,
-                 scheduling_policy: str = "fcfs"):
+                 scheduling_policy: str = "fcfs", prefix_cache: Optional[bool] = None):
         """`model`: a folder with config.json and safetensors; or `config` (a config.json dict)
         with `seed` for random weights (drawn on the host, or on the device with a stream of its
         own when `random_weights_on_device`: large models).  Option names follow the reference's server flags
@@ -73,7 +75,10 @@ class Engine:
         gpu_memory_utilization, kv_watermark_blocks, max_num_partial_prefills,
         long_prefill_token_threshold, preemption_mode, scheduling_policy (`fcfs`, or `priority`: requests with the
         smaller `SamplingParams.priority` first, and a waiting one of better priority takes the place of the worst
-        running one).
+        running one).  `prefix_cache` (the reference's environment switch FLLM_PREFIX_CACHE, rust/engine/src/runtime.rs:193-206,
+        is read when it is None; off by default here): full cache pages outlive their request, and a request that begins
+        with the same tokens starts behind them.  Its tokens are then the same as without only up to rounding, as
+        with any other change of how tokens are batched.
 
         `ahead` (the default; False: every `step()` waits for its own tokens and returns them, and the host's work per
         step adds to the step): a step is launched before the tokens of the step before it have reached the host
@@ -100,11 +105,16 @@ class Engine:
         del tensors
         self.config = typed
         self.max_model_len = self.runner.max_context
+        if prefix_cache is None:
+            prefix_cache = os.environ.get("FLLM_PREFIX_CACHE", "").strip().lower() in ("1", "on", "true", "yes")
+        if prefix_cache and self.runner.model.has_state:
+            raise ValueError("the prefix cache shares keys and values only: a model whose layers keep state of their own per "
+                             "request cannot start a request behind a shared prefix")
         self.scheduler = Scheduler(
             SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=max_batched_tokens, decode_first=decode_first,
                             watermark_pages=kv_watermark_blocks, max_partial_prefills=max_num_partial_prefills,
                             long_prefill_threshold=long_prefill_token_threshold, preemption=preemption_mode,
-                            policy=scheduling_policy),
+                            policy=scheduling_policy, prefix_cache=bool(prefix_cache)),
             self.runner.cache, self.max_model_len)
         self.sampler = Sampler(self.runner.rt)
         if eos_token_ids is None:
@@ -141,6 +151,10 @@ class Engine:
         if sid is not None:
             self.scheduler.finish(sid)
 
+    def clear_prefix_cache(self) -> int:
+        """Gives up the cached prefixes that no request uses (rust/engine/src/runtime.rs:1175-1180); returns the pages freed."""
+        return self.runner.cache.clear_prefixes()
+
     def has_unfinished(self) -> bool:
         return self.scheduler.has_work() or self._in_flight is not None
 
@@ -153,6 +167,7 @@ class Engine:
         t1 = time.perf_counter()
         self.stats.scheduler_s += t1 - t0
         self.stats.preemptions = self.scheduler.preemptions
+        self.stats.prefix_hit_tokens = self.runner.cache.prefix_hit_tokens
         earlier, self._in_flight = self._in_flight, None
         if plan is None:
             if earlier is not None:
@@ -304,6 +319,8 @@ class Engine:
         self.runner.capture_graphs(sizes, context_bounds)
         self.stats = saved
         self.scheduler.preemptions = saved.preemptions
+        self.runner.cache.clear_prefixes()
+        self.runner.cache.prefix_hit_tokens = saved.prefix_hit_tokens
         return ran
 
     # ---- whole requests -------------------------------------------------------------------

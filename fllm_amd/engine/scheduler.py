@@ -17,6 +17,11 @@ run out.  Behaviour follows the reference's scheduler (rust/engine/src/scheduler
               better priority takes the slot or the pages of the worst running sequence (never of an equal one),
               and when a decode row finds no page the worst sequence gives way instead of the newest
 
+  prefixes    with `prefix_cache` the cache manager keeps the full pages of what was computed, and a request that is
+              admitted starts behind the longest prefix of its tokens that is known there (the reference's prefix cache,
+              rust/engine/src/mem/prefix_cache.rs:414-520); a preempted sequence finds its own pages again this way
+              unless the room was needed
+
 The scheduler does the cache bookkeeping (reserve at admission and before a decode row); the
 step function commits what it ran.
 """
@@ -41,6 +46,7 @@ class SchedulerConfig:
     max_long_partial_prefills: int = 1
     preemption: str = "recompute"
     policy: str = "fcfs"                    # fcfs | priority (smaller `SamplingParams.priority` first)
+    prefix_cache: bool = False              # requests start behind the prefix of their tokens that the cache knows
 
     def __post_init__(self):
         if self.max_num_seqs <= 0 or self.max_num_batched_tokens <= 0:
@@ -90,6 +96,8 @@ class Scheduler:
         self.running: List[int] = []
         self.preemptions = 0
         self._arrivals = 0
+        if cfg.prefix_cache:
+            cache.enable_prefix_cache()
 
     # ---- queue ----------------------------------------------------------------------------
     def add(self, seq: Sequence) -> None:
@@ -108,6 +116,7 @@ class Scheduler:
         if len(seq.tokens) > self.max_model_len:
             return False
         self.cache.add_request(sid)
+        reused = self.cache.adopt_prefix(sid, seq.tokens) if self.cfg.prefix_cache else 0
         total = len(seq.tokens) + 1
         missing = self.cache.pages_missing(sid, total)
         watermark = self.cfg.watermark_pages if self.running else 0
@@ -115,7 +124,7 @@ class Scheduler:
             self.cache.free_request(sid)
             return False
         self.cache.reserve(sid, total)
-        seq.num_computed = 0
+        seq.num_computed = reused
         return True
 
     # ---- order ----------------------------------------------------------------------------
@@ -162,6 +171,17 @@ class Scheduler:
             self.waiting.remove(sid)
             self.sequences[sid].state = "running"
             self.running.append(sid)
+
+    def _remember(self, sid: int) -> None:
+        """Tells the cache which tokens the sequence's full pages hold.  A negative id stands for a token that is not
+        known yet (a step still runs); such tokens are at the end only."""
+        if not self.cfg.prefix_cache:
+            return
+        tokens = self.sequences[sid].tokens
+        known = len(tokens)
+        while known > 0 and tokens[known - 1] < 0:
+            known -= 1
+        self.cache.remember_prefix(sid, tokens, known)
 
     def _preempt(self, sid: int) -> None:
         seq = self.sequences[sid]
@@ -236,12 +256,16 @@ class Scheduler:
     # ---- after the step -------------------------------------------------------------------
     def commit_chunk(self, sid: int, count: int) -> None:
         self.sequences[sid].num_computed += count
+        self._remember(sid)
 
     def commit_decode(self, sid: int) -> None:
         seq = self.sequences[sid]
         seq.num_computed = len(seq.tokens) - 1      # the token just appended is the next decode row
+        self._remember(sid)
 
     def finish(self, sid: int) -> None:
+        if sid in self.running:
+            self._remember(sid)
         seq = self.sequences.pop(sid)
         seq.state = "finished"
         if sid in self.running:

@@ -411,3 +411,54 @@ def test_priority_policy_lets_a_better_request_overtake(ahead):
     finished = [e.request_id for e in events if e.finished]
     assert finished == ["high", "low"] and engine.stats.preemptions == 1
     engine.runner.cache.check_invariants()
+
+
+# ---- prefix cache --------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("ahead", [False, True])
+def test_requests_that_share_a_beginning_compute_it_once_and_say_the_same(ahead):
+    common = tc.random_ids(37, 512, 3)
+    prompts = [common + tc.random_ids(n, 512, 40 + n) for n in (3, 11, 6)] + [common[:20]]
+    greedy = SamplingParams(max_tokens=10)
+    want = [make_engine("B", ahead=ahead).generate([p], greedy)[0] for p in prompts]
+    engine = make_engine("B", ahead=ahead, prefix_cache=True)
+    first = engine.generate(prompts[:1], greedy)            # pages of 8 tokens: 40 + 10 - 1 computed tokens leave 6 full pages
+    assert engine.runner.cache.cached_pages() == 6 and engine.stats.prefix_hit_tokens == 0
+    rows_before = engine.stats.prefill_rows
+    rest = engine.generate(prompts[1:], greedy)
+    assert first + rest == want
+    # 32 of the 37 common tokens lie in full pages; the prompt that is nothing but a known beginning keeps 16 of its 20
+    assert engine.stats.prefix_hit_tokens == 32 + 32 + 16
+    assert engine.stats.prefill_rows - rows_before == sum(len(p) for p in prompts[1:]) - 80
+    engine.runner.cache.check_invariants()
+    assert engine.runner.cache.requests() == []
+    pool = engine.runner.cache.pools[0]
+    held = pool.num_pages - pool.available
+    assert engine.clear_prefix_cache() == held > 6
+    assert all(p.available == p.num_pages for p in engine.runner.cache.pools)
+    # the generated tokens are part of what is known: a prompt that goes on where an answer ended starts behind them
+    again = prompts[0] + first[0]
+    engine.generate([prompts[0]], greedy)
+    hits = engine.stats.prefix_hit_tokens
+    engine.generate([again + [5]], SamplingParams(max_tokens=2))
+    assert engine.stats.prefix_hit_tokens - hits == 48
+
+
+def test_few_pages_with_known_prefixes_preempt_and_give_the_same_tokens():
+    roomy = make_engine().generate(PROMPTS_A, SamplingParams(max_tokens=16))
+    for ahead in (False, True):
+        tight = make_engine(num_blocks=5, prefix_cache=True, ahead=ahead)
+        assert tight.generate(PROMPTS_A, SamplingParams(max_tokens=16)) == roomy
+        assert tight.stats.preemptions >= 1
+        tight.runner.cache.check_invariants()
+        assert tight.generate(PROMPTS_A, SamplingParams(max_tokens=16)) == roomy       # with what the first round left
+        tight.runner.cache.check_invariants()
+
+
+def test_prefix_cache_is_refused_where_pages_do_not_outlive_their_tokens_and_warm_up_leaves_none():
+    with pytest.raises(ValueError, match="keep all keys"):
+        make_engine("C", prefix_cache=True)
+    engine = make_engine(prefix_cache=True)
+    engine.warm_up()
+    assert engine.runner.cache.cached_pages() == 0 and engine.stats.prefix_hit_tokens == 0
+    assert all(p.available == p.num_pages for p in engine.runner.cache.pools)

@@ -165,6 +165,34 @@ def test_penalties_biases_min_tokens_and_min_p(dtype):
             assert agree >= len(waited[name]) - 1, name          # a near-tie may fall the other way
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_known_prefixes_are_taken_over_and_given_up(name, dtype):
+    """Requests that begin alike start behind the pages of the first; with few pages those are given up and used
+    again for other tokens, and a later request with the same beginning computes it anew."""
+    vocab = tc.CONFIGS[name]["vocab_size"]
+    page = tc.PAGE_SIZES[name]
+    common = tc.random_ids(5 * page + 3, vocab, 77)
+    prompts = [common + tc.random_ids(n, vocab, 30 + n) for n in (4, 9, 2 * page)] + [common[:3 * page]]
+    params = SamplingParams(max_tokens=12)
+    engine = make_engine(name, dtype, prefix_cache=True)
+    outputs = engine.generate(prompts[:1], params) + engine.generate(prompts[1:], params)
+    check_greedy(name, dtype, prompts, outputs)
+    assert engine.stats.prefix_hit_tokens == (5 + 5 + 2) * page
+    engine.runner.cache.check_invariants()
+    # room for one request and a little more: every request finds some of the first one's pages gone
+    others = [tc.random_ids(6 * page, vocab, 90 + i) for i in range(3)]
+    tight = make_engine(name, dtype, prefix_cache=True, num_blocks=9, max_seqs=2)
+    order = [prompts[0], others[0], prompts[1], others[1], others[2], prompts[2], prompts[0]]
+    outputs = [tight.generate([p], params)[0] for p in order]
+    check_greedy(name, dtype, order, outputs)
+    if dtype == "float32":
+        assert outputs[6] == outputs[0]
+    assert tight.runner.cache.cached_pages() <= 9 and tight.stats.prefix_hit_tokens > 0
+    tight.runner.cache.check_invariants()
+    assert tight.clear_prefix_cache() > 0 and all(p.available == p.num_pages for p in tight.runner.cache.pools)
+
+
 def test_no_garbage_collection_while_a_graph_is_captured():
     """Engines that went before leave cycles behind; their collection frees graphs and pinned buffers through the
     HIP runtime, which must not happen while a stream is capturing: the collector is off for the capture's
@@ -206,9 +234,10 @@ def test_command_line(tmp_path):
     first = record["token_ids"]
     flags = ["--repeat-penalty", "1.5", "--presence-penalty", "0.3", "--frequency-penalty", "0.2", "--repeat-last-n", "6",
              "--min-tokens", "3", "--stop-token-ids", str(first[0]), "--logit-bias", f"{first[1]}:-5,3:0.5", "--min-p", "0.1",
-             "--temperature", "0.7", "--seed", "5"]
+             "--temperature", "0.7", "--seed", "5", "--prefix-cache"]
     proc = subprocess.run(cmd + flags, cwd=ROOT, capture_output=True, text=True, timeout=110)
     assert proc.returncode == 0, proc.stderr
+    assert "prefix_hit_tokens=0" in proc.stderr
     record = json.loads(proc.stdout.strip().splitlines()[0])
     params = SamplingParams(max_tokens=8, temperature=0.7, seed=5, min_p=0.1, repetition_penalty=1.5, presence_penalty=0.3,
                             frequency_penalty=0.2, repeat_last_n=6, min_tokens=3, stop_token_ids=(first[0],),

@@ -227,3 +227,54 @@ def test_priority_orders_the_running_sequences_and_picks_the_worst_when_pages_ru
     plan = s.schedule()
     assert plan.decode == [3] and s.preemptions == 2 and s.running == [3] and set(s.waiting) == {1, 2}
     cache.check_invariants()
+
+
+# ---- prefix cache --------------------------------------------------------------------------------
+
+def test_a_request_starts_behind_the_prefix_the_cache_knows():
+    s, cache = make(pages=16, budget=8, prefix_cache=True)
+    s.add(seq(0, 11, max_tokens=1))
+    while s.has_work():
+        plan = s.schedule()
+        run_step(s, cache, plan)
+        for sid in [sid for sid, q in s.sequences.items() if q.remaining() <= 0]:
+            s.finish(sid)
+    assert cache.cached_pages() == 2 and cache.free_pages() == 16     # the keys of 11 tokens were computed: two full pages
+    s.add(seq(1, 14))                               # the same first 11 tokens and three more
+    plan = s.schedule()
+    assert plan.prefill == [(1, 8, 6)]              # two pages are taken over
+    assert cache.prefix_hit_tokens == 8
+    run_step(s, cache, plan)
+    cache.check_invariants()
+
+
+def test_a_preempted_sequence_finds_its_pages_again():
+    s, cache = make(pages=6, budget=16, prefix_cache=True)
+    s.add(seq(0, 8, max_tokens=7))
+    s.add(Sequence(seq_id=1, req_id="r1", tokens=list(range(100, 107)), prompt_len=7, sampling=SamplingParams(max_tokens=8)))
+    run_step(s, cache, s.schedule())                # both prompts: 3 + 2 pages
+    assert cache.free_pages() == 1
+    for _ in range(4):
+        run_step(s, cache, s.schedule())            # sequence 1 takes the last page with its ninth token
+    assert cache.free_pages() == 0 and cache.cached_pages() == 5
+    plan = s.schedule()                             # sequence 0 needs a fourth page: the newest gives way
+    assert s.preemptions == 1 and s.sequences[1].state == "waiting" and plan.decode == [0]
+    # sequence 1 had computed 11 tokens: its third page goes to sequence 0, its two full pages stay known
+    assert cache.pools[0].available == 0 and cache.free_pages() == 2 and cache.cached_pages() == 5
+    run_step(s, cache, plan)
+    plan = s.schedule()
+    assert plan.decode == [0] and not plan.prefill  # sequence 1 needs four pages: its own two and two more, which are not there
+    assert cache.free_pages() == 2
+    run_step(s, cache, plan)
+    assert s.sequences[0].remaining() == 0
+    s.finish(0)
+    plan = s.schedule()
+    assert plan.prefill == [(1, 8, 4)]              # it goes on behind its two pages
+    run_step(s, cache, plan)
+    cache.check_invariants()
+    # without the room for them, the same pages are given up: another request takes everything
+    s.finish(1)
+    s.add(Sequence(seq_id=2, req_id="r2", tokens=list(range(200, 222)), prompt_len=22, sampling=SamplingParams(max_tokens=1)))
+    plan = s.schedule()
+    assert plan.prefill == [(2, 0, 16)] and cache.cached_pages() == 0 and cache.free_pages() == 0
+    cache.check_invariants()
