@@ -77,6 +77,8 @@ def cmd_run(argv: List[str]) -> int:
     ap.add_argument("--repeat-last-n", type=int, default=-1, help="tokens of the history the penalties look at (negative: all)")
     ap.add_argument("--min-tokens", type=int, default=0, help="no end-of-sequence or stop id before this many generated tokens")
     ap.add_argument("--logit-bias", default="", help="comma-separated id:value pairs added to the logits")
+    ap.add_argument("--logprobs", type=int, default=None, metavar="N",
+                    help="with every token its log-probability in the model's distribution and the N likeliest tokens (at most 20)")
     ap.add_argument("--stop-token-ids", default="", help="comma-separated")
     ap.add_argument("--ignore-eos", action="store_true")
     _engine_options(ap)
@@ -100,22 +102,27 @@ def cmd_run(argv: List[str]) -> int:
                             max_tokens=args.max_tokens, stop_token_ids=stops, ignore_eos=args.ignore_eos, min_p=args.min_p,
                             repetition_penalty=args.repeat_penalty, presence_penalty=args.presence_penalty,
                             frequency_penalty=args.frequency_penalty, repeat_last_n=args.repeat_last_n,
-                            min_tokens=args.min_tokens, logit_bias=bias)
+                            min_tokens=args.min_tokens, logit_bias=bias, logprobs=args.logprobs)
     names = [f"prompt-{i}" for i in range(len(prompts))]
     for name, prompt in zip(names, prompts):
         engine.add_request(name, prompt, params)
     outputs = {n: [] for n in names}
+    logprobs = {n: [] for n in names}
     reasons = {}
     start = time.perf_counter()
     while engine.has_unfinished():
         for ev in engine.step():
             outputs[ev.request_id].append(ev.token_id)
+            if ev.logprob is not None:
+                logprobs[ev.request_id].append({"logprob": ev.logprob, "top": [[t, v] for t, v in ev.top_logprobs]})
             if ev.finished:
                 reasons[ev.request_id] = ev.finish_reason
     elapsed = time.perf_counter() - start
     for name, prompt in zip(names, prompts):
-        print(json.dumps({"request": name, "prompt_tokens": len(prompt), "token_ids": outputs[name],
-                          "finish_reason": reasons.get(name)}))
+        record = {"request": name, "prompt_tokens": len(prompt), "token_ids": outputs[name], "finish_reason": reasons.get(name)}
+        if args.logprobs is not None:
+            record["logprobs"] = logprobs[name]
+        print(json.dumps(record))
     st = engine.stats
     total = sum(len(v) for v in outputs.values())
     print(f"stats: forward_calls={st.forward_calls} rows_total={st.rows_total} max_rows={st.max_rows} "

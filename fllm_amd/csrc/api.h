@@ -156,6 +156,13 @@ int fllm_adjust_logits(float *logits, int rows, int vocab, const struct FllmAdju
                        const int32_t *seen_counts, const int32_t *bias_ids, const float *bias_values, const int32_t *blocked_ids,
                        const int32_t *last_tokens, hipStream_t stream);
 
+// Log-probabilities in the softmax of logits [rows, vocab] as they are: for each of the `wanted` rows named in
+// wanted_rows, values[(1 + top) * w] is that of tokens[row], the `top` (at most 20) values behind it those of the
+// likeliest tokens, whose ids stand at the same places of `ids` (ids[(1 + top) * w] repeats the chosen token).
+// wanted_rows are checked by the caller: they are read on the device.
+int fllm_logprobs(const float *logits, int rows, int vocab, const int32_t *wanted_rows, int wanted, const int32_t *tokens,
+                  int top, float *values, int32_t *ids, hipStream_t stream);
+
 // work: float32 [rows, vocab] scratch.  kinds: 1 every row has a temperature and neither top-k nor top-p (the draw
 // looks at every token: several workgroups share a row), 2 no row is of that kind, 3 some may be.
 int fllm_sample(const float *logits, float *work, const struct FllmSampleRow *params, int32_t *out, int rows, int vocab,

@@ -746,7 +746,111 @@ adjust_logits_kernel(float *__restrict__ logits, int vocab, const FllmAdjustRow 
         if (id >= 0 && id < vocab) w[id] = -INFINITY;
     }
 }
+
+// Log-probabilities in the distribution the model gave, the softmax of the logits as they are handed in
+// (rust/engine/src/sampling.rs:937-965): of the token that was chosen for the row and of the `top` likeliest tokens,
+// the lower id first among equals.  One workgroup a wanted row.  values[0] belongs to the chosen token, values[1..]
+// and ids[1..] to the likeliest ones; ids[0] repeats the chosen token.  A row with a NaN or +inf, or with no finite
+// value at all, has no distribution: all its values are NaN and its ids -1.
+//
+// Three passes over the row whatever `top` is: the largest value; the mass and a histogram of token counts over the
+// distance from the largest value; the tokens down to the bin in which the `top`-th lies, gathered into LDS, from
+// which the picks are then taken.  Where that list would not fit (thousands of tokens in the leading bins) or the
+// histogram does not reach `top` tokens (-inf nearly everywhere), every pick is a pass over the row instead.
+constexpr int kListed = 2048;
+__global__ void __launch_bounds__(kBlock)
+logprobs_kernel(const float *__restrict__ logits, int vocab, const int32_t *__restrict__ rows, const int32_t *__restrict__ tokens,
+                int top, float *__restrict__ values, int32_t *__restrict__ ids) {
+    __shared__ Cells cells;
+    __shared__ unsigned long long bins[kBins];
+    __shared__ float listed_v[kListed];
+    __shared__ int listed_i[kListed];
+    __shared__ int listed;
+    const int row = rows[blockIdx.x];
+    const float *w = logits + (size_t)row * vocab;
+    float *out_v = values + (size_t)blockIdx.x * (1 + top);
+    int32_t *out_i = ids + (size_t)blockIdx.x * (1 + top);
+    float largest = -INFINITY;
+    int bad = 0;
+    for_each_token(w, vocab, [&](int, float v) {
+        bad |= (v != v) || v == INFINITY;
+        if (v > largest) largest = v;
+    });
+    largest = block_largest(largest, cells);
+    bad = WholeBlock::sum(bad, cells) != 0 || !(fabsf(largest) < INFINITY);
+    for (int i = threadIdx.x; i < kBins; i += kBlock) bins[i] = 0;
+    if (threadIdx.x == 0) listed = 0;
+    __syncthreads();
+    double mass = 0.0;
+    if (!bad)
+        for_each_token(w, vocab, [&](int, float v) {
+            mass += (double)__expf(v - largest);
+            if (top > 0 && v > -INFINITY) {
+                const int b = bin_of(v, largest);
+                if (b < kBins) atomicAdd(&bins[b], 1ull);
+            }
+        });
+    const float log_mass = (float)log(WholeBlock::sum(mass, cells));
+    const int token = tokens[row];
+    if (threadIdx.x == 0) {
+        out_i[0] = token;
+        out_v[0] = bad || token < 0 || token >= vocab ? NAN : (w[token] - largest) - log_mass;
+    }
+    if (top == 0) return;
+    if (bad) {
+        for (int k = 1 + (int)threadIdx.x; k <= top; k += kBlock) out_i[k] = -1, out_v[k] = NAN;
+        return;
+    }
+    unsigned long long before = 0;
+    const int last_bin = find_bin(bins, (unsigned long long)top, cells, &before);
+    const bool from_list = last_bin < kBins && before + bins[last_bin] <= (unsigned long long)kListed;
+    __syncthreads();
+    if (from_list) {
+        for_each_token(w, vocab, [&](int i, float v) {
+            if (v > -INFINITY && bin_of(v, largest) <= last_bin) {
+                const int at = atomicAdd(&listed, 1);
+                listed_v[at] = v;
+                listed_i[at] = i;
+            }
+        });
+        __syncthreads();
+    }
+    const int count = listed;
+    Pick last = {INFINITY, -1};                   // everything comes after this
+    for (int k = 1; k <= top; k++) {
+        Pick mine = {-INFINITY, kNone};
+        auto offer = [&](int i, float v) {
+            const bool after_last = v < last.value || (v == last.value && i > last.index);
+            if (after_last && (v > mine.value || (v == mine.value && i < mine.index) || mine.index == kNone)) {
+                mine.value = v;
+                mine.index = i;
+            }
+        };
+        if (from_list) {
+            for (int j = threadIdx.x; j < count; j += kBlock) offer(listed_i[j], listed_v[j]);
+        } else {
+            for_each_token(w, vocab, offer);
+        }
+        last = block_best(mine, cells);
+        if (threadIdx.x == 0) {
+            out_i[k] = last.index == kNone ? -1 : last.index;
+            out_v[k] = last.index == kNone ? NAN : (last.value - largest) - log_mass;
+        }
+        if (last.index == kNone) last.value = -INFINITY;      // nothing is left: the rest stays empty
+    }
+}
 }  // namespace
+
+extern "C" int fllm_logprobs(const float *logits, int rows, int vocab, const int32_t *wanted_rows, int wanted,
+                             const int32_t *tokens, int top, float *values, int32_t *ids, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && vocab > 0 && wanted >= 0, "logprobs: bad sizes rows=%d vocab=%d wanted=%d", rows, vocab, wanted);
+    FLLM_REQUIRE(top >= 0 && top <= 20 && top <= vocab, "logprobs: %d alternatives asked for, at most min(20, vocabulary) are given", top);
+    if (wanted == 0) return 0;
+    FLLM_REQUIRE(logits != nullptr && wanted_rows != nullptr && tokens != nullptr && values != nullptr && ids != nullptr,
+                 "logprobs: logits, rows, tokens and both outputs are required");
+    hipLaunchKernelGGL(logprobs_kernel, dim3(wanted), dim3(kBlock), 0, stream, logits, vocab, wanted_rows, tokens, top, values, ids);
+    return fllm_check_launch("logprobs");
+}
 
 extern "C" int fllm_adjust_logits(float *logits, int rows, int vocab, const FllmAdjustRow *row_records, const int32_t *seen_ids,
                                   const int32_t *seen_counts, const int32_t *bias_ids, const float *bias_values,

@@ -9,7 +9,7 @@ from __future__ import annotations
 import os
 import time
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence as Seq, Union
+from typing import Dict, List, Optional, Sequence as Seq, Tuple, Union
 
 import torch
 
@@ -28,6 +28,8 @@ class TokenEvent:
     token_id: int
     finished: bool
     finish_reason: Optional[str] = None     # "stop" | "length"
+    logprob: Optional[float] = None         # with `SamplingParams.logprobs`: of this token in the model's distribution
+    top_logprobs: Optional[List[Tuple[int, float]]] = None     # and the likeliest tokens, (id, log-probability)
 
 
 @dataclass
@@ -57,6 +59,7 @@ class _InFlight:
     at: List[int]
     tokens: torch.Tensor
     on_host: object = None
+    logprobs: object = None      # what `Sampler.finish_logprobs` takes, when a row asked for log-probabilities
 
 
 class Engine:
@@ -203,10 +206,17 @@ class Engine:
         self.stats.rows_total += rows
         self.stats.max_rows = max(self.stats.max_rows, rows)
         requests = [SampleRequest(seqs[sid].sampling, seqs[sid].sampling.seed_for(sid), seqs[sid].draws) for sid in sampled]
-        self._adjust(logits, sampled, row_of, earlier)
+        wants_logprobs = [r for r, sid in enumerate(sampled) if seqs[sid].sampling.logprobs is not None]
+        adjusting = any(seqs[sid].sampling.adjusts_logits(seqs[sid].output_len) for sid in sampled)
+        as_given = logits.clone() if wants_logprobs and adjusting else logits
+        if adjusting:
+            self._adjust(logits, sampled, row_of, earlier)
         launched = _InFlight(sampled, [], self.sampler.launch(logits, requests))
         # queued now, before the next step is launched behind it: reading these tokens must not wait for that step
         launched.on_host = self.sampler.start_read(launched.tokens)
+        if wants_logprobs:
+            top = max(seqs[sampled[r]].sampling.logprobs for r in wants_logprobs)
+            launched.logprobs = self.sampler.start_logprobs(as_given, launched.tokens, wants_logprobs, top)
         # What does not depend on the tokens' values: the sequences grow by one (a placeholder until the
         # token is read), the prompt portions count as computed.
         for sid, _, count in plan.prefill:
@@ -231,8 +241,6 @@ class Engine:
         chosen.  A request whose newest token is still a placeholder (the step in flight chose it) has it counted on
         the device, from that step's tokens."""
         seqs = self.scheduler.sequences
-        if not any(seqs[sid].sampling.adjusts_logits(seqs[sid].output_len) for sid in sampled):
-            return
         from ..sampling.adjust import SeenTokens, row_for
         rows = []
         for sid in sampled:
@@ -248,9 +256,10 @@ class Engine:
         are and finishes the requests that end with them."""
         t0 = time.perf_counter()
         tokens = self.sampler.finish_read(step.on_host)
+        logprobs = self.sampler.finish_logprobs(step.logprobs) if step.logprobs is not None else {}
         seqs = self.scheduler.sequences
         events: List[TokenEvent] = []
-        for sid, at, token in zip(step.sampled, step.at, tokens):
+        for row, (sid, at, token) in enumerate(zip(step.sampled, step.at, tokens)):
             seq = seqs.get(sid)
             if seq is None:
                 continue                         # finished or aborted while this row was in flight
@@ -261,7 +270,11 @@ class Engine:
             if reason:
                 self.scheduler.finish(sid)
                 self._requests.pop(seq.req_id, None)
-            events.append(TokenEvent(seq.req_id, token, reason is not None, reason))
+            event = TokenEvent(seq.req_id, token, reason is not None, reason)
+            if row in logprobs:
+                event.logprob, alternatives = logprobs[row]
+                event.top_logprobs = alternatives[:seq.sampling.logprobs]
+            events.append(event)
         self.stats.postprocess_s += time.perf_counter() - t0
         return events
 

@@ -34,7 +34,7 @@ assert SAMPLE_ROW_BYTES == 32
 _lib = None
 
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 def load_library(build_if_missing: bool = True):
@@ -79,6 +79,7 @@ def load_library(build_if_missing: bool = True):
         "fllm_carry_ids": [c_void, c_void, c_void, c_int, c_int, c_void],
         "fllm_sample": [c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_adjust_logits": [c_void, c_int, c_int, c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_void],
+        "fllm_logprobs": [c_void, c_int, c_int, c_void, c_int, c_void, c_int, c_void, c_void, c_void],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -508,6 +509,22 @@ class Ops:
         self._check(self.lib.fllm_adjust_logits(_ptr(logits), rows, vocab, base, seen_ids, seen_counts, bias_ids, bias_values,
                                                 base + 4 * at, _ptr(last_tokens), self._stream()))
         return logits
+
+    def logprobs(self, logits: torch.Tensor, wanted_rows: torch.Tensor, tokens: torch.Tensor, top: int,
+                 values: torch.Tensor, ids: torch.Tensor) -> None:
+        """Log-probabilities in the softmax of float32 logits [rows, vocab] (fllm_logprobs): for each row named in
+        `wanted_rows` (int32 on the device, every one inside [0, rows): the caller's word), `values[w, 0]` is that of
+        `tokens[row]` and `values[w, 1:]`, `ids[w, 1:]` are the `top` likeliest tokens, the lower id first among equals;
+        `ids[w, 0]` repeats the chosen token.  A row with a NaN or +inf, or without a finite value, gives NaN."""
+        rows, vocab = logits.shape
+        wanted = wanted_rows.numel()
+        _dense(logits, "logits", torch.float32)
+        _dense(wanted_rows, "wanted_rows", torch.int32, (wanted,))
+        _dense(tokens, "tokens", torch.int32, (rows,))
+        _dense(values, "values", torch.float32, (wanted, 1 + top))
+        _dense(ids, "ids", torch.int32, (wanted, 1 + top))
+        self._check(self.lib.fllm_logprobs(_ptr(logits), rows, vocab, _ptr(wanted_rows), wanted, _ptr(tokens), int(top),
+                                           _ptr(values), _ptr(ids), self._stream()))
 
     def sample(self, logits: torch.Tensor, work: torch.Tensor, params: torch.Tensor, out: torch.Tensor,
                kinds: int = 3) -> torch.Tensor:

@@ -9,6 +9,7 @@ GREEDY_TEMPERATURE = 1e-5     # temperature at or below this takes the largest l
 _SEED_BASE = 0x8A5CD789635D2DFF
 _SEED_STEP = 0x9E3779B97F4A7C15
 _MASK64 = (1 << 64) - 1
+MAX_TOP_LOGPROBS = 20         # alternatives a token at most (sampling.rs:950)
 
 
 @dataclass(frozen=True)
@@ -28,6 +29,8 @@ class SamplingParams:
     logit_bias: Tuple[Tuple[int, float], ...] = ()   # (token id, what is added to its logit)
     min_tokens: int = 0               # no end-of-sequence or stop id before this many tokens were generated
     priority: int = 0                 # smaller values are served first under the `priority` scheduling policy
+    logprobs: Optional[int] = None    # None: off; n: every token comes with its log-probability in the model's own
+                                      # distribution (before penalties, temperature and filters) and the n likeliest tokens
 
     def __post_init__(self):
         if self.temperature < 0.0:
@@ -44,6 +47,8 @@ class SamplingParams:
             raise ValueError("repetition_penalty must be positive")
         if self.min_tokens < 0:
             raise ValueError("min_tokens must be nonnegative")
+        if self.logprobs is not None and not 0 <= int(self.logprobs) <= MAX_TOP_LOGPROBS:
+            raise ValueError(f"logprobs must be between 0 and {MAX_TOP_LOGPROBS} alternatives")
         object.__setattr__(self, "stop_token_ids", tuple(int(t) for t in self.stop_token_ids))
         bias = tuple((int(t), float(b)) for t, b in self.logit_bias)
         if any(t < 0 for t, _ in bias) or len({t for t, _ in bias}) != len(bias):

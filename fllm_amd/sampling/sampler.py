@@ -87,6 +87,36 @@ class Sampler:
         """The token ids of `launch` on the host (waits for the device)."""
         return cls.finish_read(cls.start_read(tokens))
 
+    def start_logprobs(self, logits: torch.Tensor, tokens: torch.Tensor, wanted: Sequence[int], top: int):
+        """Asks for the log-probabilities of `tokens[r]` and of the `top` likeliest tokens in the softmax of `logits[r]`
+        (as the model gave them: hand in the logits as they were before `adjust`), for the rows r in `wanted`.  Nothing
+        waits: the kernel and the copies to the host are queued behind what chose the tokens.  Returns what
+        `finish_logprobs` takes."""
+        wanted = [int(r) for r in wanted]
+        if any(not 0 <= r < logits.shape[0] for r in wanted):
+            raise ValueError(f"log-probabilities asked for rows {wanted} of {logits.shape[0]}")
+        top = min(int(top), logits.shape[1])
+        rows = torch.tensor(wanted, dtype=torch.int32)
+        if logits.is_cuda:
+            rows = rows.pin_memory().to(logits.device, non_blocking=True)
+        values = torch.empty((len(wanted), 1 + top), dtype=torch.float32, device=logits.device)
+        ids = torch.empty((len(wanted), 1 + top), dtype=torch.int32, device=logits.device)
+        if wanted:
+            self.rt.ops.logprobs(logits, rows, tokens, top, values, ids)
+        return wanted, self.start_read(values), self.start_read(ids)
+
+    @staticmethod
+    def finish_logprobs(pending) -> dict:
+        """{row: (log-probability of the chosen token, [(token id, log-probability), ...] likeliest first)}; waits for
+        the copies."""
+        wanted, (values, values_done), (ids, ids_done) = pending
+        for done in (values_done, ids_done):
+            if done is not None:
+                done.synchronize()
+        values, ids = values.tolist(), ids.tolist()
+        return {r: (values[w][0], [(int(i), v) for i, v in zip(ids[w][1:], values[w][1:]) if i >= 0])
+                for w, r in enumerate(wanted)}
+
     def launch(self, logits: torch.Tensor, rows: Sequence[SampleRequest]) -> torch.Tensor:
         """Starts the choice of one token per row and returns the int32 device tensor that will
         hold them; nothing waits for the device."""

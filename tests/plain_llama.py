@@ -258,6 +258,19 @@ def apply_generation_controls(logits, min_tokens, generated, eos_ids, stop_token
     return out
 
 
+def raw_logprobs(logits, token, top_n):
+    """rust/engine/src/sampling.rs:937-965: log-softmax of the float32 logits as they are, in float64 around the
+    largest value: (log-probability of `token`, the min(top_n, 20) likeliest as (id, log-probability), the lower id
+    first among equals).  A NaN or +inf anywhere, or no finite value at all, is an error there; here it is None."""
+    w = np.asarray(logits, dtype=np.float32).astype(np.float64)
+    if not 0 <= token < len(w) or np.isnan(w).any() or (w == np.inf).any() or not np.isfinite(w.max()):
+        return None
+    shifted = w - w.max()
+    logp = shifted - math.log(np.exp(shifted).sum())
+    order = sorted(range(len(w)), key=lambda i: (-logp[i], i))[:min(top_n, 20)]
+    return float(logp[token]), [(i, float(logp[i])) for i in order]
+
+
 def apply_penalties(logits, history, repetition_penalty=1.0, presence_penalty=0.0, frequency_penalty=0.0, repeat_last_n=-1,
                     logit_bias=()):
     """rust/engine/src/sampling.rs:252-274 and :579-598: over the last `repeat_last_n` tokens of the history (all of

@@ -462,3 +462,43 @@ def test_prefix_cache_is_refused_where_pages_do_not_outlive_their_tokens_and_war
     engine.warm_up()
     assert engine.runner.cache.cached_pages() == 0 and engine.stats.prefix_hit_tokens == 0
     assert all(p.available == p.num_pages for p in engine.runner.cache.pools)
+
+
+# ---- log-probabilities ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("ahead", [False, True])
+def test_events_carry_the_models_own_log_probabilities(ahead):
+    """Of every generated token and of the likeliest ones, in the distribution before penalties, temperature and
+    filters; a request that did not ask gets none; each request its own number of alternatives."""
+    cfg = tc.CONFIGS["A"]
+    _, spec = model_spec_from_config(cfg)
+    w64 = tc.to_float64(random_tensors(spec, 1, torch.float32))
+    engine = make_engine("A", ahead=ahead)
+    params = [SamplingParams(max_tokens=6, logprobs=3, repetition_penalty=1.8, logit_bias=((5, 4.0),)),
+              SamplingParams(max_tokens=6),
+              SamplingParams(max_tokens=6, logprobs=0, temperature=0.9, top_k=5, seed=3)]
+    for i, (prompt, p) in enumerate(zip(PROMPTS_A, params)):
+        engine.add_request(f"r{i}", prompt, p)
+    events = {f"r{i}": [] for i in range(3)}
+    while engine.has_unfinished():
+        for ev in engine.step():
+            events[ev.request_id].append(ev)
+    assert all(ev.logprob is None and ev.top_logprobs is None for ev in events["r1"])
+    for i in (0, 2):
+        generated = [ev.token_id for ev in events[f"r{i}"]]
+        assert len(generated) == 6
+        logits = plain_llama.forward(cfg, w64, PROMPTS_A[i] + generated)
+        for k, ev in enumerate(events[f"r{i}"]):
+            chosen, alternatives = plain_llama.raw_logprobs(logits[len(PROMPTS_A[i]) - 1 + k], ev.token_id, params[i].logprobs)
+            assert abs(ev.logprob - chosen) < 1e-4
+            assert [t for t, _ in ev.top_logprobs] == [t for t, _ in alternatives]
+            assert all(abs(a - b) < 1e-4 for (_, a), (_, b) in zip(ev.top_logprobs, alternatives))
+    assert generated_with_penalty_differs(events["r0"])
+    with pytest.raises(ValueError, match="between 0 and 20"):
+        SamplingParams(logprobs=21)
+
+
+def generated_with_penalty_differs(events):
+    """The request with a penalty and a bias did not always take the model's likeliest token: what is reported is the
+    model's distribution, not the one the token was chosen from."""
+    return any(ev.top_logprobs[0][0] != ev.token_id for ev in events)

@@ -193,6 +193,39 @@ def test_known_prefixes_are_taken_over_and_given_up(name, dtype):
     assert tight.clear_prefix_cache() > 0 and all(p.available == p.num_pages for p in tight.runner.cache.pools)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_log_probabilities_come_with_the_tokens(dtype):
+    """The model's own distribution (before the penalty that steers the choice), for the chosen token and the
+    likeliest ones, through steps launched ahead and decode graphs."""
+    cfg = tc.CONFIGS["B"]
+    _, spec = model_spec_from_config(cfg)
+    w64 = tc.to_float64(random_tensors(spec, 1, torch.float32))
+    prompts = [tc.random_ids(n, cfg["vocab_size"], 10 + n) for n in (9, 40)]
+    params = [SamplingParams(max_tokens=12, logprobs=4, repetition_penalty=1.5), SamplingParams(max_tokens=12, logprobs=20, temperature=0.8, seed=7)]
+    engine = make_engine("B", dtype)
+    for i, (prompt, p) in enumerate(zip(prompts, params)):
+        engine.add_request(f"r{i}", prompt, p)
+    events = {"r0": [], "r1": []}
+    while engine.has_unfinished():
+        for ev in engine.step():
+            events[ev.request_id].append(ev)
+    tol = 3e-6 if dtype == "float32" else 1.5e-2
+    for i, prompt in enumerate(prompts):
+        generated = [ev.token_id for ev in events[f"r{i}"]]
+        logits = plain_llama.forward(cfg, w64, prompt + generated)
+        for k, ev in enumerate(events[f"r{i}"]):
+            row = logits[len(prompt) - 1 + k]
+            want = torch.log_softmax(torch.from_numpy(np.asarray(row, dtype=np.float64)), 0)
+            allowed = 4 * tol * np.abs(row).max() + 1e-5
+            assert abs(ev.logprob - float(want[ev.token_id])) <= allowed
+            assert len(ev.top_logprobs) == params[i].logprobs
+            values = [v for _, v in ev.top_logprobs]
+            assert values == sorted(values, reverse=True) and len({t for t, _ in ev.top_logprobs}) == len(values)
+            assert all(abs(v - float(want[t])) <= allowed for t, v in ev.top_logprobs)
+            assert values[0] >= float(want.max()) - allowed and values[-1] >= float(torch.sort(want).values[-len(values)]) - allowed
+    assert engine.runner.graph_replays > 0
+
+
 def test_no_garbage_collection_while_a_graph_is_captured():
     """Engines that went before leave cycles behind; their collection frees graphs and pinned buffers through the
     HIP runtime, which must not happen while a stream is capturing: the collector is off for the capture's
@@ -234,10 +267,12 @@ def test_command_line(tmp_path):
     first = record["token_ids"]
     flags = ["--repeat-penalty", "1.5", "--presence-penalty", "0.3", "--frequency-penalty", "0.2", "--repeat-last-n", "6",
              "--min-tokens", "3", "--stop-token-ids", str(first[0]), "--logit-bias", f"{first[1]}:-5,3:0.5", "--min-p", "0.1",
-             "--temperature", "0.7", "--seed", "5", "--prefix-cache"]
+             "--temperature", "0.7", "--seed", "5", "--prefix-cache", "--logprobs", "2"]
     proc = subprocess.run(cmd + flags, cwd=ROOT, capture_output=True, text=True, timeout=110)
     assert proc.returncode == 0, proc.stderr
     assert "prefix_hit_tokens=0" in proc.stderr
+    record = json.loads(proc.stdout.strip().splitlines()[0])
+    assert len(record["logprobs"]) == len(record["token_ids"]) and all(len(e["top"]) == 2 and e["logprob"] <= 0 for e in record["logprobs"])
     record = json.loads(proc.stdout.strip().splitlines()[0])
     params = SamplingParams(max_tokens=8, temperature=0.7, seed=5, min_p=0.1, repetition_penalty=1.5, presence_penalty=0.3,
                             frequency_penalty=0.2, repeat_last_n=6, min_tokens=3, stop_token_ids=(first[0],),

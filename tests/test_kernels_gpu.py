@@ -782,6 +782,48 @@ def test_adjust_logits(ops):
     assert torch.equal(got[3], logits[3])
 
 
+@pytest.mark.parametrize("vocab,top", [(300, 0), (1000, 5), (128256, 20), (7, 7)])
+def test_logprobs(ops, vocab, top):
+    """Log-probabilities of the chosen token and the likeliest ones against the plain function: equal values come in
+    token order, -inf entries have no probability, a row with a NaN has no distribution, rows that were not asked for
+    are not touched, and only the wanted rows are read."""
+    g = gen(60 + top)
+    rows = 6
+    logits = torch.randn(rows, vocab, generator=g) * 5.0
+    best = int(logits[1].argmax())
+    logits[1, (best + 3) % vocab] = logits[1, best]           # two equal largest values
+    logits[1, vocab - 1] = logits[1, best]
+    logits[2, ::2] = -float("inf")
+    logits[3, 5 % vocab] = float("nan")
+    logits[4] = 1000.0 + torch.arange(vocab) % 3             # only three distinct values, far from zero
+    logits[5, 1:] = -float("inf")                             # one token has it all
+    tokens = torch.tensor([int(logits[r].nan_to_num(-1e30).argmax()) for r in range(rows)], dtype=torch.int32)
+    tokens[0] = vocab - 1                                      # an unlikely token was drawn
+    tokens[2] = 0                                              # one that cannot be: -inf
+    wanted = [5, 0, 1, 2, 3, 4][:rows - (1 if top == 0 else 0)]
+    values = torch.full((len(wanted), 1 + top), 7.0, device=DEV)
+    ids = torch.full((len(wanted), 1 + top), 7, dtype=torch.int32, device=DEV)
+    ops.logprobs(logits.to(DEV), torch.tensor(wanted, dtype=torch.int32, device=DEV), tokens.to(DEV), top, values, ids)
+    values, ids = values.cpu(), ids.cpu()
+    for w, r in enumerate(wanted):
+        want = plain_llama.raw_logprobs(logits[r].numpy(), int(tokens[r]), top)
+        assert int(ids[w, 0]) == int(tokens[r])
+        if want is None:
+            assert r == 3 and bool(torch.isnan(values[w]).all()) and ids[w, 1:].tolist() == [-1] * top
+            continue
+        chosen, alternatives = want
+        assert ids[w, 1:].tolist() == [i for i, _ in alternatives], (r, ids[w].tolist())
+        got = np.array([float(values[w, 0])] + values[w, 1:].tolist())
+        expected = np.array([chosen] + [v for _, v in alternatives])
+        finite = np.isfinite(expected)
+        assert np.array_equal(got[~finite], expected[~finite])
+        if finite.any():
+            assert np.abs(got[finite] - expected[finite]).max() <= 2e-6 * max(1.0, np.abs(expected[finite]).max()) + 2e-6, r
+    with pytest.raises(Exception, match="at most"):
+        ops.logprobs(logits.to(DEV), torch.tensor([0], dtype=torch.int32, device=DEV), tokens.to(DEV), 21,
+                     torch.empty(1, 22, device=DEV), torch.empty(1, 22, dtype=torch.int32, device=DEV))
+
+
 def test_sample_depends_only_on_seed_draw_and_logits(ops):
     from fllm_amd.sampling import SampleRequest, SamplingParams, pack_rows
     g = gen(18)

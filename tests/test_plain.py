@@ -347,6 +347,23 @@ def test_penalties_and_controls():
     assert P.apply_generation_controls([1.0, 2.0, 3.0, 4.0], 3, 3, [3], [1]).tolist() == [1.0, 2.0, 3.0, 4.0]
 
 
+def test_raw_logprobs():
+    """rust/engine/src/sampling.rs:970-978: stable around the largest value, ties in token order, no distribution for bad rows."""
+    logprob, top = P.raw_logprobs([1000.0, 1000.0, 999.0], 2, 2)
+    assert [i for i, _ in top] == [0, 1]
+    assert abs(logprob - (-1.0 - math.log(2.0 + math.exp(-1.0)))) < 1e-12
+    big = float(np.finfo(np.float32).max)
+    assert abs(P.raw_logprobs([big, big], 0, 0)[0] + math.log(2.0)) < 1e-12
+    assert P.raw_logprobs([float("nan")], 0, 1) is None and P.raw_logprobs([-np.inf], 0, 1) is None
+    # it is the library's log-softmax, and at most 20 alternatives come back
+    rng = np.random.default_rng(5)
+    w = rng.normal(size=300).astype(np.float32) * 4
+    logprob, top = P.raw_logprobs(w, 17, 50)
+    want = torch.log_softmax(torch.from_numpy(w).double(), 0)
+    assert abs(logprob - float(want[17])) < 1e-12 and len(top) == 20
+    assert [i for i, _ in top] == torch.argsort(want, descending=True, stable=True)[:20].tolist()
+
+
 def test_draws_follow_the_distribution_and_depend_on_seed_and_draw_only():
     logits = np.array([2.0, 1.0, 0.0, -1.0], dtype=np.float32)
     p = np.exp(logits / 0.8)
