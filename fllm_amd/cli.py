@@ -79,6 +79,10 @@ def cmd_run(argv: List[str]) -> int:
     ap.add_argument("--logit-bias", default="", help="comma-separated id:value pairs added to the logits")
     ap.add_argument("--logprobs", type=int, default=None, metavar="N",
                     help="with every token its log-probability in the model's distribution and the N likeliest tokens (at most 20)")
+    ap.add_argument("--allowed-token-ids", default="", help="comma-separated: only these tokens can be chosen")
+    ap.add_argument("--bad-words-ids", action="append", default=[], metavar="IDS",
+                    help="comma-separated token ids of a sequence that must not be generated (repeatable)")
+    ap.add_argument("--timeout", type=float, default=None, metavar="SECONDS", help="give a request up after this long")
     ap.add_argument("--stop-token-ids", default="", help="comma-separated")
     ap.add_argument("--ignore-eos", action="store_true")
     _engine_options(ap)
@@ -102,7 +106,10 @@ def cmd_run(argv: List[str]) -> int:
                             max_tokens=args.max_tokens, stop_token_ids=stops, ignore_eos=args.ignore_eos, min_p=args.min_p,
                             repetition_penalty=args.repeat_penalty, presence_penalty=args.presence_penalty,
                             frequency_penalty=args.frequency_penalty, repeat_last_n=args.repeat_last_n,
-                            min_tokens=args.min_tokens, logit_bias=bias, logprobs=args.logprobs)
+                            min_tokens=args.min_tokens, logit_bias=bias, logprobs=args.logprobs,
+                            allowed_token_ids=tuple(int(t) for t in args.allowed_token_ids.split(",") if t.strip()),
+                            bad_word_ids=tuple(tuple(int(t) for t in w.split(",") if t.strip()) for w in args.bad_words_ids),
+                            timeout_secs=args.timeout)
     names = [f"prompt-{i}" for i in range(len(prompts))]
     for name, prompt in zip(names, prompts):
         engine.add_request(name, prompt, params)
@@ -112,7 +119,8 @@ def cmd_run(argv: List[str]) -> int:
     start = time.perf_counter()
     while engine.has_unfinished():
         for ev in engine.step():
-            outputs[ev.request_id].append(ev.token_id)
+            if ev.token_id >= 0:
+                outputs[ev.request_id].append(ev.token_id)
             if ev.logprob is not None:
                 logprobs[ev.request_id].append({"logprob": ev.logprob, "top": [[t, v] for t, v in ev.top_logprobs]})
             if ev.finished:

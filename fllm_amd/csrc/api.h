@@ -139,9 +139,12 @@ struct FllmSampleRow {
 };
 // What is done to a row of logits before a token is chosen (rust/engine/src/sampling.rs:220-229, :252-274).  The
 // lists live in arrays shared by all rows: seen_ids / seen_counts [seen_off .. + seen_len) are the distinct tokens of
-// the request's history (within its window) and how often each occurs; bias_ids / bias_values; blocked_ids (to -inf).
+// the request's history (within its window) and how often each occurs; bias_ids / bias_values; blocked_ids (to -inf);
+// allowed_ids (rising; when a row has any, every other token goes to -inf); if_last / then_blocked (pairs: the second
+// goes to -inf when the newest token is the first).
 // last_row >= 0: last_tokens[last_row] (device memory, written by an earlier launch) is the newest token of the
-// history and not in the lists yet: it counts once more.  A row whose lists are empty and last_row < 0 is left alone.
+// history and not in the lists yet: it counts once more, and the pairs are judged by it.  A row whose lists are empty
+// and last_row < 0 is left alone.
 struct FllmAdjustRow {
     float repetition_penalty;   // 1: off
     float presence_penalty;
@@ -150,11 +153,22 @@ struct FllmAdjustRow {
     int32_t bias_off, bias_len;
     int32_t blocked_off, blocked_len;
     int32_t last_row;           // -1: none
+    int32_t allowed_off, allowed_len;
+    int32_t pairs_off, pairs_len;
 };
-// logits: float32 [rows, vocab], changed in place; one record a row; the id arrays may be null when no row uses them
-int fllm_adjust_logits(float *logits, int rows, int vocab, const struct FllmAdjustRow *row_records, const int32_t *seen_ids,
-                       const int32_t *seen_counts, const int32_t *bias_ids, const float *bias_values, const int32_t *blocked_ids,
-                       const int32_t *last_tokens, hipStream_t stream);
+// Device arrays that the rows' offsets point into; any may be null when no row uses it.  The struct itself is read
+// on the host, at the call.
+struct FllmAdjustLists {
+    const int32_t *seen_ids, *seen_counts;
+    const int32_t *bias_ids;
+    const float *bias_values;
+    const int32_t *blocked_ids;
+    const int32_t *allowed_ids;
+    const int32_t *if_last, *then_blocked;
+};
+// logits: float32 [rows, vocab], changed in place; one record a row (device memory)
+int fllm_adjust_logits(float *logits, int rows, int vocab, const struct FllmAdjustRow *row_records,
+                       const struct FllmAdjustLists *lists, const int32_t *last_tokens, hipStream_t stream);
 
 // Log-probabilities in the softmax of logits [rows, vocab] as they are: for each of the `wanted` rows named in
 // wanted_rows, values[(1 + top) * w] is that of tokens[row], the `top` (at most 20) values behind it those of the

@@ -717,9 +717,8 @@ __device__ __forceinline__ float penalised(float v, const FllmAdjustRow &a, int 
 }
 
 __global__ void __launch_bounds__(kAdjustBlock)
-adjust_logits_kernel(float *__restrict__ logits, int vocab, const FllmAdjustRow *__restrict__ rows, const int32_t *__restrict__ seen_ids,
-                     const int32_t *__restrict__ seen_counts, const int32_t *__restrict__ bias_ids, const float *__restrict__ bias_values,
-                     const int32_t *__restrict__ blocked_ids, const int32_t *__restrict__ last_tokens) {
+adjust_logits_kernel(float *__restrict__ logits, int vocab, const FllmAdjustRow *__restrict__ rows, const FllmAdjustLists lists,
+                     const int32_t *__restrict__ last_tokens) {
     __shared__ int last_was_listed;
     const FllmAdjustRow a = rows[blockIdx.x];
     float *w = logits + (size_t)blockIdx.x * vocab;
@@ -727,9 +726,9 @@ adjust_logits_kernel(float *__restrict__ logits, int vocab, const FllmAdjustRow 
     if (threadIdx.x == 0) last_was_listed = 0;
     __syncthreads();
     for (int j = threadIdx.x; j < a.seen_len; j += kAdjustBlock) {        // ids of a row are distinct: no two threads meet
-        const int id = seen_ids[a.seen_off + j];
+        const int id = lists.seen_ids[a.seen_off + j];
         if (id < 0 || id >= vocab) continue;
-        int count = seen_counts[a.seen_off + j];
+        int count = lists.seen_counts[a.seen_off + j];
         if (id == last) count++, last_was_listed = 1;
         w[id] = penalised(w[id], a, count);
     }
@@ -737,13 +736,28 @@ adjust_logits_kernel(float *__restrict__ logits, int vocab, const FllmAdjustRow 
     if (threadIdx.x == 0 && last >= 0 && last < vocab && !last_was_listed) w[last] = penalised(w[last], a, 1);
     __syncthreads();
     for (int j = threadIdx.x; j < a.bias_len; j += kAdjustBlock) {
-        const int id = bias_ids[a.bias_off + j];
-        if (id >= 0 && id < vocab) w[id] += bias_values[a.bias_off + j];
+        const int id = lists.bias_ids[a.bias_off + j];
+        if (id >= 0 && id < vocab) w[id] += lists.bias_values[a.bias_off + j];
     }
     __syncthreads();
     for (int j = threadIdx.x; j < a.blocked_len; j += kAdjustBlock) {
-        const int id = blocked_ids[a.blocked_off + j];
+        const int id = lists.blocked_ids[a.blocked_off + j];
         if (id >= 0 && id < vocab) w[id] = -INFINITY;
+    }
+    for (int j = threadIdx.x; j < a.pairs_len; j += kAdjustBlock) {
+        const int id = lists.then_blocked[a.pairs_off + j];
+        if (lists.if_last[a.pairs_off + j] == last && id >= 0 && id < vocab) w[id] = -INFINITY;
+    }
+    if (a.allowed_len > 0) {                       // every token that is not on the rising list
+        const int32_t *allowed = lists.allowed_ids + a.allowed_off;
+        for (int i = threadIdx.x; i < vocab; i += kAdjustBlock) {
+            int lo = 0, hi = a.allowed_len;        // the first entry >= i lies in [lo, hi]
+            while (lo < hi) {
+                const int mid = (lo + hi) / 2;
+                if (allowed[mid] < i) lo = mid + 1; else hi = mid;
+            }
+            if (lo == a.allowed_len || allowed[lo] != i) w[i] = -INFINITY;
+        }
     }
 }
 
@@ -852,14 +866,12 @@ extern "C" int fllm_logprobs(const float *logits, int rows, int vocab, const int
     return fllm_check_launch("logprobs");
 }
 
-extern "C" int fllm_adjust_logits(float *logits, int rows, int vocab, const FllmAdjustRow *row_records, const int32_t *seen_ids,
-                                  const int32_t *seen_counts, const int32_t *bias_ids, const float *bias_values,
-                                  const int32_t *blocked_ids, const int32_t *last_tokens, hipStream_t stream) {
+extern "C" int fllm_adjust_logits(float *logits, int rows, int vocab, const FllmAdjustRow *row_records, const FllmAdjustLists *lists,
+                                  const int32_t *last_tokens, hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && vocab > 0, "adjust_logits: bad sizes rows=%d vocab=%d", rows, vocab);
     if (rows == 0) return 0;
-    FLLM_REQUIRE(logits != nullptr && row_records != nullptr, "adjust_logits: logits and row records are required");
-    hipLaunchKernelGGL(adjust_logits_kernel, dim3(rows), dim3(kAdjustBlock), 0, stream, logits, vocab, row_records, seen_ids,
-                       seen_counts, bias_ids, bias_values, blocked_ids, last_tokens);
+    FLLM_REQUIRE(logits != nullptr && row_records != nullptr && lists != nullptr, "adjust_logits: logits, row records and lists are required");
+    hipLaunchKernelGGL(adjust_logits_kernel, dim3(rows), dim3(kAdjustBlock), 0, stream, logits, vocab, row_records, *lists, last_tokens);
     return fllm_check_launch("adjust_logits");
 }
 

@@ -27,7 +27,7 @@ class TokenEvent:
     request_id: str
     token_id: int
     finished: bool
-    finish_reason: Optional[str] = None     # "stop" | "length"
+    finish_reason: Optional[str] = None     # "stop" | "length" | "timeout" (then no token comes with it: token_id -1)
     logprob: Optional[float] = None         # with `SamplingParams.logprobs`: of this token in the model's distribution
     top_logprobs: Optional[List[Tuple[int, float]]] = None     # and the likeliest tokens, (id, log-probability)
 
@@ -125,6 +125,7 @@ class Engine:
         self.eos_token_ids = tuple(int(t) for t in eos_token_ids)
         self.stats = EngineStats()
         self._requests: Dict[str, int] = {}
+        self._deadlines: Dict[str, float] = {}
         self._next_seq = 0
         self.ahead = bool(ahead)
         self._in_flight: Optional[_InFlight] = None
@@ -147,7 +148,23 @@ class Engine:
         self._next_seq += 1
         self.scheduler.add(Sequence(seq_id=sid, req_id=request_id, tokens=prompt, prompt_len=len(prompt), sampling=sampling))
         self._requests[request_id] = sid
+        self._deadlines.pop(request_id, None)
+        if sampling.timeout_secs is not None:
+            self._deadlines[request_id] = time.monotonic() + float(sampling.timeout_secs)
         return sid
+
+    def expire_requests(self) -> List[str]:
+        """Gives up the requests whose `timeout_secs` have passed since they were added, waiting included, and returns
+        their ids; what they hold goes back (rust/engine/src/runtime.rs:1222-1232).  `step` calls it."""
+        if not self._deadlines:
+            return []
+        now = time.monotonic()
+        self._deadlines = {rid: d for rid, d in self._deadlines.items() if rid in self._requests}     # the others have ended
+        expired = sorted(rid for rid, deadline in self._deadlines.items() if deadline <= now)
+        for rid in expired:
+            del self._deadlines[rid]
+            self.abort_request(rid)
+        return expired
 
     def abort_request(self, request_id: str) -> None:
         sid = self._requests.pop(request_id, None)
@@ -165,6 +182,12 @@ class Engine:
     def step(self) -> List[TokenEvent]:
         """Schedules and runs one step.  Returns the tokens it produced; with `ahead`, those of the
         step before, while this one runs."""
+        timed_out = [TokenEvent(rid, -1, True, "timeout") for rid in self.expire_requests()]
+        if timed_out:
+            return timed_out + self._step()
+        return self._step()
+
+    def _step(self) -> List[TokenEvent]:
         t0 = time.perf_counter()
         plan = self.scheduler.schedule()
         t1 = time.perf_counter()
@@ -352,6 +375,6 @@ class Engine:
         outputs: Dict[str, List[int]] = {n: [] for n in names}
         while any(n in self._requests for n in names):
             for ev in self.step():
-                if ev.request_id in outputs:
+                if ev.request_id in outputs and ev.token_id >= 0:
                     outputs[ev.request_id].append(ev.token_id)
         return [outputs[n] for n in names]

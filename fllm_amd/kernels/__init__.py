@@ -27,14 +27,20 @@ class SampleRow(ctypes.Structure):
                 ("min_p", ctypes.c_float), ("seed", ctypes.c_uint64), ("draw", ctypes.c_uint64)]
 
 
+class AdjustLists(ctypes.Structure):
+    """FllmAdjustLists: device addresses of the lists that the row records of `adjust_logits` point into."""
+    _fields_ = [(name, ctypes.c_void_p) for name in ("seen_ids", "seen_counts", "bias_ids", "bias_values", "blocked_ids",
+                                                     "allowed_ids", "if_last", "then_blocked")]
+
+
 SAMPLE_ROW_BYTES = ctypes.sizeof(SampleRow)
-ADJUST_ROW_WORDS = 10         # int32 words of one FllmAdjustRow
+ADJUST_ROW_WORDS = 14         # int32 words of one FllmAdjustRow
 assert SAMPLE_ROW_BYTES == 32
 
 _lib = None
 
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 
 def load_library(build_if_missing: bool = True):
@@ -78,7 +84,7 @@ def load_library(build_if_missing: bool = True):
         "fllm_gate_up_swiglu": [c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_carry_ids": [c_void, c_void, c_void, c_int, c_int, c_void],
         "fllm_sample": [c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
-        "fllm_adjust_logits": [c_void, c_int, c_int, c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_void],
+        "fllm_adjust_logits": [c_void, c_int, c_int, c_void, c_void, c_void, c_void],
         "fllm_logprobs": [c_void, c_int, c_int, c_void, c_int, c_void, c_int, c_void, c_void, c_void],
     }
     for name, args in sig.items():
@@ -488,26 +494,28 @@ class Ops:
 
     def adjust_logits(self, logits: torch.Tensor, packed: torch.Tensor, sections: Sequence[int],
                       last_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """Penalties, biases and blocked ids on float32 logits [rows, vocab], in place (fllm_adjust_logits).  `packed`: one
-        int32 device tensor holding, one behind the other, the row records (10 words a row: the three penalties as
-        float bits, then seen_off, seen_len, bias_off, bias_len, blocked_off, blocked_len, last_row), the seen ids, the
-        seen counts, the bias ids, the bias values (float bits) and the blocked ids; `sections`: (entries of the seen
-        lists, entries of the bias lists, blocked ids), each over all rows.
+        """Penalties, biases, blocked and allowed ids on float32 logits [rows, vocab], in place (fllm_adjust_logits).
+        `packed`: one int32 device tensor holding, one behind the other, the row records (14 words a row: the three
+        penalties as float bits, then seen_off, seen_len, bias_off, bias_len, blocked_off, blocked_len, last_row,
+        allowed_off, allowed_len, pairs_off, pairs_len), the seen ids, the seen counts, the bias ids, the bias values
+        (float bits), the blocked ids, the allowed ids (rising within a row) and the pairs (first all "if the newest
+        token is" ids, then all "block" ids); `sections`: (entries of the seen lists, of the bias lists, blocked ids,
+        allowed ids, pairs), each over all rows.
         `last_tokens`: int32 device tensor that the records' last_row points into."""
         rows, vocab = logits.shape
-        seen, bias, blocked = (int(n) for n in sections)
+        seen, bias, blocked, allowed, pairs = (int(n) for n in sections)
         _dense(logits, "logits", torch.float32)
-        _dense(packed, "packed", torch.int32, (rows * ADJUST_ROW_WORDS + 2 * seen + 2 * bias + blocked,))
+        _dense(packed, "packed", torch.int32, (rows * ADJUST_ROW_WORDS + 2 * seen + 2 * bias + blocked + allowed + 2 * pairs,))
         if last_tokens is not None:
             _dense(last_tokens, "last_tokens", torch.int32)
         base = packed.data_ptr()
         at = rows * ADJUST_ROW_WORDS
-        seen_ids, seen_counts = base + 4 * at, base + 4 * (at + seen)
-        at += 2 * seen
-        bias_ids, bias_values = base + 4 * at, base + 4 * (at + bias)
-        at += 2 * bias
-        self._check(self.lib.fllm_adjust_logits(_ptr(logits), rows, vocab, base, seen_ids, seen_counts, bias_ids, bias_values,
-                                                base + 4 * at, _ptr(last_tokens), self._stream()))
+        lists = AdjustLists()
+        for name, count in (("seen_ids", seen), ("seen_counts", seen), ("bias_ids", bias), ("bias_values", bias),
+                            ("blocked_ids", blocked), ("allowed_ids", allowed), ("if_last", pairs), ("then_blocked", pairs)):
+            setattr(lists, name, base + 4 * at)
+            at += count
+        self._check(self.lib.fllm_adjust_logits(_ptr(logits), rows, vocab, base, ctypes.byref(lists), _ptr(last_tokens), self._stream()))
         return logits
 
     def logprobs(self, logits: torch.Tensor, wanted_rows: torch.Tensor, tokens: torch.Tensor, top: int,

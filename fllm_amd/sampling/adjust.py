@@ -1,5 +1,5 @@
 """What a request asks to be done to its logits before a token is chosen: penalties on tokens seen before, biases,
-and end and stop ids that `min_tokens` still blocks (rust/engine/src/sampling.rs:220-229, :252-274).  The host keeps
+end and stop ids that `min_tokens` still blocks, an allow list and bad words (rust/engine/src/sampling.rs:220-250, :252-274).  The host keeps
 the counts and packs them for the kernel; the newest token of a request may still be on the device only."""
 from __future__ import annotations
 
@@ -11,7 +11,9 @@ import torch
 
 from .params import SamplingParams
 
-ROW_WORDS = 10      # int32 words of a row record: three floats, then seen_off, seen_len, bias_off, bias_len, blocked_off, blocked_len, last_row
+# int32 words of a row record: three floats, then seen_off, seen_len, bias_off, bias_len, blocked_off, blocked_len, last_row,
+# allowed_off, allowed_len, pairs_off, pairs_len
+ROW_WORDS = 14
 
 
 class SeenTokens:
@@ -56,18 +58,42 @@ class SeenTokens:
 @dataclass
 class AdjustRow:
     """One row's share: the distinct tokens seen (within the window) with their counts (a dictionary, or the two
-    arrays of `SeenTokens.lists`), ids blocked for now, and where the newest token lies on the device when the host
-    does not know it yet."""
+    arrays of `SeenTokens.lists`), ids blocked for now, the allow list, pairs (a, b) that block b if the newest token
+    is a, and where the newest token lies on the device when the host does not know it yet."""
     params: SamplingParams
     seen: object
     blocked: Tuple[int, ...] = ()
     last_row: int = -1
+    allowed: Tuple[int, ...] = ()
+    pairs: Tuple[Tuple[int, int], ...] = ()
 
     def seen_lists(self) -> Tuple[np.ndarray, np.ndarray]:
         if isinstance(self.seen, dict):
             ids = np.fromiter((t if -(1 << 31) <= t < (1 << 31) else -1 for t in self.seen), dtype=np.int32, count=len(self.seen))
             return ids, np.fromiter(self.seen.values(), dtype=np.int32, count=len(self.seen))
         return self.seen
+
+
+def bad_word_blocks(words: Sequence[Sequence[int]], tokens: Sequence[int], known: int) -> Tuple[List[int], List[Tuple[int, int]]]:
+    """sampling.rs:241-248: the last token of a word is blocked when the tokens before it stand at the end of the history.
+    `tokens[:known]` are final; one more token may follow that only the device knows: then a word whose other tokens
+    fit is blocked on the condition that this token is the word's last but one.  Returns (blocked ids, (newest token,
+    blocked id) pairs)."""
+    blocked: List[int] = []
+    pairs: List[Tuple[int, int]] = []
+    pending = len(tokens) > known
+    for word in words:
+        *before, last = word
+        if not pending:
+            if len(before) <= known and list(tokens[known - len(before):known]) == before:
+                blocked.append(last)
+        elif not before:
+            blocked.append(last)
+        else:
+            rest = before[:-1]
+            if len(rest) <= known and list(tokens[known - len(rest):known]) == rest:
+                pairs.append((before[-1], last))
+    return blocked, pairs
 
 
 def row_for(params: SamplingParams, tokens: Sequence[int], prompt_len: int, pending_row: Optional[int], eos: Sequence[int],
@@ -93,19 +119,23 @@ def row_for(params: SamplingParams, tokens: Sequence[int], prompt_len: int, pend
                 counts[t] = counts.get(t, 0) + 1
         if pending_row is not None and n != 0:
             last_row = pending_row
-    blocked: Tuple[int, ...] = ()
+    blocked: List[int] = []
     if generated < params.min_tokens:
-        blocked = tuple(dict.fromkeys(list(eos) + list(params.stop_token_ids)))
-    return AdjustRow(params, counts, blocked, last_row)
+        blocked = list(eos) + list(params.stop_token_ids)
+    word_blocks, pairs = bad_word_blocks(params.bad_word_ids, tokens, known)
+    if pairs:
+        last_row = pending_row
+    return AdjustRow(params, counts, tuple(dict.fromkeys(blocked + word_blocks)), last_row, params.allowed_token_ids, tuple(pairs))
 
 
-def pack(rows: Sequence[Optional[AdjustRow]]) -> Tuple[torch.Tensor, Tuple[int, int, int]]:
+def pack(rows: Sequence[Optional[AdjustRow]]) -> Tuple[torch.Tensor, Tuple[int, int, int, int, int]]:
     """The kernel's input for a step's rows (None: a row left alone) as one int32 CPU tensor, and the lengths of its
-    three list sections (seen, bias, blocked)."""
+    five list sections (seen, bias, blocked, allowed, pairs)."""
     records = np.zeros((len(rows), ROW_WORDS), dtype=np.int32)
     floats = records.view(np.float32)
-    seen_ids, seen_counts, bias_ids, bias_values, blocked = [], [], [], [], []
-    n_seen = n_bias = n_blocked = 0
+    seen_ids, seen_counts, bias_ids, bias_values, blocked, allowed, if_last, then_blocked = [], [], [], [], [], [], [], []
+    n_seen = n_bias = n_blocked = n_allowed = n_pairs = 0
+    word = lambda t: t if -(1 << 31) <= t < (1 << 31) else -1
     for i, r in enumerate(rows):
         if r is None:
             floats[i, 0] = 1.0
@@ -113,16 +143,22 @@ def pack(rows: Sequence[Optional[AdjustRow]]) -> Tuple[torch.Tensor, Tuple[int, 
             continue
         p = r.params
         ids, counts = r.seen_lists()
-        floats[i, 0:3] = (p.repetition_penalty, p.presence_penalty, p.frequency_penalty)
-        records[i, 3:] = (n_seen, len(ids), n_bias, len(p.logit_bias), n_blocked, len(r.blocked), r.last_row)
+        # a window of no tokens: the penalties see nothing, not even the newest token that `last_row` names for the pairs
+        floats[i, 0:3] = (p.repetition_penalty, p.presence_penalty, p.frequency_penalty) if p.repeat_last_n != 0 else (1.0, 0.0, 0.0)
+        records[i, 3:] = (n_seen, len(ids), n_bias, len(p.logit_bias), n_blocked, len(r.blocked), r.last_row,
+                          n_allowed, len(r.allowed), n_pairs, len(r.pairs))
         seen_ids.append(ids)
         seen_counts.append(counts)
-        bias_ids.extend(t if t < (1 << 31) else -1 for t, _ in p.logit_bias)
+        bias_ids.extend(word(t) for t, _ in p.logit_bias)
         bias_values.extend(b for _, b in p.logit_bias)
-        blocked.extend(t if -(1 << 31) <= t < (1 << 31) else -1 for t in r.blocked)
+        blocked.extend(word(t) for t in r.blocked)
+        allowed.extend(min(t, (1 << 31) - 1) for t in sorted(r.allowed))
+        if_last.extend(word(a) for a, _ in r.pairs)
+        then_blocked.extend(word(b) for _, b in r.pairs)
         n_seen, n_bias, n_blocked = n_seen + len(ids), n_bias + len(p.logit_bias), n_blocked + len(r.blocked)
+        n_allowed, n_pairs = n_allowed + len(r.allowed), n_pairs + len(r.pairs)
     parts = [records.reshape(-1)] + seen_ids + seen_counts + [np.asarray(bias_ids, dtype=np.int32),
-                                                              np.asarray(bias_values, dtype=np.float32).view(np.int32),
-                                                              np.asarray(blocked, dtype=np.int32)]
+                                                              np.asarray(bias_values, dtype=np.float32).view(np.int32)]
+    parts += [np.asarray(a, dtype=np.int32) for a in (blocked, allowed, if_last, then_blocked)]
     packed = torch.from_numpy(np.concatenate(parts).astype(np.int32, copy=False))
-    return packed, (n_seen, n_bias, n_blocked)
+    return packed, (n_seen, n_bias, n_blocked, n_allowed, n_pairs)

@@ -29,6 +29,10 @@ class SamplingParams:
     logit_bias: Tuple[Tuple[int, float], ...] = ()   # (token id, what is added to its logit)
     min_tokens: int = 0               # no end-of-sequence or stop id before this many tokens were generated
     priority: int = 0                 # smaller values are served first under the `priority` scheduling policy
+    allowed_token_ids: Tuple[int, ...] = ()          # when not empty, only these tokens can be chosen
+    bad_word_ids: Tuple[Tuple[int, ...], ...] = ()   # token sequences that must not appear: the last token of one cannot
+                                                     # be chosen once the tokens before it stand at the end of the history
+    timeout_secs: Optional[float] = None             # the request is given up this long after it was added (waiting included)
     logprobs: Optional[int] = None    # None: off; n: every token comes with its log-probability in the model's own
                                       # distribution (before penalties, temperature and filters) and the n likeliest tokens
 
@@ -54,6 +58,16 @@ class SamplingParams:
         if any(t < 0 for t, _ in bias) or len({t for t, _ in bias}) != len(bias):
             raise ValueError("logit_bias needs nonnegative token ids, each once")
         object.__setattr__(self, "logit_bias", bias)
+        allowed = tuple(sorted({int(t) for t in self.allowed_token_ids}))
+        if any(t < 0 for t in allowed):
+            raise ValueError("allowed_token_ids must be nonnegative")
+        object.__setattr__(self, "allowed_token_ids", allowed)
+        words = tuple(tuple(int(t) for t in word) for word in self.bad_word_ids)
+        if any(not word or any(t < 0 for t in word) for word in words):
+            raise ValueError("bad_word_ids needs sequences of at least one nonnegative token id")
+        object.__setattr__(self, "bad_word_ids", words)
+        if self.timeout_secs is not None and not self.timeout_secs > 0.0:
+            raise ValueError("timeout_secs must be positive")
 
     @property
     def penalizes(self) -> bool:
@@ -63,7 +77,8 @@ class SamplingParams:
     def adjusts_logits(self, generated: int) -> bool:
         """Whether the logits of the next token are changed before a token is chosen: penalties, biases, or
         end and stop ids that `min_tokens` still blocks after `generated` tokens."""
-        return self.penalizes or bool(self.logit_bias) or generated < self.min_tokens
+        return (self.penalizes or bool(self.logit_bias) or generated < self.min_tokens or bool(self.allowed_token_ids)
+                or bool(self.bad_word_ids))
 
     @property
     def greedy(self) -> bool:

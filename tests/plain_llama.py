@@ -247,14 +247,27 @@ def philox_uniform_many(seed, draw, indices):
     return ((w + np.float32(0.5)) / np.float32(16777216.0)).astype(np.float32)
 
 
-def apply_generation_controls(logits, min_tokens, generated, eos_ids, stop_token_ids):
-    """rust/engine/src/sampling.rs:220-229: while fewer than `min_tokens` tokens were generated, neither an
-    end-of-sequence id nor a stop id can be chosen.  Returns a float32 copy."""
+def apply_generation_controls(logits, min_tokens, generated, eos_ids, stop_token_ids, allowed_token_ids=(), bad_word_ids=(),
+                              history=()):
+    """rust/engine/src/sampling.rs:220-250: while fewer than `min_tokens` tokens were generated, neither an
+    end-of-sequence id nor a stop id can be chosen; with an allow list, nothing outside it; the last token of a bad
+    word not when the word's other tokens are the end of `history` (prompt and generated tokens).  Returns a float32 copy."""
     out = np.asarray(logits, dtype=np.float32).copy()
     if generated < min_tokens:
         for t in list(eos_ids) + list(stop_token_ids):
             if 0 <= t < len(out):
                 out[t] = -np.inf
+    if len(allowed_token_ids):
+        keep = np.zeros(len(out), dtype=bool)
+        keep[[t for t in allowed_token_ids if 0 <= t < len(out)]] = True
+        out[~keep] = -np.inf
+    history = list(history)
+    for word in bad_word_ids:
+        if not len(word):
+            continue
+        before, last = list(word[:-1]), word[-1]
+        if len(history) >= len(before) and history[len(history) - len(before):] == before and 0 <= last < len(out):
+            out[last] = -np.inf
     return out
 
 

@@ -168,26 +168,35 @@ class ReferenceOps:
     def adjust_logits(self, logits, packed, sections, last_tokens=None):
         """The packed lists of `Ops.adjust_logits`, taken apart here and applied with the plain functions."""
         rows, vocab = logits.shape
-        seen, bias, blocked = (int(n) for n in sections)
+        seen, bias, blocked, allowed, pairs = (int(n) for n in sections)
         words = packed.cpu().numpy().astype(np.int32)
-        at = rows * 10
-        seen_ids, seen_counts = words[at:at + seen], words[at + seen:at + 2 * seen]
-        at += 2 * seen
-        bias_ids, bias_values = words[at:at + bias], words[at + bias:at + 2 * bias].view(np.float32)
-        blocked_ids = words[at + 2 * bias:at + 2 * bias + blocked]
+        at = rows * 14
+        lists = []
+        for count in (seen, seen, bias, bias, blocked, allowed, pairs, pairs):
+            lists.append(words[at:at + count])
+            at += count
+        seen_ids, seen_counts, bias_ids, bias_values, blocked_ids, allowed_ids, if_last, then_blocked = lists
+        bias_values = bias_values.view(np.float32)
         for r in range(rows):
-            rec = words[r * 10:(r + 1) * 10]
+            rec = words[r * 14:(r + 1) * 14]
             rep, pres, freq = (float(v) for v in rec[:3].view(np.float32))
-            seen_off, seen_len, bias_off, bias_len, blocked_off, blocked_len, last_row = (int(v) for v in rec[3:])
+            (seen_off, seen_len, bias_off, bias_len, blocked_off, blocked_len, last_row, allowed_off, allowed_len,
+             pairs_off, pairs_len) = (int(v) for v in rec[3:])
             history = []
             for t, n in zip(seen_ids[seen_off:seen_off + seen_len], seen_counts[seen_off:seen_off + seen_len]):
                 history += [int(t)] * int(n)
+            last = int(last_tokens[last_row]) if last_row >= 0 else -1
             if last_row >= 0:
-                history.append(int(last_tokens[last_row]))
+                history.append(last)
             row = plain_llama.apply_penalties(logits[r].float().cpu().numpy(), history, rep, pres, freq, -1,
                                               list(zip(bias_ids[bias_off:bias_off + bias_len].tolist(),
                                                        bias_values[bias_off:bias_off + bias_len].tolist())))
             row[[int(t) for t in blocked_ids[blocked_off:blocked_off + blocked_len] if 0 <= t < vocab]] = -np.inf
+            for a, b in zip(if_last[pairs_off:pairs_off + pairs_len], then_blocked[pairs_off:pairs_off + pairs_len]):
+                if int(a) == last and 0 <= b < vocab:
+                    row[int(b)] = -np.inf
+            if allowed_len:
+                row = plain_llama.apply_generation_controls(row, 0, 0, (), (), allowed_ids[allowed_off:allowed_off + allowed_len].tolist())
             logits[r] = torch.from_numpy(row).to(logits.dtype)
         return logits
 

@@ -345,7 +345,8 @@ def plain_generate(name, prompt, params, eos=()):
     seq = list(prompt)
     for draw in range(params.max_tokens):
         row = plain_llama.forward(cfg, w64, seq)[-1].astype(np.float32)
-        row = plain_llama.apply_generation_controls(row, params.min_tokens, len(seq) - len(prompt), eos, params.stop_token_ids)
+        row = plain_llama.apply_generation_controls(row, params.min_tokens, len(seq) - len(prompt), eos, params.stop_token_ids,
+                                                    params.allowed_token_ids, params.bad_word_ids, seq)
         row = plain_llama.apply_penalties(row, seq, params.repetition_penalty, params.presence_penalty, params.frequency_penalty,
                                           params.repeat_last_n, params.logit_bias)
         token = plain_llama.device_sample(row, params.temperature, params.top_k, params.top_p, params.seed or 0, draw, params.min_p)
@@ -502,3 +503,74 @@ def generated_with_penalty_differs(events):
     """The request with a penalty and a bias did not always take the model's likeliest token: what is reported is the
     model's distribution, not the one the token was chosen from."""
     return any(ev.top_logprobs[0][0] != ev.token_id for ev in events)
+
+
+# ---- allow lists, bad words, timeouts ------------------------------------------------------------
+
+@pytest.mark.parametrize("ahead", [False, True])
+def test_allow_lists_and_bad_words_match_the_plain_order(ahead):
+    """An allow list keeps every choice inside it; a bad word's last token cannot follow its other tokens, also when the
+    newest of them is still on the device (steps launched ahead); a word of one token is blocked always."""
+    free = plain_generate("A", PROMPTS_A[1], SamplingParams(max_tokens=10))
+    assert len(set(zip(free, free[1:]))) > 3
+    # what the free run said becomes forbidden: its second token after its first, its fourth after its second and third,
+    # and its fifth token anywhere
+    words = ((free[0], free[1]), (free[1], free[2], free[3]), (free[4],), (PROMPTS_A[1][-1], free[0], 9))
+    barred = SamplingParams(max_tokens=10, bad_word_ids=words)
+    fenced = SamplingParams(max_tokens=10, allowed_token_ids=(3, 200, 17, 90, 91, 92, 5000), temperature=0.8, seed=4)
+    both = SamplingParams(max_tokens=10, allowed_token_ids=tuple(range(40, 80)), bad_word_ids=((41,), (50, 51)), repetition_penalty=1.4)
+    cases = [("barred", PROMPTS_A[1], barred), ("fenced", PROMPTS_A[2], fenced), ("both", PROMPTS_A[0], both),
+             ("plain", PROMPTS_A[1], SamplingParams(max_tokens=10))]
+    engine = make_engine("A", ahead=ahead)
+    for name, prompt, params in cases:
+        engine.add_request(name, prompt, params)
+    got = {name: [] for name, _, _ in cases}
+    while engine.has_unfinished():
+        for ev in engine.step():
+            got[ev.request_id].append(ev.token_id)
+    for name, prompt, params in cases:
+        assert got[name] == plain_generate("A", prompt, params), name
+    assert got["plain"] == free and got["barred"] != free
+    assert got["barred"][0] == free[0] and got["barred"][1] != free[1] and free[4] not in got["barred"]
+    assert set(got["fenced"]) <= {3, 200, 17, 90, 91, 92} and set(got["both"]) <= set(range(40, 80)) - {41}
+
+
+def test_bad_word_blocks_with_and_without_a_token_on_the_device():
+    from fllm_amd.sampling.adjust import bad_word_blocks
+    words = [(7,), (1, 2, 3), (2, 4), (9, 9, 9, 9), (5, 1, 2, 8)]
+    assert bad_word_blocks(words, [5, 1, 2], 3) == ([7, 3, 4, 8], [])
+    assert bad_word_blocks(words, [1, 2], 2) == ([7, 3, 4], [])
+    # the newest token is not known: what would follow from each value it may have
+    assert bad_word_blocks(words, [5, 1, -1], 2) == ([7], [(2, 3), (2, 4), (2, 8)])
+    assert bad_word_blocks(words, [9, 9, -1], 2) == ([7], [(2, 4), (9, 9)])
+    assert bad_word_blocks(words, [-1], 0) == ([7], [(2, 4)])
+    with pytest.raises(ValueError, match="at least one"):
+        SamplingParams(bad_word_ids=((),))
+    with pytest.raises(ValueError, match="nonnegative"):
+        SamplingParams(allowed_token_ids=(-1,))
+
+
+def test_requests_are_given_up_when_their_time_is_over(monkeypatch):
+    """Waiting counts; the pages go back; the other requests go on (rust/engine/src/runtime.rs:1222-1232)."""
+    import fllm_amd.engine.engine as module
+    now = [100.0]
+    monkeypatch.setattr(module.time, "monotonic", lambda: now[0])
+    engine = make_engine("A", max_seqs=1)
+    engine.add_request("slow", PROMPTS_A[0], SamplingParams(max_tokens=30, timeout_secs=5.0))
+    engine.add_request("waits", PROMPTS_A[1], SamplingParams(max_tokens=4, timeout_secs=2.0))
+    engine.add_request("patient", PROMPTS_A[1], SamplingParams(max_tokens=4))
+    events = engine.step() + engine.step()
+    now[0] += 3.0                                   # the waiting request's time is over before it ever ran
+    events += engine.step()
+    assert [(e.request_id, e.token_id, e.finish_reason) for e in events if e.finished] == [("waits", -1, "timeout")]
+    now[0] += 3.0
+    assert engine.expire_requests() == ["slow"]
+    engine.runner.cache.check_invariants()
+    rest = []
+    while engine.has_unfinished():
+        rest += engine.step()
+    assert [e.token_id for e in rest if e.request_id == "patient"] == plain_greedy("A", PROMPTS_A[1], 4)
+    assert not any(e.request_id == "slow" for e in rest)
+    assert all(p.available == p.num_pages for p in engine.runner.cache.pools)
+    with pytest.raises(ValueError, match="positive"):
+        SamplingParams(timeout_secs=0.0)

@@ -131,6 +131,9 @@ def test_penalties_biases_min_tokens_and_min_p(dtype):
              ("window", prompts[2], SamplingParams(max_tokens=12, repetition_penalty=1.3, frequency_penalty=0.5, repeat_last_n=3)),
              ("held", prompts[1], SamplingParams(max_tokens=8, min_tokens=5, stop_token_ids=(free[2],), logit_bias=((free[3], 4.0), (7, -2.0)))),
              ("drawn", prompts[0], SamplingParams(max_tokens=10, temperature=0.9, top_k=30, min_p=0.08, top_p=0.9, seed=77, presence_penalty=0.6)),
+             ("barred", prompts[1], SamplingParams(max_tokens=12, bad_word_ids=((free[4], free[5]), (free[5], free[6], free[7]), (free[8],)))),
+             ("fenced", prompts[2], SamplingParams(max_tokens=10, allowed_token_ids=tuple(range(30, 90)), bad_word_ids=((31,), (40, 41)),
+                                                   temperature=0.7, seed=3)),
              ("plain", prompts[1], SamplingParams(max_tokens=12))]
 
     def run(ahead, graphs=True):
@@ -149,6 +152,7 @@ def test_penalties_biases_min_tokens_and_min_p(dtype):
     assert run(True) == waited and run(True, graphs=False) == waited
     assert waited["loops"] != free and waited["window"] != free and waited["plain"] == free[:1]
     assert len(waited["held"]) >= 5 and not set(waited["held"][:5]) & (set(eos) | {free[2]})
+    assert set(waited["fenced"]) <= set(range(30, 90)) - {31} and free[8] not in waited["barred"]
     if dtype == "float32":
         _, spec = model_spec_from_config(cfg)
         w64 = tc.to_float64(random_tensors(spec, 1, torch.float32))
@@ -156,7 +160,8 @@ def test_penalties_biases_min_tokens_and_min_p(dtype):
             seq, agree = list(prompt), 0
             for draw, token in enumerate(waited[name]):
                 row = plain_llama.forward(cfg, w64, seq)[-1].astype(np.float32)
-                row = plain_llama.apply_generation_controls(row, params.min_tokens, draw, eos, params.stop_token_ids)
+                row = plain_llama.apply_generation_controls(row, params.min_tokens, draw, eos, params.stop_token_ids,
+                                                            params.allowed_token_ids, params.bad_word_ids, seq)
                 row = plain_llama.apply_penalties(row, seq, params.repetition_penalty, params.presence_penalty,
                                                   params.frequency_penalty, params.repeat_last_n, params.logit_bias)
                 agree += token == plain_llama.device_sample(row, params.temperature, params.top_k, params.top_p, params.seed or 0,
@@ -267,7 +272,8 @@ def test_command_line(tmp_path):
     first = record["token_ids"]
     flags = ["--repeat-penalty", "1.5", "--presence-penalty", "0.3", "--frequency-penalty", "0.2", "--repeat-last-n", "6",
              "--min-tokens", "3", "--stop-token-ids", str(first[0]), "--logit-bias", f"{first[1]}:-5,3:0.5", "--min-p", "0.1",
-             "--temperature", "0.7", "--seed", "5", "--prefix-cache", "--logprobs", "2"]
+             "--temperature", "0.7", "--seed", "5", "--prefix-cache", "--logprobs", "2", "--bad-words-ids", f"{first[2]},{first[3]}",
+             "--allowed-token-ids", ",".join(str(t) for t in range(256) if t != first[4]), "--timeout", "60"]
     proc = subprocess.run(cmd + flags, cwd=ROOT, capture_output=True, text=True, timeout=110)
     assert proc.returncode == 0, proc.stderr
     assert "prefix_hit_tokens=0" in proc.stderr
@@ -276,7 +282,8 @@ def test_command_line(tmp_path):
     record = json.loads(proc.stdout.strip().splitlines()[0])
     params = SamplingParams(max_tokens=8, temperature=0.7, seed=5, min_p=0.1, repetition_penalty=1.5, presence_penalty=0.3,
                             frequency_penalty=0.2, repeat_last_n=6, min_tokens=3, stop_token_ids=(first[0],),
-                            logit_bias=((first[1], -5.0), (3, 0.5)))
+                            logit_bias=((first[1], -5.0), (3, 0.5)), bad_word_ids=((first[2], first[3]),),
+                            allowed_token_ids=tuple(t for t in range(256) if t != first[4]))
     engine = Engine(folder, dtype="float32", num_blocks=16, max_seqs=2)
     assert record["token_ids"] == engine.generate([prompt], params)[0] and first[0] not in record["token_ids"][:3]
 

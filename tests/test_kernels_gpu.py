@@ -752,34 +752,43 @@ def test_sample_rows_that_draw_from_all_tokens_share_workgroups(ops, vocab):
 
 
 def test_adjust_logits(ops):
-    """Penalties, biases and blocked ids on rows of logits against the plain functions: a row with everything, a row
+    """Penalties, biases, blocked and allowed ids on rows of logits against the plain functions: a row with everything, a row
     whose newest token is on the device only and already in its list (it counts once more), one whose newest token
-    is new to the list, a row left alone, ids outside the vocabulary ignored."""
+    is new to the list, a row left alone, ids outside the vocabulary ignored; an allow list (every other token goes,
+    at a vocabulary that is no multiple of the workgroup); pairs that block a token if the newest token, on the
+    device, is a given one, in a row without penalties and in one whose penalties look at no token."""
     from fllm_amd.sampling import SamplingParams
     from fllm_amd.sampling.adjust import AdjustRow, pack
     g = gen(41)
     vocab = 1000
-    logits = torch.randn(5, vocab, generator=g) * 3.0
+    logits = torch.randn(8, vocab, generator=g) * 3.0
     logits[0, 17] = float("nan")
     last_tokens = torch.tensor([5, 123, 999], dtype=torch.int32)
     full = SamplingParams(repetition_penalty=1.7, presence_penalty=0.3, frequency_penalty=0.2, logit_bias=((3, 2.5), (17, 1.0), (4000, 9.0)))
+    allowed = (0, 5, 6, 400, 998, 999, 4000)
     rows = [AdjustRow(full, {5: 2, 17: 1, 900: 4, 4000: 1, 44: 3}, blocked=(1, 2, 4000)),
             AdjustRow(SamplingParams(frequency_penalty=0.5), {123: 2, 7: 1}, last_row=1),
             AdjustRow(SamplingParams(repetition_penalty=0.5), {7: 1}, last_row=2),
             None,
-            AdjustRow(SamplingParams(min_tokens=3), {}, blocked=(0, 999))]
+            AdjustRow(SamplingParams(min_tokens=3), {}, blocked=(0, 999)),
+            AdjustRow(SamplingParams(allowed_token_ids=allowed, presence_penalty=1.0), {5: 1, 7: 2}, blocked=(6,), allowed=allowed),
+            AdjustRow(SamplingParams(bad_word_ids=((1, 2),)), {}, last_row=1, pairs=((123, 40), (124, 41), (123, 4000))),
+            AdjustRow(SamplingParams(repetition_penalty=3.0, repeat_last_n=0), {}, last_row=0, pairs=((5, 50), (6, 51)))]
     packed, sections = pack(rows)
     got = ops.adjust_logits(logits.clone().to(DEV), packed.to(DEV), sections, last_tokens.to(DEV)).cpu()
-    histories = [[5, 5, 17, 900, 900, 900, 900, 4000, 44, 44, 44], [123, 123, 7, 123], [7, 999], [], []]
+    histories = [[5, 5, 17, 900, 900, 900, 900, 4000, 44, 44, 44], [123, 123, 7, 123], [7, 999], [], [], [5, 7, 7], [], []]
+    also_blocked = [(), (), (), (), (), (), (40,), (50,)]
     for r, row in enumerate(rows):
         want = logits[r].numpy()
         if row is not None:
             p = row.params
             want = plain_llama.apply_penalties(want, histories[r], p.repetition_penalty, p.presence_penalty, p.frequency_penalty, -1,
                                                p.logit_bias)
-            want[[t for t in row.blocked if t < vocab]] = -np.inf
+            want[[t for t in row.blocked + also_blocked[r] if t < vocab]] = -np.inf
+            want = plain_llama.apply_generation_controls(want, 0, 0, (), (), row.allowed)
         assert np.array_equal(got[r].numpy(), want, equal_nan=True), r
     assert torch.equal(got[3], logits[3])
+    assert int(torch.isfinite(got[5]).sum()) == 5 and torch.equal(got[7, :50], logits[7, :50])
 
 
 @pytest.mark.parametrize("vocab,top", [(300, 0), (1000, 5), (128256, 20), (7, 7)])

@@ -347,6 +347,24 @@ def test_penalties_and_controls():
     assert P.apply_generation_controls([1.0, 2.0, 3.0, 4.0], 3, 3, [3], [1]).tolist() == [1.0, 2.0, 3.0, 4.0]
 
 
+def test_allow_list_and_bad_words():
+    """rust/engine/src/sampling.rs:228-249.  An allow list of one token forces it (how rust/engine/src/beam_tests.rs:130
+    scores a given continuation), one of all tokens changes nothing, ids outside the vocabulary are ignored; a bad
+    word blocks its last token only behind its other tokens, a word of one token always, a word longer than the
+    history never."""
+    row = np.array([0.5, 3.0, -1.0, 2.0, 0.0], dtype=np.float32)
+    forced = P.apply_generation_controls(row, 0, 0, (), (), allowed_token_ids=(2, 9))
+    assert P.greedy(forced) == 2 and np.isinf(forced[[0, 1, 3, 4]]).all() and forced[2] == row[2]
+    assert np.array_equal(P.apply_generation_controls(row, 0, 0, (), (), allowed_token_ids=range(5)), row)
+    words = ((1,), (4, 3), (0, 4, 0), (2, 2, 2, 2, 2, 2, 3))
+    assert np.array_equal(np.isinf(P.apply_generation_controls(row, 0, 0, (), (), (), words, history=[0, 4])), [True, True, False, True, False])
+    assert np.array_equal(np.isinf(P.apply_generation_controls(row, 0, 0, (), (), (), words, history=[4, 0])), [False, True, False, False, False])
+    assert np.array_equal(np.isinf(P.apply_generation_controls(row, 0, 0, (), (), (), words, history=[])), [False, True, False, False, False])
+    # all of them together with min_tokens: what each blocks adds up
+    out = P.apply_generation_controls(row, 2, 1, (3,), (0,), (0, 2, 3, 4), ((2, 4),), history=[2])
+    assert np.array_equal(np.isinf(out), [True, True, False, True, True])
+
+
 def test_raw_logprobs():
     """rust/engine/src/sampling.rs:970-978: stable around the largest value, ties in token order, no distribution for bad rows."""
     logprob, top = P.raw_logprobs([1000.0, 1000.0, 999.0], 2, 2)
