@@ -97,6 +97,27 @@ class CacheManager:
         self.prefix_hit_tokens += req.length
         return req.length
 
+    def share_pages(self, src_id, dst_id, tokens: int) -> int:
+        """For a request `dst_id` that holds nothing yet: puts the full pages of `src_id` that lie wholly below `tokens`
+        (and below what `src_id` has committed) into its block tables as well, and counts them as committed.  The
+        caller's word: both requests have the same tokens there.  Neither writes such a page again: each writes at and
+        behind its committed length.  Returns the tokens shared; 0 where a group has a window (its pages go back
+        while the request runs), where page sizes differ between groups, and with the prefix index on (which serves
+        the same purpose through `adopt_prefix`)."""
+        src, dst = self._get(src_id), self._get(dst_id)
+        if dst.length != 0 or any(dst.tables) or self.prefix is not None:
+            return 0
+        if any(g.window is not None for g in self.groups) or len({g.page_size for g in self.groups}) != 1:
+            return 0
+        page_size = self.groups[0].page_size
+        pages = min(src.length, int(tokens)) // page_size
+        for g in range(len(self.groups)):
+            for page in src.tables[g][:pages]:
+                self.pools[g].retain(page)
+                dst.tables[g].append(page)
+        dst.length = pages * page_size
+        return dst.length
+
     def remember_prefix(self, req_id, tokens: Sequence[int], known: Optional[int] = None) -> None:
         """Enters the full pages of a request into the index.  `tokens` are the request's tokens from its first on, of
         which the first `known` are final; pages wholly below that and below the committed length are entered.  Where

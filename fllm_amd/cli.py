@@ -70,6 +70,7 @@ def cmd_run(argv: List[str]) -> int:
     ap.add_argument("--top-p", type=float, default=1.0)
     ap.add_argument("--top-k", type=int, default=0)
     ap.add_argument("--seed", type=int, default=None)
+    ap.add_argument("--n", type=int, default=1, help="answers to every prompt (at most 16), each with draws of its own")
     ap.add_argument("--min-p", type=float, default=0.0, help="drop what weighs less than this share of the likeliest token")
     ap.add_argument("--repeat-penalty", type=float, default=1.0, help="repetition penalty on tokens seen before (1: off)")
     ap.add_argument("--presence-penalty", type=float, default=0.0)
@@ -109,28 +110,32 @@ def cmd_run(argv: List[str]) -> int:
                             min_tokens=args.min_tokens, logit_bias=bias, logprobs=args.logprobs,
                             allowed_token_ids=tuple(int(t) for t in args.allowed_token_ids.split(",") if t.strip()),
                             bad_word_ids=tuple(tuple(int(t) for t in w.split(",") if t.strip()) for w in args.bad_words_ids),
-                            timeout_secs=args.timeout)
+                            timeout_secs=args.timeout, n=args.n)
     names = [f"prompt-{i}" for i in range(len(prompts))]
     for name, prompt in zip(names, prompts):
         engine.add_request(name, prompt, params)
-    outputs = {n: [] for n in names}
-    logprobs = {n: [] for n in names}
+    outputs = {(n, k): [] for n in names for k in range(args.n)}
+    logprobs = {(n, k): [] for n in names for k in range(args.n)}
     reasons = {}
     start = time.perf_counter()
     while engine.has_unfinished():
         for ev in engine.step():
             if ev.token_id >= 0:
-                outputs[ev.request_id].append(ev.token_id)
+                outputs[ev.request_id, ev.choice].append(ev.token_id)
             if ev.logprob is not None:
-                logprobs[ev.request_id].append({"logprob": ev.logprob, "top": [[t, v] for t, v in ev.top_logprobs]})
+                logprobs[ev.request_id, ev.choice].append({"logprob": ev.logprob, "top": [[t, v] for t, v in ev.top_logprobs]})
             if ev.finished:
-                reasons[ev.request_id] = ev.finish_reason
+                for k in ([ev.choice] if ev.token_id >= 0 else range(args.n)):      # a timeout ends every answer
+                    reasons.setdefault((ev.request_id, k), ev.finish_reason)
     elapsed = time.perf_counter() - start
     for name, prompt in zip(names, prompts):
-        record = {"request": name, "prompt_tokens": len(prompt), "token_ids": outputs[name], "finish_reason": reasons.get(name)}
-        if args.logprobs is not None:
-            record["logprobs"] = logprobs[name]
-        print(json.dumps(record))
+        for k in range(args.n):
+            record = {"request": name, "prompt_tokens": len(prompt), "token_ids": outputs[name, k], "finish_reason": reasons.get((name, k))}
+            if args.n > 1:
+                record["choice"] = k
+            if args.logprobs is not None:
+                record["logprobs"] = logprobs[name, k]
+            print(json.dumps(record))
     st = engine.stats
     total = sum(len(v) for v in outputs.values())
     print(f"stats: forward_calls={st.forward_calls} rows_total={st.rows_total} max_rows={st.max_rows} "

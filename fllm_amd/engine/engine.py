@@ -28,6 +28,7 @@ class TokenEvent:
     token_id: int
     finished: bool
     finish_reason: Optional[str] = None     # "stop" | "length" | "timeout" (then no token comes with it: token_id -1)
+    choice: int = 0                         # with `SamplingParams.n` > 1: which of the answers the token belongs to
     logprob: Optional[float] = None         # with `SamplingParams.logprobs`: of this token in the model's distribution
     top_logprobs: Optional[List[Tuple[int, float]]] = None     # and the likeliest tokens, (id, log-probability)
 
@@ -124,7 +125,8 @@ class Engine:
             eos_token_ids = getattr(typed, "eos_token_ids", ()) or ()
         self.eos_token_ids = tuple(int(t) for t in eos_token_ids)
         self.stats = EngineStats()
-        self._requests: Dict[str, int] = {}
+        self._requests: Dict[str, List[int]] = {}        # the sequences of a request that have not ended: one an answer
+        self._followers: Dict[int, List[Sequence]] = {}  # further answers that wait until the first one's prompt is computed
         self._deadlines: Dict[str, float] = {}
         self._next_seq = 0
         self.ahead = bool(ahead)
@@ -145,9 +147,14 @@ class Engine:
             if not 0 <= t < self.runner.vocab_size:
                 raise ValueError(f"token id {t} is outside [0, {self.runner.vocab_size})")
         sid = self._next_seq
-        self._next_seq += 1
+        self._next_seq += sampling.n
         self.scheduler.add(Sequence(seq_id=sid, req_id=request_id, tokens=prompt, prompt_len=len(prompt), sampling=sampling))
-        self._requests[request_id] = sid
+        self._requests[request_id] = list(range(sid, sid + sampling.n))
+        if sampling.n > 1:
+            # the other answers join when the first one's prompt is in the cache, and start behind its full pages
+            self._followers[sid] = [Sequence(seq_id=sid + k, req_id=request_id, tokens=list(prompt), prompt_len=len(prompt),
+                                             sampling=sampling.for_choice(k), choice=k, fork_from=sid)
+                                    for k in range(1, sampling.n)]
         self._deadlines.pop(request_id, None)
         if sampling.timeout_secs is not None:
             self._deadlines[request_id] = time.monotonic() + float(sampling.timeout_secs)
@@ -167,9 +174,10 @@ class Engine:
         return expired
 
     def abort_request(self, request_id: str) -> None:
-        sid = self._requests.pop(request_id, None)
-        if sid is not None:
-            self.scheduler.finish(sid)
+        for sid in self._requests.pop(request_id, ()):
+            self._followers.pop(sid, None)
+            if sid in self.scheduler.sequences:
+                self.scheduler.finish(sid)
 
     def clear_prefix_cache(self) -> int:
         """Gives up the cached prefixes that no request uses (rust/engine/src/runtime.rs:1175-1180); returns the pages freed."""
@@ -251,6 +259,8 @@ class Engine:
             if not seq.sampling.greedy:
                 seq.draws += 1
             self.scheduler.commit_decode(sid)
+            for follower in self._followers.pop(sid, ()):       # the prompt is computed: the other answers may begin
+                self.scheduler.add(follower)
         if self.ahead:
             self._in_flight = launched
             events = self._resolve(earlier) if earlier is not None else []
@@ -292,8 +302,12 @@ class Engine:
             reason = "stop" if hit_stop else ("length" if hit_limit else None)
             if reason:
                 self.scheduler.finish(sid)
-                self._requests.pop(seq.req_id, None)
-            event = TokenEvent(seq.req_id, token, reason is not None, reason)
+                left = self._requests.get(seq.req_id)
+                if left is not None:
+                    left.remove(sid)
+                    if not left:
+                        del self._requests[seq.req_id]
+            event = TokenEvent(seq.req_id, token, reason is not None, reason, choice=seq.choice)
             if row in logprobs:
                 event.logprob, alternatives = logprobs[row]
                 event.top_logprobs = alternatives[:seq.sampling.logprobs]
@@ -362,7 +376,8 @@ class Engine:
     # ---- whole requests -------------------------------------------------------------------
     def generate(self, prompts: Seq[Seq[int]], sampling: Union[SamplingParams, Seq[SamplingParams], None] = None
                  ) -> List[List[int]]:
-        """Generated token ids of every prompt (token ids in, token ids out)."""
+        """Generated token ids of every prompt (token ids in, token ids out); for a prompt whose parameters ask for
+        n > 1 answers, the list of its n answers."""
         if sampling is None or isinstance(sampling, SamplingParams):
             sampling = [sampling or SamplingParams()] * len(prompts)
         if len(sampling) != len(prompts):
@@ -372,9 +387,9 @@ class Engine:
             name = f"generate-{self._next_seq}-{i}"
             self.add_request(name, p, s)
             names.append(name)
-        outputs: Dict[str, List[int]] = {n: [] for n in names}
+        outputs: Dict[str, List[List[int]]] = {n: [[] for _ in range(s.n)] for n, s in zip(names, sampling)}
         while any(n in self._requests for n in names):
             for ev in self.step():
                 if ev.request_id in outputs and ev.token_id >= 0:
-                    outputs[ev.request_id].append(ev.token_id)
-        return [outputs[n] for n in names]
+                    outputs[ev.request_id][ev.choice].append(ev.token_id)
+        return [outputs[n][0] if s.n == 1 else outputs[n] for n, s in zip(names, sampling)]

@@ -71,6 +71,8 @@ class Sequence:
     arrival: int = 0
     draws: int = 0                          # random draws taken so far
     seen: Optional[object] = None           # counts of the tokens so far, kept by the engine for requests with penalties
+    choice: int = 0                         # which of the answers to its request's prompt this sequence is
+    fork_from: Optional[int] = None         # a sequence that begins with the same tokens (the first answer, for the others)
 
     @property
     def output_len(self) -> int:
@@ -116,7 +118,7 @@ class Scheduler:
         if len(seq.tokens) > self.max_model_len:
             return False
         self.cache.add_request(sid)
-        reused = self.cache.adopt_prefix(sid, seq.tokens) if self.cfg.prefix_cache else 0
+        reused = self.cache.adopt_prefix(sid, seq.tokens) if self.cfg.prefix_cache else self._share_with_source(seq)
         total = len(seq.tokens) + 1
         missing = self.cache.pages_missing(sid, total)
         watermark = self.cfg.watermark_pages if self.running else 0
@@ -126,6 +128,19 @@ class Scheduler:
         self.cache.reserve(sid, total)
         seq.num_computed = reused
         return True
+
+    def _share_with_source(self, seq: Sequence) -> int:
+        """A further answer to a prompt starts behind the full pages of the first answer's sequence, as far as their
+        tokens are the same, if that one still runs (the reference forks the block table and copies the last block,
+        rust/engine/src/runtime.rs:437-460; here the last, partly filled page is computed again instead)."""
+        source = self.sequences.get(seq.fork_from) if seq.fork_from is not None else None
+        if source is None or source.seq_id not in self.running:
+            return 0
+        limit = min(len(seq.tokens) - 1, len(source.tokens), source.num_computed)     # the last token is always computed
+        same = limit if seq.tokens[:limit] == source.tokens[:limit] else 0
+        while same < limit and seq.tokens[same] == source.tokens[same]:
+            same += 1
+        return self.cache.share_pages(source.seq_id, seq.seq_id, same)
 
     # ---- order ----------------------------------------------------------------------------
     def _key(self, sid: int) -> Tuple[int, int]:

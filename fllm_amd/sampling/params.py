@@ -9,6 +9,8 @@ GREEDY_TEMPERATURE = 1e-5     # temperature at or below this takes the largest l
 _SEED_BASE = 0x8A5CD789635D2DFF
 _SEED_STEP = 0x9E3779B97F4A7C15
 _MASK64 = (1 << 64) - 1
+MAX_CHOICES = 16              # answers to one prompt at most (rust/engine/src/runtime.rs:399-401)
+_CHOICE_SEED_STEP = 0x9E3779B97F4A7C15
 MAX_TOP_LOGPROBS = 20         # alternatives a token at most (sampling.rs:950)
 
 
@@ -29,6 +31,7 @@ class SamplingParams:
     logit_bias: Tuple[Tuple[int, float], ...] = ()   # (token id, what is added to its logit)
     min_tokens: int = 0               # no end-of-sequence or stop id before this many tokens were generated
     priority: int = 0                 # smaller values are served first under the `priority` scheduling policy
+    n: int = 1                        # answers to the one prompt (the reference's `choices`): each with draws of its own
     allowed_token_ids: Tuple[int, ...] = ()          # when not empty, only these tokens can be chosen
     bad_word_ids: Tuple[Tuple[int, ...], ...] = ()   # token sequences that must not appear: the last token of one cannot
                                                      # be chosen once the tokens before it stand at the end of the history
@@ -51,6 +54,8 @@ class SamplingParams:
             raise ValueError("repetition_penalty must be positive")
         if self.min_tokens < 0:
             raise ValueError("min_tokens must be nonnegative")
+        if not 1 <= int(self.n) <= MAX_CHOICES:
+            raise ValueError(f"n must be between 1 and {MAX_CHOICES}")
         if self.logprobs is not None and not 0 <= int(self.logprobs) <= MAX_TOP_LOGPROBS:
             raise ValueError(f"logprobs must be between 0 and {MAX_TOP_LOGPROBS} alternatives")
         object.__setattr__(self, "stop_token_ids", tuple(int(t) for t in self.stop_token_ids))
@@ -87,6 +92,14 @@ class SamplingParams:
     def stops_on(self, token: int, eos: Sequence[int]) -> bool:
         """Explicit stop ids always stop; end-of-sequence ids unless ignored (sampling.rs:89-93)."""
         return token in self.stop_token_ids or (not self.ignore_eos and token in eos)
+
+    def for_choice(self, index: int) -> "SamplingParams":
+        """The parameters of the index-th answer: the same, with a seed of its own where one was given
+        (rust/engine/src/runtime.rs:441-444); without a seed every sequence derives its own anyway."""
+        if index == 0 or self.seed is None:
+            return self
+        from dataclasses import replace
+        return replace(self, seed=(int(self.seed) + index * _CHOICE_SEED_STEP) & _MASK64)
 
     def seed_for(self, sequence_id: int) -> int:
         """sampling.rs:193-199: the request's seed, else one derived from the sequence id."""

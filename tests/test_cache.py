@@ -377,3 +377,33 @@ def test_random_orders_with_shared_prefixes_keep_the_books(seed):
     m.clear_prefixes()
     assert m.pools[0].available == 20 and m.pools[1].available == 20 and m.cached_pages() == 0
     assert adopted > 50 and refused > 0
+
+
+def test_a_request_can_start_on_the_full_pages_of_another():
+    m = CacheManager([full(4), full(4)], [10, 10], max_requests=3)
+    m.add_request("first")
+    m.reserve("first", 11)
+    m.commit("first", 10)                           # two full pages and two tokens
+    m.add_request("second")
+    assert m.share_pages("first", "second", 9) == 8 and m.length("second") == 8
+    assert [m.table("second", g) for g in range(2)] == [m.table("first", g)[:2] for g in range(2)]
+    m.add_request("third")
+    assert m.share_pages("first", "third", 7) == 4   # only pages wholly below the tokens that are the same
+    m.reserve("second", 12)
+    assert m.table("second", 0)[2] != m.table("first", 0)[2]
+    m.check_invariants()
+    assert m.share_pages("first", "second", 9) == 0  # only for a request that holds nothing
+    m.free_request("first")
+    m.check_invariants()
+    assert m.free_pages(0) == 10 - 3                 # the shared pages stay with those who still hold them
+    m.free_request("second")
+    m.free_request("third")
+    m.check_invariants()
+    assert m.free_pages(0) == 10 and m.free_pages(1) == 10
+    # where pages go back while a request runs, nothing is shared
+    w = CacheManager([full(4), windowed(6, 4)], [10, 10], max_requests=2)
+    w.add_request("a")
+    w.reserve("a", 9)
+    w.commit("a", 9)
+    w.add_request("b")
+    assert w.share_pages("a", "b", 8) == 0

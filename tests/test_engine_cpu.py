@@ -574,3 +574,61 @@ def test_requests_are_given_up_when_their_time_is_over(monkeypatch):
     assert all(p.available == p.num_pages for p in engine.runner.cache.pools)
     with pytest.raises(ValueError, match="positive"):
         SamplingParams(timeout_secs=0.0)
+
+
+# ---- several answers to a prompt -----------------------------------------------------------------
+
+@pytest.mark.parametrize("ahead", [False, True])
+@pytest.mark.parametrize("prefix_cache", [False, True])
+def test_several_answers_share_the_prompt_and_draw_for_themselves(ahead, prefix_cache):
+    """n answers: the first computes the prompt, the others start behind its full pages (pages of 8 tokens, a prompt
+    of 40 and one of 21: 32 and 16 tokens each) and draw with seeds of their own; each is what a request of its own
+    with that seed gives.  Greedy answers are all the same."""
+    prompt = tc.random_ids(40, 512, 21)
+    other = tc.random_ids(21, 512, 22)
+    params = SamplingParams(max_tokens=8, temperature=0.9, top_k=20, seed=11, n=3)
+    engine = make_engine("B", ahead=ahead, prefix_cache=prefix_cache, max_seqs=8)
+    answers, greedy = engine.generate([prompt, other], [params, SamplingParams(max_tokens=5, n=2)])
+    assert len(answers) == 3 and len({tuple(a) for a in answers}) == 3 and greedy[0] == greedy[1] and len(greedy[0]) == 5
+    alone = make_engine("B", ahead=ahead)
+    from dataclasses import replace
+    assert answers == [alone.generate([prompt], replace(params.for_choice(k), n=1))[0] for k in range(3)]
+    assert greedy[0] == plain_greedy_b(other, 5)
+    # the prompt rows that were computed: the whole prompts once, and for every further answer what lies behind the full pages
+    assert engine.stats.prefill_rows == 40 + 2 * 8 + 21 + 5
+    engine.runner.cache.check_invariants()
+    assert engine.runner.cache.requests() == [] and not engine.has_unfinished()
+    with pytest.raises(ValueError, match="between 1 and 16"):
+        SamplingParams(n=17)
+
+
+def plain_greedy_b(prompt, count):
+    cfg = tc.CONFIGS["B"]
+    _, spec = model_spec_from_config(cfg)
+    w64 = tc.to_float64(random_tensors(spec, 1, torch.float32))
+    seq = list(prompt)
+    for _ in range(count):
+        seq.append(plain_llama.greedy(plain_llama.forward(cfg, w64, seq)[-1]))
+    return seq[len(prompt):]
+
+
+def test_answers_end_one_by_one_and_abort_together():
+    engine = make_engine("A", max_seqs=4)
+    engine.add_request("r", PROMPTS_A[1], SamplingParams(max_tokens=6, temperature=1.0, seed=2, n=3))
+    events = []
+    for _ in range(4):
+        events += engine.step()
+    assert {e.choice for e in events} == {0, 1, 2}
+    engine.abort_request("r")
+    assert not engine.scheduler.has_work() and engine.runner.cache.requests() == []
+    while engine.has_unfinished():
+        assert engine.step() == []
+    engine.add_request("r", PROMPTS_A[0], SamplingParams(max_tokens=3, n=2))
+    engine.abort_request("r")                       # before the first answer's prompt ran: the others never begin
+    assert not engine.has_unfinished() and engine._followers == {}
+    finished = []
+    engine.add_request("q", PROMPTS_A[0], SamplingParams(max_tokens=3, temperature=1.0, seed=1, n=2))
+    while engine.has_unfinished():
+        finished += [(e.choice, e.finish_reason) for e in engine.step() if e.finished]
+    assert sorted(finished) == [(0, "length"), (1, "length")]
+    engine.runner.cache.check_invariants()

@@ -231,6 +231,28 @@ def test_log_probabilities_come_with_the_tokens(dtype):
     assert engine.runner.graph_replays > 0
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_several_answers_to_a_prompt(dtype):
+    """The further answers start on the first one's full pages (which nobody writes again) and draw with seeds of
+    their own: in float32 each is the answer of a request of its own with that seed; the greedy ones agree with the
+    plain implementation."""
+    from dataclasses import replace
+    vocab = tc.CONFIGS["B"]["vocab_size"]
+    prompt, other = tc.random_ids(100, vocab, 5), tc.random_ids(37, vocab, 6)
+    drawn = SamplingParams(max_tokens=12, temperature=0.8, top_p=0.95, seed=9, n=4)
+    engine = make_engine("B", dtype, max_seqs=8)
+    answers, greedy = engine.generate([prompt, other], [drawn, SamplingParams(max_tokens=12, n=3)])
+    assert len({tuple(a) for a in answers}) == 4 and all(len(a) == 12 for a in answers)
+    check_greedy("B", dtype, [other] * 3, greedy)
+    assert engine.stats.prefill_rows == 100 + 3 * 4 + 37 + 2 * 5          # pages of 8 tokens
+    if dtype == "float32":
+        alone = make_engine("B", dtype)
+        assert answers == [alone.generate([prompt], replace(drawn.for_choice(k), n=1))[0] for k in range(4)]
+        assert greedy[0] == greedy[1] == greedy[2]
+    engine.runner.cache.check_invariants()
+    assert engine.runner.cache.requests() == []
+
+
 def test_no_garbage_collection_while_a_graph_is_captured():
     """Engines that went before leave cycles behind; their collection frees graphs and pinned buffers through the
     HIP runtime, which must not happen while a stream is capturing: the collector is off for the capture's
@@ -273,12 +295,14 @@ def test_command_line(tmp_path):
     flags = ["--repeat-penalty", "1.5", "--presence-penalty", "0.3", "--frequency-penalty", "0.2", "--repeat-last-n", "6",
              "--min-tokens", "3", "--stop-token-ids", str(first[0]), "--logit-bias", f"{first[1]}:-5,3:0.5", "--min-p", "0.1",
              "--temperature", "0.7", "--seed", "5", "--prefix-cache", "--logprobs", "2", "--bad-words-ids", f"{first[2]},{first[3]}",
-             "--allowed-token-ids", ",".join(str(t) for t in range(256) if t != first[4]), "--timeout", "60"]
+             "--allowed-token-ids", ",".join(str(t) for t in range(256) if t != first[4]), "--timeout", "60", "--n", "2"]
     proc = subprocess.run(cmd + flags, cwd=ROOT, capture_output=True, text=True, timeout=110)
     assert proc.returncode == 0, proc.stderr
     assert "prefix_hit_tokens=0" in proc.stderr
     record = json.loads(proc.stdout.strip().splitlines()[0])
     assert len(record["logprobs"]) == len(record["token_ids"]) and all(len(e["top"]) == 2 and e["logprob"] <= 0 for e in record["logprobs"])
+    second = json.loads(proc.stdout.strip().splitlines()[1])
+    assert record["choice"] == 0 and second["choice"] == 1 and second["token_ids"] != record["token_ids"]
     record = json.loads(proc.stdout.strip().splitlines()[0])
     params = SamplingParams(max_tokens=8, temperature=0.7, seed=5, min_p=0.1, repetition_penalty=1.5, presence_penalty=0.3,
                             frequency_penalty=0.2, repeat_last_n=6, min_tokens=3, stop_token_ids=(first[0],),
