@@ -152,8 +152,10 @@ class Engine:
         self._requests[request_id] = list(range(sid, sid + sampling.n))
         if sampling.n > 1:
             # the other answers join when the first one's prompt is in the cache, and start behind its full pages
+            # (not where layers keep state of their own per request: pages can be shared, such state cannot)
+            source = None if self.runner.model.has_state else sid
             self._followers[sid] = [Sequence(seq_id=sid + k, req_id=request_id, tokens=list(prompt), prompt_len=len(prompt),
-                                             sampling=sampling.for_choice(k), choice=k, fork_from=sid)
+                                             sampling=sampling.for_choice(k), choice=k, fork_from=source)
                                     for k in range(1, sampling.n)]
         self._deadlines.pop(request_id, None)
         if sampling.timeout_secs is not None:

@@ -142,6 +142,21 @@ def test_toy_architecture_steps_through_the_engine():
     runner.cache.check_invariants()
 
 
+def test_toy_state_is_never_shared_between_requests():
+    """Pages can be shared between requests that begin alike, a mixer's own state cannot: the prefix cache is refused,
+    and further answers to a prompt run the prompt themselves."""
+    from fllm_amd import Engine, SamplingParams
+    options = dict(config=TOY, seed=5, dtype="float32", num_blocks=32, max_seqs=4, ctx=128, max_batched_tokens=16)
+    with pytest.raises(ValueError, match="state of their own"):
+        Engine(prefix_cache=True, **options)
+    engine = Engine(**options)
+    prompt = tc.random_ids(40, 200, 3)
+    alone = engine.generate([prompt], SamplingParams(max_tokens=6))[0]
+    rows = engine.stats.prefill_rows
+    assert engine.generate([prompt], SamplingParams(max_tokens=6, n=3)) == [[alone] * 3]
+    assert engine.stats.prefill_rows - rows == 3 * 40
+
+
 # ---------------------------------------------------------------------------------------------
 # A feed-forward with routing and another position encoding, again without touching the framework
 # ---------------------------------------------------------------------------------------------
