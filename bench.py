@@ -44,6 +44,7 @@ CONTEXT = 8192
 PROMPT_LEN = 1024
 PREFILL_TOKENS = 2048
 PAGE_SIZE = 16
+SAMPLED = {"temperature": 0.8, "top_k": 50, "top_p": 0.9}     # the sampled point of the default run
 
 
 def linear_params(cfg, layers):
@@ -170,6 +171,9 @@ def main():
     ap.add_argument("--prompt-tokens", type=int, default=PREFILL_TOKENS,
                     help="with --prefill-only: length of the prompt; longer ones run in portions of 2,048 tokens")
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="prompt length of the decode runs (for profiling other contexts)")
+    ap.add_argument("--sampled", action="store_true",
+                    help="for profiling the sampling kernels: the decode runs draw with temperature 0.8, top-k 50 and top-p 0.9 under a "
+                         "repetition penalty of 1.1 and report 5 log-probabilities a token (the headline run is greedy)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine runs on a single MI355X, --gpus {args.gpus} is not supported")
@@ -240,7 +244,8 @@ def main():
 
     results = {}
     for batch in batches:
-        results[batch] = decode_run(engine, rng, vocab, batch, steps, warmup, args.prompt_len, f"b{batch}")
+        results[batch] = decode_run(engine, rng, vocab, batch, steps, warmup, args.prompt_len, f"b{batch}",
+                                    sampling=dict(SAMPLED, repetition_penalty=1.1, logprobs=5) if args.sampled else None)
         print(f"[bench] decode batch {batch}: {results[batch][0]:.1f} tok/s, {results[batch][1]:.3f} ms/step",
               file=sys.stderr, flush=True)
 
@@ -272,7 +277,7 @@ def main():
     if further:
         # the same batch with sampled tokens (temperature 0.8, top-k 50, top-p 0.9): what the sampler adds to a step
         result = decode_run(engine, rng, vocab, args.batch, min(steps, 64), 2, args.prompt_len, "sampled",
-                            sampling={"temperature": 0.8, "top_k": 50, "top_p": 0.9})
+                            sampling=SAMPLED)
         line["points"][f"decode_b{args.batch}_sampled"] = round(result[0], 2)
         print(f"[bench] decode batch {args.batch}, temperature 0.8, top-k 50, top-p 0.9: {result[0]:.1f} tok/s, {result[1]:.3f} ms/step",
               file=sys.stderr, flush=True)
