@@ -66,13 +66,17 @@ def cmd_run(argv: List[str]) -> int:
     ap.add_argument("--prompt-ids", action="append", default=[], help="comma-separated token ids (repeatable)")
     ap.add_argument("--prompts-file", help="JSON file: a list of token id lists")
     ap.add_argument("--max-tokens", type=int, default=64)
-    ap.add_argument("--temperature", type=float, default=0.0)
-    ap.add_argument("--top-p", type=float, default=1.0)
-    ap.add_argument("--top-k", type=int, default=0)
+    ap.add_argument("--temperature", "--temp", dest="temperature", type=float, default=None, help="0: greedy (the default)")
+    ap.add_argument("--top-p", type=float, default=None)
+    ap.add_argument("--top-k", type=int, default=None)
+    ap.add_argument("--generation-config", default="auto", metavar="auto|vllm|PATH",
+                    help="where sampling defaults come from when a flag is left out: the model folder's generation_config.json "
+                         "(auto), nowhere (vllm), or a file or folder named here; of its keys temperature, top_p, top_k, min_p "
+                         "and repetition_penalty count")
     ap.add_argument("--seed", type=int, default=None)
     ap.add_argument("--n", type=int, default=1, help="answers to every prompt (at most 16), each with draws of its own")
-    ap.add_argument("--min-p", type=float, default=0.0, help="drop what weighs less than this share of the likeliest token")
-    ap.add_argument("--repeat-penalty", type=float, default=1.0, help="repetition penalty on tokens seen before (1: off)")
+    ap.add_argument("--min-p", type=float, default=None, help="drop what weighs less than this share of the likeliest token")
+    ap.add_argument("--repeat-penalty", type=float, default=None, help="repetition penalty on tokens seen before (1: off)")
     ap.add_argument("--presence-penalty", type=float, default=0.0)
     ap.add_argument("--frequency-penalty", type=float, default=0.0)
     ap.add_argument("--repeat-last-n", type=int, default=-1, help="tokens of the history the penalties look at (negative: all)")
@@ -89,6 +93,15 @@ def cmd_run(argv: List[str]) -> int:
     _engine_options(ap)
     args = ap.parse_args(argv)
     from . import SamplingParams
+    from .config.files import generation_defaults
+    import os
+    defaults, origin = generation_defaults(args.generation_config, args.model if os.path.isdir(args.model) else None)
+    if defaults:
+        print(f"sampling defaults from {origin}: " + ", ".join(f"{k}={v}" for k, v in defaults.items()), file=sys.stderr)
+    builtin = {"temperature": 0.0, "top_p": 1.0, "top_k": 0, "min_p": 0.0, "repetition_penalty": 1.0}
+    given = {"temperature": args.temperature, "top_p": args.top_p, "top_k": args.top_k, "min_p": args.min_p,
+             "repetition_penalty": args.repeat_penalty}
+    chosen = {k: given[k] if given[k] is not None else defaults.get(k, builtin[k]) for k in builtin}
     prompts = [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids]
     if args.prompts_file:
         with open(args.prompts_file) as fh:
@@ -103,9 +116,8 @@ def cmd_run(argv: List[str]) -> int:
               file=sys.stderr)
     stops = tuple(int(t) for t in args.stop_token_ids.split(",") if t.strip())
     bias = tuple((int(t), float(b)) for t, b in (pair.split(":") for pair in args.logit_bias.split(",") if pair.strip()))
-    params = SamplingParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k, seed=args.seed,
-                            max_tokens=args.max_tokens, stop_token_ids=stops, ignore_eos=args.ignore_eos, min_p=args.min_p,
-                            repetition_penalty=args.repeat_penalty, presence_penalty=args.presence_penalty,
+    params = SamplingParams(seed=args.seed, max_tokens=args.max_tokens, stop_token_ids=stops, ignore_eos=args.ignore_eos,
+                            **chosen, presence_penalty=args.presence_penalty,
                             frequency_penalty=args.frequency_penalty, repeat_last_n=args.repeat_last_n,
                             min_tokens=args.min_tokens, logit_bias=bias, logprobs=args.logprobs,
                             allowed_token_ids=tuple(int(t) for t in args.allowed_token_ids.split(",") if t.strip()),

@@ -123,6 +123,9 @@ class Engine:
         self.sampler = Sampler(self.runner.rt)
         if eos_token_ids is None:
             eos_token_ids = getattr(typed, "eos_token_ids", ()) or ()
+            if not eos_token_ids and model is not None and os.path.isdir(model):
+                from ..config.files import generation_eos_ids
+                eos_token_ids = generation_eos_ids(model)
         self.eos_token_ids = tuple(int(t) for t in eos_token_ids)
         self.stats = EngineStats()
         self._requests: Dict[str, List[int]] = {}        # the sequences of a request that have not ended: one an answer

@@ -100,3 +100,29 @@ def test_spec_describes_every_layer():
     assert spec.head.tensors["weight"] == "lm_head.weight"
     _, tied = model_spec_from_config(tc.TINY_B)
     assert tied.head.tensors["weight"] == "model.embed_tokens.weight"
+
+
+def test_generation_defaults_of_a_model_folder(tmp_path):
+    """rust/engine/src/server/gencfg.rs:93-135, and its test at :165-190: the five sampling keys count whether or not
+    do_sample is set; values no sampler can use are dropped; `vllm` means none; a file named outright must be there."""
+    import json
+    from fllm_amd.config.files import generation_defaults, generation_eos_ids
+    folder = tmp_path / "model"
+    folder.mkdir()
+    assert generation_defaults("auto", str(folder)) == ({}, "none in the model")
+    (folder / "generation_config.json").write_text(json.dumps(
+        {"do_sample": False, "temperature": 0.6000004, "top_p": 0.9, "top_k": 0, "min_p": 1.5, "repetition_penalty": 1.1,
+         "eos_token_id": [128001, 128008, 128009], "max_length": 20}))
+    got, origin = generation_defaults("auto", str(folder))
+    assert got == {"temperature": 0.6, "top_p": 0.9, "top_k": 0, "repetition_penalty": 1.1} and origin.endswith("generation_config.json")
+    assert generation_defaults("vllm", str(folder))[0] == {}
+    assert generation_defaults(str(folder), None)[0] == got and generation_defaults(str(folder / "generation_config.json"), None)[0] == got
+    assert generation_eos_ids(str(folder)) == (128001, 128008, 128009)
+    with pytest.raises(ConfigError, match="cannot read generation defaults"):
+        generation_defaults(str(tmp_path / "nothing.json"), None)
+    (folder / "generation_config.json").write_text("{ not json")
+    assert generation_defaults("auto", str(folder)) == ({}, "none in the model") and generation_eos_ids(str(folder)) == ()
+    with pytest.raises(ConfigError, match="cannot read generation defaults"):
+        generation_defaults(str(folder), None)
+    (folder / "generation_config.json").write_text(json.dumps({"temperature": float("nan"), "top_k": -1, "top_p": True, "eos_token_id": 2}))
+    assert generation_defaults("auto", str(folder))[0] == {} and generation_eos_ids(str(folder)) == (2,)

@@ -310,6 +310,22 @@ def test_command_line(tmp_path):
                             allowed_token_ids=tuple(t for t in range(256) if t != first[4]))
     engine = Engine(folder, dtype="float32", num_blocks=16, max_seqs=2)
     assert record["token_ids"] == engine.generate([prompt], params)[0] and first[0] not in record["token_ids"][:3]
+    # sampling defaults and end-of-sequence ids that ship with the model: flags that are left out take them, `vllm` ignores them
+    with open(os.path.join(folder, "generation_config.json"), "w") as fh:
+        json.dump({"temperature": 0.9, "top_k": 12, "repetition_penalty": 1.3, "eos_token_id": [first[5]]}, fh)
+    config = json.load(open(os.path.join(folder, "config.json")))
+    config.pop("eos_token_id", None)
+    with open(os.path.join(folder, "config.json"), "w") as fh:
+        json.dump(config, fh)
+    proc = subprocess.run(cmd + ["--seed", "8", "--top-k", "20"], cwd=ROOT, capture_output=True, text=True, timeout=110)
+    assert proc.returncode == 0 and "sampling defaults from" in proc.stderr, proc.stderr
+    engine = Engine(folder, dtype="float32", num_blocks=16, max_seqs=2)
+    assert engine.eos_token_ids == (first[5],)
+    want = engine.generate([prompt], SamplingParams(max_tokens=8, temperature=0.9, top_k=20, repetition_penalty=1.3, seed=8))[0]
+    assert json.loads(proc.stdout.strip().splitlines()[0])["token_ids"] == want
+    proc = subprocess.run(cmd + ["--generation-config", "vllm"], cwd=ROOT, capture_output=True, text=True, timeout=110)
+    assert proc.returncode == 0, proc.stderr
+    assert json.loads(proc.stdout.strip().splitlines()[0])["token_ids"] == engine.generate([prompt], SamplingParams(max_tokens=8))[0]
 
 
 @pytest.mark.parametrize("budget,prompt_len", [(512, 512), (2, 40)])
