@@ -406,7 +406,7 @@ __device__ uint32_t thresholds(KeyAt key_at, WeightAt weight_at, int n, int top_
 }
 
 // Calls f(token, logit) for every token of a row, each thread of the workgroup with a share of its own: four
-// consecutive tokens a load where the row's alignment allows (two such loads in flight), single tokens at both ends.
+// consecutive tokens a load where the row's alignment allows (four such loads in flight), single tokens at both ends.
 // A thread meets its tokens in the same order in every pass.
 template <typename F>
 __device__ __forceinline__ void for_each_token(const float *__restrict__ src, int vocab, F f) {
@@ -415,15 +415,18 @@ __device__ __forceinline__ void for_each_token(const float *__restrict__ src, in
     const int quads = (vocab - head) / 4;
     const f32x4_t *q = (const f32x4_t *)(src + head);
     int i = threadIdx.x;
-    for (; i + kBlock < quads; i += 2 * kBlock) {
-        const f32x4_t a = q[i], b = q[i + kBlock];
-        const int ta = head + 4 * i, tb = head + 4 * (i + kBlock);
+    for (; i + 3 * kBlock < quads; i += 4 * kBlock) {
+        f32x4_t v[4];
 #pragma unroll
-        for (int e = 0; e < 4; e++) f(ta + e, a[e]);
+        for (int u = 0; u < 4; u++) v[u] = q[i + u * kBlock];
 #pragma unroll
-        for (int e = 0; e < 4; e++) f(tb + e, b[e]);
+        for (int u = 0; u < 4; u++) {
+            const int t = head + 4 * (i + u * kBlock);
+#pragma unroll
+            for (int e = 0; e < 4; e++) f(t + e, v[u][e]);
+        }
     }
-    if (i < quads) {
+    for (; i < quads; i += kBlock) {
         const f32x4_t a = q[i];
         const int ta = head + 4 * i;
 #pragma unroll
