@@ -741,26 +741,16 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
     if (s_seen != live_splits - 1) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
-    // The parts are read eight at a time, all loads of a group asked for before the first is used: two round trips to
-    // memory a group instead of two a part.
+    // The parts are read eight at a time, all loads of a group asked for before the first is used.  The first group's
+    // values are kept: up to eight parts (the usual case) cost one round trip to memory, not one for the largest
+    // maximum and another for the sums.
     constexpr int GRP = 8;
     for (int idx = threadIdx.x; idx < gq * D; idx += WAVES * kWave) {
         const int qi = idx / D, d = idx - qi * D;
         const size_t hrow = (size_t)row * p.heads + kvh * G + qtile * 16 + qi;
         const float *ml = p.ws_ml + hrow * p.splits * 2;
         const float *po = p.ws_o + hrow * p.splits * D + d;
-        float m = -INFINITY;
-        for (int s0 = 0; s0 < live_splits; s0 += GRP) {
-            float ms[GRP];
-#pragma unroll
-            for (int i = 0; i < GRP; i++)
-                ms[i] = s0 + i < live_splits ? __hip_atomic_load(ml + (s0 + i) * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;
-#pragma unroll
-            for (int i = 0; i < GRP; i++) m = fmaxf(m, ms[i]);
-        }
-        float l = 0.f, acc = 0.f;
-        for (int s0 = 0; s0 < live_splits; s0 += GRP) {
-            float ms[GRP], ls[GRP], os[GRP];
+        auto load_group = [&](int s0, float (&ms)[GRP], float (&ls)[GRP], float (&os)[GRP]) {
 #pragma unroll
             for (int i = 0; i < GRP; i++) {
                 const bool live = s0 + i < live_splits;
@@ -768,12 +758,34 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
                 ls[i] = live ? __hip_atomic_load(ml + (s0 + i) * 2 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
                 os[i] = live ? __hip_atomic_load(po + (size_t)(s0 + i) * D, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
             }
+        };
+        float l = 0.f, acc = 0.f;
+        auto add_group = [&](float m, const float (&ms)[GRP], const float (&ls)[GRP], const float (&os)[GRP]) {
 #pragma unroll
             for (int i = 0; i < GRP; i++) {       // in the order of the parts
                 const float f = ms[i] == -INFINITY ? 0.f : fast_exp2(ms[i] - m);
                 l += ls[i] * f;
                 acc += os[i] * f;
             }
+        };
+        float ms0[GRP], ls0[GRP], os0[GRP];
+        load_group(0, ms0, ls0, os0);
+        float m = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < GRP; i++) m = fmaxf(m, ms0[i]);
+        for (int s0 = GRP; s0 < live_splits; s0 += GRP) {
+            float ms[GRP];
+#pragma unroll
+            for (int i = 0; i < GRP; i++)
+                ms[i] = s0 + i < live_splits ? __hip_atomic_load(ml + (s0 + i) * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;
+#pragma unroll
+            for (int i = 0; i < GRP; i++) m = fmaxf(m, ms[i]);
+        }
+        add_group(m, ms0, ls0, os0);
+        for (int s0 = GRP; s0 < live_splits; s0 += GRP) {
+            float ms[GRP], ls[GRP], os[GRP];
+            load_group(s0, ms, ls, os);
+            add_group(m, ms, ls, os);
         }
         p.out[hrow * D + d] = (bf16_t)(l > 0.f ? acc / l : 0.f);
     }
