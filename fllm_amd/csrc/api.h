@@ -66,6 +66,21 @@ int fllm_norm_qkv_rope_store(const float *x, const float *norm_w, float eps, con
                              void *v_pages, int M, int heads, int kv_heads, int head_dim, int K, int page_size,
                              int store_kv, hipStream_t stream);
 
+// A norm prepared by the product before it, for steps of up to 16 rows.  fllm_linear_add_normed: out += x w^T
+// (float32 out [M, N], N a multiple of 16) and, for the RMSNorm that reads out next, next_x = out * next_w as
+// bfloat16 [M, N] and next_ssq [M, *tiles_out]: the sums of squares of out over the outputs of each tile (room for
+// M * N / 8 floats; *tiles_out, host memory, is set at the call).  The scaled forms are the norm forms above with
+// that pair in place of the float32 rows and the norm's weight.
+int fllm_linear_add_normed(const void *x, int ldx, const void *w, const float *bias, float *out, int M, int N, int K,
+                           const float *next_w, void *next_x, float *next_ssq, int *tiles_out, hipStream_t stream);
+int fllm_scaled_gate_up_swiglu(const void *xn, const float *ssq, int ssq_count, float eps, const void *w_gate_up,
+                               const float *bias, void *out, int M, int inter, int K, hipStream_t stream);
+int fllm_scaled_qkv_rope_store(const void *xn, const float *ssq, int ssq_count, float eps, const void *w_qkv, const float *bias,
+                               void *q_out, const int32_t *row_pos, const int32_t *row_seg, const int32_t *tables,
+                               int table_stride, const float *cos_table, const float *sin_table, int rope_dims, void *k_pages,
+                               void *v_pages, int M, int heads, int kv_heads, int head_dim, int K, int page_size, int store_kv,
+                               hipStream_t stream);
+
 // residual[r, :] += branch[r, :]   (residual float32 [rows, width], branch of type `dtype`)
 int fllm_add_residual(float *residual, const void *branch, int rows, int width, int dtype, hipStream_t stream);
 

@@ -5,7 +5,13 @@
 //             NORM_F32  x is the float32 residual stream; the operand is x * norm_weight and the row's
 //                       rsqrt(mean(x^2) + eps) is applied to the sums afterwards (a row scale commutes
 //                       with the product), so RMSNorm costs no pass of its own
-//   epilogue  STORE / STORE_F32 / ADD (add to the float32 residual stream)
+//             SCALED    the same norm, prepared by the product before: x * norm_weight arrives as bfloat16
+//                       rows, and every row's sum of squares in parts (one a tile of that product's
+//                       outputs), which are added in order.  Half the bytes of NORM_F32 and no conversion
+//                       (up to 16 rows)
+//   epilogue  STORE / STORE_F32 / ADD (add to the float32 residual stream; on request it also leaves what
+//                       the SCALED prologue of the next product takes: the new rows times the next norm's
+//                       weight in bfloat16, and each tile's share of the rows' sums of squares)
 //             QKV       rotate query and key lanes (pairs (2l, 2l+1)), write queries to a buffer and
 //                       keys and values straight into the pages of each row's request
 //             SWIGLU    rows n and I + n of the concatenated gate/up matrix go to one workgroup, which
@@ -44,7 +50,7 @@ __device__ __forceinline__ f32x4_t take_over(__amdgpu_buffer_rsrc_t ws, unsigned
     return (f32x4_t){__uint_as_float(bits[0]), __uint_as_float(bits[1]), __uint_as_float(bits[2]), __uint_as_float(bits[3])};
 }
 
-enum { PRO_BF16 = 0, PRO_NORM_F32 = 1 };
+enum { PRO_BF16 = 0, PRO_NORM_F32 = 1, PRO_SCALED = 2 };
 enum { EPI_STORE = 0, EPI_STORE_F32 = 1, EPI_ADD = 2, EPI_QKV = 3, EPI_SWIGLU = 4 };
 
 struct SkinnyArgs {
@@ -69,6 +75,15 @@ struct SkinnyArgs {
     int rope_dims;
     bf16_t *k_pages, *v_pages;
     int heads, kv_heads, head_dim, page_size, store_kv;
+    // ADD epilogue, on request (next_x != null): for the norm that reads the sums next
+    const float *next_w;   // [N] that norm's weight
+    bf16_t *next_x;        // [M, N] (out + sum) * next_w
+    float *next_ssq;       // [M, next_tiles] sum of squares of (out + sum) over a tile's outputs
+    int next_nt, next_tiles;   // outputs a tile (16 or 8) and tiles a row: set by the launch
+    int *next_tiles_out;   // host memory: where the launch leaves next_tiles for the caller
+    // SCALED prologue
+    const float *ssq_in;   // [M, ssq_count]
+    int ssq_count;
 };
 
 __device__ __forceinline__ bf16x4_t pack4(f32x4_t v) {
@@ -101,6 +116,7 @@ __device__ __forceinline__ void sum_waves(const f32x4_t *red, int stride_t, int 
 struct EpilogueOperands {
     bool have = false;     // resid / cs / sn hold this item's values
     f32x4_t resid;         // EPI_ADD: out[m, nb .. nb + 3]
+    f32x4_t next_w;        // EPI_ADD that prepares the next norm: that norm's weight at nb .. nb + 3
     float cs[2], sn[2];    // EPI_QKV: cosine and sine of the two pairs at nb, nb + 2
     int seg = -1, pos = 0, page = 0;   // EPI_QKV: the row's segment, position and page (do not depend on the item)
 };
@@ -120,6 +136,7 @@ __device__ __forceinline__ void load_item_operands(const SkinnyArgs &a, int m, i
     if (EPI == EPI_ADD) {
         if (nb + 3 < n_out && (a.ldo & 3) == 0 && ((uintptr_t)a.out & 15) == 0) {
             e.resid = *(const f32x4_t *)((const float *)a.out + (size_t)m * a.ldo + nb);
+            if (a.next_x != nullptr) e.next_w = *(const f32x4_t *)(a.next_w + nb);
             e.have = true;
         }
     } else if (EPI == EPI_QKV) {
@@ -139,7 +156,7 @@ template <int PRO, int EPI, int RT>
 __device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], float ss, int m, int nb, int n_out,
                                          const EpilogueOperands &e) {
     const int N = a.N, K = a.K;
-    if (PRO == PRO_NORM_F32) {
+    if (PRO != PRO_BF16) {
         const float inv = 1.0f / sqrtf(ss / (float)K + a.eps);
 #pragma unroll
         for (int t = 0; t < RT; t++) s[t] *= inv;
@@ -153,11 +170,20 @@ __device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], 
     }
     // the four outputs of a lane are neighbours in a row: one store where the row's pitch and the base keep them aligned
     const bool whole = nb + 3 < n_out && (a.ldo & 3) == 0;
-    if (EPI == EPI_ADD && e.have) {
-        *(f32x4_t *)((float *)a.out + (size_t)m * a.ldo + nb) = e.resid + s[0];
-    } else if (EPI == EPI_ADD && whole && ((uintptr_t)a.out & 15) == 0) {
+    if (EPI == EPI_ADD && (e.have || (whole && ((uintptr_t)a.out & 15) == 0))) {
         f32x4_t *dst = (f32x4_t *)((float *)a.out + (size_t)m * a.ldo + nb);
-        *dst = *dst + s[0];
+        const f32x4_t sum = (e.have ? e.resid : *dst) + s[0];
+        *dst = sum;
+        if (a.next_x != nullptr) {
+            // For the norm that reads these rows next: its operand, and this tile's share of the row's sum of squares.
+            // The lanes that hold a row's outputs of this tile sit 16 (and 32) lanes apart and are all here.
+            const f32x4_t w = e.have ? e.next_w : *(const f32x4_t *)(a.next_w + nb);
+            *(bf16x4_t *)(a.next_x + (size_t)m * a.N + nb) = pack4(sum * w);
+            float sq = sum[0] * sum[0] + sum[1] * sum[1] + sum[2] * sum[2] + sum[3] * sum[3];
+            sq += __shfl_xor(sq, 16, kWave);
+            if (a.next_nt == 16) sq += __shfl_xor(sq, 32, kWave);
+            if ((threadIdx.x & (kWave - 1)) < 16) a.next_ssq[(size_t)m * a.next_tiles + nb / a.next_nt] = sq;
+        }
     } else if (EPI == EPI_STORE && whole && ((uintptr_t)a.out & 7) == 0) {
         *(bf16x4_t *)((bf16_t *)a.out + (size_t)m * a.ldo + nb) = pack4(s[0]);
     } else if (EPI == EPI_STORE_F32 && whole && ((uintptr_t)a.out & 15) == 0) {
@@ -327,6 +353,17 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
         if (++l_j == nbw) l_j = 0, l_item++;
     };
     (void)wrow_in_tile;
+    // SCALED: the parts of the sums of squares of this wave's rows (rows wave and wave + WAVES) are asked for before
+    // anything else and added up after the staging, when they have long arrived: up to 256 parts a row, four a lane
+    f32x4_t ssq_pre[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    const bool ssq_quick = PRO == PRO_SCALED && a.ssq_count <= 4 * kWave && (a.ssq_count & 3) == 0 && ((uintptr_t)a.ssq_in & 15) == 0;
+    if (PRO == PRO_SCALED && ssq_quick && sl == 0) {
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            const int m = wave + k * WAVES;
+            if (m < M && lane * 4 < a.ssq_count) ssq_pre[k] = *(const f32x4_t *)(a.ssq_in + (size_t)m * a.ssq_count + lane * 4);
+        }
+    }
     Block b0, b1;
     issue(b0);      // in flight while the activations are staged
     issue(b1);
@@ -343,12 +380,22 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
     item_operands(0);
 
     // the wave's own columns kw0 .. kw1 of every row
-    if (PRO == PRO_NORM_F32 && lane < 16) ssq_part[wave * 16 + lane] = 0.f;
+    if (PRO != PRO_BF16 && lane < 16) ssq_part[wave * 16 + lane] = 0.f;
     __builtin_amdgcn_wave_barrier();
+    if (PRO == PRO_SCALED && sl == 0 && !ssq_quick) {
+        // the rows' sums of squares arrive in parts: wave w adds those of rows w, w + WAVES, ..., lane by lane in
+        // index order and then across the lanes, which no other row or wave changes
+        for (int m = wave; m < M; m += WAVES) {
+            float t = 0.f;
+            for (int i = lane; i < a.ssq_count; i += kWave) t += a.ssq_in[(size_t)m * a.ssq_count + i];
+            t = wave_sum(t);
+            if (lane == 0) ssq_part[wave * 16 + m] = t;
+        }
+    }
     for (int cw = kw0; cw < (XD ? 0 : kw1); cw += kWave * 8) {   // the same trips for every lane: the sums below are over the wave
         const int c0 = cw + lane * 8;
         const bool in = c0 < kw1;
-        if (PRO == PRO_BF16) {
+        if (PRO != PRO_NORM_F32) {
             const bf16_t *x = (const bf16_t *)a.x + ks0 + c0;
             for (int m0 = 0; m0 < M; m0 += 4) {
                 bf16x8_t v[4];
@@ -388,6 +435,16 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
                     ss = wave_sum(ss);
                     if (lane == 0) ssq_part[wave * 16 + m0 + i] += ss;
                 }
+            }
+        }
+    }
+    if (PRO == PRO_SCALED && ssq_quick && sl == 0) {
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            const int m = wave + k * WAVES;
+            if (m < M) {      // the same for all lanes of the wave
+                const float t = wave_sum((ssq_pre[k][0] + ssq_pre[k][1]) + (ssq_pre[k][2] + ssq_pre[k][3]));
+                if (lane == 0) ssq_part[wave * 16 + m] = t;
             }
         }
     }
@@ -436,7 +493,7 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
             do {
                 const int m = m_out, nb = tile * NT + g * 4;
                 float ss = 0.f;
-                if (PRO == PRO_NORM_F32) {
+                if (PRO != PRO_BF16) {
 #pragma unroll
                     for (int wv = 0; wv < WAVES; wv++) ss += ssq_part[wv * 16 + m];
                 }
@@ -448,7 +505,7 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
 #pragma unroll
                             for (int i = 0; i < 4; i++)
                                 __hip_atomic_store(part + t * kWave * 4 + i, s[t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        if (PRO == PRO_NORM_F32 && g == 0)
+                        if (PRO != PRO_BF16 && g == 0)
                             __hip_atomic_store(a.ws_ssq + (size_t)(tile * S + sl) * 16 + m, ss, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     }
                     // Every access to the workspace goes to the device's point of coherence by itself (agent-scope
@@ -478,7 +535,7 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
 #pragma unroll
                                 for (int i = 0; i < 4; i++)
                                     pv[j][t][i] = live ? __hip_atomic_load(src + t * kWave * 4 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
-                            ps[j] = (PRO == PRO_NORM_F32 && live)
+                            ps[j] = (PRO != PRO_BF16 && live)
                                         ? __hip_atomic_load(a.ws_ssq + (size_t)(tile * S + s0 + j) * 16 + m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
                                         : 0.f;
                         }
@@ -1003,6 +1060,11 @@ int launch_resident_plan(SkinnyArgs a, const ResidentPlan &p, int ntiles, const 
     a.S = p.S;
     a.slice = p.slice;
     a.ssq_off = (int)(p.stage + p.red);
+    if (a.next_x != nullptr) {
+        a.next_nt = TM == TM_ROWS16 ? 16 : 8;
+        a.next_tiles = ntiles;
+        if (a.next_tiles_out != nullptr) *a.next_tiles_out = ntiles;
+    }
     if (p.S > 1) {
         a.counters = (int *)ws.base;
         a.ws = (float *)((unsigned char *)ws.base + kCounterBytes);
@@ -1252,21 +1314,15 @@ extern "C" int fllm_gate_up_swiglu(const void *x, int ldx, const void *w_gate_up
     return rc;
 }
 
-extern "C" int fllm_norm_qkv_rope_store(const float *x, const float *norm_w, float eps, const void *w_qkv, const float *bias,
-                                        void *q_out, const int32_t *row_pos, const int32_t *row_seg, const int32_t *tables,
-                                        int table_stride, const float *cos_table, const float *sin_table, int rope_dims,
-                                        void *k_pages, void *v_pages, int M, int heads, int kv_heads, int head_dim, int K,
-                                        int page_size, int store_kv, hipStream_t stream) {
-    FLLM_REQUIRE(fllm_fused_decode_supported(M, K), "norm_qkv_rope_store: takes 1..64 rows and K a multiple of 8 (M=%d K=%d)", M, K);
-    FLLM_REQUIRE(aligned16(x) && aligned16(w_qkv) && aligned16(norm_w), "norm_qkv_rope_store: operands must be 16-byte aligned");
-    FLLM_REQUIRE(head_dim % 4 == 0 && rope_dims % 2 == 0 && rope_dims <= head_dim && rope_dims >= 0,
-                 "norm_qkv_rope_store: head_dim %d must be a multiple of 4 and rope_dims %d even and no larger", head_dim, rope_dims);
-    FLLM_REQUIRE(heads > 0 && kv_heads > 0 && page_size > 0 && table_stride > 0 && eps > 0.f, "norm_qkv_rope_store: bad sizes");
-    FLLM_REQUIRE(!store_kv || (k_pages && v_pages), "norm_qkv_rope_store: pages missing");
+namespace {
+// the arguments of the q/k/v forms, whatever their prologue
+SkinnyArgs qkv_args(const void *x, float eps, const void *w_qkv, const float *bias, void *q_out, const int32_t *row_pos,
+                    const int32_t *row_seg, const int32_t *tables, int table_stride, const float *cos_table,
+                    const float *sin_table, int rope_dims, void *k_pages, void *v_pages, int M, int heads, int kv_heads,
+                    int head_dim, int K, int page_size, int store_kv) {
     SkinnyArgs a = {};
     a.x = x;
     a.ldx = K;
-    a.norm_w = norm_w;
     a.eps = eps;
     a.w = (const bf16_t *)w_qkv;
     a.bias = bias;
@@ -1289,7 +1345,102 @@ extern "C" int fllm_norm_qkv_rope_store(const float *x, const float *norm_w, flo
     a.head_dim = head_dim;
     a.page_size = page_size;
     a.store_kv = store_kv;
+    return a;
+}
+}  // namespace
+
+extern "C" int fllm_norm_qkv_rope_store(const float *x, const float *norm_w, float eps, const void *w_qkv, const float *bias,
+                                        void *q_out, const int32_t *row_pos, const int32_t *row_seg, const int32_t *tables,
+                                        int table_stride, const float *cos_table, const float *sin_table, int rope_dims,
+                                        void *k_pages, void *v_pages, int M, int heads, int kv_heads, int head_dim, int K,
+                                        int page_size, int store_kv, hipStream_t stream) {
+    FLLM_REQUIRE(fllm_fused_decode_supported(M, K), "norm_qkv_rope_store: takes 1..64 rows and K a multiple of 8 (M=%d K=%d)", M, K);
+    FLLM_REQUIRE(aligned16(x) && aligned16(w_qkv) && aligned16(norm_w), "norm_qkv_rope_store: operands must be 16-byte aligned");
+    FLLM_REQUIRE(head_dim % 4 == 0 && rope_dims % 2 == 0 && rope_dims <= head_dim && rope_dims >= 0,
+                 "norm_qkv_rope_store: head_dim %d must be a multiple of 4 and rope_dims %d even and no larger", head_dim, rope_dims);
+    FLLM_REQUIRE(heads > 0 && kv_heads > 0 && page_size > 0 && table_stride > 0 && eps > 0.f, "norm_qkv_rope_store: bad sizes");
+    FLLM_REQUIRE(!store_kv || (k_pages && v_pages), "norm_qkv_rope_store: pages missing");
+    SkinnyArgs a = qkv_args(x, eps, w_qkv, bias, q_out, row_pos, row_seg, tables, table_stride, cos_table, sin_table, rope_dims,
+                            k_pages, v_pages, M, heads, kv_heads, head_dim, K, page_size, store_kv);
+    a.norm_w = norm_w;
     const int rc = dispatch<PRO_NORM_F32, EPI_QKV>(a, stream);
     FLLM_REQUIRE(rc != 1, "norm_qkv_rope_store: shape M=%d K=%d does not fit the staging area", M, K);
+    return rc;
+}
+
+// ---------------------------------------------------------------------------------------------
+// A norm prepared by the product before it (up to 16 rows)
+// ---------------------------------------------------------------------------------------------
+// out += x w^T as fllm_linear does with a float32 `out`, and for the RMSNorm that reads `out` next: next_x = out *
+// next_w as bfloat16 [M, N], and next_ssq [M, *tiles_out] the sums of squares of out over the outputs of each tile
+// (room for M * N / 8 floats).  *tiles_out (host memory) says how many parts a row has.
+extern "C" int fllm_linear_add_normed(const void *x, int ldx, const void *w, const float *bias, float *out, int M, int N, int K,
+                                      const float *next_w, void *next_x, float *next_ssq, int *tiles_out, hipStream_t stream) {
+    FLLM_REQUIRE(M >= 1 && M <= 16 && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && N >= 16 && N % 16 == 0,
+                 "linear_add_normed: takes 1..16 rows, K and ldx in steps of 8 and N in steps of 16 (M=%d N=%d K=%d ldx=%d)", M, N, K, ldx);
+    FLLM_REQUIRE(aligned16(x) && aligned16(w) && aligned16(out) && aligned16(next_w) && next_x != nullptr && next_ssq != nullptr &&
+                     ((uintptr_t)next_x & 7) == 0 && tiles_out != nullptr,
+                 "linear_add_normed: operands must be there and 16-byte aligned");
+    SkinnyArgs a = {};
+    a.x = x;
+    a.ldx = ldx;
+    a.w = (const bf16_t *)w;
+    a.bias = bias;
+    a.out = out;
+    a.ldo = N;
+    a.M = M;
+    a.N = N;
+    a.K = K;
+    a.next_w = next_w;
+    a.next_x = (bf16_t *)next_x;
+    a.next_ssq = next_ssq;
+    a.next_tiles_out = tiles_out;
+    const int rc = launch_resident<PRO_BF16, EPI_ADD>(a, stream);
+    FLLM_REQUIRE(rc != 1, "linear_add_normed: shape M=%d K=%d does not fit the staging area", M, K);
+    return rc;
+}
+
+// The forms with a norm prologue, from what fllm_linear_add_normed left: xn [M, K] bfloat16, ssq [M, ssq_count].
+extern "C" int fllm_scaled_gate_up_swiglu(const void *xn, const float *ssq, int ssq_count, float eps, const void *w_gate_up,
+                                          const float *bias, void *out, int M, int inter, int K, hipStream_t stream) {
+    FLLM_REQUIRE(M >= 1 && M <= 16 && K % 8 == 0 && K >= 8 && inter > 0 && ssq_count > 0 && eps > 0.f,
+                 "scaled_gate_up_swiglu: takes 1..16 rows and K a multiple of 8 (M=%d K=%d parts=%d)", M, K, ssq_count);
+    FLLM_REQUIRE(aligned16(xn) && aligned16(w_gate_up) && ssq != nullptr, "scaled_gate_up_swiglu: operands must be 16-byte aligned");
+    SkinnyArgs a = {};
+    a.x = xn;
+    a.ldx = K;
+    a.eps = eps;
+    a.ssq_in = ssq;
+    a.ssq_count = ssq_count;
+    a.w = (const bf16_t *)w_gate_up;
+    a.bias = bias;
+    a.out = out;
+    a.ldo = inter;
+    a.M = M;
+    a.N = 2 * inter;
+    a.K = K;
+    const int rc = launch_resident<PRO_SCALED, EPI_SWIGLU>(a, stream);
+    FLLM_REQUIRE(rc != 1, "scaled_gate_up_swiglu: shape M=%d K=%d does not fit the staging area", M, K);
+    return rc;
+}
+
+extern "C" int fllm_scaled_qkv_rope_store(const void *xn, const float *ssq, int ssq_count, float eps, const void *w_qkv,
+                                          const float *bias, void *q_out, const int32_t *row_pos, const int32_t *row_seg,
+                                          const int32_t *tables, int table_stride, const float *cos_table, const float *sin_table,
+                                          int rope_dims, void *k_pages, void *v_pages, int M, int heads, int kv_heads, int head_dim,
+                                          int K, int page_size, int store_kv, hipStream_t stream) {
+    FLLM_REQUIRE(M >= 1 && M <= 16 && K % 8 == 0 && K >= 8 && ssq_count > 0,
+                 "scaled_qkv_rope_store: takes 1..16 rows and K a multiple of 8 (M=%d K=%d parts=%d)", M, K, ssq_count);
+    FLLM_REQUIRE(aligned16(xn) && aligned16(w_qkv) && ssq != nullptr, "scaled_qkv_rope_store: operands must be 16-byte aligned");
+    FLLM_REQUIRE(head_dim % 4 == 0 && rope_dims % 2 == 0 && rope_dims <= head_dim && rope_dims >= 0,
+                 "scaled_qkv_rope_store: head_dim %d must be a multiple of 4 and rope_dims %d even and no larger", head_dim, rope_dims);
+    FLLM_REQUIRE(heads > 0 && kv_heads > 0 && page_size > 0 && table_stride > 0 && eps > 0.f, "scaled_qkv_rope_store: bad sizes");
+    FLLM_REQUIRE(!store_kv || (k_pages && v_pages), "scaled_qkv_rope_store: pages missing");
+    SkinnyArgs a = qkv_args(xn, eps, w_qkv, bias, q_out, row_pos, row_seg, tables, table_stride, cos_table, sin_table, rope_dims,
+                            k_pages, v_pages, M, heads, kv_heads, head_dim, K, page_size, store_kv);
+    a.ssq_in = ssq;
+    a.ssq_count = ssq_count;
+    const int rc = launch_resident<PRO_SCALED, EPI_QKV>(a, stream);
+    FLLM_REQUIRE(rc != 1, "scaled_qkv_rope_store: shape M=%d K=%d does not fit the staging area", M, K);
     return rc;
 }

@@ -43,6 +43,12 @@ class StepContext:
     uniform_rows: bool = False              # every segment has exactly one row
     single_from: Optional[int] = None       # the segments from this one on have one row each (None: unknown)
     single_max_context: int = 0             # largest position + 1 among those single rows
+    # A sum into the residual stream may prepare the norm that reads the stream next (`parts/base.py`, "a norm
+    # prepared ahead"): whoever arranges the parts names that norm in `then_norm` before a part runs and in
+    # `next_norm` for the part that ends a block; `prepared` is what the part left: (norm, residual stream, payload).
+    then_norm: object = None
+    next_norm: object = None
+    prepared: object = None
     _scratch: Dict = field(default_factory=dict)
 
     def no_rotation(self, rt):

@@ -135,11 +135,15 @@ class Model:
         x = self.embedding.forward(ctx, ctx.ids)
         pending = None      # a block's output that the next block adds together with its first norm
         check = self.layer_check if self.layer_check is not None and self.layer_check.active else None
-        for index, (entry, binding) in enumerate(zip(self.spec.run_order, self.bindings)):
+        order = self.spec.run_order
+        for index, (entry, binding) in enumerate(zip(order, self.bindings)):
             block = self.blocks[entry.layer]
             if check is not None:
                 check.run_block(self, block, ctx, x, binding, index, entry.layer)
                 continue
+            # the norm that reads the residual stream after this block: the first one of the block that runs next,
+            # where that block says which it is (a block may let its last sum prepare it)
+            ctx.next_norm = getattr(self.blocks[order[index + 1].layer], "mixer_norm", None) if index + 1 < len(order) else None
             if getattr(block, "takes_pending", False):
                 pending = block.forward(ctx, x, binding, pending)
             else:
@@ -147,6 +151,7 @@ class Model:
                     self.rt.ops.add_residual(x, pending)
                 pending = None
                 block.forward(ctx, x, binding)
+        ctx.next_norm = ctx.prepared = None
         if pending is not None:
             self.rt.ops.add_residual(x, pending)
         if check is not None:

@@ -7,7 +7,7 @@ library cannot be loaded or built, constructing `Ops` raises.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional, Sequence
+from typing import NamedTuple, Optional, Sequence
 
 import torch
 
@@ -27,6 +27,14 @@ class SampleRow(ctypes.Structure):
                 ("min_p", ctypes.c_float), ("seed", ctypes.c_uint64), ("draw", ctypes.c_uint64)]
 
 
+class PreparedNorm(NamedTuple):
+    """What `Ops.linear_add_prepare` leaves for the RMSNorm that reads the residual stream next: the rows times the
+    norm's weight in bfloat16, and every row's sum of squares in `parts` parts a row."""
+    x: torch.Tensor
+    ssq: torch.Tensor
+    parts: int
+
+
 class AdjustLists(ctypes.Structure):
     """FllmAdjustLists: device addresses of the lists that the row records of `adjust_logits` point into."""
     _fields_ = [(name, ctypes.c_void_p) for name in ("seen_ids", "seen_counts", "bias_ids", "bias_values", "blocked_ids",
@@ -40,7 +48,7 @@ assert SAMPLE_ROW_BYTES == 32
 _lib = None
 
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 
 def load_library(build_if_missing: bool = True):
@@ -82,6 +90,10 @@ def load_library(build_if_missing: bool = True):
                                      c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_argmax": [c_void, c_void, c_int, c_int, c_void],
         "fllm_gate_up_swiglu": [c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
+        "fllm_linear_add_normed": [c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_void, c_void, c_void, c_void, c_void],
+        "fllm_scaled_gate_up_swiglu": [c_void, c_void, c_int, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
+        "fllm_scaled_qkv_rope_store": [c_void, c_void, c_int, c_float, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void,
+                                       c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_carry_ids": [c_void, c_void, c_void, c_int, c_int, c_void],
         "fllm_sample": [c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_adjust_logits": [c_void, c_int, c_int, c_void, c_void, c_void, c_void],
@@ -291,10 +303,58 @@ class Ops:
                                               self._stream()))
         return out
 
-    def norm_gate_up_swiglu(self, x, norm_weight, eps, w_gate_up, out, bias=None):
-        """out = silu(rmsnorm(x) @ gate.T) * (rmsnorm(x) @ up.T); w_gate_up = [gate; up], out bfloat16 [M, I]."""
+    PREPARED_NORM_ROWS = 16
+
+    def prepares_norm(self, rows: int, width: int) -> bool:
+        """Whether `linear_add_prepare` serves a sum into a residual stream of this size: the fused forms are in use,
+        up to 16 rows, widths in steps of 16."""
+        return rows <= self.PREPARED_NORM_ROWS and width % 16 == 0 and self.fused_decode_supported(rows, width)
+
+    def linear_add_prepare(self, x, w, residual, next_norm_weight, bias=None) -> PreparedNorm:
+        """residual += x @ w.T (+ bias) as `linear(..., accumulate=True)` does, and in the same kernel what the RMSNorm
+        with weight `next_norm_weight` that reads `residual` next would compute first (fllm_linear_add_normed): hand the
+        result to `norm_gate_up_swiglu` / `norm_qkv_rope_store` as `prepared`.  x bfloat16 [M <= 16, K], w bfloat16 [N, K],
+        residual float32 [M, N], N a multiple of 16."""
+        M, K = x.shape
+        N = w.shape[0]
+        _need(x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1, "x must be bfloat16 rows on the GPU")
+        _dense(w, "w", torch.bfloat16, (N, K))
+        _dense(residual, "residual", torch.float32, (M, N))
+        _dense(next_norm_weight, "next_norm_weight", torch.float32, (N,))
+        if bias is not None:
+            _dense(bias, "bias", torch.float32, (N,))
+        _need(1 <= M <= self.PREPARED_NORM_ROWS and N % 16 == 0 and K % 8 == 0,
+              f"linear_add_prepare takes 1..16 rows, N in steps of 16 and K in steps of 8, not {M} x {N} x {K}")
+        xn = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+        ssq = torch.empty((M * (N // 8),), dtype=torch.float32, device=x.device)
+        parts = ctypes.c_int(0)
+        self._check(self.lib.fllm_linear_add_normed(_ptr(x), x.stride(0) if M > 1 else K, _ptr(w), _ptr(bias), _ptr(residual), M, N,
+                                                    K, _ptr(next_norm_weight), _ptr(xn), _ptr(ssq), ctypes.addressof(parts),
+                                                    self._stream()))
+        return PreparedNorm(xn, ssq, int(parts.value))
+
+    def _prepared_operands(self, prepared: PreparedNorm, w, bias, n_rows_w):
+        M, K = prepared.x.shape
+        _dense(prepared.x, "prepared.x", torch.bfloat16)
+        _dense(prepared.ssq, "prepared.ssq", torch.float32)
+        _need(prepared.parts >= 1 and prepared.ssq.numel() >= M * prepared.parts, "prepared.ssq is shorter than rows x parts")
+        _dense(w, "w", torch.bfloat16, (n_rows_w, K))
+        if bias is not None:
+            _dense(bias, "bias", torch.float32, (n_rows_w,))
+        _need(1 <= M <= self.PREPARED_NORM_ROWS and K % 8 == 0, f"a prepared norm serves 1..16 rows and widths in steps of 8, not {M} x {K}")
+        return M, K
+
+    def norm_gate_up_swiglu(self, x, norm_weight, eps, w_gate_up, out, bias=None, prepared: Optional[PreparedNorm] = None):
+        """out = silu(rmsnorm(x) @ gate.T) * (rmsnorm(x) @ up.T); w_gate_up = [gate; up], out bfloat16 [M, I].
+        `prepared`: what `linear_add_prepare` left for this norm, in place of x and norm_weight."""
         two_i = w_gate_up.shape[0]
         _need(two_i % 2 == 0, "w_gate_up needs an even number of rows")
+        if prepared is not None:
+            M, K = self._prepared_operands(prepared, w_gate_up, bias, two_i)
+            _dense(out, "out", torch.bfloat16, (M, two_i // 2))
+            self._check(self.lib.fllm_scaled_gate_up_swiglu(_ptr(prepared.x), _ptr(prepared.ssq), prepared.parts, float(eps),
+                                                            _ptr(w_gate_up), _ptr(bias), _ptr(out), M, two_i // 2, K, self._stream()))
+            return out
         M, K = self._fused_operands(x, norm_weight, w_gate_up, bias, two_i)
         _dense(out, "out", torch.bfloat16, (M, two_i // 2))
         self._check(self.lib.fllm_norm_gate_up_swiglu(_ptr(x), _ptr(norm_weight), float(eps), _ptr(w_gate_up), _ptr(bias),
@@ -330,10 +390,14 @@ class Ops:
         return out
 
     def norm_qkv_rope_store(self, x, norm_weight, eps, w_qkv, q_out, row_pos, row_seg, tables, cos, sin, k_pages, v_pages,
-                            heads, kv_heads, head_dim, rope_dims, page_size, bias=None):
+                            heads, kv_heads, head_dim, rope_dims, page_size, bias=None, prepared: Optional[PreparedNorm] = None):
         """q, k, v = rmsnorm(x) @ w_qkv.T; rotary on pairs (2l, 2l+1) of q and k; q to `q_out`
-        (bfloat16 [M, heads * head_dim]), k and v into the pages (None: not stored)."""
-        M, K = self._fused_operands(x, norm_weight, w_qkv, bias, (heads + 2 * kv_heads) * head_dim)
+        (bfloat16 [M, heads * head_dim]), k and v into the pages (None: not stored).
+        `prepared`: what `linear_add_prepare` left for this norm, in place of x and norm_weight."""
+        if prepared is not None:
+            M, K = self._prepared_operands(prepared, w_qkv, bias, (heads + 2 * kv_heads) * head_dim)
+        else:
+            M, K = self._fused_operands(x, norm_weight, w_qkv, bias, (heads + 2 * kv_heads) * head_dim)
         _dense(q_out, "q_out", torch.bfloat16, (M, heads * head_dim))
         _dense(row_pos, "row_pos", torch.int32, (M,))
         _dense(row_seg, "row_seg", torch.int32, (M,))
@@ -347,6 +411,12 @@ class Ops:
             pages = k_pages.shape[0]
             _dense(k_pages, "k_pages", torch.bfloat16, (pages, kv_heads, page_size, head_dim))
             _dense(v_pages, "v_pages", torch.bfloat16, (pages, kv_heads, head_dim, page_size))
+        if prepared is not None:
+            self._check(self.lib.fllm_scaled_qkv_rope_store(
+                _ptr(prepared.x), _ptr(prepared.ssq), prepared.parts, float(eps), _ptr(w_qkv), _ptr(bias), _ptr(q_out), _ptr(row_pos),
+                _ptr(row_seg), _ptr(tables), tables.shape[1], _ptr(cos), _ptr(sin), rope_dims, _ptr(k_pages), _ptr(v_pages), M, heads,
+                kv_heads, head_dim, K, page_size, 1 if store else 0, self._stream()))
+            return q_out
         self._check(self.lib.fllm_norm_qkv_rope_store(
             _ptr(x), _ptr(norm_weight), float(eps), _ptr(w_qkv), _ptr(bias), _ptr(q_out), _ptr(row_pos), _ptr(row_seg),
             _ptr(tables), tables.shape[1], _ptr(cos), _ptr(sin), rope_dims, _ptr(k_pages), _ptr(v_pages), M, heads, kv_heads,

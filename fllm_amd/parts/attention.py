@@ -13,7 +13,7 @@ import torch
 
 from ..config.spec import PartSpec
 from ..registry import part_class, register_part
-from .base import INIT_BIAS, INIT_MATRIX, KVNeed, Mixer
+from .base import INIT_BIAS, INIT_MATRIX, KVNeed, Mixer, add_and_prepare, take_prepared
 
 
 class PagedAttention(Mixer):
@@ -119,10 +119,11 @@ class PagedAttention(Mixer):
         else:
             cos, sin, dims, _ = ctx.no_rotation(rt)
         q = rt.empty((rows, nh * d))
+        prepared = take_prepared(ctx, norm, residual)      # the sum before this norm may have computed its first steps
         ops.norm_qkv_rope_store(residual, norm_scale, norm_eps, self.w_qkv, q, ctx.row_pos, ctx.row_seg,
                                 ctx.tables[binding.group], cos, sin, binding.k_pages if binding.writes else None,
                                 binding.v_pages if binding.writes else None, nh, nkv, d, dims, binding.page_size,
-                                bias=self.b_qkv)
+                                bias=self.b_qkv, **({"prepared": prepared} if prepared is not None else {}))
         self._attend_and_project(ctx, q, residual, binding)
         return True
 
@@ -163,7 +164,7 @@ class PagedAttention(Mixer):
                           workspace=ctx.attention_workspace(rt, rows, nh, nkv, d))
         if branch is not None:
             ops.linear(out, self.w_o, branch, bias=self.b_o)
-        else:
+        elif not add_and_prepare(ctx, ops, out, self.w_o, residual, self.b_o):
             ops.linear(out, self.w_o, residual, bias=self.b_o, accumulate=True)
 
 

@@ -31,6 +31,13 @@ Roles and their interfaces:
                 with `takes_pending = True` is called as forward(ctx, residual, binding, pending): `pending`
                 is a branch [R,H] that the block before left for it to add (or None), and it returns its
                 own such branch or None.
+                A norm prepared ahead (optional, for blocks and parts that want it): before a block runs a part whose
+                sum into `residual` is read next by a norm it knows, it names that norm in `ctx.then_norm` (for the
+                part that ends the block: `ctx.next_norm`, which whoever runs the blocks sets to the first norm of the
+                block after).  A part whose last kernel can compute that norm's first steps on the way out does so and
+                leaves `ctx.prepared = (norm, residual, payload)` (`leave_prepared`); the part that applies `norm` to
+                that very `residual` next asks `take_prepared(ctx, norm, residual)` and gets the payload or None.  A
+                block clears what its parts did not take, so nothing outlives the sum it was made from.
   embedding     forward(ctx, ids[R]) -> residual_f32[R,H].
   head          forward(ctx, h[L,H]) -> logits_f32[L,V].
 
@@ -115,3 +122,31 @@ class Norm(Part):
 
 class Block(Part):
     role = "block"
+
+
+def take_prepared(ctx, norm, residual):
+    """What the part before left for `norm` applied to `residual`, or None; whatever was left is gone afterwards."""
+    left = getattr(ctx, "prepared", None)
+    if left is None:
+        return None
+    ctx.prepared = None
+    return left[2] if left[0] is norm and left[1] is residual else None
+
+
+def leave_prepared(ctx, norm, residual, payload) -> None:
+    ctx.prepared = (norm, residual, payload)
+
+
+def add_and_prepare(ctx, ops, x, w, residual, bias) -> bool:
+    """residual += x @ w.T (+ bias) in the kernel that also prepares `ctx.then_norm`, where the kernel library has one
+    for this size and that norm says what it multiplies by (`fused_prologue`); the result is left for the norm's
+    reader.  False: nothing was done, the caller adds as usual."""
+    norm = getattr(ctx, "then_norm", None)
+    prepare = getattr(ops, "linear_add_prepare", None)
+    prologue = getattr(norm, "fused_prologue", lambda: None)() if norm is not None else None
+    if prepare is None or prologue is None or residual is None or not ops.prepares_norm(residual.shape[0], residual.shape[1]):
+        return False
+    if x.dtype != torch.bfloat16 or x.stride(0) % 8 != 0 or x.shape[1] % 8 != 0:
+        return False
+    leave_prepared(ctx, norm, residual, prepare(x, w, residual, prologue[0], bias=bias))
+    return True

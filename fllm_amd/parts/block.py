@@ -21,6 +21,20 @@ class PreNormBlock(Block):
         to be added; the return value is this block's own such output, or None when everything has
         been added.  Where a sum can ride on the norm that follows it, it costs no pass of its own."""
         ops = self.rt.ops
+        # a norm prepared ahead: what the block before left for this block's first norm, and the norms that this
+        # block's own sums are read by (the feed-forward's; the first norm of the block after)
+        incoming, ctx.prepared = getattr(ctx, "prepared", None), None
+        after = getattr(ctx, "next_norm", None)
+        try:
+            return self._forward(ctx, residual, binding, pending, incoming, after)
+        finally:
+            ctx.then_norm = None
+            left = getattr(ctx, "prepared", None)
+            if left is not None and (after is None or left[0] is not after):
+                ctx.prepared = None          # nothing outlives the sum it was made from
+
+    def _forward(self, ctx, residual, binding, pending, incoming, after):
+        ops = self.rt.ops
         add_mixer_norm = getattr(self.mixer_norm, "add_forward", None)
         add_ff_norm = getattr(self.feed_forward_norm, "add_forward", None) if self.feed_forward is not None else None
         # a part may take the residual stream and the norm before it in one fused kernel
@@ -31,7 +45,13 @@ class PreNormBlock(Block):
                 pending = None
             else:
                 fused = None     # the fused kernels read the finished residual stream: the sum rides on the norm instead
-        if fused is None or not fused(ctx, residual, self.mixer_norm, binding):
+        if fused is not None and pending is None:
+            ctx.prepared = incoming
+        ctx.then_norm = self.feed_forward_norm if self.feed_forward is not None else after
+        taken = fused is not None and fused(ctx, residual, self.mixer_norm, binding)
+        ctx.then_norm = None
+        if not taken:
+            ctx.prepared = None
             if pending is not None:
                 h = add_mixer_norm(ctx, residual, pending)
             else:
@@ -49,8 +69,15 @@ class PreNormBlock(Block):
             self.mixer.forward(ctx, h, residual, binding)
         if self.feed_forward is None:
             return None                  # a layer of a mixer alone
+        left = getattr(ctx, "prepared", None)
+        if left is not None and left[0] is not self.feed_forward_norm:
+            ctx.prepared = None
         fused = getattr(self.feed_forward, "forward_from_residual", None)
-        if fused is None or not fused(ctx, residual, self.feed_forward_norm):
+        ctx.then_norm = after
+        taken = fused is not None and fused(ctx, residual, self.feed_forward_norm)
+        ctx.then_norm = None
+        if not taken:
+            ctx.prepared = None
             h = self.feed_forward_norm.forward(ctx, residual)
             self.feed_forward.forward(ctx, h, residual)
         return None

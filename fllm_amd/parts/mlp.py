@@ -6,7 +6,7 @@ from __future__ import annotations
 import torch
 
 from ..registry import register_part
-from .base import INIT_BIAS, INIT_MATRIX, FeedForward
+from .base import INIT_BIAS, INIT_MATRIX, FeedForward, add_and_prepare, take_prepared
 
 
 class GatedMLP(FeedForward):
@@ -45,8 +45,11 @@ class GatedMLP(FeedForward):
             return False
         norm_scale, norm_eps = prologue
         act = rt.empty((rows, self.inter))
-        ops.norm_gate_up_swiglu(residual, norm_scale, norm_eps, self.w_gate_up, act, bias=self.b_gate_up)
-        ops.linear(act, self.w_down, residual, bias=self.b_down, accumulate=True)
+        prepared = take_prepared(ctx, norm, residual)      # the sum before this norm may have computed its first steps
+        ops.norm_gate_up_swiglu(residual, norm_scale, norm_eps, self.w_gate_up, act, bias=self.b_gate_up,
+                                **({"prepared": prepared} if prepared is not None else {}))
+        if not add_and_prepare(ctx, ops, act, self.w_down, residual, self.b_down):
+            ops.linear(act, self.w_down, residual, bias=self.b_down, accumulate=True)
         return True
 
     def forward_branch(self, ctx, h):

@@ -340,6 +340,65 @@ def test_norm_qkv_rope_store(ops, ref, heads, kv_heads, head_dim, rope_dims, pag
     assert torch.equal(q2[live.to(DEV)], q_gpu[live.to(DEV)])
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 4096, 14336), (8, 4096, 4096), (16, 2048, 8192), (5, 160, 432), (13, 64, 176),
+                                   (3, 8192, 28672), (8, 320, 40000), (2, 48, 96)])
+def test_a_product_prepares_the_norm_that_reads_its_sums(ops, ref, M, N, K):
+    """`linear_add_prepare` adds to the residual stream exactly as `linear` does and leaves, for the norm that comes
+    next, the rows times the norm's weight in bfloat16 (bit for bit what the norm forms compute themselves) and the rows'
+    sums of squares in parts; the gate/up and q/k/v forms fed with that pair give what they give from the float32 rows,
+    up to the order in which the squares are added.  Rows of different scale, a width per tile size, K beyond what
+    LDS holds (K slices over workgroups), several calls in a row."""
+    g = gen(70 + M)
+    x = (torch.randn(M, K, generator=g) * 0.5).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g) * 0.1
+    resid = torch.randn(M, N, generator=g) * torch.rand(M, 1, generator=g) * 6
+    nw = 1 + 0.1 * torch.randn(N, generator=g)
+    plain = ops.linear(x.to(DEV), w.to(DEV), resid.clone().to(DEV), bias=b.to(DEV), accumulate=True)
+    for _ in range(2):
+        summed = resid.clone().to(DEV)
+        prepared = ops.linear_add_prepare(x.to(DEV), w.to(DEV), summed, nw.to(DEV), bias=b.to(DEV))
+        assert torch.equal(summed, plain)
+        assert torch.equal(prepared.x, (summed * nw.to(DEV)).to(torch.bfloat16))
+        assert prepared.parts in (N // 16, N // 8)
+        squares = prepared.ssq[:M * prepared.parts].view(M, prepared.parts).double().sum(1)
+        want = summed.double().pow(2).sum(1)
+        assert float(((squares - want).abs() / want).max()) < 1e-6
+    # the products behind that norm
+    inter = 3 * N // 2 + 8
+    wgu = (torch.randn(2 * inter, N, generator=g) / math.sqrt(N)).to(torch.bfloat16).to(DEV)
+    bgu = (torch.randn(2 * inter, generator=g) * 0.1).to(DEV)
+    own = ops.norm_gate_up_swiglu(summed, nw.to(DEV), 1e-5, wgu, torch.empty(M, inter, dtype=torch.bfloat16, device=DEV), bias=bgu)
+    fed = ops.norm_gate_up_swiglu(None, None, 1e-5, wgu, torch.empty(M, inter, dtype=torch.bfloat16, device=DEV), bias=bgu, prepared=prepared)
+    want = ref.norm_gate_up_swiglu(summed.cpu(), nw, 1e-5, wgu.cpu(), torch.empty(M, inter, dtype=torch.float64), bias=bgu.cpu())
+    close(fed, want, 2 * BF16_EPS, 4e-2, f"gate/up behind a prepared norm M{M} N{N}")
+    assert float((fed.float() - own.float()).abs().max()) <= 2 * BF16_EPS * float(own.float().abs().max())
+    if N % 64 == 0:
+        heads, kv_heads, head_dim, page_size = N // 64, 1, 16, 16
+        qkv_rows = (heads + 2) * head_dim
+        wq = (torch.randn(qkv_rows, N, generator=g) / math.sqrt(N)).to(torch.bfloat16).to(DEV)
+        tables = scattered_tables(g, M, 8, M * 8 + 2).to(DEV)
+        row_pos = torch.tensor([(7 * r + 3) % 128 for r in range(M)], dtype=torch.int32, device=DEV)
+        row_seg = torch.arange(M, dtype=torch.int32, device=DEV)
+        angle = torch.rand(128, head_dim // 2, generator=g, dtype=torch.float64) * 6.28
+        cos, sin = torch.cos(angle).float().to(DEV), torch.sin(angle).float().to(DEV)
+        k0, v0 = make_pages(g, M * 8 + 2, kv_heads, page_size, head_dim, torch.bfloat16)
+        results = []
+        for kwargs in ({}, {"prepared": prepared}):
+            kp, vp = k0.to(DEV), v0.to(DEV)
+            q = ops.norm_qkv_rope_store(summed, nw.to(DEV), 1e-5, wq, torch.zeros(M, heads * head_dim, dtype=torch.bfloat16, device=DEV),
+                                        row_pos, row_seg, tables, cos, sin, kp, vp, heads, kv_heads, head_dim, head_dim, page_size, **kwargs)
+            results.append((q, kp, vp))
+        for got, base in zip(results[1], results[0]):
+            assert float((got.float() - base.float()).abs().max()) <= 2 * BF16_EPS * float(base.float().abs().max())
+    with pytest.raises(Exception, match="1..16 rows"):
+        ops.linear_add_prepare(torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV),
+                               torch.zeros(17, 32, device=DEV), torch.ones(32, device=DEV))
+    with pytest.raises(Exception, match="steps of 16"):
+        ops.linear_add_prepare(torch.zeros(2, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(24, 64, dtype=torch.bfloat16, device=DEV),
+                               torch.zeros(2, 24, device=DEV), torch.ones(24, device=DEV))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("rows,inter", [(1, 176), (13, 432), (3, 14336)])
 def test_swiglu(ops, ref, dtype, rows, inter):
