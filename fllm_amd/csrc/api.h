@@ -192,8 +192,9 @@ int fllm_adjust_logits(float *logits, int rows, int vocab, const struct FllmAdju
 int fllm_logprobs(const float *logits, int rows, int vocab, const int32_t *wanted_rows, int wanted, const int32_t *tokens,
                   int top, float *values, int32_t *ids, hipStream_t stream);
 
-// work: float32 [rows, vocab] scratch.  kinds: 1 every row has a temperature and neither top-k nor top-p (the draw
-// looks at every token: several workgroups share a row), 2 no row is of that kind, 3 some may be.
+// work: float32 [rows, vocab] scratch.  kinds: what the caller knows of the rows, a sum of 1 (some have a temperature
+// and no filter: their draw looks at every token, and several workgroups share such a row), 2 (some are of another
+// kind) and 4 (some of those have a top-k of at most 64: several workgroups share such a row as well).
 int fllm_sample(const float *logits, float *work, const struct FllmSampleRow *params, int32_t *out, int rows, int vocab,
                 int kinds, hipStream_t stream);
 

@@ -229,38 +229,46 @@ __device__ __forceinline__ int block_exclusive_scan(int v, Cells &cells, int *to
     return before + inc - v;
 }
 
-// The lowest bin b with sum(hist[0..b]) >= target, kBins when the whole histogram falls short; done by the first
-// wave, every lane over 64 bins; the same value in every thread.
+// The lowest bin b with sum(hist[0..b]) >= target, kBins when the whole histogram falls short (or target is 0); the
+// same value in every thread.  Every thread of the workgroup adds up kBins / kBlock neighbouring bins, the sums
+// before each thread come from a scan across the lanes and the waves (integers: any order of adding), and the one
+// thread in whose bins the running sum crosses the target says where.  `before`: the sum of the bins before that one.
 __device__ int find_bin(const unsigned long long *hist, unsigned long long target, Cells &cells,
                         unsigned long long *before = nullptr) {
+    constexpr int PER = kBins / kBlock;
+    static_assert(PER * kBlock == kBins, "every thread has the same number of bins");
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     __syncthreads();
-    if (threadIdx.x < kWave) {
-        const int lane = threadIdx.x;
-        constexpr int PER = kBins / kWave;
-        unsigned long long own = 0;
-        for (int i = 0; i < PER; i++) own += hist[lane * PER + i];
-        unsigned long long below = 0;      // sum of the lanes before this one
-        for (int o = 1; o < kWave; o++) {
-            const unsigned long long other = __shfl(own, (lane - o) & (kWave - 1), kWave);
-            if (lane - o >= 0) below += other;
-        }
-        int found = kBins;
-        if (lane == 0) cells.before = 0;
-        if (below < target && below + own >= target) {      // the crossing lies in this lane's bins: one lane, if any
-            unsigned long long cum = below;
-            for (int i = 0; i < PER; i++) {
-                const unsigned long long here = hist[lane * PER + i];
-                if (cum + here >= target) {
-                    found = lane * PER + i;
-                    cells.before = cum;                      // the sum of the bins before the one found
-                    break;
-                }
-                cum += here;
-            }
-        }
+    unsigned long long own[PER], sum = 0;
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) found = min(found, __shfl_xor(found, o, kWave));
-        if (lane == 0) cells.word = found;
+    for (int i = 0; i < PER; i++) {
+        own[i] = hist[threadIdx.x * PER + i];
+        sum += own[i];
+    }
+    unsigned long long upto = sum;         // this thread's bins and those of the lanes before it
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        const unsigned long long other = __shfl_up(upto, o, kWave);
+        if (lane >= o) upto += other;
+    }
+    if (lane == kWave - 1) cells.units[wave] = upto;
+    if (threadIdx.x == 0) cells.word = kBins, cells.before = 0;
+    __syncthreads();
+    unsigned long long below = upto - sum;
+#pragma unroll
+    for (int w = 0; w < kWaves; w++)
+        if (w < wave) below += cells.units[w];
+    if (below < target && below + sum >= target) {       // one thread, if any
+        unsigned long long cum = below;
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            if (cum + own[i] >= target) {
+                cells.word = threadIdx.x * PER + i;
+                cells.before = cum;
+                break;
+            }
+            cum += own[i];
+        }
     }
     __syncthreads();
     const int bin = cells.word;
@@ -405,6 +413,74 @@ __device__ uint32_t thresholds(KeyAt key_at, WeightAt weight_at, int n, int top_
     return t;
 }
 
+// The same thresholds for a short list, by one wave (all 64 lanes must call): up to 4 * kWave candidates.  Instead of
+// building each threshold bit by bit, with a sum across the lanes a bit, every lane ranks the candidates it holds
+// (lane, lane + 64, ...) against all others: how many keys are no smaller than its own, and how much they weigh,
+// added in index order.  The k-th largest key is the largest one that at least k keys are no smaller than; the top-p
+// threshold the largest one from which on the weights reach the target.  Two sums across the lanes in all.
+constexpr int kShortList = 4 * kWave;
+__device__ __forceinline__ uint32_t wave_largest_key(uint32_t v) {
+#pragma unroll
+    for (int hop = kWave / 2; hop >= 1; hop /= 2) {
+        const uint32_t other = (uint32_t)__shfl_xor((int)v, hop, kWave);
+        v = other > v ? other : v;
+    }
+    return v;
+}
+template <typename KeyAt, typename WeightAt>
+__device__ uint32_t thresholds_of_short_list(KeyAt key_at, WeightAt weight_at, int n, int top_k, bool use_k, bool use_p, float top_p,
+                                             float min_p, double total) {
+    const int lane = threadIdx.x & (kWave - 1);
+    uint32_t key[4];
+    float weight[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const int i = lane + e * kWave;
+        key[e] = i < n ? key_at(i) : 0u;
+        weight[e] = i < n ? weight_at(i) : 0.f;
+    }
+    uint32_t t = 0;
+    if (use_k) {
+        const int k = min(top_k, n);
+        int no_smaller[4] = {0, 0, 0, 0};
+        for (int j = 0; j < n; j++) {
+            const uint32_t other = key_at(j);
+#pragma unroll
+            for (int e = 0; e < 4; e++) no_smaller[e] += other >= key[e] ? 1 : 0;
+        }
+        uint32_t mine = 0;
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            if (lane + e * kWave < n && no_smaller[e] >= k && key[e] > mine) mine = key[e];
+        t = wave_largest_key(mine);
+    }
+    if (use_p) {
+        // min-p: a candidate that weighs less than min_p counts for nothing here (key 0)
+        uint32_t heavy[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) heavy[e] = weight[e] >= min_p ? key[e] : 0u;
+        const uint32_t from = t > 1u ? t : 1u;
+        double from_own[4] = {0.0, 0.0, 0.0, 0.0}, kept = 0.0;
+        for (int j = 0; j < n; j++) {
+            const float w = weight_at(j);
+            const uint32_t other = w >= min_p ? key_at(j) : 0u;
+            if (other >= from) kept += (double)w;
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (other >= heavy[e]) from_own[e] += (double)w;
+        }
+        if (use_k || min_p > 0.f) total = kept;          // top-p looks at what top-k and min-p left
+        const double target = (double)top_p * total;
+        uint32_t mine = 0;
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            if (heavy[e] != 0u && from_own[e] >= target && heavy[e] > mine) mine = heavy[e];
+        const uint32_t reached = wave_largest_key(mine);
+        t = reached > t ? reached : t;
+    }
+    return t;
+}
+
 // Calls f(token, logit) for every token of a row, each thread of the workgroup with a share of its own: four
 // consecutive tokens a load where the row's alignment allows (four such loads in flight), single tokens at both ends.
 // A thread meets its tokens in the same order in every pass.
@@ -479,16 +555,219 @@ draw_from_all_kernel(const float *__restrict__ logits, const FllmSampleRow *__re
         out[row] = token_of(all);
 }
 
+// Rows with a small top-k (the usual setting: top-k 50 with or without top-p and min-p) are shared by several
+// workgroups too.  Whatever else is asked, only the k largest logits and their equals can be chosen, and each of them
+// is among the k largest of its own stretch of the vocabulary: every part hands over those (its tokens down to the
+// bin of its k-th largest, found as the single workgroup finds them, from registers: a thread holds its eight
+// tokens), and one workgroup a row then runs the exact thresholds and the draw over what the parts handed over, at
+// most kParts x kPartCap candidates in LDS.  The parts and the order of their lists depend on the vocabulary alone,
+// not on the rows of the launch.  A part with more candidates than it may hand over (thousands of equal logits), or
+// with fewer than k tokens within reach of its largest, marks the row for `sample_kernel`, which runs behind.
+constexpr int kSmallK = 64;          // the largest top-k that goes this way
+constexpr int kParts = 16;           // parts a row at most
+constexpr int kPartTokens = 8 * kBlock;   // tokens a part at most: eight a thread
+constexpr int kPartCap = 128;        // candidates a part may hand over
+struct PartHead {
+    float largest;
+    int count;                       // -1: the row goes to sample_kernel
+};
+__device__ __forceinline__ bool takes_small_k(const FllmSampleRow &p, int vocab) {
+    return p.temperature > 1e-5f && p.top_k > 0 && p.top_k <= kSmallK && p.top_k < vocab;
+}
+
+__global__ void __launch_bounds__(kBlock)
+small_k_parts_kernel(const float *__restrict__ logits, const FllmSampleRow *__restrict__ params, int vocab, int parts, int per_part,
+                     float *__restrict__ part_v, int *__restrict__ part_i, PartHead *__restrict__ heads) {
+    __shared__ Cells cells;
+    __shared__ unsigned long long bins[kBins];
+    const int row = blockIdx.x, part = blockIdx.y;
+    const FllmSampleRow p = params[row];
+    if (!takes_small_k(p, vocab)) return;
+    const float *src = logits + (size_t)row * vocab;
+    const int lo = part * per_part, hi = min(vocab, lo + per_part);
+    float v[8];
+    float m = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int i = lo + (int)threadIdx.x + j * kBlock;
+        v[j] = i < hi ? usable(src[i]) : -INFINITY;
+        m = fmaxf(m, v[j]);
+    }
+    m = block_largest(m, cells);
+    PartHead *head = heads + (size_t)row * parts + part;
+    if (!(m > -INFINITY)) {                      // nothing finite here
+        if (threadIdx.x == 0) head->largest = m, head->count = 0;
+        return;
+    }
+    for (int i = threadIdx.x; i < kBins; i += kBlock) bins[i] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        if (!(v[j] > -INFINITY)) continue;
+        const int b = bin_of(v[j], m);
+        if (b < kBins) atomicAdd(&bins[b], 1ull);
+    }
+    const int last_bin = find_bin(bins, (unsigned long long)p.top_k, cells);
+    int mine = 0;
+#pragma unroll
+    for (int j = 0; j < 8; j++) mine += (v[j] > -INFINITY && bin_of(v[j], m) <= last_bin) ? 1 : 0;
+    int count;
+    int at = block_exclusive_scan(mine, cells, &count);
+    // (with fewer than k tokens within the histogram's reach of the largest, last_bin is kBins and the list is every
+    // finite token of the part, as in the single workgroup: handed over if that is few, else the row goes there)
+    const bool too_many = count > kPartCap;
+    if (threadIdx.x == 0) head->largest = m, head->count = too_many ? -1 : count;
+    if (too_many) return;
+    float *dst_v = part_v + ((size_t)row * parts + part) * kPartCap;
+    int *dst_i = part_i + ((size_t)row * parts + part) * kPartCap;
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+        if (v[j] > -INFINITY && bin_of(v[j], m) <= last_bin) {
+            dst_v[at] = v[j];
+            dst_i[at] = lo + (int)threadIdx.x + j * kBlock;
+            at++;
+        }
+}
+
+// One workgroup a row.  The parts' candidates together hold the row's k largest logits and their equals, and many
+// more (every part gave its own k largest): a histogram over their distance from the row's largest logit finds the
+// bin of the k-th, as the single workgroup does over the whole row, and what lies beyond it is dropped before the
+// exact thresholds and the draw run over the rest, with the same code.  done[row]: 1 the token is chosen, 0 the
+// row is left to sample_kernel.
+__global__ void __launch_bounds__(kBlock)
+small_k_finish_kernel(const FllmSampleRow *__restrict__ params, int32_t *__restrict__ out, int vocab, int parts,
+                      const float *__restrict__ part_v, const int *__restrict__ part_i, const PartHead *__restrict__ heads,
+                      int *__restrict__ done) {
+    constexpr int kMost = kParts * kPartCap;
+    __shared__ Cells cells;
+    __shared__ unsigned long long bins[kBins];       // the histogram; afterwards the candidates that are kept
+    __shared__ float all_v[kMost];
+    __shared__ int all_i[kMost];
+    __shared__ int starts[kParts + 1];
+    __shared__ int counts[kParts];
+    __shared__ float largest_of[kParts];
+    const int row = blockIdx.x;
+    const FllmSampleRow p = params[row];
+    if (!takes_small_k(p, vocab)) return;
+    if ((int)threadIdx.x < parts) {
+        const PartHead h = heads[(size_t)row * parts + threadIdx.x];
+        counts[threadIdx.x] = h.count;
+        largest_of[threadIdx.x] = h.largest;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int total = 0;
+        bool whole = true;
+        for (int q = 0; q < parts; q++) {
+            starts[q] = total;
+            if (counts[q] < 0) whole = false;
+            else total += counts[q];
+        }
+        starts[parts] = whole ? total : -1;
+    }
+    __syncthreads();
+    const int gathered = starts[parts];
+    if (gathered < 0) {
+        if (threadIdx.x == 0) done[row] = 0;
+        return;
+    }
+    float m = -INFINITY;
+    for (int q = 0; q < parts; q++) m = fmaxf(m, largest_of[q]);
+    if (threadIdx.x == 0) done[row] = 1;
+    if (!(m > -INFINITY)) {
+        if (threadIdx.x == 0) out[row] = 0;   // no finite logit: index 0, as everywhere
+        return;
+    }
+    for (int i = threadIdx.x; i < kBins; i += kBlock) bins[i] = 0;
+    {   // every slot of every part's list has a thread: all loads are asked for before the first is stored
+        constexpr int kSlots = kMost / kBlock;
+        float v[kSlots];
+        int id[kSlots], to[kSlots];
+#pragma unroll
+        for (int j = 0; j < kSlots; j++) {
+            const int slot = (int)threadIdx.x + j * kBlock, q = slot / kPartCap, i = slot - q * kPartCap;
+            to[j] = (q < parts && i < counts[q]) ? starts[q] + i : -1;
+            if (to[j] >= 0) {
+                v[j] = part_v[((size_t)row * parts + q) * kPartCap + i];
+                id[j] = part_i[((size_t)row * parts + q) * kPartCap + i];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kSlots; j++)
+            if (to[j] >= 0) all_v[to[j]] = v[j], all_i[to[j]] = id[j];
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < gathered; i += kBlock) {
+        const int b = bin_of(all_v[i], m);
+        if (b < kBins) atomicAdd(&bins[b], 1ull);
+    }
+    const int last_bin = find_bin(bins, (unsigned long long)p.top_k, cells);
+    // thread t keeps what it holds of candidates t, t + kBlock, ...: an order that depends on the lists alone
+    constexpr int kMine = kMost / kBlock;
+    int mine = 0;
+#pragma unroll
+    for (int j = 0; j < kMine; j++) {
+        const int i = (int)threadIdx.x + j * kBlock;
+        mine += (i < gathered && bin_of(all_v[i], m) <= last_bin) ? 1 : 0;
+    }
+    int count;
+    int at = block_exclusive_scan(mine, cells, &count);
+    float *logit_of = (float *)bins, *weight_of = logit_of + kMost;      // the histogram is done with
+    int *token_at = (int *)(weight_of + kMost);
+    static_assert(3 * kMost * 4 <= kBins * 8, "the kept candidates fit into the histogram's memory");
+    const float inv_t = (float)(1.0 / (double)p.temperature);
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kMine; j++) {
+        const int i = (int)threadIdx.x + j * kBlock;
+        if (i < gathered && bin_of(all_v[i], m) <= last_bin) {
+            const float v = all_v[i];
+            logit_of[at] = v;
+            weight_of[at] = expf((v - m) * inv_t);
+            token_at[at] = all_i[i];
+            at++;
+        }
+    }
+    __syncthreads();
+    const bool use_p = p.top_p > 0.f && p.top_p < 1.f;
+    const bool use_m = p.min_p > 0.f;
+    const float min_p = use_m ? p.min_p : 0.f;
+    if (threadIdx.x < kWave) {
+        auto key_at = [&](int i) { return ordered_key(logit_of[i]); };
+        auto weight_at = [&](int i) { return weight_of[i]; };
+        const uint32_t t = count <= kShortList
+                               ? thresholds_of_short_list(key_at, weight_at, count, p.top_k, true, use_p, p.top_p, min_p, 0.0)
+                               : thresholds<OneWave>(key_at, weight_at, count, p.top_k, true, use_p, p.top_p, min_p, 0.0, cells);
+        if (threadIdx.x == 0) cells.key = t;
+    }
+    __syncthreads();
+    const uint32_t threshold = cells.key;
+    Pick best = {-INFINITY, kNone};
+    for (int i = threadIdx.x; i < count; i += kBlock) {
+        const float v = logit_of[i];
+        if (ordered_key(v) < threshold) continue;
+        if (use_m && weight_of[i] < min_p) continue;
+        const int id = token_at[i];
+        const float u = uniform_of(p.seed, p.draw, (uint32_t)id);
+        const Pick here = {(v - m) * inv_t - logf(-logf(u)), id};
+        best = better_of(best, here);
+    }
+    best = block_best(best, cells);
+    if (threadIdx.x == 0) out[row] = token_of(best);
+}
+
 // `work` gives every row `vocab` 32-bit words of its own (the list of token ids); it must not overlap the logits.
 // `skip_draws_from_all`: rows with a temperature and no filter are left to `draw_from_all_kernel`.
+// `small_k_done`: rows with a small top-k whose entry is 1 have their token already (`small_k_finish_kernel`).
 __global__ void __launch_bounds__(kBlock)
 sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const FllmSampleRow *__restrict__ params,
-              int32_t *__restrict__ out, int vocab, int skip_draws_from_all) {
+              int32_t *__restrict__ out, int vocab, int skip_draws_from_all, const int *__restrict__ small_k_done) {
     __shared__ Cells cells;
     __shared__ unsigned long long bins[kBins];       // the histogram; afterwards the staged candidates
     const int row = blockIdx.x;
     const FllmSampleRow p = params[row];
     if (skip_draws_from_all && draws_from_all(p, vocab)) return;
+    if (small_k_done != nullptr && takes_small_k(p, vocab) && small_k_done[row] != 0) return;
     const float *src = logits + (size_t)row * vocab;
     if (p.temperature <= 1e-5f) {
         const Pick best = block_best(best_in_range(src, 0, vocab), cells);
@@ -569,9 +848,11 @@ sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const 
             }
             __syncthreads();
             if (threadIdx.x < kWave) {
-                const uint32_t t = thresholds<OneWave>([&](int i) { return ordered_key(logit_of[i]); },
-                                                       [&](int i) { return weight_of[i]; }, count, p.top_k, use_k, use_p,
-                                                       p.top_p, min_p, total, cells);
+                auto key_at = [&](int i) { return ordered_key(logit_of[i]); };
+                auto weight_at = [&](int i) { return weight_of[i]; };
+                const uint32_t t = count <= kShortList
+                                       ? thresholds_of_short_list(key_at, weight_at, count, p.top_k, use_k, use_p, p.top_p, min_p, total)
+                                       : thresholds<OneWave>(key_at, weight_at, count, p.top_k, use_k, use_p, p.top_p, min_p, total, cells);
                 if (threadIdx.x == 0) cells.key = t;
             }
             __syncthreads();
@@ -882,7 +1163,9 @@ extern "C" int fllm_sample(const float *logits, float *work, const FllmSampleRow
                            int vocab, int kinds, hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
     FLLM_REQUIRE(work != nullptr && params != nullptr, "sample: work and params are required");
-    FLLM_REQUIRE(kinds >= 1 && kinds <= 3, "sample: kinds %d is none of 1 (rows that draw from all tokens), 2 (other rows), 3 (both)", kinds);
+    FLLM_REQUIRE(kinds >= 1 && kinds <= 7,
+                 "sample: kinds %d is no sum of 1 (rows that draw from all tokens), 2 (other rows), 4 (rows with a top-k of at most 64 among them)",
+                 kinds);
     if (rows == 0) return 0;
     // rows with a temperature and no filter: several workgroups a row, if the device workspace is there to meet in
     void *ws = nullptr;
@@ -890,7 +1173,9 @@ extern "C" int fllm_sample(const float *logits, float *work, const FllmSampleRow
     int parts = (vocab + 8191) / 8192;
     if (parts > 64) parts = 64;
     if (parts * rows > 2048) parts = 2048 / rows;
-    const bool split = (kinds & 1) && parts > 1 && fllm_device_workspace(&ws, &ws_bytes) &&
+    const bool have_ws = fllm_device_workspace(&ws, &ws_bytes);
+    if (!have_ws) ws = nullptr, ws_bytes = 0;
+    const bool split = (kinds & 1) && parts > 1 && have_ws &&
                        (size_t)rows * sizeof(int) <= kWorkspaceCounterBytes &&
                        kWorkspaceCounterBytes + (size_t)rows * parts * 8 + (size_t)rows * 4 <= ws_bytes;
     if (split) {
@@ -902,8 +1187,31 @@ extern "C" int fllm_sample(const float *logits, float *work, const FllmSampleRow
                            per_part, pv, pi, (int *)ws, row_max);
         hipLaunchKernelGGL(draw_from_all_kernel<1>, dim3(rows, parts), dim3(kBlock), 0, stream, logits, params, out, vocab, parts,
                            per_part, pv, pi, (int *)ws, row_max);
-        if (!(kinds & 2)) return fllm_check_launch("sample");
+        if (!(kinds & 6)) return fllm_check_launch("sample");
     }
-    hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(kBlock), 0, stream, logits, work, params, out, vocab, split ? 1 : 0);
+    // rows with a small top-k: the parts of a row in workgroups of their own, then one workgroup a row; what they
+    // leave undone (done[row] 0) and every other row is sample_kernel's.  Behind the partial results of the rows that
+    // draw from all tokens in the workspace: lists, their heads, the rows' marks.
+    const int *small_k_done = nullptr;
+    const int k_parts = (vocab + kPartTokens - 1) / kPartTokens;
+    if ((kinds & 4) && k_parts >= 2 && k_parts <= kParts && ws != nullptr) {
+        const int per_part = (vocab + k_parts - 1) / k_parts;       // <= kPartTokens
+        size_t at = kWorkspaceCounterBytes + (size_t)rows * parts * 8 + (size_t)rows * 4;
+        at = (at + 255) / 256 * 256;
+        const size_t lists = (size_t)rows * k_parts * kPartCap;
+        if (at + lists * 8 + (size_t)rows * k_parts * sizeof(PartHead) + (size_t)rows * 4 <= ws_bytes) {
+            float *part_v = (float *)((unsigned char *)ws + at);
+            int *part_i = (int *)(part_v + lists);
+            PartHead *heads = (PartHead *)(part_i + lists);
+            int *done = (int *)(heads + (size_t)rows * k_parts);
+            hipLaunchKernelGGL(small_k_parts_kernel, dim3(rows, k_parts), dim3(kBlock), 0, stream, logits, params, vocab, k_parts,
+                               per_part, part_v, part_i, heads);
+            hipLaunchKernelGGL(small_k_finish_kernel, dim3(rows), dim3(kBlock), 0, stream, params, out, vocab, k_parts, part_v,
+                               part_i, heads, done);
+            small_k_done = done;
+        }
+    }
+    hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(kBlock), 0, stream, logits, work, params, out, vocab, split ? 1 : 0,
+                       small_k_done);
     return fllm_check_launch("sample");
 }

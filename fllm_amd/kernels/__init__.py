@@ -605,10 +605,11 @@ class Ops:
                                            _ptr(values), _ptr(ids), self._stream()))
 
     def sample(self, logits: torch.Tensor, work: torch.Tensor, params: torch.Tensor, out: torch.Tensor,
-               kinds: int = 3) -> torch.Tensor:
-        """`params`: uint8 GPU tensor [rows, 32] holding `SampleRow` records.  `kinds`: what the caller knows of the rows:
-        1 all of them have a temperature and no top-k or top-p (their draw looks at every token, and several
-        workgroups share a row), 2 none of them is of that kind, 3 (default) some may be."""
+               kinds: int = 7) -> torch.Tensor:
+        """`params`: uint8 GPU tensor [rows, 32] holding `SampleRow` records.  `kinds`: what the caller knows of the rows,
+        a sum of 1 (some have a temperature and no filter: their draw looks at every token, and several workgroups
+        share such a row), 2 (some are of another kind) and 4 (some of those have a top-k of at most 64: several
+        workgroups share such a row as well); 7 when nothing is known."""
         rows, vocab = logits.shape
         _dense(logits, "logits", torch.float32)
         _dense(work, "work", torch.float32, (rows, vocab))

@@ -17,6 +17,7 @@ class SampleRequest:
     draw: int
 
 
+SMALL_TOP_K = 64     # rows with a top-k up to this are shared by several workgroups (the kernel's own limit)
 _RECORD = 32   # bytes of one row record: float temperature, float top_p, int32 top_k, float min_p, uint64 seed, uint64 draw
 
 
@@ -136,5 +137,7 @@ class Sampler:
             vocab = logits.shape[1]
             from_all = [draws_from_all(r.params, vocab) for r in rows]
             kinds = 1 if all(from_all) else (3 if any(from_all) else 2)
+            if any(0 < int(r.params.top_k) <= SMALL_TOP_K and not r.params.greedy for r in rows):
+                kinds |= 4          # rows with a small top-k: several workgroups a row
             self.rt.ops.sample(logits, work, params, out, kinds)
         return out

@@ -810,6 +810,45 @@ def test_sample_rows_that_draw_from_all_tokens_share_workgroups(ops, vocab):
     assert int(counters.to(torch.int64).sum()) == 0
 
 
+@pytest.mark.parametrize("vocab", [20000, 128256, 140000])
+def test_sample_rows_with_a_small_top_k_share_workgroups(ops, vocab):
+    """Rows with a top-k of at most 64 are cut into parts for several workgroups (vocabularies of 8,193 to 131,072
+    tokens); every token is the plain sampler's, with or without the caller's hint, beside rows of other kinds: equal
+    logits at the threshold (all kept), thousands of equal logits (the part hands the row back), a distribution so
+    peaked that fewer than k tokens lie within the histogram's reach, -inf nearly everywhere, min-p and top-p behind
+    top-k, k = 1 and k = 64, and a top-k of 65 that goes the old way."""
+    from fllm_amd.sampling import SampleRequest, SamplingParams, pack_rows
+    g = gen(31)
+    params = [SamplingParams(temperature=0.8, top_k=50, top_p=0.9), SamplingParams(temperature=1.0, top_k=5),
+              SamplingParams(temperature=1.3, top_k=64, min_p=0.05, top_p=0.7), SamplingParams(temperature=0.7, top_k=1),
+              SamplingParams(temperature=1.0, top_k=40), SamplingParams(temperature=1.0, top_k=40), SamplingParams(temperature=2.0, top_k=30),
+              SamplingParams(temperature=1.0, top_k=10), SamplingParams(temperature=0.9, top_k=65, top_p=0.95),
+              SamplingParams(temperature=1.0), SamplingParams(temperature=0.0), SamplingParams(temperature=1.1, top_p=0.5)]
+    logits = torch.randn(len(params), vocab, generator=g) * 3.0
+    logits[1, 100:140] = float(logits[1].max()) + 1.0                 # forty equal largest logits and a top-k of 5: all stay
+    logits[4, :] = torch.round(logits[4])                              # a few distinct values: thousands of equals in a part
+    logits[5, :] = -200.0 + 0.001 * torch.randn(vocab, generator=g)    # peaked: three tokens far above everything else
+    logits[5, [7, vocab // 2, vocab - 1]] = torch.tensor([0.0, -0.5, -1.0])
+    logits[6, :] = float("-inf")
+    logits[6, [3, 9000, vocab - 2]] = torch.tensor([1.0, 0.5, 2.0])
+    logits[7, ::3] = float("nan")
+
+    def draw(kinds, d):
+        reqs = [SampleRequest(p, seed=900 + i, draw=d) for i, p in enumerate(params)]
+        out = torch.full((len(params),), -1, dtype=torch.int32, device=DEV)
+        ops.sample(logits.to(DEV), torch.empty(len(params), vocab, device=DEV), pack_rows(reqs).to(DEV), out, kinds)
+        return out.cpu().tolist()
+
+    for d in range(4):
+        want = [plain_llama.device_sample(logits[i].numpy(), p.temperature, p.top_k, p.top_p, 900 + i, d, p.min_p) for i, p in enumerate(params)]
+        assert draw(7, d) == want, d
+        assert draw(3, d) == want, d                # without the hint the single workgroup does it
+    assert {draw(7, d)[1] for d in range(12)} <= set(range(100, 140)) and len({draw(7, d)[1] for d in range(12)}) > 3
+    counters = type(ops)._workspaces[torch.cuda.current_device()][: 64 * 1024]
+    torch.cuda.synchronize()
+    assert int(counters.to(torch.int64).sum()) == 0
+
+
 def test_adjust_logits(ops):
     """Penalties, biases, blocked and allowed ids on rows of logits against the plain functions: a row with everything, a row
     whose newest token is on the device only and already in its list (it counts once more), one whose newest token
