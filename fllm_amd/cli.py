@@ -33,6 +33,8 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--kv-watermark-blocks", type=int, default=0)
     ap.add_argument("--max-num-partial-prefills", type=int, default=0)
     ap.add_argument("--long-prefill-token-threshold", type=int, default=0)
+    ap.add_argument("--max-long-partial-prefills", type=int, default=1,
+                    help="prompts longer than the threshold that may be in their portions at once")
     ap.add_argument("--preemption-mode", default="recompute", choices=["recompute", "none"])
     ap.add_argument("--scheduling-policy", default="fcfs", choices=["fcfs", "priority"])
     ap.add_argument("--prefix-cache", action="store_true", default=None,
@@ -54,7 +56,8 @@ def _make_engine(args, model):
                   max_batched_tokens=args.max_batched_tokens, block_size=args.kv_block_size, num_blocks=args.kv_blocks,
                   gpu_memory_utilization=args.gpu_memory_utilization, kv_watermark_blocks=args.kv_watermark_blocks,
                   max_num_partial_prefills=args.max_num_partial_prefills,
-                  long_prefill_token_threshold=args.long_prefill_token_threshold, preemption_mode=args.preemption_mode,
+                  long_prefill_token_threshold=args.long_prefill_token_threshold,
+                  max_long_partial_prefills=args.max_long_partial_prefills, preemption_mode=args.preemption_mode,
                   decode_first=args.chunked_prefill_policy == "decode-first", ahead=args.ahead,
                   scheduling_policy=args.scheduling_policy, prefix_cache=args.prefix_cache,
                   check_layers=args.check_layers)
@@ -65,7 +68,7 @@ def cmd_run(argv: List[str]) -> int:
     ap.add_argument("model")
     ap.add_argument("--prompt-ids", action="append", default=[], help="comma-separated token ids (repeatable)")
     ap.add_argument("--prompts-file", help="JSON file: a list of token id lists")
-    ap.add_argument("--max-tokens", type=int, default=64)
+    ap.add_argument("--max-tokens", "--max-new", dest="max_tokens", type=int, default=64)
     ap.add_argument("--temperature", "--temp", dest="temperature", type=float, default=None, help="0: greedy (the default)")
     ap.add_argument("--top-p", type=float, default=None)
     ap.add_argument("--top-k", type=int, default=None)
@@ -73,6 +76,8 @@ def cmd_run(argv: List[str]) -> int:
                     help="where sampling defaults come from when a flag is left out: the model folder's generation_config.json "
                          "(auto), nowhere (vllm), or a file or folder named here; of its keys temperature, top_p, top_k, min_p "
                          "and repetition_penalty count")
+    ap.add_argument("--no-generation-config", dest="generation_config", action="store_const", const="vllm",
+                    help="the same as --generation-config vllm")
     ap.add_argument("--seed", type=int, default=None)
     ap.add_argument("--n", type=int, default=1, help="answers to every prompt (at most 16), each with draws of its own")
     ap.add_argument("--min-p", type=float, default=None, help="drop what weighs less than this share of the likeliest token")

@@ -68,7 +68,7 @@ class Engine:
                  dtype: str = "bfloat16", device: str = "cuda:0", ctx: Optional[int] = None, max_seqs: int = 16,
                  max_batched_tokens: int = 512, block_size: int = 16, num_blocks: Optional[int] = None,
                  gpu_memory_utilization: float = 0.90, decode_first: bool = True, kv_watermark_blocks: int = 0,
-                 max_num_partial_prefills: int = 0, long_prefill_token_threshold: int = 0,
+                 max_num_partial_prefills: int = 0, long_prefill_token_threshold: int = 0, max_long_partial_prefills: int = 1,
                  preemption_mode: str = "recompute", eos_token_ids: Optional[Seq[int]] = None,
                  random_weights_on_device: bool = False, ops=None, ahead: bool = True, check_layers: int = 0,
                  scheduling_policy: str = "fcfs", prefix_cache: Optional[bool] = None):
@@ -77,7 +77,7 @@ class Engine:
         own when `random_weights_on_device`: large models).  Option names follow the reference's server flags
         (rust/engine/src/bin/serve.rs:530-557, :681-782): ctx, max_seqs, max_batched_tokens,
         gpu_memory_utilization, kv_watermark_blocks, max_num_partial_prefills,
-        long_prefill_token_threshold, preemption_mode, scheduling_policy (`fcfs`, or `priority`: requests with the
+        long_prefill_token_threshold, max_long_partial_prefills, preemption_mode, scheduling_policy (`fcfs`, or `priority`: requests with the
         smaller `SamplingParams.priority` first, and a waiting one of better priority takes the place of the worst
         running one).  `prefix_cache` (the reference's environment switch FLLM_PREFIX_CACHE, rust/engine/src/runtime.rs:193-206,
         is read when it is None; off by default here): full cache pages outlive their request, and a request that begins
@@ -117,7 +117,8 @@ class Engine:
         self.scheduler = Scheduler(
             SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=max_batched_tokens, decode_first=decode_first,
                             watermark_pages=kv_watermark_blocks, max_partial_prefills=max_num_partial_prefills,
-                            long_prefill_threshold=long_prefill_token_threshold, preemption=preemption_mode,
+                            long_prefill_threshold=long_prefill_token_threshold,
+                            max_long_partial_prefills=max_long_partial_prefills, preemption=preemption_mode,
                             policy=scheduling_policy, prefix_cache=bool(prefix_cache)),
             self.runner.cache, self.max_model_len)
         self.sampler = Sampler(self.runner.rt)
