@@ -401,10 +401,13 @@ def test_toy_norm_keeps_the_fused_decode_kernels_and_a_layer_may_lack_a_feed_for
     tensors = {k: v.float() for k, v in random_tensors(spec, 23, torch.bfloat16).items()}
     runner = ModelRunner(spec, tensors, dtype=dtype, page_size=16, max_tokens=256, max_requests=4)
     assert runner.use_graphs and runner.model.blocks[0].feed_forward is None
-    calls = {"norm_qkv_rope_store": 0, "norm_gate_up_swiglu": 0}
+    calls = {"norm_qkv_rope_store": 0, "norm_gate_up_swiglu": 0, "linear_add_prepare": 0}
+    fed = {"norm_qkv_rope_store": 0, "norm_gate_up_swiglu": 0}       # calls that got a norm prepared by the sum before
     for name in calls:
         def counted(*args, _fn=getattr(runner.rt.ops, name), _name=name, **kw):
             calls[_name] += 1
+            if kw.get("prepared") is not None:
+                fed[_name] += 1
             return _fn(*args, **kw)
         setattr(runner.rt.ops, name, counted)
     try:
@@ -427,8 +430,12 @@ def test_toy_norm_keeps_the_fused_decode_kernels_and_a_layer_may_lack_a_feed_for
         assert err <= tol * np.abs(want).max(), err
     if dtype == "bfloat16":      # the decode steps went through the kernels that norm on the way in, and through graphs
         assert calls["norm_qkv_rope_store"] >= 2 and calls["norm_gate_up_swiglu"] >= 1 and runner.graph_replays >= 8
+        # the toy norm says what it multiplies by, so the sums before it prepare it: every norm but a step's first one
+        # comes prepared (a layer without a feed-forward prepares the first norm of the layer after)
+        assert calls["linear_add_prepare"] > 0 and fed["norm_qkv_rope_store"] + fed["norm_gate_up_swiglu"] == calls["linear_add_prepare"]
+        assert 2 * fed["norm_qkv_rope_store"] == calls["norm_qkv_rope_store"] and fed["norm_gate_up_swiglu"] == calls["norm_gate_up_swiglu"]
     else:
-        assert calls == {"norm_qkv_rope_store": 0, "norm_gate_up_swiglu": 0}
+        assert calls == {"norm_qkv_rope_store": 0, "norm_gate_up_swiglu": 0, "linear_add_prepare": 0}
 
 
 def test_state_slot_is_handed_over_cleared():
