@@ -1109,10 +1109,13 @@ int launch_resident(const SkinnyArgs &a, hipStream_t stream) {
         ResidentPlan p = plan_resident(a.M, a.K, tiles16, RT, ws, x_direct);
         if (p.S == 0) return 1;
         // 8-row tiles (two K halves a product) when the rows allow it and the 16-row tiles come to between half a
-        // tile and two tiles per slot, unevenly: 384 tiles on 512 slots run as long as 512 would
+        // tile and two tiles per slot, unevenly: 384 tiles on 512 slots run as long as 512 would.  Also when the 16-row
+        // tiles fill no more than half of the compute units (narrow models): twice the workgroups, each with half the
+        // weights (128 tiles of 2,048 x 8,192: 12.7 -> 9.4 us at one row; 192 tiles gain nothing, 7.7 -> 8.1 us, and at
+        // 256 tiles it is the other way round, 26.9 -> 32.3 us)
         const int slots = device_cus() * p.per_cu;
-        const bool dual = a.M <= 8 && p.S == 1 && fllm_option_dual_k() && 2 * tiles16 > slots && tiles16 < 2 * slots &&
-                          tiles16 % slots != 0;
+        const bool uneven = 2 * tiles16 > slots && tiles16 < 2 * slots && tiles16 % slots != 0;
+        const bool dual = a.M <= 8 && p.S == 1 && fllm_option_dual_k() && (uneven || 2 * tiles16 <= device_cus());
         if constexpr (PRO == PRO_BF16) {
             if (x_direct) {
                 if (dual) return launch_resident_plan<PRO, EPI, TM_DUALK, 8, true>(a, p, tiles8, ws, stream);
