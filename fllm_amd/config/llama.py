@@ -19,13 +19,28 @@ _EPS_KEYS = ("rms_norm_eps", "layer_norm_eps", "norm_epsilon", "layer_norm_epsil
 
 @dataclass(frozen=True)
 class RopeScaling:
-    """`kind` is one of "none", "linear", "llama3"."""
+    """`kind` is one of "none", "linear", "llama3", "yarn", "longrope".
+
+    yarn (plan.rs:1433-1477 → config.rs:1558-1569): `extrapolation`, `attention`, `beta_fast`, `beta_slow`,
+    `truncate` are the values the reference's engine reads, with its defaults; `attention` is the checkpoint's
+    magnitude of cos and sin (`attention_factor`, or the quotient of the `mscale` pair), None for the built-in
+    1 + 0.1 ln(factor).  longrope (plan.rs:1507-1548): per-lane divisors for
+    contexts up to `original_max_position` (`short_factor`) and beyond (`long_factor`); `attention` multiplies
+    cos and sin.  `dynamic` with an `alpha` only changes the base (plan.rs:1339-1343) and leaves kind "none".
+    """
 
     kind: str = "none"
     factor: float = 1.0
     low_freq_factor: float = 1.0
     high_freq_factor: float = 4.0
     original_max_position: int = 0
+    extrapolation: float = 1.0
+    attention: Optional[float] = None
+    beta_fast: float = 32.0
+    beta_slow: float = 1.0
+    truncate: bool = True
+    short_factor: Tuple[float, ...] = ()
+    long_factor: Tuple[float, ...] = ()
 
 
 @dataclass(frozen=True)
@@ -112,7 +127,12 @@ class LlamaConfig:
             rope_dims = int(round(head_dim * partial))
         if head_dim % 2 != 0 or rope_dims % 2 != 0 or rope_dims <= 0 or rope_dims > head_dim:
             raise ConfigError("the decoder requires even head and rotary dimensions")
-        scaling = _rope_scaling(rope_raw, rope_kind, cfg)
+        if rope_kind == "dynamic" and _float(rope_raw, "alpha") is not None:
+            # plan.rs:1339-1343: the NTK-aware base; nothing else of the scaling is kept (:1376)
+            theta = theta * _float(rope_raw, "alpha") ** (head_dim / (head_dim - 2.0))
+            scaling = RopeScaling()
+        else:
+            scaling = _rope_scaling(rope_raw, rope_kind, cfg, rope_dims, max_position)
 
         windows = _layer_windows(cfg, layers)
 
@@ -173,6 +193,26 @@ class LlamaConfig:
                 "low_freq_factor": s.low_freq_factor,
                 "high_freq_factor": s.high_freq_factor,
                 "original_max_position_embeddings": s.original_max_position,
+            }
+        elif s.kind == "yarn":
+            out["rope_scaling"] = {
+                "rope_type": "yarn",
+                "factor": s.factor,
+                "original_max_position_embeddings": s.original_max_position,
+                "beta_fast": s.beta_fast,
+                "beta_slow": s.beta_slow,
+                "extrapolation_factor": s.extrapolation,
+                "truncate": s.truncate,
+            }
+            if s.attention is not None:
+                out["rope_scaling"]["attention_factor"] = s.attention
+        elif s.kind == "longrope":
+            out["rope_scaling"] = {
+                "rope_type": "longrope",
+                "short_factor": list(s.short_factor),
+                "long_factor": list(s.long_factor),
+                "original_max_position_embeddings": s.original_max_position,
+                "attention_factor": s.attention,
             }
         windows = [w for w in self.layer_windows if w is not None]
         if windows:
@@ -238,7 +278,7 @@ def _rope_params(cfg: Dict[str, Any]) -> Tuple[Dict[str, Any], str, Optional[flo
     return raw, kind, theta
 
 
-def _rope_scaling(raw: Dict[str, Any], kind: str, cfg: Dict[str, Any]) -> RopeScaling:
+def _rope_scaling(raw: Dict[str, Any], kind: str, cfg: Dict[str, Any], rope_dims: int, ctx: int) -> RopeScaling:
     if kind == "default":
         return RopeScaling()
     if kind == "linear":
@@ -261,6 +301,50 @@ def _rope_scaling(raw: Dict[str, Any], kind: str, cfg: Dict[str, Any]) -> RopeSc
             raise ConfigError("invalid llama3 rope_scaling values")
         return RopeScaling(kind="llama3", factor=factor, low_freq_factor=low, high_freq_factor=high,
                            original_max_position=int(original))
+    if kind == "yarn":
+        # plan.rs:1433-1477 (config.json keys) and config.rs:1558-1569 (the engine's defaults)
+        factor = _float(raw, "factor")
+        if factor is None:
+            raise ConfigError("yarn rope_scaling requires factor")
+        original = _first(_uint(raw, "original_max_position_embeddings"), _uint(cfg, "original_max_position_embeddings"))
+        if original is None:
+            raise ConfigError("yarn rope_scaling requires original_max_position_embeddings")
+        if not factor > 0.0 or original == 0:
+            raise ConfigError("invalid yarn rope_scaling values")
+        magnitude = lambda m: 0.1 * m * math.log(factor) + 1.0
+        given = _float(raw, "attention_factor")
+        if given is None:
+            a, b = _float(raw, "mscale"), _float(raw, "mscale_all_dim")
+            if a is not None and b is not None:
+                given = magnitude(a) / magnitude(b)
+        return RopeScaling(kind="yarn", factor=factor, original_max_position=original, attention=given,
+                           beta_fast=_first(_float(raw, "beta_fast"), 32.0),
+                           beta_slow=_first(_float(raw, "beta_slow"), 1.0),
+                           extrapolation=_first(_float(raw, "extrapolation_factor"), 1.0),
+                           truncate=raw.get("truncate") is not False)
+    if kind in ("longrope", "su"):
+        # plan.rs:1507-1548
+        def factors(key: str) -> Tuple[float, ...]:
+            v = raw.get(key)
+            if not isinstance(v, list):
+                raise ConfigError(f"longrope scaling requires {key}")
+            return tuple(float(x) for x in v if isinstance(x, (int, float)) and not isinstance(x, bool))
+        short, long = factors("short_factor"), factors("long_factor")
+        lanes = rope_dims // 2
+        if len(short) != lanes or len(long) != lanes:
+            raise ConfigError(f"longrope factors must have {lanes} entries")
+        original = _first(_uint(raw, "original_max_position_embeddings"), _uint(cfg, "original_max_position_embeddings"), ctx)
+        if original == 0 or any(not f > 0.0 for f in short + long):
+            raise ConfigError("invalid longrope scaling values")
+        scale = ctx / original
+        default = math.sqrt(1.0 + math.log(scale) / math.log(original)) if scale > 1.0 else 1.0
+        return RopeScaling(kind="longrope", original_max_position=original,
+                           attention=_first(_float(raw, "attention_factor"), default),
+                           short_factor=short, long_factor=long)
+    if kind in ("dynamic", "dynamic-ntk", "dynamic_ntk"):
+        # the reference's planner passes the kind on (plan.rs:1379-1392) and its engine then refuses the model
+        # with these words (rust/engine/src/config.rs:1570); only `dynamic` with an `alpha` runs (above)
+        raise ConfigError('unsupported rope scaling type "dynamic"')
     raise ConfigError(f"unsupported rope_scaling type {kind!r}")
 
 

@@ -27,6 +27,13 @@ def build_spec(cfg: LlamaConfig) -> ModelSpec:
         "low_freq_factor": s.low_freq_factor,
         "high_freq_factor": s.high_freq_factor,
         "original_max_position": s.original_max_position,
+        "extrapolation": s.extrapolation,
+        "attention": s.attention,
+        "beta_fast": s.beta_fast,
+        "beta_slow": s.beta_slow,
+        "truncate": s.truncate,
+        "short_factor": s.short_factor,
+        "long_factor": s.long_factor,
         "max_position": cfg.max_position,
     }
     layers = []

@@ -34,6 +34,12 @@ def read_sizes(cfg):
     out["theta"] = float(scaling.get("rope_theta", cfg.get("rope_theta", 10000.0)))
     out["rope_kind"] = str(scaling.get("rope_type", scaling.get("type", "default"))).lower()
     out["rope_scaling"] = scaling
+    out["context"] = out["model_context"] = cfg.get("max_position_embeddings", 40960)
+    if out["rope_kind"] == "dynamic" and "alpha" in scaling:
+        # rust/checkpoint/src/plan.rs:1339-1343: the base grows, nothing else of the scaling stays (:1376)
+        d = float(out["head_dim"])
+        out["theta"] *= float(scaling["alpha"]) ** (d / (d - 2.0))
+        out["rope_kind"] = "default"
     partial = cfg.get("partial_rotary_factor", 1.0)
     out["rope_dims"] = int(round(out["head_dim"] * partial))
     window = cfg.get("sliding_window") or 0
@@ -78,10 +84,82 @@ def llama3_divisors(dims, theta, factor, low, high, original):
     return np.array(out, dtype=np.float32)
 
 
-def rope_tables(positions, dims, theta, kind="default", scaling=None):
+def yarn_values(scaling, cfg_original=None):
+    """What the engine's YaRN tables are built from, out of the keys of config.json
+    (rust/checkpoint/src/plan.rs:1433-1477 writes them as float32 metadata, rust/engine/src/config.rs:1558-1569 reads
+    them with these defaults): the checkpoint's `attention_factor` (or mscale quotient) h replaces the built-in
+    magnitude 1 + 0.1 ln(factor), so the engine's factor is h / (1 + 0.1 ln(factor))."""
+    factor = float(scaling["factor"])
+    magnitude = lambda m: 0.1 * m * math.log(factor) + 1.0
+    h = scaling.get("attention_factor")
+    if h is None and "mscale" in scaling and "mscale_all_dim" in scaling:
+        h = magnitude(float(scaling["mscale"])) / magnitude(float(scaling["mscale_all_dim"]))
+    return {
+        "factor": np.float32(factor),
+        "original": int(scaling.get("original_max_position_embeddings", cfg_original)),
+        "extrapolation": np.float32(scaling.get("extrapolation_factor", 1.0)),
+        "attention": np.float32(1.0 if h is None else float(h) / magnitude(1.0)),
+        "beta_fast": np.float32(scaling.get("beta_fast", 32.0)),
+        "beta_slow": np.float32(scaling.get("beta_slow", 1.0)),
+        "truncate": scaling.get("truncate") is not False,
+    }
+
+
+def yarn_tables(positions, inverse, dims, base, y):
+    """rust/engine/src/rope.rs:70-110 with :15-23, all in float32 up to the phase: a lane's angle is a mix of the
+    plain angle (position * inverse) and the interpolated one (that divided by the factor); the lanes below the
+    correction dimension of `beta_fast` keep the plain angle, those above that of `beta_slow` the interpolated
+    one, a straight ramp between; cos and sin are multiplied by attention * (1 + 0.1 ln(factor))."""
+    f = np.float32
+    two_pi = f(2.0) * f(math.pi)
+
+    def correction_dim(rotations):
+        return f(f(dims) * np.log(f(f(y["original"]) / f(rotations * two_pi))) / f(f(2.0) * np.log(f(base))))
+
+    low, high = correction_dim(y["beta_fast"]), correction_dim(y["beta_slow"])
+    if y["truncate"]:
+        low, high = np.floor(low), np.ceil(high)
+    low, high = max(low, f(0.0)), min(high, f(dims - 1))
+    scale = f(1.0) / y["factor"]
+    lanes = np.arange(len(inverse), dtype=np.float32)
+    ramp = f(1.0) - np.clip((lanes - low) / max(f(high - low), f(0.001)), f(0.0), f(1.0)).astype(np.float32)
+    pos = np.asarray(positions, dtype=np.float32)
+    extrapolated = (pos[:, None] * inverse[None, :]).astype(np.float32)
+    interpolated = (scale * extrapolated).astype(np.float32)
+    if y["extrapolation"] != 0.0:
+        mix = (ramp * y["extrapolation"]).astype(np.float32)[None, :]
+        theta = (interpolated * (f(1.0) - mix) + extrapolated * mix).astype(np.float32)
+        magnitude = f(y["attention"] * f(f(1.0) + f(0.1) * np.log(f(f(1.0) / scale))))
+    else:
+        theta, magnitude = interpolated, y["attention"]
+    phase = theta.astype(np.float64)
+    cos = (np.cos(phase).astype(np.float32) * magnitude).astype(np.float32)
+    sin = (np.sin(phase).astype(np.float32) * magnitude).astype(np.float32)
+    return cos.astype(np.float64), sin.astype(np.float64)
+
+
+def longrope_values(scaling, dims, context):
+    """rust/checkpoint/src/plan.rs:1507-1548: the two lists of dims/2 factors, the original context (the model's
+    own context when the key is missing) and the factor on cos and sin: `attention_factor`, else
+    sqrt(1 + ln(context / original) / ln(original)) when the context is longer than the original one, else 1."""
+    short = np.array(scaling["short_factor"], dtype=np.float32)
+    long = np.array(scaling["long_factor"], dtype=np.float32)
+    assert len(short) == len(long) == dims // 2
+    original = int(scaling.get("original_max_position_embeddings", context))
+    ratio = context / original
+    attention = scaling.get("attention_factor")
+    if attention is None:
+        attention = math.sqrt(1.0 + math.log(ratio) / math.log(original)) if ratio > 1.0 else 1.0
+    return short, long, original, np.float32(attention)
+
+
+def rope_tables(positions, dims, theta, kind="default", scaling=None, context=None, model_context=None):
     """rust/engine/src/rope.rs:38-68: inverse frequencies in float32 (divided by the per-lane
     divisors when there are any), phase = position * inverse in float32 (`linear` scaling divides
-    the position, :53-62), cos and sin in float64.  Returns float64 [len(positions), dims/2]."""
+    the position, :53-62), cos and sin in float64.  `yarn`: see yarn_tables.  `longrope` (:30-36, :58-66): the
+    frequencies are divided by the long factors when the engine's tables reach beyond the original context
+    (`context` positions; the model's own context, `model_context`, when left out), by the short ones otherwise,
+    and cos and sin are multiplied by the attention factor in float32.  Returns float64 [len(positions), dims/2]."""
     scaling = scaling or {}
     half = dims // 2
     lanes = np.arange(half, dtype=np.float32)
@@ -97,10 +175,20 @@ def rope_tables(positions, dims, theta, kind="default", scaling=None):
                                              float(scaling["original_max_position_embeddings"]))).astype(np.float32)
     elif kind == "linear":
         scale = np.float32(1.0) / np.float32(scaling["factor"])
+    elif kind == "yarn":
+        return yarn_tables(positions, inverse, dims, np.float32(theta), yarn_values(scaling))
+    elif kind in ("longrope", "su"):
+        model_context = model_context or context or 40960
+        short, long, original, magnitude = longrope_values(scaling, dims, model_context)
+        inverse = (inverse / (long if (context or model_context) > original else short)).astype(np.float32)
     elif kind != "default":
         raise ValueError(kind)
     pos = np.asarray(positions, dtype=np.float32) * scale
     phase = (pos[:, None] * inverse[None, :]).astype(np.float32).astype(np.float64)
+    if kind in ("longrope", "su"):
+        cos = (np.cos(phase).astype(np.float32) * magnitude).astype(np.float32)
+        sin = (np.sin(phase).astype(np.float32) * magnitude).astype(np.float32)
+        return cos.astype(np.float64), sin.astype(np.float64)
     return np.cos(phase), np.sin(phase)
 
 
@@ -172,18 +260,23 @@ def attention_layer(x, weights, prefix, sizes, layer, positions):
     q = linear(x, g("q_proj.weight"), g("q_proj.bias")).reshape(T, heads, d)
     k = linear(x, g("k_proj.weight"), g("k_proj.bias")).reshape(T, kv_heads, d)
     v = linear(x, g("v_proj.weight"), g("v_proj.bias")).reshape(T, kv_heads, d)
-    cos, sin = rope_tables(positions, sizes["rope_dims"], sizes["theta"], sizes["rope_kind"], sizes["rope_scaling"])
+    cos, sin = rope_tables(positions, sizes["rope_dims"], sizes["theta"], sizes["rope_kind"], sizes["rope_scaling"],
+                           sizes["context"], sizes["model_context"])
     q = apply_rope(q, cos, sin, sizes["rope_dims"])
     k = apply_rope(k, cos, sin, sizes["rope_dims"])
     o = attention(q, k, v, 1.0 / math.sqrt(d), sizes["windows"][layer])
     return linear(o.reshape(T, heads * d), g("o_proj.weight"), g("o_proj.bias"))
 
 
-def forward(cfg, weights, token_ids, first_position=0):
+def forward(cfg, weights, token_ids, first_position=0, context=None):
     """Logits [T, vocab] of a whole sequence (rust/engine/src/rust_decoder.rs:8531-8701 and
     :8706-9117): embedding; per layer x += attention(norm(x)), x += mlp(norm(x)); final norm;
-    head (the embedding table when `tie_word_embeddings`, rust_decoder.rs:2503-2507)."""
+    head (the embedding table when `tie_word_embeddings`, rust_decoder.rs:2503-2507).  `context`: the positions the
+    engine is set up for (rust/engine/src/model.rs:307), the model's own context when left out; only `longrope`
+    looks at it."""
     sizes = read_sizes(cfg)
+    if context is not None:
+        sizes["context"] = context
     ids = np.asarray(token_ids, dtype=np.int64)
     positions = np.arange(first_position, first_position + len(ids))
     x = np.asarray(weights["model.embed_tokens.weight"], dtype=np.float64)[ids]

@@ -1,5 +1,6 @@
 """Configuration and registry: keys, defaults and refusals."""
 import copy
+import math
 
 import pytest
 
@@ -48,6 +49,32 @@ def test_rope_parameters_form():
     assert LlamaConfig.from_dict(cfg) == LlamaConfig.from_dict(tc.TINY_B)
 
 
+def test_yarn_longrope_and_dynamic_keys():
+    """plan.rs:1433-1477, :1507-1548, :1339-1343."""
+    f = LlamaConfig.from_dict(tc.TINY_F).rope_scaling
+    assert (f.kind, f.factor, f.original_max_position, f.beta_fast, f.beta_slow) == ("yarn", 4.0, 64, 16.0, 2.0)
+    assert f.extrapolation == 1.0 and f.truncate and f.attention is None
+    cfg = copy.deepcopy(tc.TINY_F)
+    cfg["rope_scaling"].update(mscale=1.0, mscale_all_dim=0.5, truncate=False, extrapolation_factor=0.5)
+    del cfg["rope_scaling"]["original_max_position_embeddings"]
+    cfg["original_max_position_embeddings"] = 32                       # the model's own key stands in
+    y = LlamaConfig.from_dict(cfg).rope_scaling
+    assert y.original_max_position == 32 and not y.truncate and y.extrapolation == 0.5
+    assert abs(y.attention - (1 + 0.1 * math.log(4.0)) / (1 + 0.05 * math.log(4.0))) < 1e-12
+    cfg["rope_scaling"]["attention_factor"] = 1.5                      # goes before the pair
+    assert LlamaConfig.from_dict(cfg).rope_scaling.attention == 1.5
+    g = LlamaConfig.from_dict(tc.TINY_G)
+    assert g.rope_dims == 24 and g.rope_scaling.kind == "longrope" and len(g.rope_scaling.long_factor) == 12
+    assert abs(g.rope_scaling.attention - math.sqrt(1 + math.log(160 / 48) / math.log(48))) < 1e-12
+    cfg = copy.deepcopy(tc.TINY_G)
+    del cfg["rope_scaling"]["original_max_position_embeddings"]        # then the model's context is the original one
+    s = LlamaConfig.from_dict(cfg).rope_scaling
+    assert s.original_max_position == 160 and s.attention == 1.0
+    cfg = dict(tc.TINY_A, rope_scaling={"rope_type": "dynamic", "alpha": 4.0})
+    d = LlamaConfig.from_dict(cfg)
+    assert d.rope_scaling.kind == "none" and abs(d.rope_theta - 10000.0 * 4.0 ** (16 / 14)) < 1e-6
+
+
 def test_windows():
     c = LlamaConfig.from_dict(tc.TINY_C)
     assert c.layer_windows == (24, None, 24, None) and c.rope_dims == 24
@@ -74,7 +101,12 @@ def test_windows():
     ({"rms_norm_eps": 0.0}, "invalid rms_norm_eps"),
     ({"rope_scaling": {"rope_type": "llama3", "original_max_position_embeddings": 64}}, "requires factor"),
     ({"rope_scaling": {"rope_type": "llama3", "factor": 8.0}}, "requires original_max_position_embeddings"),
-    ({"rope_scaling": {"rope_type": "yarn", "factor": 8.0}}, "unsupported rope_scaling type"),
+    ({"rope_scaling": {"rope_type": "yarn", "factor": 8.0}}, "yarn rope_scaling requires original_max_position_embeddings"),
+    ({"rope_scaling": {"rope_type": "yarn", "original_max_position_embeddings": 64}}, "yarn rope_scaling requires factor"),
+    ({"rope_scaling": {"rope_type": "longrope", "long_factor": [1.0] * 8}}, "longrope scaling requires short_factor"),
+    ({"rope_scaling": {"rope_type": "su", "short_factor": [1.0] * 8, "long_factor": [1.0] * 7}}, "longrope factors must have 8 entries"),
+    ({"rope_scaling": {"rope_type": "dynamic", "factor": 2.0}}, 'unsupported rope scaling type "dynamic"'),
+    ({"rope_scaling": {"rope_type": "proportional", "factor": 2.0}}, "unsupported rope_scaling type"),
     ({"rope_scaling": {"type": "linear"}}, "linear rope_scaling requires factor"),
     ({"head_dim": 15}, "even head and rotary dimensions"),
     ({"quantization_config": {"bits": 4}}, "quantized"),

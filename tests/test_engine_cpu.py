@@ -25,7 +25,7 @@ def runner_for(name, max_tokens, **kw):
     return cfg, tc.to_float64(tensors), r
 
 
-@pytest.mark.parametrize("name,lengths", [("A", [5, 17, 40]), ("C", [30, 70])])
+@pytest.mark.parametrize("name,lengths", [("A", [5, 17, 40]), ("C", [30, 70]), ("F", [20, 70]), ("G", [49, 60])])
 @pytest.mark.parametrize("family", ["whole", "last32", "portions", "mixed"])
 def test_every_way_of_cutting_gives_the_plain_logits(tmp_path, name, lengths, family):
     requests = {f"r{i}": tc.random_ids(n, tc.CONFIGS[name]["vocab_size"], 50 + i) for i, n in enumerate(lengths)}

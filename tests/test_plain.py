@@ -52,6 +52,87 @@ def test_linear_scaling_divides_the_position():
     assert np.allclose(linear[8], plain[2], atol=1e-6)
 
 
+def test_yarn_reference_vector():
+    """rust/engine/src/rope.rs:153-175: 8 dims, base 10000, factor 4, original context 64, beta 32 / 1, truncated:
+    the fastest lane keeps its angle and only grows by 1 + 0.1 ln 4, the slowest turns a quarter as far."""
+    yarn = {"factor": 4.0, "original_max_position_embeddings": 64}
+    pc, ps = P.rope_tables(range(40), 8, 10000.0)
+    yc, ys = P.rope_tables(range(40), 8, 10000.0, "yarn", yarn)
+    magnitude = 1.0 + 0.1 * math.log(4.0)
+    angle = lambda c, s, p, l: math.atan2(s[p, l], c[p, l])
+    assert abs(angle(yc, ys, 30, 0) - angle(pc, ps, 30, 0)) < 1e-5
+    assert abs(math.hypot(yc[30, 0], ys[30, 0]) - magnitude) < 1e-5
+    assert abs(angle(yc, ys, 30, 3) - angle(pc, ps, 30, 3) / 4.0) < 1e-5
+    # a wrong direction of the ramp would interpolate the fast lane instead: 30 rad / 4 is another angle
+    assert abs(angle(yc, ys, 30, 0) - math.atan2(math.sin(7.5), math.cos(7.5))) > 0.1
+
+
+def test_yarn_special_cases():
+    plain = P.rope_tables(range(50), 16, 10000.0)
+    # factor 1: both angles are the same and ln 1 = 0: plain rotary
+    one = P.rope_tables(range(50), 16, 10000.0, "yarn", {"factor": 1.0, "original_max_position_embeddings": 32})
+    assert np.allclose(one[0], plain[0], atol=1e-6) and np.allclose(one[1], plain[1], atol=1e-6)
+    # no extrapolation at all: linear scaling times the attention factor alone (rope.rs:87-91, :97-101)
+    lin = P.rope_tables(range(50), 16, 10000.0, "linear", {"factor": 4.0})
+    flat = P.rope_tables(range(50), 16, 10000.0, "yarn", {"factor": 4.0, "original_max_position_embeddings": 32,
+                                                           "extrapolation_factor": 0.0})
+    assert np.allclose(flat[0], lin[0], atol=1e-6) and np.allclose(flat[1], lin[1], atol=1e-6)
+    # the checkpoint's attention_factor IS the magnitude: it replaces 1 + 0.1 ln(factor) (plan.rs:1460-1476)
+    given = P.rope_tables(range(50), 16, 10000.0, "yarn", {"factor": 4.0, "original_max_position_embeddings": 32,
+                                                            "attention_factor": 1.25})
+    assert np.allclose(np.hypot(given[0], given[1]), 1.25, atol=1e-6)
+    # the pair of mscales gives the quotient of their magnitudes
+    pair = P.rope_tables(range(50), 16, 10000.0, "yarn", {"factor": 4.0, "original_max_position_embeddings": 32,
+                                                           "mscale": 1.0, "mscale_all_dim": 0.5})
+    want = (1 + 0.1 * math.log(4.0)) / (1 + 0.05 * math.log(4.0))
+    assert np.allclose(np.hypot(pair[0], pair[1]), want, atol=1e-6)
+    # lanes between the two correction dimensions lie between both angles: 64 dims, original 2048: low 8, high 21
+    y = P.yarn_values({"factor": 8.0, "original_max_position_embeddings": 2048})
+    assert (y["beta_fast"], y["beta_slow"], y["truncate"], float(y["attention"])) == (32.0, 1.0, True, 1.0)
+    yc, ys = P.rope_tables([100], 64, 10000.0, "yarn", {"factor": 8.0, "original_max_position_embeddings": 2048})
+    pc, ps = P.rope_tables([100], 64, 10000.0)
+    turn = lambda c, s, l: math.atan2(s[0, l], c[0, l])
+    inv = lambda l: 10000.0 ** (-2.0 * l / 64)
+    for lane in (0, 5, 8):
+        assert abs(turn(yc, ys, lane) - turn(pc, ps, lane)) < 1e-4               # up to low: untouched
+    for lane in (21, 25, 31):
+        assert abs(turn(yc, ys, lane) - 100 * inv(lane) / 8.0) < 1e-5            # from high on: position / 8
+    mid = 100 * inv(14)
+    assert mid / 8.0 + 0.1 < turn(yc, ys, 14) < mid - 0.1 < math.pi              # between: between
+    want = mid / 8.0 * (1 - (1 - 6 / 13)) + mid * (1 - 6 / 13)                   # the ramp is a straight line in the lane
+    assert abs(turn(yc, ys, 14) - want) < 1e-5
+
+
+def test_longrope_chooses_factors_by_the_context():
+    """rust/engine/src/rope.rs:30-36, :58-66; the magnitude of rust/checkpoint/src/plan.rs:1533-1538."""
+    short = [1.0, 1.5, 2.0, 2.5]
+    long = [1.0, 3.0, 6.0, 9.0]
+    s = {"short_factor": short, "long_factor": long, "original_max_position_embeddings": 64}
+    plain = P.rope_tables(range(20), 8, 10000.0)
+    angle = lambda c, s_, p, l: math.atan2(s_[p, l], c[p, l])
+    within = P.rope_tables(range(20), 8, 10000.0, "longrope", s, context=64, model_context=256)
+    beyond = P.rope_tables(range(20), 8, 10000.0, "longrope", s, context=65, model_context=256)
+    magnitude = math.sqrt(1.0 + math.log(4.0) / math.log(64.0))
+    for tables, factors in ((within, short), (beyond, long)):
+        assert np.allclose(np.hypot(*tables), magnitude, atol=1e-6)
+        for lane in range(4):
+            assert abs(angle(*tables, 12, lane) - angle(*plain, 12, lane) / factors[lane]) < 1e-5
+    # a model that is no longer than its original context: magnitude 1; with all factors 1 plain rotary
+    ones = {"short_factor": [1.0] * 4, "long_factor": [1.0] * 4, "original_max_position_embeddings": 64}
+    same = P.rope_tables(range(20), 8, 10000.0, "su", ones, context=64, model_context=64)
+    assert np.allclose(same[0], plain[0], atol=1e-7) and np.allclose(same[1], plain[1], atol=1e-7)
+    fixed = P.rope_tables(range(20), 8, 10000.0, "longrope", dict(ones, attention_factor=1.5), context=64, model_context=64)
+    assert np.allclose(np.hypot(*fixed), 1.5, atol=1e-6)
+
+
+def test_dynamic_alpha_only_changes_the_base():
+    """rust/checkpoint/src/plan.rs:1339-1343."""
+    cfg = {"hidden_size": 64, "num_attention_heads": 4, "num_hidden_layers": 1, "intermediate_size": 8, "head_dim": 16,
+           "rope_theta": 10000.0, "rope_scaling": {"rope_type": "dynamic", "alpha": 4.0, "factor": 2.0}}
+    sizes = P.read_sizes(cfg)
+    assert sizes["rope_kind"] == "default" and abs(sizes["theta"] - 10000.0 * 4.0 ** (16 / 14)) < 1e-6
+
+
 def test_llama3_divisors_reference_vector():
     """rust/checkpoint/src/plan.rs:3219-3232: head_dim 16, theta 5e5, factor 8, low 1, high 4,
     original 8192: 8 divisors, the first 1.0, the last 8.0."""
@@ -158,9 +239,9 @@ def weights():
     return out
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "F", "G"])
 def test_a_shift_of_all_positions_changes_nothing(weights, name):
-    """Rotary attention sees distances only (also with per-lane or linear scaling)."""
+    """Rotary attention sees distances only (also with per-lane, linear, yarn or longrope scaling)."""
     cfg = tc.CONFIGS[name]
     ids = tc.random_ids(20, cfg["vocab_size"], 1)
     a = P.forward(cfg, weights[name], ids)

@@ -14,7 +14,8 @@ import trace_tools as tt
 pytestmark = pytest.mark.gpu
 
 LENGTHS = {"A": [5, 17, 31, 70, 128, 100], "B": [1, 9, 40, 100, 256, 130], "C": [3, 50, 190, 77, 120, 64],
-           "D": [700, 3, 130, 1000, 64], "E": [300, 45, 130, 500, 64, 90]}
+           "D": [700, 3, 130, 1000, 64], "E": [300, 45, 130, 500, 64, 90], "F": [4, 60, 256, 33, 150, 90],
+           "G": [2, 48, 160, 49, 100, 70]}
 # |engine - plain| <= tol * max|plain logit| ; float32 engine against a float64 reference, and
 # bfloat16 (8 bits of mantissa in weights, activations and cache) against the same.  About three times the largest
 # error any case here has shown on the MI355X (float32 7.0e-7, bfloat16 5.7e-3; the test session prints them).
@@ -65,7 +66,7 @@ def make_runner(folder, dtype, page_size, max_tokens, use_graphs=True):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F", "G"])
 @pytest.mark.parametrize("family", ["whole", "last32", "portions", "mixed"])
 def test_replay(models, tmp_path, name, dtype, family):
     folder, cfg, requests, plain = models[name]
