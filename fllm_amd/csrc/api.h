@@ -129,6 +129,11 @@ int fllm_carry_ids(int32_t *ids, const int32_t *source, const int32_t *previous,
 // Probes for measurements: a kernel that only reads `bytes` from `src` (`sink`: 4 bytes a workgroup, left alone),
 // and one that only multiplies (32x32x16 bfloat16 MFMA, `blocks` workgroups of 8 waves; `sink`: 2 KiB a workgroup;
 // returns the floating-point operations of the launch, negative on error).  The caller times them.
+// out[i] = element i of the random tensor with key (key_lo, key_hi): kind 0 a normal number of deviation 0.02, kind 1
+// a norm weight 1 + U(-0.1, 0.1); the generator that fllm_amd/weights/random_init.py specifies, bit for bit what
+// that module computes on the host.  `dtype` 0 float32, 1 bfloat16 (rounded to nearest even).
+int fllm_random_fill(void *out, uint64_t count, uint32_t key_lo, uint32_t key_hi, int kind, int dtype, hipStream_t stream);
+
 int fllm_probe_read(const void *src, size_t bytes, void *sink, int blocks, hipStream_t stream);
 double fllm_probe_mfma_bf16(void *sink, int blocks, int iters, hipStream_t stream);
 

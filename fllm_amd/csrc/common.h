@@ -91,3 +91,24 @@ template <int NW> __device__ __forceinline__ float block_max(float v, float *scr
     for (int i = 0; i < NW; i++) total = fmaxf(total, scratch[i]);
     return total;
 }
+
+// Philox-4x32 with ten rounds (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3"): the counter words in,
+// the output words in their place.  The sampler's draws and the random-weights generator use it.
+struct Philox {
+    uint32_t c0, c1, c2, c3;
+    __device__ __forceinline__ void ten_rounds(uint32_t key_lo, uint32_t key_hi) {
+#pragma unroll
+        for (int round = 0; round < 10; round++) {
+            const uint64_t left = (uint64_t)0xD2511F53u * c0;
+            const uint64_t right = (uint64_t)0xCD9E8D57u * c2;
+            const uint32_t next0 = (uint32_t)(right >> 32) ^ c1 ^ key_lo;
+            const uint32_t next2 = (uint32_t)(left >> 32) ^ c3 ^ key_hi;
+            c1 = (uint32_t)right;
+            c3 = (uint32_t)left;
+            c0 = next0;
+            c2 = next2;
+            key_lo += 0x9E3779B9u;
+            key_hi += 0xBB67AE85u;
+        }
+    }
+};

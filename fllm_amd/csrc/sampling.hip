@@ -145,25 +145,6 @@ argmax_split_kernel(const float *__restrict__ logits, int32_t *__restrict__ out,
 // counter words by fixed odd constants and mixes the halves of the products with the other words and the key; the
 // key moves on by the golden-ratio and sqrt(3) - 1 constants.
 // ---------------------------------------------------------------------------------------------
-struct Philox {
-    uint32_t c0, c1, c2, c3;
-    __device__ __forceinline__ void ten_rounds(uint32_t key_lo, uint32_t key_hi) {
-#pragma unroll
-        for (int round = 0; round < 10; round++) {
-            const uint64_t left = (uint64_t)0xD2511F53u * c0;
-            const uint64_t right = (uint64_t)0xCD9E8D57u * c2;
-            const uint32_t next0 = (uint32_t)(right >> 32) ^ c1 ^ key_lo;
-            const uint32_t next2 = (uint32_t)(left >> 32) ^ c3 ^ key_hi;
-            c1 = (uint32_t)right;
-            c3 = (uint32_t)left;
-            c0 = next0;
-            c2 = next2;
-            key_lo += 0x9E3779B9u;
-            key_hi += 0xBB67AE85u;
-        }
-    }
-};
-
 // The uniform number of (seed, draw, token): the counter is (token, 0, draw), the key is the seed; the top 24 bits of
 // the first output word, centred in their cell, so that the number lies strictly between 0 and 1.
 __device__ __forceinline__ float uniform_of(uint64_t seed, uint64_t draw, uint32_t token) {

@@ -48,7 +48,7 @@ assert SAMPLE_ROW_BYTES == 32
 _lib = None
 
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 
 def load_library(build_if_missing: bool = True):
@@ -113,6 +113,8 @@ def load_library(build_if_missing: bool = True):
     lib.fllm_probe_read.restype = c_int
     lib.fllm_probe_mfma_bf16.argtypes = [c_void, c_int, c_int, c_void]
     lib.fllm_probe_mfma_bf16.restype = ctypes.c_double
+    lib.fllm_random_fill.argtypes = [c_void, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint32, c_int, c_int, c_void]
+    lib.fllm_random_fill.restype = c_int
     lib.fllm_set_fast_kernels.argtypes = [c_int]
     lib.fllm_set_fast_kernels.restype = None
     lib.fllm_attention_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int, c_int]
@@ -200,6 +202,16 @@ class Ops:
             raise KernelError(f"kernels of device {device} were launched on stream {seen:#x} before and are now asked for on "
                               f"stream {handle:#x}: they share the device workspace and must stay on one stream")
         return handle
+
+    def random_fill(self, out: torch.Tensor, key, kind: int) -> torch.Tensor:
+        """Fills `out` with the random tensor of `key` (two 32-bit words): kind 0 normal numbers of deviation 0.02, kind 1
+        norm weights; the generator of `fllm_amd.weights.random_init`."""
+        _dense(out, "out")
+        _need(out.dtype in _DTYPE_CODE, f"out dtype {out.dtype} unsupported")
+        with torch.cuda.device(out.device):
+            self._check(self.lib.fllm_random_fill(_ptr(out), out.numel(), int(key[0]), int(key[1]), int(kind),
+                                                  _DTYPE_CODE[out.dtype], self._stream()))
+        return out
 
     def embed(self, ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
         rows = ids.numel()

@@ -51,6 +51,45 @@ BF16_EPS = 2.0 ** -8
 
 
 # ---------------------------------------------------------------------------------------------
+# random weights: the device draws what the host draws
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(1,), (5,), (130, 77), ((1 << 21) + 3,), (515, 4099)])
+def test_random_weights_are_the_same_bits_on_the_host_and_on_the_device(ops, dtype, shape):
+    from fllm_amd.parts.base import INIT_MATRIX, INIT_NORM
+    from fllm_amd.weights.random_init import random_tensor
+    as_int = torch.int32 if dtype == torch.float32 else torch.int16
+    for kind in (INIT_MATRIX, INIT_NORM):
+        host = random_tensor("model.layers.3.x.weight", shape, kind, 12, dtype, "cpu")
+        device = random_tensor("model.layers.3.x.weight", shape, kind, 12, dtype, DEV, ops)
+        assert device.is_cuda and device.shape == host.shape and device.dtype == dtype
+        differ = (host.view(as_int) != device.cpu().view(as_int)).sum().item()
+        assert differ == 0, f"{kind} {dtype} {shape}: {differ} elements differ"
+
+
+def test_random_model_on_the_device_is_the_model_of_the_host():
+    """An engine whose random weights are drawn on the device computes what the plain implementation computes from the
+    weights drawn on the host: a benchmark's model can be replayed."""
+    import tiny_configs as tc
+    from fllm_amd import Engine, SamplingParams
+    from fllm_amd.registry import model_spec_from_config
+    from fllm_amd.weights import random_tensors
+    cfg = tc.TINY_A
+    _, spec = model_spec_from_config(cfg)
+    host = random_tensors(spec, 4, torch.float32)
+    on_device = random_tensors(spec, 4, torch.float32, device=DEV)
+    assert all(torch.equal(host[n], on_device[n].cpu()) for n in host)
+    engine = Engine(config=cfg, seed=4, dtype="float32", ctx=128, max_seqs=2, block_size=16, num_blocks=16,
+                    random_weights_on_device=True)
+    prompt = tc.random_ids(9, cfg["vocab_size"], 3)
+    tokens = engine.generate([prompt], SamplingParams(max_tokens=6))[0]
+    w64, seq = tc.to_float64(host), list(prompt)
+    for t in tokens:
+        assert t == plain_llama.greedy(plain_llama.forward(cfg, w64, seq)[-1])
+        seq.append(t)
+
+
+# ---------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("rows,width,vocab", [(1, 64, 256), (13, 160, 515), (5, 4104, 1000)])
 def test_embed(ops, ref, dtype, rows, width, vocab):

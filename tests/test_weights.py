@@ -5,6 +5,7 @@ import os
 import struct
 
 import pytest
+import numpy as np
 import torch
 
 import tiny_configs as tc
@@ -138,3 +139,71 @@ def test_sharded_checkpoint(tmp_path):
         json.dump({"weight_map": {names[0]: "../evil.safetensors"}}, fh)
     with pytest.raises(SafetensorsError, match="plain file name"):
         open_checkpoint(str(tmp_path))
+
+
+def _scalar_random_value(seed, name, index, norm_weight):
+    """The generator's specification (the module text of fllm_amd/weights/random_init.py) written out for ONE element
+    with Python integers and NumPy float32 scalars, every operation rounded on its own."""
+    import hashlib
+    import math
+    f = np.float32
+    digest = hashlib.sha256(f"{seed}:{name}".encode()).digest()
+    k = [int.from_bytes(digest[:4], "little"), int.from_bytes(digest[4:8], "little")]
+    c = [index & 0xFFFFFFFF, index >> 32, 0, 0]
+    for _ in range(10):
+        left, right = 0xD2511F53 * c[0], 0xCD9E8D57 * c[2]
+        c = [((right >> 32) ^ c[1] ^ k[0]) & 0xFFFFFFFF, right & 0xFFFFFFFF, ((left >> 32) ^ c[3] ^ k[1]) & 0xFFFFFFFF, left & 0xFFFFFFFF]
+        k = [(k[0] + 0x9E3779B9) & 0xFFFFFFFF, (k[1] + 0xBB67AE85) & 0xFFFFFFFF]
+    w0, w1 = c[0], c[1]
+    if norm_weight:
+        u = (f(w0 >> 9) + f(0.5)) / f(2 ** 23)
+        return f(1.0) + (u * f(0.2) - f(0.1))
+    v = 2 * (w0 >> 9) + 1
+    e = v.bit_length()                       # v = m 2^e with m in [1/2, 1)
+    m = f(v) / f(2.0 ** e)
+    if m < f(math.sqrt(0.5)):
+        m, e = m * f(2.0), e - 1
+    s = (m - f(1.0)) / (m + f(1.0))
+    s2 = s * s
+    series = f(1.0 / 9.0)
+    for t in (1.0 / 7.0, 1.0 / 5.0, 1.0 / 3.0, 1.0):
+        series = series * s2 + f(t)
+    log_u = f(e - 24) * f(math.log(2.0)) + (f(2.0) * s) * series
+    radius = np.sqrt(max(f(-2.0) * log_u, f(0.0)))
+    angle = w1 >> 9
+    quadrant, j = angle >> 21, angle & ((1 << 21) - 1)
+    x = ((f(j) + f(0.5)) / f(2 ** 21)) * f(math.pi / 2)
+    x2 = x * x
+    sine = f(-1.0 / math.factorial(11))
+    for n in (9, 7, 5, 3):
+        sine = sine * x2 + f((-1.0) ** (n // 2) / math.factorial(n))
+    sine = x * (sine * x2 + f(1.0))
+    cosine = f(1.0 / math.factorial(12))
+    for n in (10, 8, 6, 4, 2):
+        cosine = cosine * x2 + f((-1.0) ** (n // 2) / math.factorial(n))
+    cosine = cosine * x2 + f(1.0)
+    turn = [cosine, -sine, -cosine, sine][quadrant]
+    return f(0.02) * (radius * turn)
+
+
+def test_random_generator_follows_its_specification():
+    from fllm_amd.parts.base import INIT_MATRIX, INIT_NORM
+    from fllm_amd.weights.random_init import random_tensor
+    count = (1 << 20) + 37                                          # longer than one piece of the host's evaluation
+    for kind, norm_weight in ((INIT_MATRIX, False), (INIT_NORM, True)):
+        t = random_tensor("model.some.weight", (count,), kind, 5, torch.float32)
+        for i in list(range(40)) + [1 << 20, (1 << 20) - 1, count - 1]:
+            want = _scalar_random_value(5, "model.some.weight", i, norm_weight)
+            assert t[i].item() == float(want), (kind, i)
+        # an element depends on (seed, name, index) only: not on the tensor's size or shape
+        small = random_tensor("model.some.weight", (7, 11), kind, 5, torch.float32)
+        assert torch.equal(small.reshape(-1), t[:77])
+        assert not torch.equal(random_tensor("model.other.weight", (77,), kind, 5, torch.float32), t[:77])
+        # bfloat16 is the float32 value rounded to nearest even
+        assert torch.equal(random_tensor("model.some.weight", (77,), kind, 5, torch.bfloat16), t[:77].to(torch.bfloat16))
+    # what the distribution is meant to be
+    z = random_tensor("w", (1 << 18,), INIT_MATRIX, 9, torch.float32).double() / 0.02
+    assert abs(z.mean()) < 0.01 and abs(z.std() - 1) < 0.01 and abs((z ** 4).mean() - 3) < 0.1 and abs((z ** 3).mean()) < 0.05
+    assert 0.66 < (z.abs() < 1).double().mean() < 0.70 and z.abs().max() > 4.0
+    u = random_tensor("w", (1 << 18,), INIT_NORM, 9, torch.float32).double()
+    assert 0.9 <= u.min() < 0.9001 and 1.0999 < u.max() <= 1.1 and abs(u.mean() - 1) < 1e-3 and abs(u.std() - 0.2 / 12 ** 0.5) < 1e-3
