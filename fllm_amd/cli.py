@@ -169,7 +169,7 @@ def cmd_inspect(argv: List[str]) -> int:
     args = ap.parse_args(argv)
     from .config.files import read_config_json
     from .registry import model_spec_from_config
-    from .weights.loader import check_tensors, expected_tensors
+    from .weights.loader import canonical_names, check_tensors, expected_tensors
     from .weights.safetensors_io import open_checkpoint
     typed, spec = model_spec_from_config(read_config_json(args.model))
     print(f"architecture: {spec.architecture}")
@@ -177,7 +177,7 @@ def cmd_inspect(argv: List[str]) -> int:
     required, _, _ = expected_tensors(spec)
     print(f"tensors expected: {len(required)}, parameters: {sum(int(__import__('math').prod(s)) for s in required.values()):,}")
     found = open_checkpoint(args.model)
-    check_tensors(spec, {n: f.entries[n].shape for n, (f, _) in found.items()})
+    check_tensors(spec, {canonical: found[n][0].entries[n].shape for n, canonical in canonical_names(spec, found).items()})
     dtypes = sorted({f.entries[n].dtype for n, (f, _) in found.items()})
     print(f"checkpoint: {len(found)} tensors, stored as {', '.join(dtypes)}: ok")
     return 0

@@ -77,6 +77,11 @@ class ModelSpec:
     head: PartSpec
     # tensor names a checkpoint may hold that do not affect the forward pass
     ignorable_tensors: Tuple[str, ...] = ()
+    # checkpoints that nest the model under other names: (prefix, replacement) rules, the first that fits a tensor's
+    # name applies; then tensors whose name begins with one of `skipped_tensor_prefixes` are left aside (towers of
+    # other modalities beside the language model)
+    tensor_renames: Tuple[Tuple[str, str], ...] = ()
+    skipped_tensor_prefixes: Tuple[str, ...] = ()
 
     def validate(self) -> None:
         for i, entry in enumerate(self.run_order):

@@ -93,6 +93,12 @@ def build_spec(cfg: LlamaConfig) -> ModelSpec:
         head=PartSpec("linear", {"vocab_size": cfg.vocab_size, "hidden_size": cfg.hidden_size},
                       {"weight": head_tensor}),
         ignorable_tensors=tuple(ignorable),
+        # multimodal checkpoints nest the language model and carry towers that are not run (plan.rs:2624-2650)
+        tensor_renames=(("model.language_model.", "model."), ("language_model.model.", "model."),
+                        ("language_model.lm_head.", "lm_head."), ("language_model.", "model.")),
+        skipped_tensor_prefixes=("model.visual.", "visual.", "vision_tower.", "model.vision_tower.",
+                                 "multi_modal_projector.", "model.multi_modal_projector.", "model.vision_",
+                                 "vision_model.", "vit_large_projector."),
     )
 
 

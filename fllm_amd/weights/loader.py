@@ -65,6 +65,27 @@ def expected_tensors(spec: ModelSpec):
     return required, optional, init
 
 
+def canonical_names(spec: ModelSpec, names) -> Dict[str, str]:
+    """Checkpoint tensor name -> the name the model knows it by, after the architecture's renaming rules
+    (`ModelSpec.tensor_renames`); tensors under a skipped prefix are left out.  Two tensors that come to the same
+    name are an error (the reference refuses duplicate targets, rust/checkpoint/src/plan.rs:3068-3093)."""
+    out: Dict[str, str] = {}
+    taken: Dict[str, str] = {}
+    for name in names:
+        canonical = name
+        for prefix, replacement in spec.tensor_renames:
+            if name.startswith(prefix):
+                canonical = replacement + name[len(prefix):]
+                break
+        if any(canonical.startswith(p) for p in spec.skipped_tensor_prefixes):
+            continue
+        if canonical in taken:
+            raise ValueError(f"checkpoint tensors {taken[canonical]!r} and {name!r} both stand for {canonical!r}")
+        taken[canonical] = name
+        out[name] = canonical
+    return out
+
+
 def check_tensors(spec: ModelSpec, shapes: Dict[str, tuple]) -> None:
     """Raises `WeightsError` unless `shapes` (name -> shape of what a checkpoint holds) fits."""
     required, optional, _ = expected_tensors(spec)
@@ -83,12 +104,13 @@ def check_tensors(spec: ModelSpec, shapes: Dict[str, tuple]) -> None:
 def load_checkpoint(model_dir: str, spec: ModelSpec) -> Dict[str, torch.Tensor]:
     """Name -> CPU tensor in the stored dtype (views of the mapped files; integer tensors as
     int32) for every tensor the model takes."""
-    found = open_checkpoint(model_dir)
-    check_tensors(spec, {n: f.entries[n].shape for n, (f, _) in found.items()})
+    stored = open_checkpoint(model_dir)
+    found = {canonical: stored[name] for name, canonical in canonical_names(spec, stored).items()}
+    check_tensors(spec, {n: f.entries[stored_name].shape for n, (f, stored_name) in found.items()})
     required, optional, _ = expected_tensors(spec)
     out: Dict[str, torch.Tensor] = {}
     for n in list(required) + [o for o in optional if o in found]:
-        t = found[n][0].tensor(n)
+        t = found[n][0].tensor(found[n][1])
         if not t.dtype.is_floating_point:
             t = t.to(torch.int32)
         out[n] = t

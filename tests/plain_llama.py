@@ -261,7 +261,7 @@ def attention_layer(x, weights, prefix, sizes, layer, positions):
     k = linear(x, g("k_proj.weight"), g("k_proj.bias")).reshape(T, kv_heads, d)
     v = linear(x, g("v_proj.weight"), g("v_proj.bias")).reshape(T, kv_heads, d)
     cos, sin = rope_tables(positions, sizes["rope_dims"], sizes["theta"], sizes["rope_kind"], sizes["rope_scaling"],
-                           sizes["context"], sizes["model_context"])
+                           sizes.get("context"), sizes.get("model_context"))
     q = apply_rope(q, cos, sin, sizes["rope_dims"])
     k = apply_rope(k, cos, sin, sizes["rope_dims"])
     o = attention(q, k, v, 1.0 / math.sqrt(d), sizes["windows"][layer])

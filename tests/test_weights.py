@@ -207,3 +207,29 @@ def test_random_generator_follows_its_specification():
     assert 0.66 < (z.abs() < 1).double().mean() < 0.70 and z.abs().max() > 4.0
     u = random_tensor("w", (1 << 18,), INIT_NORM, 9, torch.float32).double()
     assert 0.9 <= u.min() < 0.9001 and 1.0999 < u.max() <= 1.1 and abs(u.mean() - 1) < 1e-3 and abs(u.std() - 0.2 / 12 ** 0.5) < 1e-3
+
+
+def test_nested_language_model_names(tmp_path):
+    """rust/checkpoint/src/plan.rs:2624-2650: `model.language_model.X` is `model.X`, `language_model.model.X` and
+    `language_model.lm_head.X` lose their first part, any other `language_model.X` is `model.X`; vision towers are
+    left aside."""
+    from safetensors.torch import save_file
+    _, spec = model_spec_from_config(tc.TINY_A)
+    tensors = random_tensors(spec, 2, torch.float32)
+    with open(tmp_path / "config.json", "w") as fh:
+        json.dump(tc.TINY_A, fh)
+    for form in (lambda n: "model.language_model." + n[len("model."):] if n.startswith("model.") else n,
+                 lambda n: "language_model." + n,
+                 lambda n: "language_model." + n[len("model."):] if n.startswith("model.") else "language_model." + n):
+        stored = {form(n): t for n, t in tensors.items()}
+        stored["vision_tower.patch.weight"] = torch.zeros(3, 3)
+        stored["model.visual.blocks.0.weight"] = torch.zeros(2)
+        assert set(stored) != set(tensors)
+        save_file(stored, str(tmp_path / "model.safetensors"))
+        loaded = load_checkpoint(str(tmp_path), spec)
+        assert set(loaded) == set(tensors) and all(torch.equal(loaded[n], tensors[n]) for n in tensors)
+    stored = dict(tensors)
+    stored["language_model.model.norm.weight"] = tensors["model.norm.weight"].clone()
+    save_file(stored, str(tmp_path / "model.safetensors"))
+    with pytest.raises(ValueError, match="both stand for 'model.norm.weight'"):
+        load_checkpoint(str(tmp_path), spec)
