@@ -5,7 +5,10 @@ weights, synthetic token ids.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers N] [--shape 8b|1b|70b] [--no-further]
 
 A step is one decode step of the whole engine (scheduler, step function, sampling), with steps
-launched ahead of the tokens of the step before them (--no-ahead: each step waits for the last).  The one
+launched ahead of the tokens of the step before them (--no-ahead: each step waits for the last).  Every headline
+figure (batch 1, 8, 64 and the prefill) is the median of --repeats (3) timed runs of K steps, each with requests of its own;
+"runs_ms_per_step" lists them all.  "kernels" gives the device time of the kernels a batch-8 decode step and a prefill
+step spend most on, in microseconds a step, from a short profiled run behind the timed ones.  The one
 JSON line on standard output holds decoded tokens per second at the default batch (8), the same
 at batch 1 and 64 under "points", a 2,048-token prefill under "prefill" and the decode step's
 share of the HBM roofline under "roofline": of the published peaks (8 TB/s, 2.5 PFLOP/s), and under "measured_peak" /
@@ -145,12 +148,68 @@ def decode_run(engine, rng, vocab, batch, steps, warmup, prompt_len, tag, sampli
     return tokens / elapsed, elapsed / steps * 1e3, [c + steps / 2.0 for c in contexts]
 
 
+def median_run(runs):
+    """Of several (tokens/s, ms a step, contexts) the one with the median time a step."""
+    ordered = sorted(runs, key=lambda r: r[1])
+    return ordered[len(ordered) // 2]
+
+
+def short_kernel_name(name):
+    """`void (anonymous namespace)::kernel<1, 2>(Args, int)` -> `kernel<1, 2>`; a mangled name -> its function's name;
+    a kernel of the GEMM library -> `gemm_library_MT<its tile>`."""
+    import re
+    tile = re.search(r"Cijk_.*?(MT\d+x\d+x\d+)", name)
+    if tile:
+        return "gemm_library_" + tile.group(1)
+    mangled = re.match(r"_ZN?(?:12_GLOBAL__N_1)?(\d+)", name)
+    if mangled:
+        return name[mangled.end():mangled.end() + int(mangled.group(1))]
+    name = name.replace("void ", "").replace("(anonymous namespace)::", "")
+    depth = 0
+    for i, ch in enumerate(name):
+        depth += ch == "<"
+        depth -= ch == ">"
+        if ch == "(" and depth == 0:
+            return name[:i]
+    return name
+
+
+def kernel_breakdown(run_steps, steps, top=8):
+    """Device time by kernel over `steps` calls of `run_steps()` (one engine step each), in microseconds a step: the
+    `top` longest by name and the rest as "other".  What the reference prints as its BatchStats per phase
+    (rust/engine/src/runtime.rs:20-40) is per kernel here.  None when the profiler gives nothing."""
+    import torch
+    from torch.profiler import ProfilerActivity, profile
+    try:
+        with profile(activities=[ProfilerActivity.CUDA]) as prof:
+            for _ in range(steps):
+                run_steps()
+            torch.cuda.synchronize()
+        by_name = {}
+        for e in prof.key_averages():
+            if e.device_time_total > 0:
+                name = short_kernel_name(e.key)
+                by_name[name] = by_name.get(name, 0.0) + e.device_time_total / steps
+        rows = list(by_name.items())
+    except Exception as exc:                                   # a profiler that cannot attach must not cost the run its line
+        print(f"[bench] no kernel breakdown: {exc}", file=sys.stderr, flush=True)
+        return None
+    rows.sort(key=lambda r: -r[1])
+    out = {name: round(us, 1) for name, us in rows[:top]}
+    if rows[top:]:
+        out["other"] = round(sum(us for _, us in rows[top:]), 1)
+    out["total"] = round(sum(us for _, us in rows), 1)
+    return out or None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=248, help="timed decode steps (with the warm-up: 256 generated tokens a request)")
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--repeats", type=int, default=3, help="timed runs of each headline figure; the median is reported")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the profiled steps that give the per-kernel times")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="8b",
                     help="layer sizes: Llama-3.1-8B (the default, the headline configuration), Llama-3.2-1B or Llama-3.1-70B")
     ap.add_argument("--layers", type=int, default=None,
@@ -242,12 +301,16 @@ def main():
     def share(result, model=cfg, layers=args.layers):
         return decode_step_bytes(model, layers, result[2]) / (result[1] * 1e-3) / 1e9 / HBM_PEAK_GBS
 
-    results = {}
+    results, all_runs = {}, {}
+    repeats = max(1, args.repeats)
     for batch in batches:
-        results[batch] = decode_run(engine, rng, vocab, batch, steps, warmup, args.prompt_len, f"b{batch}",
-                                    sampling=dict(SAMPLED, repetition_penalty=1.1, logprobs=5) if args.sampled else None)
-        print(f"[bench] decode batch {batch}: {results[batch][0]:.1f} tok/s, {results[batch][1]:.3f} ms/step",
-              file=sys.stderr, flush=True)
+        runs = [decode_run(engine, rng, vocab, batch, steps, warmup, args.prompt_len, f"b{batch}r{r}",
+                           sampling=dict(SAMPLED, repetition_penalty=1.1, logprobs=5) if args.sampled else None)
+                for r in range(repeats)]
+        results[batch] = median_run(runs)
+        all_runs[batch] = [round(r[1], 4) for r in runs]
+        print(f"[bench] decode batch {batch}: {results[batch][0]:.1f} tok/s, {results[batch][1]:.3f} ms/step (median of "
+              f"{', '.join(f'{r[1]:.3f}' for r in runs)})", file=sys.stderr, flush=True)
 
     value, ms_per_step, contexts = results[args.batch]
     step_bytes = decode_step_bytes(cfg, args.layers, contexts)
@@ -264,16 +327,54 @@ def main():
                    "kv_dtype": "bf16", "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "timed_runs": repeats, "value_of_runs": "median",
+        "runs_ms_per_step": {f"decode_b{b}": v for b, v in all_runs.items()},
     }
     if not args.no_points:
         line["points"] = {"decode_b1": round(results[1][0], 2), "decode_b64": round(results[64][0], 2)}
         for b in (1, 64):
             line["points"][f"decode_b{b}_hbm_frac"] = round(share(results[b]), 4)
-        best = prefill_run()
+        prefills = sorted(prefill_run() for _ in range(repeats))
+        best = prefills[len(prefills) // 2]
         flops = prefill_flops(cfg, args.layers, PREFILL_TOKENS)
         line["prefill"] = {"value": round(PREFILL_TOKENS / best, 1), "tokens": PREFILL_TOKENS, "ms": round(best * 1e3, 3),
-                           "frac": round(flops / best / (MFMA_PEAK_TFLOPS["bf16"] * 1e12), 4)}
-        print(f"[bench] prefill {PREFILL_TOKENS} tokens: {best * 1e3:.2f} ms", file=sys.stderr, flush=True)
+                           "frac": round(flops / best / (MFMA_PEAK_TFLOPS["bf16"] * 1e12), 4),
+                           "achieved_tflops": round(flops / best / 1e12, 1), "peak_tflops": MFMA_PEAK_TFLOPS["bf16"]}
+        line["runs_ms_per_step"]["prefill"] = [round(p * 1e3, 3) for p in prefills]
+        print(f"[bench] prefill {PREFILL_TOKENS} tokens: {best * 1e3:.2f} ms (median of "
+              f"{', '.join(f'{p * 1e3:.2f}' for p in prefills)})", file=sys.stderr, flush=True)
+        if not args.no_kernels:
+            line["kernels"] = {}
+            prompts = iter(range(10 ** 6))
+
+            def one_prompt():
+                engine.add_request(f"profiled-{next(prompts)}", rng.integers(0, vocab, PREFILL_TOKENS).tolist(),
+                                   SamplingParams(max_tokens=1, ignore_eos=True))
+                while engine.has_unfinished():
+                    engine.step()
+
+            one_prompt()
+            found = kernel_breakdown(one_prompt, 2)
+            if found:
+                line["kernels"]["prefill_us"] = found
+            # a decode batch of its own for the profiled steps: prompts, a few steps untimed, then five profiled steps
+            names = [f"profiled-b{args.batch}-{i}" for i in range(args.batch)]
+            for name in names:
+                engine.add_request(name, rng.integers(0, vocab, args.prompt_len).tolist(),
+                                   SamplingParams(max_tokens=64, ignore_eos=True))
+            got = {n: 0 for n in names}
+            while min(got.values()) < 4:
+                for ev in engine.step():
+                    got[ev.request_id] += 1
+            found = kernel_breakdown(engine.step, 5)
+            if found:
+                line["kernels"][f"decode_b{args.batch}_us"] = found
+            for name in names:
+                engine.abort_request(name)
+            while engine.has_unfinished():
+                engine.step()
+            for phase, found in line["kernels"].items():
+                print(f"[bench] kernels, {phase}: " + ", ".join(f"{k} {v}" for k, v in found.items()), file=sys.stderr, flush=True)
     if further:
         # the same batch with sampled tokens (temperature 0.8, top-k 50, top-p 0.9): what the sampler adds to a step
         result = decode_run(engine, rng, vocab, args.batch, min(steps, 64), 2, args.prompt_len, "sampled",

@@ -43,6 +43,18 @@ def test_the_line_of_a_short_run():
     assert (roofline["bound"], roofline["peak"], roofline["unit"]) == ("hbm", 8000.0, "GB/s")
     assert abs(roofline["frac"] - roofline["achieved"] / roofline["peak"]) < 1e-3 and 0 < roofline["frac"] < 1
     assert line["points"]["decode_b1"] > 0 and line["points"]["decode_b64"] > line["points"]["decode_b1"]
+    # every headline figure is the median of three timed runs, all of them listed
+    runs = line["runs_ms_per_step"]
+    assert line["timed_runs"] == 3 and set(runs) == {"decode_b1", "decode_b8", "decode_b64", "prefill"}
+    assert all(len(v) == 3 for v in runs.values())
+    assert sorted(runs["decode_b8"])[1] == line["ms_per_step"] and sorted(runs["prefill"])[1] == line["prefill"]["ms"]
+    flops = line["prefill"]["achieved_tflops"] * 1e12
+    assert abs(flops / (line["prefill"]["peak_tflops"] * 1e12) - line["prefill"]["frac"]) < 1e-3
+    # the kernels a step's time goes to, in microseconds a step: they add up to most of the step
+    for phase, ms in (("decode_b8_us", line["ms_per_step"]), ("prefill_us", line["prefill"]["ms"])):
+        kernels = line["kernels"][phase]
+        assert len(kernels) >= 4 and 0.5 * ms * 1e3 < kernels["total"] < 1.2 * ms * 1e3, (phase, kernels, ms)
+        assert abs(sum(v for k, v in kernels.items() if k != "total") - kernels["total"]) < 1.0
 
 
 @pytest.mark.gpu
