@@ -30,10 +30,11 @@ SIZES = {
     "1b": config(2, 2048, 32, 8, 64, 8192, 32.0, True),
     "70b": config(1, 8192, 64, 8, 128, 28672, 8.0, False),
 }
-# |engine - plain| <= tol * max|plain logit|.  Largest errors seen on the MI355X: float32 9.1e-6; bfloat16 1.6e-2 (8b),
+# |engine - plain| <= tol * max|plain logit|, and the engine's largest logit of every row is the plain implementation's
+# or within twice that of it.  Largest errors seen on the MI355X: float32 9.1e-6; bfloat16 1.5e-2 (8b),
 # 1.2e-2 (1b), 1.4e-2 (70b).  The plain kernels (one float32 chain per element, bfloat16 only where tensors are stored)
 # are as far from the plain implementation at these widths (1.3e-2 at the 8b sizes): the distance is the storage type's.
-TOL = {"float32": 2e-5, "bfloat16": 3e-2}
+TOL = {"float32": 2e-5, "bfloat16": 2e-2}
 LADDER = [10] * 40 + [14] * 16 + [18] * 7 + [22]          # 64 requests; 64, 24, 8 and 1 of them are left as they end
 
 
@@ -99,6 +100,12 @@ def test_steps_at_benchmark_sizes(cases, tmp_path, name, dtype):
             assert err.max() <= TOL[dtype], (f"{name} {dtype} {family}: request {rid}: error {err.max():.3e} of the largest logit at "
                                              f"position {int(err.argmax())}; first position over the limit: "
                                              f"{int(np.argmax(err > TOL[dtype]))}")
+            # the greedy token of every row: the plain implementation's, or one that nearly ties with it there
+            chosen, best = logits.argmax(axis=1), want.argmax(axis=1)
+            rows = np.arange(len(want))
+            gap = (want[rows, best] - want[rows, chosen]) / np.abs(want).max(axis=1)
+            assert gap.max() <= 2 * TOL[dtype], (f"{name} {dtype} {family}: request {rid}: position {int(gap.argmax())} takes token "
+                                                 f"{int(chosen[gap.argmax()])}, the plain implementation {int(best[gap.argmax()])}")
         runner.cache.check_invariants()
         assert all(pool.available == pool.num_pages for pool in runner.cache.pools)
     print(f"observed errors {name} {dtype}: " + ", ".join(f"{k} {v:.2e}" for k, v in worst.items()))

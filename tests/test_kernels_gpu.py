@@ -208,6 +208,30 @@ def test_linear_bf16_library_path(library_ops, ref, M, N, K, mode, bias):
     _linear_case(library_ops, ref, torch.bfloat16, M, N, K, mode, bias, branch_rounded=(mode == "add" and not bias))
 
 
+@pytest.mark.parametrize("K,row_counts", [(4096, (1, 8, 16, 64)), (2048, (1,)), (8192, (1,))])
+def test_vocabulary_projection_at_the_benchmark_sizes(ops, library_ops, K, row_counts):
+    """The product that ends every step, at the sizes the benchmark times: 128,256 outputs in float32 from bfloat16
+    operands, widths of the 8B, 1B and 70B shapes; up to 16 rows on this library's kernel, 64 rows through the GEMM
+    library as the engine sends them.  Against the float64 product; a row gives the same bits alone and in a batch."""
+    N = 128256
+    g = gen(46)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    x = torch.randn(max(row_counts), K, generator=g).to(torch.bfloat16)
+    w64, wg = w.double(), w.to(DEV)
+    want = x.double() @ w64.T
+    mag = (x.double().abs() @ w64.abs().T).max().item()
+    alone = None
+    for M in row_counts:
+        which = library_ops if M > 16 else ops
+        out = which.linear(x[:M].to(DEV), wg, torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV))
+        close(out, want[:M], 1e-6, 4e-7 * mag + 1e-6, f"vocabulary projection M{M} K{K}")
+        assert torch.equal(out.argmax(-1).cpu(), want[:M].argmax(-1)), f"M{M} K{K}: another largest logit"
+        if M == 1:
+            alone = out[0].clone()
+        elif M <= 16:
+            assert torch.equal(out[0], alone), f"M{M} K{K}: row 0 differs from the row computed alone"
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("rows,width", [(1, 64), (13, 4099), (300, 4096)])
 def test_add_residual(ops, dtype, rows, width):

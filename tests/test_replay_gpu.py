@@ -97,6 +97,26 @@ def test_replay(models, tmp_path, name, dtype, family):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("page_size", [4, 12, 32, 64, 128])
+@pytest.mark.parametrize("name,family", [("A", "mixed"), ("D", "mixed"), ("D", "last32"), ("E", "portions")])
+def test_replay_at_other_page_sizes(models, tmp_path, name, family, page_size, dtype):
+    """Pages of 4 to 128 tokens, among them a size that is no power of two: the matrix-core attention kernels take pages
+    of 8 to 64 tokens, the others run the plain kernels; pages are still used again."""
+    folder, cfg, requests, plain = models[name]
+    steps = {"last32": tt.last_tokens_one_by_one, "portions": tt.portions,
+             "mixed": lambda r: tt.mixed(r, seed=6, refeed=[rid for rid, t in r.items() if len(t) >= 60][:1])}[family](requests)
+    steps = tt.number(steps)
+    runner = make_runner(folder, dtype, page_size, tt.live_tokens_bound(steps, round_to=max(64, page_size)))
+    handed_out = tt.record_allocations(runner.cache)
+    got = tt.run_in_process(runner, steps, cfg["vocab_size"], str(tmp_path))
+    check(got, plain, dtype, f"{name} {dtype} {family} page {page_size}")
+    runner.cache.check_invariants()
+    assert all(pool.available == pool.num_pages for pool in runner.cache.pools), "pages were lost"
+    for pages in handed_out:
+        assert len(pages) > len(set(pages)), "the trace was meant to use pages again"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["B", "D"])
 def test_single_rows_beside_portions_take_the_decode_kernel(models, tmp_path, monkeypatch, name, dtype):
     """In a step that mixes portions of prompts with single tokens the single rows go to the decode kernel once their
