@@ -94,7 +94,7 @@ def test_sampled_generation_is_reproducible(dtype):
             agree += token == plain_llama.device_sample(logits, 0.8, 0, 1.0, 4242, draw)
             seq.append(token)
         # one of the 24 may differ: the draw is the largest of logit / T + noise, and where the two largest of those
-        # lie closer together than the engine's logits are to the plain ones (bfloat16: about 1e-2 of the largest
+        # lie closer together than the engine's float32 logits are to the plain float64 ones (about 1e-6 of the largest
         # logit) either may come out; from then on the comparison follows the engine's token, so one miss stays one
         assert agree >= 23, f"{24 - agree} of 24 sampled tokens are not what the plain sampler draws from the plain logits"
     assert make_engine("B", dtype).generate(prompts, SamplingParams(max_tokens=24, temperature=0.8, seed=1)) != a

@@ -212,7 +212,8 @@ def test_linear_bf16_library_path(library_ops, ref, M, N, K, mode, bias):
 def test_vocabulary_projection_at_the_benchmark_sizes(ops, library_ops, K, row_counts):
     """The product that ends every step, at the sizes the benchmark times: 128,256 outputs in float32 from bfloat16
     operands, widths of the 8B, 1B and 70B shapes; up to 16 rows on this library's kernel, 64 rows through the GEMM
-    library as the engine sends them.  Against the float64 product; a row gives the same bits alone and in a batch."""
+    library as the engine sends them.  Against the float64 product.  On this library's kernel a row's bits do not depend
+    on the rows beside it; up to 8 rows (one tile shape) they are also the bits of the row computed alone."""
     N = 128256
     g = gen(46)
     w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
@@ -229,7 +230,12 @@ def test_vocabulary_projection_at_the_benchmark_sizes(ops, library_ops, K, row_c
         if M == 1:
             alone = out[0].clone()
         elif M <= 16:
-            assert torch.equal(out[0], alone), f"M{M} K{K}: row 0 differs from the row computed alone"
+            if M <= 8:
+                assert torch.equal(out[0], alone), f"M{M} K{K}: row 0 differs from the row computed alone"
+            others = x[:M].clone()
+            others[1:] = torch.randn(M - 1, K, generator=g).to(torch.bfloat16)
+            again = which.linear(others.to(DEV), wg, torch.empty((M, N), dtype=torch.float32, device=DEV))
+            assert torch.equal(again[0], out[0]), f"M{M} K{K}: row 0 depends on the rows beside it"
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
