@@ -27,7 +27,8 @@ class GroupSpec:
     """Cache-owning run entries with one need.  `window` None: all keys are kept."""
     entries: tuple
     kv_heads: int
-    head_dim: int
+    k_dim: int
+    v_dim: int
     window: Optional[int]
     page_size: int
 
@@ -80,22 +81,56 @@ class CacheManager:
         self._idle.pop(node, None)
         req.shared.append(node)
 
-    def adopt_prefix(self, req_id, tokens: Sequence[int]) -> int:
+    def _known_prefix(self, tokens: Sequence[int], with_state: bool) -> List[PrefixNode]:
+        """The nodes of the longest known prefix of `tokens` that leaves at least the last token to be computed; where
+        the model keeps state per request (`with_state`), only as far as a node that holds a copy of that state."""
+        if self.prefix is None:
+            return []
+        nodes = self.prefix.match(tokens, (len(tokens) - 1) // self.prefix.page_size)
+        if with_state:
+            while nodes and nodes[-1].state is None:
+                nodes.pop()
+        return nodes
+
+    def probe_prefix(self, tokens: Sequence[int], with_state: bool = False):
+        """(pages, idle) of what `adopt_prefix` would take over: how many pages, and how many of them no request holds
+        at the moment (those count among `free_pages` until they are adopted).  Changes nothing."""
+        nodes = self._known_prefix(tokens, with_state)
+        return len(nodes), sum(1 for n in nodes if n.holders == 0)
+
+    def adopt_prefix(self, req_id, tokens: Sequence[int], with_state: bool = False):
         """For a request that holds nothing yet: puts the pages of the longest known prefix of `tokens` into its block
         tables, leaving at least the last token to be computed.  Returns the number of tokens taken over; the request
-        holds them as if it had committed them."""
+        holds them as if it had committed them.  `with_state`: only as far as a page behind which a copy of the
+        model's per-request state was kept (`keep_state`); then (tokens, that copy) is returned."""
         req = self._get(req_id)
         if self.prefix is None or req.length != 0 or any(req.tables):
-            return 0
+            return (0, None) if with_state else 0
         page_size = self.prefix.page_size
-        for node in self.prefix.match(tokens, (len(tokens) - 1) // page_size):
+        for node in self._known_prefix(tokens, with_state):
             for g, page in enumerate(node.pages):
                 self.pools[g].retain(page)
                 req.tables[g].append(page)
             self._hold(req, node)
         req.length = len(req.shared) * page_size
         self.prefix_hit_tokens += req.length
+        if with_state:
+            return req.length, (req.shared[-1].state if req.shared else None)
         return req.length
+
+    def keep_state(self, req_id, tokens: int, state) -> bool:
+        """Keeps `state` (whatever the caller copies a request's fixed-size state into) with the known prefix that ends
+        behind the request's first `tokens` tokens, which must be whole pages that `remember_prefix` has entered.
+        False: there is no such prefix (the prefix cache is off, or the page was not entered)."""
+        req = self._get(req_id)
+        if self.prefix is None or tokens <= 0 or tokens % self.prefix.page_size != 0:
+            return False
+        index = tokens // self.prefix.page_size - 1
+        if index >= len(req.shared):
+            return False
+        if req.shared[index].state is None:
+            req.shared[index].state = state
+        return True
 
     def share_pages(self, src_id, dst_id, tokens: int) -> int:
         """For a request `dst_id` that holds nothing yet: puts the full pages of `src_id` that lie wholly below `tokens`
@@ -107,6 +142,9 @@ class CacheManager:
         src, dst = self._get(src_id), self._get(dst_id)
         if dst.length != 0 or any(dst.tables) or self.prefix is not None:
             return 0
+        if not self.groups:                     # a model without keys and values: nothing to share but the position
+            dst.length = min(src.length, int(tokens))
+            return dst.length
         if any(g.window is not None for g in self.groups) or len({g.page_size for g in self.groups}) != 1:
             return 0
         page_size = self.groups[0].page_size

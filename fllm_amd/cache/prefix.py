@@ -13,7 +13,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 
 
 class PrefixNode:
-    __slots__ = ("parent", "key", "pages", "children", "holders")
+    __slots__ = ("parent", "key", "pages", "children", "holders", "state")
 
     def __init__(self, parent: Optional["PrefixNode"], key: Tuple[int, ...], pages: Tuple[int, ...]):
         self.parent = parent
@@ -21,6 +21,7 @@ class PrefixNode:
         self.pages = pages               # one page a cache group
         self.children: Dict[Tuple[int, ...], "PrefixNode"] = {}
         self.holders = 0                 # live requests whose block tables name these pages
+        self.state = None                # for models with per-request state: a copy of it as it was behind this page
 
 
 class PrefixIndex:

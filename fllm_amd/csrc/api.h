@@ -146,6 +146,7 @@ int fllm_argmax(const float *logits, int32_t *out, int rows, int vocab, hipStrea
 // until the process ends; the call allocates nothing and needs no fllm_set_device_workspace.  At most 256 rows
 // (more are refused; any vocabulary).  Same result as fllm_argmax.  All calls on one GPU share that GPU's array:
 // calls that overlap on one GPU (different streams, different threads) race; calls in stream order do not.  The
+// entry point takes any stream and checks nothing of this: keeping one call in flight a device is the caller's duty.  The
 // first call on a device looks up the array's address (once per device); make it outside a graph capture.
 int fllm_argmax_static(const float *logits, int32_t *out, int rows, int vocab, hipStream_t stream);
 

@@ -528,14 +528,13 @@ attn_tile32_kernel(AttnArgs p) {
                 __hip_atomic_store(mine + (db * 16 + i) * kThreads + threadIdx.x, o[db][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(mine + DB * 16 * kThreads + threadIdx.x, m_run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(mine + (DB * 16 + 1) * kThreads + threadIdx.x, l_run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_s_waitcnt(0);      // the part has arrived before it is counted
+        parts_published();      // the part has arrived before it is counted
         __syncthreads();
         int *counter = p.counters + group;
         if (threadIdx.x == 0) s_seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (s_seen != parts - 1) return;
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        parts_visible();
         if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
         float m_all = -INFINITY;
         for (int i0 = 0; i0 < parts; i0 += 8) {       // eight loads in flight at a time
@@ -732,14 +731,13 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
     // The split that arrives last adds the parts up, in the order of the splits: the result does not depend on
     // which one that is.  Its partial sums have arrived before it is counted.
     __shared__ int s_seen;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);
+    parts_published();
     __syncthreads();
     int *counter = p.counters + ((size_t)row * p.kv_heads + kvh) * qtiles + qtile;
     if (threadIdx.x == 0) s_seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (s_seen != live_splits - 1) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    parts_visible();
     if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
     // The parts are read eight at a time, all loads of a group asked for before the first is used.  The first group's
     // values are kept: up to eight parts (the usual case) cost one round trip to memory, not one for the largest

@@ -42,6 +42,34 @@ int fllm_option_dual_k(void);
 constexpr size_t kWorkspaceCounterBytes = 64 * 1024;      // plans.h counts with the same number (checked where both are seen)
 bool fllm_device_workspace(void **base, size_t *bytes);
 
+// Workgroups of one launch that meet in the workspace: a workgroup leaves its partial results there (relaxed
+// agent-scope atomic stores, or the sc0 sc1 buffer stores of linear_skinny.hip), calls parts_published() and then
+// counts itself with a relaxed agent-scope add; the workgroup that counts last calls parts_visible() and reads the
+// parts of all (relaxed agent-scope atomic loads, sc0 sc1 buffer loads).
+//
+// FLLM_HANDOVER_SCOPE "agent" makes the two calls the release and acquire fences at agent scope that the HIP memory
+// model asks for.  On gfx950 such a release writes the die's whole L2 back and the acquire drops it, and a decode
+// step of 8 rows at the Llama-3.1-8B sizes takes 4.76 ms instead of 3.73 (measured; its K-sliced products and split
+// contexts hand over 200 times a step), 3.41 instead of 3.34 ms at one row.  The default is therefore the form that
+// rests on what the hardware does with these particular accesses, which is all the hand-over needs:
+//   1. every part is written by stores with the sc1 bit (what an agent-scope atomic store is on gfx950): they are
+//      written through to the memory side, which all eight dies share, and do not stay in the writer's L2;
+//   2. s_waitcnt vmcnt(0) returns when those stores have been acknowledged from there;
+//   3. only then is the counter's add issued, an atomic performed at the same memory-side point;
+//   4. the reader issues its loads after the add that told it it is last has returned, and they carry sc1 too: they
+//      are served from the memory side, not from a line its own die's L2 may still hold.
+// A compiler fence at workgroup scope keeps the compiler from moving the stores, the add and the loads across each other.
+// What this depends on and a change of hardware or compiler could break: that sc1 stores are acknowledged only once
+// visible to the other dies (2), and that agent-scope atomic loads never hit in a die's L2 (4).
+#ifndef FLLM_HANDOVER_SCOPE
+#define FLLM_HANDOVER_SCOPE "workgroup"
+#endif
+__device__ __forceinline__ void parts_published() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, FLLM_HANDOVER_SCOPE);
+    __builtin_amdgcn_s_waitcnt(0);
+}
+__device__ __forceinline__ void parts_visible() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, FLLM_HANDOVER_SCOPE); }
+
 #define FLLM_REQUIRE(cond, ...)            \
     do {                                   \
         if (!(cond)) {                     \

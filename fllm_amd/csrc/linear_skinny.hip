@@ -511,13 +511,12 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
                     // Every access to the workspace goes to the device's point of coherence by itself (agent-scope
                     // atomics), so no cache has to be written back or dropped: it is enough that the wave's partial
                     // sums have arrived there before the item is counted.
-                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                    __builtin_amdgcn_s_waitcnt(0);
+                    parts_published();
                     int seen = 0;
                     if (lane == 0) seen = __hip_atomic_fetch_add(a.counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     seen = __shfl(seen, 0, kWave);
                     if (seen != S - 1) break;       // another workgroup finishes this tile
-                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                    parts_visible();
                     if (lane == 0) __hip_atomic_store(a.counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
                     if (!owner || m >= M) break;
 #pragma unroll
@@ -702,13 +701,12 @@ skinny_wide_kernel(SkinnyArgs a) {
                 if (mt == MT - 1) {
                     // every access to the workspace goes to the device's point of coherence by itself: it is enough
                     // that the wave's partial sums have arrived there before the tile is counted
-                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                    __builtin_amdgcn_s_waitcnt(0);
+                    parts_published();
                     int seen = 0;
                     if (lane == 0) seen = __hip_atomic_fetch_add(a.counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     seen = __shfl(seen, 0, kWave);
                     if (seen == S - 1) {        // the last slice of this tile: add the parts in slice order
-                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                        parts_visible();
                         if (lane == 0) __hip_atomic_store(a.counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
                         for (int mt2 = 0; mt2 < MT; mt2++) {
@@ -884,9 +882,7 @@ skinny_slab_kernel(SkinnyArgs a, int cells_off) {
     // squares in the workspace, counts the tile, and whoever counts last adds the S parts in slice order and runs
     // the epilogue.  None of this may make the wave wait, or the weights stop streaming, so it is spread over three
     // item ends: the parts are sent at the end of their own item; the tile is counted at the end of the item after,
-    // when the loads that were asked for since have pushed the parts' stores out of the queue of outstanding memory
-    // operations (they complete in the order of their issue, so waiting until only the newest loads are outstanding
-    // is waiting for nothing that is not needed anyway); the count is looked at one item later still.
+    // behind a release fence (the stores have had an item's time by then); the count is looked at one item later still.
     const bool owner = EPI == EPI_SWIGLU ? g < 2 : true;      // 8-output tiles: lanes g < 2 hold gate rows, g >= 2 the up rows
     const __amdgpu_buffer_rsrc_t wsb = workspace_buffer(a.ws);
     int sent_tile = -1;                     // parts sent, tile not counted yet
@@ -907,7 +903,7 @@ skinny_slab_kernel(SkinnyArgs a, int cells_off) {
         const int tile = counted_tile;
         counted_tile = -1;
         if (__shfl(counted_raw, 0, kWave) != S - 1) return;      // another workgroup finishes this tile
-        asm volatile("" ::: "memory");
+        parts_visible();
         if (lane == 0) __hip_atomic_store(a.counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
         // one block of 16 rows after the other (few registers: this runs in the middle of the stream of weights); the
         // parts of two slices are asked for before the first is added, and they are added in slice order
@@ -947,14 +943,12 @@ skinny_slab_kernel(SkinnyArgs a, int cells_off) {
             finish_rows(tile, mt, s, ss);
         }
     };
-    // `drained`: nothing more will be asked for, wait for everything; otherwise wait until only the loads that the
-    // item just finished asked for are outstanding (8 a chunk, up to two chunks): the parts were sent before them.
-    auto count = [&](bool drained) __attribute__((always_inline)) {
+    // The parts were sent at the end of the item before: by now their stores have had an item's time to complete, and
+    // the release fence waits for whatever of them has not (loads and stores of a wave may complete out of their order
+    // of issue with respect to each other, so counting outstanding operations cannot stand in for it).
+    auto count = [&]() __attribute__((always_inline)) {
         if (sent_tile < 0) return;
-        if (drained) __builtin_amdgcn_s_waitcnt(0);
-        else if (nchunks >= 2) __builtin_amdgcn_s_waitcnt(0x4F70);      // vmcnt(16), nothing else waited for
-        else __builtin_amdgcn_s_waitcnt(0x0F78);                        // vmcnt(8)
-        asm volatile("" ::: "memory");
+        parts_published();
         if (lane == 0) counted_raw = __hip_atomic_fetch_add(a.counters + sent_tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         counted_tile = sent_tile;
         sent_tile = -1;
@@ -979,7 +973,7 @@ skinny_slab_kernel(SkinnyArgs a, int cells_off) {
         item++;
         if (S > 1) {
             look();
-            count(false);
+            count();
         }
         f32x4_t s[MT][RT];
         float ss[MT];
@@ -1024,7 +1018,7 @@ skinny_slab_kernel(SkinnyArgs a, int cells_off) {
     }
     if (S > 1) {       // what the last items left to do
         look();
-        count(true);
+        count();
         look();
     }
 }

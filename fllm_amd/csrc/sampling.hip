@@ -111,12 +111,12 @@ __device__ __forceinline__ bool meet_and_merge(Pick best, int row, int part, int
     if (threadIdx.x == 0) {
         __hip_atomic_store(partial_v + (size_t)row * parts + part, best.value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(partial_i + (size_t)row * parts + part, best.index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_s_waitcnt(0);      // the part has arrived before it is counted
+        parts_published();      // the part has arrived before it is counted
         cells.word = __hip_atomic_fetch_add(counters + row, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (cells.word != parts - 1) return false;
+    parts_visible();
     if (threadIdx.x == 0) __hip_atomic_store(counters + row, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     Pick mine = {-INFINITY, kNone};
     if ((int)threadIdx.x < parts) {

@@ -17,11 +17,11 @@ import torch
 class CacheBinding:
     """Where one run entry keeps its keys and values (and state)."""
     group: int                              # index into StepContext.tables
-    k_pages: Optional[torch.Tensor]         # [pages, kv_heads, page_size, head_dim]
-    v_pages: Optional[torch.Tensor]         # [pages, kv_heads, head_dim, page_size]
+    k_pages: Optional[torch.Tensor]         # [pages, kv_heads, page_size, k_dim]
+    v_pages: Optional[torch.Tensor]         # [pages, kv_heads, v_dim, page_size]
     page_size: int
     writes: bool                            # False: the entry reads another entry's cache
-    state: Optional[torch.Tensor] = None    # [max_requests, *shape], for mixers with fixed-size state
+    state: object = None                    # [max_requests, *shape], or name -> such a tensor: mixers with fixed-size state
 
 
 @dataclass

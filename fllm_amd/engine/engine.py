@@ -111,15 +111,14 @@ class Engine:
         self.max_model_len = self.runner.max_context
         if prefix_cache is None:
             prefix_cache = os.environ.get("FLLM_PREFIX_CACHE", "").strip().lower() in ("1", "on", "true", "yes")
-        if prefix_cache and self.runner.model.has_state:
-            raise ValueError("the prefix cache shares keys and values only: a model whose layers keep state of their own per "
-                             "request cannot start a request behind a shared prefix")
         self.scheduler = Scheduler(
             SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=max_batched_tokens, decode_first=decode_first,
                             watermark_pages=kv_watermark_blocks, max_partial_prefills=max_num_partial_prefills,
                             long_prefill_threshold=long_prefill_token_threshold,
                             max_long_partial_prefills=max_long_partial_prefills, preemption=preemption_mode,
-                            policy=scheduling_policy, prefix_cache=bool(prefix_cache)),
+                            policy=scheduling_policy, prefix_cache=bool(prefix_cache),
+                            state_checkpoints=self.runner.model.has_state,
+                            portion_multiple=self.runner.model.portion_multiple),
             self.runner.cache, self.max_model_len)
         self.sampler = Sampler(self.runner.rt)
         if eos_token_ids is None:
@@ -152,14 +151,14 @@ class Engine:
                 raise ValueError(f"token id {t} is outside [0, {self.runner.vocab_size})")
         sid = self._next_seq
         self._next_seq += sampling.n
-        self.scheduler.add(Sequence(seq_id=sid, req_id=request_id, tokens=prompt, prompt_len=len(prompt), sampling=sampling))
+        self.scheduler.add(Sequence(seq_id=sid, req_id=request_id, tokens=prompt, prompt_len=len(prompt), sampling=sampling,
+                                    forks=sampling.n > 1))
         self._requests[request_id] = list(range(sid, sid + sampling.n))
         if sampling.n > 1:
             # the other answers join when the first one's prompt is in the cache, and start behind its full pages
-            # (not where layers keep state of their own per request: pages can be shared, such state cannot)
-            source = None if self.runner.model.has_state else sid
+            # (where layers keep state of their own per request: behind the place where that state was copied)
             self._followers[sid] = [Sequence(seq_id=sid + k, req_id=request_id, tokens=list(prompt), prompt_len=len(prompt),
-                                             sampling=sampling.for_choice(k), choice=k, fork_from=source)
+                                             sampling=sampling.for_choice(k), choice=k, fork_from=sid)
                                     for k in range(1, sampling.n)]
         self._deadlines.pop(request_id, None)
         if sampling.timeout_secs is not None:
@@ -229,6 +228,8 @@ class Engine:
             token = seqs[sid].tokens[-1]
             entries.append(StepEntry(sid, [token], [0], carry=row_of[sid] if token == PENDING else None))
             sampled.append(sid)
+        for sid, state in self.scheduler.take_restores():         # requests that start behind a shared beginning
+            self.runner.restore_state(sid, state)
         try:
             logits = self.runner.step(entries, previous_tokens=earlier.tokens if earlier is not None else None)
         except Exception:
@@ -258,6 +259,8 @@ class Engine:
         # token is read), the prompt portions count as computed.
         for sid, _, count in plan.prefill:
             self.scheduler.commit_chunk(sid, count)
+        for sid, tokens in self.scheduler.take_checkpoints():     # copied now, on the step's stream, before the next step
+            self.scheduler.keep_checkpoint(sid, tokens, self.runner.snapshot_state(sid))
         for sid in sampled:
             seq = seqs[sid]
             launched.at.append(len(seq.tokens))

@@ -1,6 +1,7 @@
 """A model put together from parts as its `ModelSpec` says, and the plan of its caches."""
 from __future__ import annotations
 
+import math
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
@@ -44,11 +45,16 @@ class Model:
         """Groups cache-owning run entries by what they need; entries that read another entry's
         cache join that entry's group."""
         self.kv_needs: List[Optional[KVNeed]] = []
-        self.state_needs: List[Optional[StateNeed]] = []
+        self.state_needs: List[object] = []          # per run entry None, a StateNeed, or a dict of named ones
+        self.portion_multiple = 1                    # a prompt is cut on multiples of every mixer's own multiple
         for entry in self.spec.run_order:
             mixer = self.blocks[entry.layer].mixer
             self.kv_needs.append(mixer.cache_need())
             self.state_needs.append(mixer.state_need())
+            multiple = int(getattr(mixer, "portion_multiple", lambda: 1)())
+            if multiple <= 0:
+                raise ValueError(f"run entry of layer {entry.layer}: portion_multiple() must be positive, is {multiple}")
+            self.portion_multiple = self.portion_multiple * multiple // math.gcd(self.portion_multiple, multiple)
         keys: List[Tuple] = []
         self.entry_group: List[Optional[int]] = [None] * len(self.spec.run_order)
         self.entry_index: List[Optional[int]] = [None] * len(self.spec.run_order)   # index inside the group's tensors
@@ -60,14 +66,14 @@ class Model:
             if entry.reads_cache_of is not None:
                 src = entry.reads_cache_of
                 src_need = self.kv_needs[src]
-                if src_need is None or (src_need.kv_heads, src_need.head_dim) != (need.kv_heads, need.head_dim):
+                if src_need is None or (src_need.kv_heads, src_need.k_dim, src_need.v_dim) != (need.kv_heads, need.k_dim, need.v_dim):
                     raise ValueError(f"run entry {i} cannot read the cache of entry {src}: different geometry")
                 if src_need.window is not None and (need.window is None or need.window > src_need.window):
                     raise ValueError(f"run entry {i} needs more keys than entry {src} keeps")
                 self.entry_group[i] = self.entry_group[src]
                 self.entry_index[i] = self.entry_index[src]
                 continue
-            key = (need.kv_heads, need.head_dim, need.window)
+            key = (need.kv_heads, need.k_dim, need.v_dim, need.window)
             if key not in keys:
                 keys.append(key)
                 members.append([])
@@ -79,13 +85,13 @@ class Model:
         self.group_members = members
 
     def group_specs(self, page_size: int) -> List[GroupSpec]:
-        return [GroupSpec(entries=tuple(m), kv_heads=k[0], head_dim=k[1], window=k[2], page_size=page_size)
+        return [GroupSpec(entries=tuple(m), kv_heads=k[0], k_dim=k[1], v_dim=k[2], window=k[3], page_size=page_size)
                 for k, m in zip(self.group_keys, self.group_members)]
 
     def cache_bytes_per_page(self, page_size: int) -> List[int]:
         """Bytes a page of each group costs (keys and values of all the group's run entries)."""
         elem = torch.empty((), dtype=self.rt.dtype).element_size()
-        return [2 * len(m) * k[0] * k[1] * page_size * elem for k, m in zip(self.group_keys, self.group_members)]
+        return [len(m) * k[0] * (k[1] + k[2]) * page_size * elem for k, m in zip(self.group_keys, self.group_members)]
 
     def allocate_caches(self, page_size: int, pages_per_group: Sequence[int], max_requests: int,
                         max_step_tokens: Optional[int] = None) -> CacheManager:
@@ -99,17 +105,17 @@ class Model:
         self.null_pages = [int(n) for n in pages_per_group]
         self.k_store, self.v_store = [], []
         for g, n in zip(groups, pages_per_group):
-            self.k_store.append(torch.zeros((len(g.entries), n + 1, g.kv_heads, page_size, g.head_dim),
+            self.k_store.append(torch.zeros((len(g.entries), n + 1, g.kv_heads, page_size, g.k_dim),
                                             dtype=rt.dtype, device=rt.device))
-            self.v_store.append(torch.zeros((len(g.entries), n + 1, g.kv_heads, g.head_dim, page_size),
+            self.v_store.append(torch.zeros((len(g.entries), n + 1, g.kv_heads, g.v_dim, page_size),
                                             dtype=rt.dtype, device=rt.device))
         self.bindings = []
         for i, entry in enumerate(self.spec.run_order):
             g = self.entry_group[i]
-            state = None
-            if self.state_needs[i] is not None:
-                need = self.state_needs[i]
-                state = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=rt.device)
+            arena = lambda need: torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=rt.device)
+            need = self.state_needs[i]
+            state = None if need is None else ({name: arena(n) for name, n in need.items()} if isinstance(need, dict)
+                                               else arena(need))
             if g is None:
                 self.bindings.append(CacheBinding(group=-1, k_pages=None, v_pages=None, page_size=page_size,
                                                   writes=False, state=state))
@@ -119,11 +125,32 @@ class Model:
                                               page_size=page_size, writes=entry.reads_cache_of is None, state=state))
         return CacheManager(groups, list(pages_per_group), max_requests, max_step_tokens=max_step_tokens)
 
+    def state_arenas(self):
+        """(run entry, name or None, arena [max_requests, *shape]) of every state tensor the model keeps."""
+        for index, binding in enumerate(self.bindings):
+            if isinstance(binding.state, dict):
+                for name, arena in binding.state.items():
+                    yield index, name, arena
+            elif binding.state is not None:
+                yield index, None, binding.state
+
     def clear_state(self, slot: int) -> None:
         """Zeros the fixed-size state of every run entry in one request slot (a request's first step)."""
-        for binding in self.bindings:
-            if binding.state is not None:
-                binding.state[slot].zero_()
+        for _, _, arena in self.state_arenas():
+            arena[slot].zero_()
+
+    def snapshot_state(self, slot: int):
+        """A copy of everything the model keeps in one request slot, for `restore_state`
+        (the reference's sequence state snapshots, rust/engine/src/rust_decoder/state_api.rs:14-80)."""
+        return [(index, name, arena[slot].clone()) for index, name, arena in self.state_arenas()]
+
+    def restore_state(self, slot: int, snapshot) -> None:
+        """Puts a snapshot (of this model, of any slot) into `slot`."""
+        arenas = {(index, name): arena for index, name, arena in self.state_arenas()}
+        if sorted(arenas, key=str) != sorted(((i, n) for i, n, _ in snapshot), key=str):
+            raise ValueError("the snapshot is not one of this model's state")
+        for index, name, saved in snapshot:
+            arenas[(index, name)][slot].copy_(saved)
 
     @property
     def has_state(self) -> bool:
@@ -143,7 +170,7 @@ class Model:
                 continue
             # the norm that reads the residual stream after this block: the first one of the block that runs next,
             # where that block says which it is (a block may let its last sum prepare it)
-            ctx.next_norm = getattr(self.blocks[order[index + 1].layer], "mixer_norm", None) if index + 1 < len(order) else None
+            ctx.next_norm = self.blocks[order[index + 1].layer].first_norm() if index + 1 < len(order) else None
             if getattr(block, "takes_pending", False):
                 pending = block.forward(ctx, x, binding, pending)
             else:

@@ -203,6 +203,21 @@ class ModelRunner:
             start = self.cache.length(e.req_id) if self.cache.has_request(e.req_id) else 0
             if start + n > self.max_context:
                 raise StepError(f"request {e.req_id!r} would hold {start + n} tokens, the context is {self.max_context}")
+            multiple = self.model.portion_multiple
+            if multiple > 1 and n > 1 and start % multiple != 0:
+                raise StepError(f"request {e.req_id!r} brings a portion of {n} tokens at position {start}: portions of this "
+                                f"model begin on multiples of {multiple}")
+
+    # ---- per-request state of fixed size ----------------------------------------------------
+    def snapshot_state(self, req_id):
+        """A copy of everything the model's layers keep for `req_id` outside the pages, as it is after the steps
+        launched so far (the reference's rust/engine/src/rust_decoder/state_api.rs:84-120); [] for a model without."""
+        return self.model.snapshot_state(self.cache.slot(req_id))
+
+    def restore_state(self, req_id, snapshot) -> None:
+        """Puts a snapshot of this model into the slot of `req_id` (a request that the cache manager knows: its length
+        says how many tokens the state stands for, state_api.rs:122-160).  The next step of the request goes on there."""
+        self.model.restore_state(self.cache.slot(req_id), snapshot)
 
     def step(self, entries: Sequence[StepEntry], previous_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Runs the entries as one batch and returns float32 logits [wanted, vocab] on the device,

@@ -21,12 +21,22 @@ run out.  Behaviour follows the reference's scheduler (rust/engine/src/scheduler
               admitted starts behind the longest prefix of its tokens that is known there (the reference's prefix cache,
               rust/engine/src/mem/prefix_cache.rs:414-520); a preempted sequence finds its own pages again this way
               unless the room was needed
+  state       for a model whose layers keep state of fixed size per request (`state_checkpoints`): such state cannot be
+              shared by pointing at pages, it has to be copied at the position where two requests part.  A prompt whose
+              beginning may serve others (the prefix cache is on, or further answers to it wait) is cut so that one
+              portion ends on its last page boundary; the engine copies the state there (`take_checkpoints`), and a
+              request that starts behind shared pages gets the copy put into its slot before its first step
+              (`take_restores`).  The reference does the same with its state checkpoints (scheduler.rs:383-388, :536-560,
+              :598-612; rust/engine/src/runtime.rs:979-1011)
+  multiples   `portion_multiple`: a portion that does not end its prompt ends on a multiple of so many tokens (mixers
+              whose kernels work on fixed chunks of positions ask for it)
 
 The scheduler does the cache bookkeeping (reserve at admission and before a decode row); the
 step function commits what it ran.
 """
 from __future__ import annotations
 
+import math
 from collections import deque
 from dataclasses import dataclass, field
 from typing import Deque, Dict, List, Optional, Tuple
@@ -47,6 +57,8 @@ class SchedulerConfig:
     preemption: str = "recompute"
     policy: str = "fcfs"                    # fcfs | priority (smaller `SamplingParams.priority` first)
     prefix_cache: bool = False              # requests start behind the prefix of their tokens that the cache knows
+    state_checkpoints: bool = False         # the model keeps state per request: shared beginnings need a copy of it
+    portion_multiple: int = 1               # portions that do not end a prompt end on multiples of this
 
     def __post_init__(self):
         if self.max_num_seqs <= 0 or self.max_num_batched_tokens <= 0:
@@ -55,6 +67,8 @@ class SchedulerConfig:
             raise ValueError("preemption must be 'recompute' or 'none'")
         if self.policy not in ("fcfs", "priority"):
             raise ValueError("scheduling policy must be 'fcfs' or 'priority'")
+        if self.portion_multiple <= 0:
+            raise ValueError("portion_multiple must be positive")
 
 
 @dataclass
@@ -73,6 +87,8 @@ class Sequence:
     seen: Optional[object] = None           # counts of the tokens so far, kept by the engine for requests with penalties
     choice: int = 0                         # which of the answers to its request's prompt this sequence is
     fork_from: Optional[int] = None         # a sequence that begins with the same tokens (the first answer, for the others)
+    forks: bool = False                     # further answers will start behind this sequence's prompt
+    checkpoint_at: Optional[int] = None     # tokens after which the model's per-request state is to be copied
 
     @property
     def output_len(self) -> int:
@@ -100,6 +116,11 @@ class Scheduler:
         self._arrivals = 0
         if cfg.prefix_cache:
             cache.enable_prefix_cache()
+        # per-request state of the model (`state_checkpoints`): copies the engine took, by sequence: (tokens, copy);
+        # what it has to copy after the step it is about to run, and what it has to put back before it
+        self.state_copies: Dict[int, Tuple[int, object]] = {}
+        self._checkpoints: List[Tuple[int, int]] = []
+        self._restores: List[Tuple[int, object]] = []
 
     # ---- queue ----------------------------------------------------------------------------
     def add(self, seq: Sequence) -> None:
@@ -117,30 +138,96 @@ class Scheduler:
         seq = self.sequences[sid]
         if len(seq.tokens) > self.max_model_len:
             return False
+        with_state = self.cfg.state_checkpoints
         self.cache.add_request(sid)
-        reused = self.cache.adopt_prefix(sid, seq.tokens) if self.cfg.prefix_cache else self._share_with_source(seq)
         total = len(seq.tokens) + 1
-        missing = self.cache.pages_missing(sid, total)
         watermark = self.cfg.watermark_pages if self.running else 0
-        if any(m + watermark > self.cache.free_pages(g) for g, m in enumerate(missing)):
-            self.cache.free_request(sid)
-            return False
+        state = None
+        if self.cfg.prefix_cache:
+            # looked up without taking hold: a request that does not fit yet leaves the index as it was (its hits are
+            # not counted, the pages it would use keep their place in the order in which unused ones are given up)
+            known, idle = self.cache.probe_prefix(seq.tokens, with_state)
+            missing = self.cache.pages_missing(sid, total)
+            if any(m - known + watermark > self.cache.free_pages(g) - idle for g, m in enumerate(missing)):
+                self.cache.free_request(sid)
+                return False
+            reused = self.cache.adopt_prefix(sid, seq.tokens, with_state)
+            if with_state:
+                reused, state = reused
+        else:
+            reused, state = self._share_with_source(seq)
+            missing = self.cache.pages_missing(sid, total)
+            if any(m + watermark > self.cache.free_pages(g) for g, m in enumerate(missing)):
+                self.cache.free_request(sid)
+                return False
         self.cache.reserve(sid, total)
         seq.num_computed = reused
+        if state is not None:
+            self._restores.append((sid, state))
+        seq.checkpoint_at = None
+        if with_state and (self.cfg.prefix_cache or seq.forks):
+            unit = self._checkpoint_unit()
+            boundary = (len(seq.tokens) - 1) // unit * unit          # the last token is always computed
+            if unit > 0 and boundary > reused:
+                seq.checkpoint_at = boundary
         return True
 
-    def _share_with_source(self, seq: Sequence) -> int:
+    def _checkpoint_unit(self) -> int:
+        """State is copied where pages end and portions may end; 0: the page sizes of the groups differ."""
+        sizes = {g.page_size for g in self.cache.groups}
+        if len(sizes) > 1:
+            return 0
+        page, multiple = (sizes.pop() if sizes else 1), self.cfg.portion_multiple
+        return page * multiple // math.gcd(page, multiple)
+
+    def _share_with_source(self, seq: Sequence) -> Tuple[int, object]:
         """A further answer to a prompt starts behind the full pages of the first answer's sequence, as far as their
         tokens are the same, if that one still runs (the reference forks the block table and copies the last block,
-        rust/engine/src/runtime.rs:437-460; here the last, partly filled page is computed again instead)."""
+        rust/engine/src/runtime.rs:437-460; here the last, partly filled page is computed again instead).  Where the
+        model keeps state per request, only as far as the place where that state was copied.  Returns the tokens shared
+        and the copy of the state to start from (None without)."""
         source = self.sequences.get(seq.fork_from) if seq.fork_from is not None else None
         if source is None or source.seq_id not in self.running:
-            return 0
+            return 0, None
         limit = min(len(seq.tokens) - 1, len(source.tokens), source.num_computed)     # the last token is always computed
+        state = None
+        if self.cfg.state_checkpoints:
+            tokens, state = self.state_copies.get(source.seq_id, (0, None))
+            if state is None or tokens > limit:
+                return 0, None
+            limit = tokens
         same = limit if seq.tokens[:limit] == source.tokens[:limit] else 0
         while same < limit and seq.tokens[same] == source.tokens[same]:
             same += 1
-        return self.cache.share_pages(source.seq_id, seq.seq_id, same)
+        if state is not None and same != limit:
+            return 0, None
+        shared = self.cache.share_pages(source.seq_id, seq.seq_id, same)
+        if state is not None and shared != limit:
+            if shared:                                   # cannot be: the copy was taken where the source's pages end
+                raise RuntimeError(f"{shared} tokens shared, the state was copied behind {limit}")
+            return 0, None
+        return shared, state
+
+    def take_checkpoints(self) -> List[Tuple[int, int]]:
+        """(sequence, tokens) of the sequences whose portion of the step just committed ended where their state is to be
+        copied: the caller copies it now, before the next step, and hands it to `keep_checkpoint`."""
+        due, self._checkpoints = self._checkpoints, []
+        return due
+
+    def keep_checkpoint(self, sid: int, tokens: int, state) -> None:
+        seq = self.sequences.get(sid)
+        if seq is None:
+            return
+        if seq.forks:
+            self.state_copies[sid] = (tokens, state)
+        if self.cfg.prefix_cache:
+            self.cache.keep_state(sid, tokens, state)
+
+    def take_restores(self) -> List[Tuple[int, object]]:
+        """(sequence, copy of a state) for the sequences admitted since the last call that start behind a shared
+        beginning: the caller puts the copy into the sequence's slot before it runs the step."""
+        due, self._restores = self._restores, []
+        return [(sid, state) for sid, state in due if sid in self.running]
 
     # ---- order ----------------------------------------------------------------------------
     def _key(self, sid: int) -> Tuple[int, int]:
@@ -206,6 +293,8 @@ class Scheduler:
         seq.num_computed = 0
         seq.prefill_target = len(seq.tokens)
         seq.state = "waiting"
+        seq.checkpoint_at = None
+        self.state_copies.pop(sid, None)
         self.running.remove(sid)
         self.waiting.appendleft(sid)
 
@@ -234,6 +323,12 @@ class Scheduler:
             if is_long and long_prefills >= max(1, self.cfg.max_long_partial_prefills):
                 continue
             chunk = min(todo, prefill_budget)
+            if seq.checkpoint_at is not None and seq.num_computed < seq.checkpoint_at < seq.num_computed + chunk:
+                chunk = seq.checkpoint_at - seq.num_computed     # state can only be copied between two portions
+            if self.cfg.portion_multiple > 1 and chunk < todo:
+                chunk -= (seq.num_computed + chunk) % self.cfg.portion_multiple
+                if chunk <= 0:
+                    continue                                     # no room for a whole multiple in this step
             if not self.cache.can_reserve(sid, seq.num_computed + chunk):
                 break
             self.cache.reserve(sid, seq.num_computed + chunk)
@@ -270,8 +365,13 @@ class Scheduler:
 
     # ---- after the step -------------------------------------------------------------------
     def commit_chunk(self, sid: int, count: int) -> None:
-        self.sequences[sid].num_computed += count
+        seq = self.sequences[sid]
+        seq.num_computed += count
         self._remember(sid)
+        if seq.checkpoint_at is not None and seq.num_computed >= seq.checkpoint_at:
+            if seq.num_computed == seq.checkpoint_at:
+                self._checkpoints.append((sid, seq.checkpoint_at))
+            seq.checkpoint_at = None
 
     def commit_decode(self, sid: int) -> None:
         seq = self.sequences[sid]
@@ -283,6 +383,7 @@ class Scheduler:
             self._remember(sid)
         seq = self.sequences.pop(sid)
         seq.state = "finished"
+        self.state_copies.pop(sid, None)
         if sid in self.running:
             self.running.remove(sid)
         if sid in self.waiting:

@@ -41,6 +41,9 @@ class PagedAttention(Mixer):
             raise ValueError(f"head count {self.heads} is not a multiple of key/value head count {self.kv_heads}")
         if self.window is not None and self.window <= 0:
             raise ValueError("an attention window must be positive")
+        if spec.get("value_head_dim") not in (None, self.head_dim):
+            raise ValueError(f"this attention's kernels read keys and values of one width: values of "
+                             f"{spec.get('value_head_dim')} beside keys of {self.head_dim} need a mixer of their own")
         position = spec.get("position")
         self.position = None
         if position is not None:
@@ -84,7 +87,7 @@ class PagedAttention(Mixer):
         return torch.tensor([h * head_dim + j for h in range(heads) for j in one], dtype=torch.long)
 
     def cache_need(self):
-        return KVNeed(self.kv_heads, self.head_dim, self.window)
+        return KVNeed(self.kv_heads, self.head_dim, self.head_dim, self.window)     # keys and values of one width: what the kernels take
 
     def forward(self, ctx, h, residual, binding, branch=None):
         rt, ops = self.rt, self.rt.ops

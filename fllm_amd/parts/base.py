@@ -16,9 +16,12 @@ Roles and their interfaces:
                 (0: lanes l and l + dims/2, 1: lanes 2l and 2l + 1).  Optional: `score_slopes`, a float32 device
                 vector [heads]: every score gets score_slopes[head] * (key position - row position) added (an
                 encoding that biases scores by distance; such layers run the plain attention kernel).
-  mixer         cache_need() / state_need() say what the cache manager must keep for it;
+  mixer         cache_need() / state_need() say what the cache manager must keep for it (keys and values of widths
+                of their own; one state tensor or several named ones); portion_multiple() on which multiples of
+                tokens a prompt may be cut;
                 forward(ctx, h[R,H], residual_f32[R,H], binding) adds its output to `residual`.
-                State of fixed size: `binding.state[slot]` belongs to one live request (slot = ctx.seg_slots[s] on the
+                State of fixed size: `binding.state[slot]` (`binding.state[name][slot]` when the mixer named several)
+                belongs to one live request (slot = ctx.seg_slots[s] on the
                 host, ctx.slots[s] on the device).  The step function hands it over filled with zeros at the first
                 step of a request it has not seen before (also one that was freed and is fed again from position 0),
                 touches it at no other time, and runs a request's rows in position order, `seg_pos_start[s]` being the
@@ -60,11 +63,19 @@ INIT_BIAS = "bias"         # N(0, 0.02)
 
 @dataclass(frozen=True)
 class KVNeed:
-    """Keys and values of `kv_heads` heads of `head_dim` per token; `window` keys back (the
-    token itself included) or all of them when None."""
+    """Per token, keys of `kv_heads` heads of `k_dim` values and values of as many heads of `v_dim` (`k_dim` when left
+    out; 0: the mixer caches keys alone); `window` keys back (the token itself included) or all of them when None.
+    The pages are shaped from both widths; what a mixer's kernels can read is the mixer's matter."""
     kv_heads: int
-    head_dim: int
+    k_dim: int
+    v_dim: Optional[int] = None
     window: Optional[int] = None
+
+    def __post_init__(self):
+        if self.v_dim is None:
+            object.__setattr__(self, "v_dim", self.k_dim)
+        if self.kv_heads <= 0 or self.k_dim <= 0 or self.v_dim < 0:
+            raise ValueError(f"a cache of {self.kv_heads} heads with keys of {self.k_dim} and values of {self.v_dim}")
 
 
 @dataclass(frozen=True)
@@ -94,8 +105,16 @@ class Mixer(Part):
     def cache_need(self) -> Optional[KVNeed]:
         return None
 
-    def state_need(self) -> Optional[StateNeed]:
+    def state_need(self):
+        """None, one `StateNeed` (then `binding.state[slot]` is the request's tensor), or a dict of named ones of any
+        shapes and types (then `binding.state[name][slot]`)."""
         return None
+
+    def portion_multiple(self) -> int:
+        """A portion of a prompt that does not end the prompt must hold a multiple of this many tokens (a mixer whose
+        kernels work on fixed chunks of positions); 1: any cut.  The scheduler cuts accordingly and the step function
+        refuses other cuts."""
+        return 1
 
     def forward(self, ctx, h, residual, binding) -> None:
         raise NotImplementedError
@@ -122,6 +141,11 @@ class Norm(Part):
 
 class Block(Part):
     role = "block"
+
+    def first_norm(self):
+        """The norm this block applies to the residual stream first, if whoever ends the block before may prepare it
+        (`ctx.next_norm`); None: the block says nothing, and nothing is prepared for it."""
+        return None
 
 
 def take_prepared(ctx, norm, residual):

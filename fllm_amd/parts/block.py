@@ -14,6 +14,9 @@ class PreNormBlock(Block):
         self.mixer_norm = norms["mixer"]
         self.feed_forward_norm = norms["feed_forward"] if feed_forward is not None else None
 
+    def first_norm(self):
+        return self.mixer_norm
+
     takes_pending = True     # forward accepts a branch that the block before has not added yet, and may hand one on
 
     def forward(self, ctx, residual, binding, pending=None):

@@ -51,6 +51,10 @@ class Sampler:
         the rows' `last_row` points into."""
         if all(r is None for r in rows):
             return logits
+        pointing = [r.last_row for r in rows if r is not None and r.last_row >= 0]
+        if pointing and (last_tokens is None or max(pointing) >= last_tokens.numel()):
+            raise ValueError(f"rows name their newest token at index {max(pointing)} of `last_tokens`, which "
+                             + ("was not given" if last_tokens is None else f"holds {last_tokens.numel()} tokens"))
         from .adjust import pack
         packed, sections = pack(rows)
         if logits.is_cuda:

@@ -31,11 +31,11 @@ def test_pool_is_lifo_and_counts_references():
 
 
 def full(page_size=4):
-    return GroupSpec(entries=(0, 1), kv_heads=2, head_dim=16, window=None, page_size=page_size)
+    return GroupSpec(entries=(0, 1), kv_heads=2, k_dim=16, v_dim=16, window=None, page_size=page_size)
 
 
 def windowed(window, page_size=4):
-    return GroupSpec(entries=(2,), kv_heads=2, head_dim=16, window=window, page_size=page_size)
+    return GroupSpec(entries=(2,), kv_heads=2, k_dim=16, v_dim=16, window=window, page_size=page_size)
 
 
 def test_reserve_commit_free():

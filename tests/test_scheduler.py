@@ -8,7 +8,7 @@ from fllm_amd.sampling import SamplingParams
 
 
 def make(pages, max_seqs=4, budget=8, page_size=4, **kw):
-    cache = CacheManager([GroupSpec(entries=(0,), kv_heads=1, head_dim=16, window=None, page_size=page_size)], [pages],
+    cache = CacheManager([GroupSpec(entries=(0,), kv_heads=1, k_dim=16, v_dim=16, window=None, page_size=page_size)], [pages],
                          max_requests=max_seqs)
     return Scheduler(SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=budget, **kw), cache, max_model_len=64), cache
 
@@ -277,4 +277,71 @@ def test_a_preempted_sequence_finds_its_pages_again():
     s.add(Sequence(seq_id=2, req_id="r2", tokens=list(range(200, 222)), prompt_len=22, sampling=SamplingParams(max_tokens=1)))
     plan = s.schedule()
     assert plan.prefill == [(2, 0, 16)] and cache.cached_pages() == 0 and cache.free_pages() == 0
+    cache.check_invariants()
+
+
+def test_a_blocked_request_leaves_the_prefix_index_as_it_was():
+    """The request at the head of the queue is tried at every call while it does not fit: its hits are counted once, when
+    it is admitted, and the pages it would take over keep their place among the unused ones."""
+    s, cache = make(pages=8, budget=32, prefix_cache=True)
+    for sid, first in ((0, 0), (1, 100)):           # two prompts of 9 tokens leave two known pages each
+        s.add(Sequence(seq_id=sid, req_id=f"r{sid}", tokens=list(range(first, first + 9)), prompt_len=9,
+                       sampling=SamplingParams(max_tokens=1)))
+        while s.has_work():
+            run_step(s, cache, s.schedule())
+            for done in [d for d, q in s.sequences.items() if q.remaining() <= 0]:
+                s.finish(done)
+    assert cache.cached_pages() == 4 and cache.prefix_hit_tokens == 0
+    order = list(cache._idle)
+    s.add(Sequence(seq_id=2, req_id="r2", tokens=list(range(300, 320)), prompt_len=20, sampling=SamplingParams(max_tokens=12)))
+    run_step(s, cache, s.schedule())                # 6 pages held: the unused prefixes of request 0 had to go
+    assert cache.pools[0].available == 0 and cache.free_pages() == 2
+    order = list(cache._idle)
+    assert len(order) == 2
+    # the first prompt of request 1 again, and more: it needs 2 known + 3 further pages, 2 + 0 are there
+    s.add(Sequence(seq_id=3, req_id="r3", tokens=list(range(100, 117)), prompt_len=17, sampling=SamplingParams(max_tokens=1)))
+    for _ in range(3):
+        plan = s.schedule()
+        assert plan.prefill == [] and plan.decode == [2] and 3 in s.waiting
+        assert cache.prefix_hit_tokens == 0 and list(cache._idle) == order
+        run_step(s, cache, plan)
+    cache.check_invariants()
+    s.finish(2)
+    plan = s.schedule()
+    assert plan.prefill == [(3, 8, 9)] and cache.prefix_hit_tokens == 8
+    cache.check_invariants()
+
+
+def test_portions_end_on_multiples_and_at_the_place_where_state_is_copied():
+    """scheduler.rs:383-388: a portion ends exactly on the boundary that is worth keeping; and a model may ask for
+    portions that begin on multiples of some number of tokens."""
+    s, cache = make(pages=32, budget=10, page_size=4, portion_multiple=3)
+    s.add(seq(0, 29))
+    cuts = []
+    while s.sequences[0].num_computed < 29:
+        plan = s.schedule()
+        cuts += plan.prefill
+        run_step(s, cache, plan)
+    assert cuts == [(0, 0, 9), (0, 9, 9), (0, 18, 9), (0, 27, 2)]          # multiples of 3 until the prompt ends
+    s, cache = make(pages=32, budget=10, page_size=4, portion_multiple=3, state_checkpoints=True, prefix_cache=True)
+    s.add(seq(0, 29))
+    cuts, copied = [], []
+    while s.sequences[0].num_computed < 29:
+        plan = s.schedule()
+        cuts += plan.prefill
+        run_step(s, cache, plan)
+        for sid, tokens in s.take_checkpoints():
+            copied.append((sid, tokens, s.sequences[sid].num_computed))
+            s.keep_checkpoint(sid, tokens, "copy of the state behind 24 tokens")
+    # pages of 4 and multiples of 3: the state is copied behind 24 tokens, the last place below the last token that is both
+    assert cuts == [(0, 0, 9), (0, 9, 9), (0, 18, 6), (0, 24, 5)] and copied == [(0, 24, 24)]
+    s.finish(0)
+    s.add(Sequence(seq_id=1, req_id="r1", tokens=list(range(26)) + [77, 78], prompt_len=28, sampling=SamplingParams(max_tokens=1)))
+    plan = s.schedule()
+    assert plan.prefill == [(1, 24, 4)] and s.take_restores() == [(1, "copy of the state behind 24 tokens")]
+    # a prompt that shares fewer pages than the copy stands for starts from nothing: pages alone are not enough
+    s.add(Sequence(seq_id=2, req_id="r2", tokens=list(range(20)) + [90] * 8, prompt_len=28, sampling=SamplingParams(max_tokens=1)))
+    run_step(s, cache, plan)
+    plan = s.schedule()
+    assert (2, 0, 9) in plan.prefill and s.take_restores() == []
     cache.check_invariants()

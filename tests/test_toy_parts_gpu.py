@@ -78,8 +78,8 @@ register_architecture(Architecture("toy-state", ("ToyStateModel",), lambda c: c,
 TOY = {"model_type": "toy-state", "hidden_size": 64, "vocab_size": 200, "decay": 0.75}
 
 
-def plain_toy(w, ids):
-    """The same model, whole sequence, float64."""
+def plain_toy(w, ids, first_mixer=None):
+    """The same model, whole sequence, float64.  `first_mixer`: the output [T, hidden] of another first mixer."""
     x = w["embed"][np.asarray(ids)]
     T = len(ids)
 
@@ -105,7 +105,7 @@ def plain_toy(w, ids):
     for t in range(T):
         state = 0.75 * state + h[t]
         out[t] = w["layers.0.mix.w"] @ state
-    x = mlp(x + out, 0)
+    x = mlp(x + (out if first_mixer is None else first_mixer), 0)
     x, first_cache = attention(x)
     x, _ = attention(x)
     x, _ = attention(x, kv_from=first_cache)
@@ -142,19 +142,149 @@ def test_toy_architecture_steps_through_the_engine():
     runner.cache.check_invariants()
 
 
-def test_toy_state_is_never_shared_between_requests():
-    """Pages can be shared between requests that begin alike, a mixer's own state cannot: the prefix cache is refused,
-    and further answers to a prompt run the prompt themselves."""
+def check_shared_beginnings(engine_options):
+    """Pages can be shared between requests that begin alike by naming them twice; a mixer's own state has to be copied
+    where the requests part.  Further answers to a prompt, and requests behind a known prefix, start from such a copy
+    and give the tokens of a request that ran alone.  (Also run on the CPU by tests/test_toy_state_cpu.py.)"""
     from fllm_amd import Engine, SamplingParams
-    options = dict(config=TOY, seed=5, dtype="float32", num_blocks=32, max_seqs=4, ctx=128, max_batched_tokens=16)
-    with pytest.raises(ValueError, match="state of their own"):
-        Engine(prefix_cache=True, **options)
+    options = dict(config=TOY, seed=5, dtype="float32", num_blocks=32, max_seqs=4, ctx=128, max_batched_tokens=24)
+    options.update(engine_options)
     engine = Engine(**options)
     prompt = tc.random_ids(40, 200, 3)
     alone = engine.generate([prompt], SamplingParams(max_tokens=6))[0]
     rows = engine.stats.prefill_rows
+    assert rows == 40
+    # three answers: the first one's prompt is cut at its last page boundary (32), the state is copied there, and the
+    # other two compute the 8 tokens behind it
     assert engine.generate([prompt], SamplingParams(max_tokens=6, n=3)) == [[alone] * 3]
-    assert engine.stats.prefill_rows - rows == 3 * 40
+    assert engine.stats.prefill_rows - rows == 40 + 2 * 8
+    engine.runner.cache.check_invariants()
+    # sampled answers differ from each other and are what each seed gives alone
+    params = SamplingParams(max_tokens=6, n=3, temperature=0.9, seed=11)
+    together = engine.generate([prompt], params)[0]
+    from dataclasses import replace
+    single = [Engine(**options).generate([prompt], replace(params.for_choice(k), n=1))[0] for k in range(3)]
+    assert together == single and len({tuple(t) for t in together}) > 1
+    # the prefix cache: a second request with the same beginning starts behind the copy
+    cached = Engine(prefix_cache=True, **options)
+    other = prompt[:35] + tc.random_ids(9, 200, 4)
+    want_other = engine.generate([other], SamplingParams(max_tokens=6))[0]
+    assert cached.generate([prompt], SamplingParams(max_tokens=6))[0] == alone
+    rows = cached.stats.prefill_rows
+    assert cached.generate([prompt], SamplingParams(max_tokens=6))[0] == alone
+    assert cached.stats.prefill_rows - rows == 8 and cached.stats.prefix_hit_tokens == 32
+    rows = cached.stats.prefill_rows
+    assert cached.generate([other], SamplingParams(max_tokens=6))[0] == want_other
+    assert cached.stats.prefill_rows - rows == 44 - 32          # pages without a copy of the state behind them do not count
+    assert cached.generate([prompt, other], SamplingParams(max_tokens=6, n=2)) == [[alone] * 2, [want_other] * 2]
+    cached.runner.cache.check_invariants()
+
+
+def test_toy_state_is_copied_where_requests_part():
+    check_shared_beginnings({})
+
+
+class RunningMean(Mixer):
+    """output_t = W mean(x_0 .. x_t): a sum and a count per request, two tensors of different shape and type.  It asks
+    for portions that begin on multiples of four tokens, as a mixer whose kernels work on chunks of positions would."""
+
+    @classmethod
+    def tensor_shapes(cls, spec):
+        return {"w": ((spec["hidden_size"], spec["hidden_size"]), INIT_MATRIX)}
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        self.hidden = spec["hidden_size"]
+        self.w = rt.matrix(weights["w"])
+
+    def state_need(self):
+        return {"sum": StateNeed((self.hidden,), torch.float32), "count": StateNeed((1,), torch.int32)}
+
+    def portion_multiple(self):
+        return 4
+
+    def forward(self, ctx, h, residual, binding):
+        row = 0
+        for rows, start, slot in zip(ctx.seg_rows, ctx.seg_pos_start, ctx.seg_slots):
+            total, count = binding.state["sum"][slot], binding.state["count"][slot]
+            assert rows == 1 or start % 4 == 0, "a portion that begins off a multiple of four"
+            assert int(count) == start, "the state is not the one left behind the position before"
+            for r in range(row, row + rows):
+                total.add_(h[r].float())
+                count.add_(1)
+                residual[r] += self.w.float() @ (total / count.float())
+            row += rows
+
+
+register_part("mixer", "running_mean", RunningMean)
+
+
+def mean_spec(cfg):
+    spec = toy_spec(cfg)
+    mixer = PartSpec("running_mean", {"hidden_size": cfg["hidden_size"]}, {"w": "layers.0.mix.w"})
+    first = LayerSpec(spec.layers[0].block, mixer, spec.layers[0].feed_forward, spec.layers[0].norms)
+    return ModelSpec("toy-mean", spec.hidden_size, spec.vocab_size, spec.max_position, spec.embedding,
+                     (first, spec.layers[1]), spec.run_order, spec.final_norm, spec.head)
+
+
+register_architecture(Architecture("toy-mean", ("ToyMeanModel",), lambda c: c, mean_spec))
+MEAN = {"model_type": "toy-mean", "hidden_size": 64, "vocab_size": 200, "decay": 0.0}
+
+
+def plain_mean_greedy(w, prompt, count):
+    """Greedy tokens of the running-mean model, whole sequences, float64: plain_toy with the mean in place of the
+    decaying sum (a decay of 1 and a division by the position)."""
+    def logits(ids):
+        x = w["embed"][np.asarray(ids)]
+        h = P.rms_norm(x, w["layers.0.n1"], 1e-5)
+        mean = np.cumsum(h, axis=0) / np.arange(1, len(ids) + 1)[:, None]
+        return mean @ w["layers.0.mix.w"].T
+    seq, out = list(prompt), []
+    for _ in range(count):
+        # the rest of the model is plain_toy's: run it with the first mixer's output swapped in
+        out.append(int(np.argmax(plain_toy(w, seq, first_mixer=logits(seq))[-1])))
+        seq.append(out[-1])
+    return out
+
+
+def check_two_state_tensors(engine_options):
+    from fllm_amd import Engine, SamplingParams
+    from fllm_amd.engine import StepError
+    options = dict(config=MEAN, seed=8, dtype="float32", num_blocks=32, max_seqs=4, ctx=128, max_batched_tokens=22)
+    options.update(engine_options)
+    engine = Engine(**options)
+    state = engine.runner.model.bindings[0].state
+    assert set(state) == {"sum", "count"} and state["sum"].shape == (4, 64) and state["count"].dtype == torch.int32
+    assert engine.runner.model.portion_multiple == 4 and engine.scheduler.cfg.portion_multiple == 4
+    _, spec = model_spec_from_config(MEAN)
+    w64 = tc.to_float64(random_tensors(spec, 8, torch.float32))
+    prompt = tc.random_ids(45, 200, 6)
+    want = plain_mean_greedy(w64, prompt, 5)
+    # a budget of 22 tokens a step: the scheduler cuts 20 + 12 (the page boundary at 32, where the state is copied) + 13
+    assert engine.generate([prompt], SamplingParams(max_tokens=5, n=3)) == [[want] * 3]
+    assert engine.stats.prefill_rows == 45 + 2 * 13
+    # snapshots hold both tensors; one of another model is refused
+    engine.add_request("r", prompt[:9], SamplingParams(max_tokens=2))
+    engine.step()
+    sid = engine.scheduler.running[0]
+    snapshot = engine.runner.snapshot_state(sid)
+    assert sorted(name for _, name, _ in snapshot) == ["count", "sum"] and int(snapshot[0][2] if snapshot[0][1] == "count" else snapshot[1][2]) == 9
+    with pytest.raises(ValueError, match="not one of this model"):
+        engine.runner.restore_state(sid, snapshot[:1])
+    engine.abort_request("r")
+    while engine.has_unfinished():
+        engine.step()
+    # the step function refuses a portion that begins off a multiple
+    runner = engine.runner
+    runner.step([StepEntry("p", prompt[:6], [])])
+    with pytest.raises(StepError, match="multiples of 4"):
+        runner.step([StepEntry("p", prompt[6:9], [])])
+    runner.step([StepEntry("p", prompt[6:7], [])])             # single tokens go anywhere
+    runner.free_request("p")
+
+
+def test_toy_mixer_with_two_state_tensors_and_portions_on_multiples():
+    check_two_state_tensors({})
 
 
 # ---------------------------------------------------------------------------------------------
