@@ -84,7 +84,21 @@ struct SkinnyArgs {
     // SCALED prologue
     const float *ssq_in;   // [M, ssq_count]
     int ssq_count;
+#ifdef FLLM_TIMELINE
+    unsigned long long *timeline;   // measurement builds only: [workgroup][8] times of the 100 MHz clock
+#endif
 };
+
+#ifdef FLLM_TIMELINE
+#define FLLM_STAMP(a, k)                                                                                   \
+    do {                                                                                                   \
+        if ((a).timeline != nullptr && threadIdx.x == 0) (a).timeline[blockIdx.x * 8 + (k)] = __builtin_amdgcn_s_memrealtime(); \
+    } while (0)
+#else
+#define FLLM_STAMP(a, k) \
+    do {                 \
+    } while (0)
+#endif
 
 __device__ __forceinline__ bf16x4_t pack4(f32x4_t v) {
     bf16x4_t p;
@@ -303,6 +317,7 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int r = lane & 15, g = lane >> 4;
     const int M = a.M, N = a.N, K = a.K, S = a.S;
+    FLLM_STAMP(a, 0);
     const int n_out = EPI == EPI_SWIGLU ? N / 2 : N;
     const int ntiles = (n_out + NT - 1) / NT;
     const int pitch = a.slice + 8;
@@ -341,9 +356,17 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
             if (row >= row_limit) row = row_limit - 1;
             if (TM == TM_GATEUP) row += (r >> 3) * n_out;
             const int kb = kr0 + l_j * KB;
+#ifdef FLLM_TILED_PROBE
+            // timing experiment only (wrong sums): the addresses a tile-major weight layout would give
+            const bf16_t *wp = a.w + (size_t)(tile0 + l_item * tstride) * NT * (TM == TM_GATEUP ? 2 : 1) * K + (size_t)((kw0 + l_j * KB) / KB) * (16 * KB) + lane * 8 - (size_t)0;
+            (void)row;
+#pragma unroll
+            for (int u = 0; u < U; u++) buf.w[u] = kb + u * 32 < kr1 ? *(const bf16x8_t *)(wp + u * 512) : zero8();
+#else
             const bf16_t *wp = a.w + (size_t)row * K + ks0 + kb;
 #pragma unroll
             for (int u = 0; u < U; u++) buf.w[u] = kb + u * 32 < kr1 ? *(const bf16x8_t *)(wp + u * 32) : zero8();
+#endif
             if (XD) {
                 const bf16_t *xp = (const bf16_t *)a.x + (size_t)xrow_i * a.ldx + ks0 + kb;
 #pragma unroll
@@ -454,6 +477,7 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
     int item = 0, j = 0;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
     const bf16_t *xrow = xs + xrow_i * pitch + kr0;
+    FLLM_STAMP(a, 1);
 
     auto step = [&](Block &buf) {
         bf16x8_t xf[U];
@@ -466,10 +490,17 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
 #pragma unroll
         for (int u = 0; u < U; u++) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(buf.w[u], xf[u], acc, 0, 0, 0);
         issue(buf);      // the block two ahead takes this one's registers
+#ifdef FLLM_TIMELINE
+        if (item == 0 && j == 0) {
+            asm volatile("" ::"v"(acc));      // the first block's products have been issued: its loads had arrived
+            FLLM_STAMP(a, 2);
+        }
+#endif
         if (++j < nbw) return;
         // the item is complete: the waves' sums meet in LDS; one wave (they take turns) adds them up and goes on
         // to the epilogue while the others start the next item
         j = 0;
+        if (item == my_items - 1) FLLM_STAMP(a, 3);
         red[wave * kWave + lane] = acc;
         acc = (f32x4_t){0.f, 0.f, 0.f, 0.f};
         __syncthreads();
@@ -562,6 +593,7 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
         step(b0);
         if (q + 1 < total) step(b1);
     }
+    FLLM_STAMP(a, 4);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1048,9 +1080,16 @@ ResidentPlan plan_resident(int M, int K, int ntiles, int rt, const Workspace &ws
     return fllm_plan::plan_resident(M, K, ntiles, rt, ws.bytes, ws.base != nullptr, x_direct, fllm_option_linear_slices());
 }
 
+#ifdef FLLM_TIMELINE
+unsigned long long *g_timeline = nullptr;
+#endif
+
 template <int PRO, int EPI, int TM, int WAVES, bool XD = false>
 int launch_resident_plan(SkinnyArgs a, const ResidentPlan &p, int ntiles, const Workspace &ws, hipStream_t stream) {
     constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
+#ifdef FLLM_TIMELINE
+    a.timeline = g_timeline;
+#endif
     a.S = p.S;
     a.slice = p.slice;
     a.ssq_off = (int)(p.stage + p.red);
@@ -1441,3 +1480,8 @@ extern "C" int fllm_scaled_qkv_rope_store(const void *xn, const float *ssq, int 
     FLLM_REQUIRE(rc != 1, "scaled_qkv_rope_store: shape M=%d K=%d does not fit the staging area", M, K);
     return rc;
 }
+
+#ifdef FLLM_TIMELINE
+// measurement builds only: device memory for [workgroups][8] clock readings of the next resident launches (null: off)
+extern "C" void fllm_set_timeline(unsigned long long *buffer) { g_timeline = buffer; }
+#endif
