@@ -471,3 +471,13 @@ def test_draws_follow_the_distribution_and_depend_on_seed_and_draw_only():
     assert np.all(np.abs(counts - p) < 0.03)
     assert P.device_sample(logits, 0.8, 0, 1.0, 5, 17) == P.device_sample(logits, 0.8, 0, 1.0, 5, 17)
     assert len({P.device_sample(logits, 1.5, 0, 1.0, s, 0) for s in range(40)}) > 1
+
+
+def test_the_smoke_run_carries_the_same_plain_model(weights):
+    """__graft_entry__.smoke() compares the engine with a plain model of its own, so that it runs from that file and the
+    package alone; here that one is held against this folder's."""
+    import __graft_entry__ as entry
+    cfg = entry.SMOKE_CONFIG
+    assert cfg == {k: v for k, v in tc.TINY_A.items()}
+    ids = tc.random_ids(23, cfg["vocab_size"], 5)
+    assert np.allclose(entry.plain_logits(cfg, weights["A"], ids), P.forward(cfg, weights["A"], ids), rtol=0, atol=1e-12)
