@@ -225,6 +225,8 @@ def main():
                     help="skip the points beyond the headline configuration: decoding at contexts of 8,192 and 32,768 tokens, and "
                          "the Llama-3.2-1B sizes (decoding at batch 1 and the mixed workload of 64 requests)")
     ap.add_argument("--no-ahead", action="store_true", help="every step waits for the tokens of the step before it")
+    ap.add_argument("--no-weight-tiles", action="store_true",
+                    help="without the tile-major copies of the output and down projection matrices that decode steps of up to 16 rows read")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run the 2,048-token prefill steps alone and print their time (for profiling); no JSON line")
     ap.add_argument("--prompt-tokens", type=int, default=PREFILL_TOKENS,
@@ -262,7 +264,8 @@ def main():
     t0 = time.time()
     engine = Engine(config=cfg, seed=0, dtype="bfloat16", device="cuda:0", ctx=most_context, max_seqs=max(batches),
                     max_batched_tokens=PREFILL_TOKENS, block_size=PAGE_SIZE, num_blocks=-(-need_tokens // PAGE_SIZE),
-                    decode_first=True, random_weights_on_device=True, ahead=not args.no_ahead)
+                    decode_first=True, random_weights_on_device=True, ahead=not args.no_ahead,
+                    decode_weight_tiles=False if args.no_weight_tiles else "auto")
     print(f"[bench] engine ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
     rng = np.random.default_rng(0)
     vocab = cfg["vocab_size"]

@@ -71,8 +71,26 @@ int fllm_norm_qkv_rope_store(const float *x, const float *norm_w, float eps, con
 // bfloat16 [M, N] and next_ssq [M, *tiles_out]: the sums of squares of out over the outputs of each tile (room for
 // M * N / 8 floats; *tiles_out, host memory, is set at the call).  The scaled forms are the norm forms above with
 // that pair in place of the float32 rows and the norm's weight.
+// w_tiles (may be null): the tile-major copy of w, see below.
 int fllm_linear_add_normed(const void *x, int ldx, const void *w, const float *bias, float *out, int M, int N, int K,
-                           const float *next_w, void *next_x, float *next_ssq, int *tiles_out, hipStream_t stream);
+                           const float *next_w, void *next_x, float *next_ssq, int *tiles_out, const void *w_tiles,
+                           hipStream_t stream);
+
+// Tile-major weights for the products of decode steps that add into the residual stream (output and down
+// projections).  A decode-shaped product feeds 16 weight rows x 32 columns to a matrix-core instruction, 16 bytes a
+// lane: from a row-major matrix that is 64 bytes of each of 16 rows a load, and the memory pipeline of a compute unit
+// looks up 64 cache lines for it; from the tile-major copy it is 1 KiB in a row, 8 lines, and the product of 8 or 16 rows
+// takes no longer than that of one (down projection of the 8B sizes: 29 -> 24 us at 8 rows).  The copy costs the
+// matrix's memory a second time, which a GPU with 288 GB affords; row-major stays for the products of 17 rows and more.
+//   fllm_weight_tiles_supported  1 where the kernels take tiles: N >= 16, K a multiple of 1,024
+//   fllm_weight_tiles_elements   bfloat16 elements of the copy: N rounded up to 16, times K
+//   fllm_tile_weights            writes the copy: [tile of 16 rows][block of 128 columns][k-step of 32][lane][8]
+//   fllm_linear_add_tiled        out += x w^T (+ bias), float32 out, 1..16 rows; with w_tiles where it can
+int fllm_weight_tiles_supported(int N, int K);
+size_t fllm_weight_tiles_elements(int N, int K);
+int fllm_tile_weights(const void *w, void *tiles, int N, int K, hipStream_t stream);
+int fllm_linear_add_tiled(const void *x, int ldx, const void *w, const void *w_tiles, const float *bias, float *out, int ldo,
+                          int M, int N, int K, hipStream_t stream);
 int fllm_scaled_gate_up_swiglu(const void *xn, const float *ssq, int ssq_count, float eps, const void *w_gate_up,
                                const float *bias, void *out, int M, int inter, int K, hipStream_t stream);
 int fllm_scaled_qkv_rope_store(const void *xn, const float *ssq, int ssq_count, float eps, const void *w_qkv, const float *bias,

@@ -59,6 +59,7 @@ struct SkinnyArgs {
     const float *norm_w;
     float eps;
     const bf16_t *w;
+    const bf16_t *w_tiles;   // the same matrix tile by tile (fllm_tile_weights), or null
     const float *bias;
     void *out;
     int ldo;
@@ -303,10 +304,11 @@ __device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], 
 // result does not depend on which workgroup came last.
 enum { TM_ROWS16 = 0, TM_DUALK = 1, TM_GATEUP = 2 };
 
-template <int PRO, int EPI, int TM, int WAVES, bool XD>
+template <int PRO, int EPI, int TM, int WAVES, bool XD, bool WT = false>
 __global__ void __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4, 4)))   // 16 waves a CU: 128 registers
 skinny_resident_kernel(SkinnyArgs a, int red_off) {
     static_assert(!XD || PRO == PRO_BF16, "activations straight from global memory: the bfloat16 prologue only");
+    static_assert(!WT || (TM == TM_ROWS16 && XD), "tile-major weights: 16-row tiles, one slice");
     constexpr int U = 4;                           // k-steps of 32 per block: four 16-byte loads per lane
     constexpr int KB = 32 * U;                     // K elements of one range per block
     constexpr int RB = 4;                          // rows of activations staged at a time (more would spill registers)
@@ -356,17 +358,17 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
             if (row >= row_limit) row = row_limit - 1;
             if (TM == TM_GATEUP) row += (r >> 3) * n_out;
             const int kb = kr0 + l_j * KB;
-#ifdef FLLM_TILED_PROBE
-            // timing experiment only (wrong sums): the addresses a tile-major weight layout would give
-            const bf16_t *wp = a.w + (size_t)(tile0 + l_item * tstride) * NT * (TM == TM_GATEUP ? 2 : 1) * K + (size_t)((kw0 + l_j * KB) / KB) * (16 * KB) + lane * 8 - (size_t)0;
-            (void)row;
+            if (WT) {
+                // tile-major weights (fllm_tile_weights): the 16 rows x 128 columns of a block lie together in the order
+                // the lanes take them, so a load instruction reads 1 KiB in a row instead of 64 bytes of each of 16 rows
+                const bf16_t *wp = a.w_tiles + (size_t)(tile0 + l_item * tstride) * 16 * K + (size_t)((kw0 + l_j * KB) / KB) * (16 * KB) + lane * 8;
 #pragma unroll
-            for (int u = 0; u < U; u++) buf.w[u] = kb + u * 32 < kr1 ? *(const bf16x8_t *)(wp + u * 512) : zero8();
-#else
-            const bf16_t *wp = a.w + (size_t)row * K + ks0 + kb;
+                for (int u = 0; u < U; u++) buf.w[u] = kb + u * 32 < kr1 ? *(const bf16x8_t *)(wp + u * (16 * 32)) : zero8();
+            } else {
+                const bf16_t *wp = a.w + (size_t)row * K + ks0 + kb;
 #pragma unroll
-            for (int u = 0; u < U; u++) buf.w[u] = kb + u * 32 < kr1 ? *(const bf16x8_t *)(wp + u * 32) : zero8();
-#endif
+                for (int u = 0; u < U; u++) buf.w[u] = kb + u * 32 < kr1 ? *(const bf16x8_t *)(wp + u * 32) : zero8();
+            }
             if (XD) {
                 const bf16_t *xp = (const bf16_t *)a.x + (size_t)xrow_i * a.ldx + ks0 + kb;
 #pragma unroll
@@ -1084,7 +1086,7 @@ ResidentPlan plan_resident(int M, int K, int ntiles, int rt, const Workspace &ws
 unsigned long long *g_timeline = nullptr;
 #endif
 
-template <int PRO, int EPI, int TM, int WAVES, bool XD = false>
+template <int PRO, int EPI, int TM, int WAVES, bool XD = false, bool WT = false>
 int launch_resident_plan(SkinnyArgs a, const ResidentPlan &p, int ntiles, const Workspace &ws, hipStream_t stream) {
     constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
 #ifdef FLLM_TIMELINE
@@ -1108,14 +1110,33 @@ int launch_resident_plan(SkinnyArgs a, const ResidentPlan &p, int ntiles, const 
     const int groups = fllm_plan::resident_groups(p, ntiles, device_cus());
     static bool attribute_set = false;   // more than the default 64 KiB of dynamic LDS has to be asked for once
     if (!attribute_set) {
-        const hipError_t e = hipFuncSetAttribute((const void *)skinny_resident_kernel<PRO, EPI, TM, WAVES, XD>,
+        const hipError_t e = hipFuncSetAttribute((const void *)skinny_resident_kernel<PRO, EPI, TM, WAVES, XD, WT>,
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         FLLM_REQUIRE(e == hipSuccess, "linear_skinny: cannot raise the LDS limit: %s", hipGetErrorString(e));
         attribute_set = true;
     }
-    hipLaunchKernelGGL((skinny_resident_kernel<PRO, EPI, TM, WAVES, XD>), dim3(groups * p.S), dim3(WAVES * kWave), p.smem, stream,
+    hipLaunchKernelGGL((skinny_resident_kernel<PRO, EPI, TM, WAVES, XD, WT>), dim3(groups * p.S), dim3(WAVES * kWave), p.smem, stream,
                        a, (int)p.stage);
     return fllm_check_launch("linear_skinny");
+}
+
+// Tile-major weights serve matrices whose eight waves' K ranges are whole blocks of 128 columns.
+bool tiles_fit(int N, int K) { return N >= 16 && K >= 1024 && K % 1024 == 0; }
+
+// tiles[T][B][u][lane][8] = w[16 T + lane % 16][128 B + 32 u + 8 (lane / 16) ...]: tile T of 16 rows, block B of 128 columns,
+// k-step u of 32, and inside it the 16 bytes of each of the 64 lanes of a wave in lane order; rows past N are zeros
+__global__ void __launch_bounds__(256) tile_weights_kernel(const bf16_t *__restrict__ w, bf16_t *__restrict__ tiles, int N, int K, size_t pieces) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const int blocks = K / 128;
+    for (size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x; v < pieces; v += stride) {
+        const int lane = (int)(v & 63), u = (int)((v >> 6) & 3);
+        const size_t tb = v >> 8;
+        const int B = (int)(tb % blocks);
+        const size_t T = tb / blocks;
+        const size_t n = T * 16 + (lane & 15);
+        const int k = B * 128 + u * 32 + (lane >> 4) * 8;
+        *(bf16x8_t *)(tiles + v * 8) = n < (size_t)N ? *(const bf16x8_t *)(w + n * K + k) : zero8();
+    }
 }
 
 template <int PRO, int EPI>
@@ -1150,6 +1171,10 @@ int launch_resident(const SkinnyArgs &a, hipStream_t stream) {
         const bool uneven = 2 * tiles16 > slots && tiles16 < 2 * slots && tiles16 % slots != 0;
         const bool dual = a.M <= 8 && p.S == 1 && fllm_option_dual_k() && (uneven || 2 * tiles16 <= device_cus());
         if constexpr (PRO == PRO_BF16) {
+            if constexpr (EPI == EPI_ADD) {     // the output and down projections: their tile-major copy, where there is one
+                if (x_direct && !dual && a.w_tiles != nullptr && tiles_fit(a.N, a.K))
+                    return launch_resident_plan<PRO, EPI, TM_ROWS16, 8, true, true>(a, p, tiles16, ws, stream);
+            }
             if (x_direct) {
                 if (dual) return launch_resident_plan<PRO, EPI, TM_DUALK, 8, true>(a, p, tiles8, ws, stream);
                 return launch_resident_plan<PRO, EPI, TM_ROWS16, 8, true>(a, p, tiles16, ws, stream);
@@ -1410,17 +1435,57 @@ extern "C" int fllm_norm_qkv_rope_store(const float *x, const float *norm_w, flo
 // out += x w^T as fllm_linear does with a float32 `out`, and for the RMSNorm that reads `out` next: next_x = out *
 // next_w as bfloat16 [M, N], and next_ssq [M, *tiles_out] the sums of squares of out over the outputs of each tile
 // (room for M * N / 8 floats).  *tiles_out (host memory) says how many parts a row has.
+extern "C" int fllm_weight_tiles_supported(int N, int K) { return tiles_fit(N, K) ? 1 : 0; }
+
+extern "C" size_t fllm_weight_tiles_elements(int N, int K) { return (size_t)((N + 15) / 16) * 16 * (size_t)K; }
+
+extern "C" int fllm_tile_weights(const void *w, void *tiles, int N, int K, hipStream_t stream) {
+    FLLM_REQUIRE(tiles_fit(N, K), "tile_weights: takes matrices of at least 16 rows whose width is a multiple of 1,024 (N=%d K=%d)", N, K);
+    FLLM_REQUIRE(w != nullptr && tiles != nullptr && aligned16(w) && aligned16(tiles), "tile_weights: operands must be there and 16-byte aligned");
+    const size_t pieces = fllm_weight_tiles_elements(N, K) / 8;
+    const size_t want = (pieces + 255) / 256;
+    hipLaunchKernelGGL(tile_weights_kernel, dim3((unsigned int)(want < 65536 ? want : 65536)), dim3(256), 0, stream, (const bf16_t *)w,
+                       (bf16_t *)tiles, N, K, pieces);
+    return fllm_check_launch("tile_weights");
+}
+
+// out += x w^T (+ bias) for 1..16 bfloat16 rows and a float32 `out`, as fllm_linear in mode 2; `w_tiles` (may be null):
+// the tile-major copy of w, which the kernel streams instead where the launch it chooses can.
+extern "C" int fllm_linear_add_tiled(const void *x, int ldx, const void *w, const void *w_tiles, const float *bias, float *out, int ldo,
+                                     int M, int N, int K, hipStream_t stream) {
+    FLLM_REQUIRE(M >= 1 && M <= 16 && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && ldx >= K && ldo >= N,
+                 "linear_add_tiled: takes 1..16 rows, K and ldx in steps of 8 (M=%d N=%d K=%d ldx=%d ldo=%d)", M, N, K, ldx, ldo);
+    FLLM_REQUIRE(aligned16(x) && aligned16(w) && out != nullptr && (w_tiles == nullptr || aligned16(w_tiles)),
+                 "linear_add_tiled: operands must be there and 16-byte aligned");
+    SkinnyArgs a = {};
+    a.x = x;
+    a.ldx = ldx;
+    a.w = (const bf16_t *)w;
+    a.w_tiles = (const bf16_t *)w_tiles;
+    a.bias = bias;
+    a.out = out;
+    a.ldo = ldo;
+    a.M = M;
+    a.N = N;
+    a.K = K;
+    const int rc = launch_resident<PRO_BF16, EPI_ADD>(a, stream);
+    FLLM_REQUIRE(rc != 1, "linear_add_tiled: shape M=%d K=%d does not fit the staging area", M, K);
+    return rc;
+}
+
 extern "C" int fllm_linear_add_normed(const void *x, int ldx, const void *w, const float *bias, float *out, int M, int N, int K,
-                                      const float *next_w, void *next_x, float *next_ssq, int *tiles_out, hipStream_t stream) {
+                                      const float *next_w, void *next_x, float *next_ssq, int *tiles_out, const void *w_tiles,
+                                      hipStream_t stream) {
     FLLM_REQUIRE(M >= 1 && M <= 16 && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && N >= 16 && N % 16 == 0,
                  "linear_add_normed: takes 1..16 rows, K and ldx in steps of 8 and N in steps of 16 (M=%d N=%d K=%d ldx=%d)", M, N, K, ldx);
     FLLM_REQUIRE(aligned16(x) && aligned16(w) && aligned16(out) && aligned16(next_w) && next_x != nullptr && next_ssq != nullptr &&
-                     ((uintptr_t)next_x & 7) == 0 && tiles_out != nullptr,
+                     ((uintptr_t)next_x & 7) == 0 && tiles_out != nullptr && (w_tiles == nullptr || aligned16(w_tiles)),
                  "linear_add_normed: operands must be there and 16-byte aligned");
     SkinnyArgs a = {};
     a.x = x;
     a.ldx = ldx;
     a.w = (const bf16_t *)w;
+    a.w_tiles = (const bf16_t *)w_tiles;
     a.bias = bias;
     a.out = out;
     a.ldo = N;

@@ -71,7 +71,7 @@ class Engine:
                  max_num_partial_prefills: int = 0, long_prefill_token_threshold: int = 0, max_long_partial_prefills: int = 1,
                  preemption_mode: str = "recompute", eos_token_ids: Optional[Seq[int]] = None,
                  random_weights_on_device: bool = False, ops=None, ahead: bool = True, check_layers: int = 0,
-                 scheduling_policy: str = "fcfs", prefix_cache: Optional[bool] = None):
+                 scheduling_policy: str = "fcfs", prefix_cache: Optional[bool] = None, decode_weight_tiles="auto"):
         """`model`: a folder with config.json and safetensors; or `config` (a config.json dict)
         with `seed` for random weights (drawn on the host, or on the device with a stream of its
         own when `random_weights_on_device`: large models).  Option names follow the reference's server flags
@@ -91,6 +91,9 @@ class Engine:
         this one, and `step()` returns the events of the step before.  A request that stops at a
         token (end of sequence, stop id) has one more row in flight by then; that row is dropped.
 
+        `decode_weight_tiles` (True, False, "auto": while memory is plentiful): a second copy of the output and down
+        projection matrices in the order decode steps read them (`Runtime.tile_for_decode`).
+
         `check_layers`: the first so many steps run every layer also with the plain kernels and print, layer by
         layer, how far the two are apart, the largest value, a checksum and NaN/Inf counts (`runner.check_layers`)."""
         if (model is None) == (config is None):
@@ -105,7 +108,8 @@ class Engine:
             tensors = random_tensors(spec, seed, parse_dtype(dtype), device=device if random_weights_on_device else "cpu")
         self.runner = ModelRunner(spec, tensors, dtype=dtype, device=device, page_size=block_size, num_pages=num_blocks,
                                   max_requests=max_seqs, max_context=ctx, memory_utilization=gpu_memory_utilization,
-                                  ops=ops, typed_config=typed, max_step_tokens=max_batched_tokens)
+                                  ops=ops, typed_config=typed, max_step_tokens=max_batched_tokens,
+                                  decode_weight_tiles=decode_weight_tiles)
         del tensors
         self.config = typed
         self.max_model_len = self.runner.max_context

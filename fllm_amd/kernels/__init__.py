@@ -7,7 +7,8 @@ library cannot be loaded or built, constructing `Ops` raises.
 from __future__ import annotations
 
 import ctypes
-from typing import NamedTuple, Optional, Sequence
+import weakref
+from typing import Dict, NamedTuple, Optional, Sequence, Tuple
 
 import torch
 
@@ -48,7 +49,7 @@ assert SAMPLE_ROW_BYTES == 32
 _lib = None
 
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 
 def load_library(build_if_missing: bool = True):
@@ -90,7 +91,9 @@ def load_library(build_if_missing: bool = True):
                                      c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_argmax": [c_void, c_void, c_int, c_int, c_void],
         "fllm_gate_up_swiglu": [c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
-        "fllm_linear_add_normed": [c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_void, c_void, c_void, c_void, c_void],
+        "fllm_linear_add_normed": [c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_void, c_void, c_void, c_void, c_void, c_void],
+        "fllm_tile_weights": [c_void, c_void, c_int, c_int, c_void],
+        "fllm_linear_add_tiled": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_void],
         "fllm_scaled_gate_up_swiglu": [c_void, c_void, c_int, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_scaled_qkv_rope_store": [c_void, c_void, c_int, c_float, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void,
                                        c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
@@ -115,6 +118,10 @@ def load_library(build_if_missing: bool = True):
     lib.fllm_probe_mfma_bf16.restype = ctypes.c_double
     lib.fllm_random_fill.argtypes = [c_void, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint32, c_int, c_int, c_void]
     lib.fllm_random_fill.restype = c_int
+    lib.fllm_weight_tiles_supported.argtypes = [c_int, c_int]
+    lib.fllm_weight_tiles_supported.restype = c_int
+    lib.fllm_weight_tiles_elements.argtypes = [c_int, c_int]
+    lib.fllm_weight_tiles_elements.restype = c_size
     lib.fllm_set_fast_kernels.argtypes = [c_int]
     lib.fllm_set_fast_kernels.restype = None
     lib.fllm_attention_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int, c_int]
@@ -171,6 +178,33 @@ class Ops:
             torch.cuda.synchronize()
             self._check(self.lib.fllm_set_device_workspace(_ptr(buf), buf.numel()))
         Ops._workspaces[device] = buf
+
+    # ---- tile-major copies of weights for decode steps --------------------------------------------------
+    _tiles: Dict[int, Tuple[tuple, torch.Tensor]] = {}     # address of a weight matrix -> (its shape, its tile-major copy)
+
+    def tile_for_decode(self, w: torch.Tensor) -> bool:
+        """Keeps beside `w` (bfloat16 [N, K] on the GPU) a copy in the order in which the products of decode steps that
+        add into the residual stream read it (`fllm_tile_weights`); `linear(..., accumulate=True)` and
+        `linear_add_prepare` find it by the matrix's address and use it for steps of up to 16 rows.  The copy is given up
+        with `w`.  False: nothing was made (another type or place, a shape the kernels do not take tiles of)."""
+        if not (w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()):
+            return False
+        N, K = w.shape
+        if not self.lib.fllm_weight_tiles_supported(N, K):
+            return False
+        key = w.data_ptr()
+        if key in Ops._tiles and Ops._tiles[key][0] == (N, K):
+            return True
+        tiles = torch.empty(int(self.lib.fllm_weight_tiles_elements(N, K)), dtype=torch.bfloat16, device=w.device)
+        with torch.cuda.device(w.device):
+            self._check(self.lib.fllm_tile_weights(_ptr(w), _ptr(tiles), N, K, self._stream()))
+        Ops._tiles[key] = ((N, K), tiles)
+        weakref.finalize(w, Ops._tiles.pop, key, None)
+        return True
+
+    def _tiles_of(self, w: torch.Tensor) -> Optional[torch.Tensor]:
+        held = Ops._tiles.get(w.data_ptr())
+        return held[1] if held is not None and held[0] == tuple(w.shape) else None
 
     def set_fast_kernels(self, on: bool) -> None:
         """Off: bfloat16 calls run the plain kernels (tests compare the two)."""
@@ -283,6 +317,11 @@ class Ops:
             return out
         ldx = x.stride(0) if M > 1 else K
         ldo = out.stride(0) if M > 1 else N
+        tiles = self._tiles_of(w) if mode == OUT_ADD_F32 and M <= 16 and Ops._tiles else None
+        if tiles is not None and ldx % 8 == 0 and K % 8 == 0:
+            self._check(self.lib.fllm_linear_add_tiled(_ptr(x), ldx, _ptr(w), _ptr(tiles), _ptr(bias), _ptr(out), ldo, M, N, K,
+                                                       self._stream()))
+            return out
         self._check(self.lib.fllm_linear(_ptr(x), ldx, _ptr(w), _ptr(bias), _ptr(out), ldo, M, N, K, _DTYPE_CODE[x.dtype],
                                          mode, self._stream()))
         return out
@@ -342,7 +381,7 @@ class Ops:
         parts = ctypes.c_int(0)
         self._check(self.lib.fllm_linear_add_normed(_ptr(x), x.stride(0) if M > 1 else K, _ptr(w), _ptr(bias), _ptr(residual), M, N,
                                                     K, _ptr(next_norm_weight), _ptr(xn), _ptr(ssq), ctypes.addressof(parts),
-                                                    self._stream()))
+                                                    _ptr(self._tiles_of(w)) if Ops._tiles else None, self._stream()))
         return PreparedNorm(xn, ssq, int(parts.value))
 
     def _prepared_operands(self, prepared: PreparedNorm, w, bias, n_rows_w):

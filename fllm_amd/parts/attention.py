@@ -66,6 +66,7 @@ class PagedAttention(Mixer):
         self.w_qkv = torch.cat([reorder(rt.matrix(weights["q"]), order_q), reorder(rt.matrix(weights["k"]), order_k),
                                 rt.matrix(weights["v"])], dim=0).contiguous()
         self.w_o = rt.matrix(weights["o"])
+        rt.tile_for_decode(self.w_o)
         biases = [reorder(None if weights.get("q_bias") is None else rt.vector(weights["q_bias"]), order_q),
                   reorder(None if weights.get("k_bias") is None else rt.vector(weights["k_bias"]), order_k),
                   None if weights.get("v_bias") is None else rt.vector(weights["v_bias"])]

@@ -26,6 +26,7 @@ class GatedMLP(FeedForward):
         self.inter = int(spec["intermediate_size"])
         self.w_gate_up = torch.cat([rt.matrix(weights["gate"]), rt.matrix(weights["up"])], dim=0).contiguous()
         self.w_down = rt.matrix(weights["down"])
+        rt.tile_for_decode(self.w_down)
         gb, ub = weights.get("gate_bias"), weights.get("up_bias")
         self.b_gate_up = None
         if gb is not None or ub is not None:

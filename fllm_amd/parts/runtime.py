@@ -12,13 +12,16 @@ class Runtime:
     (matrices, activations and pages in bfloat16; residual stream, norms, softmax, rotary angles
     and logits in float32).  `ops` is the kernel library (`fllm_amd.kernels.Ops`)."""
 
-    def __init__(self, device: torch.device, dtype: torch.dtype, ops, max_context: int):
+    def __init__(self, device: torch.device, dtype: torch.dtype, ops, max_context: int, decode_weight_tiles="auto"):
         if dtype not in (torch.float32, torch.bfloat16):
             raise ValueError(f"compute dtype must be float32 or bfloat16, not {dtype}")
         self.device = torch.device(device)
         self.dtype = dtype
         self.ops = ops
         self.max_context = int(max_context)
+        # second copies of some weight matrices in the order decode steps read them (`tile_for_decode`): True, False, or
+        # "auto": as long as a copy is a small part of the memory that is still free
+        self.decode_weight_tiles = decode_weight_tiles
         # weak: a placed tensor lives as long as a part holds it (pieces of a concatenated matrix are freed)
         self._placed = weakref.WeakValueDictionary()
         self.shared: Dict[Any, Any] = {}      # tables several parts share (rotary tables)
@@ -39,6 +42,20 @@ class Runtime:
     def vector(self, t: torch.Tensor) -> torch.Tensor:
         """Norm weights and biases: float32 (exact for both storage types)."""
         return self._place(t, torch.float32)
+
+    def tile_for_decode(self, w: torch.Tensor) -> None:
+        """For a matrix whose product adds into the residual stream in decode steps: lets the kernel library keep a
+        tile-major copy beside it, where it has such kernels and the memory is there (288 GB a device are laid out for
+        bandwidth: the copy costs the matrix's bytes again and takes a fifth off such a product at 8 rows)."""
+        make = getattr(self.ops, "tile_for_decode", None)
+        if not self.decode_weight_tiles or make is None or self.dtype != torch.bfloat16 or not w.is_cuda:
+            return
+        if self.decode_weight_tiles == "auto":
+            free, _ = torch.cuda.mem_get_info(self.device)
+            if w.numel() * w.element_size() > free // 20:
+                self.decode_weight_tiles = False          # the device is filling up: no further copies
+                return
+        make(w)
 
     def forget_host_tensors(self) -> None:
         self._placed.clear()

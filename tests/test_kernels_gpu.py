@@ -238,6 +238,44 @@ def test_vocabulary_projection_at_the_benchmark_sizes(ops, library_ops, K, row_c
             assert torch.equal(again[0], out[0]), f"M{M} K{K}: row 0 depends on the rows beside it"
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 4096, 14336), (16, 2048, 8192), (5, 4104, 1024), (8, 40, 1024), (3, 8192, 2048),
+                                   (16, 4096, 14336), (2, 24, 3072), (9, 1000, 2048)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_products_that_add_read_the_tile_major_copy(ops, ref, M, N, K, bias):
+    """The output and down projections of decode steps keep a second copy of their matrix, tile by tile in the order the
+    lanes of a wave take it (`Ops.tile_for_decode`): `linear(..., accumulate=True)` and `linear_add_prepare` find it by
+    the matrix's address.  The sums are those of the row-major matrix bit for bit (the same products in the same order),
+    and the float64 product's within rounding; the copy holds every element at its place."""
+    g = gen(47)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).to(DEV)
+    b = torch.randn(N, generator=g).to(DEV) if bias else None
+    base = torch.randn(M, N, generator=g).to(DEV)
+    plain = ops.linear(x, w, base.clone(), bias=b, accumulate=True)
+    twin = w.clone()                                         # the same values at another address: that one gets the copy
+    assert ops.tile_for_decode(twin) and ops._tiles_of(twin) is not None and ops._tiles_of(w) is None
+    tiles = ops._tiles_of(twin).view(-1, K // 128, 4, 4, 16, 8)          # [tile][block][k-step][lane / 16][lane % 16][8]
+    back = tiles.permute(0, 4, 1, 2, 3, 5).reshape(-1, K)                 # [16 tile + lane % 16][128 block + 32 step + 8 (lane / 16) + j]
+    assert torch.equal(back[:N], w) and not back[N:].any()
+    tiled = ops.linear(x, twin, base.clone(), bias=b, accumulate=True)
+    assert torch.equal(tiled, plain), f"M{M} N{N} K{K}: the tile-major copy gives other sums"
+    want = ref.linear(x.cpu(), w.cpu(), base.double().cpu(), bias=None if b is None else b.cpu(), accumulate=True)
+    mag = (x.double().abs() @ w.double().abs().T).max().item()
+    close(tiled, want, 1e-6, 4e-7 * mag + 1e-6, f"tile-major M{M} N{N} K{K}")
+    if N % 16 == 0:
+        norm_w = (1.0 + 0.1 * torch.randn(N, generator=g)).to(DEV)
+        r1, r2 = base.clone(), base.clone()
+        a = ops.linear_add_prepare(x, w, r1, norm_w, bias=b)
+        c = ops.linear_add_prepare(x, twin, r2, norm_w, bias=b)
+        assert torch.equal(r1, r2) and torch.equal(a.x, c.x) and a.parts == c.parts
+        assert torch.equal(a.ssq[:M * a.parts], c.ssq[:M * c.parts])
+    key = twin.data_ptr()
+    del twin, tiles, back
+    assert key not in type(ops)._tiles                       # the copy goes with its matrix
+    assert not ops.tile_for_decode(torch.zeros(64, 1000, dtype=torch.bfloat16, device=DEV))       # widths it does not take
+    assert not ops.tile_for_decode(torch.zeros(64, 1024, dtype=torch.float32, device=DEV))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("rows,width", [(1, 64), (13, 4099), (300, 4096)])
 def test_add_residual(ops, dtype, rows, width):
