@@ -52,9 +52,9 @@ attention_generic_kernel(const T *__restrict__ q, int q_stride, const T *__restr
         float s = -INFINITY;
         if (key < n) {
             const int page = tbl[key / page_size], off = key % page_size;
-            const T *kr = k_pages + (((size_t)page * kv_heads + kvh) * page_size + off) * head_dim;
+            const T *kr = k_pages + key_offset(page, kv_heads, kvh, page_size, head_dim, off, 0);     // chunk c / 8 lies c / 8 * page_size * 8 on
             float dot = 0.f;
-            for (int c = 0; c < head_dim; c++) dot = fmaf(qs[c], to_f32<T>(kr[c]), dot);
+            for (int c = 0; c < head_dim; c++) dot = fmaf(qs[c], to_f32<T>(kr[(size_t)(c >> 3) * page_size * 8 + (c & 7)]), dot);
             s = dot * scale;
             if (head_slopes != nullptr) s = fmaf(head_slopes[h], (float)(key - pos), s);   // a bias by distance (<= 0 keys back)
         }
@@ -103,6 +103,7 @@ int attention_any(const void *q, int q_stride, const void *k_pages, const void *
     FLLM_REQUIRE(rows >= 0 && heads > 0 && kv_heads > 0 && head_dim > 0 && page_size > 0 && table_stride > 0 && num_pages > 0,
                  "attention: bad sizes");
     FLLM_REQUIRE(heads % kv_heads == 0, "attention: %d heads are not a multiple of %d key/value heads", heads, kv_heads);
+    FLLM_REQUIRE(head_dim % 8 == 0, "attention: head size %d; keys lie in chunks of 8 values in a page, head sizes come in steps of 8", head_dim);
     FLLM_REQUIRE(num_segs > 0 && seg_start != nullptr, "attention: segment starts are required");
     FLLM_REQUIRE(single_from >= 0 && single_from <= num_segs, "attention: single_from %d is outside 0..%d", single_from, num_segs);
     FLLM_REQUIRE(q_stride >= heads * head_dim, "attention: q_stride %d is shorter than heads*head_dim", q_stride);

@@ -179,12 +179,12 @@ attn_tile_kernel(AttnArgs p) {
     for (int k0 = kbegin; k0 <= p_last; k0 += KT) {
         __syncthreads();   // the previous tile has been read
         for (int ch = threadIdx.x; ch < KT * D / 8; ch += kThreads) {
-            const int key = ch / (D / 8), dc = ch % (D / 8);
+            const int key = ch % KT, dc = ch / KT;       // neighbouring threads take neighbouring keys: that is how they lie in a page
             const int kabs = k0 + key;
             bf16x8_t v = zero8();
             if (kabs >= lo_tile && kabs <= p_last) {
                 const int page = tbl[kabs >> psh], off = kabs & pmask;
-                v = *(const bf16x8_t *)(p.kp + (((size_t)page * nkv + kvh) * ps + off) * D + dc * 8);
+                v = *(const bf16x8_t *)(p.kp + key_offset(page, nkv, kvh, ps, D, off, dc * 8));
             }
             *(bf16x8_t *)(Ks + key * KP + dc * 8) = v;
         }
@@ -351,9 +351,9 @@ attn_tile32_kernel(AttnArgs p) {
 #pragma unroll
     for (int c = 0; c < CH; c++) {
         const int ch = threadIdx.x + c * kThreads;
-        const int key = ch >> (LD - 3), dc = ch & (D / 8 - 1);
+        const int key = ch & (KT - 1), dc = ch / KT;     // neighbouring threads take neighbouring keys: that is how they lie in a page
         k_key[c] = key;
-        k_in_page[c] = (kvh * ps + (key & pmask)) * D + dc * 8;
+        k_in_page[c] = (int)key_offset(0, nkv, kvh, ps, D, key & pmask, dc * 8);
         // A key's row in LDS: bits 2 and 3 of the key swapped, which is where the products read it (row q of a 32-key
         // block is key 16 (q / 16) + 8 (q / 4 % 2) + 4 (q / 8 % 2) + q % 4, see the table above, and that map is this swap): the 8 lanes of a 128-byte LDS access then read 8
         // consecutive rows, 16 bytes further along the banks each, instead of hitting every bank twice.
@@ -623,37 +623,45 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
     for (int dt = 0; dt < DT; dt++) o[dt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
 
+    // A block is 32 keys: two score tiles of 16.  Row c of tile j is key kb + 16 j + c, so that a load of the tile's keys
+    // (chunks 4 kk + g of 16 neighbouring tokens) is 1 KiB in a row where a page holds 16 tokens or more.  Lane (c, g) then
+    // holds the scores of keys kb + 16 j + 4 g + i, i = 0..3, and takes exactly those eight keys' values as its operand
+    // of the second product: two runs of four neighbouring tokens of V^T, 8 bytes each.
     // The page numbers of a block are asked for one block ahead, so that a block waits for one memory latency
     // (its keys and values), not for two in a row.
-    auto block_pages = [&](int kb, int &kpage, int &vpage) {
-        const int grp = kb + (c >> 2) * 8, vkey = kb + g * 8;
-        kpage = (kb < end && grp < n && grp + 8 > lo) ? tbl[grp >> psh] : 0;
-        vpage = (kb < end && vkey < n && vkey + 8 > lo) ? tbl[vkey >> psh] : 0;
-    };
-    int kpage_next, vpage_next;
-    block_pages(begin + wave * 32, kpage_next, vpage_next);
-    for (int kb = begin + wave * 32; kb < end; kb += WAVES * 32) {
-        // keys: A row c of tile j is key kb + 8*(c/4) + 4*j + c%4; both tiles of a lane lie in one group of 8.
-        // values: lane (c, g) loads V^T[d = 16 dt + c][keys kb + 8g .. + 7].  All loads of the block are
-        // issued before the first product: one memory latency per block.
-        const int grp = kb + (c >> 2) * 8;
-        const bool gload = grp < n && grp + 8 > lo;
-        const int vkey = kb + g * 8;
-        const bool vload = vkey < n && vkey + 8 > lo;
-        const int kpage = kpage_next, vpage = vpage_next;
-        block_pages(kb + WAVES * 32, kpage_next, vpage_next);
-        bf16x8_t kf[2][KD], vf[DT];
+    auto block_pages = [&](int kb, int (&kpage)[2], int (&vpage)[2]) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            const int key = grp + j * 4 + (c & 3);
-            const bool valid = gload && key >= lo && key < n;
-            const bf16_t *kr = p.kp + (((size_t)kpage * nkv + kvh) * ps + (key & pmask)) * D + g * 8;
-#pragma unroll
-            for (int kk = 0; kk < KD; kk++) kf[j][kk] = valid ? *(const bf16x8_t *)(kr + kk * 32) : zero8();
+            const int key = kb + 16 * j + c, vkey = kb + 16 * j + 4 * g;
+            kpage[j] = (kb < end && key < n && key >= lo) ? tbl[key >> psh] : 0;
+            vpage[j] = (kb < end && vkey < n && vkey + 4 > lo) ? tbl[vkey >> psh] : 0;
         }
-        const bf16_t *vr = p.vp + (((size_t)vpage * nkv + kvh) * D + c) * ps + (vkey & pmask);
+    };
+    int kpage_next[2], vpage_next[2];
+    block_pages(begin + wave * 32, kpage_next, vpage_next);
+    for (int kb = begin + wave * 32; kb < end; kb += WAVES * 32) {
+        int kpage[2], vpage[2];
 #pragma unroll
-        for (int dt = 0; dt < DT; dt++) vf[dt] = vload ? *(const bf16x8_t *)(vr + (size_t)dt * 16 * ps) : zero8();
+        for (int j = 0; j < 2; j++) kpage[j] = kpage_next[j], vpage[j] = vpage_next[j];
+        block_pages(kb + WAVES * 32, kpage_next, vpage_next);
+        // All loads of the block are issued before the first product: one memory latency per block.
+        bf16x8_t kf[2][KD];
+        bf16x4_t vf[2][DT];
+        bool vtail[2];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int key = kb + 16 * j + c;
+            const bool valid = key >= lo && key < n;
+            const bf16_t *kr = p.kp + key_offset(kpage[j], nkv, kvh, ps, D, key & pmask, g * 8);
+#pragma unroll
+            for (int kk = 0; kk < KD; kk++) kf[j][kk] = valid ? *(const bf16x8_t *)(kr + (size_t)kk * 4 * ps * 8) : zero8();
+            const int vkey = kb + 16 * j + 4 * g;
+            const bool vload = vkey < n && vkey + 4 > lo;
+            vtail[j] = vload && vkey + 4 > n;
+            const bf16_t *vr = p.vp + (((size_t)vpage[j] * nkv + kvh) * D + c) * ps + (vkey & pmask);
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) vf[j][dt] = vload ? *(const bf16x4_t *)(vr + (size_t)dt * 16 * ps) : (bf16x4_t){(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
+        }
 
         f32x4_t s[2];
 #pragma unroll
@@ -666,22 +674,24 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const int key = kb + g * 8 + j * 4 + i;
+                const int key = kb + 16 * j + 4 * g + i;
                 const bool vis = key >= lo && key < n;
                 s[j][i] = vis ? s[j][i] * p.scale_log2 : -INFINITY;
             }
         float alpha;
         softmax_step<2>(s, m_run, l_run, alpha);
         const bf16x8_t pf = pack_p(s[0], s[1]);
-        const bool tail = vload && vkey + 8 > n;
 #pragma unroll
         for (int dt = 0; dt < DT; dt++) {
-            bf16x8_t a = vf[dt];
-            if (tail) {   // slots past the last token hold whatever an earlier request left
+            bf16x8_t a;
 #pragma unroll
-                for (int e = 0; e < 8; e++)
-                    if (vkey + e >= n) a[e] = (bf16_t)0.0f;
-            }
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    // slots past the last token hold whatever an earlier request left
+                    const bool past = vtail[j] && kb + 16 * j + 4 * g + e >= n;
+                    a[4 * j + e] = past ? (bf16_t)0.0f : vf[j][dt][e];
+                }
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf, o[dt] * alpha, 0, 0, 0);
         }
     }

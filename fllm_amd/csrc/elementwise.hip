@@ -159,14 +159,13 @@ rope_kv_store_kernel(T *__restrict__ qkv, const int32_t *__restrict__ row_pos, c
         const int ia = pairing ? 2 * l : l, ib = pairing ? 2 * l + 1 : l + half;
         const T *head = krow + (size_t)h * head_dim;
         const float a = to_f32<T>(head[ia]), b = to_f32<T>(head[ib]);
-        T *dst = k_pages + (((size_t)page * kv_heads + h) * page_size + off) * head_dim;
-        dst[ia] = from_f32<T>(a * cs[l] - b * sn[l]);
-        dst[ib] = from_f32<T>(b * cs[l] + a * sn[l]);
+        k_pages[key_offset(page, kv_heads, h, page_size, head_dim, off, ia)] = from_f32<T>(a * cs[l] - b * sn[l]);
+        k_pages[key_offset(page, kv_heads, h, page_size, head_dim, off, ib)] = from_f32<T>(b * cs[l] + a * sn[l]);
     }
     const int rest = head_dim - rope_dims;
     for (int i = threadIdx.x; i < kv_heads * rest; i += kBlock) {
         const int h = i / rest, c = rope_dims + (i - h * rest);
-        k_pages[(((size_t)page * kv_heads + h) * page_size + off) * head_dim + c] = krow[(size_t)h * head_dim + c];
+        k_pages[key_offset(page, kv_heads, h, page_size, head_dim, off, c)] = krow[(size_t)h * head_dim + c];
     }
     // values, stored transposed inside the page: [head_dim][token]
     for (int i = threadIdx.x; i < kv_heads * head_dim; i += kBlock) {
@@ -331,7 +330,7 @@ rope_kv_store_vec_kernel(bf16_t *__restrict__ qkv, const int32_t *__restrict__ r
             }
         }
         if (h < heads) *(bf16x8_t *)(row + (size_t)h * head_dim + c) = v;
-        else *(bf16x8_t *)(k_pages + (((size_t)s_page[i] * kv_heads + (h - heads)) * page_size + s_off[i]) * head_dim + c) = v;
+        else *(bf16x8_t *)(k_pages + key_offset(s_page[i], kv_heads, h - heads, page_size, head_dim, s_off[i], c)) = v;
     }
     if (!store_kv) return;
     if (!run) {
@@ -371,6 +370,7 @@ extern "C" int fllm_rope_kv_store(void *qkv, const int32_t *row_pos, const int32
                  "rope_kv_store: rope_dims %d must be even and at most head_dim %d", rope_dims, head_dim);
     FLLM_REQUIRE(pairing == 0 || pairing == 1, "rope_kv_store: unknown pairing %d", pairing);
     FLLM_REQUIRE(!store_kv || (k_pages && v_pages && num_pages > 0), "rope_kv_store: pages missing");
+    FLLM_REQUIRE(head_dim % 8 == 0, "rope_kv_store: head size %d; keys lie in chunks of 8 values in a page, head sizes come in steps of 8", head_dim);
     (void)table_positions;
     if (rows == 0) return 0;
     if (dtype == FLLM_F32)

@@ -261,7 +261,7 @@ __device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], 
             const int off = pos % a.page_size;
             if (hd < a.heads + a.kv_heads) {
                 const int kvh = hd - a.heads;
-                bf16_t *kd = a.k_pages + (((size_t)page * a.kv_heads + kvh) * a.page_size + off) * d + j;
+                bf16_t *kd = a.k_pages + key_offset(page, a.kv_heads, kvh, a.page_size, d, off, j);      // j .. j + 3 lie in one chunk of 8
                 if (((uintptr_t)a.k_pages & 7) == 0) {      // head_dim and j are multiples of 4
                     *(bf16x4_t *)kd = pack4(v4);
                 } else {
@@ -389,9 +389,13 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
             if (m < M && lane * 4 < a.ssq_count) ssq_pre[k] = *(const f32x4_t *)(a.ssq_in + (size_t)m * a.ssq_count + lane * 4);
         }
     }
-    Block b0, b1;
-    issue(b0);      // in flight while the activations are staged
-    issue(b1);
+#ifndef FLLM_BLOCKS_IN_FLIGHT
+#define FLLM_BLOCKS_IN_FLIGHT 2
+#endif
+    constexpr int NB = XD ? 2 : FLLM_BLOCKS_IN_FLIGHT;      // blocks of weights a wave has asked for ahead of its products
+    Block bl[NB];
+#pragma unroll
+    for (int i = 0; i < NB; i++) issue(bl[i]);      // in flight while the activations are staged
     // what the epilogue reads besides the sums: the part that belongs to this lane's row now, the part that belongs
     // to an item when the wave whose turn it is to finish the item starts on it
     const int m_out = TM == TM_DUALK ? (r & 7) : r;
@@ -591,9 +595,10 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
     };
 
     const int total = my_items * nbw;
-    for (int q = 0; q < total; q += 2) {
-        step(b0);
-        if (q + 1 < total) step(b1);
+    for (int q = 0; q < total; q += NB) {
+#pragma unroll
+        for (int i = 0; i < NB; i++)
+            if (i == 0 || q + i < total) step(bl[i]);
     }
     FLLM_STAMP(a, 4);
 }
@@ -1417,8 +1422,8 @@ extern "C" int fllm_norm_qkv_rope_store(const float *x, const float *norm_w, flo
                                         int page_size, int store_kv, hipStream_t stream) {
     FLLM_REQUIRE(fllm_fused_decode_supported(M, K), "norm_qkv_rope_store: takes 1..64 rows and K a multiple of 8 (M=%d K=%d)", M, K);
     FLLM_REQUIRE(aligned16(x) && aligned16(w_qkv) && aligned16(norm_w), "norm_qkv_rope_store: operands must be 16-byte aligned");
-    FLLM_REQUIRE(head_dim % 4 == 0 && rope_dims % 2 == 0 && rope_dims <= head_dim && rope_dims >= 0,
-                 "norm_qkv_rope_store: head_dim %d must be a multiple of 4 and rope_dims %d even and no larger", head_dim, rope_dims);
+    FLLM_REQUIRE(head_dim % 8 == 0 && rope_dims % 2 == 0 && rope_dims <= head_dim && rope_dims >= 0,
+                 "norm_qkv_rope_store: head_dim %d must be a multiple of 8 and rope_dims %d even and no larger", head_dim, rope_dims);
     FLLM_REQUIRE(heads > 0 && kv_heads > 0 && page_size > 0 && table_stride > 0 && eps > 0.f, "norm_qkv_rope_store: bad sizes");
     FLLM_REQUIRE(!store_kv || (k_pages && v_pages), "norm_qkv_rope_store: pages missing");
     SkinnyArgs a = qkv_args(x, eps, w_qkv, bias, q_out, row_pos, row_seg, tables, table_stride, cos_table, sin_table, rope_dims,
@@ -1533,8 +1538,8 @@ extern "C" int fllm_scaled_qkv_rope_store(const void *xn, const float *ssq, int 
     FLLM_REQUIRE(M >= 1 && M <= 16 && K % 8 == 0 && K >= 8 && ssq_count > 0,
                  "scaled_qkv_rope_store: takes 1..16 rows and K a multiple of 8 (M=%d K=%d parts=%d)", M, K, ssq_count);
     FLLM_REQUIRE(aligned16(xn) && aligned16(w_qkv) && ssq != nullptr, "scaled_qkv_rope_store: operands must be 16-byte aligned");
-    FLLM_REQUIRE(head_dim % 4 == 0 && rope_dims % 2 == 0 && rope_dims <= head_dim && rope_dims >= 0,
-                 "scaled_qkv_rope_store: head_dim %d must be a multiple of 4 and rope_dims %d even and no larger", head_dim, rope_dims);
+    FLLM_REQUIRE(head_dim % 8 == 0 && rope_dims % 2 == 0 && rope_dims <= head_dim && rope_dims >= 0,
+                 "scaled_qkv_rope_store: head_dim %d must be a multiple of 8 and rope_dims %d even and no larger", head_dim, rope_dims);
     FLLM_REQUIRE(heads > 0 && kv_heads > 0 && page_size > 0 && table_stride > 0 && eps > 0.f, "scaled_qkv_rope_store: bad sizes");
     FLLM_REQUIRE(!store_kv || (k_pages && v_pages), "scaled_qkv_rope_store: pages missing");
     SkinnyArgs a = qkv_args(xn, eps, w_qkv, bias, q_out, row_pos, row_seg, tables, table_stride, cos_table, sin_table, rope_dims,

@@ -17,7 +17,7 @@ import torch
 class CacheBinding:
     """Where one run entry keeps its keys and values (and state)."""
     group: int                              # index into StepContext.tables
-    k_pages: Optional[torch.Tensor]         # [pages, kv_heads, page_size, k_dim]
+    k_pages: Optional[torch.Tensor]         # [pages, kv_heads, *KVNeed.key_page_shape]: [page_size, k_dim], or chunked [k_dim / n, page_size, n]
     v_pages: Optional[torch.Tensor]         # [pages, kv_heads, v_dim, page_size]
     page_size: int
     writes: bool                            # False: the entry reads another entry's cache

@@ -2,7 +2,7 @@
 from __future__ import annotations
 
 import math
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Dict, List, NamedTuple, Optional, Sequence, Tuple
 
 import torch
 
@@ -13,6 +13,15 @@ from ..parts.runtime import Runtime
 from ..registry import part_class
 from ..weights.loader import part_weights
 from .context import CacheBinding, StepContext
+
+
+class GroupKey(NamedTuple):
+    """What run entries must have in common to share the pages of one cache group."""
+    kv_heads: int
+    k_dim: int
+    v_dim: int
+    window: Optional[int]
+    key_chunk: int
 
 
 class Model:
@@ -55,7 +64,7 @@ class Model:
             if multiple <= 0:
                 raise ValueError(f"run entry of layer {entry.layer}: portion_multiple() must be positive, is {multiple}")
             self.portion_multiple = self.portion_multiple * multiple // math.gcd(self.portion_multiple, multiple)
-        keys: List[Tuple] = []
+        keys: List[GroupKey] = []
         self.entry_group: List[Optional[int]] = [None] * len(self.spec.run_order)
         self.entry_index: List[Optional[int]] = [None] * len(self.spec.run_order)   # index inside the group's tensors
         members: List[List[int]] = []
@@ -66,14 +75,15 @@ class Model:
             if entry.reads_cache_of is not None:
                 src = entry.reads_cache_of
                 src_need = self.kv_needs[src]
-                if src_need is None or (src_need.kv_heads, src_need.k_dim, src_need.v_dim) != (need.kv_heads, need.k_dim, need.v_dim):
+                if src_need is None or ((src_need.kv_heads, src_need.k_dim, src_need.v_dim, src_need.key_chunk)
+                                        != (need.kv_heads, need.k_dim, need.v_dim, need.key_chunk)):
                     raise ValueError(f"run entry {i} cannot read the cache of entry {src}: different geometry")
                 if src_need.window is not None and (need.window is None or need.window > src_need.window):
                     raise ValueError(f"run entry {i} needs more keys than entry {src} keeps")
                 self.entry_group[i] = self.entry_group[src]
                 self.entry_index[i] = self.entry_index[src]
                 continue
-            key = (need.kv_heads, need.k_dim, need.v_dim, need.window)
+            key = GroupKey(need.kv_heads, need.k_dim, need.v_dim, need.window, need.key_chunk)
             if key not in keys:
                 keys.append(key)
                 members.append([])
@@ -85,13 +95,13 @@ class Model:
         self.group_members = members
 
     def group_specs(self, page_size: int) -> List[GroupSpec]:
-        return [GroupSpec(entries=tuple(m), kv_heads=k[0], k_dim=k[1], v_dim=k[2], window=k[3], page_size=page_size)
+        return [GroupSpec(entries=tuple(m), kv_heads=k.kv_heads, k_dim=k.k_dim, v_dim=k.v_dim, window=k.window, page_size=page_size)
                 for k, m in zip(self.group_keys, self.group_members)]
 
     def cache_bytes_per_page(self, page_size: int) -> List[int]:
         """Bytes a page of each group costs (keys and values of all the group's run entries)."""
         elem = torch.empty((), dtype=self.rt.dtype).element_size()
-        return [len(m) * k[0] * (k[1] + k[2]) * page_size * elem for k, m in zip(self.group_keys, self.group_members)]
+        return [len(m) * k.kv_heads * (k.k_dim + k.v_dim) * page_size * elem for k, m in zip(self.group_keys, self.group_members)]
 
     def allocate_caches(self, page_size: int, pages_per_group: Sequence[int], max_requests: int,
                         max_step_tokens: Optional[int] = None) -> CacheManager:
@@ -105,7 +115,8 @@ class Model:
         self.null_pages = [int(n) for n in pages_per_group]
         self.k_store, self.v_store = [], []
         for g, n in zip(groups, pages_per_group):
-            self.k_store.append(torch.zeros((len(g.entries), n + 1, g.kv_heads, page_size, g.k_dim),
+            need = self.kv_needs[g.entries[0]]            # the group's entries agree on what they need
+            self.k_store.append(torch.zeros((len(g.entries), n + 1, g.kv_heads, *need.key_page_shape(page_size)),
                                             dtype=rt.dtype, device=rt.device))
             self.v_store.append(torch.zeros((len(g.entries), n + 1, g.kv_heads, g.v_dim, page_size),
                                             dtype=rt.dtype, device=rt.device))

@@ -132,7 +132,7 @@ class ModelRunner:
         keeps a window when steps are bounded, the window and one step."""
         caps = []
         for key in self.model.group_keys:
-            window = key[2]
+            window = key.window
             each = -(-self.max_context // self.page_size)
             if window is not None and self.max_step_tokens is not None:
                 each = min(each, CacheManager.window_pages_bound(window, self.page_size, self.max_step_tokens))
@@ -148,7 +148,7 @@ class ModelRunner:
             return caps
         free, total = torch.cuda.mem_get_info(self.device)
         budget = int(free - (1.0 - utilization) * total) - (2 << 30)   # room for activations and logits
-        bounded = [key[2] is not None and self.max_step_tokens is not None for key in self.model.group_keys]
+        bounded = [key.window is not None and self.max_step_tokens is not None for key in self.model.group_keys]
         pages = [cap if b else 0 for cap, b in zip(caps, bounded)]
         budget -= sum(n * size for n, size in zip(pages, per_page))
         rest = [g for g, b in enumerate(bounded) if not b]

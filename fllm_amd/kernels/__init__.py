@@ -460,7 +460,7 @@ class Ops:
         store = k_pages is not None
         if store:
             pages = k_pages.shape[0]
-            _dense(k_pages, "k_pages", torch.bfloat16, (pages, kv_heads, page_size, head_dim))
+            _dense(k_pages, "k_pages", torch.bfloat16, (pages, kv_heads, head_dim // 8, page_size, 8))
             _dense(v_pages, "v_pages", torch.bfloat16, (pages, kv_heads, head_dim, page_size))
         if prepared is not None:
             self._check(self.lib.fllm_scaled_qkv_rope_store(
@@ -510,9 +510,10 @@ class Ops:
         _need(cos.dim() == 2 and cos.shape[1] == half, f"rotary tables must be [positions, {half}]")
         store = k_pages is not None
         num_pages = 0
+        _need(head_dim % 8 == 0, f"head size {head_dim}: keys are stored in chunks of 8 values")
         if store:
             num_pages = k_pages.shape[0]
-            _dense(k_pages, "k_pages", qkv.dtype, (num_pages, kv_heads, page_size, head_dim))
+            _dense(k_pages, "k_pages", qkv.dtype, (num_pages, kv_heads, head_dim // 8, page_size, 8))
             _dense(v_pages, "v_pages", qkv.dtype, (num_pages, kv_heads, head_dim, page_size))
         self._check(self.lib.fllm_rope_kv_store(
             _ptr(qkv), _ptr(row_pos), _ptr(row_seg), _ptr(tables), tables.shape[1], _ptr(cos), _ptr(sin), cos.shape[0],
@@ -537,7 +538,7 @@ class Ops:
               f"q must be [rows, {heads * head_dim}] with unit column stride")
         _need(q.dtype in _DTYPE_CODE, f"dtype {q.dtype} unsupported")
         num_pages = k_pages.shape[0]
-        _dense(k_pages, "k_pages", q.dtype, (num_pages, kv_heads, page_size, head_dim))
+        _dense(k_pages, "k_pages", q.dtype, (num_pages, kv_heads, head_dim // 8, page_size, 8))
         _dense(v_pages, "v_pages", q.dtype, (num_pages, kv_heads, head_dim, page_size))
         _dense(tables, "tables", torch.int32)
         _need(tables.dim() == 2, "tables must be [segments, pages]")

@@ -73,7 +73,7 @@ def _paged(dev, dtype, segs, kv_heads, head_dim, page_size):
     pages_each = -(-ctx // page_size)
     num_pages = len(segs) * pages_each + 1
     tables = torch.randperm(num_pages, device=dev)[: len(segs) * pages_each].to(torch.int32).view(len(segs), pages_each)
-    k = torch.randn(num_pages, kv_heads, page_size, head_dim, device=dev).to(dtype)
+    k = torch.randn(num_pages, kv_heads, head_dim // 8, page_size, 8, device=dev).to(dtype)      # keys chunk by chunk in a page
     v = torch.randn(num_pages, kv_heads, head_dim, page_size, device=dev).to(dtype)
     row_pos = torch.tensor([p + i for p, n in segs for i in range(n)], dtype=torch.int32, device=dev)
     row_seg = torch.tensor([s for s, (_, n) in enumerate(segs) for _ in range(n)], dtype=torch.int32, device=dev)
@@ -99,7 +99,7 @@ def _rope_kv(ops, dev, report):
         report(f"rope q {dtype}", _err(qkv.view(-1, heads + 2 * kv_heads, d)[:, :heads], rotated[:, :heads]), tol)
         pages = tables[row_seg.long(), (row_pos // ps).long()].long()
         offs = (row_pos % ps).long()
-        report(f"rope k pages {dtype}", _err(k[pages, :, offs, :], rotated[:, heads:]), tol)
+        report(f"rope k pages {dtype}", _err(k[pages, :, :, offs, :].reshape(len(pages), kv_heads, d), rotated[:, heads:]), tol)
         report(f"v pages {dtype}", _err(v[pages, :, :, offs], view[:, heads + kv_heads:]), 0.0)
 
 
@@ -116,7 +116,7 @@ def _attention(ops, dev, report):
                 lo = max(0, pos + 1 - window) if window else 0
                 keys = torch.arange(lo, pos + 1, device=dev)
                 pg, off = tables[seg, (keys // ps).long()].long(), (keys % ps).long()
-                kk = k[pg, :, off, :].double().repeat_interleave(heads // kv_heads, 1)      # [n, heads, d]
+                kk = k[pg, :, :, off, :].double().reshape(len(keys), kv_heads, d).repeat_interleave(heads // kv_heads, 1)      # [n, heads, d]
                 vv = v[pg, :, :, off].double().repeat_interleave(heads // kv_heads, 1)
                 sc = torch.einsum("hd,nhd->hn", q[r].double().view(heads, d), kk) * d ** -0.5
                 want[r] = torch.einsum("hn,nhd->hd", torch.softmax(sc, -1), vv)

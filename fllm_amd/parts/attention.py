@@ -18,6 +18,7 @@ from .base import INIT_BIAS, INIT_MATRIX, KVNeed, Mixer, add_and_prepare, take_p
 
 class PagedAttention(Mixer):
     graph_safe = True      # forward launches kernels only: no per-step decision on the host
+    KEY_CHUNK = 8          # values of a key that lie together in a page (csrc/common.h, key_offset)
 
     @classmethod
     def tensor_shapes(cls, spec):
@@ -41,6 +42,9 @@ class PagedAttention(Mixer):
             raise ValueError(f"head count {self.heads} is not a multiple of key/value head count {self.kv_heads}")
         if self.window is not None and self.window <= 0:
             raise ValueError("an attention window must be positive")
+        if self.head_dim % self.KEY_CHUNK != 0:
+            raise ValueError(f"head size {self.head_dim}: the attention kernels store keys in chunks of {self.KEY_CHUNK} values, "
+                             f"head sizes come in steps of {self.KEY_CHUNK}")
         if spec.get("value_head_dim") not in (None, self.head_dim):
             raise ValueError(f"this attention's kernels read keys and values of one width: values of "
                              f"{spec.get('value_head_dim')} beside keys of {self.head_dim} need a mixer of their own")
@@ -88,7 +92,8 @@ class PagedAttention(Mixer):
         return torch.tensor([h * head_dim + j for h in range(heads) for j in one], dtype=torch.long)
 
     def cache_need(self):
-        return KVNeed(self.kv_heads, self.head_dim, self.head_dim, self.window)     # keys and values of one width: what the kernels take
+        # keys and values of one width, keys in chunks of 8 values (16 bytes in bfloat16): what the kernels take
+        return KVNeed(self.kv_heads, self.head_dim, self.head_dim, self.window, key_chunk=self.KEY_CHUNK)
 
     def forward(self, ctx, h, residual, binding, branch=None):
         rt, ops = self.rt, self.rt.ops

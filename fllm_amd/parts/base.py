@@ -65,17 +65,28 @@ INIT_BIAS = "bias"         # N(0, 0.02)
 class KVNeed:
     """Per token, keys of `kv_heads` heads of `k_dim` values and values of as many heads of `v_dim` (`k_dim` when left
     out; 0: the mixer caches keys alone); `window` keys back (the token itself included) or all of them when None.
-    The pages are shaped from both widths; what a mixer's kernels can read is the mixer's matter."""
+    The pages are shaped from both widths; what a mixer's kernels can read is the mixer's matter.  `key_chunk`: 0 stores
+    a token's keys together ([page][kv_head][token][k_dim]); n > 0 stores them in chunks of n values, chunk by chunk over
+    the tokens of a page ([page][kv_head][k_dim / n][token][n]), the order this library's attention kernels read."""
     kv_heads: int
     k_dim: int
     v_dim: Optional[int] = None
     window: Optional[int] = None
+    key_chunk: int = 0
 
     def __post_init__(self):
         if self.v_dim is None:
             object.__setattr__(self, "v_dim", self.k_dim)
         if self.kv_heads <= 0 or self.k_dim <= 0 or self.v_dim < 0:
             raise ValueError(f"a cache of {self.kv_heads} heads with keys of {self.k_dim} and values of {self.v_dim}")
+        if self.key_chunk < 0 or (self.key_chunk and self.k_dim % self.key_chunk != 0):
+            raise ValueError(f"keys of {self.k_dim} values cannot be stored in chunks of {self.key_chunk}")
+
+    def key_page_shape(self, page_size: int) -> Tuple[int, ...]:
+        """Shape of the keys of one key/value head in one page."""
+        if self.key_chunk:
+            return (self.k_dim // self.key_chunk, page_size, self.key_chunk)
+        return (page_size, self.k_dim)
 
 
 @dataclass(frozen=True)

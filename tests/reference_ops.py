@@ -120,7 +120,8 @@ class ReferenceOps:
                 continue
             page = int(tables[seg, pos // page_size])
             off = pos % page_size
-            k_pages[page, :, off, :] = view[r, heads:heads + kv_heads, :]
+            # keys lie chunk by chunk in a page: [page][kv_head][head_dim / 8][token][8]
+            k_pages[page, :, :, off, :] = view[r, heads:heads + kv_heads, :].reshape(kv_heads, head_dim // 8, 8)
             v_pages[page, :, :, off] = view[r, heads + kv_heads:, :]
 
     def attention_workspace_bytes(self, rows, heads, kv_heads, head_dim, max_context):
@@ -141,7 +142,7 @@ class ReferenceOps:
             keys = torch.arange(lo, n, device=q.device)
             pages = tables[seg, (keys // page_size).long()].long()
             offs = (keys % page_size).long()
-            k = k_pages[pages, :, offs, :].double()          # [n, kv_heads, d]
+            k = k_pages[pages, :, :, offs, :].double().reshape(len(keys), kv_heads, head_dim)     # [n, kv_heads, d]
             v = v_pages[pages, :, :, offs].double()          # [n, kv_heads, d]
             qr = q[r].double().view(heads, head_dim)
             for h in range(heads):

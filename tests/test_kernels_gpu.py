@@ -437,7 +437,7 @@ def test_norm_qkv_rope_store(ops, ref, heads, kv_heads, head_dim, rope_dims, pag
     for r in range(rows):
         if row_seg[r] >= 0:
             untouched[int(tables[int(row_seg[r]), int(row_pos[r]) // page_size]), int(row_pos[r]) % page_size] = False
-    assert torch.equal(k_gpu.cpu().permute(0, 2, 1, 3)[untouched], k0.permute(0, 2, 1, 3)[untouched])
+    assert torch.equal(k_gpu.cpu().permute(0, 3, 1, 2, 4)[untouched], k0.permute(0, 3, 1, 2, 4)[untouched])
     assert torch.equal(v_gpu.cpu().permute(0, 3, 1, 2)[untouched], v0.permute(0, 3, 1, 2)[untouched])
     # reading another entry's cache: queries only
     k2, v2 = k0.to(DEV), v0.to(DEV)
@@ -521,7 +521,9 @@ def test_swiglu(ops, ref, dtype, rows, inter):
 
 # ---------------------------------------------------------------------------------------------
 def make_pages(g, num_pages, kv_heads, page_size, head_dim, dtype):
-    k = torch.randn(num_pages, kv_heads, page_size, head_dim, generator=g).to(dtype)
+    """Pages as the kernels lay them out: keys chunk by chunk [page][kv_head][head_dim / 8][token][8], values
+    [page][kv_head][head_dim][token]."""
+    k = torch.randn(num_pages, kv_heads, head_dim // 8, page_size, 8, generator=g).to(dtype)
     v = torch.randn(num_pages, kv_heads, head_dim, page_size, generator=g).to(dtype)
     return k, v
 
@@ -609,7 +611,7 @@ def attention_case(ops, ref, dtype, heads, kv_heads, head_dim, page_size, segs, 
             page, off = int(tables[s, far // page_size]), far % page_size
             for h in range(heads):
                 q = qkv[r - 1, h * head_dim:(h + 1) * head_dim].float()
-                k[page, h // (heads // kv_heads), off, :] = (q * (12.0 / q.norm() ** 2 * math.sqrt(head_dim))).to(dtype)
+                k[page, h // (heads // kv_heads), :, off, :] = (q * (12.0 / q.norm() ** 2 * math.sqrt(head_dim))).to(dtype).view(-1, 8)
     q = qkv[:, : heads * head_dim]
     scale = head_dim ** -0.5
     want = ref.attention(q, k, v, tables, row_pos, row_seg, seg_start, torch.empty(rows, heads * head_dim, dtype=torch.float64),
@@ -760,7 +762,7 @@ def test_attention_with_scores_biased_by_distance(ops, ref, dtype, heads, kv_hea
     assert (biased.float() - plain.float()).abs().max() > 0.05
     from fllm_amd.kernels import KernelError
     q = torch.zeros(1, heads * head_dim, dtype=dtype, device=DEV)
-    pages = torch.zeros(2, kv_heads, 16, head_dim, dtype=dtype, device=DEV)
+    pages = torch.zeros(2, kv_heads, head_dim // 8, 16, 8, dtype=dtype, device=DEV)
     ints = lambda *v: torch.tensor(v, dtype=torch.int32, device=DEV)
     with pytest.raises(KernelError, match="head_slopes"):        # one slope too few
         ops.attention(q, pages, pages.view(2, kv_heads, head_dim, 16), ints(0).view(1, 1), ints(0), ints(0), ints(0, 1),

@@ -112,7 +112,7 @@ def test_attention_part(rt, heads, kv_heads, head_dim, window, rows, first):
     need = part.cache_need()
     assert (need.kv_heads, need.k_dim, need.v_dim, need.window) == (kv_heads, head_dim, head_dim, window)
     ctx, pages = whole_prompt_context(rows)
-    binding = CacheBinding(group=0, k_pages=torch.zeros(pages, kv_heads, 16, head_dim, dtype=rt.dtype, device=DEV),
+    binding = CacheBinding(group=0, k_pages=torch.zeros(pages, kv_heads, head_dim // 8, 16, 8, dtype=rt.dtype, device=DEV),
                            v_pages=torch.zeros(pages, kv_heads, head_dim, 16, dtype=rt.dtype, device=DEV), page_size=16,
                            writes=True)
     x = torch.randn(rows, hidden, generator=torch.Generator().manual_seed(7)).to(rt.dtype)
