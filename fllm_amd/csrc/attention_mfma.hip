@@ -179,7 +179,9 @@ attn_tile_kernel(AttnArgs p) {
     for (int k0 = kbegin; k0 <= p_last; k0 += KT) {
         __syncthreads();   // the previous tile has been read
         for (int ch = threadIdx.x; ch < KT * D / 8; ch += kThreads) {
-            const int key = ch % KT, dc = ch / KT;       // neighbouring threads take neighbouring keys: that is how they lie in a page
+            // the chunks in the order in which they lie in a page: token fastest, then the key's chunks, then the tile's pages
+            const int wsh = psh < 6 ? psh : 6;           // log2 of the tokens of a page that lie in this tile (KT is 64)
+            const int key = ((ch >> (wsh + LD - 3)) << wsh) | (ch & ((1 << wsh) - 1)), dc = (ch >> wsh) & (D / 8 - 1);
             const int kabs = k0 + key;
             bf16x8_t v = zero8();
             if (kabs >= lo_tile && kabs <= p_last) {
@@ -351,7 +353,10 @@ attn_tile32_kernel(AttnArgs p) {
 #pragma unroll
     for (int c = 0; c < CH; c++) {
         const int ch = threadIdx.x + c * kThreads;
-        const int key = ch & (KT - 1), dc = ch / KT;     // neighbouring threads take neighbouring keys: that is how they lie in a page
+        // the chunks in the order in which they lie in a page (token fastest, then the key's chunks, then the tile's pages):
+        // a load instruction of a wave reads 1 KiB in a row where a page holds 16 tokens or more
+        const int wsh = psh < 6 ? psh : 6;               // log2 of the tokens of a page that lie in this tile (KT is 64)
+        const int key = ((ch >> (wsh + LD - 3)) << wsh) | (ch & ((1 << wsh) - 1)), dc = (ch >> wsh) & (D / 8 - 1);
         k_key[c] = key;
         k_in_page[c] = (int)key_offset(0, nkv, kvh, ps, D, key & pmask, dc * 8);
         // A key's row in LDS: bits 2 and 3 of the key swapped, which is where the products read it (row q of a 32-key
