@@ -34,6 +34,7 @@ int fllm_option_x_direct(void);
 // products of 17 to 64 rows: 1 (default) the kernel that suits the shape; 0 activations pass through LDS in chunks wherever
 // that kernel can serve; 2 a K slice of the activations stays in LDS wherever that kernel can serve
 int fllm_option_slab(void);
+int fllm_option_wide_waves(void);
 // 1: decode-shaped products of up to 8 rows use 8-row weight tiles with two K halves a product (default); 0: 16-row tiles
 int fllm_option_dual_k(void);
 

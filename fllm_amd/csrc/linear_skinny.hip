@@ -615,18 +615,19 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
 // b / S, b / S + G / S, ...  With S > 1 a wave leaves its tile's sums in the workspace and counts
 // the tile; the wave that counts the last slice adds the S partial sums in slice order and runs
 // the epilogue (as in the resident kernel).
-template <int MT, int EPI>
-__global__ void __launch_bounds__(4 * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// WT: the weights come from their tile-major copy (fllm_tile_weights, fllm_tile_weights_gate_up), K a multiple of 256.
+template <int MT, int EPI, bool WT = false, int WAVES = 4>
+__global__ void __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
 skinny_wide_kernel(SkinnyArgs a) {
-    constexpr int WAVES = 4, THREADS = WAVES * kWave;
+    constexpr int THREADS = WAVES * kWave;
     constexpr int KC = 256;                        // columns per chunk
     constexpr int KS = KC / 32;                    // MFMA k-steps per chunk
     constexpr int XP = KC + 8;                     // pitch of an activation row in LDS
     constexpr int ROWS = MT * 16;
-    constexpr int XL = ROWS * (KC / 8) / THREADS;  // 16-byte activation loads per thread and chunk
+    constexpr int XPIECES = ROWS * (KC / 8);       // 16-byte pieces of a chunk of activations
+    constexpr int XL = (XPIECES + THREADS - 1) / THREADS;   // loads per thread and chunk
     constexpr int NT = EPI == EPI_SWIGLU ? 8 : 16; // outputs per row and tile
     constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
-    static_assert(ROWS * (KC / 8) % THREADS == 0, "the chunk divides evenly over the threads");
     __shared__ __attribute__((aligned(16))) bf16_t xs[2][ROWS * XP];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int r = lane & 15, g = lane >> 4;
@@ -657,9 +658,16 @@ skinny_wide_kernel(SkinnyArgs a) {
         if (row >= n_out) row = n_out - 1;    // past the end: computed from a valid row, never stored
         if (EPI == EPI_SWIGLU) row += (r >> 3) * n_out;
         const int kb = w_chunk * KC + g * 8;
-        const bf16_t *wp = a.w + (size_t)row * K + ks0;
+        if (WT) {
+            // a chunk is two blocks of 128 columns of the tile, each 4 KiB in the order the lanes take it
+            const bf16_t *wp = a.w_tiles + (size_t)min(tile, ntiles - 1) * 16 * K + (size_t)((ks0 + w_chunk * KC) >> 7) * 2048 + lane * 8;
 #pragma unroll
-        for (int u = 0; u < KS; u++) buf[u] = *(const bf16x8_t *)(live ? wp + min(kb + u * 32, kcn - 8) : zeros);
+            for (int u = 0; u < KS; u++) buf[u] = *(const bf16x8_t *)(live ? wp + (u >> 2) * 2048 + (u & 3) * 512 : zeros);
+        } else {
+            const bf16_t *wp = a.w + (size_t)row * K + ks0;
+#pragma unroll
+            for (int u = 0; u < KS; u++) buf[u] = *(const bf16x8_t *)(live ? wp + min(kb + u * 32, kcn - 8) : zeros);
+        }
         if (++w_chunk == nchunks) w_chunk = 0, w_item++;
     };
     // activations: the chunk index within the slice is all that matters (every item walks the same slice)
@@ -669,7 +677,7 @@ skinny_wide_kernel(SkinnyArgs a) {
         for (int i = 0; i < XL; i++) {
             const int idx = threadIdx.x + i * THREADS;
             const int m = idx / (KC / 8), c = (idx - m * (KC / 8)) * 8 + chunk * KC;
-            xr[i] = *(const bf16x8_t *)((m < M && c < kcn) ? x + (size_t)m * a.ldx + ks0 + c : zeros);
+            xr[i] = *(const bf16x8_t *)((m < M && c < kcn && idx < XPIECES) ? x + (size_t)m * a.ldx + ks0 + c : zeros);
         }
     };
     auto store_x = [&](int buffer) {
@@ -677,7 +685,7 @@ skinny_wide_kernel(SkinnyArgs a) {
         for (int i = 0; i < XL; i++) {
             const int idx = threadIdx.x + i * THREADS;
             const int m = idx / (KC / 8), c = (idx - m * (KC / 8)) * 8;
-            *(bf16x8_t *)(&xs[buffer][m * XP + c]) = xr[i];
+            if (XPIECES % THREADS == 0 || idx < XPIECES) *(bf16x8_t *)(&xs[buffer][m * XP + c]) = xr[i];
         }
     };
 
@@ -729,17 +737,15 @@ skinny_wide_kernel(SkinnyArgs a) {
             const int m = mt * 16 + r;
             bool finish = tile < ntiles;
             if (S > 1 && tile < ntiles) {       // wave-uniform: the whole wave takes part in the hand-over
-                float *part = a.ws + (((size_t)tile * S + sl) * MT + mt) * RT * kWave * 4 + (size_t)lane * 4;
+                const __amdgpu_buffer_rsrc_t wsb = workspace_buffer(a.ws);
+                const unsigned int part = (unsigned int)(((((size_t)tile * S + sl) * MT + mt) * RT * kWave + lane) * 16);
                 if (owner && m < M) {
 #pragma unroll
-                    for (int t = 0; t < RT; t++)
-#pragma unroll
-                        for (int i = 0; i < 4; i++)
-                            __hip_atomic_store(part + t * kWave * 4 + i, s[t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    for (int t = 0; t < RT; t++) hand_over(wsb, part + t * kWave * 16, s[t]);
                 }
                 if (mt == MT - 1) {
-                    // every access to the workspace goes to the device's point of coherence by itself: it is enough
-                    // that the wave's partial sums have arrived there before the tile is counted
+                    // the pieces pass by the caches on both ways: it is enough that the wave's own have arrived in
+                    // memory before the tile is counted
                     parts_published();
                     int seen = 0;
                     if (lane == 0) seen = __hip_atomic_fetch_add(a.counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -750,18 +756,28 @@ skinny_wide_kernel(SkinnyArgs a) {
 #pragma unroll
                         for (int mt2 = 0; mt2 < MT; mt2++) {
                             const int m2 = mt2 * 16 + r;
-                            if (!owner || m2 >= M || nb >= n_out) continue;
+                            const bool mine = owner && m2 < M && nb < n_out;
                             f32x4_t t2[RT];
 #pragma unroll
                             for (int t = 0; t < RT; t++) t2[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-                            for (int s2 = 0; s2 < S; s2++) {
-                                const float *src = a.ws + (((size_t)tile * S + s2) * MT + mt2) * RT * kWave * 4 + (size_t)lane * 4;
+                            // the parts of up to eight slices are asked for together (one trip to memory, not one a
+                            // slice) and added in slice order; every lane loads, so that no load sits behind a branch
+                            for (int s0 = 0; s0 < S; s0 += 8) {
+                                f32x4_t pv[8][RT];
 #pragma unroll
-                                for (int t = 0; t < RT; t++)
+                                for (int j = 0; j < 8; j++) {
+                                    const int s2 = s0 + j < S ? s0 + j : s0;
+                                    const unsigned int src = (unsigned int)(((((size_t)tile * S + s2) * MT + mt2) * RT * kWave + lane) * 16);
 #pragma unroll
-                                    for (int i = 0; i < 4; i++)
-                                        t2[t][i] += __hip_atomic_load(src + t * kWave * 4 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                    for (int t = 0; t < RT; t++) pv[j][t] = take_over(wsb, src + t * kWave * 16);
+                                }
+#pragma unroll
+                                for (int j = 0; j < 8; j++)
+#pragma unroll
+                                    for (int t = 0; t < RT; t++)
+                                        if (s0 + j < S) t2[t] += pv[j][t];
                             }
+                            if (!mine) continue;
                             EpilogueOperands eo;
                             epilogue<PRO_BF16, EPI, RT>(a, t2, 0.f, m2, nb, n_out, eo);
                         }
@@ -1130,7 +1146,10 @@ bool tiles_fit(int N, int K) { return N >= 16 && K >= 1024 && K % 1024 == 0; }
 
 // tiles[T][B][u][lane][8] = w[16 T + lane % 16][128 B + 32 u + 8 (lane / 16) ...]: tile T of 16 rows, block B of 128 columns,
 // k-step u of 32, and inside it the 16 bytes of each of the 64 lanes of a wave in lane order; rows past N are zeros
-__global__ void __launch_bounds__(256) tile_weights_kernel(const bf16_t *__restrict__ w, bf16_t *__restrict__ tiles, int N, int K, size_t pieces) {
+// `half_rows` > 0: w is a gate matrix on top of an up matrix of `half_rows` rows each, and tile T is rows 8 T .. 8 T + 7 of
+// the one followed by the same rows of the other, as the SwiGLU epilogue wants them
+__global__ void __launch_bounds__(256) tile_weights_kernel(const bf16_t *__restrict__ w, bf16_t *__restrict__ tiles, int N, int K, size_t pieces,
+                                                           int half_rows) {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     const int blocks = K / 128;
     for (size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x; v < pieces; v += stride) {
@@ -1138,9 +1157,16 @@ __global__ void __launch_bounds__(256) tile_weights_kernel(const bf16_t *__restr
         const size_t tb = v >> 8;
         const int B = (int)(tb % blocks);
         const size_t T = tb / blocks;
-        const size_t n = T * 16 + (lane & 15);
+        const int r = lane & 15;
+        size_t n = T * 16 + r;
+        bool there = n < (size_t)N;
+        if (half_rows > 0) {
+            const size_t o = T * 8 + (r & 7);
+            there = o < (size_t)half_rows;
+            n = o + (size_t)(r >> 3) * half_rows;
+        }
         const int k = B * 128 + u * 32 + (lane >> 4) * 8;
-        *(bf16x8_t *)(tiles + v * 8) = n < (size_t)N ? *(const bf16x8_t *)(w + n * K + k) : zero8();
+        *(bf16x8_t *)(tiles + v * 8) = there ? *(const bf16x8_t *)(w + n * K + k) : zero8();
     }
 }
 
@@ -1194,29 +1220,37 @@ int launch_resident(const SkinnyArgs &a, hipStream_t stream) {
     }
 }
 
+template <int MT, int EPI, bool WT, int WAVES>
+int launch_wide_kernel(const SkinnyArgs &a, int grid, hipStream_t stream) {
+    hipLaunchKernelGGL((skinny_wide_kernel<MT, EPI, WT, WAVES>), dim3(grid), dim3(WAVES * kWave), 0, stream, a);
+    return fllm_check_launch("linear_wide");
+}
+
 template <int MT, int EPI>
 int launch_wide(SkinnyArgs a, hipStream_t stream) {
-    constexpr int WAVES = 4;
     constexpr int NT = EPI == EPI_SWIGLU ? 8 : 16;
     constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
     const int n_out = EPI == EPI_SWIGLU ? a.N / 2 : a.N;
     const int ntiles = (n_out + NT - 1) / NT;
-    const int ngroups = (ntiles + WAVES - 1) / WAVES;
     void *base = nullptr;
     size_t bytes = 0;
     const bool have_ws = fllm_device_workspace(&base, &bytes);
-    const fllm_plan::ChunkPlan p = fllm_plan::plan_chunks(a.K, ntiles, MT, RT, bytes, have_ws, device_cus(), fllm_option_linear_slices());
+    // workgroups of seven or eight waves only with the weights' tile-major copy (they were measured with it)
+    const bool tiled = a.w_tiles != nullptr && a.K % 256 == 0;
+    const fllm_plan::ChunkPlan p =
+        tiled ? fllm_plan::plan_chunks_balanced(a.K, ntiles, MT, RT, bytes, have_ws, device_cus(), fllm_option_linear_slices(),
+                                                fllm_option_wide_waves())
+              : fllm_plan::plan_chunks(a.K, ntiles, MT, RT, bytes, have_ws, device_cus(), fllm_option_linear_slices(), 4);
     a.S = p.S;
     a.slice = p.slice;
     if (p.S > 1) {
         a.counters = (int *)base;
         a.ws = (float *)((unsigned char *)base + kWorkspaceCounterBytes);
     }
-    const int per_slice = p.grid / p.S;
-    const int S = p.S;
-    (void)ngroups;
-    hipLaunchKernelGGL((skinny_wide_kernel<MT, EPI>), dim3(per_slice * S), dim3(WAVES * kWave), 0, stream, a);
-    return fllm_check_launch("linear_wide");
+    if (!tiled) return launch_wide_kernel<MT, EPI, false, 4>(a, p.grid, stream);
+    if (p.waves == 7) return launch_wide_kernel<MT, EPI, true, 7>(a, p.grid, stream);
+    if (p.waves == 8) return launch_wide_kernel<MT, EPI, true, 8>(a, p.grid, stream);
+    return launch_wide_kernel<MT, EPI, true, 4>(a, p.grid, stream);
 }
 
 using fllm_plan::SlabPlan;
@@ -1450,16 +1484,50 @@ extern "C" int fllm_tile_weights(const void *w, void *tiles, int N, int K, hipSt
     const size_t pieces = fllm_weight_tiles_elements(N, K) / 8;
     const size_t want = (pieces + 255) / 256;
     hipLaunchKernelGGL(tile_weights_kernel, dim3((unsigned int)(want < 65536 ? want : 65536)), dim3(256), 0, stream, (const bf16_t *)w,
-                       (bf16_t *)tiles, N, K, pieces);
+                       (bf16_t *)tiles, N, K, pieces, 0);
     return fllm_check_launch("tile_weights");
+}
+
+extern "C" size_t fllm_weight_tiles_elements_gate_up(int inter, int K) { return (size_t)((inter + 7) / 8) * 16 * (size_t)K; }
+
+// The copy for the gate/up product with its SwiGLU epilogue: w is [2 inter][K], gate rows first.
+extern "C" int fllm_tile_weights_gate_up(const void *w, void *tiles, int inter, int K, hipStream_t stream) {
+    FLLM_REQUIRE(tiles_fit(2 * inter, K), "tile_weights_gate_up: takes matrices whose width is a multiple of 1,024 (inter=%d K=%d)", inter, K);
+    FLLM_REQUIRE(w != nullptr && tiles != nullptr && aligned16(w) && aligned16(tiles), "tile_weights_gate_up: operands must be there and 16-byte aligned");
+    const size_t pieces = fllm_weight_tiles_elements_gate_up(inter, K) / 8;
+    const size_t want = (pieces + 255) / 256;
+    hipLaunchKernelGGL(tile_weights_kernel, dim3((unsigned int)(want < 65536 ? want : 65536)), dim3(256), 0, stream, (const bf16_t *)w,
+                       (bf16_t *)tiles, 2 * inter, K, pieces, inter);
+    return fllm_check_launch("tile_weights_gate_up");
+}
+
+// fllm_gate_up_swiglu for 17..64 rows with the weights' tile-major copy (fllm_tile_weights_gate_up; may be null)
+extern "C" int fllm_gate_up_swiglu_tiled(const void *x, int ldx, const void *w_gate_up, const void *w_tiles, const float *bias, void *out,
+                                         int M, int inter, int K, hipStream_t stream) {
+    FLLM_REQUIRE(M >= 17 && M <= 64 && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && inter > 0,
+                 "gate_up_swiglu_tiled: takes 17..64 rows and K, ldx in steps of 8 (M=%d K=%d ldx=%d)", M, K, ldx);
+    FLLM_REQUIRE(aligned16(x) && aligned16(w_gate_up) && (w_tiles == nullptr || aligned16(w_tiles)),
+                 "gate_up_swiglu_tiled: operands must be 16-byte aligned");
+    SkinnyArgs a = {};
+    a.x = x;
+    a.ldx = ldx;
+    a.w = (const bf16_t *)w_gate_up;
+    a.w_tiles = (const bf16_t *)w_tiles;
+    a.bias = bias;
+    a.out = out;
+    a.ldo = inter;
+    a.M = M;
+    a.N = 2 * inter;
+    a.K = K;
+    return dispatch_wide<EPI_SWIGLU>(a, stream);
 }
 
 // out += x w^T (+ bias) for 1..16 bfloat16 rows and a float32 `out`, as fllm_linear in mode 2; `w_tiles` (may be null):
 // the tile-major copy of w, which the kernel streams instead where the launch it chooses can.
 extern "C" int fllm_linear_add_tiled(const void *x, int ldx, const void *w, const void *w_tiles, const float *bias, float *out, int ldo,
                                      int M, int N, int K, hipStream_t stream) {
-    FLLM_REQUIRE(M >= 1 && M <= 16 && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && ldx >= K && ldo >= N,
-                 "linear_add_tiled: takes 1..16 rows, K and ldx in steps of 8 (M=%d N=%d K=%d ldx=%d ldo=%d)", M, N, K, ldx, ldo);
+    FLLM_REQUIRE(M >= 1 && M <= 64 && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && ldx >= K && ldo >= N,
+                 "linear_add_tiled: takes 1..64 rows, K and ldx in steps of 8 (M=%d N=%d K=%d ldx=%d ldo=%d)", M, N, K, ldx, ldo);
     FLLM_REQUIRE(aligned16(x) && aligned16(w) && out != nullptr && (w_tiles == nullptr || aligned16(w_tiles)),
                  "linear_add_tiled: operands must be there and 16-byte aligned");
     SkinnyArgs a = {};
@@ -1473,7 +1541,7 @@ extern "C" int fllm_linear_add_tiled(const void *x, int ldx, const void *w, cons
     a.M = M;
     a.N = N;
     a.K = K;
-    const int rc = launch_resident<PRO_BF16, EPI_ADD>(a, stream);
+    const int rc = M <= 16 ? launch_resident<PRO_BF16, EPI_ADD>(a, stream) : dispatch_wide<EPI_ADD>(a, stream);
     FLLM_REQUIRE(rc != 1, "linear_add_tiled: shape M=%d K=%d does not fit the staging area", M, K);
     return rc;
 }

@@ -76,25 +76,29 @@ inline int resident_groups(const ResidentPlan &p, int ntiles, int cus) {
 
 // ---- products of 17 to 64 rows, activations in chunks through LDS ----
 struct ChunkPlan {
-    int S = 1, slice = 0, grid = 0;
+    int S = 1, slice = 0, grid = 0, waves = 4;
 };
 inline size_t chunk_workspace_need(int ntiles, int S, int mt, int rt) {
     return kCounterBytes + (size_t)ntiles * S * mt * rt * kWaveLanes * 4 * kF32;
 }
-inline ChunkPlan plan_chunks(int K, int ntiles, int mt, int rt, size_t ws_bytes, bool have_ws, int cus, int forced) {
-    const int ngroups = (ntiles + 3) / 4;
-    const int slots = 2 * cus;        // two workgroups of four waves a compute unit
+// `waves`: row tiles (waves) of a workgroup; a compute unit holds eight waves of this kernel, two workgroups of four or
+// one of five to eight
+inline ChunkPlan plan_chunks(int K, int ntiles, int mt, int rt, size_t ws_bytes, bool have_ws, int cus, int forced, int waves = 4) {
+    const int ngroups = (ntiles + waves - 1) / waves;
+    const int slots = 8 / waves * cus;
     // K slices: as many as fill the chip with the row groups there are, each at least two chunks long
     int S = 1;
     while (S < 8 && ngroups * S * 2 <= slots && (K + 2 * S - 1) / (2 * S) >= 512) S *= 2;
     if (forced > 0) S = forced;
     while (S > 1) {
-        if (have_ws && chunk_workspace_need(ntiles, S, mt, rt) <= ws_bytes && (size_t)ntiles * sizeof(int) <= kCounterBytes &&
+        const size_t need = chunk_workspace_need(ntiles, S, mt, rt);      // the kernel's offsets into it are 32 bits
+        if (have_ws && need <= ws_bytes && need - kCounterBytes <= 0x7fffffffu && (size_t)ntiles * sizeof(int) <= kCounterBytes &&
             (K + S - 1) / S >= 256)
             break;
         S /= 2;
     }
     ChunkPlan p;
+    p.waves = waves;
     p.S = S;
     p.slice = ((K + S - 1) / S + 255) / 256 * 256;
     if (S > 1 && (long)(S - 1) * p.slice >= K) p.S = S = (K + p.slice - 1) / p.slice;   // no empty slice
@@ -103,6 +107,30 @@ inline ChunkPlan plan_chunks(int K, int ntiles, int mt, int rt, size_t ws_bytes,
     if (per_slice > ngroups) per_slice = ngroups;
     p.grid = per_slice * S;
     return p;
+}
+// What the busiest compute unit streams under a plan, in weight rows x columns: its workgroups' row tiles over their
+// slices, as often as the row groups of a slice come round.
+inline long chunk_plan_cost(const ChunkPlan &p, int ntiles) {
+    const int ngroups = (ntiles + p.waves - 1) / p.waves;
+    const int per_slice = p.grid / p.S;
+    const long rounds = (ngroups + per_slice - 1) / per_slice;
+    return rounds * (8 / p.waves) * p.waves * (long)p.slice;
+}
+// The number of waves (four, seven or eight) whose plan leaves the least to the busiest compute unit; four on a tie.
+// 1,792 tiles over 256 compute units are seven a unit: workgroups of seven waves take a tile each in one round, where
+// four or eight waves leave an eighth of the device idle in the last round.
+inline ChunkPlan plan_chunks_balanced(int K, int ntiles, int mt, int rt, size_t ws_bytes, bool have_ws, int cus, int forced,
+                                      int forced_waves) {
+    if (forced_waves == 4 || forced_waves == 7 || forced_waves == 8)
+        return plan_chunks(K, ntiles, mt, rt, ws_bytes, have_ws, cus, forced, forced_waves);
+    ChunkPlan best = plan_chunks(K, ntiles, mt, rt, ws_bytes, have_ws, cus, forced, 4);
+    long best_cost = chunk_plan_cost(best, ntiles);
+    for (int waves = 7; waves <= 8; waves++) {
+        const ChunkPlan p = plan_chunks(K, ntiles, mt, rt, ws_bytes, have_ws, cus, forced, waves);
+        const long cost = chunk_plan_cost(p, ntiles);
+        if (cost < best_cost) best = p, best_cost = cost;
+    }
+    return best;
 }
 
 // ---- products of 17 to 64 rows, a K slice of the activations resident in LDS ----

@@ -33,6 +33,8 @@ static int g_linear_slices = 0;
 static int g_dual_k = 1;
 static int g_x_direct = 1;
 int fllm_option_x_direct(void) { return g_x_direct; }
+static int g_wide_waves = 0;      // 0: planned
+int fllm_option_wide_waves(void) { return g_wide_waves; }
 static int g_slab = 1;
 int fllm_option_slab(void) { return g_slab; }
 static int g_fused_merge = 1;
@@ -53,6 +55,10 @@ extern "C" int fllm_set_option(const char *name, int value) {
     }
     if (strcmp(name, "linear.slab") == 0) {
         g_slab = value < 0 ? 0 : (value > 2 ? 2 : value);
+        return 0;
+    }
+    if (strcmp(name, "linear.wide_waves") == 0) {
+        g_wide_waves = (value == 4 || value == 7 || value == 8) ? value : 0;
         return 0;
     }
     if (strcmp(name, "linear.x_direct") == 0) {

@@ -93,6 +93,8 @@ def load_library(build_if_missing: bool = True):
         "fllm_gate_up_swiglu": [c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_linear_add_normed": [c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_void, c_void, c_void, c_void, c_void, c_void],
         "fllm_tile_weights": [c_void, c_void, c_int, c_int, c_void],
+        "fllm_tile_weights_gate_up": [c_void, c_void, c_int, c_int, c_void],
+        "fllm_gate_up_swiglu_tiled": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_linear_add_tiled": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_void],
         "fllm_scaled_gate_up_swiglu": [c_void, c_void, c_int, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_scaled_qkv_rope_store": [c_void, c_void, c_int, c_float, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void,
@@ -122,6 +124,8 @@ def load_library(build_if_missing: bool = True):
     lib.fllm_weight_tiles_supported.restype = c_int
     lib.fllm_weight_tiles_elements.argtypes = [c_int, c_int]
     lib.fllm_weight_tiles_elements.restype = c_size
+    lib.fllm_weight_tiles_elements_gate_up.argtypes = [c_int, c_int]
+    lib.fllm_weight_tiles_elements_gate_up.restype = c_size
     lib.fllm_set_fast_kernels.argtypes = [c_int]
     lib.fllm_set_fast_kernels.restype = None
     lib.fllm_attention_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int, c_int]
@@ -182,29 +186,45 @@ class Ops:
     # ---- tile-major copies of weights for decode steps --------------------------------------------------
     _tiles: Dict[int, Tuple[tuple, torch.Tensor]] = {}     # address of a weight matrix -> (its shape, its tile-major copy)
 
-    def tile_for_decode(self, w: torch.Tensor) -> bool:
-        """Keeps beside `w` (bfloat16 [N, K] on the GPU) a copy in the order in which the products of decode steps that
-        add into the residual stream read it (`fllm_tile_weights`); `linear(..., accumulate=True)` and
-        `linear_add_prepare` find it by the matrix's address and use it for steps of up to 16 rows.  The copy is given up
-        with `w`.  False: nothing was made (another type or place, a shape the kernels do not take tiles of)."""
+    def tile_for_decode(self, w: torch.Tensor, gate_up: bool = False) -> bool:
+        """Keeps beside `w` (bfloat16 [N, K] on the GPU) a copy in the order in which the products of decode steps read
+        it (`fllm_tile_weights`): `linear(..., accumulate=True)` and `linear_add_prepare` find it by the matrix's address
+        and use it for steps of up to 64 rows.  `gate_up`: w is [gate; up] and the copy is for `gate_up_swiglu` at 17 to
+        64 rows (8 gate rows and the same 8 up rows a tile, `fllm_tile_weights_gate_up`).  The copy is given up with
+        `w`.  False: nothing was made (another type or place, a shape the kernels do not take tiles of)."""
         if not (w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()):
             return False
         N, K = w.shape
-        if not self.lib.fllm_weight_tiles_supported(N, K):
+        if not self.lib.fllm_weight_tiles_supported(N, K) or (gate_up and N % 2 != 0):
             return False
         key = w.data_ptr()
-        if key in Ops._tiles and Ops._tiles[key][0] == (N, K):
+        kind = (N, K, bool(gate_up))
+        if key in Ops._tiles and Ops._tiles[key][0] == kind:
             return True
-        tiles = torch.empty(int(self.lib.fllm_weight_tiles_elements(N, K)), dtype=torch.bfloat16, device=w.device)
         with torch.cuda.device(w.device):
-            self._check(self.lib.fllm_tile_weights(_ptr(w), _ptr(tiles), N, K, self._stream()))
-        Ops._tiles[key] = ((N, K), tiles)
+            if gate_up:
+                tiles = torch.empty(int(self.lib.fllm_weight_tiles_elements_gate_up(N // 2, K)), dtype=torch.bfloat16, device=w.device)
+                self._check(self.lib.fllm_tile_weights_gate_up(_ptr(w), _ptr(tiles), N // 2, K, self._stream()))
+            else:
+                tiles = torch.empty(int(self.lib.fllm_weight_tiles_elements(N, K)), dtype=torch.bfloat16, device=w.device)
+                self._check(self.lib.fllm_tile_weights(_ptr(w), _ptr(tiles), N, K, self._stream()))
+        Ops._tiles[key] = (kind, tiles)
         weakref.finalize(w, Ops._tiles.pop, key, None)
         return True
 
-    def _tiles_of(self, w: torch.Tensor) -> Optional[torch.Tensor]:
+    def _tiles_of(self, w: torch.Tensor, gate_up: bool = False) -> Optional[torch.Tensor]:
         held = Ops._tiles.get(w.data_ptr())
-        return held[1] if held is not None and held[0] == tuple(w.shape) else None
+        return held[1] if held is not None and held[0] == (w.shape[0], w.shape[1], bool(gate_up)) else None
+
+    # 17 to 64 rows beside the GEMM library: with the tile-major copies the own products of the feed-forward (gate/up
+    # with its SwiGLU epilogue, down with the residual sum) are faster than the library's products and the SwiGLU kernel
+    # (measured at the 8B sizes, 64 / 32 rows: gate/up 48 / 44 us against 55 / 53, down 34 / 28 against 40 / 31)
+    def own_feed_forward(self, rows: int, w_gate_up: torch.Tensor, w_down: torch.Tensor) -> bool:
+        """Whether a bfloat16 step of 17 to 64 rows whose products would go to the GEMM library should take
+        `gate_up_swiglu` and `linear(..., accumulate=True)` for its feed-forward instead: when both matrices have their
+        tile-major copies."""
+        return (self.library_gemm_from is not None and self.library_gemm_from <= rows <= self.GATE_UP_SWIGLU_ROWS and bool(Ops._tiles)
+                and self._tiles_of(w_gate_up, gate_up=True) is not None and self._tiles_of(w_down) is not None)
 
     def set_fast_kernels(self, on: bool) -> None:
         """Off: bfloat16 calls run the plain kernels (tests compare the two)."""
@@ -306,6 +326,13 @@ class Ops:
             mode = OUT_STORE_F32
         if bias is not None:
             _dense(bias, "bias", torch.float32, (N,))
+        ldx = x.stride(0) if M > 1 else K
+        ldo = out.stride(0) if M > 1 else N
+        tiles = self._tiles_of(w) if mode == OUT_ADD_F32 and M <= 64 and Ops._tiles else None
+        if tiles is not None and ldx % 8 == 0 and K % 8 == 0:
+            self._check(self.lib.fllm_linear_add_tiled(_ptr(x), ldx, _ptr(w), _ptr(tiles), _ptr(bias), _ptr(out), ldo, M, N, K,
+                                                       self._stream()))
+            return out
         if (self.library_gemm_from is not None and M >= self.library_gemm_from and x.dtype == torch.bfloat16
                 and bias is None):
             if mode == OUT_STORE:
@@ -314,13 +341,6 @@ class Ops:
                 torch.mm(x, w.t(), out_dtype=torch.float32, out=out)     # bfloat16 operands, float32 sums stored as they are
             else:
                 self.add_residual(out, torch.matmul(x, w.t()))
-            return out
-        ldx = x.stride(0) if M > 1 else K
-        ldo = out.stride(0) if M > 1 else N
-        tiles = self._tiles_of(w) if mode == OUT_ADD_F32 and M <= 16 and Ops._tiles else None
-        if tiles is not None and ldx % 8 == 0 and K % 8 == 0:
-            self._check(self.lib.fllm_linear_add_tiled(_ptr(x), ldx, _ptr(w), _ptr(tiles), _ptr(bias), _ptr(out), ldo, M, N, K,
-                                                       self._stream()))
             return out
         self._check(self.lib.fllm_linear(_ptr(x), ldx, _ptr(w), _ptr(bias), _ptr(out), ldo, M, N, K, _DTYPE_CODE[x.dtype],
                                          mode, self._stream()))
@@ -436,6 +456,11 @@ class Ops:
             _dense(bias, "bias", torch.float32, (two_i,))
         _dense(out, "out", torch.bfloat16, (M, two_i // 2))
         _need(1 <= M <= self.GATE_UP_SWIGLU_ROWS and K % 8 == 0, f"gate_up_swiglu takes 1..64 rows and widths in steps of 8, not {M} x {K}")
+        tiles = self._tiles_of(w_gate_up, gate_up=True) if M >= 17 and Ops._tiles else None
+        if tiles is not None and x.stride(0) % 8 == 0:
+            self._check(self.lib.fllm_gate_up_swiglu_tiled(_ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(tiles), _ptr(bias), _ptr(out), M,
+                                                           two_i // 2, K, self._stream()))
+            return out
         self._check(self.lib.fllm_gate_up_swiglu(_ptr(x), x.stride(0) if M > 1 else K, _ptr(w_gate_up), _ptr(bias), _ptr(out), M,
                                                  two_i // 2, K, self._stream()))
         return out

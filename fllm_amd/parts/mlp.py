@@ -27,6 +27,7 @@ class GatedMLP(FeedForward):
         self.w_gate_up = torch.cat([rt.matrix(weights["gate"]), rt.matrix(weights["up"])], dim=0).contiguous()
         self.w_down = rt.matrix(weights["down"])
         rt.tile_for_decode(self.w_down)
+        rt.tile_for_decode(self.w_gate_up, gate_up=True)     # for steps of 17 to 64 rows
         gb, ub = weights.get("gate_bias"), weights.get("up_bias")
         self.b_gate_up = None
         if gb is not None or ub is not None:
@@ -53,6 +54,12 @@ class GatedMLP(FeedForward):
             ops.linear(act, self.w_down, residual, bias=self.b_down, accumulate=True)
         return True
 
+    def _own_products(self, rows: int) -> bool:
+        """17 to 64 rows: the kernel library may prefer its own products to the GEMM library's (it does when both matrices
+        have their tile-major copies)."""
+        own = getattr(self.rt.ops, "own_feed_forward", None)
+        return own is not None and self.rt.dtype == torch.bfloat16 and own(rows, self.w_gate_up, self.w_down)
+
     def forward_branch(self, ctx, h):
         """The output as a tensor of its own instead of a sum into the residual stream (large bfloat16
         steps whose products go to the GEMM library, which has no residual epilogue): the block lets
@@ -62,6 +69,8 @@ class GatedMLP(FeedForward):
         start = getattr(ops, "library_gemm_from", None)
         if rt.dtype != torch.bfloat16 or start is None or rows < start or self.b_down is not None:
             return None
+        if self._own_products(rows):
+            return None          # `forward` runs the own products, which add into the residual stream themselves
         act = rt.empty((rows, self.inter))
         if (getattr(ops, "prefers_own_gate_up", None) is not None and ops.prefers_own_gate_up(rows, self.w_gate_up)
                 and self.hidden % 8 == 0 and h.stride(0) % 8 == 0):
@@ -79,7 +88,7 @@ class GatedMLP(FeedForward):
         rows = h.shape[0]
         start = getattr(ops, "library_gemm_from", None)
         if (rt.dtype == torch.bfloat16 and rows <= getattr(ops, "GATE_UP_SWIGLU_ROWS", 0) and self.hidden % 8 == 0
-                and h.stride(0) % 8 == 0 and (start is None or rows < start)):
+                and h.stride(0) % 8 == 0 and (start is None or rows < start or self._own_products(rows))):
             # decode batches that the hand-written products serve: the activation is the epilogue of the gate/up product
             act = rt.empty((rows, self.inter))
             ops.gate_up_swiglu(h, self.w_gate_up, act, bias=self.b_gate_up)

@@ -43,7 +43,7 @@ class Runtime:
         """Norm weights and biases: float32 (exact for both storage types)."""
         return self._place(t, torch.float32)
 
-    def tile_for_decode(self, w: torch.Tensor) -> None:
+    def tile_for_decode(self, w: torch.Tensor, gate_up: bool = False) -> None:
         """For a matrix whose product adds into the residual stream in decode steps: lets the kernel library keep a
         tile-major copy beside it, where it has such kernels and the memory is there (288 GB a device are laid out for
         bandwidth: the copy costs the matrix's bytes again and takes a fifth off such a product at 8 rows)."""
@@ -55,7 +55,7 @@ class Runtime:
             if w.numel() * w.element_size() > free // 20:
                 self.decode_weight_tiles = False          # the device is filling up: no further copies
                 return
-        make(w)
+        make(w, gate_up=True) if gate_up else make(w)
 
     def forget_host_tensors(self) -> None:
         self._placed.clear()

@@ -91,7 +91,11 @@ int main() {
                                 const int nt = rt == 2 ? 8 : 16;
                                 const int ntiles = (int)ceil_div(rt == 2 ? N / 2 : N, nt);
                                 if (ntiles == 0) continue;
-                                const ChunkPlan c = plan_chunks(K, ntiles, mt, rt, ws_bytes, have_ws, cus, forced);
+                              for (int waves : {0, 4, 7, 8}) {
+                                const ChunkPlan c = plan_chunks_balanced(K, ntiles, mt, rt, ws_bytes, have_ws, cus, forced, waves);
+                                REQUIRE(c.waves == 4 || c.waves == 7 || c.waves == 8, "chunks waves %d", c.waves);
+                                REQUIRE(waves == 0 || c.waves == waves, "chunks waves %d forced %d", c.waves, waves);
+                                REQUIRE(c.grid / c.S <= (int)ceil_div(ntiles, c.waves), "chunks grid %d beyond the row groups", c.grid);
                                 slices_cover(K, c.S, c.slice, "chunks");
                                 REQUIRE(c.grid >= 1 && c.grid % c.S == 0, "chunks grid %d S %d", c.grid, c.S);
                                 if (c.S > 1) {
@@ -102,7 +106,9 @@ int main() {
                                     for (int tile : {0, ntiles - 1})
                                         for (int sl : {0, c.S - 1})
                                             touch(buf, (((size_t)tile * c.S + sl) * mt) * rt * kWaveLanes * 4, (size_t)mt * rt * kWaveLanes * 4);
+                                    REQUIRE(need - kCounterBytes <= 0x7fffffffu, "chunks workspace offsets");
                                 }
+                              }
                                 for (int norm = 0; norm < 2; norm++) {
                                     const int M = mt * 16 - 3;
                                     const SlabPlan s = plan_slab(M, ntiles, K, mt, rt, norm != 0, nt, ws_bytes, have_ws, cus, forced);

@@ -276,6 +276,75 @@ def test_products_that_add_read_the_tile_major_copy(ops, ref, M, N, K, bias):
     assert not ops.tile_for_decode(torch.zeros(64, 1024, dtype=torch.float32, device=DEV))
 
 
+@pytest.mark.parametrize("waves", [0, 4, 7, 8])
+@pytest.mark.parametrize("M,N,K,bias", [(17, 4096, 4096, False), (64, 4096, 14336, False), (33, 1000, 2048, True), (48, 24, 1024, True),
+                                        (64, 4104, 3072, False), (20, 16, 7168, False)])
+def test_products_of_17_to_64_rows_that_add_read_the_tile_major_copy(ops, ref, M, N, K, bias, waves):
+    """From 17 rows on the products that add into the residual stream take four to eight row tiles a workgroup and the
+    activations through LDS in chunks; with the tile-major copy they read 1 KiB a load instruction and may take
+    workgroups of seven or eight waves (`linear.wide_waves`; 0 lets the plan choose).  The sums are those of the row-major
+    matrix bit for bit whatever the number of waves, and the float64 product's within rounding."""
+    g = gen(53)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).to(DEV)
+    b = torch.randn(N, generator=g).to(DEV) if bias else None
+    base = torch.randn(M, N, generator=g).to(DEV)
+    from fllm_amd.kernels import _ptr
+    plain = base.clone()                                     # the row-major matrix through the same kernel
+    ops._check(ops.lib.fllm_linear_add_tiled(_ptr(x), x.stride(0), _ptr(w), None, _ptr(b), _ptr(plain), N, M, N, K, ops._stream()))
+    twin = w.clone()
+    assert ops.tile_for_decode(twin)
+    ops.set_option("linear.wide_waves", waves)
+    try:
+        tiled = ops.linear(x, twin, base.clone(), bias=b, accumulate=True)
+        again = ops.linear(x, twin, base.clone(), bias=b, accumulate=True)
+    finally:
+        ops.set_option("linear.wide_waves", 0)
+    assert torch.equal(tiled, again), "two launches differ"
+    want = ref.linear(x.cpu(), w.cpu(), base.double().cpu(), bias=None if b is None else b.cpu(), accumulate=True)
+    mag = (x.double().abs() @ w.double().abs().T).max().item()
+    close(tiled, want, 1e-6, 4e-7 * mag + 1e-6, f"tile-major M{M} N{N} K{K} waves {waves}")
+    # the slices a plan cuts K into depend on the number of waves, and with them the order of the sums: bit-equal to the
+    # row-major matrix under the plan that the row-major matrix gets (four waves)
+    ops.set_option("linear.wide_waves", 4)
+    try:
+        four = ops.linear(x, twin, base.clone(), bias=b, accumulate=True)
+    finally:
+        ops.set_option("linear.wide_waves", 0)
+    assert torch.equal(four, plain), f"M{M} N{N} K{K}: the tile-major copy gives other sums"
+
+
+@pytest.mark.parametrize("waves", [0, 4, 7, 8])
+@pytest.mark.parametrize("M,inter,K,bias", [(17, 14336, 4096, False), (64, 14336, 4096, False), (40, 1000, 2048, True), (64, 12, 1024, True),
+                                            (29, 8192, 2048, False), (64, 1796, 1024, False)])
+def test_gate_up_of_17_to_64_rows_reads_the_tile_major_copy(ops, ref, M, inter, K, bias, waves):
+    """`gate_up_swiglu` from 17 rows on with the copy that holds 8 gate rows and the same 8 up rows a tile
+    (`tile_for_decode(w, gate_up=True)`): the copy holds every element at its place, the outputs are those of the
+    row-major matrix bit for bit (one slice of K: the same products in the same order) and the float64 result's within
+    bfloat16 rounding."""
+    g = gen(59)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(2 * inter, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).to(DEV)
+    b = torch.randn(2 * inter, generator=g).to(DEV) if bias else None
+    from fllm_amd.kernels import _ptr
+    plain = torch.empty((M, inter), dtype=torch.bfloat16, device=DEV)        # the row-major matrix through the same kernel
+    ops._check(ops.lib.fllm_gate_up_swiglu_tiled(_ptr(x), x.stride(0), _ptr(w), None, _ptr(b), _ptr(plain), M, inter, K, ops._stream()))
+    twin = w.clone()
+    assert ops.tile_for_decode(twin, gate_up=True) and ops._tiles_of(twin) is None and ops._tiles_of(twin, gate_up=True) is not None
+    tiles = ops._tiles_of(twin, gate_up=True).view(-1, K // 128, 4, 4, 2, 8, 8)     # [tile][block][k-step][lane / 16][gate, up][row % 8][8]
+    back = tiles.permute(4, 0, 5, 1, 2, 3, 6).reshape(2, -1, K)                      # [gate, up][8 tile + row % 8][128 block + 32 step + 8 (lane / 16) + j]
+    assert torch.equal(back[0, :inter], w[:inter]) and torch.equal(back[1, :inter], w[inter:]) and not back[:, inter:].any()
+    ops.set_option("linear.wide_waves", waves)
+    try:
+        tiled = ops.gate_up_swiglu(x, twin, torch.empty((M, inter), dtype=torch.bfloat16, device=DEV), bias=b)
+    finally:
+        ops.set_option("linear.wide_waves", 0)
+    want = ref.gate_up_swiglu(x.cpu(), w.cpu(), torch.empty((M, inter), dtype=torch.float64), bias=None if b is None else b.cpu())
+    close(tiled.float(), want, 2 * BF16_EPS, 1e-4, f"gate/up tile-major M{M} I{inter} K{K} waves {waves}")
+    same = (tiled == plain).float().mean().item()        # another number of waves may cut K into other slices
+    assert same == 1.0 if waves == 4 else same > 0.999, f"M{M} I{inter} K{K} waves {waves}: {1 - same:.2%} of the outputs differ from the row-major matrix's"
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("rows,width", [(1, 64), (13, 4099), (300, 4096)])
 def test_add_residual(ops, dtype, rows, width):
