@@ -16,7 +16,7 @@ int fllm_abi_version(void);
 void fllm_set_fast_kernels(int on);
 // Switches a kernel variant (for measurements and tests): "attention.tile32" 0/1; "linear.slices" n
 // (0: chosen by shape); "linear.dual_k" 0/1; "linear.x_direct" 0/1; "attention.fused_merge" 0/1;
-// "attention.prefill_parts" 0/1; "linear.slab" 0/1/2.  0 on success.
+// "attention.prefill_parts" 0/1; "linear.slab" 0/1/2; "linear.wide_waves" 0 (planned)/4/7/8.  0 on success.
 int fllm_set_option(const char *name, int value);
 
 // out[r, :] = scale * table[ids[r], :]            out: float32 [rows, width]
@@ -66,12 +66,13 @@ int fllm_norm_qkv_rope_store(const float *x, const float *norm_w, float eps, con
                              void *v_pages, int M, int heads, int kv_heads, int head_dim, int K, int page_size,
                              int store_kv, hipStream_t stream);
 
-// A norm prepared by the product before it, for steps of up to 16 rows.  fllm_linear_add_normed: out += x w^T
+// A norm prepared by the product before it, for steps of up to 64 rows.  fllm_linear_add_normed: out += x w^T
 // (float32 out [M, N], N a multiple of 16) and, for the RMSNorm that reads out next, next_x = out * next_w as
 // bfloat16 [M, N] and next_ssq [M, *tiles_out]: the sums of squares of out over the outputs of each tile (room for
 // M * N / 8 floats; *tiles_out, host memory, is set at the call).  The scaled forms are the norm forms above with
 // that pair in place of the float32 rows and the norm's weight.
-// w_tiles (may be null): the tile-major copy of w, see below.
+// w_tiles (may be null up to 16 rows): the tile-major copy of w, see below; the scaled forms of 17 to 64 rows need it, and K
+// in steps of 256.
 int fllm_linear_add_normed(const void *x, int ldx, const void *w, const float *bias, float *out, int M, int N, int K,
                            const float *next_w, void *next_x, float *next_ssq, int *tiles_out, const void *w_tiles,
                            hipStream_t stream);
@@ -81,23 +82,37 @@ int fllm_linear_add_normed(const void *x, int ldx, const void *w, const float *b
 // lane: from a row-major matrix that is 64 bytes of each of 16 rows a load, and the memory pipeline of a compute unit
 // looks up 64 cache lines for it; from the tile-major copy it is 1 KiB in a row, 8 lines, and the product of 8 or 16 rows
 // takes no longer than that of one (down projection of the 8B sizes: 29 -> 24 us at 8 rows).  The copy costs the
-// matrix's memory a second time, which a GPU with 288 GB affords; row-major stays for the products of 17 rows and more.
+// matrix's memory a second time, which a GPU with 288 GB affords; row-major stays for the GEMM library's products.
+// Steps of 17 to 64 rows read the copies too (four to eight row tiles a workgroup, the activations through LDS in chunks):
+// the feed-forward and q/k/v products with their fused prologues and epilogues then beat the library's products and
+// the separate norm, rotary and SwiGLU kernels.
 //   fllm_weight_tiles_supported  1 where the kernels take tiles: N >= 16, K a multiple of 1,024
 //   fllm_weight_tiles_elements   bfloat16 elements of the copy: N rounded up to 16, times K
 //   fllm_tile_weights            writes the copy: [tile of 16 rows][block of 128 columns][k-step of 32][lane][8]
-//   fllm_linear_add_tiled        out += x w^T (+ bias), float32 out, 1..16 rows; with w_tiles where it can
+//   fllm_linear_add_tiled        out += x w^T (+ bias), float32 out, 1..64 rows; with w_tiles where it can
+//   fllm_tile_weights_gate_up    the copy of [gate; up] ([2 inter][K]) for the SwiGLU epilogue of 17 to 64 rows: tile T holds
+//                                gate rows 8 T .. 8 T + 7 and then the same up rows; fllm_weight_tiles_elements_gate_up elements
+//   fllm_gate_up_swiglu_tiled    fllm_gate_up_swiglu for 17..64 rows with that copy (null: row-major)
 int fllm_weight_tiles_supported(int N, int K);
 size_t fllm_weight_tiles_elements(int N, int K);
 int fllm_tile_weights(const void *w, void *tiles, int N, int K, hipStream_t stream);
 int fllm_linear_add_tiled(const void *x, int ldx, const void *w, const void *w_tiles, const float *bias, float *out, int ldo,
                           int M, int N, int K, hipStream_t stream);
+size_t fllm_weight_tiles_elements_gate_up(int inter, int K);
+int fllm_tile_weights_gate_up(const void *w, void *tiles, int inter, int K, hipStream_t stream);
+int fllm_gate_up_swiglu_tiled(const void *x, int ldx, const void *w_gate_up, const void *w_tiles, const float *bias, void *out, int M,
+                              int inter, int K, hipStream_t stream);
 int fllm_scaled_gate_up_swiglu(const void *xn, const float *ssq, int ssq_count, float eps, const void *w_gate_up,
-                               const float *bias, void *out, int M, int inter, int K, hipStream_t stream);
+                               const float *bias, void *out, int M, int inter, int K, const void *w_tiles, hipStream_t stream);
 int fllm_scaled_qkv_rope_store(const void *xn, const float *ssq, int ssq_count, float eps, const void *w_qkv, const float *bias,
                                void *q_out, const int32_t *row_pos, const int32_t *row_seg, const int32_t *tables,
                                int table_stride, const float *cos_table, const float *sin_table, int rope_dims, void *k_pages,
                                void *v_pages, int M, int heads, int kv_heads, int head_dim, int K, int page_size, int store_kv,
-                               hipStream_t stream);
+                               const void *w_tiles, hipStream_t stream);
+
+// The pair that fllm_linear_add_normed leaves, from float32 rows that no such product wrote: xn = x * weight as bfloat16
+// [rows, width] and ssq [rows] (one part a row).
+int fllm_prepare_norm(const float *x, const float *weight, void *xn, float *ssq, int rows, int width, hipStream_t stream);
 
 // residual[r, :] += branch[r, :]   (residual float32 [rows, width], branch of type `dtype`)
 int fllm_add_residual(float *residual, const void *branch, int rows, int width, int dtype, hipStream_t stream);

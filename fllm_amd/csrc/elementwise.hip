@@ -79,6 +79,26 @@ rmsnorm_kernel(float *__restrict__ x, const B *__restrict__ branch, const int32_
     }
 }
 
+// What a product that adds into the residual stream leaves for the RMSNorm behind it (fllm_linear_add_normed), made
+// from rows that no such product wrote (the first layer's): xn = x * weight in bfloat16 and the row's sum of squares as
+// one part, added in the order of rmsnorm_kernel.
+__global__ void __launch_bounds__(kBlock)
+prepare_norm_kernel(const float *__restrict__ x, const float *__restrict__ weight, bf16_t *__restrict__ xn, float *__restrict__ ssq,
+                    int width) {
+    __shared__ float scratch[kWaves];
+    const int r = blockIdx.x;
+    const float *src = x + (size_t)r * width;
+    bf16_t *dst = xn + (size_t)r * width;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < width; c += kBlock) {
+        const float v = src[c];
+        ss += v * v;
+        dst[c] = (bf16_t)(v * weight[c]);
+    }
+    ss = block_sum<kWaves>(ss, scratch);
+    if (threadIdx.x == 0) ssq[r] = ss;
+}
+
 template <typename T>
 __global__ void __launch_bounds__(kBlock)
 swiglu_kernel(const T *__restrict__ gu, T *__restrict__ out, int inter) {
@@ -234,6 +254,14 @@ extern "C" int fllm_add_rmsnorm(float *x, const void *branch, int branch_dtype, 
         return dispatch_rmsnorm<float>(x, (const float *)branch, nullptr, weight, out, count, width, eps, out_dtype, stream);
     FLLM_REQUIRE(branch_dtype == FLLM_BF16, "add_rmsnorm: unknown dtype %d", branch_dtype);
     return dispatch_rmsnorm<bf16_t>(x, (const bf16_t *)branch, nullptr, weight, out, count, width, eps, out_dtype, stream);
+}
+
+extern "C" int fllm_prepare_norm(const float *x, const float *weight, void *xn, float *ssq, int rows, int width, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && width > 0 && x != nullptr && weight != nullptr && xn != nullptr && ssq != nullptr,
+                 "prepare_norm: bad operands rows=%d width=%d", rows, width);
+    if (rows == 0) return 0;
+    hipLaunchKernelGGL(prepare_norm_kernel, dim3(rows), dim3(kBlock), 0, stream, x, weight, (bf16_t *)xn, ssq, width);
+    return fllm_check_launch("prepare_norm");
 }
 
 extern "C" int fllm_swiglu(const void *gate_up, void *out, int rows, int inter, int dtype, hipStream_t stream) {

@@ -616,9 +616,12 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
 // the tile; the wave that counts the last slice adds the S partial sums in slice order and runs
 // the epilogue (as in the resident kernel).
 // WT: the weights come from their tile-major copy (fllm_tile_weights, fllm_tile_weights_gate_up), K a multiple of 256.
-template <int MT, int EPI, bool WT = false, int WAVES = 4>
+// PRO_SCALED: the rows are what the product before prepared for an RMSNorm (fllm_linear_add_normed); the row's scale,
+// from the parts of its sum of squares, multiplies the finished sums.
+template <int MT, int EPI, bool WT = false, int WAVES = 4, int PRO = PRO_BF16>
 __global__ void __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
 skinny_wide_kernel(SkinnyArgs a) {
+    static_assert(PRO == PRO_BF16 || PRO == PRO_SCALED, "rows arrive in bfloat16");
     constexpr int THREADS = WAVES * kWave;
     constexpr int KC = 256;                        // columns per chunk
     constexpr int KS = KC / 32;                    // MFMA k-steps per chunk
@@ -692,6 +695,39 @@ skinny_wide_kernel(SkinnyArgs a) {
     bf16x8_t wa[KS], wb[KS];
     issue_w(wa);
     issue_w(wb);
+    __shared__ float ssq_rows[PRO == PRO_SCALED ? ROWS : 1];
+    if (PRO == PRO_SCALED) {
+        // A row's sum of squares arrives in parts (up to a few hundred).  Four neighbouring threads share a row: each adds
+        // a quarter of the parts in index order, all its loads asked for together, and the quarters are added in order:
+        // the same sum for a row whatever the batch and the workgroup, and one trip to memory for all rows at once.
+        static_assert(THREADS >= 4 * ROWS, "four threads a row");
+        const int m = threadIdx.x >> 2, q = threadIdx.x & 3;
+        float t = 0.f;
+        if (threadIdx.x < 4 * ROWS) {      // whole waves: ROWS is a multiple of 16
+            const int per = (a.ssq_count + 3) / 4;
+            const int i0 = min(q * per, a.ssq_count), i1 = min(i0 + per, a.ssq_count);
+            if (m < M) {
+                const float *parts = a.ssq_in + (size_t)m * a.ssq_count;
+                if ((per & 3) == 0 && (a.ssq_count & 3) == 0 && ((uintptr_t)a.ssq_in & 15) == 0) {
+#pragma unroll 4
+                    for (int i = i0; i < i1; i += 4) {
+                        const f32x4_t v = *(const f32x4_t *)(parts + i);
+                        t += v[0];
+                        t += v[1];
+                        t += v[2];
+                        t += v[3];
+                    }
+                } else {
+                    for (int i = i0; i < i1; i++) t += parts[i];
+                }
+            }
+            const float t1 = __shfl_xor(t, 1, kWave);
+            const float pair = (q & 1) ? t1 + t : t + t1;          // quarter 2 k, then quarter 2 k + 1
+            const float other = __shfl_xor(pair, 2, kWave);
+            const float sum = (q & 2) ? other + pair : pair + other;
+            if (q == 0 && m < M) ssq_rows[m] = sum;
+        }
+    }
     if (total > 0) {
         load_x(0);
         store_x(0);
@@ -779,7 +815,8 @@ skinny_wide_kernel(SkinnyArgs a) {
                             }
                             if (!mine) continue;
                             EpilogueOperands eo;
-                            epilogue<PRO_BF16, EPI, RT>(a, t2, 0.f, m2, nb, n_out, eo);
+                            load_row_operands<EPI>(a, m2, eo);
+                            epilogue<PRO, EPI, RT>(a, t2, PRO == PRO_SCALED ? ssq_rows[m2] : 0.f, m2, nb, n_out, eo);
                         }
                     }
                 }
@@ -787,7 +824,8 @@ skinny_wide_kernel(SkinnyArgs a) {
             }
             if (finish && owner && m < M && nb < n_out) {
                 EpilogueOperands eo;
-                epilogue<PRO_BF16, EPI, RT>(a, s, 0.f, m, nb, n_out, eo);
+                load_row_operands<EPI>(a, m, eo);
+                epilogue<PRO, EPI, RT>(a, s, PRO == PRO_SCALED ? ssq_rows[m] : 0.f, m, nb, n_out, eo);
             }
         }
     };
@@ -1220,13 +1258,14 @@ int launch_resident(const SkinnyArgs &a, hipStream_t stream) {
     }
 }
 
-template <int MT, int EPI, bool WT, int WAVES>
+template <int MT, int EPI, bool WT, int WAVES, int PRO>
 int launch_wide_kernel(const SkinnyArgs &a, int grid, hipStream_t stream) {
-    hipLaunchKernelGGL((skinny_wide_kernel<MT, EPI, WT, WAVES>), dim3(grid), dim3(WAVES * kWave), 0, stream, a);
+    hipLaunchKernelGGL((skinny_wide_kernel<MT, EPI, WT, WAVES, PRO>), dim3(grid), dim3(WAVES * kWave), 0, stream, a);
     return fllm_check_launch("linear_wide");
 }
 
-template <int MT, int EPI>
+// 1: the shape is not served (the scaled prologue and the q/k/v epilogue only with the tile-major copy)
+template <int MT, int EPI, int PRO = PRO_BF16>
 int launch_wide(SkinnyArgs a, hipStream_t stream) {
     constexpr int NT = EPI == EPI_SWIGLU ? 8 : 16;
     constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
@@ -1247,10 +1286,22 @@ int launch_wide(SkinnyArgs a, hipStream_t stream) {
         a.counters = (int *)base;
         a.ws = (float *)((unsigned char *)base + kWorkspaceCounterBytes);
     }
-    if (!tiled) return launch_wide_kernel<MT, EPI, false, 4>(a, p.grid, stream);
-    if (p.waves == 7) return launch_wide_kernel<MT, EPI, true, 7>(a, p.grid, stream);
-    if (p.waves == 8) return launch_wide_kernel<MT, EPI, true, 8>(a, p.grid, stream);
-    return launch_wide_kernel<MT, EPI, true, 4>(a, p.grid, stream);
+    if (a.next_x != nullptr) {
+        a.next_nt = NT;
+        a.next_tiles = ntiles;
+        *a.next_tiles_out = ntiles;
+    }
+    constexpr bool kTiledOnly = PRO != PRO_BF16 || EPI == EPI_QKV;
+    constexpr bool kHasTiles = EPI == EPI_ADD || EPI == EPI_SWIGLU || EPI == EPI_QKV;     // the matrices that get copies
+    if constexpr (kHasTiles) {
+        if (tiled) {
+            if (p.waves == 7) return launch_wide_kernel<MT, EPI, true, 7, PRO>(a, p.grid, stream);
+            if (p.waves == 8) return launch_wide_kernel<MT, EPI, true, 8, PRO>(a, p.grid, stream);
+            return launch_wide_kernel<MT, EPI, true, 4, PRO>(a, p.grid, stream);
+        }
+    }
+    if constexpr (kTiledOnly) return 1;
+    else return launch_wide_kernel<MT, EPI, false, 4, PRO_BF16>(a, p.grid, stream);
 }
 
 using fllm_plan::SlabPlan;
@@ -1293,12 +1344,12 @@ int dispatch_slab(const SkinnyArgs &a, hipStream_t stream) {
     return launch_slab<PRO, EPI, 4>(a, stream);
 }
 
-template <int EPI>
+template <int EPI, int PRO = PRO_BF16>
 int dispatch_wide(const SkinnyArgs &a, hipStream_t stream) {
     const int mt = (a.M + 15) / 16;
-    if (mt == 2) return launch_wide<2, EPI>(a, stream);
-    if (mt == 3) return launch_wide<3, EPI>(a, stream);
-    return launch_wide<4, EPI>(a, stream);
+    if (mt == 2) return launch_wide<2, EPI, PRO>(a, stream);
+    if (mt == 3) return launch_wide<3, EPI, PRO>(a, stream);
+    return launch_wide<4, EPI, PRO>(a, stream);
 }
 
 template <int PRO, int EPI>
@@ -1549,8 +1600,8 @@ extern "C" int fllm_linear_add_tiled(const void *x, int ldx, const void *w, cons
 extern "C" int fllm_linear_add_normed(const void *x, int ldx, const void *w, const float *bias, float *out, int M, int N, int K,
                                       const float *next_w, void *next_x, float *next_ssq, int *tiles_out, const void *w_tiles,
                                       hipStream_t stream) {
-    FLLM_REQUIRE(M >= 1 && M <= 16 && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && N >= 16 && N % 16 == 0,
-                 "linear_add_normed: takes 1..16 rows, K and ldx in steps of 8 and N in steps of 16 (M=%d N=%d K=%d ldx=%d)", M, N, K, ldx);
+    FLLM_REQUIRE(M >= 1 && M <= 64 && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && N >= 16 && N % 16 == 0,
+                 "linear_add_normed: takes 1..64 rows, K and ldx in steps of 8 and N in steps of 16 (M=%d N=%d K=%d ldx=%d)", M, N, K, ldx);
     FLLM_REQUIRE(aligned16(x) && aligned16(w) && aligned16(out) && aligned16(next_w) && next_x != nullptr && next_ssq != nullptr &&
                      ((uintptr_t)next_x & 7) == 0 && tiles_out != nullptr && (w_tiles == nullptr || aligned16(w_tiles)),
                  "linear_add_normed: operands must be there and 16-byte aligned");
@@ -1569,17 +1620,23 @@ extern "C" int fllm_linear_add_normed(const void *x, int ldx, const void *w, con
     a.next_x = (bf16_t *)next_x;
     a.next_ssq = next_ssq;
     a.next_tiles_out = tiles_out;
-    const int rc = launch_resident<PRO_BF16, EPI_ADD>(a, stream);
+    const int rc = M <= 16 ? launch_resident<PRO_BF16, EPI_ADD>(a, stream) : dispatch_wide<EPI_ADD>(a, stream);
     FLLM_REQUIRE(rc != 1, "linear_add_normed: shape M=%d K=%d does not fit the staging area", M, K);
     return rc;
 }
 
 // The forms with a norm prologue, from what fllm_linear_add_normed left: xn [M, K] bfloat16, ssq [M, ssq_count].
+// From 17 rows on they need the weights' tile-major copy (`w_tiles`, of fllm_tile_weights_gate_up and fllm_tile_weights) and
+// K in steps of 256.
 extern "C" int fllm_scaled_gate_up_swiglu(const void *xn, const float *ssq, int ssq_count, float eps, const void *w_gate_up,
-                                          const float *bias, void *out, int M, int inter, int K, hipStream_t stream) {
-    FLLM_REQUIRE(M >= 1 && M <= 16 && K % 8 == 0 && K >= 8 && inter > 0 && ssq_count > 0 && eps > 0.f,
-                 "scaled_gate_up_swiglu: takes 1..16 rows and K a multiple of 8 (M=%d K=%d parts=%d)", M, K, ssq_count);
-    FLLM_REQUIRE(aligned16(xn) && aligned16(w_gate_up) && ssq != nullptr, "scaled_gate_up_swiglu: operands must be 16-byte aligned");
+                                          const float *bias, void *out, int M, int inter, int K, const void *w_tiles,
+                                          hipStream_t stream) {
+    FLLM_REQUIRE(M >= 1 && M <= 64 && K % 8 == 0 && K >= 8 && inter > 0 && ssq_count > 0 && eps > 0.f,
+                 "scaled_gate_up_swiglu: takes 1..64 rows and K a multiple of 8 (M=%d K=%d parts=%d)", M, K, ssq_count);
+    FLLM_REQUIRE(aligned16(xn) && aligned16(w_gate_up) && ssq != nullptr && (w_tiles == nullptr || aligned16(w_tiles)),
+                 "scaled_gate_up_swiglu: operands must be 16-byte aligned");
+    FLLM_REQUIRE(M <= 16 || (w_tiles != nullptr && K % 256 == 0),
+                 "scaled_gate_up_swiglu: from 17 rows on it takes the tile-major copy and K in steps of 256 (M=%d K=%d)", M, K);
     SkinnyArgs a = {};
     a.x = xn;
     a.ldx = K;
@@ -1593,6 +1650,10 @@ extern "C" int fllm_scaled_gate_up_swiglu(const void *xn, const float *ssq, int 
     a.M = M;
     a.N = 2 * inter;
     a.K = K;
+    if (M > 16) {
+        a.w_tiles = (const bf16_t *)w_tiles;
+        return dispatch_wide<EPI_SWIGLU, PRO_SCALED>(a, stream);
+    }
     const int rc = launch_resident<PRO_SCALED, EPI_SWIGLU>(a, stream);
     FLLM_REQUIRE(rc != 1, "scaled_gate_up_swiglu: shape M=%d K=%d does not fit the staging area", M, K);
     return rc;
@@ -1602,10 +1663,13 @@ extern "C" int fllm_scaled_qkv_rope_store(const void *xn, const float *ssq, int 
                                           const float *bias, void *q_out, const int32_t *row_pos, const int32_t *row_seg,
                                           const int32_t *tables, int table_stride, const float *cos_table, const float *sin_table,
                                           int rope_dims, void *k_pages, void *v_pages, int M, int heads, int kv_heads, int head_dim,
-                                          int K, int page_size, int store_kv, hipStream_t stream) {
-    FLLM_REQUIRE(M >= 1 && M <= 16 && K % 8 == 0 && K >= 8 && ssq_count > 0,
-                 "scaled_qkv_rope_store: takes 1..16 rows and K a multiple of 8 (M=%d K=%d parts=%d)", M, K, ssq_count);
-    FLLM_REQUIRE(aligned16(xn) && aligned16(w_qkv) && ssq != nullptr, "scaled_qkv_rope_store: operands must be 16-byte aligned");
+                                          int K, int page_size, int store_kv, const void *w_tiles, hipStream_t stream) {
+    FLLM_REQUIRE(M >= 1 && M <= 64 && K % 8 == 0 && K >= 8 && ssq_count > 0,
+                 "scaled_qkv_rope_store: takes 1..64 rows and K a multiple of 8 (M=%d K=%d parts=%d)", M, K, ssq_count);
+    FLLM_REQUIRE(aligned16(xn) && aligned16(w_qkv) && ssq != nullptr && (w_tiles == nullptr || aligned16(w_tiles)),
+                 "scaled_qkv_rope_store: operands must be 16-byte aligned");
+    FLLM_REQUIRE(M <= 16 || (w_tiles != nullptr && K % 256 == 0),
+                 "scaled_qkv_rope_store: from 17 rows on it takes the tile-major copy and K in steps of 256 (M=%d K=%d)", M, K);
     FLLM_REQUIRE(head_dim % 8 == 0 && rope_dims % 2 == 0 && rope_dims <= head_dim && rope_dims >= 0,
                  "scaled_qkv_rope_store: head_dim %d must be a multiple of 8 and rope_dims %d even and no larger", head_dim, rope_dims);
     FLLM_REQUIRE(heads > 0 && kv_heads > 0 && page_size > 0 && table_stride > 0 && eps > 0.f, "scaled_qkv_rope_store: bad sizes");
@@ -1614,6 +1678,10 @@ extern "C" int fllm_scaled_qkv_rope_store(const void *xn, const float *ssq, int 
                             k_pages, v_pages, M, heads, kv_heads, head_dim, K, page_size, store_kv);
     a.ssq_in = ssq;
     a.ssq_count = ssq_count;
+    if (M > 16) {
+        a.w_tiles = (const bf16_t *)w_tiles;
+        return dispatch_wide<EPI_QKV, PRO_SCALED>(a, stream);
+    }
     const int rc = launch_resident<PRO_SCALED, EPI_QKV>(a, stream);
     FLLM_REQUIRE(rc != 1, "scaled_qkv_rope_store: shape M=%d K=%d does not fit the staging area", M, K);
     return rc;

@@ -49,7 +49,7 @@ assert SAMPLE_ROW_BYTES == 32
 _lib = None
 
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 
 def load_library(build_if_missing: bool = True):
@@ -96,9 +96,10 @@ def load_library(build_if_missing: bool = True):
         "fllm_tile_weights_gate_up": [c_void, c_void, c_int, c_int, c_void],
         "fllm_gate_up_swiglu_tiled": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_linear_add_tiled": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_void],
-        "fllm_scaled_gate_up_swiglu": [c_void, c_void, c_int, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
+        "fllm_scaled_gate_up_swiglu": [c_void, c_void, c_int, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_void, c_void],
         "fllm_scaled_qkv_rope_store": [c_void, c_void, c_int, c_float, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void,
-                                       c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
+                                       c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void, c_void],
+        "fllm_prepare_norm": [c_void, c_void, c_void, c_void, c_int, c_int, c_void],
         "fllm_carry_ids": [c_void, c_void, c_void, c_int, c_int, c_void],
         "fllm_sample": [c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_adjust_logits": [c_void, c_int, c_int, c_void, c_void, c_void, c_void],
@@ -375,16 +376,47 @@ class Ops:
         return out
 
     PREPARED_NORM_ROWS = 16
+    CHUNK_KERNEL_ROWS = 64   # what those kernels take
+    CHUNK_ROWS = 48          # steps of 17 to this many rows take the fused forms of the kernels that pass the activations through
+                             # LDS in chunks (measured at the 8B sizes: 4 to 5 % of a step at 17 and 32 rows, 1 % at 48; from 49
+                             # rows on the library's q/k/v and output products beside the own feed-forward are 1 % faster)
 
-    def prepares_norm(self, rows: int, width: int) -> bool:
+    def fused_form(self, rows: int, width: int, w: torch.Tensor, gate_up: bool = False) -> Optional[str]:
+        """Which fused kernels serve a product of `rows` rows with the matrix `w` behind an RMSNorm of `width`:
+        "resident" (up to `fused_decode_rows` rows), "chunks" (17 to 64 rows: they need the norm prepared, by
+        `linear_add_prepare` or `prepare_norm`, and the tile-major copy of `w`) or None."""
+        if self.fused_decode_supported(rows, width):
+            return "resident"
+        if (self.fused_decode_rows < rows <= self.CHUNK_ROWS and (self.library_gemm_from is None or rows >= self.library_gemm_from)
+                and self.fused_decode_rows >= self.PREPARED_NORM_ROWS and width % 256 == 0 and Ops._tiles
+                and self._tiles_of(w, gate_up=gate_up) is not None):
+            return "chunks"
+        return None
+
+    def prepares_norm(self, rows: int, width: int, w: Optional[torch.Tensor] = None) -> bool:
         """Whether `linear_add_prepare` serves a sum into a residual stream of this size: the fused forms are in use,
-        up to 16 rows, widths in steps of 16."""
-        return rows <= self.PREPARED_NORM_ROWS and width % 16 == 0 and self.fused_decode_supported(rows, width)
+        up to 16 rows, or up to 64 with the tile-major copy of the matrix `w`; widths in steps of 16."""
+        if width % 16 != 0:
+            return False
+        if rows <= self.PREPARED_NORM_ROWS:
+            return self.fused_decode_supported(rows, width)
+        return w is not None and self.fused_form(rows, w.shape[1], w) == "chunks"      # the product's own width counts
+
+    def prepare_norm(self, x: torch.Tensor, norm_weight: torch.Tensor) -> PreparedNorm:
+        """What `linear_add_prepare` leaves for an RMSNorm, from float32 rows that no such product wrote (a model's first
+        layer): the rows times the norm's weight in bfloat16 and each row's sum of squares as one part."""
+        M, K = x.shape
+        _dense(x, "x", torch.float32)
+        _dense(norm_weight, "norm_weight", torch.float32, (K,))
+        xn = torch.empty((M, K), dtype=torch.bfloat16, device=x.device)
+        ssq = torch.empty((M,), dtype=torch.float32, device=x.device)
+        self._check(self.lib.fllm_prepare_norm(_ptr(x), _ptr(norm_weight), _ptr(xn), _ptr(ssq), M, K, self._stream()))
+        return PreparedNorm(xn, ssq, 1)
 
     def linear_add_prepare(self, x, w, residual, next_norm_weight, bias=None) -> PreparedNorm:
         """residual += x @ w.T (+ bias) as `linear(..., accumulate=True)` does, and in the same kernel what the RMSNorm
         with weight `next_norm_weight` that reads `residual` next would compute first (fllm_linear_add_normed): hand the
-        result to `norm_gate_up_swiglu` / `norm_qkv_rope_store` as `prepared`.  x bfloat16 [M <= 16, K], w bfloat16 [N, K],
+        result to `norm_gate_up_swiglu` / `norm_qkv_rope_store` as `prepared`.  x bfloat16 [M <= 64, K], w bfloat16 [N, K],
         residual float32 [M, N], N a multiple of 16."""
         M, K = x.shape
         N = w.shape[0]
@@ -394,8 +426,8 @@ class Ops:
         _dense(next_norm_weight, "next_norm_weight", torch.float32, (N,))
         if bias is not None:
             _dense(bias, "bias", torch.float32, (N,))
-        _need(1 <= M <= self.PREPARED_NORM_ROWS and N % 16 == 0 and K % 8 == 0,
-              f"linear_add_prepare takes 1..16 rows, N in steps of 16 and K in steps of 8, not {M} x {N} x {K}")
+        _need(1 <= M <= self.CHUNK_KERNEL_ROWS and N % 16 == 0 and K % 8 == 0,
+              f"linear_add_prepare takes 1..64 rows, N in steps of 16 and K in steps of 8, not {M} x {N} x {K}")
         xn = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
         ssq = torch.empty((M * (N // 8),), dtype=torch.float32, device=x.device)
         parts = ctypes.c_int(0)
@@ -412,8 +444,17 @@ class Ops:
         _dense(w, "w", torch.bfloat16, (n_rows_w, K))
         if bias is not None:
             _dense(bias, "bias", torch.float32, (n_rows_w,))
-        _need(1 <= M <= self.PREPARED_NORM_ROWS and K % 8 == 0, f"a prepared norm serves 1..16 rows and widths in steps of 8, not {M} x {K}")
+        _need(1 <= M <= self.CHUNK_KERNEL_ROWS and K % 8 == 0, f"a prepared norm serves 1..64 rows and widths in steps of 8, not {M} x {K}")
         return M, K
+
+    def _chunk_tiles(self, M: int, K: int, w: torch.Tensor, gate_up: bool = False) -> Optional[torch.Tensor]:
+        """The tile-major copy that a prepared norm of more than 16 rows needs (None up to 16 rows)."""
+        if M <= self.PREPARED_NORM_ROWS:
+            return None
+        tiles = self._tiles_of(w, gate_up=gate_up)
+        _need(tiles is not None and K % 256 == 0,
+              f"a prepared norm of {M} rows needs the tile-major copy of the matrix (tile_for_decode) and a width in steps of 256, not {K}")
+        return tiles
 
     def norm_gate_up_swiglu(self, x, norm_weight, eps, w_gate_up, out, bias=None, prepared: Optional[PreparedNorm] = None):
         """out = silu(rmsnorm(x) @ gate.T) * (rmsnorm(x) @ up.T); w_gate_up = [gate; up], out bfloat16 [M, I].
@@ -424,7 +465,8 @@ class Ops:
             M, K = self._prepared_operands(prepared, w_gate_up, bias, two_i)
             _dense(out, "out", torch.bfloat16, (M, two_i // 2))
             self._check(self.lib.fllm_scaled_gate_up_swiglu(_ptr(prepared.x), _ptr(prepared.ssq), prepared.parts, float(eps),
-                                                            _ptr(w_gate_up), _ptr(bias), _ptr(out), M, two_i // 2, K, self._stream()))
+                                                            _ptr(w_gate_up), _ptr(bias), _ptr(out), M, two_i // 2, K,
+                                                            _ptr(self._chunk_tiles(M, K, w_gate_up, gate_up=True)), self._stream()))
             return out
         M, K = self._fused_operands(x, norm_weight, w_gate_up, bias, two_i)
         _dense(out, "out", torch.bfloat16, (M, two_i // 2))
@@ -491,7 +533,7 @@ class Ops:
             self._check(self.lib.fllm_scaled_qkv_rope_store(
                 _ptr(prepared.x), _ptr(prepared.ssq), prepared.parts, float(eps), _ptr(w_qkv), _ptr(bias), _ptr(q_out), _ptr(row_pos),
                 _ptr(row_seg), _ptr(tables), tables.shape[1], _ptr(cos), _ptr(sin), rope_dims, _ptr(k_pages), _ptr(v_pages), M, heads,
-                kv_heads, head_dim, K, page_size, 1 if store else 0, self._stream()))
+                kv_heads, head_dim, K, page_size, 1 if store else 0, _ptr(self._chunk_tiles(M, K, w_qkv)), self._stream()))
             return q_out
         self._check(self.lib.fllm_norm_qkv_rope_store(
             _ptr(x), _ptr(norm_weight), float(eps), _ptr(w_qkv), _ptr(bias), _ptr(q_out), _ptr(row_pos), _ptr(row_seg),

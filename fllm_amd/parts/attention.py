@@ -13,7 +13,7 @@ import torch
 
 from ..config.spec import PartSpec
 from ..registry import part_class, register_part
-from .base import INIT_BIAS, INIT_MATRIX, KVNeed, Mixer, add_and_prepare, take_prepared
+from .base import INIT_BIAS, INIT_MATRIX, KVNeed, Mixer, add_and_prepare, fused_form, take_prepared
 
 
 class PagedAttention(Mixer):
@@ -71,6 +71,7 @@ class PagedAttention(Mixer):
                                 rt.matrix(weights["v"])], dim=0).contiguous()
         self.w_o = rt.matrix(weights["o"])
         rt.tile_for_decode(self.w_o)
+        rt.tile_for_decode(self.w_qkv)       # for steps of 17 to 64 rows
         biases = [reorder(None if weights.get("q_bias") is None else rt.vector(weights["q_bias"]), order_q),
                   reorder(None if weights.get("k_bias") is None else rt.vector(weights["k_bias"]), order_k),
                   None if weights.get("v_bias") is None else rt.vector(weights["v_bias"])]
@@ -117,9 +118,8 @@ class PagedAttention(Mixer):
         rt, ops = self.rt, self.rt.ops
         rows = residual.shape[0]
         prologue = getattr(norm, "fused_prologue", lambda: None)()
-        if (rt.dtype != torch.bfloat16 or self.pairing != 1 or prologue is None
-                or not hasattr(ops, "norm_qkv_rope_store") or not ops.fused_decode_supported(rows, self.hidden)
-                or self.head_dim % 4 != 0):
+        form = fused_form(ops, rows, self.hidden, self.w_qkv) if hasattr(ops, "norm_qkv_rope_store") else None
+        if rt.dtype != torch.bfloat16 or self.pairing != 1 or prologue is None or form is None or self.head_dim % 4 != 0:
             return False
         norm_scale, norm_eps = prologue
         nh, nkv, d = self.heads, self.kv_heads, self.head_dim
@@ -129,6 +129,8 @@ class PagedAttention(Mixer):
             cos, sin, dims, _ = ctx.no_rotation(rt)
         q = rt.empty((rows, nh * d))
         prepared = take_prepared(ctx, norm, residual)      # the sum before this norm may have computed its first steps
+        if prepared is None and form == "chunks":
+            prepared = ops.prepare_norm(residual, norm_scale)
         ops.norm_qkv_rope_store(residual, norm_scale, norm_eps, self.w_qkv, q, ctx.row_pos, ctx.row_seg,
                                 ctx.tables[binding.group], cos, sin, binding.k_pages if binding.writes else None,
                                 binding.v_pages if binding.writes else None, nh, nkv, d, dims, binding.page_size,

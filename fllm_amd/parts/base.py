@@ -172,6 +172,16 @@ def leave_prepared(ctx, norm, residual, payload) -> None:
     ctx.prepared = (norm, residual, payload)
 
 
+def fused_form(ops, rows: int, width: int, w, gate_up: bool = False):
+    """Which of the kernel library's fused kernels serve a product of `rows` rows with the matrix `w` behind a norm of
+    `width`: "resident" (the norm is folded in or prepared), "chunks" (more rows: the norm must be prepared,
+    `ops.prepare_norm` does it where the product before has not) or None."""
+    ask = getattr(ops, "fused_form", None)
+    if ask is not None:
+        return ask(rows, width, w, gate_up=gate_up)
+    return "resident" if ops.fused_decode_supported(rows, width) else None
+
+
 def add_and_prepare(ctx, ops, x, w, residual, bias) -> bool:
     """residual += x @ w.T (+ bias) in the kernel that also prepares `ctx.then_norm`, where the kernel library has one
     for this size and that norm says what it multiplies by (`fused_prologue`); the result is left for the norm's
@@ -179,7 +189,10 @@ def add_and_prepare(ctx, ops, x, w, residual, bias) -> bool:
     norm = getattr(ctx, "then_norm", None)
     prepare = getattr(ops, "linear_add_prepare", None)
     prologue = getattr(norm, "fused_prologue", lambda: None)() if norm is not None else None
-    if prepare is None or prologue is None or residual is None or not ops.prepares_norm(residual.shape[0], residual.shape[1]):
+    if prepare is None or prologue is None or residual is None:
+        return False
+    rows, width = residual.shape
+    if not (ops.prepares_norm(rows, width, w) if rows > 16 else ops.prepares_norm(rows, width)):
         return False
     if x.dtype != torch.bfloat16 or x.stride(0) % 8 != 0 or x.shape[1] % 8 != 0:
         return False

@@ -6,7 +6,7 @@ from __future__ import annotations
 import torch
 
 from ..registry import register_part
-from .base import INIT_BIAS, INIT_MATRIX, FeedForward, add_and_prepare, take_prepared
+from .base import INIT_BIAS, INIT_MATRIX, FeedForward, add_and_prepare, fused_form, take_prepared
 
 
 class GatedMLP(FeedForward):
@@ -42,12 +42,14 @@ class GatedMLP(FeedForward):
         rt, ops = self.rt, self.rt.ops
         rows = residual.shape[0]
         prologue = getattr(norm, "fused_prologue", lambda: None)()
-        if (rt.dtype != torch.bfloat16 or prologue is None
-                or not hasattr(ops, "norm_gate_up_swiglu") or not ops.fused_decode_supported(rows, self.hidden)):
+        form = fused_form(ops, rows, self.hidden, self.w_gate_up, gate_up=True) if hasattr(ops, "norm_gate_up_swiglu") else None
+        if rt.dtype != torch.bfloat16 or prologue is None or form is None:
             return False
         norm_scale, norm_eps = prologue
         act = rt.empty((rows, self.inter))
         prepared = take_prepared(ctx, norm, residual)      # the sum before this norm may have computed its first steps
+        if prepared is None and form == "chunks":
+            prepared = ops.prepare_norm(residual, norm_scale)
         ops.norm_gate_up_swiglu(residual, norm_scale, norm_eps, self.w_gate_up, act, bias=self.b_gate_up,
                                 **({"prepared": prepared} if prepared is not None else {}))
         if not add_and_prepare(ctx, ops, act, self.w_down, residual, self.b_down):

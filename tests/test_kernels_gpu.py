@@ -567,12 +567,78 @@ def test_a_product_prepares_the_norm_that_reads_its_sums(ops, ref, M, N, K):
             results.append((q, kp, vp))
         for got, base in zip(results[1], results[0]):
             assert float((got.float() - base.float()).abs().max()) <= 2 * BF16_EPS * float(base.float().abs().max())
-    with pytest.raises(Exception, match="1..16 rows"):
-        ops.linear_add_prepare(torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV),
-                               torch.zeros(17, 32, device=DEV), torch.ones(32, device=DEV))
+    with pytest.raises(Exception, match="1..64 rows"):
+        ops.linear_add_prepare(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV),
+                               torch.zeros(65, 32, device=DEV), torch.ones(32, device=DEV))
     with pytest.raises(Exception, match="steps of 16"):
         ops.linear_add_prepare(torch.zeros(2, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(24, 64, dtype=torch.bfloat16, device=DEV),
                                torch.zeros(2, 24, device=DEV), torch.ones(24, device=DEV))
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 4096, 4096), (64, 4096, 14336), (33, 1024, 2048), (48, 2048, 1024), (64, 2048, 8192)])
+def test_prepared_norms_of_17_to_64_rows(ops, ref, M, N, K):
+    """Steps of 17 to 64 rows run the same five kernels a layer as smaller ones, on the kernels that pass the
+    activations through LDS in chunks and read the tile-major copies: the sum into the residual stream prepares the
+    next norm, the gate/up and q/k/v products take the prepared rows and scale their sums by the row's norm.  Against
+    the float64 results, against the same forms fed with the float32 rows (another kernel), and with the preparation
+    made by `prepare_norm` (a model's first layer)."""
+    g = gen(170 + M)
+    x = (torch.randn(M, K, generator=g) * 0.5).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).to(DEV)
+    resid = (torch.randn(M, N, generator=g) * torch.rand(M, 1, generator=g) * 6).to(DEV)
+    nw = (1 + 0.1 * torch.randn(N, generator=g)).to(DEV)
+    few = min(M, ops.CHUNK_ROWS)                             # the kernels take up to 64 rows, steps use them up to CHUNK_ROWS
+    assert ops.tile_for_decode(w) and ops.fused_form(few, K, w) == "chunks" and ops.prepares_norm(few, N, w)
+    assert ops.fused_form(few, K, w.clone()) is None         # no copy: the library's products and the separate kernels serve
+    assert ops.fused_form(ops.CHUNK_ROWS + 1, K, w) is None
+    summed = resid.clone()
+    prepared = ops.linear_add_prepare(x, w, summed, nw)
+    want = ref.linear(x.cpu(), w.cpu(), resid.double().cpu(), accumulate=True)
+    mag = (x.double().abs() @ w.double().abs().T).max().item()
+    close(summed, want, 1e-6, 4e-7 * mag + 1e-6, f"sum M{M} N{N} K{K}")
+    assert torch.equal(summed, ops.linear(x, w, resid.clone(), accumulate=True))
+    assert torch.equal(prepared.x, (summed * nw).to(torch.bfloat16)) and prepared.parts == N // 16
+    squares = prepared.ssq[:M * prepared.parts].view(M, prepared.parts).double().sum(1)
+    assert float(((squares - summed.double().pow(2).sum(1)).abs() / summed.double().pow(2).sum(1)).max()) < 1e-6
+    first = ops.prepare_norm(summed, nw)
+    assert torch.equal(first.x, prepared.x) and first.parts == 1
+    assert float(((first.ssq.double() - squares).abs() / squares).max()) < 1e-6
+    # the products behind that norm
+    inter = 3 * N // 2 + 8
+    wgu = (torch.randn(2 * inter, N, generator=g) / math.sqrt(N)).to(torch.bfloat16).to(DEV)
+    bgu = (torch.randn(2 * inter, generator=g) * 0.1).to(DEV)
+    assert ops.tile_for_decode(wgu, gate_up=True) and ops.fused_form(few, N, wgu, gate_up=True) == "chunks"
+    want = ref.norm_gate_up_swiglu(summed.cpu(), nw.cpu(), 1e-5, wgu.cpu(), torch.empty(M, inter, dtype=torch.float64), bias=bgu.cpu())
+    own = ops.norm_gate_up_swiglu(summed, nw, 1e-5, wgu, torch.empty(M, inter, dtype=torch.bfloat16, device=DEV), bias=bgu)
+    for pair in (prepared, first):
+        fed = ops.norm_gate_up_swiglu(None, None, 1e-5, wgu, torch.empty(M, inter, dtype=torch.bfloat16, device=DEV), bias=bgu, prepared=pair)
+        close(fed, want, 2 * BF16_EPS, 4e-2, f"gate/up behind a prepared norm M{M} N{N}")
+        assert float((fed.float() - own.float()).abs().max()) <= 2 * BF16_EPS * float(own.float().abs().max())
+    heads, kv_heads, head_dim, page_size = N // 64, 2, 16, 16
+    qkv_rows = (heads + 2 * kv_heads) * head_dim
+    wq = (torch.randn(qkv_rows, N, generator=g) / math.sqrt(N)).to(torch.bfloat16).to(DEV)
+    assert ops.tile_for_decode(wq)
+    tables = scattered_tables(g, M, 8, M * 8 + 2).to(DEV)
+    row_pos = torch.tensor([(7 * r + 3) % 128 for r in range(M)], dtype=torch.int32, device=DEV)
+    row_seg = torch.arange(M, dtype=torch.int32, device=DEV)
+    row_seg[M // 2] = -1                                   # a padding row stores nothing
+    angle = torch.rand(128, head_dim // 2, generator=g, dtype=torch.float64) * 6.28
+    cos, sin = torch.cos(angle).float().to(DEV), torch.sin(angle).float().to(DEV)
+    k0, v0 = make_pages(g, M * 8 + 2, kv_heads, page_size, head_dim, torch.bfloat16)
+    results = []
+    for kwargs in ({}, {"prepared": prepared}, {"prepared": first}):
+        kp, vp = k0.to(DEV), v0.to(DEV)
+        q = ops.norm_qkv_rope_store(summed, nw, 1e-5, wq, torch.zeros(M, heads * head_dim, dtype=torch.bfloat16, device=DEV),
+                                    row_pos, row_seg, tables, cos, sin, kp, vp, heads, kv_heads, head_dim, head_dim, page_size, **kwargs)
+        results.append((q, kp, vp))
+    live = row_seg >= 0
+    for other in results[1:]:
+        for got, base in zip(other, results[0]):
+            got, base = (got[live], base[live]) if got.shape[0] == M else (got, base)
+            assert float((got.float() - base.float()).abs().max()) <= 2 * BF16_EPS * float(base.float().abs().max())
+    assert torch.equal(results[1][0][~live], torch.zeros_like(results[1][0][~live]))
+    with pytest.raises(Exception, match="tile-major copy"):
+        ops.norm_gate_up_swiglu(None, None, 1e-5, wgu.clone(), torch.empty(M, inter, dtype=torch.bfloat16, device=DEV), prepared=prepared)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
