@@ -255,7 +255,7 @@ def main():
     further = not (args.no_points or args.no_further or args.prefill_only) and args.shape == "8b"
     long_contexts = (8192, 32768) if further else ()
     long_steps = 32
-    batches = [args.batch] if args.no_points or args.prefill_only else sorted({1, args.batch, 64})
+    batches = [args.batch] if args.no_points or args.prefill_only else sorted({1, args.batch, 32, 64})
     prompt_tokens = args.prompt_tokens if args.prefill_only else PREFILL_TOKENS
     runs = [(b, args.prompt_len, steps) for b in batches] + [(args.batch, c, long_steps) for c in long_contexts]
     held = [prompt + warmup + count + decode_slack(b, prompt) for b, prompt, count in runs]      # tokens a request comes to hold
@@ -319,7 +319,7 @@ def main():
     step_bytes = decode_step_bytes(cfg, args.layers, contexts)
     achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
     line = {
-        "metric": f"decode tok/s at batch {args.batch} ({SHAPE_NAMES[args.shape]}, {args.prompt_len:,}-token prompts); points: batch 1/64; prefill: 2,048 tokens",
+        "metric": f"decode tok/s at batch {args.batch} ({SHAPE_NAMES[args.shape]}, {args.prompt_len:,}-token prompts); points: batch 1/32/64; prefill: 2,048 tokens",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic token ids, random-init weights N(0, 0.02)",
@@ -334,8 +334,9 @@ def main():
         "runs_ms_per_step": {f"decode_b{b}": v for b, v in all_runs.items()},
     }
     if not args.no_points:
-        line["points"] = {"decode_b1": round(results[1][0], 2), "decode_b64": round(results[64][0], 2)}
-        for b in (1, 64):
+        line["points"] = {"decode_b1": round(results[1][0], 2), "decode_b64": round(results[64][0], 2),
+                          "decode_b32": round(results[32][0], 2)}
+        for b in (1, 32, 64):
             line["points"][f"decode_b{b}_hbm_frac"] = round(share(results[b]), 4)
         prefills = sorted(prefill_run() for _ in range(repeats))
         best = prefills[len(prefills) // 2]

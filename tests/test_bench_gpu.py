@@ -45,7 +45,7 @@ def test_the_line_of_a_short_run():
     assert line["points"]["decode_b1"] > 0 and line["points"]["decode_b64"] > line["points"]["decode_b1"]
     # every headline figure is the median of three timed runs, all of them listed
     runs = line["runs_ms_per_step"]
-    assert line["timed_runs"] == 3 and set(runs) == {"decode_b1", "decode_b8", "decode_b64", "prefill"}
+    assert line["timed_runs"] == 3 and set(runs) == {"decode_b1", "decode_b8", "decode_b32", "decode_b64", "prefill"}
     assert all(len(v) == 3 for v in runs.values())
     assert sorted(runs["decode_b8"])[1] == line["ms_per_step"] and sorted(runs["prefill"])[1] == line["prefill"]["ms"]
     flops = line["prefill"]["achieved_tflops"] * 1e12
