@@ -91,8 +91,8 @@ class Engine:
         this one, and `step()` returns the events of the step before.  A request that stops at a
         token (end of sequence, stop id) has one more row in flight by then; that row is dropped.
 
-        `decode_weight_tiles` (True, False, "auto": while memory is plentiful): a second copy of the output and down
-        projection matrices in the order decode steps read them (`Runtime.tile_for_decode`).
+        `decode_weight_tiles` (True, False, "auto": within half of the memory that is free once the weights are placed):
+        second copies of the layers' matrices in the order decode steps read them (`Runtime.tile_for_decode`).
 
         `check_layers`: the first so many steps run every layer also with the plain kernels and print, layer by
         layer, how far the two are apart, the largest value, a checksum and NaN/Inf counts (`runner.check_layers`)."""
@@ -109,7 +109,7 @@ class Engine:
         self.runner = ModelRunner(spec, tensors, dtype=dtype, device=device, page_size=block_size, num_pages=num_blocks,
                                   max_requests=max_seqs, max_context=ctx, memory_utilization=gpu_memory_utilization,
                                   ops=ops, typed_config=typed, max_step_tokens=max_batched_tokens,
-                                  decode_weight_tiles=decode_weight_tiles)
+                                  decode_weight_tiles=decode_weight_tiles, consume_tensors=True)
         del tensors
         self.config = typed
         self.max_model_len = self.runner.max_context

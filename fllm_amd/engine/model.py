@@ -25,7 +25,7 @@ class GroupKey(NamedTuple):
 
 
 class Model:
-    def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], rt: Runtime):
+    def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], rt: Runtime, consume_tensors: bool = False):
         spec.validate()
         self.spec = spec
         self.rt = rt
@@ -33,6 +33,7 @@ class Model:
         def make(role, part, **extra):
             return part_class(role, part.kind)(part, part_weights(part, tensors), rt, **extra)
 
+        rt.collect_tile_requests()       # copies of matrices for decode steps are made when all weights are placed
         self.embedding = make("embedding", spec.embedding)
         self.blocks = []
         for layer in spec.layers:
@@ -45,6 +46,9 @@ class Model:
             self.blocks.append(make("block", layer.block, **placed))
         self.final_norm = make("norm", spec.final_norm)
         self.head = make("head", spec.head)
+        if consume_tensors:
+            tensors.clear()              # the parts hold what they use; what they joined into one matrix is given back
+        self.decode_tile_bytes = rt.tiles_for_model()
         self.bindings: List[CacheBinding] = []
         self.layer_check = None          # a diagnostics.LayerCheck while layers are being checked
         self._plan_caches()

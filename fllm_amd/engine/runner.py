@@ -65,13 +65,15 @@ class ModelRunner:
                  num_pages: Union[int, Sequence[int], None] = None,
                  max_requests: int = 16, max_context: Optional[int] = None, memory_utilization: float = 0.90,
                  ops=None, typed_config=None, use_graphs: bool = True, max_step_tokens: Optional[int] = None,
-                 decode_weight_tiles="auto"):
+                 decode_weight_tiles="auto", consume_tensors: bool = False):
         """`num_pages`: pages of every cache group (one number) or of each group (a list); by default what
         `max_tokens` tokens need, else what fits on the card.  `max_step_tokens`: the most tokens of one request
         that a step may bring (more are refused); with it, groups that keep a window of keys are made no larger than
         `max_requests` requests can fill.  `decode_weight_tiles`: True, False or "auto" (while memory is plentiful): the
         matrices whose products add into the residual stream keep a second, tile-major copy for decode steps
-        (`Runtime.tile_for_decode`)."""
+        (`Runtime.tile_for_decode`).  `consume_tensors`: the caller has no further use for `tensors`; the dictionary is
+        emptied once the parts hold what they need, so that pieces the parts have joined into one matrix (q, k and v;
+        gate and up) do not stay on the device beside it while the copies and the cache are sized."""
         self.spec = spec
         self.config = typed_config
         self.device = torch.device(device)
@@ -85,7 +87,7 @@ class ModelRunner:
         self.max_context = int(min(max_context or spec.max_position, spec.max_position))
         self.rt = Runtime(self.device, self.dtype, ops, self.max_context, decode_weight_tiles)
         check_tensors(spec, {n: tuple(t.shape) for n, t in tensors.items()})
-        self.model = Model(spec, tensors, self.rt)
+        self.model = Model(spec, tensors, self.rt, consume_tensors=consume_tensors)
         self.vocab_size = spec.vocab_size
         num_groups = len(self.model.group_keys)
         self.max_requests = max_requests

@@ -27,7 +27,7 @@ class GatedMLP(FeedForward):
         self.w_gate_up = torch.cat([rt.matrix(weights["gate"]), rt.matrix(weights["up"])], dim=0).contiguous()
         self.w_down = rt.matrix(weights["down"])
         rt.tile_for_decode(self.w_down)
-        rt.tile_for_decode(self.w_gate_up, gate_up=True)     # for steps of 17 to 64 rows
+        rt.tile_for_decode(self.w_gate_up, gate_up=True, priority=1)     # for steps of 17 to 64 rows
         gb, ub = weights.get("gate_bias"), weights.get("up_bias")
         self.b_gate_up = None
         if gb is not None or ub is not None:
