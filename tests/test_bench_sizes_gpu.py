@@ -1,8 +1,10 @@
 """Whole steps of the engine at the layer sizes that the benchmark times (Llama-3.1-8B, Llama-3.2-1B and
 Llama-3.1-70B widths, with few layers and a small vocabulary), against the plain implementation: requests whole, in
-portions, with the last tokens one by one, mixed with four live requests, and decoded in batches of 64, 24, 8 and 1
+portions, with the last tokens one by one, mixed with four live requests, and decoded in batches of 64, 40, 24, 8 and 1
 rows through the captured graphs, in float32 and in bfloat16.  The kernel variants that only these sizes select (K
-slices of the decode products, their 8-row tiles, eight query heads a key/value head) run here inside a model.
+slices of the decode products, their 8-row tiles, eight query heads a key/value head, the tile-major copies of the
+matrices and the fused forms of 17 to 48 rows that read them) run here inside a model; `options` is a model of such
+widths with what the others lack: biases on every product, a sliding window on one layer, a partial rotary width.
 The reference compares whole-model logits the same way (rust/engine/src/tiny_models.rs:946-1005,
 scripts/verify_architectures.py:1-70)."""
 import numpy as np
@@ -29,13 +31,15 @@ SIZES = {
     "8b": config(2, 4096, 32, 8, 128, 14336, 8.0, False),
     "1b": config(2, 2048, 32, 8, 64, 8192, 32.0, True),
     "70b": config(1, 8192, 64, 8, 128, 28672, 8.0, False),
+    "options": dict(config(2, 1024, 8, 2, 128, 3072, 8.0, True), partial_rotary_factor=0.5, sliding_window=40,
+                    layer_types=["sliding_attention", "full_attention"]),
 }
 # |engine - plain| <= tol * max|plain logit|, and the engine's largest logit of every row is the plain implementation's
 # or within twice that of it.  Largest errors seen on the MI355X: float32 9.1e-6; bfloat16 1.5e-2 (8b),
 # 1.2e-2 (1b), 1.4e-2 (70b).  The plain kernels (one float32 chain per element, bfloat16 only where tensors are stored)
 # are as far from the plain implementation at these widths (1.3e-2 at the 8b sizes): the distance is the storage type's.
 TOL = {"float32": 2e-5, "bfloat16": 2e-2}
-LADDER = [10] * 40 + [14] * 16 + [18] * 7 + [22]          # 64 requests; 64, 24, 8 and 1 of them are left as they end
+LADDER = [10] * 24 + [12] * 16 + [14] * 16 + [18] * 7 + [22]          # 64 requests; 64, 40, 24, 8 and 1 of them are left as they end
 
 
 @pytest.fixture(scope="module")
@@ -49,7 +53,7 @@ def cases():
             from fllm_amd.weights import random_tensors
             cfg = SIZES[name]
             _, spec = model_spec_from_config(cfg)
-            tensors = {k: v.to(torch.float32) for k, v in random_tensors(spec, 77, torch.bfloat16).items()}
+            tensors = {k: v.to(torch.float32) for k, v in random_tensors(spec, 77, torch.bfloat16, with_optional=(name == "options")).items()}
             lengths = {"w": 300, "m0": 90, "m1": 150, "m2": 60, "m3": 200}
             requests = {rid: tc.random_ids(n, cfg["vocab_size"], 7 + i) for i, (rid, n) in enumerate(lengths.items())}
             ladder = {f"d{i}": tc.random_ids(n, cfg["vocab_size"], 500 + i) for i, n in enumerate(LADDER)}
@@ -75,7 +79,7 @@ def ladder_steps(ladder, head=6):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["8b", "1b", "70b"])
+@pytest.mark.parametrize("name", ["8b", "1b", "70b", "options"])
 def test_steps_at_benchmark_sizes(cases, tmp_path, name, dtype):
     from fllm_amd.engine import ModelRunner
     cfg, spec, tensors, requests, ladder, plain = cases(name)
@@ -111,4 +115,9 @@ def test_steps_at_benchmark_sizes(cases, tmp_path, name, dtype):
     print(f"observed errors {name} {dtype}: " + ", ".join(f"{k} {v:.2e}" for k, v in worst.items()))
     if dtype == "bfloat16":
         rows_seen = {key[0] for key in runner._graphs}
-        assert {1, 8, 24, 64} <= rows_seen, f"decode graphs of {sorted(rows_seen)} rows ran"
+        assert {1, 8, 24, 40, 64} <= rows_seen, f"decode graphs of {sorted(rows_seen)} rows ran"
+        ops = runner.rt.ops                      # the steps of 24 and 40 rows ran the fused forms that read the copies
+        for block in runner.model.blocks:
+            assert ops.fused_form(24, cfg["hidden_size"], block.mixer.w_qkv) == "chunks"
+            assert ops.fused_form(40, cfg["hidden_size"], block.feed_forward.w_gate_up, gate_up=True) == "chunks"
+            assert ops.own_feed_forward(64, block.feed_forward.w_gate_up, block.feed_forward.w_down)
