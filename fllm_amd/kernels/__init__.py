@@ -219,12 +219,15 @@ class Ops:
 
     # 17 to 64 rows beside the GEMM library: with the tile-major copies the own products of the feed-forward (gate/up
     # with its SwiGLU epilogue, down with the residual sum) are faster than the library's products and the SwiGLU kernel
-    # (measured at the 8B sizes, 64 / 32 rows: gate/up 48 / 44 us against 55 / 53, down 34 / 28 against 40 / 31)
+    # (measured at the 8B sizes, 64 / 32 rows: gate/up 48 / 44 us against 55 / 53, down 34 / 28 against 40 / 31; at the 1B
+    # sizes, 67 MB of gate and up weights, the library is 3 % of a 64-row step ahead, hence the same floor on the bytes
+    # as for `prefers_own_gate_up`)
     def own_feed_forward(self, rows: int, w_gate_up: torch.Tensor, w_down: torch.Tensor) -> bool:
         """Whether a bfloat16 step of 17 to 64 rows whose products would go to the GEMM library should take
         `gate_up_swiglu` and `linear(..., accumulate=True)` for its feed-forward instead: when both matrices have their
         tile-major copies."""
         return (self.library_gemm_from is not None and self.library_gemm_from <= rows <= self.GATE_UP_SWIGLU_ROWS and bool(Ops._tiles)
+                and w_gate_up.numel() * w_gate_up.element_size() >= self.OWN_GATE_UP_BYTES
                 and self._tiles_of(w_gate_up, gate_up=True) is not None and self._tiles_of(w_down) is not None)
 
     def set_fast_kernels(self, on: bool) -> None:

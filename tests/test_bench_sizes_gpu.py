@@ -120,4 +120,5 @@ def test_steps_at_benchmark_sizes(cases, tmp_path, name, dtype):
         for block in runner.model.blocks:
             assert ops.fused_form(24, cfg["hidden_size"], block.mixer.w_qkv) == "chunks"
             assert ops.fused_form(40, cfg["hidden_size"], block.feed_forward.w_gate_up, gate_up=True) == "chunks"
-            assert ops.own_feed_forward(64, block.feed_forward.w_gate_up, block.feed_forward.w_down)
+            large = block.feed_forward.w_gate_up.numel() * 2 >= ops.OWN_GATE_UP_BYTES       # small matrices: the library's products
+            assert ops.own_feed_forward(64, block.feed_forward.w_gate_up, block.feed_forward.w_down) == large
