@@ -69,9 +69,8 @@ __device__ __forceinline__ bf16x8_t zero8() {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // floats that one part of a shared row tile leaves for the merge (tile32 kernel): head_dim / 2 outputs, a maximum
-// and a sum for each of its 256 lanes
-__host__ __device__ constexpr size_t kPartFloats(int head_dim) { return fllm_plan::part_floats(head_dim); }
-static_assert(kThreads == 256, "part_floats counts 256 threads");
+// and a sum for each of its lanes
+__host__ __device__ constexpr size_t kPartFloats(int head_dim, int threads) { return fllm_plan::part_floats(head_dim, threads); }
 
 // Online-softmax update of one query row held across the four lane groups of a wave.
 // s: NS score tiles (already scaled and masked with -inf); returns the P^T operands.
@@ -259,7 +258,7 @@ attn_tile_kernel(AttnArgs p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// tile kernel on 32x32x16 products: 128 (token, head-of-group) rows per workgroup
+// tile kernel on 32x32x16 products: 128 or 256 (token, head-of-group) rows per workgroup
 // ---------------------------------------------------------------------------------------------
 // v_mfma_f32_32x32x16_bf16: A lane l holds A[m = l%32][k = 8*(l/32) .. +7], B lane l holds
 // B[k = 8*(l/32) .. +7][n = l%32], D lane l holds D[m = 8*(i/4) + 4*(l/32) + i%4][n = l%32], i = 0..15.
@@ -271,21 +270,25 @@ attn_tile_kernel(AttnArgs p) {
 // from global memory into registers while the current one is multiplied, the scale is folded into
 // the exponent (one fused multiply-add per score), tiles wholly below the diagonal skip the mask,
 // and the outputs are rescaled only when a row's maximum moved.
-template <int D>
-__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// WAVES: 4 (128 rows a workgroup, two workgroups a compute unit) or 8 (256 rows, one workgroup a compute unit: a key or
+// value fetched from L2 serves twice the rows; 128 rows over 16,384 keys ask L2 for 6.9 TB/s, which is about what it
+// hands to the compute units).
+template <int D, int WAVES>
+__global__ void __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
 attn_tile32_kernel(AttnArgs p) {
+    constexpr int THREADS = WAVES * kWave;
     constexpr int KT = 64;          // keys per tile
     constexpr int KP = D + 8;       // pitch of a key row in LDS
     constexpr int VP = KT + 8;      // pitch of a value row (one head_dim lane, KT keys) in LDS
     constexpr int DS = D / 16, DB = D / 32;
-    constexpr int CH = KT * D / 8 / kThreads;   // 16-byte chunks per thread and tile (K and V each)
+    constexpr int CH = KT * D / 8 / THREADS;   // 16-byte chunks per thread and tile (K and V each)
     constexpr int LD = D == 64 ? 6 : 7;         // log2(D)
     static_assert(CH >= 1 && (D == 64 || D == 128), "this tiling takes head_dim 64 or 128");
     __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KP];
     __shared__ __attribute__((aligned(16))) bf16_t Vs[D * VP];
     __shared__ int s_tile[2];
     const int G = p.heads / p.kv_heads;
-    const int TQ = 128 / G;         // tokens per tile
+    const int TQ = WAVES * 32 / G;  // tokens per tile
     // blockIdx.x = (row tile, key/value head), the head fastest: workgroups start in the order of their row tiles,
     // longest contexts first, whatever their head, and with 8 heads each of the 8 dies sees the keys of one head only
     const int group = blockIdx.x;
@@ -352,7 +355,7 @@ attn_tile32_kernel(AttnArgs p) {
     int k_key[CH], v_koff[CH], k_in_page[CH], v_in_page[CH], k_lds[CH], v_lds[CH];
 #pragma unroll
     for (int c = 0; c < CH; c++) {
-        const int ch = threadIdx.x + c * kThreads;
+        const int ch = threadIdx.x + c * THREADS;
         // the chunks in the order in which they lie in a page (token fastest, then the key's chunks, then the tile's pages):
         // a load instruction of a wave reads 1 KiB in a row where a page holds 16 tokens or more
         const int wsh = psh < 6 ? psh : 6;               // log2 of the tokens of a page that lie in this tile (KT is 64)
@@ -524,15 +527,15 @@ attn_tile32_kernel(AttnArgs p) {
         // its own values (the parts share the assignment of rows to lanes); the part that arrives last adds them up
         // in the order of the parts, so the result does not depend on which one that is.
         __shared__ int s_seen;
-        float *slot = p.parts_ws + (size_t)group * gridDim.y * kPartFloats(D);
-        float *mine = slot + (size_t)blockIdx.y * kPartFloats(D);
+        float *slot = p.parts_ws + (size_t)group * gridDim.y * kPartFloats(D, THREADS);
+        float *mine = slot + (size_t)blockIdx.y * kPartFloats(D, THREADS);
 #pragma unroll
         for (int db = 0; db < DB; db++)
 #pragma unroll
             for (int i = 0; i < 16; i++)
-                __hip_atomic_store(mine + (db * 16 + i) * kThreads + threadIdx.x, o[db][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(mine + DB * 16 * kThreads + threadIdx.x, m_run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(mine + (DB * 16 + 1) * kThreads + threadIdx.x, l_run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(mine + (db * 16 + i) * THREADS + threadIdx.x, o[db][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(mine + DB * 16 * THREADS + threadIdx.x, m_run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(mine + (DB * 16 + 1) * THREADS + threadIdx.x, l_run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         parts_published();      // the part has arrived before it is counted
         __syncthreads();
         int *counter = p.counters + group;
@@ -546,7 +549,7 @@ attn_tile32_kernel(AttnArgs p) {
             float mp[8];
 #pragma unroll
             for (int i = 0; i < 8; i++)
-                mp[i] = i0 + i < parts ? __hip_atomic_load(slot + (size_t)(i0 + i) * kPartFloats(D) + DB * 16 * kThreads + threadIdx.x,
+                mp[i] = i0 + i < parts ? __hip_atomic_load(slot + (size_t)(i0 + i) * kPartFloats(D, THREADS) + DB * 16 * THREADS + threadIdx.x,
                                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
                                        : -INFINITY;
 #pragma unroll
@@ -558,16 +561,16 @@ attn_tile32_kernel(AttnArgs p) {
             for (int i = 0; i < 16; i++) o[db][i] = 0.f;
         l_run = 0.f;
         for (int i = 0; i < parts; i++) {
-            const float *from = slot + (size_t)i * kPartFloats(D);
-            const float mi = __hip_atomic_load(from + DB * 16 * kThreads + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float *from = slot + (size_t)i * kPartFloats(D, THREADS);
+            const float mi = __hip_atomic_load(from + DB * 16 * THREADS + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             const float f = mi == -INFINITY ? 0.f : fast_exp2((mi - m_all) * sc);
-            l_run = fmaf(__hip_atomic_load(from + (DB * 16 + 1) * kThreads + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT),
+            l_run = fmaf(__hip_atomic_load(from + (DB * 16 + 1) * THREADS + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT),
                          f, l_run);
 #pragma unroll
             for (int db = 0; db < DB; db++)
 #pragma unroll
                 for (int j = 0; j < 16; j++)
-                    o[db][j] = fmaf(__hip_atomic_load(from + (db * 16 + j) * kThreads + threadIdx.x, __ATOMIC_RELAXED,
+                    o[db][j] = fmaf(__hip_atomic_load(from + (db * 16 + j) * THREADS + threadIdx.x, __ATOMIC_RELAXED,
                                                       __HIP_MEMORY_SCOPE_AGENT), f, o[db][j]);
         }
     }
@@ -851,9 +854,31 @@ int device_slots() {   // workgroups of the tile32 kernel that the device holds 
 
 // How the tile32 kernel shares the key tiles of a row tile among workgroups (plans.h), with the device's slots and
 // the option that is set by hand.
-int prefill_part_plan(int tiles, int kv_heads, int rows, int max_context, int window, size_t room, int *max_parts) {
-    return fllm_plan::prefill_part_plan(tiles, kv_heads, rows, max_context, window, room, device_slots(), fllm_option_prefill_parts(),
+int prefill_part_plan(int tiles, int kv_heads, int rows, int max_context, int window, size_t room, int slots, int *max_parts) {
+    return fllm_plan::prefill_part_plan(tiles, kv_heads, rows, max_context, window, room, slots, fllm_option_prefill_parts(),
                                         max_parts);
+}
+
+// Prompt portions on the 32x32x16 products: WAVES * 32 rows a workgroup.
+template <int D, int WAVES>
+int launch_tile32(const AttnArgs &a, int max_context, hipStream_t stream) {
+    const int G = a.heads / a.kv_heads;
+    const int TQ = WAVES * 32 / G;
+    const int tiles = (a.rows + TQ - 1) / TQ + a.num_segs;   // upper bound; surplus workgroups leave at once
+    AttnArgs p = a;
+    int max_parts = 1;
+    void *dev_ws = nullptr;
+    size_t dev_ws_bytes = 0;
+    if (fllm_option_prefill_parts() && fllm_device_workspace(&dev_ws, &dev_ws_bytes) && dev_ws_bytes > kWorkspaceCounterBytes) {
+        p.part_tiles = prefill_part_plan(tiles, a.kv_heads, a.rows, max_context, a.window,
+                                         (dev_ws_bytes - kWorkspaceCounterBytes) / (kPartFloats(D, WAVES * kWave) * sizeof(float)),
+                                         device_slots() * 4 / WAVES, &max_parts);
+        p.counters = (int *)dev_ws;
+        p.parts_ws = (float *)((unsigned char *)dev_ws + kWorkspaceCounterBytes);
+    }
+    FLLM_REQUIRE(tiles >= 1 && (long)tiles * a.kv_heads <= 0x7fffffffL && max_parts <= 65535, "attention: grid too large");
+    hipLaunchKernelGGL((attn_tile32_kernel<(D >= 64 ? D : 64), WAVES>), dim3(tiles * a.kv_heads, max_parts), dim3(WAVES * kWave), 0, stream, p);
+    return fllm_check_launch("attention_tile32");
 }
 
 template <int D>
@@ -895,22 +920,11 @@ int launch(const AttnArgs &a, int uniform_rows, int max_context, void *workspace
                                a.heads, p.splits);
         return fllm_check_launch("attention_decode");
     }
-    if (D >= 64 && G <= 64 && fllm_option_tile32()) {   // 128 rows per workgroup on 32x32x16 products
-        const int TQ = 128 / G;
-        const int tiles = (a.rows + TQ - 1) / TQ + a.num_segs;   // upper bound; surplus workgroups leave at once
-        AttnArgs p = a;
-        int max_parts = 1;
-        void *dev_ws = nullptr;
-        size_t dev_ws_bytes = 0;
-        if (fllm_option_prefill_parts() && fllm_device_workspace(&dev_ws, &dev_ws_bytes) && dev_ws_bytes > kWorkspaceCounterBytes) {
-            p.part_tiles = prefill_part_plan(tiles, a.kv_heads, a.rows, max_context, a.window,
-                                             (dev_ws_bytes - kWorkspaceCounterBytes) / (kPartFloats(D) * sizeof(float)), &max_parts);
-            p.counters = (int *)dev_ws;
-            p.parts_ws = (float *)((unsigned char *)dev_ws + kWorkspaceCounterBytes);
-        }
-        FLLM_REQUIRE(tiles >= 1 && (long)tiles * a.kv_heads <= 0x7fffffffL && max_parts <= 65535, "attention: grid too large");
-        hipLaunchKernelGGL(attn_tile32_kernel<(D >= 64 ? D : 64)>, dim3(tiles * a.kv_heads, max_parts), dim3(kThreads), 0, stream, p);
-        return fllm_check_launch("attention_tile32");
+    if (D >= 64 && G <= 64 && fllm_option_tile32()) {   // 128 or 256 rows per workgroup on 32x32x16 products
+        // 256 rows where they leave no compute unit without a workgroup: twice the rows for every key fetched from L2
+        const int wide = fllm_option_tile32_rows();
+        const bool rows256 = wide == 256 || (wide == 0 && (long)((a.rows + 256 / G - 1) / (256 / G)) * a.kv_heads >= device_slots() / 2);
+        return rows256 ? launch_tile32<D, 8>(a, max_context, stream) : launch_tile32<D, 4>(a, max_context, stream);
     }
     const int TQ = 64 / G;
     const int tiles = (a.rows + TQ - 1) / TQ + a.num_segs;   // upper bound; surplus workgroups leave at once

@@ -220,8 +220,8 @@ inline size_t decode_lds_bytes(int head_dim, int group) {
 inline bool decode_counters_fit(int rows, int kv_heads, int qtiles) { return (size_t)rows * kv_heads * qtiles * sizeof(int) <= kCounterBytes; }
 
 // ---- prompt attention: the key tiles of a row tile shared among workgroups ----
-// what a part of a row tile leaves behind, in floats: every thread of the 256 its outputs (head_dim / 2), a maximum and a sum
-constexpr size_t part_floats(int head_dim) { return (size_t)256 * (head_dim / 2 + 2); }
+// what a part of a row tile leaves behind, in floats: every thread of the workgroup its outputs (head_dim / 2), a maximum and a sum
+constexpr size_t part_floats(int head_dim, int threads = 256) { return (size_t)threads * (head_dim / 2 + 2); }
 // The most key tiles one workgroup takes (0: row tiles are not shared) and the most parts a row tile can have.  Row
 // tiles are shared when, one workgroup each, they would leave workgroup slots of the device empty: a part then has
 // about the key tiles that a slot sees in all when every slot is taken, and at least 8, since every part pays for

@@ -33,6 +33,8 @@ static int g_linear_slices = 0;
 static int g_dual_k = 1;
 static int g_x_direct = 1;
 int fllm_option_x_direct(void) { return g_x_direct; }
+static int g_tile32_rows = 0;     // 0: chosen by the launch; 128 or 256
+int fllm_option_tile32_rows(void) { return g_tile32_rows; }
 static int g_wide_waves = 0;      // 0: planned
 int fllm_option_wide_waves(void) { return g_wide_waves; }
 static int g_slab = 1;
@@ -55,6 +57,10 @@ extern "C" int fllm_set_option(const char *name, int value) {
     }
     if (strcmp(name, "linear.slab") == 0) {
         g_slab = value < 0 ? 0 : (value > 2 ? 2 : value);
+        return 0;
+    }
+    if (strcmp(name, "attention.tile32_rows") == 0) {
+        g_tile32_rows = (value == 128 || value == 256) ? value : 0;
         return 0;
     }
     if (strcmp(name, "linear.wide_waves") == 0) {

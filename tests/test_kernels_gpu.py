@@ -840,6 +840,28 @@ def test_attention_bf16_tile_kernel_of_64_rows(ops, ref, heads, kv_heads, head_d
         ops.set_option("attention.tile32", 1)
 
 
+@pytest.mark.parametrize("rows", [128, 256])
+@pytest.mark.parametrize("prefill_parts", [1, 0])
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(8, 2, 64, 16), (32, 8, 128, 16), (8, 8, 64, 32), (16, 1, 128, 16), (6, 3, 64, 8)])
+@pytest.mark.parametrize("segs,window", [(CHUNK_SEGS[3], None), (CHUNK_SEGS[4], None), (CHUNK_SEGS[5], None), (CHUNK_SEGS[7], 100),
+                                          ([(640, 64)], 300), ([(0, 700), (1500, 40), (3, 300)], None), ([(0, 1100)], None)])
+def test_attention_bf16_row_tiles_of_128_and_256(ops, ref, rows, prefill_parts, heads, kv_heads, head_dim, page_size, segs, window):
+    """The prompt kernel takes 128 rows a workgroup or 256 (one workgroup a compute unit: a key fetched from L2 serves
+    twice the rows); a launch picks by how many row tiles it has, `attention.tile32_rows` by hand.  Both against the plain
+    reference, with and without row tiles shared between workgroups, with a far key that stands out."""
+    ops.set_option("attention.tile32_rows", rows)
+    ops.set_option("attention.prefill_parts", prefill_parts)
+    try:
+        attention_case(ops, ref, torch.bfloat16, heads, kv_heads, head_dim, page_size, segs, window, 23, spike=True, calls=2)
+    finally:
+        ops.set_option("attention.tile32_rows", 0)
+        ops.set_option("attention.prefill_parts", 1)
+    torch.cuda.synchronize()
+    from fllm_amd.kernels import Ops
+    counters = Ops._workspaces[torch.cuda.current_device()][: 64 * 1024]
+    assert int(counters.to(torch.int64).sum()) == 0
+
+
 @pytest.mark.parametrize("fused_merge", [1, 0])
 @pytest.mark.parametrize("heads,kv_heads,head_dim,page_size", [(8, 2, 64, 16), (32, 8, 128, 16), (5, 1, 32, 8)])
 @pytest.mark.parametrize("segs,bound,window", [([(999, 1), (5, 1), (640, 1)], 2048, None), ([(1100, 1)], 4096, None),
