@@ -921,9 +921,11 @@ int launch(const AttnArgs &a, int uniform_rows, int max_context, void *workspace
         return fllm_check_launch("attention_decode");
     }
     if (D >= 64 && G <= 64 && fllm_option_tile32()) {   // 128 or 256 rows per workgroup on 32x32x16 products
-        // 256 rows where they leave no compute unit without a workgroup: twice the rows for every key fetched from L2
+        // 256 rows where they leave no compute unit without a workgroup and the contexts are long: twice the rows for
+        // every key fetched from L2 (inside a model: 3 % at contexts of 2,048 to 16,384 keys, nothing or a loss below)
         const int wide = fllm_option_tile32_rows();
-        const bool rows256 = wide == 256 || (wide == 0 && (long)((a.rows + 256 / G - 1) / (256 / G)) * a.kv_heads >= device_slots() / 2);
+        const bool rows256 = wide == 256 || (wide == 0 && max_context > 4096 &&
+                                             (long)((a.rows + 256 / G - 1) / (256 / G)) * a.kv_heads >= device_slots() / 2);
         return rows256 ? launch_tile32<D, 8>(a, max_context, stream) : launch_tile32<D, 4>(a, max_context, stream);
     }
     const int TQ = 64 / G;
