@@ -89,6 +89,9 @@ def cmd_run(argv: List[str]) -> int:
     ap.add_argument("--logit-bias", default="", help="comma-separated id:value pairs added to the logits")
     ap.add_argument("--logprobs", type=int, default=None, metavar="N",
                     help="with every token its log-probability in the model's distribution and the N likeliest tokens (at most 20)")
+    ap.add_argument("--logprobs-mode", choices=["raw_logprobs", "processed_logprobs"], default="raw_logprobs",
+                    help="processed_logprobs: the log-probabilities are those of the distribution a token was drawn from "
+                         "(after penalties, temperature and filters) instead of the model's own")
     ap.add_argument("--allowed-token-ids", default="", help="comma-separated: only these tokens can be chosen")
     ap.add_argument("--bad-words-ids", action="append", default=[], metavar="IDS",
                     help="comma-separated token ids of a sequence that must not be generated (repeatable)")
@@ -125,6 +128,7 @@ def cmd_run(argv: List[str]) -> int:
                             **chosen, presence_penalty=args.presence_penalty,
                             frequency_penalty=args.frequency_penalty, repeat_last_n=args.repeat_last_n,
                             min_tokens=args.min_tokens, logit_bias=bias, logprobs=args.logprobs,
+                            logprobs_processed=args.logprobs_mode == "processed_logprobs",
                             allowed_token_ids=tuple(int(t) for t in args.allowed_token_ids.split(",") if t.strip()),
                             bad_word_ids=tuple(tuple(int(t) for t in w.split(",") if t.strip()) for w in args.bad_words_ids),
                             timeout_secs=args.timeout, n=args.n)

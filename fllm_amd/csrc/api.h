@@ -232,6 +232,13 @@ int fllm_adjust_logits(float *logits, int rows, int vocab, const struct FllmAdju
 int fllm_logprobs(const float *logits, int rows, int vocab, const int32_t *wanted_rows, int wanted, const int32_t *tokens,
                   int top, float *values, int32_t *ids, hipStream_t stream);
 
+// The same for the distribution a token was drawn from: logits as the sampler saw them (penalties and biases applied),
+// divided by the temperature, over the tokens that top-k, min-p and top-p leave (params: the records fllm_sample got,
+// one a row); a greedy row is a point mass.  A chosen token that the filters leave out has -inf; where fewer than `top`
+// tokens are left the rest of ids is -1.
+int fllm_logprobs_processed(const float *logits, int rows, int vocab, const int32_t *wanted_rows, int wanted, const int32_t *tokens,
+                            const struct FllmSampleRow *params, int top, float *values, int32_t *ids, hipStream_t stream);
+
 // work: float32 [rows, vocab] scratch.  kinds: what the caller knows of the rows, a sum of 1 (some have a temperature
 // and no filter: their draw looks at every token, and several workgroups share such a row), 2 (some are of another
 // kind) and 4 (some of those have a top-k of at most 64: several workgroups share such a row as well).

@@ -462,6 +462,32 @@ __device__ uint32_t thresholds_of_short_list(KeyAt key_at, WeightAt weight_at, i
     return t;
 }
 
+// The threshold of a list too long for LDS, by the whole workgroup: top-k over `key_at` (key 0: not a candidate), then
+// top-p over `heavy_key_at`, which is key_at with 0 for a candidate that min-p drops.  `all_units`: with top-p alone, the
+// mass of every finite logit in units of 2^-40, listed or not.  `bins`: kBins cells of LDS.
+template <typename KeyAt, typename WeightAt, typename HeavyKeyAt>
+__device__ uint32_t threshold_of_long_list(KeyAt key_at, WeightAt weight_at, HeavyKeyAt heavy_key_at, int count, int top_k, bool use_k,
+                                           bool use_p, bool use_m, float top_p, unsigned long long all_units, unsigned long long *bins,
+                                           Cells &cells) {
+    uint32_t t = 0;
+    unsigned long long whole = all_units;
+    if (use_k) t = key_by_histograms<false>(key_at, weight_at, count, 0u, (unsigned long long)min(top_k, count), bins, cells);
+    if (use_p) {
+        if (use_k || use_m) {
+            unsigned long long mine = 0;
+            for (int i = threadIdx.x; i < count; i += kBlock) {
+                const uint32_t key = heavy_key_at(i);
+                if (key != 0 && key >= t) mine += units_of(weight_at(i));
+            }
+            whole = block_units(mine, cells);
+        }
+        unsigned long long target = (unsigned long long)((double)top_p * (double)whole);
+        if (target == 0) target = 1;
+        t = key_by_histograms<true>(heavy_key_at, weight_at, count, t, target, bins, cells);
+    }
+    return t;
+}
+
 // Calls f(token, logit) for every token of a row, each thread of the workgroup with a share of its own: four
 // consecutive tokens a load where the row's alignment allows (four such loads in flight), single tokens at both ends.
 // A thread meets its tokens in the same order in every pass.
@@ -847,22 +873,8 @@ sample_kernel(const float *__restrict__ logits, float *__restrict__ work, const 
                 const float v = usable(src[list[i]]);
                 return expf((v - m) * inv_t) >= min_p ? ordered_key(v) : 0u;
             };
-            uint32_t t = 0;
-            unsigned long long whole = all_units;        // top-p alone: the mass of every finite logit, listed or not
-            if (use_k) t = key_by_histograms<false>(key_at, weight_at, count, 0u, (unsigned long long)min(p.top_k, count), bins, cells);
-            if (use_p) {
-                if (use_k || use_m) {
-                    unsigned long long mine = 0;
-                    for (int i = threadIdx.x; i < count; i += kBlock) {
-                        const uint32_t key = heavy_key_at(i);
-                        if (key != 0 && key >= t) mine += units_of(weight_at(i));
-                    }
-                    whole = block_units(mine, cells);
-                }
-                unsigned long long target = (unsigned long long)((double)p.top_p * (double)whole);
-                if (target == 0) target = 1;
-                t = key_by_histograms<true>(heavy_key_at, weight_at, count, t, target, bins, cells);
-            }
+            const uint32_t t = threshold_of_long_list(key_at, weight_at, heavy_key_at, count, p.top_k, use_k, use_p, use_m, p.top_p,
+                                                      all_units, bins, cells);
             threshold = t;
         }
     }
@@ -1118,7 +1130,109 @@ logprobs_kernel(const float *__restrict__ logits, int vocab, const int32_t *__re
         if (last.index == kNone) last.value = -INFINITY;      // nothing is left: the rest stays empty
     }
 }
+// Log-probabilities in the distribution a token was drawn from (rust/engine/src/sampling.rs, `logprobs_processed` and
+// `processed_distribution`; its test :1542-1556): the softmax of logits / T over the tokens that top-k, min-p and top-p
+// leave, in that order and with the ties kept as the sampler keeps them; a greedy row is a point mass on the first
+// largest logit.  `logits` are the ones the sampler saw (penalties and biases applied).  values[0] belongs to the chosen
+// token (-inf if the filters leave it out), values[1..] and ids[1..] to the likeliest of the tokens that are left, fewer
+// than `top` if fewer are left (then ids -1, values NaN).  One workgroup a wanted row; the thresholds are found as
+// `sample_kernel` finds them for a list that does not fit into LDS (histograms over the keys' bits), over the whole row.
+__global__ void __launch_bounds__(kBlock)
+processed_logprobs_kernel(const float *__restrict__ logits, int vocab, const int32_t *__restrict__ rows, const int32_t *__restrict__ tokens,
+                          const FllmSampleRow *__restrict__ params, int top, float *__restrict__ values, int32_t *__restrict__ ids) {
+    __shared__ Cells cells;
+    __shared__ unsigned long long bins[kBins];
+    const int row = rows[blockIdx.x];
+    const FllmSampleRow p = params[row];
+    const float *src = logits + (size_t)row * vocab;
+    float *out_v = values + (size_t)blockIdx.x * (1 + top);
+    int32_t *out_i = ids + (size_t)blockIdx.x * (1 + top);
+    const int token = tokens[row];
+    float m = -INFINITY;
+    for_each_token(src, vocab, [&](int, float v) { m = fmaxf(m, usable(v)); });
+    m = block_largest(m, cells);
+    if (!(m > -INFINITY)) {      // no finite logit: no distribution
+        for (int k = threadIdx.x; k <= top; k += kBlock) out_i[k] = k == 0 ? token : -1, out_v[k] = NAN;
+        return;
+    }
+    const bool greedy = !(p.temperature > 1e-5f);
+    const float inv_t = greedy ? 1.0f : (float)(1.0 / (double)p.temperature);
+    const bool use_k = !greedy && p.top_k > 0 && p.top_k < vocab;
+    const bool use_p = !greedy && p.top_p > 0.f && p.top_p < 1.f;
+    const bool use_m = !greedy && p.min_p > 0.f;
+    const float min_p = use_m ? p.min_p : 0.f;
+    auto key_at = [&](int i) {
+        const float v = usable(src[i]);
+        return v > -INFINITY ? ordered_key(v) : 0u;      // key 0: not a candidate
+    };
+    auto weight_at = [&](int i) { return expf((usable(src[i]) - m) * inv_t); };
+    auto heavy_key_at = [&](int i) {
+        const float v = usable(src[i]);
+        return (v > -INFINITY && expf((v - m) * inv_t) >= min_p) ? ordered_key(v) : 0u;
+    };
+    uint32_t threshold = 0;
+    if (greedy) {
+        threshold = ordered_key(m);                      // the largest logit alone; among equals the first (below)
+    } else if (use_k || use_p) {
+        unsigned long long mine = 0;
+        if (use_p && !use_k && !use_m)
+            for (int i = threadIdx.x; i < vocab; i += kBlock)
+                if (key_at(i) != 0) mine += units_of(weight_at(i));
+        const unsigned long long all_units = block_units(mine, cells);
+        threshold = threshold_of_long_list(key_at, weight_at, heavy_key_at, vocab, p.top_k, use_k, use_p, use_m, p.top_p, all_units,
+                                           bins, cells);
+    }
+    // what is left, and its mass
+    auto left = [&](int i, float v) { return v > -INFINITY && ordered_key(v) >= threshold && (!use_m || expf((v - m) * inv_t) >= min_p); };
+    double mass = 0.0;
+    Pick first = {-INFINITY, kNone};
+    for (int i = threadIdx.x; i < vocab; i += kBlock) {
+        const float v = usable(src[i]);
+        if (!left(i, v)) continue;
+        mass += (double)expf((v - m) * inv_t);
+        first = better_of(first, Pick{v, i});
+    }
+    first = block_best(first, cells);
+    const float log_mass = greedy ? 0.f : (float)log(WholeBlock::sum(mass, cells));
+    auto value_of = [&](int i, float v) { return greedy ? 0.f : (v - m) * inv_t - log_mass; };
+    if (threadIdx.x == 0) {
+        const float v = token >= 0 && token < vocab ? usable(src[token]) : -INFINITY;
+        const bool in = token >= 0 && token < vocab && left(token, v) && (!greedy || token == first.index);
+        out_i[0] = token;
+        out_v[0] = in ? value_of(token, v) : -INFINITY;
+    }
+    Pick last = {INFINITY, -1};                   // everything comes after this
+    for (int k = 1; k <= top; k++) {
+        Pick mine = {-INFINITY, kNone};
+        if (!(greedy && k > 1))
+            for (int i = threadIdx.x; i < vocab; i += kBlock) {
+                const float v = usable(src[i]);
+                if (!left(i, v)) continue;
+                const bool after_last = v < last.value || (v == last.value && i > last.index);
+                if (after_last && (v > mine.value || (v == mine.value && i < mine.index) || mine.index == kNone)) mine = Pick{v, i};
+            }
+        last = block_best(mine, cells);
+        if (threadIdx.x == 0) {
+            out_i[k] = last.index == kNone ? -1 : last.index;
+            out_v[k] = last.index == kNone ? NAN : value_of(last.index, last.value);
+        }
+        if (last.index == kNone) last.value = -INFINITY;      // nothing is left: the rest stays empty
+    }
+}
 }  // namespace
+
+extern "C" int fllm_logprobs_processed(const float *logits, int rows, int vocab, const int32_t *wanted_rows, int wanted,
+                                       const int32_t *tokens, const FllmSampleRow *params, int top, float *values, int32_t *ids,
+                                       hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && vocab > 0 && wanted >= 0, "logprobs_processed: bad sizes rows=%d vocab=%d wanted=%d", rows, vocab, wanted);
+    FLLM_REQUIRE(top >= 0 && top <= 20 && top <= vocab, "logprobs_processed: %d alternatives asked for, at most min(20, vocabulary) are given", top);
+    if (wanted == 0) return 0;
+    FLLM_REQUIRE(logits != nullptr && wanted_rows != nullptr && tokens != nullptr && params != nullptr && values != nullptr && ids != nullptr,
+                 "logprobs_processed: logits, rows, tokens, sampling records and both outputs are required");
+    hipLaunchKernelGGL(processed_logprobs_kernel, dim3(wanted), dim3(kBlock), 0, stream, logits, vocab, wanted_rows, tokens, params, top,
+                       values, ids);
+    return fllm_check_launch("logprobs_processed");
+}
 
 extern "C" int fllm_logprobs(const float *logits, int rows, int vocab, const int32_t *wanted_rows, int wanted,
                              const int32_t *tokens, int top, float *values, int32_t *ids, hipStream_t stream) {

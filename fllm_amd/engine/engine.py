@@ -30,6 +30,7 @@ class TokenEvent:
     finish_reason: Optional[str] = None     # "stop" | "length" | "timeout" (then no token comes with it: token_id -1)
     choice: int = 0                         # with `SamplingParams.n` > 1: which of the answers the token belongs to
     logprob: Optional[float] = None         # with `SamplingParams.logprobs`: of this token in the model's distribution
+                                            # (with `logprobs_processed`: in the one it was drawn from)
     top_logprobs: Optional[List[Tuple[int, float]]] = None     # and the likeliest tokens, (id, log-probability)
 
 
@@ -249,8 +250,10 @@ class Engine:
         self.stats.max_rows = max(self.stats.max_rows, rows)
         requests = [SampleRequest(seqs[sid].sampling, seqs[sid].sampling.seed_for(sid), seqs[sid].draws) for sid in sampled]
         wants_logprobs = [r for r, sid in enumerate(sampled) if seqs[sid].sampling.logprobs is not None]
+        wants_processed = [r for r in wants_logprobs if seqs[sampled[r]].sampling.logprobs_processed]
+        wants_raw = [r for r in wants_logprobs if r not in wants_processed]
         adjusting = any(seqs[sid].sampling.adjusts_logits(seqs[sid].output_len) for sid in sampled)
-        as_given = logits.clone() if wants_logprobs and adjusting else logits
+        as_given = logits.clone() if wants_raw and adjusting else logits
         if adjusting:
             self._adjust(logits, sampled, row_of, earlier)
         launched = _InFlight(sampled, [], self.sampler.launch(logits, requests))
@@ -258,7 +261,8 @@ class Engine:
         launched.on_host = self.sampler.start_read(launched.tokens)
         if wants_logprobs:
             top = max(seqs[sampled[r]].sampling.logprobs for r in wants_logprobs)
-            launched.logprobs = self.sampler.start_logprobs(as_given, launched.tokens, wants_logprobs, top)
+            launched.logprobs = self.sampler.start_logprobs(as_given, launched.tokens, wants_raw, top, processed=wants_processed,
+                                                            seen=logits, requests=requests)
         # What does not depend on the tokens' values: the sequences grow by one (a placeholder until the
         # token is read), the prompt portions count as computed.
         for sid, _, count in plan.prefill:

@@ -49,7 +49,7 @@ assert SAMPLE_ROW_BYTES == 32
 _lib = None
 
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 
 def load_library(build_if_missing: bool = True):
@@ -104,6 +104,7 @@ def load_library(build_if_missing: bool = True):
         "fllm_sample": [c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_adjust_logits": [c_void, c_int, c_int, c_void, c_void, c_void, c_void],
         "fllm_logprobs": [c_void, c_int, c_int, c_void, c_int, c_void, c_int, c_void, c_void, c_void],
+        "fllm_logprobs_processed": [c_void, c_int, c_int, c_void, c_int, c_void, c_void, c_int, c_void, c_void, c_void],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -725,6 +726,23 @@ class Ops:
         _dense(ids, "ids", torch.int32, (wanted, 1 + top))
         self._check(self.lib.fllm_logprobs(_ptr(logits), rows, vocab, _ptr(wanted_rows), wanted, _ptr(tokens), int(top),
                                            _ptr(values), _ptr(ids), self._stream()))
+
+    def logprobs_processed(self, logits: torch.Tensor, wanted_rows: torch.Tensor, tokens: torch.Tensor, params: torch.Tensor,
+                           top: int, values: torch.Tensor, ids: torch.Tensor) -> None:
+        """As `logprobs`, in the distribution each token was drawn from (fllm_logprobs_processed): `logits` are what the
+        sampler saw (penalties and biases applied), `params` the `SampleRow` records `sample` took (uint8 [rows, 32]):
+        temperature, then top-k, min-p and top-p with the sampler's ties; a greedy row is a point mass.  A chosen token
+        that the filters leave out gives -inf; where fewer than `top` tokens are left, the rest of `ids` is -1."""
+        rows, vocab = logits.shape
+        wanted = wanted_rows.numel()
+        _dense(logits, "logits", torch.float32)
+        _dense(wanted_rows, "wanted_rows", torch.int32, (wanted,))
+        _dense(tokens, "tokens", torch.int32, (rows,))
+        _dense(params, "params", torch.uint8, (rows, SAMPLE_ROW_BYTES))
+        _dense(values, "values", torch.float32, (wanted, 1 + top))
+        _dense(ids, "ids", torch.int32, (wanted, 1 + top))
+        self._check(self.lib.fllm_logprobs_processed(_ptr(logits), rows, vocab, _ptr(wanted_rows), wanted, _ptr(tokens), _ptr(params),
+                                                     int(top), _ptr(values), _ptr(ids), self._stream()))
 
     def sample(self, logits: torch.Tensor, work: torch.Tensor, params: torch.Tensor, out: torch.Tensor,
                kinds: int = 7) -> torch.Tensor:

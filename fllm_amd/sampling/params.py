@@ -38,6 +38,9 @@ class SamplingParams:
     timeout_secs: Optional[float] = None             # the request is given up this long after it was added (waiting included)
     logprobs: Optional[int] = None    # None: off; n: every token comes with its log-probability in the model's own
                                       # distribution (before penalties, temperature and filters) and the n likeliest tokens
+    logprobs_processed: bool = False  # the reference's `logprobs_mode: processed_logprobs`: the log-probabilities are those
+                                      # of the distribution the token was drawn from (after penalties, temperature and
+                                      # filters; greedy: a point mass), the alternatives the likeliest tokens that are left
 
     def __post_init__(self):
         if self.temperature < 0.0:

@@ -3,7 +3,7 @@ otherwise (temperature, top-k, top-p, Gumbel-max draw keyed by seed and draw num
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import List, Sequence
+from typing import List, Optional, Sequence
 
 import torch
 
@@ -92,23 +92,35 @@ class Sampler:
         """The token ids of `launch` on the host (waits for the device)."""
         return cls.finish_read(cls.start_read(tokens))
 
-    def start_logprobs(self, logits: torch.Tensor, tokens: torch.Tensor, wanted: Sequence[int], top: int):
+    def start_logprobs(self, logits: torch.Tensor, tokens: torch.Tensor, wanted: Sequence[int], top: int,
+                       processed: Sequence[int] = (), seen: Optional[torch.Tensor] = None,
+                       requests: Optional[Sequence[SampleRequest]] = None):
         """Asks for the log-probabilities of `tokens[r]` and of the `top` likeliest tokens in the softmax of `logits[r]`
-        (as the model gave them: hand in the logits as they were before `adjust`), for the rows r in `wanted`.  Nothing
-        waits: the kernel and the copies to the host are queued behind what chose the tokens.  Returns what
+        (as the model gave them: hand in the logits as they were before `adjust`), for the rows r in `wanted`.  The
+        rows in `processed` get theirs in the distribution they were drawn from instead (`SamplingParams.
+        logprobs_processed`): from `seen`, the logits as the sampler saw them, and `requests`, what `launch` took.
+        Nothing waits: the kernels and the copies to the host are queued behind what chose the tokens.  Returns what
         `finish_logprobs` takes."""
-        wanted = [int(r) for r in wanted]
-        if any(not 0 <= r < logits.shape[0] for r in wanted):
-            raise ValueError(f"log-probabilities asked for rows {wanted} of {logits.shape[0]}")
+        wanted, processed = [int(r) for r in wanted], [int(r) for r in processed]
+        if any(not 0 <= r < logits.shape[0] for r in wanted + processed):
+            raise ValueError(f"log-probabilities asked for rows {wanted + processed} of {logits.shape[0]}")
+        if processed and (seen is None or requests is None or len(requests) != logits.shape[0]):
+            raise ValueError("processed log-probabilities need the logits the sampler saw and its requests, one a row")
         top = min(int(top), logits.shape[1])
-        rows = torch.tensor(wanted, dtype=torch.int32)
+        rows = torch.tensor(wanted + processed, dtype=torch.int32)
         if logits.is_cuda:
             rows = rows.pin_memory().to(logits.device, non_blocking=True)
-        values = torch.empty((len(wanted), 1 + top), dtype=torch.float32, device=logits.device)
-        ids = torch.empty((len(wanted), 1 + top), dtype=torch.int32, device=logits.device)
+        values = torch.empty((len(wanted) + len(processed), 1 + top), dtype=torch.float32, device=logits.device)
+        ids = torch.empty((len(wanted) + len(processed), 1 + top), dtype=torch.int32, device=logits.device)
+        n = len(wanted)
         if wanted:
-            self.rt.ops.logprobs(logits, rows, tokens, top, values, ids)
-        return wanted, self.start_read(values), self.start_read(ids)
+            self.rt.ops.logprobs(logits, rows[:n], tokens, top, values[:n], ids[:n])
+        if processed:
+            params = pack_rows(requests)
+            if seen.is_cuda:
+                params = params.pin_memory().to(seen.device, non_blocking=True)
+            self.rt.ops.logprobs_processed(seen, rows[n:], tokens, params, top, values[n:], ids[n:])
+        return wanted + processed, self.start_read(values), self.start_read(ids)
 
     @staticmethod
     def finish_logprobs(pending) -> dict:

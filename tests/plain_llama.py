@@ -377,6 +377,29 @@ def raw_logprobs(logits, token, top_n):
     return float(logp[token]), [(i, float(logp[i])) for i in order]
 
 
+def processed_logprobs(logits, token, top_n, temperature, top_k=0, top_p=1.0, min_p=0.0):
+    """rust/engine/src/sampling.rs:365-381 and :928-935 (`logprobs_mode: processed_logprobs`): the log-probabilities of
+    the distribution a token is drawn from.  A greedy request (temperature <= 1e-5) is a point mass on the first largest
+    logit; otherwise the softmax of logits / T over the tokens the sampler still draws from (`device_survivors`, with its
+    ties kept).  Returns (log-probability of `token`, -inf outside the support; the min(top_n, 20) likeliest of the
+    tokens that are left as (id, log-probability), the lower id first among equals), or None without a finite logit."""
+    w = np.asarray(logits, dtype=np.float32)
+    finite = np.where(np.isfinite(w), w, -np.inf)
+    if not np.isfinite(finite).any():
+        return None
+    if temperature <= 1e-5:
+        first = greedy(finite)
+        return (0.0 if token == first else -math.inf), [(first, 0.0)][:min(top_n, 20)]
+    left = device_survivors(logits, temperature, top_k, top_p, min_p)
+    alive = np.isfinite(left)
+    inv_t = np.float32(1.0 / float(temperature))
+    scaled = ((finite - finite.max()) * inv_t).astype(np.float32).astype(np.float64)
+    log_mass = math.log(np.exp(scaled[alive]).sum())
+    logp = np.where(alive, scaled - log_mass, -np.inf)
+    order = sorted(np.flatnonzero(alive).tolist(), key=lambda i: (-logp[i], i))[:min(top_n, 20)]
+    return float(logp[token]), [(i, float(logp[i])) for i in order]
+
+
 def apply_penalties(logits, history, repetition_penalty=1.0, presence_penalty=0.0, frequency_penalty=0.0, repeat_last_n=-1,
                     logit_bias=()):
     """rust/engine/src/sampling.rs:252-274 and :579-598: over the last `repeat_last_n` tokens of the history (all of

@@ -214,6 +214,23 @@ class ReferenceOps:
                 ids[w, 1 + k] = got[1][k][0] if k < len(got[1]) else -1
                 values[w, 1 + k] = got[1][k][1] if k < len(got[1]) else float("nan")
 
+    def logprobs_processed(self, logits, wanted_rows, tokens, params, top, values, ids):
+        rec = np.frombuffer(params.cpu().numpy().tobytes(), dtype=np.dtype([("temperature", "<f4"), ("top_p", "<f4"), ("top_k", "<i4"),
+                                                                            ("min_p", "<f4"), ("seed", "<u8"), ("draw", "<u8")]))
+        for w, r in enumerate(int(r) for r in wanted_rows):
+            p = rec[r]
+            got = plain_llama.processed_logprobs(logits[r].float().cpu().numpy(), int(tokens[r]), top, float(p["temperature"]),
+                                                 int(p["top_k"]), float(p["top_p"]), float(p["min_p"]))
+            ids[w, 0] = int(tokens[r])
+            if got is None:
+                values[w] = float("nan")
+                ids[w, 1:] = torch.tensor([-1] * top, dtype=ids.dtype)
+                continue
+            values[w, 0] = got[0]
+            for k in range(top):
+                ids[w, 1 + k] = got[1][k][0] if k < len(got[1]) else -1
+                values[w, 1 + k] = got[1][k][1] if k < len(got[1]) else float("nan")
+
     def sample(self, logits, work, params, out, kinds=3):
         raw = params.cpu().numpy().tobytes()
         rec = np.frombuffer(raw, dtype=np.dtype([("temperature", "<f4"), ("top_p", "<f4"), ("top_k", "<i4"),

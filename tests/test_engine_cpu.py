@@ -1,6 +1,8 @@
 """The step function, the scheduler and generation on the CPU, with the plain kernels of
 tests/reference_ops.py in place of the HIP library: what is tested here is the engine's own
 logic (batches, pages, portions, preemption), not the kernels."""
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -497,6 +499,43 @@ def test_events_carry_the_models_own_log_probabilities(ahead):
     assert generated_with_penalty_differs(events["r0"])
     with pytest.raises(ValueError, match="between 0 and 20"):
         SamplingParams(logprobs=21)
+
+
+@pytest.mark.parametrize("ahead", [False, True])
+def test_events_carry_the_log_probabilities_of_the_distribution_drawn_from(ahead):
+    """`logprobs_processed`: after penalties, biases, temperature and filters; beside a request that asks for the
+    model's own in the same steps."""
+    cfg = tc.CONFIGS["A"]
+    _, spec = model_spec_from_config(cfg)
+    w64 = tc.to_float64(random_tensors(spec, 1, torch.float32))
+    engine = make_engine("A", ahead=ahead)
+    params = [SamplingParams(max_tokens=6, logprobs=3, logprobs_processed=True, repetition_penalty=1.8, logit_bias=((5, 4.0),)),
+              SamplingParams(max_tokens=6, logprobs=2),
+              SamplingParams(max_tokens=6, logprobs=4, logprobs_processed=True, temperature=0.9, top_k=3, seed=3)]
+    for i, (prompt, p) in enumerate(zip(PROMPTS_A, params)):
+        engine.add_request(f"r{i}", prompt, p)
+    events = {f"r{i}": [] for i in range(3)}
+    while engine.has_unfinished():
+        for ev in engine.step():
+            events[ev.request_id].append(ev)
+    for i in range(3):
+        generated = [ev.token_id for ev in events[f"r{i}"]]
+        logits = plain_llama.forward(cfg, w64, PROMPTS_A[i] + generated)
+        for k, ev in enumerate(events[f"r{i}"]):
+            row = logits[len(PROMPTS_A[i]) - 1 + k]
+            p = params[i]
+            if p.logprobs_processed:
+                seen = plain_llama.apply_penalties(row, PROMPTS_A[i] + generated[:k], p.repetition_penalty, p.presence_penalty,
+                                                   p.frequency_penalty, p.repeat_last_n, p.logit_bias)
+                chosen, alternatives = plain_llama.processed_logprobs(seen, ev.token_id, p.logprobs, p.temperature, p.top_k, p.top_p, p.min_p)
+            else:
+                chosen, alternatives = plain_llama.raw_logprobs(row, ev.token_id, p.logprobs)
+            assert abs(ev.logprob - chosen) < 1e-4, (i, k)
+            assert [t for t, _ in ev.top_logprobs] == [t for t, _ in alternatives], (i, k)
+            assert all(abs(a - b) < 1e-4 for (_, a), (_, b) in zip(ev.top_logprobs, alternatives))
+    # greedy with a penalty: a point mass on the token that was taken; top-k 3: three alternatives whatever was asked for
+    assert all(ev.logprob == 0.0 and ev.top_logprobs == [(ev.token_id, 0.0)] for ev in events["r0"])
+    assert all(len(ev.top_logprobs) == 3 and math.isfinite(ev.logprob) for ev in events["r2"])
 
 
 def generated_with_penalty_differs(events):

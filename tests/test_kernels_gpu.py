@@ -1197,6 +1197,53 @@ def test_logprobs(ops, vocab, top):
                      torch.empty(1, 22, device=DEV), torch.empty(1, 22, dtype=torch.int32, device=DEV))
 
 
+@pytest.mark.parametrize("vocab,top", [(300, 3), (1000, 5), (128256, 20), (7, 7)])
+def test_logprobs_of_the_distribution_a_token_was_drawn_from(ops, vocab, top):
+    """`logprobs_processed` against the plain function: greedy rows are point masses, sampled rows the softmax of
+    logits / T over what top-k, min-p and top-p leave (ties at a threshold kept, as the sampler keeps them); a token
+    outside the support has -inf, fewer survivors than alternatives leave the rest empty, and the token the sampler
+    draws from the same records lies inside the support."""
+    from fllm_amd.sampling import SampleRequest, SamplingParams, pack_rows
+    g = gen(80 + top)
+    settings = [dict(temperature=0.0), dict(temperature=0.8), dict(temperature=1.3, top_k=4), dict(temperature=0.7, top_p=0.6),
+                dict(temperature=1.0, top_k=50, top_p=0.9, min_p=0.02), dict(temperature=0.9, min_p=0.1), dict(temperature=0.5, top_k=2),
+                dict(temperature=1.1, top_k=3)]
+    rows = len(settings)
+    logits = torch.randn(rows, vocab, generator=g) * 3.0
+    logits[2, ::3] = -float("inf")
+    best = int(logits[7].argmax())
+    logits[7, (best + 1) % vocab] = logits[7, best]            # equal values at the top: top-k keeps its ties
+    logits[7, (best + 2) % vocab] = logits[7, best]
+    logits[7, (best + 3) % vocab] = logits[7, best]
+    requests = [SampleRequest(SamplingParams(**s), seed=11 + r, draw=r) for r, s in enumerate(settings)]
+    params = pack_rows(requests).to(DEV)
+    drawn = torch.empty(rows, dtype=torch.int32, device=DEV)
+    ops.sample(logits.to(DEV), torch.empty(rows, vocab, device=DEV), params, drawn)
+    tokens = drawn.cpu().clone()
+    tokens[6] = int(torch.argsort(logits[6], descending=True)[min(5, vocab - 1)])      # a token top-k 2 leaves out
+    wanted = [3, 0, 1, 2, 4, 5, 6, 7]
+    values = torch.full((len(wanted), 1 + top), 7.0, device=DEV)
+    ids = torch.full((len(wanted), 1 + top), 7, dtype=torch.int32, device=DEV)
+    ops.logprobs_processed(logits.to(DEV), torch.tensor(wanted, dtype=torch.int32, device=DEV), tokens.to(DEV), params, top, values, ids)
+    values, ids = values.cpu(), ids.cpu()
+    for w, r in enumerate(wanted):
+        s = settings[r]
+        chosen, alternatives = plain_llama.processed_logprobs(logits[r].numpy(), int(tokens[r]), top, s["temperature"], s.get("top_k", 0),
+                                                              s.get("top_p", 1.0), s.get("min_p", 0.0))
+        assert int(ids[w, 0]) == int(tokens[r])
+        assert ids[w, 1:].tolist() == [i for i, _ in alternatives] + [-1] * (top - len(alternatives)), (r, ids[w].tolist())
+        got = np.array([float(values[w, 0])] + values[w, 1:1 + len(alternatives)].tolist())
+        expected = np.array([chosen] + [v for _, v in alternatives])
+        finite = np.isfinite(expected)
+        assert np.array_equal(got[~finite], expected[~finite]), r
+        assert np.abs(got[finite] - expected[finite]).max() <= 2e-5, r
+        assert bool(torch.isnan(values[w, 1 + len(alternatives):]).all())
+        if r != 6:
+            assert math.isfinite(float(values[w, 0])), f"row {r}: the sampler drew a token outside the support"
+    assert float(values[wanted.index(6), 0]) == -math.inf and float(values[wanted.index(0), 0]) == 0.0
+    assert len([i for i in ids[wanted.index(7), 1:].tolist() if i >= 0]) == min(top, 4)       # four equal largest values survive top-k 3
+
+
 def test_sample_depends_only_on_seed_draw_and_logits(ops):
     from fllm_amd.sampling import SampleRequest, SamplingParams, pack_rows
     g = gen(18)

@@ -463,6 +463,36 @@ def test_raw_logprobs():
     assert [i for i, _ in top] == torch.argsort(want, descending=True, stable=True)[:20].tolist()
 
 
+def test_processed_logprobs():
+    """rust/engine/src/sampling.rs:1542-1556: the reference's own vector (only the survivors of top-k are listed, their
+    probabilities add up to one, a token outside the support has probability zero, greedy is a point mass), and the
+    softmax of logits / T over what the filters leave against the library's."""
+    logits = [3.0, 2.0, 1.0, 0.0, -1.0]
+    chosen, top = P.processed_logprobs(logits, 1, 5, 1.0, top_k=3)
+    assert [i for i, _ in top] == [0, 1, 2] and abs(sum(math.exp(v) for _, v in top) - 1.0) < 1e-6
+    assert abs(chosen - top[1][1]) < 1e-12
+    assert P.processed_logprobs(logits, 4, 5, 1.0, top_k=3)[0] == -math.inf
+    assert P.processed_logprobs(logits, 0, 3, 0.0) == (0.0, [(0, 0.0)])
+    assert P.processed_logprobs(logits, 2, 3, 0.0)[0] == -math.inf
+    assert P.processed_logprobs([-np.inf, float("nan")], 0, 1, 1.0) is None
+    rng = np.random.default_rng(8)
+    w = rng.normal(size=200).astype(np.float32) * 3
+    # no filter: log-softmax of w / T
+    chosen, top = P.processed_logprobs(w, 17, 20, 0.7)
+    want = torch.log_softmax(torch.from_numpy(w).double() / 0.7, 0)
+    assert abs(chosen - float(want[17])) < 1e-5 and [i for i, _ in top] == torch.argsort(want, descending=True, stable=True)[:20].tolist()
+    # top-k 6 and top-p 0.5: the renormalized head of that distribution; min-p drops what is 20 times lighter than the top
+    order = torch.argsort(want, descending=True, stable=True).tolist()
+    head = want[order[:6]].exp()
+    kept = int(np.flatnonzero(np.cumsum((head / head.sum()).numpy()) >= 0.5)[0]) + 1
+    chosen, top = P.processed_logprobs(w, order[0], 20, 0.7, top_k=6, top_p=0.5)
+    assert [i for i, _ in top] == order[:kept] and abs(sum(math.exp(v) for _, v in top) - 1.0) < 1e-6
+    assert abs(chosen - math.log(float(head[0] / head[:kept].sum()))) < 1e-5
+    assert P.processed_logprobs(w, order[kept], 20, 0.7, top_k=6, top_p=0.5)[0] == -math.inf
+    _, top = P.processed_logprobs(w, order[0], 20, 0.7, min_p=0.05)
+    assert [i for i, _ in top] == [i for i in order if float(want[i] - want[order[0]]) >= math.log(0.05)][:20]
+
+
 def test_draws_follow_the_distribution_and_depend_on_seed_and_draw_only():
     logits = np.array([2.0, 1.0, 0.0, -1.0], dtype=np.float32)
     p = np.exp(logits / 0.8)
