@@ -16,7 +16,7 @@ int fllm_abi_version(void);
 void fllm_set_fast_kernels(int on);
 // Switches a kernel variant (for measurements and tests): "attention.tile32" 0/1; "linear.slices" n
 // (0: chosen by shape); "linear.dual_k" 0/1; "linear.x_direct" 0/1; "attention.fused_merge" 0/1;
-// "attention.prefill_parts" 0/1; "linear.slab" 0/1/2; "linear.wide_waves" 0 (planned)/4/7/8;
+// "attention.prefill_parts" 0/1; "linear.slab" 0/1/2; "linear.wide_waves" 0 (planned)/4/7/8; "linear.resident_tiles" 0/1;
 // "attention.tile32_rows" 0 (chosen by the launch)/128/256.  0 on success.
 int fllm_set_option(const char *name, int value);
 

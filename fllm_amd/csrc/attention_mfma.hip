@@ -592,6 +592,13 @@ attn_tile32_kernel(AttnArgs p) {
 // ---------------------------------------------------------------------------------------------
 // decode kernel
 // ---------------------------------------------------------------------------------------------
+// A decode step reads the keys and values of a request once, so these loads carry the non-temporal hint (a step of
+// the 8B sizes at batch 8: 4.75 -> 4.62 ms at contexts of 8,192, 8.88 -> 8.34 ms at 32,768; 6.20 -> 6.02 ms at batch 64).
+#ifdef FLLM_CACHE_TEMPORAL
+#define FLLM_CACHE_LOAD(ptr) (*(ptr))
+#else
+#define FLLM_CACHE_LOAD(ptr) __builtin_nontemporal_load(ptr)
+#endif
 template <int D, int WAVES>
 __global__ void __launch_bounds__(WAVES * kWave)
 attn_decode_kernel(AttnArgs p, int qtiles) {
@@ -662,13 +669,13 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
             const bool valid = key >= lo && key < n;
             const bf16_t *kr = p.kp + key_offset(kpage[j], nkv, kvh, ps, D, key & pmask, g * 8);
 #pragma unroll
-            for (int kk = 0; kk < KD; kk++) kf[j][kk] = valid ? *(const bf16x8_t *)(kr + (size_t)kk * 4 * ps * 8) : zero8();
+            for (int kk = 0; kk < KD; kk++) kf[j][kk] = valid ? FLLM_CACHE_LOAD((const bf16x8_t *)(kr + (size_t)kk * 4 * ps * 8)) : zero8();
             const int vkey = kb + 16 * j + 4 * g;
             const bool vload = vkey < n && vkey + 4 > lo;
             vtail[j] = vload && vkey + 4 > n;
             const bf16_t *vr = p.vp + (((size_t)vpage[j] * nkv + kvh) * D + c) * ps + (vkey & pmask);
 #pragma unroll
-            for (int dt = 0; dt < DT; dt++) vf[j][dt] = vload ? *(const bf16x4_t *)(vr + (size_t)dt * 16 * ps) : (bf16x4_t){(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
+            for (int dt = 0; dt < DT; dt++) vf[j][dt] = vload ? FLLM_CACHE_LOAD((const bf16x4_t *)(vr + (size_t)dt * 16 * ps)) : (bf16x4_t){(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
         }
 
         f32x4_t s[2];

@@ -35,6 +35,7 @@ int fllm_option_x_direct(void);
 // that kernel can serve; 2 a K slice of the activations stays in LDS wherever that kernel can serve
 int fllm_option_slab(void);
 int fllm_option_wide_waves(void);
+int fllm_option_resident_tiles(void);
 int fllm_option_tile32_rows(void);
 // 1: decode-shaped products of up to 8 rows use 8-row weight tiles with two K halves a product (default); 0: 16-row tiles
 int fllm_option_dual_k(void);

@@ -304,11 +304,22 @@ __device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], 
 // result does not depend on which workgroup came last.
 enum { TM_ROWS16 = 0, TM_DUALK = 1, TM_GATEUP = 2 };
 
+// A load of weights.  Every weight is read once a step, so the loads carry the non-temporal hint: the lines do not
+// push the activations, which every workgroup reads again, out of the caches (a decode step of the 8B sizes: 3.68 ->
+// 3.60 ms at batch 8, 4.69 -> 4.53 at 32, 6.30 -> 6.19 at 64).
+__device__ __forceinline__ bf16x8_t load_weights(const bf16_t *p) {
+#ifdef FLLM_WEIGHTS_TEMPORAL
+    return *(const bf16x8_t *)p;
+#else
+    return __builtin_nontemporal_load((const bf16x8_t *)p);
+#endif
+}
+
 template <int PRO, int EPI, int TM, int WAVES, bool XD, bool WT = false>
 __global__ void __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4, 4)))   // 16 waves a CU: 128 registers
 skinny_resident_kernel(SkinnyArgs a, int red_off) {
     static_assert(!XD || PRO == PRO_BF16, "activations straight from global memory: the bfloat16 prologue only");
-    static_assert(!WT || (TM == TM_ROWS16 && XD), "tile-major weights: 16-row tiles, one slice");
+    static_assert(!WT || TM == TM_ROWS16, "tile-major weights: whole 16-row tiles, one slice");
     constexpr int U = 4;                           // k-steps of 32 per block: four 16-byte loads per lane
     constexpr int KB = 32 * U;                     // K elements of one range per block
     constexpr int RB = 4;                          // rows of activations staged at a time (more would spill registers)
@@ -363,11 +374,11 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
                 // the lanes take them, so a load instruction reads 1 KiB in a row instead of 64 bytes of each of 16 rows
                 const bf16_t *wp = a.w_tiles + (size_t)(tile0 + l_item * tstride) * 16 * K + (size_t)((kw0 + l_j * KB) / KB) * (16 * KB) + lane * 8;
 #pragma unroll
-                for (int u = 0; u < U; u++) buf.w[u] = kb + u * 32 < kr1 ? *(const bf16x8_t *)(wp + u * (16 * 32)) : zero8();
+                for (int u = 0; u < U; u++) buf.w[u] = kb + u * 32 < kr1 ? load_weights(wp + u * (16 * 32)) : zero8();
             } else {
                 const bf16_t *wp = a.w + (size_t)row * K + ks0 + kb;
 #pragma unroll
-                for (int u = 0; u < U; u++) buf.w[u] = kb + u * 32 < kr1 ? *(const bf16x8_t *)(wp + u * 32) : zero8();
+                for (int u = 0; u < U; u++) buf.w[u] = kb + u * 32 < kr1 ? load_weights(wp + u * 32) : zero8();
             }
             if (XD) {
                 const bf16_t *xp = (const bf16_t *)a.x + (size_t)xrow_i * a.ldx + ks0 + kb;
@@ -665,11 +676,11 @@ skinny_wide_kernel(SkinnyArgs a) {
             // a chunk is two blocks of 128 columns of the tile, each 4 KiB in the order the lanes take it
             const bf16_t *wp = a.w_tiles + (size_t)min(tile, ntiles - 1) * 16 * K + (size_t)((ks0 + w_chunk * KC) >> 7) * 2048 + lane * 8;
 #pragma unroll
-            for (int u = 0; u < KS; u++) buf[u] = *(const bf16x8_t *)(live ? wp + (u >> 2) * 2048 + (u & 3) * 512 : zeros);
+            for (int u = 0; u < KS; u++) buf[u] = load_weights(live ? wp + (u >> 2) * 2048 + (u & 3) * 512 : zeros);
         } else {
             const bf16_t *wp = a.w + (size_t)row * K + ks0;
 #pragma unroll
-            for (int u = 0; u < KS; u++) buf[u] = *(const bf16x8_t *)(live ? wp + min(kb + u * 32, kcn - 8) : zeros);
+            for (int u = 0; u < KS; u++) buf[u] = load_weights(live ? wp + min(kb + u * 32, kcn - 8) : zeros);
         }
         if (++w_chunk == nchunks) w_chunk = 0, w_item++;
     };
@@ -898,7 +909,7 @@ skinny_slab_kernel(SkinnyArgs a, int cells_off) {
         const int kb = ((w_chunk + phase) % nchunks) * KC + g * 8;
         const bf16_t *wp = a.w + (size_t)row * K + ks0;
 #pragma unroll
-        for (int u = 0; u < KS; u++) buf[u] = *(const bf16x8_t *)(live ? wp + min(kb + u * 32, kcn - 8) : zeros);
+        for (int u = 0; u < KS; u++) buf[u] = load_weights(live ? wp + min(kb + u * 32, kcn - 8) : zeros);
         if (++w_chunk == nchunks) w_chunk = 0, w_item++;
     };
     bf16x8_t wa[KS], wb[KS];
@@ -1208,6 +1219,12 @@ __global__ void __launch_bounds__(256) tile_weights_kernel(const bf16_t *__restr
     }
 }
 
+// Whether a staged launch (activations in LDS) may stream the tile-major copy: one slice, and every wave's K range whole
+// blocks of 128 columns
+bool staged_tiles_fit(const SkinnyArgs &a, const ResidentPlan &p, int n_out) {
+    return a.w_tiles != nullptr && p.S == 1 && tiles_fit(n_out, a.K) && a.K % (p.waves * 128) == 0;
+}
+
 template <int PRO, int EPI>
 int launch_resident(const SkinnyArgs &a, hipStream_t stream) {
     constexpr int RT = EPI == EPI_SWIGLU ? 2 : 1;
@@ -1247,6 +1264,16 @@ int launch_resident(const SkinnyArgs &a, hipStream_t stream) {
             if (x_direct) {
                 if (dual) return launch_resident_plan<PRO, EPI, TM_DUALK, 8, true>(a, p, tiles8, ws, stream);
                 return launch_resident_plan<PRO, EPI, TM_ROWS16, 8, true>(a, p, tiles16, ws, stream);
+            }
+        }
+        if constexpr (EPI == EPI_QKV) {
+            // q/k/v behind a prepared norm: whole 16-row tiles from the tile-major copy, where there is one, rather than
+            // 8-row tiles of the matrix (4,096 x 6,144: 13.2 -> 12.4 us at one row, 15.2 -> 15.0 at 8, 19.6 -> 18.1 at 16).
+            // Reading the activations straight from global memory as the output projection does is slower here
+            // (14.0, 15.4, 18.3 us), and the gate/up product gains nothing from its copy (41.1 us at one row either way).
+            if (!x_direct && fllm_option_resident_tiles() && staged_tiles_fit(a, p, a.N)) {
+                if (p.waves == 8) return launch_resident_plan<PRO, EPI, TM_ROWS16, 8, false, true>(a, p, tiles16, ws, stream);
+                return launch_resident_plan<PRO, EPI, TM_ROWS16, 16, false, true>(a, p, tiles16, ws, stream);
             }
         }
         if (dual) {
@@ -1650,10 +1677,8 @@ extern "C" int fllm_scaled_gate_up_swiglu(const void *xn, const float *ssq, int 
     a.M = M;
     a.N = 2 * inter;
     a.K = K;
-    if (M > 16) {
-        a.w_tiles = (const bf16_t *)w_tiles;
-        return dispatch_wide<EPI_SWIGLU, PRO_SCALED>(a, stream);
-    }
+    a.w_tiles = (const bf16_t *)w_tiles;
+    if (M > 16) return dispatch_wide<EPI_SWIGLU, PRO_SCALED>(a, stream);
     const int rc = launch_resident<PRO_SCALED, EPI_SWIGLU>(a, stream);
     FLLM_REQUIRE(rc != 1, "scaled_gate_up_swiglu: shape M=%d K=%d does not fit the staging area", M, K);
     return rc;
@@ -1678,10 +1703,8 @@ extern "C" int fllm_scaled_qkv_rope_store(const void *xn, const float *ssq, int 
                             k_pages, v_pages, M, heads, kv_heads, head_dim, K, page_size, store_kv);
     a.ssq_in = ssq;
     a.ssq_count = ssq_count;
-    if (M > 16) {
-        a.w_tiles = (const bf16_t *)w_tiles;
-        return dispatch_wide<EPI_QKV, PRO_SCALED>(a, stream);
-    }
+    a.w_tiles = (const bf16_t *)w_tiles;
+    if (M > 16) return dispatch_wide<EPI_QKV, PRO_SCALED>(a, stream);
     const int rc = launch_resident<PRO_SCALED, EPI_QKV>(a, stream);
     FLLM_REQUIRE(rc != 1, "scaled_qkv_rope_store: shape M=%d K=%d does not fit the staging area", M, K);
     return rc;

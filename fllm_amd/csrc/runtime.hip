@@ -37,6 +37,8 @@ static int g_tile32_rows = 0;     // 0: chosen by the launch; 128 or 256
 int fllm_option_tile32_rows(void) { return g_tile32_rows; }
 static int g_wide_waves = 0;      // 0: planned
 int fllm_option_wide_waves(void) { return g_wide_waves; }
+static int g_resident_tiles = 1;  // q/k/v of up to 16 rows behind a prepared norm streams its tile-major copy (16-row tiles)
+int fllm_option_resident_tiles(void) { return g_resident_tiles; }
 static int g_slab = 1;
 int fllm_option_slab(void) { return g_slab; }
 static int g_fused_merge = 1;
@@ -61,6 +63,10 @@ extern "C" int fllm_set_option(const char *name, int value) {
     }
     if (strcmp(name, "attention.tile32_rows") == 0) {
         g_tile32_rows = (value == 128 || value == 256) ? value : 0;
+        return 0;
+    }
+    if (strcmp(name, "linear.resident_tiles") == 0) {
+        g_resident_tiles = value != 0;
         return 0;
     }
     if (strcmp(name, "linear.wide_waves") == 0) {

@@ -452,10 +452,11 @@ class Ops:
         return M, K
 
     def _chunk_tiles(self, M: int, K: int, w: torch.Tensor, gate_up: bool = False) -> Optional[torch.Tensor]:
-        """The tile-major copy that a prepared norm of more than 16 rows needs (None up to 16 rows)."""
+        """The tile-major copy that a prepared norm of more than 16 rows needs; up to 16 rows the kernel streams it
+        where there is one and the launch it chooses can."""
+        tiles = self._tiles_of(w, gate_up=gate_up) if Ops._tiles else None
         if M <= self.PREPARED_NORM_ROWS:
-            return None
-        tiles = self._tiles_of(w, gate_up=gate_up)
+            return tiles
         _need(tiles is not None and K % 256 == 0,
               f"a prepared norm of {M} rows needs the tile-major copy of the matrix (tile_for_decode) and a width in steps of 256, not {K}")
         return tiles

@@ -575,6 +575,49 @@ def test_a_product_prepares_the_norm_that_reads_its_sums(ops, ref, M, N, K):
                                torch.zeros(2, 24, device=DEV), torch.ones(24, device=DEV))
 
 
+@pytest.mark.parametrize("M,heads,kv_heads,head_dim,K,bias", [(1, 32, 8, 128, 4096, False), (8, 32, 8, 128, 4096, True), (16, 32, 8, 128, 4096, False),
+                                                              (5, 6, 2, 80, 2048, True), (11, 3, 1, 16, 1024, True), (9, 8, 4, 64, 3072, False)])
+def test_qkv_of_up_to_16_rows_streams_the_tile_major_copy(ops, ref, M, heads, kv_heads, head_dim, K, bias):
+    """Up to 16 rows the q/k/v product behind a prepared norm reads whole 16-row tiles from the tile-major copy where
+    there is one and the launch fits it; without the copy (or with the switch off) it reads the matrix, in 8-row tiles
+    where those fill the device better.  All of them against the form that norms the float32 rows itself."""
+    g = gen(300 + M + heads)
+    page_size = 16
+    rows = (torch.randn(M, K, generator=g) * torch.rand(M, 1, generator=g) * 4).to(DEV)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV)
+    n = (heads + 2 * kv_heads) * head_dim
+    wq = (torch.randn(n, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).to(DEV)
+    bq = (torch.randn(n, generator=g) * 0.1).to(DEV) if bias else None
+    prepared = ops.prepare_norm(rows, nw)
+    tables = scattered_tables(g, M, 8, M * 8 + 2).to(DEV)
+    row_pos = torch.tensor([(7 * r + 3) % 128 for r in range(M)], dtype=torch.int32, device=DEV)
+    row_seg = torch.arange(M, dtype=torch.int32, device=DEV)
+    angle = torch.rand(128, head_dim // 2, generator=g, dtype=torch.float64) * 6.28
+    cos, sin = torch.cos(angle).float().to(DEV), torch.sin(angle).float().to(DEV)
+    k0, v0 = make_pages(g, M * 8 + 2, kv_heads, page_size, head_dim, torch.bfloat16)
+
+    def product(**kwargs):
+        kp, vp = k0.to(DEV), v0.to(DEV)
+        q = ops.norm_qkv_rope_store(rows, nw, 1e-5, wq, torch.zeros(M, heads * head_dim, dtype=torch.bfloat16, device=DEV), row_pos, row_seg,
+                                    tables, cos, sin, kp, vp, heads, kv_heads, head_dim, head_dim, page_size, bias=bq, **kwargs)
+        return q, kp, vp
+
+    base = product()
+    without = product(prepared=prepared)
+    assert ops.tile_for_decode(wq) == (K % 1024 == 0)
+    with_copy = product(prepared=prepared)
+    ops.set_option("linear.resident_tiles", 0)
+    try:
+        switched_off = product(prepared=prepared)
+    finally:
+        ops.set_option("linear.resident_tiles", 1)
+    for a, b in zip(switched_off, without):
+        assert torch.equal(a, b)
+    for other in (without, with_copy):
+        for got, want in zip(other, base):
+            assert float((got.float() - want.float()).abs().max()) <= 2 * BF16_EPS * float(want.float().abs().max())
+
+
 @pytest.mark.parametrize("M,N,K", [(17, 4096, 4096), (64, 4096, 14336), (33, 1024, 2048), (48, 2048, 1024), (64, 2048, 8192)])
 def test_prepared_norms_of_17_to_64_rows(ops, ref, M, N, K):
     """Steps of 17 to 64 rows run the same five kernels a layer as smaller ones, on the kernels that pass the
