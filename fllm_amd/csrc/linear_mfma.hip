@@ -13,7 +13,7 @@
 #include "common.h"
 
 int fllm_linear_bf16_skinny(const void *x, int ldx, const void *w, const float *bias, void *out, int ldo, int M, int N,
-                            int K, int out_mode, hipStream_t stream);   // linear_skinny.hip; 1: shape declined
+                            int K, int out_mode, hipStream_t stream, const void *w_tiles = nullptr);   // linear_skinny.hip; 1: shape declined
 
 namespace {
 

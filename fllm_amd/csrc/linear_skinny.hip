@@ -304,14 +304,19 @@ __device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], 
 // result does not depend on which workgroup came last.
 enum { TM_ROWS16 = 0, TM_DUALK = 1, TM_GATEUP = 2 };
 
-// A load of weights.  Every weight is read once a step, so the loads carry the non-temporal hint: the lines do not
-// push the activations, which every workgroup reads again, out of the caches (a decode step of the 8B sizes: 3.68 ->
-// 3.60 ms at batch 8, 4.69 -> 4.53 at 32, 6.30 -> 6.19 at 64).
+// A load of weights.  Every weight is read once a step, so the loads from the tile-major copies carry the
+// non-temporal hint: the lines do not push the activations, which every workgroup reads again, out of the caches, and a
+// kernel that only reads gets 7.1 instead of 6.3 TB/s with it.  Only where a load instruction takes whole 128-byte
+// lines, though: from the matrix as the checkpoint has it an instruction takes half a line of each of 16 rows and the
+// next one the other half, and with the hint the second asks memory again (4,096 x 28,672 at one row: 41.0 us plain,
+// 43.0 with the hint, 38.0 with hint and copy; the vocabulary projection 176.8 us plain, 187.8 with the hint).
+template <bool STREAMED>
 __device__ __forceinline__ bf16x8_t load_weights(const bf16_t *p) {
 #ifdef FLLM_WEIGHTS_TEMPORAL
     return *(const bf16x8_t *)p;
 #else
-    return __builtin_nontemporal_load((const bf16x8_t *)p);
+    if (STREAMED) return __builtin_nontemporal_load((const bf16x8_t *)p);
+    return *(const bf16x8_t *)p;
 #endif
 }
 
@@ -319,7 +324,7 @@ template <int PRO, int EPI, int TM, int WAVES, bool XD, bool WT = false>
 __global__ void __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(4, 4)))   // 16 waves a CU: 128 registers
 skinny_resident_kernel(SkinnyArgs a, int red_off) {
     static_assert(!XD || PRO == PRO_BF16, "activations straight from global memory: the bfloat16 prologue only");
-    static_assert(!WT || TM == TM_ROWS16, "tile-major weights: whole 16-row tiles, one slice");
+    static_assert(!WT || TM != TM_DUALK, "tile-major weights: whole 16-row tiles (or 8 gate and 8 up rows), one slice");
     constexpr int U = 4;                           // k-steps of 32 per block: four 16-byte loads per lane
     constexpr int KB = 32 * U;                     // K elements of one range per block
     constexpr int RB = 4;                          // rows of activations staged at a time (more would spill registers)
@@ -374,11 +379,11 @@ skinny_resident_kernel(SkinnyArgs a, int red_off) {
                 // the lanes take them, so a load instruction reads 1 KiB in a row instead of 64 bytes of each of 16 rows
                 const bf16_t *wp = a.w_tiles + (size_t)(tile0 + l_item * tstride) * 16 * K + (size_t)((kw0 + l_j * KB) / KB) * (16 * KB) + lane * 8;
 #pragma unroll
-                for (int u = 0; u < U; u++) buf.w[u] = kb + u * 32 < kr1 ? load_weights(wp + u * (16 * 32)) : zero8();
+                for (int u = 0; u < U; u++) buf.w[u] = kb + u * 32 < kr1 ? load_weights<true>(wp + u * (16 * 32)) : zero8();
             } else {
                 const bf16_t *wp = a.w + (size_t)row * K + ks0 + kb;
 #pragma unroll
-                for (int u = 0; u < U; u++) buf.w[u] = kb + u * 32 < kr1 ? load_weights(wp + u * 32) : zero8();
+                for (int u = 0; u < U; u++) buf.w[u] = kb + u * 32 < kr1 ? load_weights<false>(wp + u * 32) : zero8();
             }
             if (XD) {
                 const bf16_t *xp = (const bf16_t *)a.x + (size_t)xrow_i * a.ldx + ks0 + kb;
@@ -676,11 +681,11 @@ skinny_wide_kernel(SkinnyArgs a) {
             // a chunk is two blocks of 128 columns of the tile, each 4 KiB in the order the lanes take it
             const bf16_t *wp = a.w_tiles + (size_t)min(tile, ntiles - 1) * 16 * K + (size_t)((ks0 + w_chunk * KC) >> 7) * 2048 + lane * 8;
 #pragma unroll
-            for (int u = 0; u < KS; u++) buf[u] = load_weights(live ? wp + (u >> 2) * 2048 + (u & 3) * 512 : zeros);
+            for (int u = 0; u < KS; u++) buf[u] = load_weights<true>(live ? wp + (u >> 2) * 2048 + (u & 3) * 512 : zeros);
         } else {
             const bf16_t *wp = a.w + (size_t)row * K + ks0;
 #pragma unroll
-            for (int u = 0; u < KS; u++) buf[u] = load_weights(live ? wp + min(kb + u * 32, kcn - 8) : zeros);
+            for (int u = 0; u < KS; u++) buf[u] = load_weights<false>(live ? wp + min(kb + u * 32, kcn - 8) : zeros);
         }
         if (++w_chunk == nchunks) w_chunk = 0, w_item++;
     };
@@ -909,7 +914,7 @@ skinny_slab_kernel(SkinnyArgs a, int cells_off) {
         const int kb = ((w_chunk + phase) % nchunks) * KC + g * 8;
         const bf16_t *wp = a.w + (size_t)row * K + ks0;
 #pragma unroll
-        for (int u = 0; u < KS; u++) buf[u] = load_weights(live ? wp + min(kb + u * 32, kcn - 8) : zeros);
+        for (int u = 0; u < KS; u++) buf[u] = load_weights<false>(live ? wp + min(kb + u * 32, kcn - 8) : zeros);
         if (++w_chunk == nchunks) w_chunk = 0, w_item++;
     };
     bf16x8_t wa[KS], wb[KS];
@@ -1239,6 +1244,10 @@ int launch_resident(const SkinnyArgs &a, hipStream_t stream) {
     if constexpr (EPI == EPI_SWIGLU) {
         const ResidentPlan p = plan_resident(a.M, a.K, tiles8, RT, ws, false);
         if (p.S == 0) return 1;
+        if (fllm_option_resident_tiles() && staged_tiles_fit(a, p, n_out)) {    // the copy of fllm_tile_weights_gate_up
+            if (p.waves == 8) return launch_resident_plan<PRO, EPI, TM_GATEUP, 8, false, true>(a, p, tiles8, ws, stream);
+            return launch_resident_plan<PRO, EPI, TM_GATEUP, 16, false, true>(a, p, tiles8, ws, stream);
+        }
         if (p.waves == 8) return launch_resident_plan<PRO, EPI, TM_GATEUP, 8>(a, p, tiles8, ws, stream);
         return launch_resident_plan<PRO, EPI, TM_GATEUP, 16>(a, p, tiles8, ws, stream);
     } else {
@@ -1266,11 +1275,11 @@ int launch_resident(const SkinnyArgs &a, hipStream_t stream) {
                 return launch_resident_plan<PRO, EPI, TM_ROWS16, 8, true>(a, p, tiles16, ws, stream);
             }
         }
-        if constexpr (EPI == EPI_QKV) {
-            // q/k/v behind a prepared norm: whole 16-row tiles from the tile-major copy, where there is one, rather than
-            // 8-row tiles of the matrix (4,096 x 6,144: 13.2 -> 12.4 us at one row, 15.2 -> 15.0 at 8, 19.6 -> 18.1 at 16).
-            // Reading the activations straight from global memory as the output projection does is slower here
-            // (14.0, 15.4, 18.3 us), and the gate/up product gains nothing from its copy (41.1 us at one row either way).
+        if constexpr ((EPI == EPI_QKV && PRO == PRO_SCALED) || (EPI == EPI_STORE_F32 && PRO == PRO_BF16)) {
+            // q/k/v behind a prepared norm and the vocabulary projection: whole 16-row tiles from the tile-major copy,
+            // where there is one, rather than the matrix (in 8-row tiles where those fill the device better).  Reading
+            // the activations straight from global memory as the output projection does is slower for q/k/v
+            // (4,096 x 6,144 at 1, 8, 16 rows: 14.0, 15.4, 18.3 us against 12.4, 15.0, 18.1 staged).
             if (!x_direct && fllm_option_resident_tiles() && staged_tiles_fit(a, p, a.N)) {
                 if (p.waves == 8) return launch_resident_plan<PRO, EPI, TM_ROWS16, 8, false, true>(a, p, tiles16, ws, stream);
                 return launch_resident_plan<PRO, EPI, TM_ROWS16, 16, false, true>(a, p, tiles16, ws, stream);
@@ -1406,12 +1415,13 @@ bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 // The decode-shaped product of fllm_linear.  0: launched, negative: error, 1: shape declined.
 int fllm_linear_bf16_skinny(const void *x, int ldx, const void *w, const float *bias, void *out, int ldo, int M, int N,
-                            int K, int out_mode, hipStream_t stream) {
+                            int K, int out_mode, hipStream_t stream, const void *w_tiles) {
     if (M > 64 || K % 8 != 0 || ldx % 8 != 0 || !aligned16(x) || !aligned16(w)) return 1;
     SkinnyArgs a = {};
     a.x = x;
     a.ldx = ldx;
     a.w = (const bf16_t *)w;
+    a.w_tiles = M <= 16 && out_mode == 1 ? (const bf16_t *)w_tiles : nullptr;     // the form that streams it
     a.bias = bias;
     a.out = out;
     a.ldo = ldo;
@@ -1621,6 +1631,19 @@ extern "C" int fllm_linear_add_tiled(const void *x, int ldx, const void *w, cons
     a.K = K;
     const int rc = M <= 16 ? launch_resident<PRO_BF16, EPI_ADD>(a, stream) : dispatch_wide<EPI_ADD>(a, stream);
     FLLM_REQUIRE(rc != 1, "linear_add_tiled: shape M=%d K=%d does not fit the staging area", M, K);
+    return rc;
+}
+
+// out = x w^T (+ bias) for 1..16 bfloat16 rows and a float32 `out` (the vocabulary projection of a decode step), as
+// fllm_linear in mode 1, from the tile-major copy of w where the launch it chooses can stream it.
+extern "C" int fllm_linear_f32_tiled(const void *x, int ldx, const void *w, const void *w_tiles, const float *bias, float *out, int ldo,
+                                     int M, int N, int K, hipStream_t stream) {
+    FLLM_REQUIRE(M >= 1 && M <= 16 && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && ldx >= K && ldo >= N,
+                 "linear_f32_tiled: takes 1..16 rows, K and ldx in steps of 8 (M=%d N=%d K=%d ldx=%d ldo=%d)", M, N, K, ldx, ldo);
+    FLLM_REQUIRE(aligned16(x) && aligned16(w) && out != nullptr && (w_tiles == nullptr || aligned16(w_tiles)),
+                 "linear_f32_tiled: operands must be there and 16-byte aligned");
+    const int rc = fllm_linear_bf16_skinny(x, ldx, w, bias, out, ldo, M, N, K, 1, stream, w_tiles);
+    FLLM_REQUIRE(rc != 1, "linear_f32_tiled: shape M=%d K=%d does not fit the staging area", M, K);
     return rc;
 }
 

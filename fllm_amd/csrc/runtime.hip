@@ -189,4 +189,4 @@ extern "C" double fllm_probe_mfma_bf16(void *sink, int blocks, int iters, hipStr
 }
 
 extern "C" const char *fllm_last_error(void) { return g_error; }
-extern "C" int fllm_abi_version(void) { return 10; }   // 10: fllm_logprobs_processed, fllm_prepare_norm.  9: tiles for 17 to 64 rows, fllm_scaled_* take w_tiles.  8: weight tiles.  7: fllm_random_fill.  2: fllm_attention takes single_from; probes.  3: fllm_sample takes kinds.  4: fllm_logprobs.  5: FllmAdjustLists.  6: fllm_linear_add_normed, fllm_scaled_*
+extern "C" int fllm_abi_version(void) { return 11; }   // 11: fllm_linear_f32_tiled.  10: fllm_logprobs_processed, fllm_prepare_norm.  9: tiles for 17 to 64 rows, fllm_scaled_* take w_tiles.  8: weight tiles.  7: fllm_random_fill.  2: fllm_attention takes single_from; probes.  3: fllm_sample takes kinds.  4: fllm_logprobs.  5: FllmAdjustLists.  6: fllm_linear_add_normed, fllm_scaled_*

@@ -49,7 +49,7 @@ assert SAMPLE_ROW_BYTES == 32
 _lib = None
 
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 
 def load_library(build_if_missing: bool = True):
@@ -96,6 +96,7 @@ def load_library(build_if_missing: bool = True):
         "fllm_tile_weights_gate_up": [c_void, c_void, c_int, c_int, c_void],
         "fllm_gate_up_swiglu_tiled": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_linear_add_tiled": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_void],
+        "fllm_linear_f32_tiled": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_void],
         "fllm_scaled_gate_up_swiglu": [c_void, c_void, c_int, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_void, c_void],
         "fllm_scaled_qkv_rope_store": [c_void, c_void, c_int, c_float, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void,
                                        c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void, c_void],
@@ -190,10 +191,10 @@ class Ops:
 
     def tile_for_decode(self, w: torch.Tensor, gate_up: bool = False) -> bool:
         """Keeps beside `w` (bfloat16 [N, K] on the GPU) a copy in the order in which the products of decode steps read
-        it (`fllm_tile_weights`): `linear(..., accumulate=True)` and `linear_add_prepare` find it by the matrix's address
-        and use it for steps of up to 64 rows.  `gate_up`: w is [gate; up] and the copy is for `gate_up_swiglu` at 17 to
-        64 rows (8 gate rows and the same 8 up rows a tile, `fllm_tile_weights_gate_up`).  The copy is given up with
-        `w`.  False: nothing was made (another type or place, a shape the kernels do not take tiles of)."""
+        it (`fllm_tile_weights`): `linear(..., accumulate=True)`, `linear_add_prepare`, the forms behind a prepared norm
+        and `linear` with float32 logits of up to 16 rows find it by the matrix's address and use it for steps of up to 64
+        rows.  `gate_up`: w is [gate; up] and the copy holds 8 gate rows and the same 8 up rows a tile
+        (`fllm_tile_weights_gate_up`), for `norm_gate_up_swiglu` and `gate_up_swiglu`.  The copy is given up with `w`.  False: nothing was made (another type or place, a shape the kernels do not take tiles of)."""
         if not (w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()):
             return False
         N, K = w.shape
@@ -333,10 +334,10 @@ class Ops:
             _dense(bias, "bias", torch.float32, (N,))
         ldx = x.stride(0) if M > 1 else K
         ldo = out.stride(0) if M > 1 else N
-        tiles = self._tiles_of(w) if mode == OUT_ADD_F32 and M <= 64 and Ops._tiles else None
+        tiles = self._tiles_of(w) if Ops._tiles and (M <= 64 if mode == OUT_ADD_F32 else mode == OUT_STORE_F32 and M <= 16) else None
         if tiles is not None and ldx % 8 == 0 and K % 8 == 0:
-            self._check(self.lib.fllm_linear_add_tiled(_ptr(x), ldx, _ptr(w), _ptr(tiles), _ptr(bias), _ptr(out), ldo, M, N, K,
-                                                       self._stream()))
+            entry = self.lib.fllm_linear_add_tiled if mode == OUT_ADD_F32 else self.lib.fllm_linear_f32_tiled
+            self._check(entry(_ptr(x), ldx, _ptr(w), _ptr(tiles), _ptr(bias), _ptr(out), ldo, M, N, K, self._stream()))
             return out
         if (self.library_gemm_from is not None and M >= self.library_gemm_from and x.dtype == torch.bfloat16
                 and bias is None):

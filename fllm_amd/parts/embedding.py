@@ -37,6 +37,7 @@ class LinearHead(Part):
         super().__init__(spec, weights, rt)
         self.weight = rt.matrix(weights["weight"])
         self.vocab = int(spec["vocab_size"])
+        rt.tile_for_decode(self.weight, priority=2)      # read once a step of up to 16 rows: after the layers' copies
 
     def forward(self, ctx, h):
         logits = self.rt.empty((h.shape[0], self.vocab), torch.float32)

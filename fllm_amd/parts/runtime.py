@@ -50,7 +50,7 @@ class Runtime:
         bytes again and takes a fifth off such a product at 8 rows).  `gate_up`: w is [gate; up], see the library.
         `priority`: while a model is being built the copies are only asked for, and made when it is whole
         (`tiles_for_model`), the lower numbers first: 0 for copies that every decode step reads (output and down
-        projections), 1 for those of steps of 17 to 64 rows only."""
+        projections), 1 for the layers' other matrices, 2 for the vocabulary projection (once a step)."""
         make = getattr(self.ops, "tile_for_decode", None)
         if not self.decode_weight_tiles or make is None or self.dtype != torch.bfloat16 or not w.is_cuda:
             return
