@@ -1328,7 +1328,7 @@ int launch_wide(SkinnyArgs a, hipStream_t stream) {
         *a.next_tiles_out = ntiles;
     }
     constexpr bool kTiledOnly = PRO != PRO_BF16 || EPI == EPI_QKV;
-    constexpr bool kHasTiles = EPI == EPI_ADD || EPI == EPI_SWIGLU || EPI == EPI_QKV;     // the matrices that get copies
+    constexpr bool kHasTiles = EPI == EPI_ADD || EPI == EPI_SWIGLU || EPI == EPI_QKV || EPI == EPI_STORE_F32;     // the matrices that get copies
     if constexpr (kHasTiles) {
         if (tiled) {
             if (p.waves == 7) return launch_wide_kernel<MT, EPI, true, 7, PRO>(a, p.grid, stream);
@@ -1634,14 +1634,28 @@ extern "C" int fllm_linear_add_tiled(const void *x, int ldx, const void *w, cons
     return rc;
 }
 
-// out = x w^T (+ bias) for 1..16 bfloat16 rows and a float32 `out` (the vocabulary projection of a decode step), as
+// out = x w^T (+ bias) for 1..64 bfloat16 rows and a float32 `out` (the vocabulary projection of a decode step), as
 // fllm_linear in mode 1, from the tile-major copy of w where the launch it chooses can stream it.
 extern "C" int fllm_linear_f32_tiled(const void *x, int ldx, const void *w, const void *w_tiles, const float *bias, float *out, int ldo,
                                      int M, int N, int K, hipStream_t stream) {
-    FLLM_REQUIRE(M >= 1 && M <= 16 && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && ldx >= K && ldo >= N,
-                 "linear_f32_tiled: takes 1..16 rows, K and ldx in steps of 8 (M=%d N=%d K=%d ldx=%d ldo=%d)", M, N, K, ldx, ldo);
+    FLLM_REQUIRE(M >= 1 && M <= 64 && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && ldx >= K && ldo >= N,
+                 "linear_f32_tiled: takes 1..64 rows, K and ldx in steps of 8 (M=%d N=%d K=%d ldx=%d ldo=%d)", M, N, K, ldx, ldo);
     FLLM_REQUIRE(aligned16(x) && aligned16(w) && out != nullptr && (w_tiles == nullptr || aligned16(w_tiles)),
                  "linear_f32_tiled: operands must be there and 16-byte aligned");
+    if (M > 16) {
+        SkinnyArgs a = {};
+        a.x = x;
+        a.ldx = ldx;
+        a.w = (const bf16_t *)w;
+        a.w_tiles = (const bf16_t *)w_tiles;
+        a.bias = bias;
+        a.out = out;
+        a.ldo = ldo;
+        a.M = M;
+        a.N = N;
+        a.K = K;
+        return dispatch_wide<EPI_STORE_F32>(a, stream);
+    }
     const int rc = fllm_linear_bf16_skinny(x, ldx, w, bias, out, ldo, M, N, K, 1, stream, w_tiles);
     FLLM_REQUIRE(rc != 1, "linear_f32_tiled: shape M=%d K=%d does not fit the staging area", M, K);
     return rc;

@@ -334,7 +334,7 @@ class Ops:
             _dense(bias, "bias", torch.float32, (N,))
         ldx = x.stride(0) if M > 1 else K
         ldo = out.stride(0) if M > 1 else N
-        tiles = self._tiles_of(w) if Ops._tiles and (M <= 64 if mode == OUT_ADD_F32 else mode == OUT_STORE_F32 and M <= 16) else None
+        tiles = self._tiles_of(w) if Ops._tiles and M <= 64 and mode in (OUT_ADD_F32, OUT_STORE_F32) else None
         if tiles is not None and ldx % 8 == 0 and K % 8 == 0:
             entry = self.lib.fllm_linear_add_tiled if mode == OUT_ADD_F32 else self.lib.fllm_linear_f32_tiled
             self._check(entry(_ptr(x), ldx, _ptr(w), _ptr(tiles), _ptr(bias), _ptr(out), ldo, M, N, K, self._stream()))
