@@ -90,11 +90,11 @@ int fllm_linear_add_normed(const void *x, int ldx, const void *w, const float *b
 //   fllm_weight_tiles_supported  1 where the kernels take tiles: N >= 16, K a multiple of 1,024
 //   fllm_weight_tiles_elements   bfloat16 elements of the copy: N rounded up to 16, times K
 //   fllm_tile_weights            writes the copy: [tile of 16 rows][block of 128 columns][k-step of 32][lane][8]
-//   fllm_linear_add_tiled        out += x w^T (+ bias), float32 out, 1..64 rows; with w_tiles where it can
+//   fllm_linear_add_tiled        out += x w^T (+ bias), float32 out, 1..128 rows (beyond 64: w_tiles required, K in steps of 256)
 //   fllm_linear_f32_tiled        out = x w^T (+ bias), float32 out, 1..64 rows (the vocabulary projection); with w_tiles where it can
 //   fllm_tile_weights_gate_up    the copy of [gate; up] ([2 inter][K]) for the SwiGLU epilogue of 17 to 64 rows: tile T holds
 //                                gate rows 8 T .. 8 T + 7 and then the same up rows; fllm_weight_tiles_elements_gate_up elements
-//   fllm_gate_up_swiglu_tiled    fllm_gate_up_swiglu for 17..64 rows with that copy (null: row-major)
+//   fllm_gate_up_swiglu_tiled    fllm_gate_up_swiglu for 17..128 rows with that copy (null: row-major, up to 64 rows)
 int fllm_weight_tiles_supported(int N, int K);
 size_t fllm_weight_tiles_elements(int N, int K);
 int fllm_tile_weights(const void *w, void *tiles, int N, int K, hipStream_t stream);

@@ -50,6 +50,7 @@ __device__ __forceinline__ f32x4_t take_over(__amdgpu_buffer_rsrc_t ws, unsigned
     return (f32x4_t){__uint_as_float(bits[0]), __uint_as_float(bits[1]), __uint_as_float(bits[2]), __uint_as_float(bits[3])};
 }
 
+constexpr int kWideRows = 128;            // the most rows of the kernel that passes the activations through LDS in chunks
 enum { PRO_BF16 = 0, PRO_NORM_F32 = 1, PRO_SCALED = 2 };
 enum { EPI_STORE = 0, EPI_STORE_F32 = 1, EPI_ADD = 2, EPI_QKV = 3, EPI_SWIGLU = 4 };
 
@@ -814,17 +815,18 @@ skinny_wide_kernel(SkinnyArgs a) {
                             for (int t = 0; t < RT; t++) t2[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
                             // the parts of up to eight slices are asked for together (one trip to memory, not one a
                             // slice) and added in slice order; every lane loads, so that no load sits behind a branch
-                            for (int s0 = 0; s0 < S; s0 += 8) {
-                                f32x4_t pv[8][RT];
+                            constexpr int GRP = MT > 4 ? 4 : 8;      // (with more row tiles the registers are needed elsewhere)
+                            for (int s0 = 0; s0 < S; s0 += GRP) {
+                                f32x4_t pv[GRP][RT];
 #pragma unroll
-                                for (int j = 0; j < 8; j++) {
+                                for (int j = 0; j < GRP; j++) {
                                     const int s2 = s0 + j < S ? s0 + j : s0;
                                     const unsigned int src = (unsigned int)(((((size_t)tile * S + s2) * MT + mt2) * RT * kWave + lane) * 16);
 #pragma unroll
                                     for (int t = 0; t < RT; t++) pv[j][t] = take_over(wsb, src + t * kWave * 16);
                                 }
 #pragma unroll
-                                for (int j = 0; j < 8; j++)
+                                for (int j = 0; j < GRP; j++)
 #pragma unroll
                                     for (int t = 0; t < RT; t++)
                                         if (s0 + j < S) t2[t] += pv[j][t];
@@ -1312,10 +1314,14 @@ int launch_wide(SkinnyArgs a, hipStream_t stream) {
     const bool have_ws = fllm_device_workspace(&base, &bytes);
     // workgroups of seven or eight waves only with the weights' tile-major copy (they were measured with it)
     const bool tiled = a.w_tiles != nullptr && a.K % 256 == 0;
+    if (MT > 4 && !tiled) return 1;
+    // more than 64 rows: eight waves share the chunk of activations, which then fills LDS (and the prologue of a
+    // prepared norm has four threads a row)
     const fllm_plan::ChunkPlan p =
-        tiled ? fllm_plan::plan_chunks_balanced(a.K, ntiles, MT, RT, bytes, have_ws, device_cus(), fllm_option_linear_slices(),
-                                                fllm_option_wide_waves())
-              : fllm_plan::plan_chunks(a.K, ntiles, MT, RT, bytes, have_ws, device_cus(), fllm_option_linear_slices(), 4);
+        MT > 4 ? fllm_plan::plan_chunks(a.K, ntiles, MT, RT, bytes, have_ws, device_cus(), fllm_option_linear_slices(), 8)
+        : tiled ? fllm_plan::plan_chunks_balanced(a.K, ntiles, MT, RT, bytes, have_ws, device_cus(), fllm_option_linear_slices(),
+                                                  fllm_option_wide_waves())
+                : fllm_plan::plan_chunks(a.K, ntiles, MT, RT, bytes, have_ws, device_cus(), fllm_option_linear_slices(), 4);
     a.S = p.S;
     a.slice = p.slice;
     if (p.S > 1) {
@@ -1329,15 +1335,19 @@ int launch_wide(SkinnyArgs a, hipStream_t stream) {
     }
     constexpr bool kTiledOnly = PRO != PRO_BF16 || EPI == EPI_QKV;
     constexpr bool kHasTiles = EPI == EPI_ADD || EPI == EPI_SWIGLU || EPI == EPI_QKV || EPI == EPI_STORE_F32;     // the matrices that get copies
-    if constexpr (kHasTiles) {
-        if (tiled) {
-            if (p.waves == 7) return launch_wide_kernel<MT, EPI, true, 7, PRO>(a, p.grid, stream);
-            if (p.waves == 8) return launch_wide_kernel<MT, EPI, true, 8, PRO>(a, p.grid, stream);
-            return launch_wide_kernel<MT, EPI, true, 4, PRO>(a, p.grid, stream);
+    if constexpr (MT > 4) {
+        return launch_wide_kernel<MT, EPI, true, 8, PRO>(a, p.grid, stream);
+    } else {
+        if constexpr (kHasTiles) {
+            if (tiled) {
+                if (p.waves == 7) return launch_wide_kernel<MT, EPI, true, 7, PRO>(a, p.grid, stream);
+                if (p.waves == 8) return launch_wide_kernel<MT, EPI, true, 8, PRO>(a, p.grid, stream);
+                return launch_wide_kernel<MT, EPI, true, 4, PRO>(a, p.grid, stream);
+            }
         }
+        if constexpr (kTiledOnly) return 1;
+        else return launch_wide_kernel<MT, EPI, false, 4, PRO_BF16>(a, p.grid, stream);
     }
-    if constexpr (kTiledOnly) return 1;
-    else return launch_wide_kernel<MT, EPI, false, 4, PRO_BF16>(a, p.grid, stream);
 }
 
 using fllm_plan::SlabPlan;
@@ -1385,7 +1395,14 @@ int dispatch_wide(const SkinnyArgs &a, hipStream_t stream) {
     const int mt = (a.M + 15) / 16;
     if (mt == 2) return launch_wide<2, EPI, PRO>(a, stream);
     if (mt == 3) return launch_wide<3, EPI, PRO>(a, stream);
-    return launch_wide<4, EPI, PRO>(a, stream);
+    if (mt == 4) return launch_wide<4, EPI, PRO>(a, stream);
+    // 65 to 128 rows: six or eight row tiles, from the tile-major copies only, for the feed-forward's two products (the
+    // GEMM library's down projection of this many rows leaves half of the device idle; its other products are as fast)
+    if constexpr (PRO == PRO_BF16 && (EPI == EPI_ADD || EPI == EPI_SWIGLU)) {
+        if (mt <= 6) return launch_wide<6, EPI, PRO>(a, stream);
+        if (mt <= 8) return launch_wide<8, EPI, PRO>(a, stream);
+    }
+    return 1;
 }
 
 template <int PRO, int EPI>
@@ -1592,8 +1609,9 @@ extern "C" int fllm_tile_weights_gate_up(const void *w, void *tiles, int inter, 
 // fllm_gate_up_swiglu for 17..64 rows with the weights' tile-major copy (fllm_tile_weights_gate_up; may be null)
 extern "C" int fllm_gate_up_swiglu_tiled(const void *x, int ldx, const void *w_gate_up, const void *w_tiles, const float *bias, void *out,
                                          int M, int inter, int K, hipStream_t stream) {
-    FLLM_REQUIRE(M >= 17 && M <= 64 && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && inter > 0,
-                 "gate_up_swiglu_tiled: takes 17..64 rows and K, ldx in steps of 8 (M=%d K=%d ldx=%d)", M, K, ldx);
+    FLLM_REQUIRE(M >= 17 && M <= kWideRows && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && inter > 0,
+                 "gate_up_swiglu_tiled: takes 17..128 rows and K, ldx in steps of 8 (M=%d K=%d ldx=%d)", M, K, ldx);
+    FLLM_REQUIRE(M <= 64 || (w_tiles != nullptr && K % 256 == 0), "gate_up_swiglu_tiled: beyond 64 rows it takes the tile-major copy and K in steps of 256 (M=%d K=%d)", M, K);
     FLLM_REQUIRE(aligned16(x) && aligned16(w_gate_up) && (w_tiles == nullptr || aligned16(w_tiles)),
                  "gate_up_swiglu_tiled: operands must be 16-byte aligned");
     SkinnyArgs a = {};
@@ -1614,8 +1632,9 @@ extern "C" int fllm_gate_up_swiglu_tiled(const void *x, int ldx, const void *w_g
 // the tile-major copy of w, which the kernel streams instead where the launch it chooses can.
 extern "C" int fllm_linear_add_tiled(const void *x, int ldx, const void *w, const void *w_tiles, const float *bias, float *out, int ldo,
                                      int M, int N, int K, hipStream_t stream) {
-    FLLM_REQUIRE(M >= 1 && M <= 64 && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && ldx >= K && ldo >= N,
-                 "linear_add_tiled: takes 1..64 rows, K and ldx in steps of 8 (M=%d N=%d K=%d ldx=%d ldo=%d)", M, N, K, ldx, ldo);
+    FLLM_REQUIRE(M >= 1 && M <= kWideRows && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && ldx >= K && ldo >= N,
+                 "linear_add_tiled: takes 1..128 rows, K and ldx in steps of 8 (M=%d N=%d K=%d ldx=%d ldo=%d)", M, N, K, ldx, ldo);
+    FLLM_REQUIRE(M <= 64 || (w_tiles != nullptr && K % 256 == 0), "linear_add_tiled: beyond 64 rows it takes the tile-major copy and K in steps of 256 (M=%d K=%d)", M, K);
     FLLM_REQUIRE(aligned16(x) && aligned16(w) && out != nullptr && (w_tiles == nullptr || aligned16(w_tiles)),
                  "linear_add_tiled: operands must be there and 16-byte aligned");
     SkinnyArgs a = {};
@@ -1664,8 +1683,9 @@ extern "C" int fllm_linear_f32_tiled(const void *x, int ldx, const void *w, cons
 extern "C" int fllm_linear_add_normed(const void *x, int ldx, const void *w, const float *bias, float *out, int M, int N, int K,
                                       const float *next_w, void *next_x, float *next_ssq, int *tiles_out, const void *w_tiles,
                                       hipStream_t stream) {
-    FLLM_REQUIRE(M >= 1 && M <= 64 && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && N >= 16 && N % 16 == 0,
-                 "linear_add_normed: takes 1..64 rows, K and ldx in steps of 8 and N in steps of 16 (M=%d N=%d K=%d ldx=%d)", M, N, K, ldx);
+    FLLM_REQUIRE(M >= 1 && M <= kWideRows && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && N >= 16 && N % 16 == 0,
+                 "linear_add_normed: takes 1..128 rows, K and ldx in steps of 8 and N in steps of 16 (M=%d N=%d K=%d ldx=%d)", M, N, K, ldx);
+    FLLM_REQUIRE(M <= 64 || (w_tiles != nullptr && K % 256 == 0), "linear_add_normed: beyond 64 rows it takes the tile-major copy and K in steps of 256 (M=%d K=%d)", M, K);
     FLLM_REQUIRE(aligned16(x) && aligned16(w) && aligned16(out) && aligned16(next_w) && next_x != nullptr && next_ssq != nullptr &&
                      ((uintptr_t)next_x & 7) == 0 && tiles_out != nullptr && (w_tiles == nullptr || aligned16(w_tiles)),
                  "linear_add_normed: operands must be there and 16-byte aligned");

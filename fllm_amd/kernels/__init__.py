@@ -219,16 +219,17 @@ class Ops:
         held = Ops._tiles.get(w.data_ptr())
         return held[1] if held is not None and held[0] == (w.shape[0], w.shape[1], bool(gate_up)) else None
 
-    # 17 to 64 rows beside the GEMM library: with the tile-major copies the own products of the feed-forward (gate/up
+    # 17 to 128 rows beside the GEMM library: with the tile-major copies the own products of the feed-forward (gate/up
     # with its SwiGLU epilogue, down with the residual sum) are faster than the library's products and the SwiGLU kernel
     # (measured at the 8B sizes, 64 / 32 rows: gate/up 48 / 44 us against 55 / 53, down 34 / 28 against 40 / 31; at the 1B
     # sizes, 67 MB of gate and up weights, the library is 3 % of a 64-row step ahead, hence the same floor on the bytes
     # as for `prefers_own_gate_up`)
     def own_feed_forward(self, rows: int, w_gate_up: torch.Tensor, w_down: torch.Tensor) -> bool:
-        """Whether a bfloat16 step of 17 to 64 rows whose products would go to the GEMM library should take
+        """Whether a bfloat16 step of 17 to 128 rows whose products would go to the GEMM library should take
         `gate_up_swiglu` and `linear(..., accumulate=True)` for its feed-forward instead: when both matrices have their
         tile-major copies."""
-        return (self.library_gemm_from is not None and self.library_gemm_from <= rows <= self.GATE_UP_SWIGLU_ROWS and bool(Ops._tiles)
+        return (self.library_gemm_from is not None and self.library_gemm_from <= rows <= self.GATE_UP_SWIGLU_TILED_ROWS and bool(Ops._tiles)
+                and (rows <= 64 or (w_gate_up.shape[1] % 256 == 0 and w_down.shape[1] % 256 == 0))
                 and w_gate_up.numel() * w_gate_up.element_size() >= self.OWN_GATE_UP_BYTES
                 and self._tiles_of(w_gate_up, gate_up=True) is not None and self._tiles_of(w_down) is not None)
 
@@ -334,8 +335,9 @@ class Ops:
             _dense(bias, "bias", torch.float32, (N,))
         ldx = x.stride(0) if M > 1 else K
         ldo = out.stride(0) if M > 1 else N
-        tiles = self._tiles_of(w) if Ops._tiles and M <= 64 and mode in (OUT_ADD_F32, OUT_STORE_F32) else None
-        if tiles is not None and ldx % 8 == 0 and K % 8 == 0:
+        tiles = (self._tiles_of(w) if Ops._tiles and ((mode == OUT_ADD_F32 and M <= self.ADD_KERNEL_ROWS) or (mode == OUT_STORE_F32 and M <= 64))
+                 else None)
+        if tiles is not None and ldx % 8 == 0 and K % 8 == 0 and (M <= 64 or K % 256 == 0):
             entry = self.lib.fllm_linear_add_tiled if mode == OUT_ADD_F32 else self.lib.fllm_linear_f32_tiled
             self._check(entry(_ptr(x), ldx, _ptr(w), _ptr(tiles), _ptr(bias), _ptr(out), ldo, M, N, K, self._stream()))
             return out
@@ -381,7 +383,10 @@ class Ops:
         return out
 
     PREPARED_NORM_ROWS = 16
-    CHUNK_KERNEL_ROWS = 64   # what those kernels take
+    CHUNK_KERNEL_ROWS = 64   # what those kernels take behind a prepared norm
+    ADD_KERNEL_ROWS = 128    # and as sums into the residual stream or with the SwiGLU epilogue (beyond 64 rows from the tile-major
+                             # copies only): the feed-forward of steps of up to 128 rows, whose down projection the GEMM library
+                             # runs on half of the device (96 / 128 rows of the 8B sizes: 39 / 53 us against 63 / 75)
     CHUNK_ROWS = 48          # steps of 17 to this many rows take the fused forms of the kernels that pass the activations through
                              # LDS in chunks (measured at the 8B sizes: 4 to 5 % of a step at 17 and 32 rows, 1 % at 48; from 49
                              # rows on the library's q/k/v and output products beside the own feed-forward are 1 % faster)
@@ -431,8 +436,8 @@ class Ops:
         _dense(next_norm_weight, "next_norm_weight", torch.float32, (N,))
         if bias is not None:
             _dense(bias, "bias", torch.float32, (N,))
-        _need(1 <= M <= self.CHUNK_KERNEL_ROWS and N % 16 == 0 and K % 8 == 0,
-              f"linear_add_prepare takes 1..64 rows, N in steps of 16 and K in steps of 8, not {M} x {N} x {K}")
+        _need(1 <= M <= self.ADD_KERNEL_ROWS and N % 16 == 0 and K % 8 == 0,
+              f"linear_add_prepare takes 1..128 rows, N in steps of 16 and K in steps of 8, not {M} x {N} x {K}")
         xn = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
         ssq = torch.empty((M * (N // 8),), dtype=torch.float32, device=x.device)
         parts = ctypes.c_int(0)
@@ -480,7 +485,8 @@ class Ops:
                                                       _ptr(out), M, two_i // 2, K, self._stream()))
         return out
 
-    GATE_UP_SWIGLU_ROWS = 64
+    GATE_UP_SWIGLU_ROWS = 64          # from the matrix as the checkpoint has it
+    GATE_UP_SWIGLU_TILED_ROWS = 128   # from its tile-major copy, widths in steps of 256
     # Beside the GEMM library: up to this many rows, and from this many bytes of gate and up weights on, the own
     # product with the SwiGLU epilogue is faster than the library's product and a SwiGLU kernel behind it (measured at
     # 17 and 32 rows: 6.5 and 4.6 us a layer at 235 MB of weights; slower at 64 rows, and at 67 MB of weights).
@@ -503,8 +509,10 @@ class Ops:
         if bias is not None:
             _dense(bias, "bias", torch.float32, (two_i,))
         _dense(out, "out", torch.bfloat16, (M, two_i // 2))
-        _need(1 <= M <= self.GATE_UP_SWIGLU_ROWS and K % 8 == 0, f"gate_up_swiglu takes 1..64 rows and widths in steps of 8, not {M} x {K}")
+        _need(1 <= M <= self.GATE_UP_SWIGLU_TILED_ROWS and K % 8 == 0, f"gate_up_swiglu takes 1..128 rows and widths in steps of 8, not {M} x {K}")
         tiles = self._tiles_of(w_gate_up, gate_up=True) if M >= 17 and Ops._tiles else None
+        _need(M <= 64 or (tiles is not None and K % 256 == 0 and x.stride(0) % 8 == 0),
+              f"gate_up_swiglu takes more than 64 rows only with the tile-major copy of the matrix and widths in steps of 256, not {M} x {K}")
         if tiles is not None and x.stride(0) % 8 == 0:
             self._check(self.lib.fllm_gate_up_swiglu_tiled(_ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(tiles), _ptr(bias), _ptr(out), M,
                                                            two_i // 2, K, self._stream()))

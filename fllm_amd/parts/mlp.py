@@ -89,8 +89,8 @@ class GatedMLP(FeedForward):
         rt, ops = self.rt, self.rt.ops
         rows = h.shape[0]
         start = getattr(ops, "library_gemm_from", None)
-        if (rt.dtype == torch.bfloat16 and rows <= getattr(ops, "GATE_UP_SWIGLU_ROWS", 0) and self.hidden % 8 == 0
-                and h.stride(0) % 8 == 0 and (start is None or rows < start or self._own_products(rows))):
+        if (rt.dtype == torch.bfloat16 and self.hidden % 8 == 0 and h.stride(0) % 8 == 0
+                and (self._own_products(rows) or (rows <= getattr(ops, "GATE_UP_SWIGLU_ROWS", 0) and (start is None or rows < start)))):
             # decode batches that the hand-written products serve: the activation is the epilogue of the gate/up product
             act = rt.empty((rows, self.inter))
             ops.gate_up_swiglu(h, self.w_gate_up, act, bias=self.b_gate_up)

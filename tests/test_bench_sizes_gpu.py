@@ -122,3 +122,6 @@ def test_steps_at_benchmark_sizes(cases, tmp_path, name, dtype):
             assert ops.fused_form(40, cfg["hidden_size"], block.feed_forward.w_gate_up, gate_up=True) == "chunks"
             large = block.feed_forward.w_gate_up.numel() * 2 >= ops.OWN_GATE_UP_BYTES       # small matrices: the library's products
             assert ops.own_feed_forward(64, block.feed_forward.w_gate_up, block.feed_forward.w_down) == large
+            # and so did the whole request of 90 tokens (six row tiles a workgroup), but no step of more than 128 rows
+            assert ops.own_feed_forward(90, block.feed_forward.w_gate_up, block.feed_forward.w_down) == large
+            assert not ops.own_feed_forward(150, block.feed_forward.w_gate_up, block.feed_forward.w_down)

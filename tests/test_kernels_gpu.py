@@ -336,6 +336,48 @@ def test_products_of_17_to_64_rows_that_add_read_the_tile_major_copy(ops, ref, M
     assert torch.equal(four, plain), f"M{M} N{N} K{K}: the tile-major copy gives other sums"
 
 
+@pytest.mark.parametrize("M,N,K,bias", [(65, 4096, 4096, False), (128, 4096, 14336, False), (96, 1000, 2048, True), (100, 24, 1024, True),
+                                        (128, 4104, 3072, False), (97, 2048, 8192, False), (80, 16, 7168, True)])
+def test_products_of_65_to_128_rows(ops, ref, M, N, K, bias):
+    """65 to 128 rows: six or eight row tiles a workgroup of eight waves, from the tile-major copies only, for the two
+    products of the feed-forward.  The sum into the residual stream with and without the preparation of the next norm and
+    gate/up from bfloat16 rows, each against the float64 result; two launches give the same bits; the other forms refuse."""
+    g = gen(61 + M)
+    x = (torch.randn(M, K, generator=g) * 0.5).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).to(DEV)
+    b = (torch.randn(N, generator=g) * 0.1).to(DEV) if bias else None
+    resid = (torch.randn(M, N, generator=g) * torch.rand(M, 1, generator=g) * 6).to(DEV)
+    assert ops.tile_for_decode(w)
+    want = ref.linear(x.cpu(), w.cpu(), resid.double().cpu(), bias=None if b is None else b.cpu(), accumulate=True)
+    mag = (x.double().abs() @ w.double().abs().T).max().item()
+    summed = ops.linear(x, w, resid.clone(), bias=b, accumulate=True)
+    close(summed, want, 1e-6, 4e-7 * mag + 1e-6, f"sum M{M} N{N} K{K}")
+    assert torch.equal(summed, ops.linear(x, w, resid.clone(), bias=b, accumulate=True)), "two launches differ"
+    with pytest.raises(Exception, match="tile-major copy|steps of 256"):
+        ops.gate_up_swiglu(x, torch.zeros(64, K, dtype=torch.bfloat16, device=DEV), torch.empty(M, 32, dtype=torch.bfloat16, device=DEV))
+    if N % 1024 != 0:
+        return
+    nw = (1 + 0.1 * torch.randn(N, generator=g)).to(DEV)
+    assert ops.fused_form(M, K, w) is None and not ops.prepares_norm(M, N, w)      # steps of this many rows do not use it
+    prepared_sum = resid.clone()
+    prepared = ops.linear_add_prepare(x, w, prepared_sum, nw, bias=b)
+    assert torch.equal(prepared_sum, summed)
+    assert torch.equal(prepared.x, (summed * nw).to(torch.bfloat16)) and prepared.parts == N // 16
+    squares = prepared.ssq[:M * prepared.parts].view(M, prepared.parts).double().sum(1)
+    assert float(((squares - summed.double().pow(2).sum(1)).abs() / summed.double().pow(2).sum(1)).max()) < 1e-6
+    inter = 3 * N // 2 + 8
+    wgu = (torch.randn(2 * inter, N, generator=g) / math.sqrt(N)).to(torch.bfloat16).to(DEV)
+    bgu = (torch.randn(2 * inter, generator=g) * 0.1).to(DEV)
+    assert ops.tile_for_decode(wgu, gate_up=True)
+    want_act = ref.norm_gate_up_swiglu(summed.cpu(), nw.cpu(), 1e-5, wgu.cpu(), torch.empty(M, inter, dtype=torch.float64), bias=bgu.cpu())
+    normed = ops.rmsnorm(summed, nw, 1e-5, torch.empty(M, N, dtype=torch.bfloat16, device=DEV))
+    act = ops.gate_up_swiglu(normed, wgu, torch.empty(M, inter, dtype=torch.bfloat16, device=DEV), bias=bgu)
+    close(act, want_act, 2 * BF16_EPS, 4e-2, f"gate/up M{M} N{N}")
+    assert torch.equal(act, ops.gate_up_swiglu(normed, wgu, torch.empty(M, inter, dtype=torch.bfloat16, device=DEV), bias=bgu))
+    with pytest.raises(Exception, match="1..64 rows"):
+        ops.norm_gate_up_swiglu(None, None, 1e-5, wgu, torch.empty(M, inter, dtype=torch.bfloat16, device=DEV), bias=bgu, prepared=prepared)
+
+
 @pytest.mark.parametrize("waves", [0, 4, 7, 8])
 @pytest.mark.parametrize("M,inter,K,bias", [(17, 14336, 4096, False), (64, 14336, 4096, False), (40, 1000, 2048, True), (64, 12, 1024, True),
                                             (29, 8192, 2048, False), (64, 1796, 1024, False)])
@@ -589,7 +631,10 @@ def test_a_product_prepares_the_norm_that_reads_its_sums(ops, ref, M, N, K):
             results.append((q, kp, vp))
         for got, base in zip(results[1], results[0]):
             assert float((got.float() - base.float()).abs().max()) <= 2 * BF16_EPS * float(base.float().abs().max())
-    with pytest.raises(Exception, match="1..64 rows"):
+    with pytest.raises(Exception, match="1..128 rows"):
+        ops.linear_add_prepare(torch.zeros(129, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV),
+                               torch.zeros(129, 32, device=DEV), torch.ones(32, device=DEV))
+    with pytest.raises(Exception, match="tile-major copy"):      # beyond 64 rows only from the copy
         ops.linear_add_prepare(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV),
                                torch.zeros(65, 32, device=DEV), torch.ones(32, device=DEV))
     with pytest.raises(Exception, match="steps of 16"):
