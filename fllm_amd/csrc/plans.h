@@ -71,6 +71,10 @@ inline int resident_groups(const ResidentPlan &p, int ntiles, int cus) {
     int groups = cus * p.per_cu / p.S;
     if (groups < 1) groups = 1;
     if (groups > ntiles) groups = ntiles;
+    // no more workgroups than give every one the same number of tiles: 1,792 tiles on 512 slots are 448 workgroups of 4
+    // tiles, not 256 of 4 beside 256 of 3 that wait for them (gate/up of the 8B sizes at 8 rows: 40.2 -> 39.6 us)
+    const int rounds = (ntiles + groups - 1) / groups;
+    groups = (ntiles + rounds - 1) / rounds;
     return groups;       // the grid is groups * S
 }
 
