@@ -1396,11 +1396,13 @@ int dispatch_wide(const SkinnyArgs &a, hipStream_t stream) {
     if (mt == 2) return launch_wide<2, EPI, PRO>(a, stream);
     if (mt == 3) return launch_wide<3, EPI, PRO>(a, stream);
     if (mt == 4) return launch_wide<4, EPI, PRO>(a, stream);
-    // 65 to 128 rows: six or eight row tiles, from the tile-major copies only, for the feed-forward's two products (the
+    // 65 to 128 rows: five to eight row tiles, from the tile-major copies only, for the feed-forward's two products (the
     // GEMM library's down projection of this many rows leaves half of the device idle; its other products are as fast)
     if constexpr (PRO == PRO_BF16 && (EPI == EPI_ADD || EPI == EPI_SWIGLU)) {
-        if (mt <= 6) return launch_wide<6, EPI, PRO>(a, stream);
-        if (mt <= 8) return launch_wide<8, EPI, PRO>(a, stream);
+        if (mt == 5) return launch_wide<5, EPI, PRO>(a, stream);
+        if (mt == 6) return launch_wide<6, EPI, PRO>(a, stream);
+        if (mt == 7) return launch_wide<7, EPI, PRO>(a, stream);
+        if (mt == 8) return launch_wide<8, EPI, PRO>(a, stream);
     }
     return 1;
 }

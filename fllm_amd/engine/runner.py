@@ -40,9 +40,9 @@ def parse_dtype(name: Union[str, torch.dtype]) -> torch.dtype:
 
 
 # Decode steps are padded to these row counts and replayed as HIP graphs (the reference's
-# buckets: rust/engine/src/rust_decoder.rs:1037; 96 is this engine's own, where the feed-forward's kernels take six row
-# tiles instead of eight: a step of 96 requests 8.7 -> 7.9 ms at the 8B sizes).
-GRAPH_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64, 96, 128, 256)
+# buckets: rust/engine/src/rust_decoder.rs:1037; 80, 96 and 112 are this engine's own, where the feed-forward's kernels
+# take five, six or seven row tiles instead of eight: a step of 96 requests 8.7 -> 7.9 ms at the 8B sizes).
+GRAPH_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64, 80, 96, 112, 128, 256)
 
 
 class StepError(ValueError):

@@ -337,9 +337,10 @@ def test_products_of_17_to_64_rows_that_add_read_the_tile_major_copy(ops, ref, M
 
 
 @pytest.mark.parametrize("M,N,K,bias", [(65, 4096, 4096, False), (128, 4096, 14336, False), (96, 1000, 2048, True), (100, 24, 1024, True),
-                                        (128, 4104, 3072, False), (97, 2048, 8192, False), (80, 16, 7168, True)])
+                                        (128, 4104, 3072, False), (97, 2048, 8192, False), (80, 16, 7168, True), (72, 4096, 14336, False),
+                                        (112, 2048, 4096, False)])
 def test_products_of_65_to_128_rows(ops, ref, M, N, K, bias):
-    """65 to 128 rows: six or eight row tiles a workgroup of eight waves, from the tile-major copies only, for the two
+    """65 to 128 rows: five to eight row tiles a workgroup of eight waves, from the tile-major copies only, for the two
     products of the feed-forward.  The sum into the residual stream with and without the preparation of the next norm and
     gate/up from bfloat16 rows, each against the float64 result; two launches give the same bits; the other forms refuse."""
     g = gen(61 + M)
