@@ -54,7 +54,7 @@ int fllm_set_device_workspace(void *workspace, size_t bytes);
 //                             queries as bfloat16 [M, heads * head_dim] and keys and values into the pages
 //                             (layouts and row/segment/table arguments as fllm_rope_kv_store)
 int fllm_fused_decode_supported(int M, int K);
-// out = silu(x gate^T) * (x up^T) for bfloat16 rows x [M, K] (1..64 rows, row stride ldx), w = [gate; up] ([2 I, K])
+// out = silu(x gate^T) * (x up^T) for bfloat16 rows x [M, K] (1..64 rows, row stride ldx; fllm_gate_up_swiglu_tiled: to 128), w = [gate; up] ([2 I, K])
 int fllm_gate_up_swiglu(const void *x, int ldx, const void *w_gate_up, const float *bias, void *out, int M, int inter,
                         int K, hipStream_t stream);
 int fllm_norm_linear(const float *x, const float *norm_w, float eps, const void *w, const float *bias, void *out, int M,
@@ -67,7 +67,7 @@ int fllm_norm_qkv_rope_store(const float *x, const float *norm_w, float eps, con
                              void *v_pages, int M, int heads, int kv_heads, int head_dim, int K, int page_size,
                              int store_kv, hipStream_t stream);
 
-// A norm prepared by the product before it, for steps of up to 64 rows.  fllm_linear_add_normed: out += x w^T
+// A norm prepared by the product before it, for steps of up to 64 rows (the sum itself: up to 128).  fllm_linear_add_normed: out += x w^T
 // (float32 out [M, N], N a multiple of 16) and, for the RMSNorm that reads out next, next_x = out * next_w as
 // bfloat16 [M, N] and next_ssq [M, *tiles_out]: the sums of squares of out over the outputs of each tile (room for
 // M * N / 8 floats; *tiles_out, host memory, is set at the call).  The scaled forms are the norm forms above with
@@ -84,7 +84,8 @@ int fllm_linear_add_normed(const void *x, int ldx, const void *w, const float *b
 // looks up 64 cache lines for it; from the tile-major copy it is 1 KiB in a row, 8 lines, and the product of 8 or 16 rows
 // takes no longer than that of one (down projection of the 8B sizes: 29 -> 24 us at 8 rows).  The copy costs the
 // matrix's memory a second time, which a GPU with 288 GB affords; row-major stays for the GEMM library's products.
-// Steps of 17 to 64 rows read the copies too (four to eight row tiles a workgroup, the activations through LDS in chunks):
+// Steps of 17 to 64 rows read the copies too (four to eight weight tiles a workgroup, the activations through LDS in chunks;
+// the two products of the feed-forward up to 128 rows):
 // the feed-forward and q/k/v products with their fused prologues and epilogues then beat the library's products and
 // the separate norm, rotary and SwiGLU kernels.
 //   fllm_weight_tiles_supported  1 where the kernels take tiles: N >= 16, K a multiple of 1,024

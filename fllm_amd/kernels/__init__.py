@@ -192,8 +192,8 @@ class Ops:
     def tile_for_decode(self, w: torch.Tensor, gate_up: bool = False) -> bool:
         """Keeps beside `w` (bfloat16 [N, K] on the GPU) a copy in the order in which the products of decode steps read
         it (`fllm_tile_weights`): `linear(..., accumulate=True)`, `linear_add_prepare`, the forms behind a prepared norm
-        and `linear` with float32 logits of up to 16 rows find it by the matrix's address and use it for steps of up to 64
-        rows.  `gate_up`: w is [gate; up] and the copy holds 8 gate rows and the same 8 up rows a tile
+        and `linear` with float32 logits find it by the matrix's address and use it for steps of up to 64 rows (sums into a
+        float32 `out` and `gate_up_swiglu`: up to 128).  `gate_up`: w is [gate; up] and the copy holds 8 gate rows and the same 8 up rows a tile
         (`fllm_tile_weights_gate_up`), for `norm_gate_up_swiglu` and `gate_up_swiglu`.  The copy is given up with `w`.  False: nothing was made (another type or place, a shape the kernels do not take tiles of)."""
         if not (w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()):
             return False
@@ -500,7 +500,8 @@ class Ops:
                 and w_gate_up.numel() * w_gate_up.element_size() >= self.OWN_GATE_UP_BYTES)
 
     def gate_up_swiglu(self, x, w_gate_up, out, bias=None):
-        """out = silu(x @ gate.T) * (x @ up.T) for up to 64 bfloat16 rows; w_gate_up = [gate; up], out bfloat16 [M, I]."""
+        """out = silu(x @ gate.T) * (x @ up.T) for up to 64 bfloat16 rows, up to 128 with the tile-major copy of w_gate_up
+        ([gate; up]); out bfloat16 [M, I]."""
         M, K = x.shape
         two_i = w_gate_up.shape[0]
         _need(two_i % 2 == 0, "w_gate_up needs an even number of rows")

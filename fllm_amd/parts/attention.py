@@ -71,7 +71,7 @@ class PagedAttention(Mixer):
                                 rt.matrix(weights["v"])], dim=0).contiguous()
         self.w_o = rt.matrix(weights["o"])
         rt.tile_for_decode(self.w_o)
-        rt.tile_for_decode(self.w_qkv, priority=1)       # for steps of 17 to 64 rows
+        rt.tile_for_decode(self.w_qkv, priority=1)
         biases = [reorder(None if weights.get("q_bias") is None else rt.vector(weights["q_bias"]), order_q),
                   reorder(None if weights.get("k_bias") is None else rt.vector(weights["k_bias"]), order_k),
                   None if weights.get("v_bias") is None else rt.vector(weights["v_bias"])]

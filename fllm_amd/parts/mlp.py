@@ -27,7 +27,7 @@ class GatedMLP(FeedForward):
         self.w_gate_up = torch.cat([rt.matrix(weights["gate"]), rt.matrix(weights["up"])], dim=0).contiguous()
         self.w_down = rt.matrix(weights["down"])
         rt.tile_for_decode(self.w_down)
-        rt.tile_for_decode(self.w_gate_up, gate_up=True, priority=1)     # for steps of 17 to 64 rows
+        rt.tile_for_decode(self.w_gate_up, gate_up=True, priority=1)
         gb, ub = weights.get("gate_bias"), weights.get("up_bias")
         self.b_gate_up = None
         if gb is not None or ub is not None:
@@ -57,7 +57,7 @@ class GatedMLP(FeedForward):
         return True
 
     def _own_products(self, rows: int) -> bool:
-        """17 to 64 rows: the kernel library may prefer its own products to the GEMM library's (it does when both matrices
+        """17 to 128 rows: the kernel library may prefer its own products to the GEMM library's (it does when both matrices
         have their tile-major copies)."""
         own = getattr(self.rt.ops, "own_feed_forward", None)
         return own is not None and self.rt.dtype == torch.bfloat16 and own(rows, self.w_gate_up, self.w_down)
