@@ -193,8 +193,9 @@ class Ops:
         """Keeps beside `w` (bfloat16 [N, K] on the GPU) a copy in the order in which the products of decode steps read
         it (`fllm_tile_weights`): `linear(..., accumulate=True)`, `linear_add_prepare`, the forms behind a prepared norm
         and `linear` with float32 logits find it by the matrix's address and use it for steps of up to 64 rows (sums into a
-        float32 `out` and `gate_up_swiglu`: up to 128).  `gate_up`: w is [gate; up] and the copy holds 8 gate rows and the same 8 up rows a tile
-        (`fllm_tile_weights_gate_up`), for `norm_gate_up_swiglu` and `gate_up_swiglu`.  The copy is given up with `w`.  False: nothing was made (another type or place, a shape the kernels do not take tiles of)."""
+        float32 `out` and `gate_up_swiglu`: up to 128).  `gate_up`: w is [gate; up] and the copy holds 8 gate rows and the
+        same 8 up rows a tile (`fllm_tile_weights_gate_up`), for `norm_gate_up_swiglu` and `gate_up_swiglu`.  The copy is
+        given up with `w`.  False: nothing was made (another type or place, a shape the kernels do not take tiles of)."""
         if not (w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()):
             return False
         N, K = w.shape
