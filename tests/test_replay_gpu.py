@@ -185,3 +185,31 @@ def test_decode_graphs_and_eager_steps_agree(models, tmp_path, name, dtype):
             assert np.array_equal(a, b), f"{rid}: graph and eager steps differ in float32"
         else:
             assert np.abs(a - b).max() <= TOL[dtype] * np.abs(want).max()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,count", [("A", 100), ("B", 75)])
+def test_decode_steps_of_many_requests(models, tmp_path, name, count, dtype):
+    """Decode steps of 65 to 128 requests are padded to 80, 96, 112 or 128 rows and replayed as graphs like the smaller
+    ones: every request's logits are those of the plain implementation, and the rows that pad a step store nothing."""
+    from fllm_amd.engine import ModelRunner
+    folder, cfg, _, _ = models[name]
+    from safetensors.torch import load_file
+    w64 = tc.to_float64(load_file(os.path.join(folder, "model.safetensors")))
+    lengths = [6 + (i * 7) % 5 for i in range(count)]              # 6 to 10 tokens: requests end at different steps
+    requests = {f"n{i}": tc.random_ids(n, cfg["vocab_size"], 900 + i) for i, n in enumerate(lengths)}
+    plain = {rid: plain_llama.forward(cfg, w64, toks) for rid, toks in requests.items()}
+    head = 4
+    steps = [{"entries": [{"id": rid, "tokens": toks[:head], "want": list(range(head))} for rid, toks in requests.items()], "end": []}]
+    for at in range(head, max(lengths)):
+        live = {rid: toks for rid, toks in requests.items() if len(toks) > at}
+        steps.append({"entries": [{"id": rid, "tokens": [toks[at]], "want": [0]} for rid, toks in live.items()],
+                      "end": [rid for rid, toks in live.items() if len(toks) == at + 1]})
+    runner = ModelRunner.from_folder(folder, dtype=dtype, page_size=tc.PAGE_SIZES[name], max_tokens=count * 64, max_requests=count)
+    got = tt.run_in_process(runner, tt.number(steps), cfg["vocab_size"], str(tmp_path / "many"))
+    check(got, plain, dtype, f"many {name} {dtype}")
+    runner.cache.check_invariants()
+    assert all(pool.available == pool.num_pages for pool in runner.cache.pools)
+    if runner.use_graphs:
+        rows_seen = {key[0] for key in runner._graphs}
+        assert rows_seen & {80, 96, 112, 128}, f"decode graphs of {sorted(rows_seen)} rows ran"
