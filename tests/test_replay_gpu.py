@@ -18,7 +18,7 @@ LENGTHS = {"A": [5, 17, 31, 70, 128, 100], "B": [1, 9, 40, 100, 256, 130], "C": 
            "G": [2, 48, 160, 49, 100, 70]}
 # |engine - plain| <= tol * max|plain logit| ; float32 engine against a float64 reference, and
 # bfloat16 (8 bits of mantissa in weights, activations and cache) against the same.  About three times the largest
-# error any case here has shown on the MI355X (float32 7.0e-7, bfloat16 5.7e-3; the test session prints them).
+# error any case here has shown on the MI355X (float32 7.9e-7, bfloat16 6.0e-3; the test session prints them).
 TOL = {"float32": 3e-6, "bfloat16": 1.5e-2}
 
 
