@@ -147,12 +147,15 @@ def _need(cond: bool, msg: str) -> None:
 
 
 def _dense(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
-    _need(t.is_cuda, f"{name} must be on the GPU")
-    _need(t.is_contiguous(), f"{name} must be contiguous")
-    if dtype is not None:
-        _need(t.dtype == dtype, f"{name} must be {dtype}, is {t.dtype}")
-    if shape is not None:
-        _need(tuple(t.shape) == tuple(shape), f"{name} must have shape {tuple(shape)}, has {tuple(t.shape)}")
+    # (every launch checks its operands: the messages are put together only when a check fails)
+    if not t.is_cuda:
+        raise KernelError(f"{name} must be on the GPU")
+    if not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, is {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{name} must have shape {tuple(shape)}, has {tuple(t.shape)}")
 
 
 class Ops:
@@ -254,8 +257,13 @@ class Ops:
         at zero, partial results behind them), so launches on one device must not overlap: all of them go to one stream
         (a stream that is capturing a graph stands for the stream the graph will be replayed on).  A launch on a second
         stream of the same device is refused."""
-        stream = torch.cuda.current_stream()
-        handle, device = stream.cuda_stream, stream.device_index
+        raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+        if raw is not None:               # the handle without a Stream object around it (a launch asks for it every time)
+            device = torch.cuda.current_device()
+            handle = raw(device)
+        else:
+            stream = torch.cuda.current_stream()
+            handle, device = stream.cuda_stream, stream.device_index
         seen = Ops._streams.get(device)
         if seen is None:
             if not torch.cuda.is_current_stream_capturing():
